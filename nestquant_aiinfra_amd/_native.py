@@ -1,0 +1,98 @@
+"""ctypes binding of libnqhip.so (the C ABI declared in include/nqhip.h).
+
+The library is the only compute path of this package: if it is missing, every
+operator raises.  There is no CPU or eager-PyTorch fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from pathlib import Path
+
+import torch
+
+LIBRARY_PATH = Path(__file__).resolve().parent / "libnqhip.so"
+
+NQ_OK = 0
+NQ_ERR_ARGUMENT = -1
+NQ_ERR_SHAPE = -2
+NQ_ERR_LAUNCH = -3
+NQ_ERR_WORKSPACE = -4
+
+NQ_F32, NQ_BF16, NQ_F16 = 0, 1, 2
+_DTYPE_TAGS = {torch.float32: NQ_F32, torch.bfloat16: NQ_BF16, torch.float16: NQ_F16}
+
+_c = ctypes
+_ptr, _i32, _i64, _size = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_size_t
+
+# name -> (restype, argtypes); must list every symbol include/nqhip.h declares
+SIGNATURES = {
+    "nq_abi_version": (_i32, []),
+    "nq_last_error": (_c.c_char_p, []),
+    "nq_e8_nearest": (_i32, [_ptr, _ptr, _i64, _ptr]),
+    "nq_quantize_rows": (_i32, [_ptr, _i32, _i64, _i64, _i32, _ptr, _i32, _i32, _i64, _i64,
+                                _ptr, _ptr, _ptr, _ptr]),
+    "nq_dequantize_rows": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i64, _i64,
+                                  _ptr, _i32, _ptr]),
+    "nq_w4a4_gemv": (_i32, [_ptr] * 8 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
+                                         _size, _ptr]),
+    "nq_w4a4_gemv_workspace_bytes": (_size, [_i32, _i32, _i32, _i32]),
+}
+
+_LIB: ctypes.CDLL | None = None
+
+
+class NativeLibraryMissing(RuntimeError):
+    pass
+
+
+def library() -> ctypes.CDLL:
+    """Load libnqhip.so once; raise loudly when it has not been built."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    if not LIBRARY_PATH.exists():
+        raise NativeLibraryMissing(
+            f"{LIBRARY_PATH} is missing: build it with `python -m nestquant_aiinfra_amd.build` "
+            "(there is no fallback path)"
+        )
+    lib = ctypes.CDLL(str(LIBRARY_PATH))
+    for name, (restype, argtypes) in SIGNATURES.items():
+        function = getattr(lib, name)
+        function.restype = restype
+        function.argtypes = argtypes
+    _LIB = lib
+    return lib
+
+
+def dtype_tag(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_TAGS[dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dtype}; expected float32, bfloat16 or float16") from None
+
+
+def stream_handle(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def check(status: int) -> None:
+    """Translate a C-ABI status into the exception class the reference raises."""
+    if status == NQ_OK:
+        return
+    message = (library().nq_last_error() or b"").decode("utf-8", "replace")
+    if status in (NQ_ERR_ARGUMENT, NQ_ERR_SHAPE):
+        raise ValueError(message)
+    raise RuntimeError(message)
+
+
+def require_cuda(*tensors: torch.Tensor) -> torch.device:
+    device = tensors[0].device
+    for tensor in tensors:
+        if tensor.device.type != "cuda":
+            raise ValueError("tensors must live on the GPU (device type 'cuda' under ROCm)")
+        if tensor.device != device:
+            raise ValueError("tensors must share one device")
+        if not tensor.is_contiguous():
+            raise RuntimeError("tensors must be contiguous")
+    return device

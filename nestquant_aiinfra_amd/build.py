@@ -1,0 +1,69 @@
+"""Builds libnqhip.so (the gfx950 kernels behind the C ABI in include/nqhip.h) in-tree.
+
+    python -m nestquant_aiinfra_amd.build
+
+hipcc cross-compiles for gfx950 without a GPU.  Flags that are part of the contract:
+  -ffp-contract=off   the codec's float32 operation order is specified; fused
+                      multiply-adds appear only where the source spells fmaf;
+  -fhip-fp32-correctly-rounded-divide-sqrt   IEEE division and sqrt on the device;
+  -packed-fp32-ops off   no packed-FP32 VALU instructions.
+"""
+
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PACKAGE = Path(__file__).resolve().parent
+CSRC = PACKAGE / "csrc"
+LIBRARY = PACKAGE / "libnqhip.so"
+ARCH = "gfx950"
+
+FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC",
+    "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function", "-Wno-unknown-pragmas",
+]
+
+
+def sources() -> list[Path]:
+    return sorted(CSRC.glob("*.hip"))
+
+
+def build(verbose: bool = False) -> Path:
+    """Compile every csrc/*.hip for gfx950 and link libnqhip.so.  Always recompiles."""
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    objects = []
+
+    def compile_one(source: Path) -> Path:
+        obj = source.with_suffix(".o")
+        command = [hipcc, *FLAGS, "-c", str(source), "-o", str(obj)]
+        if verbose:
+            print(" ".join(command), flush=True)
+        result = subprocess.run(command, capture_output=True, text=True)
+        # the host pass warns that it does not know the packed-fp32 feature: harmless
+        noise = "is not a recognized feature for this target"
+        stderr = "\n".join(line for line in result.stderr.splitlines() if noise not in line)
+        if result.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {source.name}:\n{stderr}")
+        if verbose and stderr.strip():
+            print(stderr, file=sys.stderr)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(8, len(sources()) or 1)) as pool:
+        objects = list(pool.map(compile_one, sources()))
+    link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(LIBRARY), *map(str, objects)]
+    result = subprocess.run(link, capture_output=True, text=True)
+    if result.returncode != 0:
+        raise RuntimeError(f"link failed:\n{result.stderr}")
+    for obj in objects:
+        obj.unlink(missing_ok=True)
+    return LIBRARY
+
+
+if __name__ == "__main__":
+    print(build(verbose="-v" in sys.argv))

@@ -1,0 +1,166 @@
+"""NQPK v1: fixed-width, LSB-first byte streams of E8 residue codes and beta ids.
+
+Container layout and error behaviour follow nestquant/core/packing.py:18-225:
+header ``<4sBBHHQQ`` = magic "NQPK", version 1, ndim, q, beta_count, code bytes, beta
+bytes; then ndim little-endian u64 dims; then the two payloads.  Value ``i`` of a flat
+stream occupies bits ``[(i % per_byte) * width, +width)`` of byte ``i // per_byte``.
+"""
+
+from __future__ import annotations
+
+import math
+import struct
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+_HEADER = struct.Struct("<4sBBHHQQ")
+_MAGIC = b"NQPK"
+_VERSION = 1
+
+
+def bits_for_cardinality(cardinality: int) -> int:
+    if cardinality < 1:
+        raise ValueError("cardinality must be positive")
+    return max(1, math.ceil(math.log2(cardinality)))
+
+
+def _ceil_bytes(count: int, width: int) -> int:
+    return (count * width + 7) // 8
+
+
+def _check_cardinalities(q: int, beta_count: int) -> None:
+    if q < 2 or q > 256 or beta_count < 1 or beta_count > 256:
+        raise ValueError("q must be in [2, 256] and beta_count in [1, 256]")
+    if bits_for_cardinality(q) not in (1, 2, 4, 8) or bits_for_cardinality(beta_count) not in (1, 2, 4, 8):
+        raise ValueError("packing format supports only 1, 2, 4, or 8 bits per value")
+
+
+def pack_unsigned(values: np.ndarray, width: int) -> bytes:
+    flat = np.ascontiguousarray(values, dtype=np.uint8).reshape(-1)
+    per_byte = 8 // width
+    padded = np.zeros(_ceil_bytes(flat.size, width) * per_byte, dtype=np.uint8)
+    padded[: flat.size] = flat
+    lanes = padded.reshape(-1, per_byte).astype(np.uint16)
+    shifts = (np.arange(per_byte, dtype=np.uint16) * width)[None, :]
+    return np.bitwise_or.reduce(lanes << shifts, axis=1).astype(np.uint8).tobytes()
+
+
+def unpack_unsigned(payload: bytes, count: int, width: int) -> np.ndarray:
+    if len(payload) != _ceil_bytes(count, width):
+        raise ValueError("payload size does not match expected packed value count")
+    packed = np.frombuffer(payload, dtype=np.uint8)
+    per_byte = 8 // width
+    remainder = count % per_byte
+    if remainder and int(packed[-1]) >> (remainder * width):
+        raise ValueError("nonzero padding bits in packed payload")
+    shifts = (np.arange(per_byte, dtype=np.uint8) * width)[None, :]
+    values = (packed[:, None] >> shifts) & ((1 << width) - 1)
+    return values.reshape(-1)[:count].copy()
+
+
+@dataclass(frozen=True)
+class PackedNestQuantIndices:
+    """Packed residue and beta-index streams of one quantized tensor."""
+
+    shape: tuple[int, ...]
+    q: int
+    beta_count: int
+    code_payload: bytes
+    beta_payload: bytes
+
+    @property
+    def code_bit_width(self) -> int:
+        return bits_for_cardinality(self.q)
+
+    @property
+    def beta_index_bit_width(self) -> int:
+        return bits_for_cardinality(self.beta_count)
+
+    @property
+    def header_bytes(self) -> int:
+        return _HEADER.size + 8 * len(self.shape)
+
+    @property
+    def serialized_bytes(self) -> int:
+        return self.header_bytes + len(self.code_payload) + len(self.beta_payload)
+
+    def to_bytes(self) -> bytes:
+        if len(self.shape) < 2 or len(self.shape) > 255 or any(d < 1 for d in self.shape) or self.shape[-1] != 8:
+            raise ValueError("shape must contain 2 to 255 positive dimensions and end in 8")
+        _check_cardinalities(self.q, self.beta_count)
+        if (len(self.code_payload) != _ceil_bytes(math.prod(self.shape), self.code_bit_width)
+                or len(self.beta_payload) != _ceil_bytes(math.prod(self.shape[:-1]), self.beta_index_bit_width)):
+            raise ValueError("payload lengths do not match tensor shape and bit widths")
+        header = _HEADER.pack(_MAGIC, _VERSION, len(self.shape), self.q, self.beta_count,
+                              len(self.code_payload), len(self.beta_payload))
+        return header + struct.pack(f"<{len(self.shape)}Q", *self.shape) + self.code_payload + self.beta_payload
+
+    @classmethod
+    def from_bytes(cls, data) -> "PackedNestQuantIndices":
+        view = memoryview(data)
+        if len(view) < _HEADER.size:
+            raise ValueError("input is shorter than the NestQuant packing header")
+        magic, version, ndim, q, beta_count, code_len, beta_len = _HEADER.unpack_from(view)
+        if magic != _MAGIC:
+            raise ValueError("invalid NestQuant packing magic")
+        if version != _VERSION:
+            raise ValueError(f"unsupported NestQuant packing version: {version}")
+        if ndim < 2:
+            raise ValueError("packed code shape must include rows and 8D block dimension")
+        _check_cardinalities(q, beta_count)
+        shape_end = _HEADER.size + 8 * ndim
+        if len(view) < shape_end:
+            raise ValueError("truncated tensor shape in packing header")
+        shape = struct.unpack_from(f"<{ndim}Q", view, _HEADER.size)
+        if any(d < 1 for d in shape) or shape[-1] != 8:
+            raise ValueError("shape must be positive and end with E8 dimension 8")
+        if code_len != _ceil_bytes(math.prod(shape), bits_for_cardinality(q)):
+            raise ValueError("residue payload length disagrees with header shape")
+        if beta_len != _ceil_bytes(math.prod(shape[:-1]), bits_for_cardinality(beta_count)):
+            raise ValueError("beta-index payload length disagrees with header shape")
+        if len(view) != shape_end + code_len + beta_len:
+            raise ValueError("packed container has trailing or truncated payload bytes")
+        return cls(tuple(shape), q, beta_count, bytes(view[shape_end:shape_end + code_len]),
+                   bytes(view[shape_end + code_len:]))
+
+    def unpack(self, *, device: torch.device | str = "cpu") -> tuple[torch.Tensor, torch.Tensor]:
+        """Host-side inspection helper: int64 codes ``shape`` and beta ids ``shape[:-1]``."""
+        codes = unpack_unsigned(self.code_payload, math.prod(self.shape), self.code_bit_width)
+        betas = unpack_unsigned(self.beta_payload, math.prod(self.shape[:-1]), self.beta_index_bit_width)
+        if codes.size and int(codes.max()) >= self.q:
+            raise ValueError("decoded residue is outside [0, q)")
+        if betas.size and int(betas.max()) >= self.beta_count:
+            raise ValueError("decoded beta index is outside [0, beta_count)")
+        return (torch.from_numpy(codes.astype(np.int64)).reshape(self.shape).to(device),
+                torch.from_numpy(betas.astype(np.int64)).reshape(self.shape[:-1]).to(device))
+
+
+def pack_nestquant_indices(codes: torch.Tensor, beta_indices: torch.Tensor, *, q: int,
+                           beta_count: int) -> PackedNestQuantIndices:
+    """Pack integer code / beta-id tensors (nestquant/core/packing.py:137-171)."""
+    integer = (torch.int8, torch.uint8, torch.int16, torch.int32, torch.int64)
+    if not isinstance(codes, torch.Tensor) or codes.dtype not in integer:
+        raise TypeError("codes must be an integer torch.Tensor")
+    if not isinstance(beta_indices, torch.Tensor) or beta_indices.dtype not in integer:
+        raise TypeError("beta_indices must be an integer torch.Tensor")
+    if codes.ndim < 2 or codes.shape[-1] != 8:
+        raise ValueError("codes must end in E8 dimension 8")
+    if tuple(beta_indices.shape) != tuple(codes.shape[:-1]):
+        raise ValueError("beta_indices shape must equal codes.shape[:-1]")
+    if q < 2 or q > 256:
+        raise ValueError("q must be in [2, 256]")
+    if beta_count < 1 or beta_count > 256:
+        raise ValueError("beta_count must be in [1, 256]")
+    code_width, beta_width = bits_for_cardinality(q), bits_for_cardinality(beta_count)
+    if code_width not in (1, 2, 4, 8) or beta_width not in (1, 2, 4, 8):
+        raise ValueError("this format version supports only bit widths 1, 2, 4, or 8")
+    for tensor, cardinality in ((codes, q), (beta_indices, beta_count)):
+        if tensor.numel() and (int(tensor.min()) < 0 or int(tensor.max()) >= cardinality):
+            raise ValueError(f"all values must be in [0, {cardinality})")
+    return PackedNestQuantIndices(
+        tuple(codes.shape), q, beta_count,
+        pack_unsigned(codes.detach().to(torch.uint8).cpu().numpy(), code_width),
+        pack_unsigned(beta_indices.detach().to(torch.uint8).cpu().numpy(), beta_width),
+    )

@@ -1,0 +1,183 @@
+"""NQRT v4: one packed NestQuant weight tensor with stateless-dither metadata.
+
+Byte layout follows nestquant/core/tensor_checkpoint.py:28-31, 124-256: header
+``<4sBBIQQQ`` = "NQRT", version, dither mode, len(metadata), len(indices), len(norms),
+len(dither); compact JSON metadata (fixed key order, ``separators=(",", ":")``); an NQPK
+blob of shape ``(rows, features / 8, 8)``; row norms in ``output_dtype``.
+
+Only what the packed execution path consumes is implemented: dither mode 3 (seed +
+``lcg31_mix_v1``) and mode 0 (no dither), versions 2-4.  Records carrying a stored dither
+tensor or a generator state (modes 1, 2) or version 1 are rejected: the packed kernels
+cannot run them either (nestquant/runtime/triton_fused_linear.py:146-165).
+"""
+
+from __future__ import annotations
+
+import json
+import struct
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from .codec import (CURRENT_CODEC_SEMANTICS, LEGACY_CODEC_SEMANTICS, STATELESS_DITHER_ALGORITHM,
+                    STATELESS_MODULUS, UPSTREAM_CODEC_SEMANTICS)
+from .packing import PackedNestQuantIndices
+
+_HEADER = struct.Struct("<4sBBIQQQ")
+_MAGIC = b"NQRT"
+_VERSION = 4
+_DTYPE_TO_NAME = {torch.float16: "float16", torch.bfloat16: "bfloat16",
+                  torch.float32: "float32", torch.float64: "float64"}
+_NAME_TO_DTYPE = {name: dtype for dtype, name in _DTYPE_TO_NAME.items()}
+_NUMPY_VIEW = {torch.float16: np.float16, torch.float32: np.float32, torch.float64: np.float64}
+
+
+def _tensor_to_bytes(tensor: torch.Tensor) -> bytes:
+    tensor = tensor.detach().cpu().contiguous()
+    if tensor.dtype == torch.bfloat16:
+        return tensor.view(torch.int16).numpy().tobytes()
+    return tensor.numpy().tobytes()
+
+
+def _tensor_from_bytes(blob: bytes, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+    if dtype == torch.bfloat16:
+        return torch.from_numpy(np.frombuffer(blob, dtype=np.int16).copy()).view(torch.bfloat16).reshape(shape)
+    return torch.from_numpy(np.frombuffer(blob, dtype=_NUMPY_VIEW[dtype]).copy()).reshape(shape)
+
+
+def _validate_stateless(seed, algorithm) -> None:
+    if isinstance(seed, bool) or not isinstance(seed, int) or not 0 <= seed < STATELESS_MODULUS:
+        raise ValueError("dither_seed must be an integer in [0, 2**31)")
+    if algorithm != STATELESS_DITHER_ALGORITHM:
+        raise ValueError(f"unsupported stateless dither algorithm: {algorithm}")
+
+
+@dataclass(frozen=True)
+class PackedNestQuantTensor:
+    """Self-contained serialized data of one quantized matrix tensor."""
+
+    tensor_name: str
+    indices: PackedNestQuantIndices
+    row_norms: torch.Tensor
+    betas: tuple[float, ...]
+    feature_count: int
+    output_dtype: torch.dtype
+    dither: torch.Tensor | None = None
+    dither_generator_state: bytes | None = None
+    dither_generator_device: str | None = None
+    dither_torch_version: str | None = None
+    dither_seed: int | None = None
+    dither_algorithm: str | None = None
+    codec_semantics: str = CURRENT_CODEC_SEMANTICS
+
+    def _validate(self) -> None:
+        if not self.tensor_name or not isinstance(self.tensor_name, str):
+            raise ValueError("tensor_name must be a nonempty string")
+        if self.dither is not None or self.dither_generator_state is not None:
+            raise ValueError("only seed-based (stateless) dither is supported by the packed path")
+        if self.output_dtype not in _DTYPE_TO_NAME:
+            raise ValueError("unsupported row-norm dtype")
+        rows = self.indices.shape[0]
+        if self.indices.shape != (rows, self.feature_count // 8, 8) or self.feature_count <= 0 or self.feature_count % 8:
+            raise ValueError("metadata feature shape disagrees with packed indices")
+        if tuple(self.row_norms.shape) != (rows,) or self.row_norms.dtype != self.output_dtype:
+            raise ValueError("row norms must be one value per row in output_dtype")
+        if len(self.betas) != self.indices.beta_count:
+            raise ValueError("beta table length disagrees with packed beta_count")
+        if self.codec_semantics not in {UPSTREAM_CODEC_SEMANTICS, LEGACY_CODEC_SEMANTICS}:
+            raise ValueError("unsupported tensor checkpoint codec semantics")
+        if self.dither_seed is not None:
+            _validate_stateless(self.dither_seed, self.dither_algorithm)
+
+    @property
+    def serialized_bytes(self) -> int:
+        return len(self.to_bytes())
+
+    def to_bytes(self) -> bytes:
+        self._validate()
+        dither_mode = 3 if self.dither_seed is not None else 0
+        metadata = json.dumps({
+            "tensor_name": self.tensor_name,
+            "q": self.indices.q,
+            "beta_count": self.indices.beta_count,
+            "betas": list(self.betas),
+            "rows": self.indices.shape[0],
+            "feature_count": self.feature_count,
+            "output_dtype": _DTYPE_TO_NAME[self.output_dtype],
+            "dither_generator_device": None,
+            "dither_torch_version": None,
+            "dither_seed": self.dither_seed,
+            "dither_algorithm": self.dither_algorithm,
+            "codec_semantics": self.codec_semantics,
+        }, ensure_ascii=False, separators=(",", ":")).encode("utf-8")
+        indices_blob = self.indices.to_bytes()
+        norms_blob = _tensor_to_bytes(self.row_norms)
+        header = _HEADER.pack(_MAGIC, _VERSION, dither_mode, len(metadata), len(indices_blob),
+                              len(norms_blob), 0)
+        return header + metadata + indices_blob + norms_blob
+
+    @classmethod
+    def from_bytes(cls, data) -> "PackedNestQuantTensor":
+        view = memoryview(data)
+        if len(view) < 5:
+            raise ValueError("input is shorter than the tensor checkpoint header")
+        if bytes(view[:4]) != _MAGIC:
+            raise ValueError("invalid tensor checkpoint magic")
+        version = int(view[4])
+        if version not in (2, 3, 4):
+            raise ValueError(f"unsupported tensor checkpoint version: {version}")
+        if len(view) < _HEADER.size:
+            raise ValueError("input is shorter than the v2 tensor checkpoint header")
+        _, _, dither_mode, metadata_len, indices_len, norms_len, dither_len = _HEADER.unpack_from(view)
+        if dither_mode not in (0, 1, 2, 3):
+            raise ValueError("invalid dither storage mode")
+        if dither_mode in (1, 2):
+            raise ValueError("stored-dither and generator-state records are not supported by the packed path")
+        offset = _HEADER.size
+        if offset + metadata_len + indices_len + norms_len + dither_len != len(view):
+            raise ValueError("tensor checkpoint payload lengths do not match file size")
+        if dither_len:
+            raise ValueError("dither payload exists for a payload-free mode")
+        try:
+            metadata = json.loads(bytes(view[offset:offset + metadata_len]).decode("utf-8"))
+        except (UnicodeDecodeError, json.JSONDecodeError) as error:
+            raise ValueError("invalid tensor checkpoint metadata") from error
+        offset += metadata_len
+        indices = PackedNestQuantIndices.from_bytes(view[offset:offset + indices_len])
+        offset += indices_len
+        norms_blob = bytes(view[offset:offset + norms_len])
+        try:
+            dtype = _NAME_TO_DTYPE[metadata["output_dtype"]]
+            rows = int(metadata["rows"])
+            features = int(metadata["feature_count"])
+            name = metadata["tensor_name"]
+            betas = tuple(float(value) for value in metadata["betas"])
+        except (KeyError, TypeError, ValueError) as error:
+            raise ValueError("missing or invalid tensor checkpoint metadata fields") from error
+        if not isinstance(name, str):
+            raise ValueError("invalid tensor name")
+        if metadata.get("q") != indices.q or metadata.get("beta_count") != indices.beta_count:
+            raise ValueError("metadata disagrees with packed index parameters")
+        if indices.shape != (rows, features // 8, 8) or features <= 0 or features % 8:
+            raise ValueError("metadata feature shape disagrees with packed indices")
+        if len(norms_blob) != rows * torch.empty((), dtype=dtype).element_size():
+            raise ValueError("row norm payload size disagrees with metadata")
+        seed = metadata.get("dither_seed") if dither_mode == 3 else None
+        algorithm = metadata.get("dither_algorithm") if dither_mode == 3 else None
+        if dither_mode == 3:
+            if version < 4:
+                raise ValueError("stateless dither requires NQRT v4")
+            _validate_stateless(seed, algorithm)
+        semantics = metadata.get("codec_semantics") if version >= 3 else LEGACY_CODEC_SEMANTICS
+        record = cls(tensor_name=name, indices=indices,
+                     row_norms=_tensor_from_bytes(norms_blob, (rows,), dtype), betas=betas,
+                     feature_count=features, output_dtype=dtype, dither_seed=seed,
+                     dither_algorithm=algorithm, codec_semantics=semantics)
+        record._validate()
+        return record
+
+    def dequantize(self, *, device: torch.device | str = "cuda") -> torch.Tensor:
+        """Float32 reconstruction on the GPU (QuantizedRows.dequantize semantics)."""
+        from ..runtime.w4a4_linear import dequantize_record
+        return dequantize_record(self, device=device)

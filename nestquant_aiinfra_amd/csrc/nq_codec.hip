@@ -1,0 +1,321 @@
+// E8 codec kernels: nearest point, row quantiser with multi-beta selection (NQA4 / NQKV4
+// encoder) and its inverse.  Reference: nestquant/core/quantizer.py:214-301, 39-51;
+// nestquant/runtime/nqkv_page.py:97-185, 332-372, 446-456, 22-95; nestquant/runtime/cuda_e8.cu:8-59.
+#include "nq_e8.hip.h"
+#include "nq_host.h"
+
+#include <math.h>
+
+namespace nq {
+
+// ---------------------------------------------------------------------------------------
+// e8_nearest: one lane per vector, two 128-bit loads and stores per lane.
+// ---------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) e8_nearest_kernel(const float4 *x, float4 *out, int64_t count) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    const float4 lo = x[2 * i], hi = x[2 * i + 1];
+    const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    float r[8];
+    e8_nearest(v, r);
+    out[2 * i] = make_float4(r[0], r[1], r[2], r[3]);
+    out[2 * i + 1] = make_float4(r[4], r[5], r[6], r[7]);
+}
+
+// ---------------------------------------------------------------------------------------
+// Row quantiser.
+//
+// A workgroup owns `rows_per_wg` consecutive rows, staged once in LDS as float32.
+//   phase 1  coalesced load (+ promotion) of the rows into LDS;
+//   phase 2  row norms in the reference's order: eight interleaved fused-multiply-add
+//            chains (element i feeds chain i % 8), chains added 0..7, sqrt; eight lanes
+//            per row run the chains, the rest of the workgroup waits;
+//   phase 3  one lane per (block, beta) pair: a quad of lanes evaluates the four betas of
+//            one block, the per-block argmin (first minimum) is a two-step quad exchange,
+//            the winning lane stores the 32-bit code word, and the 2-bit ids of four
+//            neighbouring blocks are merged into one byte with two more exchanges.
+// ---------------------------------------------------------------------------------------
+template <typename T> __device__ __forceinline__ float load_as_f32(const T *p, int64_t i);
+template <> __device__ __forceinline__ float load_as_f32<float>(const float *p, int64_t i) { return p[i]; }
+template <> __device__ __forceinline__ float load_as_f32<uint16_t>(const uint16_t *p, int64_t i) {
+    return bf16_to_f32(p[i]);
+}
+struct half_bits { uint16_t v; };
+template <> __device__ __forceinline__ float load_as_f32<half_bits>(const half_bits *p, int64_t i) {
+    return f16_to_f32(p[i].v);
+}
+
+// exchange with the lane whose id differs in bit 0 / bit 1 (inside a quad)
+__device__ __forceinline__ uint32_t quad_xor1(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+}
+__device__ __forceinline__ uint32_t quad_xor2(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+}
+
+template <typename T, bool kDithered>
+__global__ void __launch_bounds__(1024)
+quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, float inv_q,
+                     const float *__restrict__ betas, int beta_count, float sqrt_n,
+                     uint32_t seed_plus_offset, uint32_t *__restrict__ codes,
+                     uint8_t *__restrict__ beta_ids, float *__restrict__ norms, int rows_per_wg) {
+    extern __shared__ float lds[];
+    float *row_scale = lds + (size_t)rows_per_wg * n;
+    const int tid = threadIdx.x;
+    const int64_t row0 = (int64_t)blockIdx.x * rows_per_wg;
+    const int blocks_per_row = n >> 3;
+
+    // phase 1
+    const int64_t first = row0 * n, limit = rows * (int64_t)n;
+    for (int idx = tid; idx < rows_per_wg * n; idx += blockDim.x) {
+        const int64_t g = first + idx;
+        lds[idx] = g < limit ? load_as_f32<T>(x, g) : 0.0f;
+    }
+    __syncthreads();
+
+    // phase 2
+    if (tid < 8 * rows_per_wg) {
+        const int r = tid >> 3, lane = tid & 7;
+        const float *row = lds + (size_t)r * n + lane;
+        float acc = 0.0f;
+#pragma unroll 8
+        for (int i = 0; i < blocks_per_row; i++) {
+            const float v = row[8 * i];
+            acc = __builtin_fmaf(v, v, acc);
+        }
+        float total = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; k++) total = total + __shfl(acc, (tid & 56) + k, 64);
+        const float norm = __builtin_sqrtf(total);
+        if (lane == 0) {
+            // math.sqrt(n) / norm is evaluated as (1 / norm) * float32(sqrt(n))
+            row_scale[r] = norm > 0.0f ? (1.0f / norm) * sqrt_n : 0.0f;
+            if (row0 + r < rows) norms[row0 + r] = norm;
+        }
+    }
+    __syncthreads();
+
+    // phase 3
+    const int pairs = rows_per_wg * blocks_per_row * 4;
+    for (int p = tid; p < pairs; p += blockDim.x) {
+        const int blk = p >> 2, bi = p & 3;
+        const int r = blk / blocks_per_row, b = blk - r * blocks_per_row;
+        const float scale = row_scale[r];
+        const float4 lo = *reinterpret_cast<const float4 *>(lds + (size_t)r * n + 8 * b);
+        const float4 hi = *reinterpret_cast<const float4 *>(lds + (size_t)r * n + 8 * b + 4);
+        const float raw[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        const bool live = bi < beta_count;
+        const float beta = betas[live ? bi : 0];
+        const int64_t row = row0 + r;
+        const int64_t gblock = row * blocks_per_row + b;
+        float y[8], z[8], code[8], p8[8], recon[8], dither[8];
+        if (kDithered) dither_block(seed_plus_offset + (uint32_t)gblock * 8u, dither);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            y[j] = raw[j] * scale;
+            z[j] = y[j] / beta;                 // IEEE division
+            if (kDithered) z[j] = z[j] + dither[j];
+        }
+        encode_block(z, q, inv_q, code);
+        e8_coset_point(code, p8);
+        if (kDithered) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) p8[j] = p8[j] - dither[j];
+        }
+        reduce_coset_point(p8, q, recon);
+        float err = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float d = recon[j] * beta - y[j];
+            err = err + d * d;
+        }
+        if (!live) err = __builtin_inff();
+
+        // first minimum over the quad: order by (err, beta index)
+        uint32_t best_err = __float_as_uint(err), best = (uint32_t)bi;
+        {
+            const uint32_t oe = quad_xor1(best_err), oi = quad_xor1(best);
+            const float fe = __uint_as_float(oe), me = __uint_as_float(best_err);
+            const bool take = fe < me || (fe == me && oi < best);
+            best_err = take ? oe : best_err;
+            best = take ? oi : best;
+        }
+        {
+            const uint32_t oe = quad_xor2(best_err), oi = quad_xor2(best);
+            const float fe = __uint_as_float(oe), me = __uint_as_float(best_err);
+            const bool take = fe < me || (fe == me && oi < best);
+            best = take ? oi : best;
+        }
+        if (best == (uint32_t)bi && row < rows) codes[gblock] = pack_codeword(code);
+
+        // four consecutive blocks (16 lanes) share one beta byte
+        uint32_t byte = best << (2 * (b & 3));
+        byte |= (uint32_t)__shfl_xor((int)byte, 4, 64);
+        byte |= (uint32_t)__shfl_xor((int)byte, 8, 64);
+        if ((p & 15) == 0 && row < rows) beta_ids[gblock >> 2] = (uint8_t)byte;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Dequantise rows: one lane per block.
+// ---------------------------------------------------------------------------------------
+template <bool kDithered>
+__global__ void __launch_bounds__(256)
+dequantize_rows_kernel(const uint32_t *__restrict__ codes, const uint8_t *__restrict__ beta_ids,
+                       const float *__restrict__ norms, const float *__restrict__ betas,
+                       int64_t blocks, int blocks_per_row, float q, float sqrt_n,
+                       uint32_t seed_plus_offset, void *__restrict__ out, int out_dtype) {
+    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= blocks) return;
+    const int64_t row = g / blocks_per_row;
+    float v[8];
+    decode_codeword<kDithered>(codes[g], q, seed_plus_offset + (uint32_t)g * 8u, v);
+    const float beta = betas[(beta_ids[g >> 2] >> (2 * (g & 3))) & 3];
+    const float scale = norms[row] / sqrt_n;            // IEEE division (tensor / python float)
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = (v[j] * beta) * scale;
+    if (out_dtype == NQ_F32) {
+        float4 *o = reinterpret_cast<float4 *>(out) + 2 * g;
+        o[0] = make_float4(v[0], v[1], v[2], v[3]);
+        o[1] = make_float4(v[4], v[5], v[6], v[7]);
+    } else if (out_dtype == NQ_BF16) {
+        uint4 w;
+        w.x = f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+        w.y = f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+        w.z = f32_to_bf16(v[4]) | ((uint32_t)f32_to_bf16(v[5]) << 16);
+        w.w = f32_to_bf16(v[6]) | ((uint32_t)f32_to_bf16(v[7]) << 16);
+        reinterpret_cast<uint4 *>(out)[g] = w;
+    } else {
+        _Float16 *o = reinterpret_cast<_Float16 *>(out) + 8 * g;
+#pragma unroll
+        for (int j = 0; j < 8; j++) o[j] = (_Float16)v[j];
+    }
+}
+
+}  // namespace nq
+
+extern "C" int nq_e8_nearest(const float *x_dev, float *out_dev, int64_t count, void *stream) {
+    NQ_REQUIRE(count >= 0, NQ_ERR_SHAPE, "nq_e8_nearest: count must be non-negative");
+    if (count == 0) return NQ_OK;
+    NQ_REQUIRE(x_dev && out_dev, NQ_ERR_ARGUMENT, "nq_e8_nearest: null pointer");
+    NQ_REQUIRE(nq::aligned(x_dev, 16) && nq::aligned(out_dev, 16), NQ_ERR_ARGUMENT,
+               "nq_e8_nearest: pointers must be 16-byte aligned");
+    const int threads = 256;
+    const int64_t grid = (count + threads - 1) / threads;
+    NQ_REQUIRE(grid <= 0x7fffffff, NQ_ERR_SHAPE, "nq_e8_nearest: too many vectors");
+    hipLaunchKernelGGL(nq::e8_nearest_kernel, dim3((unsigned)grid), dim3(threads), 0,
+                       (hipStream_t)stream, reinterpret_cast<const float4 *>(x_dev),
+                       reinterpret_cast<float4 *>(out_dev), count);
+    return nq::check_launch("nq_e8_nearest");
+}
+
+namespace {
+
+template <typename T, bool kDithered>
+int launch_quantize(const void *x, int64_t rows, int n, int q, const float *betas, int beta_count,
+                    uint32_t seed_plus_offset, uint8_t *codes, uint8_t *beta_ids, float *norms,
+                    hipStream_t stream) {
+    const int pairs_per_row = n / 2;
+    const int target = pairs_per_row < 256 ? 256 : (pairs_per_row < 1024 ? pairs_per_row : 1024);
+    int rows_per_wg = target / pairs_per_row;
+    if (rows_per_wg < 1) rows_per_wg = 1;
+    if (rows_per_wg > rows) rows_per_wg = (int)rows;
+    int threads = rows_per_wg * pairs_per_row;
+    if (threads > 1024) threads = 1024;
+    if (threads < 64) threads = 64;
+    const size_t lds_bytes = ((size_t)rows_per_wg * n + rows_per_wg) * sizeof(float);
+    auto kernel = nq::quantize_rows_kernel<T, kDithered>;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                (int)lds_bytes);
+        if (status != hipSuccess)
+            return nq::fail(NQ_ERR_LAUNCH, "nq_quantize_rows: cannot reserve %zu bytes of LDS: %s",
+                            lds_bytes, hipGetErrorString(status));
+    }
+    const int64_t grid = (rows + rows_per_wg - 1) / rows_per_wg;
+    if (grid > 0x7fffffff) return nq::fail(NQ_ERR_SHAPE, "nq_quantize_rows: too many rows");
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(threads), lds_bytes, stream,
+                       reinterpret_cast<const T *>(x), rows, n, (float)q, 1.0f / (float)q, betas,
+                       beta_count, (float)sqrt((double)n), seed_plus_offset,
+                       reinterpret_cast<uint32_t *>(codes), beta_ids, norms, rows_per_wg);
+    return nq::check_launch("nq_quantize_rows");
+}
+
+}  // namespace
+
+extern "C" int nq_quantize_rows(const void *x_dev, int x_dtype, int64_t rows, int64_t n, int q,
+                                const float *betas_dev, int beta_count, int has_dither, int64_t seed,
+                                int64_t block_offset, uint8_t *codes_dev, uint8_t *beta_ids_dev,
+                                float *norms_dev, void *stream) {
+    NQ_REQUIRE(rows >= 1 && n >= 1, NQ_ERR_SHAPE, "nq_quantize_rows: rows and n must be positive");
+    NQ_REQUIRE(n % 32 == 0, NQ_ERR_SHAPE,
+               "nq_quantize_rows: feature count %lld must be a multiple of 32", (long long)n);
+    NQ_REQUIRE(n <= 32768, NQ_ERR_SHAPE, "nq_quantize_rows: feature count %lld exceeds 32768",
+               (long long)n);
+    NQ_REQUIRE(q >= 2 && q <= 16, NQ_ERR_SHAPE, "nq_quantize_rows: q must be in [2, 16] for 4-bit codes");
+    NQ_REQUIRE(beta_count >= 1 && beta_count <= 4, NQ_ERR_SHAPE,
+               "nq_quantize_rows: beta_count must be in [1, 4] for 2-bit ids");
+    NQ_REQUIRE(x_dev && betas_dev && codes_dev && beta_ids_dev && norms_dev, NQ_ERR_ARGUMENT,
+               "nq_quantize_rows: null pointer");
+    NQ_REQUIRE(nq::aligned(codes_dev, 4), NQ_ERR_ARGUMENT, "nq_quantize_rows: codes must be 4-byte aligned");
+    uint32_t seed_plus_offset = 0;
+    if (has_dither) {
+        NQ_REQUIRE(seed >= 0 && seed < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
+                   "nq_quantize_rows: seed must be in [0, 2**31)");
+        NQ_REQUIRE(block_offset >= 0 && block_offset + rows * (n / 8) <= ((int64_t)1 << 28), NQ_ERR_SHAPE,
+                   "nq_quantize_rows: block range exceeds the stateless dither counter space");
+        seed_plus_offset = (uint32_t)((uint64_t)seed + (uint64_t)block_offset * 8u);
+    }
+    hipStream_t s = (hipStream_t)stream;
+#define NQ_DISPATCH_QUANTIZE(T)                                                                    \
+    (has_dither ? launch_quantize<T, true>(x_dev, rows, (int)n, q, betas_dev, beta_count,           \
+                                           seed_plus_offset, codes_dev, beta_ids_dev, norms_dev, s) \
+                : launch_quantize<T, false>(x_dev, rows, (int)n, q, betas_dev, beta_count, 0u,      \
+                                            codes_dev, beta_ids_dev, norms_dev, s))
+    switch (x_dtype) {
+        case NQ_F32: return NQ_DISPATCH_QUANTIZE(float);
+        case NQ_BF16: return NQ_DISPATCH_QUANTIZE(uint16_t);
+        case NQ_F16: return NQ_DISPATCH_QUANTIZE(nq::half_bits);
+        default: return nq::fail(NQ_ERR_ARGUMENT, "nq_quantize_rows: unknown dtype tag %d", x_dtype);
+    }
+#undef NQ_DISPATCH_QUANTIZE
+}
+
+extern "C" int nq_dequantize_rows(const uint8_t *codes_dev, const uint8_t *beta_ids_dev,
+                                  const float *norms_dev, const float *betas_dev, int64_t rows,
+                                  int64_t n, int q, int has_dither, int64_t seed,
+                                  int64_t block_offset, void *out_dev, int out_dtype, void *stream) {
+    NQ_REQUIRE(rows >= 1 && n >= 1, NQ_ERR_SHAPE, "nq_dequantize_rows: rows and n must be positive");
+    NQ_REQUIRE(n % 32 == 0, NQ_ERR_SHAPE,
+               "nq_dequantize_rows: feature count %lld must be a multiple of 32", (long long)n);
+    NQ_REQUIRE(q >= 2 && q <= 16, NQ_ERR_SHAPE, "nq_dequantize_rows: q must be in [2, 16]");
+    NQ_REQUIRE(out_dtype == NQ_F32 || out_dtype == NQ_BF16 || out_dtype == NQ_F16, NQ_ERR_ARGUMENT,
+               "nq_dequantize_rows: unknown dtype tag %d", out_dtype);
+    NQ_REQUIRE(codes_dev && beta_ids_dev && norms_dev && betas_dev && out_dev, NQ_ERR_ARGUMENT,
+               "nq_dequantize_rows: null pointer");
+    NQ_REQUIRE(nq::aligned(codes_dev, 4) && nq::aligned(out_dev, 16), NQ_ERR_ARGUMENT,
+               "nq_dequantize_rows: codes need 4-byte and out 16-byte alignment");
+    const int64_t blocks = rows * (n / 8);
+    if (has_dither) {
+        NQ_REQUIRE(seed >= 0 && seed < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
+                   "nq_dequantize_rows: seed must be in [0, 2**31)");
+        NQ_REQUIRE(block_offset >= 0 && block_offset + blocks <= ((int64_t)1 << 28), NQ_ERR_SHAPE,
+                   "nq_dequantize_rows: block range exceeds the stateless dither counter space");
+    }
+    const int threads = 256;
+    const int64_t grid = (blocks + threads - 1) / threads;
+    NQ_REQUIRE(grid <= 0x7fffffff, NQ_ERR_SHAPE, "nq_dequantize_rows: too many blocks");
+    const uint32_t seed_plus_offset = (uint32_t)((uint64_t)seed + (uint64_t)block_offset * 8u);
+    const float sqrt_n = (float)sqrt((double)n);
+    const uint32_t *codes = reinterpret_cast<const uint32_t *>(codes_dev);
+    if (has_dither)
+        hipLaunchKernelGGL(nq::dequantize_rows_kernel<true>, dim3((unsigned)grid), dim3(threads), 0,
+                           (hipStream_t)stream, codes, beta_ids_dev, norms_dev, betas_dev, blocks,
+                           (int)(n / 8), (float)q, sqrt_n, seed_plus_offset, out_dev, out_dtype);
+    else
+        hipLaunchKernelGGL(nq::dequantize_rows_kernel<false>, dim3((unsigned)grid), dim3(threads), 0,
+                           (hipStream_t)stream, codes, beta_ids_dev, norms_dev, betas_dev, blocks,
+                           (int)(n / 8), (float)q, sqrt_n, 0u, out_dev, out_dtype);
+    return nq::check_launch("nq_dequantize_rows");
+}

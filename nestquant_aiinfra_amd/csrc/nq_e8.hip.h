@@ -1,0 +1,186 @@
+// Device-side E8 codec primitives shared by every kernel of the packed W4A4KV4 path.
+//
+// One lane owns one 8-dimensional block: all eight coordinates live in registers, so
+// the nearest-point search needs no cross-lane traffic and its eight-term sums are
+// naturally sequential.  The float32 operation order below is the contract: it
+// reproduces the reference's CPU arithmetic (torch on the host) so that codes, beta
+// ids and every decode of an undithered code agree bit for bit:
+//   * squares are rounded, then added j = 0..7 in order (the translation unit is built
+//     with -ffp-contract=off, so `a + b * b` never fuses);
+//   * divisions are IEEE (correctly rounded), never reciprocal multiplies;
+//   * v_rndne rounds half to even; the first index wins argmax / argmin ties;
+//   * the half-coset residual is (x - 0.5) - rint(x - 0.5);
+//   * equal coset distances select the half-integer coset.
+// Reference semantics: nestquant/core/lattice.py:18-81, nestquant/core/codec.py:30-224.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nq {
+
+// lattice.py:18-34.  Nearest point of D8 (integer vectors with even coordinate sum).
+// `e` returns the residual p - a of the returned point on every coordinate.
+__device__ __forceinline__ void d8_nearest(const float (&p)[8], float (&a)[8], float (&e)[8]) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        a[j] = __builtin_rintf(p[j]);
+        e[j] = p[j] - a[j];          // exact
+        sum = sum + a[j];
+    }
+    // remainder(sum, 2) != 0 without an integer conversion (also right for huge sums)
+    const bool odd = __builtin_amdgcn_fractf(sum * 0.5f) != 0.0f;
+    const float m = fmaxf(fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3]))),
+                          fmaxf(fmaxf(fabsf(e[4]), fabsf(e[5])), fmaxf(fabsf(e[6]), fabsf(e[7]))));
+    bool done = !odd;                // an even sum needs no correction
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const bool hit = !done && (fabsf(e[j]) == m);   // first coordinate with the largest |residual|
+        done = done || hit;
+        const float dir = __builtin_copysignf(1.0f, e[j]);   // residual >= 0 -> +1 (a residual is never -0)
+        const float moved = a[j] + dir;
+        const float moved_e = e[j] - dir;               // == p - moved, both correctly rounded
+        a[j] = hit ? moved : a[j];
+        e[j] = hit ? moved_e : e[j];
+    }
+}
+
+// lattice.py:37-81, tie_break "upstream_half".  Returns the nearest E8 point of x.
+__device__ __forceinline__ void e8_nearest(const float (&x)[8], float (&out)[8]) {
+    float a[8], ea[8], xm[8], b[8], eb[8];
+    d8_nearest(x, a, ea);
+#pragma unroll
+    for (int j = 0; j < 8; j++) xm[j] = x[j] - 0.5f;
+    d8_nearest(xm, b, eb);
+    float da = 0.0f, db = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        b[j] = b[j] + 0.5f;
+        const float t = x[j] - b[j];     // the reference recomputes x - point for both cosets
+        da = da + ea[j] * ea[j];         // ea[j] == x[j] - a[j]
+        db = db + t * t;
+    }
+    const bool pick_a = da < db;         // ties go to the half-integer coset
+#pragma unroll
+    for (int j = 0; j < 8; j++) out[j] = pick_a ? a[j] : b[j];
+}
+
+// Integer generator coordinates of a lattice point (closed form of codec.py:89-96,
+// as in nestquant/runtime/nqkv_page.py:141-148); every step is exact in float32.
+__device__ __forceinline__ void e8_coords(const float (&l)[8], float (&c)[8]) {
+    c[7] = 2.0f * l[7];
+    c[6] = l[6] - l[7];
+#pragma unroll
+    for (int j = 5; j >= 1; j--) c[j] = (l[j] + c[j + 1]) - l[7];
+    c[0] = 0.5f * ((l[0] + c[1]) - l[7]);
+}
+
+// codec.py:30-42: coset point G * c of an integer code (exact).
+__device__ __forceinline__ void e8_coset_point(const float (&c)[8], float (&p)[8]) {
+    const float h = 0.5f * c[7];
+    p[0] = (2.0f * c[0] - c[1]) + h;
+#pragma unroll
+    for (int j = 1; j < 6; j++) p[j] = (c[j] - c[j + 1]) + h;
+    p[6] = c[6] + h;
+    p[7] = h;
+}
+
+// Non-negative residue of an integer-valued float modulo q (torch.remainder, codec.py:97).
+__device__ __forceinline__ float mod_q(float c, float q, float inv_q) {
+    float r = c - q * __builtin_rintf(c * inv_q);   // in [-q/2 - 1, q/2 + 1], exact
+    r = (r < 0.0f) ? r + q : r;
+    r = (r >= q) ? r - q : r;
+    return r;
+}
+
+// Eight 4-bit codes of one block, little-endian nibbles (packing.py:191-208).
+__device__ __forceinline__ void unpack_codeword(uint32_t word, float (&c)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) c[j] = (float)((word >> (4 * j)) & 15u);
+}
+
+__device__ __forceinline__ uint32_t pack_codeword(const float (&c)[8]) {
+    uint32_t word = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) word |= ((uint32_t)c[j]) << (4 * j);
+    return word;
+}
+
+// codec.py:53-102 `encode_nested` for one block: codes in [0, q) as floats.
+__device__ __forceinline__ void encode_block(const float (&x)[8], float q, float inv_q, float (&code)[8]) {
+    float lattice[8], c[8];
+    e8_nearest(x, lattice);
+    e8_coords(lattice, c);
+#pragma unroll
+    for (int j = 0; j < 8; j++) code[j] = mod_q(c[j], q, inv_q);
+}
+
+// codec.py:105-142 `decode_nested` for one block given its coset point (already minus
+// the dither when there is one): the minimum-energy representative p - q * Q(p / q).
+__device__ __forceinline__ void reduce_coset_point(const float (&p)[8], float q, float (&out)[8]) {
+    float z[8], k[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) z[j] = p[j] / q;         // IEEE division
+    e8_nearest(z, k);
+#pragma unroll
+    for (int j = 0; j < 8; j++) out[j] = p[j] - q * k[j]; // exact
+}
+
+// codec.py:213-222 / nestquant/runtime/nqrt4_device.cuh:7-17: lcg31_mix_v1.  Only the
+// low 31 bits of every stage matter, so masks are folded into bit-field extracts.
+__device__ __forceinline__ uint32_t lcg31_mix(uint32_t counter_plus_seed) {
+    uint32_t v = counter_plus_seed;
+    v ^= (v >> 16) & 0x7fffu;                 // bits 16..30 of the masked value
+    v = v * 1103515245u + 12345u;
+    v ^= (v >> 13) & 0x3ffffu;                // bits 13..30
+    v = v * 134775813u + 1u;
+    v ^= (v >> 16) & 0x7fffu;
+    return v & 0x7fffffffu;
+}
+
+// codec.py:222-224: u = float32(v) * 2^-30 in [0, 2], then d = u - Q_E8(u).
+__device__ __forceinline__ void dither_block(uint32_t first_counter_plus_seed, float (&d)[8]) {
+    float u[8], n[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+        u[j] = (float)lcg31_mix(first_counter_plus_seed + (uint32_t)j) * (2.0f / 2147483648.0f);
+    e8_nearest(u, n);
+#pragma unroll
+    for (int j = 0; j < 8; j++) d[j] = u[j] - n[j];
+}
+
+// Decode one packed block to lattice units (no beta / norm scale yet).
+// counter_plus_seed is the low 32 bits of (global_block * 8 + seed); dithered == false
+// skips the dither (activations and KV pages).
+template <bool kDithered>
+__device__ __forceinline__ void decode_codeword(uint32_t word, float q, uint32_t counter_plus_seed,
+                                                float (&out)[8]) {
+    float c[8], p[8];
+    unpack_codeword(word, c);
+    e8_coset_point(c, p);
+    if (kDithered) {
+        float d[8];
+        dither_block(counter_plus_seed, d);
+#pragma unroll
+        for (int j = 0; j < 8; j++) p[j] = p[j] - d[j];
+    }
+    reduce_coset_point(p, q, out);
+}
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t bits) {
+    return __uint_as_float(((uint32_t)bits) << 16);
+}
+
+// float32 -> bfloat16, round to nearest even (finite inputs).
+__device__ __forceinline__ uint16_t f32_to_bf16(float x) {
+    uint32_t bits = __float_as_uint(x);
+    bits += 0x7fffu + ((bits >> 16) & 1u);
+    return (uint16_t)(bits >> 16);
+}
+
+__device__ __forceinline__ float f16_to_f32(uint16_t bits) {
+    return (float)__builtin_bit_cast(_Float16, bits);
+}
+
+}  // namespace nq

@@ -1,0 +1,342 @@
+"""Packed W4A4 operators: NQA4 activation encoder, NQRT4 weight preparation, and the
+linear kernels that consume both without ever materialising a BF16 matrix.
+
+Names, argument meaning and error behaviour mirror the reference's Python surface:
+  quantize_activation_cuda / PreparedNQA4Activation   nestquant/runtime/triton_w4a4_linear.py:489-617
+  prepare_fused_linear / PreparedNQRTLinear           nestquant/runtime/triton_fused_linear.py:135-165
+  can_use_w4a4_* / linear_packed_w4a4_*               nestquant/runtime/cuda_w4a4_mma.py:44-619
+Every operator calls the HIP library through its C ABI; there is no other compute path.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Any, Sequence
+
+import torch
+
+from .. import _native
+from ..core.codec import STATELESS_DITHER_ALGORITHM, UPSTREAM_CODEC_SEMANTICS
+from ..core.packing import PackedNestQuantIndices, bits_for_cardinality
+from ..core.tensor_checkpoint import PackedNestQuantTensor
+
+
+# --------------------------------------------------------------------------------------
+# containers
+# --------------------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class PreparedNQA4Activation:
+    """GPU-resident packed activation rows consumed without BF16 expansion."""
+
+    code_payload: torch.Tensor
+    beta_payload: torch.Tensor
+    row_norms: torch.Tensor
+    beta_table: torch.Tensor
+    original_shape: tuple[int, ...]
+    q: int
+    code_width: int
+    beta_width: int
+    output_dtype: torch.dtype
+
+    @property
+    def token_count(self) -> int:
+        return math.prod(self.original_shape[:-1])
+
+    @property
+    def feature_count(self) -> int:
+        return self.original_shape[-1]
+
+    @property
+    def resident_bytes(self) -> int:
+        return sum(t.numel() * t.element_size()
+                   for t in (self.code_payload, self.beta_payload, self.row_norms, self.beta_table))
+
+
+@dataclass(frozen=True)
+class PreparedNQRTLinear:
+    """GPU-resident packed streams and metadata of one NQRT4 weight."""
+
+    record: Any          # PackedNestQuantTensor (ours or the reference's: same attributes)
+    code_payload: torch.Tensor
+    beta_payload: torch.Tensor
+    row_norms: torch.Tensor
+    beta_table: torch.Tensor
+
+
+# --------------------------------------------------------------------------------------
+# encoders
+# --------------------------------------------------------------------------------------
+
+def _beta_values(betas: Sequence[float]) -> tuple[float, ...]:
+    try:
+        values = tuple(float(value) for value in betas)
+    except (TypeError, ValueError) as error:
+        raise TypeError("betas must be a nonempty sequence of numbers") from error
+    if not values or any(not math.isfinite(value) or value <= 0 for value in values):
+        raise ValueError("betas must be positive finite values")
+    return values
+
+
+def quantize_rows_packed(rows: torch.Tensor, *, q: int, beta_table: torch.Tensor,
+                         dither_seed: int | None = None, block_offset: int = 0
+                         ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Encode ``rows`` [R, n] (float32 / bfloat16 / float16, on the GPU) into packed 4-bit
+    codes, packed 2-bit beta ids and float32 row norms with one kernel launch."""
+    device = _native.require_cuda(rows, beta_table)
+    if rows.ndim != 2:
+        raise ValueError("rows must have shape [rows, features]")
+    count, n = rows.shape
+    codes = torch.empty(count * n // 2, dtype=torch.uint8, device=device)
+    beta_ids = torch.empty(count * n // 32, dtype=torch.uint8, device=device)
+    norms = torch.empty(count, dtype=torch.float32, device=device)
+    _native.check(_native.library().nq_quantize_rows(
+        rows.data_ptr(), _native.dtype_tag(rows.dtype), count, n, q, beta_table.data_ptr(),
+        beta_table.numel(), int(dither_seed is not None), int(dither_seed or 0), block_offset,
+        codes.data_ptr(), beta_ids.data_ptr(), norms.data_ptr(), _native.stream_handle(device)))
+    return codes, beta_ids, norms
+
+
+def quantize_activation_cuda(inputs: torch.Tensor, *, q: int, betas: Sequence[float],
+                             beta_table: torch.Tensor | None = None) -> PreparedNQA4Activation:
+    """Encode floating activations into packed NQA4 payloads on the GPU.
+
+    BF16 / FP16 inputs are promoted to float32 inside the kernel (the reference promotes
+    with ``.float()`` first, triton_w4a4_linear.py:599); results are identical.
+    """
+    if not isinstance(inputs, torch.Tensor) or not inputs.is_floating_point():
+        raise TypeError("inputs must be a floating-point tensor")
+    if inputs.device.type != "cuda" or inputs.ndim < 1 or inputs.numel() == 0:
+        raise ValueError("inputs must be a nonempty CUDA tensor")
+    if inputs.shape[-1] % 8:
+        raise ValueError("activation feature dimension must be divisible by 8")
+    beta_values = _beta_values(betas)
+    code_width = bits_for_cardinality(q)
+    beta_width = bits_for_cardinality(len(beta_values))
+    if code_width not in {1, 2, 4, 8} or beta_width not in {1, 2, 4, 8}:
+        raise ValueError("packed activation fields require 1, 2, 4, or 8 bits")
+    if code_width != 4 or beta_width != 2:
+        raise ValueError("the HIP encoder packs 4-bit codes and 2-bit beta ids (q in [9, 16], 3 or 4 betas)")
+    rows = inputs.reshape(-1, inputs.shape[-1])
+    if rows.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        rows = rows.float()
+    rows = rows.contiguous()
+    if beta_table is None:
+        beta_table = torch.tensor(beta_values, device=inputs.device, dtype=torch.float32)
+    codes, beta_ids, norms = quantize_rows_packed(rows, q=q, beta_table=beta_table)
+    return PreparedNQA4Activation(
+        code_payload=codes, beta_payload=beta_ids, row_norms=norms, beta_table=beta_table,
+        original_shape=tuple(inputs.shape), q=q, code_width=code_width, beta_width=beta_width,
+        output_dtype=inputs.dtype,
+    )
+
+
+def quantize_weight_nqrt4(weight: torch.Tensor, *, q: int = 14, betas: Sequence[float],
+                          dither_seed: int, tensor_name: str = "weight") -> PackedNestQuantTensor:
+    """Quantize an (already rotated) weight [N, K] on the GPU into an NQRT v4 record with
+    stateless dither: the offline step of nestquant/core/quantizer.py:214-301 followed by
+    PackedNestQuantTensor.from_quantized_rows (nestquant/core/tensor_checkpoint.py:59-118)."""
+    if not isinstance(weight, torch.Tensor) or not weight.is_floating_point() or weight.ndim != 2:
+        raise TypeError("weight must be a floating-point matrix")
+    beta_values = _beta_values(betas)
+    table = torch.tensor(beta_values, device=weight.device, dtype=torch.float32)
+    rows = weight.contiguous()
+    dtype = rows.dtype if rows.dtype in (torch.float32, torch.bfloat16, torch.float16) else torch.float32
+    codes, beta_ids, norms = quantize_rows_packed(rows.to(dtype), q=q, beta_table=table,
+                                                  dither_seed=dither_seed)
+    n_out, k = weight.shape
+    indices = PackedNestQuantIndices((n_out, k // 8, 8), q, len(beta_values),
+                                     codes.cpu().numpy().tobytes(), beta_ids.cpu().numpy().tobytes())
+    return PackedNestQuantTensor(
+        tensor_name=tensor_name, indices=indices, row_norms=norms.to(dtype).cpu(), betas=beta_values,
+        feature_count=k, output_dtype=dtype, dither_seed=dither_seed,
+        dither_algorithm=STATELESS_DITHER_ALGORITHM,
+    )
+
+
+def _payload_tensor(payload: bytes, device: torch.device) -> torch.Tensor:
+    return torch.frombuffer(bytearray(payload), dtype=torch.uint8).to(device)
+
+
+def prepare_fused_linear(record: Any, *, device: torch.device | str = "cuda") -> PreparedNQRTLinear:
+    """Copy only the packed NQRT streams and compact metadata to the target GPU."""
+    for attribute in ("indices", "row_norms", "betas", "feature_count", "dither_seed",
+                      "dither_algorithm", "codec_semantics"):
+        if not hasattr(record, attribute):
+            raise TypeError("record must be a PackedNestQuantTensor")
+    target = torch.device(device)
+    if target.type != "cuda" or not torch.cuda.is_available():
+        raise ValueError("fused Linear preparation requires a GPU (device type 'cuda')")
+    if record.dither_seed is None or record.dither_algorithm != STATELESS_DITHER_ALGORITHM:
+        raise ValueError("fused Linear requires NQRT v4 stateless dither")
+    if record.codec_semantics != UPSTREAM_CODEC_SEMANTICS:
+        raise ValueError("fused Linear requires upstream E8 semantics")
+    return PreparedNQRTLinear(
+        record=record,
+        code_payload=_payload_tensor(record.indices.code_payload, target),
+        beta_payload=_payload_tensor(record.indices.beta_payload, target),
+        row_norms=record.row_norms.to(device=target, dtype=torch.float32),
+        beta_table=torch.tensor(record.betas, device=target, dtype=torch.float32),
+    )
+
+
+# --------------------------------------------------------------------------------------
+# decoders (diagnostics and container round trips)
+# --------------------------------------------------------------------------------------
+
+def dequantize_rows_packed(codes: torch.Tensor, beta_ids: torch.Tensor, norms: torch.Tensor,
+                           beta_table: torch.Tensor, *, rows: int, features: int, q: int,
+                           dither_seed: int | None = None, block_offset: int = 0,
+                           output_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    device = _native.require_cuda(codes, beta_ids, norms, beta_table)
+    out = torch.empty((rows, features), dtype=output_dtype, device=device)
+    _native.check(_native.library().nq_dequantize_rows(
+        codes.data_ptr(), beta_ids.data_ptr(), norms.data_ptr(), beta_table.data_ptr(), rows,
+        features, q, int(dither_seed is not None), int(dither_seed or 0), block_offset,
+        out.data_ptr(), _native.dtype_tag(output_dtype), _native.stream_handle(device)))
+    return out
+
+
+def dequantize_record(record: Any, *, device: torch.device | str = "cuda") -> torch.Tensor:
+    prepared = prepare_fused_linear(record, device=device)
+    rows = record.indices.shape[0]
+    return dequantize_rows_packed(prepared.code_payload, prepared.beta_payload, prepared.row_norms,
+                                  prepared.beta_table, rows=rows, features=record.feature_count,
+                                  q=record.indices.q, dither_seed=record.dither_seed)
+
+
+def decode_packed_a4(activation: PreparedNQA4Activation,
+                     output_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """Decode packed NQA4 rows (diagnostic; mirrors decode_packed_a4_triton_diagnostic,
+    triton_w4a4_linear.py:522-556, and decode_a4_m16 of the CUDA extension)."""
+    if not isinstance(activation, PreparedNQA4Activation):
+        raise TypeError("activation must be PreparedNQA4Activation")
+    out = dequantize_rows_packed(
+        activation.code_payload, activation.beta_payload, activation.row_norms,
+        activation.beta_table, rows=activation.token_count, features=activation.feature_count,
+        q=activation.q, output_dtype=output_dtype or activation.output_dtype)
+    return out.reshape(*activation.original_shape)
+
+
+# --------------------------------------------------------------------------------------
+# predicates
+# --------------------------------------------------------------------------------------
+
+def _common_ok(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear,
+               feature_multiple: int, row_multiple: int) -> bool:
+    record = weight.record
+    tensors = (activation.code_payload, activation.beta_payload, activation.row_norms,
+               activation.beta_table, weight.code_payload, weight.beta_payload,
+               weight.row_norms, weight.beta_table)
+    return bool(
+        activation.feature_count == record.feature_count
+        and activation.q == 14 and activation.code_width == 4 and activation.beta_width == 2
+        and activation.beta_table.numel() == 4
+        and record.feature_count % feature_multiple == 0
+        and record.indices.shape[0] % row_multiple == 0
+        and record.indices.q == 14 and record.indices.code_bit_width == 4
+        and record.indices.beta_count == 4 and record.indices.beta_index_bit_width == 2
+        and record.dither_seed is not None
+        and record.dither_algorithm == STATELESS_DITHER_ALGORITHM
+        and record.codec_semantics == UPSTREAM_CODEC_SEMANTICS
+        and all(t.is_contiguous() for t in tensors)
+        and all(t.device == activation.code_payload.device for t in tensors)
+    )
+
+
+# The HIP kernels stream 128-bit words per lane, so K must be a multiple of 32 (the
+# reference's CUDA kernels accept multiples of 8 / 16); rows need no alignment.
+def can_use_w4a4_gemv_m1(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear) -> bool:
+    return activation.token_count == 1 and _common_ok(activation, weight, 32, 1)
+
+
+def can_use_w4a4_mma_small_m(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear) -> bool:
+    return activation.token_count in (2, 4, 8) and _common_ok(activation, weight, 32, 1)
+
+
+# --------------------------------------------------------------------------------------
+# linear kernels, M = 1..8
+# --------------------------------------------------------------------------------------
+
+def _gemv(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *, split_k: int,
+          output_dtype: torch.dtype) -> torch.Tensor:
+    lib = _native.library()
+    device = activation.code_payload.device
+    m, k, n = activation.token_count, activation.feature_count, weight.record.indices.shape[0]
+    out = torch.empty((m, n), dtype=output_dtype, device=device)
+    need = lib.nq_w4a4_gemv_workspace_bytes(m, k, n, split_k)
+    workspace = torch.empty(need, dtype=torch.uint8, device=device) if need else None
+    _native.check(lib.nq_w4a4_gemv(
+        activation.code_payload.data_ptr(), activation.beta_payload.data_ptr(),
+        activation.row_norms.data_ptr(), activation.beta_table.data_ptr(),
+        weight.code_payload.data_ptr(), weight.beta_payload.data_ptr(),
+        weight.row_norms.data_ptr(), weight.beta_table.data_ptr(), m, k, n, 0,
+        int(weight.record.dither_seed), split_k, out.data_ptr(), _native.dtype_tag(output_dtype),
+        None if workspace is None else workspace.data_ptr(), need, _native.stream_handle(device)))
+    return out.reshape(*activation.original_shape[:-1], n)
+
+
+def _kernel_dtype(activation: PreparedNQA4Activation) -> torch.dtype:
+    # BF16 results are rounded once, from the FP32 accumulator, inside the kernel; any
+    # other output dtype goes through FP32 exactly like the reference's `.to(dtype)`.
+    return torch.bfloat16 if activation.output_dtype == torch.bfloat16 else torch.float32
+
+
+def linear_packed_w4a4_gemv_m1(activation: PreparedNQA4Activation,
+                               weight: PreparedNQRTLinear) -> torch.Tensor:
+    """Packed-word direct W4A4 GEMV for one token."""
+    if not can_use_w4a4_gemv_m1(activation, weight):
+        raise ValueError("activation or packed weight is unsupported by W4A4 M1")
+    return _gemv(activation, weight, split_k=0,
+                 output_dtype=_kernel_dtype(activation)).to(activation.output_dtype)
+
+
+def linear_packed_w4a4_gemv_m1_fp32_probe(activation: PreparedNQA4Activation,
+                                          weight: PreparedNQRTLinear) -> torch.Tensor:
+    """The M1 accumulator before output-dtype rounding."""
+    if not can_use_w4a4_gemv_m1(activation, weight):
+        raise ValueError("activation or packed weight is unsupported by W4A4 M1")
+    return _gemv(activation, weight, split_k=0, output_dtype=torch.float32)
+
+
+def linear_packed_w4a4_gemv_m1_splitk_probe(activation: PreparedNQA4Activation,
+                                            weight: PreparedNQRTLinear, *,
+                                            split_k: int) -> torch.Tensor:
+    """Deterministic long-K M1 split-K: slices are reduced in ascending order."""
+    if not can_use_w4a4_gemv_m1(activation, weight):
+        raise ValueError("activation or packed weight is unsupported by W4A4 M1")
+    if split_k not in (2, 4, 8):
+        raise ValueError("split_k must be 2, 4, or 8")
+    return _gemv(activation, weight, split_k=split_k,
+                 output_dtype=_kernel_dtype(activation)).to(activation.output_dtype)
+
+
+def linear_packed_w4a4_gemv_m1_splitk_fp32_probe(activation: PreparedNQA4Activation,
+                                                 weight: PreparedNQRTLinear, *,
+                                                 split_k: int) -> torch.Tensor:
+    if not can_use_w4a4_gemv_m1(activation, weight):
+        raise ValueError("activation or packed weight is unsupported by W4A4 M1")
+    if split_k not in (2, 4, 8):
+        raise ValueError("split_k must be 2, 4, or 8")
+    return _gemv(activation, weight, split_k=split_k, output_dtype=torch.float32)
+
+
+def linear_packed_w4a4_mma_small_m(activation: PreparedNQA4Activation,
+                                   weight: PreparedNQRTLinear) -> torch.Tensor:
+    """M in {2, 4, 8}: each weight block is decoded once and reused by every token."""
+    if not can_use_w4a4_mma_small_m(activation, weight):
+        raise ValueError("activation or packed weight is unsupported by small-M probe")
+    return _gemv(activation, weight, split_k=0,
+                 output_dtype=_kernel_dtype(activation)).to(activation.output_dtype)
+
+
+def linear_packed_w4a4_mma_small_m_splitk_probe(activation: PreparedNQA4Activation,
+                                                weight: PreparedNQRTLinear, *,
+                                                split_k: int) -> torch.Tensor:
+    if not can_use_w4a4_mma_small_m(activation, weight):
+        raise ValueError("activation or packed weight is unsupported by small-M")
+    if split_k not in (2, 4, 8):
+        raise ValueError("split_k must be 2, 4, or 8")
+    return _gemv(activation, weight, split_k=split_k,
+                 output_dtype=_kernel_dtype(activation)).to(activation.output_dtype)

@@ -41,12 +41,13 @@
 /* lattice.py:18-34 `_nearest_even_sum_integer` */
 static void d8_nearest(const float *p, float *out) {
     float residual[8];
-    int parity = 0;
+    float sum = 0.0f;
     for (int j = 0; j < 8; j++) {
         out[j] = rintf(p[j]);                 /* torch.round: half to even */
         residual[j] = p[j] - out[j];
-        parity ^= ((long long)out[j]) & 1;    /* remainder(sum, 2) != 0 */
+        sum = sum + out[j];                   /* rounded.sum(dim=-1), float32 */
     }
+    const int parity = fmodf(sum, 2.0f) != 0.0f;   /* remainder(sum, 2) != 0 */
     int best = 0;
     float best_abs = fabsf(residual[0]);
     for (int j = 1; j < 8; j++) {             /* argmax keeps the first index */

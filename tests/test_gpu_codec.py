@@ -1,0 +1,189 @@
+"""GPU parity of the E8 codec kernels, called through the C ABI, against the CPU oracle
+and the reference's golden vectors.  Integer outputs (codes, beta ids, packed bytes) and
+float32 decodes must be bit-exact; row norms are bit-exact too."""
+
+import hashlib
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ACTIVATION_BETAS, KEY_BETAS, Q, VALUE_BETAS, WEIGHT_BETAS
+from gpu_util import bits, outlier_rows, student_t_rows
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from nestquant_aiinfra_amd.runtime import w4a4_linear
+    assert torch.cuda.is_available()
+    return w4a4_linear
+
+
+def _table(betas):
+    return torch.tensor([float(b) for b in betas], dtype=torch.float32, device="cuda")
+
+
+def _check_rows(rt, oracle, x: torch.Tensor, betas, *, dither_seed=None, dtype=torch.float32):
+    xd = x.to(dtype).cuda()
+    codes, beta_ids, norms = rt.quantize_rows_packed(xd, q=Q, beta_table=_table(betas), dither_seed=dither_seed)
+    xf = xd.float().cpu().numpy()
+    rows, n = xf.shape
+    dither = None if dither_seed is None else oracle.dither_stateless(rows * n // 8, dither_seed).reshape(rows, n // 8, 8)
+    oc, ob, on = oracle.quantize_rows(xf, Q, betas, dither=dither)
+    assert np.array_equal(bits(norms), on)
+    assert np.array_equal(bits(codes), oracle.pack_unsigned(oc, 4))
+    assert np.array_equal(bits(beta_ids), oracle.pack_unsigned(ob, 2))
+    return codes, beta_ids, norms, (oc, ob, on)
+
+
+def test_e8_nearest_matches_golden(golden):
+    from nestquant_aiinfra_amd import _native
+    x = torch.from_numpy(golden["e8_x"]).cuda()
+    out = torch.empty_like(x)
+    _native.check(_native.library().nq_e8_nearest(x.data_ptr(), out.data_ptr(), x.shape[0], 0))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(out), golden["e8_point"])
+
+
+def test_quantize_rows_matches_reference_golden(rt, golden):
+    for name in ("qr64", "qr2048"):
+        x = torch.from_numpy(golden[f"{name}_x"]).cuda()
+        codes, beta_ids, norms = rt.quantize_rows_packed(x, q=Q, beta_table=_table(ACTIVATION_BETAS))
+        assert np.array_equal(bits(norms), golden[f"{name}_norms"]), name
+        assert np.array_equal(bits(codes).reshape(-1, 4).view(np.uint32).reshape(-1),
+                              _pack_words(golden[f"{name}_codes"])), name
+        assert np.array_equal(bits(beta_ids), _pack_ids(golden[f"{name}_beta"])), name
+        rows, n = x.shape
+        deq = rt.dequantize_rows_packed(codes, beta_ids, norms, _table(ACTIVATION_BETAS), rows=rows, features=n, q=Q)
+        assert np.array_equal(bits(deq), golden[f"{name}_deq"]), name
+
+
+def _pack_words(codes):
+    c = codes.reshape(-1, 8).astype(np.uint32)
+    return sum(c[:, j] << (4 * j) for j in range(8)).astype(np.uint32)
+
+
+def _pack_ids(beta):
+    b = beta.reshape(-1, 4).astype(np.uint8)
+    return (b[:, 0] | (b[:, 1] << 2) | (b[:, 2] << 4) | (b[:, 3] << 6)).astype(np.uint8)
+
+
+@pytest.mark.parametrize("rows,n,kind,dtype", [
+    (1, 2048, "student", torch.bfloat16),
+    (8, 8192, "student", torch.bfloat16),
+    (17, 2048, "outlier", torch.bfloat16),
+    (40, 2048, "outlier", torch.float32),
+    (128, 64, "normal", torch.bfloat16),        # one KV page side: 16 tokens x 8 heads
+    (5, 32, "normal", torch.float32),
+    (3, 96, "normal", torch.float16),
+    (2, 16384, "normal", torch.float32),
+])
+def test_quantize_rows_matches_oracle(rt, oracle, rows, n, kind, dtype):
+    if kind == "student":
+        x = student_t_rows(rows, n, seed=rows * 1000 + n)
+    elif kind == "outlier":
+        x = outlier_rows(rows, n, seed=rows * 1000 + n + 1)
+    else:
+        x = torch.from_numpy(np.random.default_rng(n + rows).standard_normal((rows, n)).astype(np.float32))
+    x = torch.from_numpy(oracle.hadamard(x.numpy())) if n & (n - 1) == 0 else x
+    if rows > 2:
+        x[1] = 0.0                                 # a zero row must stay zero
+    _check_rows(rt, oracle, x, ACTIVATION_BETAS, dtype=dtype)
+
+
+def test_quantize_rows_key_value_tables_and_three_betas(rt, oracle):
+    x = torch.from_numpy(np.random.default_rng(77).standard_normal((128, 64)).astype(np.float32))
+    _check_rows(rt, oracle, x, KEY_BETAS, dtype=torch.bfloat16)
+    _check_rows(rt, oracle, x, VALUE_BETAS, dtype=torch.bfloat16)
+    _check_rows(rt, oracle, x, (0.25, 0.5, 1.0))
+
+
+def test_dithered_weight_encoder_matches_golden_record(rt, golden, golden_meta):
+    w = torch.from_numpy(golden["nqrt_w"]).cuda()
+    record = rt.quantize_weight_nqrt4(w, q=Q, betas=WEIGHT_BETAS, dither_seed=golden_meta["nqrt_seed"],
+                                      tensor_name="model.layers.0.self_attn.q_proj.weight")
+    assert np.array_equal(np.frombuffer(record.indices.code_payload, np.uint8), golden["nqrt_code_payload"])
+    assert np.array_equal(np.frombuffer(record.indices.beta_payload, np.uint8), golden["nqrt_beta_payload"])
+    assert np.array_equal(record.row_norms.numpy(), golden["nqrt_norms"])
+    # container bytes are identical to the reference's serialisation
+    assert np.array_equal(np.frombuffer(record.to_bytes(), np.uint8), golden["nqrt_bytes"])
+    assert np.array_equal(bits(record.dequantize(device="cuda")), golden["nqrt_deq"])
+
+
+def test_dithered_encoder_and_decoder_match_oracle(rt, oracle):
+    rng = np.random.default_rng(5)
+    w = oracle.hadamard((0.02 * rng.standard_normal((96, 2048))).astype(np.float32))
+    codes, beta_ids, norms, (oc, ob, on) = _check_rows(rt, oracle, torch.from_numpy(w), WEIGHT_BETAS, dither_seed=20261101)
+    deq = rt.dequantize_rows_packed(codes, beta_ids, norms, _table(WEIGHT_BETAS), rows=96, features=2048, q=Q,
+                                    dither_seed=20261101)
+    assert np.array_equal(bits(deq), oracle.dequantize_rows(oc, ob, on, WEIGHT_BETAS, Q, seed=20261101))
+    # a shard keeps its global block offset (row-parallel split of the same tensor)
+    part = rt.quantize_rows_packed(torch.from_numpy(w[32:64]).cuda(), q=Q, beta_table=_table(WEIGHT_BETAS),
+                                   dither_seed=20261101, block_offset=32 * 256)
+    assert np.array_equal(bits(part[0]), bits(codes).reshape(96, -1)[32:64].reshape(-1))
+
+
+def test_undithered_decode_matches_golden_boundary_blocks(rt, golden):
+    codes = golden["decode_codes"]                       # [8195, 8]; pad to a multiple of 4 blocks
+    pad = (-codes.shape[0]) % 4
+    codes = np.concatenate([codes, np.zeros((pad, 8), np.uint8)])
+    words = torch.from_numpy(_pack_words(codes).view(np.uint8).copy()).cuda()
+    blocks = codes.shape[0]
+    ids = torch.zeros(blocks // 4, dtype=torch.uint8, device="cuda")
+    # one "row" of n = 8 * blocks features with norm sqrt(n) and beta 1 leaves lattice units
+    n = 8 * blocks
+    norm = torch.tensor([np.sqrt(np.float64(n))], dtype=torch.float32, device="cuda")
+    table = torch.tensor([1.0, 1.0, 1.0, 1.0], dtype=torch.float32, device="cuda")
+    out = rt.dequantize_rows_packed(words, ids, norm, table, rows=1, features=n, q=Q)
+    expect = golden["decode_out"]
+    got = bits(out).reshape(-1, 8)[: expect.shape[0]]
+    scale = np.float32(norm.item()) / np.float32(np.sqrt(np.float64(n)))
+    assert scale == 1.0
+    assert np.array_equal(got, expect)
+
+
+def test_config1_full_size_payload_hashes(rt, oracle, golden_meta):
+    """2048 x 2048 plumbing case at full size: SHA-256 of the packed streams equals the
+    reference's, for the undithered (A4) and the dithered (NQRT4) encoder."""
+    ref = golden_meta["config1"]
+    g = torch.Generator().manual_seed(58)
+    x0 = torch.randn(2048, 2048, generator=g)
+    signs = (2 * torch.randint(0, 2, (2048,), generator=g) - 1).float()
+    xr = torch.from_numpy(oracle.hadamard((x0 * signs).numpy()))
+    assert hashlib.sha256(xr.numpy().tobytes()).hexdigest() == ref["input_sha256"]
+    sha = lambda t: hashlib.sha256(bits(t).tobytes()).hexdigest()
+    codes, beta_ids, norms = rt.quantize_rows_packed(xr.cuda(), q=Q, beta_table=_table(ACTIVATION_BETAS))
+    assert sha(codes) == ref["A_code_sha256"]
+    assert sha(beta_ids) == ref["A_beta_sha256"]
+    assert sha(norms) == ref["A_norm_sha256"]
+    codes, beta_ids, _ = rt.quantize_rows_packed(xr.cuda(), q=Q, beta_table=_table(WEIGHT_BETAS),
+                                                 dither_seed=ref["dither_seed"])
+    assert sha(codes) == ref["B_code_sha256"]
+    assert sha(beta_ids) == ref["B_beta_sha256"]
+
+
+def test_largest_prefill_activation_is_bit_exact_and_decodes_close(rt, oracle):
+    """The benchmark's largest activation (384 x 8192, outlier channels, rotated) at full
+    size: bit-exact against the oracle, and the decode is a 4-bit-quality reconstruction."""
+    x = torch.from_numpy(oracle.hadamard(outlier_rows(384, 8192, seed=3001).numpy()))
+    codes, beta_ids, norms, _ = _check_rows(rt, oracle, x, ACTIVATION_BETAS, dtype=torch.bfloat16)
+    deq = rt.dequantize_rows_packed(codes, beta_ids, norms, _table(ACTIVATION_BETAS), rows=384, features=8192, q=Q)
+    xf = x.to(torch.bfloat16).float().cuda()
+    rel = (deq - xf).norm(dim=1) / xf.norm(dim=1)
+    assert torch.isfinite(deq).all() and float(rel.max()) < 0.12
+
+
+def test_errors_are_reported_like_the_reference(rt):
+    x = torch.randn(2, 40, device="cuda")
+    with pytest.raises(ValueError):
+        rt.quantize_rows_packed(x, q=Q, beta_table=_table(ACTIVATION_BETAS))      # 40 % 32 != 0
+    with pytest.raises(ValueError):
+        rt.quantize_activation_cuda(torch.randn(2, 12, device="cuda"), q=Q, betas=ACTIVATION_BETAS)
+    with pytest.raises(TypeError):
+        rt.quantize_activation_cuda(torch.zeros(2, 16, dtype=torch.int32, device="cuda"), q=Q, betas=ACTIVATION_BETAS)
+    with pytest.raises(ValueError):
+        rt.quantize_activation_cuda(torch.randn(2, 32), q=Q, betas=ACTIVATION_BETAS)  # CPU tensor
+    with pytest.raises(RuntimeError, match="contiguous"):
+        rt.quantize_rows_packed(torch.randn(64, 4, device="cuda").t(), q=Q, beta_table=_table(ACTIVATION_BETAS))

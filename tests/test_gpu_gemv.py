@@ -1,0 +1,127 @@
+"""GPU parity of the packed W4A4 decode linear (M = 1..8), through the C ABI.
+
+Bar: max |y - y_ref| / max |y_ref| <= 1e-2 against the oracle's decode-then-FP32 matmul
+(the reference's own acceptance for this product is atol .02-.04 / rtol .01 between its
+kernels, tests/unit/runtime/test_cuda_w4a4_mma.py:99-133).  A second, tighter check
+compares with the same product taken on BF16-rounded operands (what every reference
+kernel multiplies): <= 2e-3, which leaves only the FP32 accumulation order.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ACTIVATION_BETAS, Q, WEIGHT_BETAS
+from gpu_util import bits, oracle_weight, relative_error, student_t_rows
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = 1e-2
+BF16_TOLERANCE = 2e-3
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from nestquant_aiinfra_amd.runtime import w4a4_linear
+    return w4a4_linear
+
+
+def _record(rt, codes, beta, norms, k, seed):
+    from nestquant_aiinfra_amd.core.packing import PackedNestQuantIndices
+    from nestquant_aiinfra_amd.core.tensor_checkpoint import PackedNestQuantTensor
+    import oracle as o
+    n_out = norms.shape[0]
+    indices = PackedNestQuantIndices((n_out, k // 8, 8), Q, 4, o.pack_unsigned(codes, 4).tobytes(),
+                                     o.pack_unsigned(beta, 2).tobytes())
+    return PackedNestQuantTensor("w", indices, torch.from_numpy(norms), tuple(WEIGHT_BETAS), k, torch.float32,
+                                 dither_seed=seed, dither_algorithm="lcg31_mix_v1")
+
+
+def _references(oracle, activation, rt, wc, wb, wn, seed):
+    """(FP32-operand reference, BF16-operand reference) from the oracle's decodes."""
+    m, k = activation.token_count, activation.feature_count
+    a_codes = oracle.unpack_unsigned(bits(activation.code_payload), m * k, 4)
+    a_beta = oracle.unpack_unsigned(bits(activation.beta_payload), m * k // 8, 2)
+    a_hat = oracle.dequantize_rows(a_codes, a_beta, bits(activation.row_norms), ACTIVATION_BETAS, Q)
+    w_hat = oracle.dequantize_rows(wc, wb, wn, WEIGHT_BETAS, Q, seed=seed)
+    return oracle.matmul_nt(a_hat, w_hat), oracle.matmul_nt(oracle.bf16_round(a_hat), oracle.bf16_round(w_hat))
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("k,n_out", [(256, 64), (2048, 136), (4096, 40)])
+def test_small_shapes_match_oracle(rt, oracle, m, k, n_out):
+    seed = 20261101 + m
+    _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=1000 + k + n_out, dither_seed=seed)
+    weight = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
+    x = torch.from_numpy(oracle.hadamard(student_t_rows(m, k, seed=2001 + m).numpy())).to(torch.bfloat16).cuda()
+    activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS)
+    ref32, ref16 = _references(oracle, activation, rt, wc, wb, wn, seed)
+    y = rt._gemv(activation, weight, split_k=0, output_dtype=torch.float32)
+    assert relative_error(bits(y), ref32) <= TOLERANCE
+    assert relative_error(bits(y), ref16) <= BF16_TOLERANCE
+    y16 = rt._gemv(activation, weight, split_k=0, output_dtype=torch.bfloat16)
+    assert relative_error(bits(y16.float()), ref32) <= TOLERANCE
+    if k >= 512:
+        for split in (2, 4, 8):
+            if (k // split) % 32:
+                continue
+            ys = rt._gemv(activation, weight, split_k=split, output_dtype=torch.float32)
+            assert relative_error(bits(ys), ref16) <= BF16_TOLERANCE
+            again = rt._gemv(activation, weight, split_k=split, output_dtype=torch.float32)
+            assert torch.equal(ys, again)                     # deterministic reduction
+
+
+@pytest.mark.parametrize("name,k,n_out,wseed,dseed", [("q_proj", 2048, 2048, 1001, 20261101),
+                                                      ("down_proj", 8192, 2048, 1002, 20261102)])
+def test_llama_1b_projection_shapes(rt, oracle, name, k, n_out, wseed, dseed):
+    """Full-size decode shapes, M = 1 and M = 8, weights encoded on the GPU."""
+    rng = np.random.default_rng(wseed)
+    w = torch.from_numpy(oracle.hadamard((0.02 * rng.standard_normal((n_out, k))).astype(np.float32)))
+    record = rt.quantize_weight_nqrt4(w.cuda(), q=Q, betas=WEIGHT_BETAS, dither_seed=dseed, tensor_name=name)
+    weight = rt.prepare_fused_linear(record, device="cuda")
+    wc = oracle.unpack_unsigned(np.frombuffer(record.indices.code_payload, np.uint8), n_out * k, 4)
+    wb = oracle.unpack_unsigned(np.frombuffer(record.indices.beta_payload, np.uint8), n_out * k // 8, 2)
+    wn = record.row_norms.numpy()
+    for m in (1, 8):
+        x = torch.from_numpy(oracle.hadamard(student_t_rows(m, k, seed=2001).numpy())).to(torch.bfloat16).cuda()
+        activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS)
+        ref32, ref16 = _references(oracle, activation, rt, wc, wb, wn, dseed)
+        fn = rt.linear_packed_w4a4_gemv_m1 if m == 1 else rt.linear_packed_w4a4_mma_small_m
+        y = fn(activation, weight)
+        assert y.dtype == torch.bfloat16 and tuple(y.shape) == (m, n_out)
+        assert relative_error(bits(y.float()), ref32) <= TOLERANCE
+        if m == 1:
+            y32 = rt.linear_packed_w4a4_gemv_m1_fp32_probe(activation, weight)
+            assert relative_error(bits(y32), ref16) <= BF16_TOLERANCE
+            ys = rt.linear_packed_w4a4_gemv_m1_splitk_fp32_probe(activation, weight, split_k=8)
+            assert relative_error(bits(ys), ref16) <= BF16_TOLERANCE
+
+
+def test_linearity_in_the_row_norm(rt, oracle):
+    """Scaling an activation's row norm scales its output row (size-independent property)."""
+    k, n_out, seed = 2048, 64, 20261103
+    _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=3, dither_seed=seed)
+    weight = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
+    x = student_t_rows(2, k, seed=4).cuda()
+    a = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS)
+    y1 = rt._gemv(a, weight, split_k=1, output_dtype=torch.float32)
+    import dataclasses
+    a2 = dataclasses.replace(a, row_norms=a.row_norms * 2.0)        # power of two: exact in BF16 and FP32
+    y2 = rt._gemv(a2, weight, split_k=1, output_dtype=torch.float32)
+    assert torch.equal(y2, 2.0 * y1)
+
+
+def test_predicates_and_errors(rt, oracle):
+    k, n_out, seed = 256, 16, 7
+    _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=3, dither_seed=seed)
+    weight = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
+    a1 = rt.quantize_activation_cuda(torch.randn(1, k, device="cuda"), q=Q, betas=ACTIVATION_BETAS)
+    a3 = rt.quantize_activation_cuda(torch.randn(3, k, device="cuda"), q=Q, betas=ACTIVATION_BETAS)
+    assert rt.can_use_w4a4_gemv_m1(a1, weight) and not rt.can_use_w4a4_gemv_m1(a3, weight)
+    assert not rt.can_use_w4a4_mma_small_m(a3, weight)
+    with pytest.raises(ValueError):
+        rt.linear_packed_w4a4_gemv_m1(a3, weight)
+    with pytest.raises(ValueError):
+        rt.linear_packed_w4a4_gemv_m1_splitk_probe(a1, weight, split_k=3)
+    other = rt.quantize_activation_cuda(torch.randn(1, 512, device="cuda"), q=Q, betas=ACTIVATION_BETAS)
+    assert not rt.can_use_w4a4_gemv_m1(other, weight)
