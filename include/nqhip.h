@@ -63,6 +63,9 @@ int nq_e8_nearest(const float *x_dev, float *out_dev, int64_t count, void *strea
  * block_offset + r * n/8 + b and `seed` is added before the lattice search and removed
  * after it: this is the NQRT4 weight encoder (nestquant/core/quantizer.py:214-301 with
  * generate_e8_dither_stateless, nestquant/core/codec.py:176-224).
+ * decoded_bf16_dev (optional, may be NULL): BF16 [rows, n] decode of the stored codes,
+ * bf16((decode * beta) * (norm / sqrt(n))), which the linear kernels accept in place of
+ * decoding the packed activation again.
  * Requires n % 32 == 0, n <= 32768, 2 <= q <= 16.
  * Replaces: _quantize_rows_cuda_fused + _nqkv_encode_kernel + _pack_unsigned_cuda,
  * nestquant/runtime/nqkv_page.py:332-372, 97-185, 446-456 (called by
@@ -72,7 +75,7 @@ int nq_e8_nearest(const float *x_dev, float *out_dev, int64_t count, void *strea
 int nq_quantize_rows(const void *x_dev, int x_dtype, int64_t rows, int64_t n, int q,
                      const float *betas_dev, int beta_count, int has_dither, int64_t seed,
                      int64_t block_offset, uint8_t *codes_dev, uint8_t *beta_ids_dev,
-                     float *norms_dev, void *stream);
+                     float *norms_dev, void *decoded_bf16_dev, void *stream);
 
 /*
  * Inverse of nq_quantize_rows: out[r, :] = (decode(codes) * beta[id]) * (norm[r] / sqrt(n)).
@@ -91,26 +94,54 @@ int nq_dequantize_rows(const uint8_t *codes_dev, const uint8_t *beta_ids_dev,
 
 /*
  * Packed W4A4 linear for decode, M = 1..8 tokens: y[m, n] = sum_k bf16(a[m, k]) * bf16(w[n, k]),
- * FP32 accumulation, both operands decoded in registers from their packed streams
- * (weights with regenerated dither; counter = weight_offset * 8 + n * K + k).
- *   act_*    NQA4 streams of [M, K]  (codes M*K/2 B, beta ids M*K/32 B, norms f32[M], betas f32[4])
- *   w_*      NQRT4 streams of [N, K] (codes N*K/2 B, beta ids N*K/32 B, norms f32[N], betas f32[4])
- *   out_dev  [M, N] of out_dtype (NQ_F32 or NQ_BF16)
- *   split_k  1, 2, 4 or 8 slices of K reduced in ascending order (deterministic); 0 lets
- *            the library choose.  split_k > 1 needs nq_w4a4_gemv_workspace_bytes() bytes.
- * Requires q = 14, K % 256 == 0, (K / split_k) % 256 == 0, 1 <= M <= 8.
+ * FP32 accumulation; the weight is decoded in registers from its packed stream (dither
+ * regenerated; counter = weight_offset * 8 + n * K + k).
+ *   act_*            NQA4 streams of [M, K] (codes M*K/2 B, beta ids M*K/32 B, norms f32[M], betas f32[4])
+ *   act_decoded_dev  optional BF16 [M, K] decode of the same activation (from nq_quantize_rows);
+ *                    when NULL the packed streams are decoded once into the workspace,
+ *                    when given the packed streams may be NULL
+ *   w_*              NQRT4 streams of [N, K] (codes N*K/2 B, beta ids N*K/32 B, norms f32[N], betas f32[4])
+ *   out_dev          [M, N] of out_dtype (NQ_F32 or NQ_BF16)
+ *   split_k          1, 2, 4 or 8 slices of K reduced in ascending order (deterministic); 0 lets
+ *                    the library choose
+ *   workspace_dev    at least nq_w4a4_gemv_workspace_bytes() bytes, 16-byte aligned (may be
+ *                    NULL when that is 0)
+ * Requires q = 14, K % 32 == 0, (K / split_k) % 32 == 0, 1 <= M <= 8.
  * Replaces: run_m1 / run_m1_splitk_probe / run_small_m / run_small_m_splitk_probe of the
  * torch extension, nestquant/runtime/nqrt4_w4a4_mma_binding.cpp:3-46, kernels
  * nestquant/runtime/nqrt4_w4a4_mma.cu:901-947, 952-1001, 411-420, 229-286.
  */
 int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
                  const float *act_norms_dev, const float *act_betas_dev,
-                 const uint8_t *w_codes_dev, const uint8_t *w_beta_ids_dev,
-                 const float *w_norms_dev, const float *w_betas_dev, int m, int k, int n,
-                 int64_t weight_offset, int64_t weight_seed, int split_k, void *out_dev,
-                 int out_dtype, void *workspace_dev, size_t workspace_bytes, void *stream);
+                 const void *act_decoded_dev, const uint8_t *w_codes_dev,
+                 const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
+                 const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
+                 int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
+                 void *workspace_dev, size_t workspace_bytes, void *stream);
 
-size_t nq_w4a4_gemv_workspace_bytes(int m, int k, int n, int split_k);
+size_t nq_w4a4_gemv_workspace_bytes(int m, int k, int n, int split_k, int have_decoded_activation);
+
+/*
+ * Packed W4A4 linear for prefill, any M >= 1 (meant for M >= 9): same product and same
+ * arguments as nq_w4a4_gemv, computed on the matrix cores (v_mfma_f32_32x32x16_bf16).  The
+ * weight tile is decoded once per call into double-buffered LDS as MFMA B fragments; ragged
+ * M is padded to a multiple of 32 with zero rows inside the kernel and M above 512 is
+ * processed in chunks of 512 rows.  split_k in {0 (library picks), 1, 2, 4, 8, 16}.
+ * Requires q = 14, K % 128 == 0, (K / split_k) % 128 == 0.
+ * Replaces: run_m16 / run_large_m_staged of the torch extension
+ * (nestquant/runtime/nqrt4_w4a4_mma_binding.cpp:3-46, kernels
+ * nestquant/runtime/nqrt4_w4a4_mma.cu:124-171, 606-667) and the Python chunk-and-pad wrapper
+ * linear_packed_w4a4_mma_chunked_staged (nestquant/runtime/cuda_w4a4_mma.py:393-484).
+ */
+int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
+                 const float *act_norms_dev, const float *act_betas_dev,
+                 const void *act_decoded_dev, const uint8_t *w_codes_dev,
+                 const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
+                 const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
+                 int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
+                 void *workspace_dev, size_t workspace_bytes, void *stream);
+
+size_t nq_w4a4_gemm_workspace_bytes(int m, int k, int n, int split_k, int have_decoded_activation);
 
 #ifdef __cplusplus
 }

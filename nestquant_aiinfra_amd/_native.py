@@ -31,12 +31,15 @@ SIGNATURES = {
     "nq_last_error": (_c.c_char_p, []),
     "nq_e8_nearest": (_i32, [_ptr, _ptr, _i64, _ptr]),
     "nq_quantize_rows": (_i32, [_ptr, _i32, _i64, _i64, _i32, _ptr, _i32, _i32, _i64, _i64,
-                                _ptr, _ptr, _ptr, _ptr]),
+                                _ptr, _ptr, _ptr, _ptr, _ptr]),
     "nq_dequantize_rows": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i64, _i64,
                                   _ptr, _i32, _ptr]),
-    "nq_w4a4_gemv": (_i32, [_ptr] * 8 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
+    "nq_w4a4_gemv": (_i32, [_ptr] * 9 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
                                          _size, _ptr]),
-    "nq_w4a4_gemv_workspace_bytes": (_size, [_i32, _i32, _i32, _i32]),
+    "nq_w4a4_gemv_workspace_bytes": (_size, [_i32, _i32, _i32, _i32, _i32]),
+    "nq_w4a4_gemm": (_i32, [_ptr] * 9 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
+                                         _size, _ptr]),
+    "nq_w4a4_gemm_workspace_bytes": (_size, [_i32, _i32, _i32, _i32, _i32]),
 }
 
 _LIB: ctypes.CDLL | None = None

@@ -35,15 +35,40 @@ __global__ void __launch_bounds__(256) e8_nearest_kernel(const float4 *x, float4
 //            the winning lane stores the 32-bit code word, and the 2-bit ids of four
 //            neighbouring blocks are merged into one byte with two more exchanges.
 // ---------------------------------------------------------------------------------------
-template <typename T> __device__ __forceinline__ float load_as_f32(const T *p, int64_t i);
-template <> __device__ __forceinline__ float load_as_f32<float>(const float *p, int64_t i) { return p[i]; }
-template <> __device__ __forceinline__ float load_as_f32<uint16_t>(const uint16_t *p, int64_t i) {
-    return bf16_to_f32(p[i]);
-}
+// 16-byte global load of consecutive elements, promoted to float32 and stored to LDS
 struct half_bits { uint16_t v; };
-template <> __device__ __forceinline__ float load_as_f32<half_bits>(const half_bits *p, int64_t i) {
-    return f16_to_f32(p[i].v);
-}
+template <typename T> struct RowLoader;
+template <> struct RowLoader<float> {
+    static constexpr int kPerVector = 4;
+    static __device__ __forceinline__ void load(const float *x, int64_t v, float *dst) {
+        *reinterpret_cast<float4 *>(dst) = reinterpret_cast<const float4 *>(x)[v];
+    }
+    static __device__ __forceinline__ float scalar(const float *x, int64_t i) { return x[i]; }
+};
+template <> struct RowLoader<uint16_t> {
+    static constexpr int kPerVector = 8;
+    static __device__ __forceinline__ void load(const uint16_t *x, int64_t v, float *dst) {
+        const uint4 raw = reinterpret_cast<const uint4 *>(x)[v];
+        reinterpret_cast<float4 *>(dst)[0] = make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                                                         __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u));
+        reinterpret_cast<float4 *>(dst)[1] = make_float4(__uint_as_float(raw.z << 16), __uint_as_float(raw.z & 0xffff0000u),
+                                                         __uint_as_float(raw.w << 16), __uint_as_float(raw.w & 0xffff0000u));
+    }
+    static __device__ __forceinline__ float scalar(const uint16_t *x, int64_t i) { return bf16_to_f32(x[i]); }
+};
+template <> struct RowLoader<half_bits> {
+    static constexpr int kPerVector = 8;
+    static __device__ __forceinline__ void load(const half_bits *x, int64_t v, float *dst) {
+        const uint4 raw = reinterpret_cast<const uint4 *>(x)[v];
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            dst[2 * j] = f16_to_f32((uint16_t)(w[j] & 0xffffu));
+            dst[2 * j + 1] = f16_to_f32((uint16_t)(w[j] >> 16));
+        }
+    }
+    static __device__ __forceinline__ float scalar(const half_bits *x, int64_t i) { return f16_to_f32(x[i].v); }
+};
 
 // exchange with the lane whose id differs in bit 0 / bit 1 (inside a quad)
 __device__ __forceinline__ uint32_t quad_xor1(uint32_t v) {
@@ -58,18 +83,39 @@ __global__ void __launch_bounds__(1024)
 quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, float inv_q,
                      const float *__restrict__ betas, int beta_count, float sqrt_n,
                      uint32_t seed_plus_offset, uint32_t *__restrict__ codes,
-                     uint8_t *__restrict__ beta_ids, float *__restrict__ norms, int rows_per_wg) {
+                     uint8_t *__restrict__ beta_ids, float *__restrict__ norms,
+                     uint4 *__restrict__ decoded, int rows_per_wg, int slices, int vector_loads) {
     extern __shared__ float lds[];
     float *row_scale = lds + (size_t)rows_per_wg * n;
+    float *row_norm = row_scale + rows_per_wg;
     const int tid = threadIdx.x;
-    const int64_t row0 = (int64_t)blockIdx.x * rows_per_wg;
+    // With few rows a single row is spread over `slices` workgroups (rows_per_wg == 1): each
+    // stages the whole row and repeats the norm, then encodes its own range of blocks.
+    const int slice = blockIdx.x % slices;
+    const int64_t row0 = (int64_t)(blockIdx.x / slices) * rows_per_wg;
     const int blocks_per_row = n >> 3;
 
     // phase 1
     const int64_t first = row0 * n, limit = rows * (int64_t)n;
-    for (int idx = tid; idx < rows_per_wg * n; idx += blockDim.x) {
-        const int64_t g = first + idx;
-        lds[idx] = g < limit ? load_as_f32<T>(x, g) : 0.0f;
+    if (vector_loads) {
+        // n is a multiple of 32, so every row is a whole number of 16-byte vectors
+        constexpr int kPer = RowLoader<T>::kPerVector;
+        const int vectors = rows_per_wg * n / kPer;
+#pragma unroll 4
+        for (int v = tid; v < vectors; v += blockDim.x) {
+            const int64_t g = first + (int64_t)v * kPer;
+            if (g < limit) {
+                RowLoader<T>::load(x, g / kPer, lds + v * kPer);
+            } else {
+#pragma unroll
+                for (int j = 0; j < kPer; j++) lds[v * kPer + j] = 0.0f;
+            }
+        }
+    } else {
+        for (int idx = tid; idx < rows_per_wg * n; idx += blockDim.x) {
+            const int64_t g = first + idx;
+            lds[idx] = g < limit ? RowLoader<T>::scalar(x, g) : 0.0f;
+        }
     }
     __syncthreads();
 
@@ -78,10 +124,14 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
         const int r = tid >> 3, lane = tid & 7;
         const float *row = lds + (size_t)r * n + lane;
         float acc = 0.0f;
+        // n is a multiple of 32: four chain steps per trip, many trips in flight
 #pragma unroll 8
-        for (int i = 0; i < blocks_per_row; i++) {
-            const float v = row[8 * i];
-            acc = __builtin_fmaf(v, v, acc);
+        for (int i = 0; i < blocks_per_row; i += 4) {
+            const float v0 = row[8 * i], v1 = row[8 * i + 8], v2 = row[8 * i + 16], v3 = row[8 * i + 24];
+            acc = __builtin_fmaf(v0, v0, acc);
+            acc = __builtin_fmaf(v1, v1, acc);
+            acc = __builtin_fmaf(v2, v2, acc);
+            acc = __builtin_fmaf(v3, v3, acc);
         }
         float total = 0.0f;
 #pragma unroll
@@ -90,14 +140,16 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
         if (lane == 0) {
             // math.sqrt(n) / norm is evaluated as (1 / norm) * float32(sqrt(n))
             row_scale[r] = norm > 0.0f ? (1.0f / norm) * sqrt_n : 0.0f;
-            if (row0 + r < rows) norms[row0 + r] = norm;
+            row_norm[r] = norm;
+            if (row0 + r < rows && slice == 0) norms[row0 + r] = norm;
         }
     }
     __syncthreads();
 
     // phase 3
-    const int pairs = rows_per_wg * blocks_per_row * 4;
-    for (int p = tid; p < pairs; p += blockDim.x) {
+    const int slice_pairs = rows_per_wg * blocks_per_row * 4 / slices;     // a multiple of 16
+    const int pairs = slice_pairs * (slice + 1);
+    for (int p = slice_pairs * slice + tid; p < pairs; p += blockDim.x) {
         const int blk = p >> 2, bi = p & 3;
         const int r = blk / blocks_per_row, b = blk - r * blocks_per_row;
         const float scale = row_scale[r];
@@ -146,7 +198,18 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
             const bool take = fe < me || (fe == me && oi < best);
             best = take ? oi : best;
         }
-        if (best == (uint32_t)bi && row < rows) codes[gblock] = pack_codeword(code);
+        if (best == (uint32_t)bi && row < rows) {
+            codes[gblock] = pack_codeword(code);
+            if (decoded) {
+                // the BF16 decode of the stored code, as the linear kernels consume it
+                const float back = row_norm[r] / sqrt_n;
+                uint32_t h[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) h[j] = f32_to_bf16((recon[j] * beta) * back);
+                decoded[gblock] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16),
+                                             h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+            }
+        }
 
         // four consecutive blocks (16 lanes) share one beta byte
         uint32_t byte = best << (2 * (b & 3));
@@ -214,7 +277,7 @@ namespace {
 template <typename T, bool kDithered>
 int launch_quantize(const void *x, int64_t rows, int n, int q, const float *betas, int beta_count,
                     uint32_t seed_plus_offset, uint8_t *codes, uint8_t *beta_ids, float *norms,
-                    hipStream_t stream) {
+                    void *decoded, hipStream_t stream) {
     const int pairs_per_row = n / 2;
     const int target = pairs_per_row < 256 ? 256 : (pairs_per_row < 1024 ? pairs_per_row : 1024);
     int rows_per_wg = target / pairs_per_row;
@@ -222,8 +285,18 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
     if (rows_per_wg > rows) rows_per_wg = (int)rows;
     int threads = rows_per_wg * pairs_per_row;
     if (threads > 1024) threads = 1024;
+    // few long rows (decode activations): spread each row over several workgroups of 256
+    // lanes so that the whole chip encodes it; beta bytes need 16-pair alignment
+    int slices = 1;
+    if (rows_per_wg == 1 && pairs_per_row > 256) {
+        const int64_t wanted = 1024 / rows;                 // about four workgroups per CU in total
+        while (slices * 2 <= wanted && pairs_per_row / (slices * 2) >= 256 &&
+               pairs_per_row % (slices * 2 * 16) == 0)
+            slices *= 2;
+        if (slices > 1) threads = 256;
+    }
     if (threads < 64) threads = 64;
-    const size_t lds_bytes = ((size_t)rows_per_wg * n + rows_per_wg) * sizeof(float);
+    const size_t lds_bytes = ((size_t)rows_per_wg * n + 2 * rows_per_wg) * sizeof(float);
     auto kernel = nq::quantize_rows_kernel<T, kDithered>;
     if (lds_bytes > 48 * 1024) {
         hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -233,12 +306,14 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
             return nq::fail(NQ_ERR_LAUNCH, "nq_quantize_rows: cannot reserve %zu bytes of LDS: %s",
                             lds_bytes, hipGetErrorString(status));
     }
-    const int64_t grid = (rows + rows_per_wg - 1) / rows_per_wg;
+    const int64_t grid = ((rows + rows_per_wg - 1) / rows_per_wg) * slices;
     if (grid > 0x7fffffff) return nq::fail(NQ_ERR_SHAPE, "nq_quantize_rows: too many rows");
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(threads), lds_bytes, stream,
                        reinterpret_cast<const T *>(x), rows, n, (float)q, 1.0f / (float)q, betas,
                        beta_count, (float)sqrt((double)n), seed_plus_offset,
-                       reinterpret_cast<uint32_t *>(codes), beta_ids, norms, rows_per_wg);
+                       reinterpret_cast<uint32_t *>(codes), beta_ids, norms,
+                       reinterpret_cast<uint4 *>(decoded), rows_per_wg, slices,
+                       (int)nq::aligned(x, 16));
     return nq::check_launch("nq_quantize_rows");
 }
 
@@ -247,7 +322,7 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
 extern "C" int nq_quantize_rows(const void *x_dev, int x_dtype, int64_t rows, int64_t n, int q,
                                 const float *betas_dev, int beta_count, int has_dither, int64_t seed,
                                 int64_t block_offset, uint8_t *codes_dev, uint8_t *beta_ids_dev,
-                                float *norms_dev, void *stream) {
+                                float *norms_dev, void *decoded_bf16_dev, void *stream) {
     NQ_REQUIRE(rows >= 1 && n >= 1, NQ_ERR_SHAPE, "nq_quantize_rows: rows and n must be positive");
     NQ_REQUIRE(n % 32 == 0, NQ_ERR_SHAPE,
                "nq_quantize_rows: feature count %lld must be a multiple of 32", (long long)n);
@@ -259,6 +334,8 @@ extern "C" int nq_quantize_rows(const void *x_dev, int x_dtype, int64_t rows, in
     NQ_REQUIRE(x_dev && betas_dev && codes_dev && beta_ids_dev && norms_dev, NQ_ERR_ARGUMENT,
                "nq_quantize_rows: null pointer");
     NQ_REQUIRE(nq::aligned(codes_dev, 4), NQ_ERR_ARGUMENT, "nq_quantize_rows: codes must be 4-byte aligned");
+    NQ_REQUIRE(!decoded_bf16_dev || nq::aligned(decoded_bf16_dev, 16), NQ_ERR_ARGUMENT,
+               "nq_quantize_rows: decoded output must be 16-byte aligned");
     uint32_t seed_plus_offset = 0;
     if (has_dither) {
         NQ_REQUIRE(seed >= 0 && seed < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
@@ -270,9 +347,10 @@ extern "C" int nq_quantize_rows(const void *x_dev, int x_dtype, int64_t rows, in
     hipStream_t s = (hipStream_t)stream;
 #define NQ_DISPATCH_QUANTIZE(T)                                                                    \
     (has_dither ? launch_quantize<T, true>(x_dev, rows, (int)n, q, betas_dev, beta_count,           \
-                                           seed_plus_offset, codes_dev, beta_ids_dev, norms_dev, s) \
+                                           seed_plus_offset, codes_dev, beta_ids_dev, norms_dev,  \
+                                           decoded_bf16_dev, s)                                     \
                 : launch_quantize<T, false>(x_dev, rows, (int)n, q, betas_dev, beta_count, 0u,      \
-                                            codes_dev, beta_ids_dev, norms_dev, s))
+                                            codes_dev, beta_ids_dev, norms_dev, decoded_bf16_dev, s))
     switch (x_dtype) {
         case NQ_F32: return NQ_DISPATCH_QUANTIZE(float);
         case NQ_BF16: return NQ_DISPATCH_QUANTIZE(uint16_t);

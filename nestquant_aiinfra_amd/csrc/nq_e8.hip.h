@@ -19,49 +19,70 @@
 
 namespace nq {
 
-// lattice.py:18-34.  Nearest point of D8 (integer vectors with even coordinate sum).
-// `e` returns the residual p - a of the returned point on every coordinate.
-__device__ __forceinline__ void d8_nearest(const float (&p)[8], float (&a)[8], float (&e)[8]) {
-    float sum = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        a[j] = __builtin_rintf(p[j]);
-        e[j] = p[j] - a[j];          // exact
-        sum = sum + a[j];
-    }
-    // remainder(sum, 2) != 0 without an integer conversion (also right for huge sums)
-    const bool odd = __builtin_amdgcn_fractf(sum * 0.5f) != 0.0f;
-    const float m = fmaxf(fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3]))),
-                          fmaxf(fmaxf(fabsf(e[4]), fabsf(e[5])), fmaxf(fabsf(e[6]), fabsf(e[7]))));
-    bool done = !odd;                // an even sum needs no correction
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const bool hit = !done && (fabsf(e[j]) == m);   // first coordinate with the largest |residual|
-        done = done || hit;
-        const float dir = __builtin_copysignf(1.0f, e[j]);   // residual >= 0 -> +1 (a residual is never -0)
-        const float moved = a[j] + dir;
-        const float moved_e = e[j] - dir;               // == p - moved, both correctly rounded
-        a[j] = hit ? moved : a[j];
-        e[j] = hit ? moved_e : e[j];
-    }
+__device__ __forceinline__ float max_abs8(const float (&e)[8]) {
+    return fmaxf(fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3]))),
+                 fmaxf(fmaxf(fabsf(e[4]), fabsf(e[5])), fmaxf(fabsf(e[6]), fabsf(e[7]))));
 }
 
-// lattice.py:37-81, tie_break "upstream_half".  Returns the nearest E8 point of x.
+// remainder(sum, 2) != 0 for an integer-valued float, without an integer conversion
+// (also right for sums too large to convert)
+__device__ __forceinline__ bool is_odd(float sum) { return __builtin_amdgcn_fractf(sum * 0.5f) != 0.0f; }
+
+// lattice.py:37-81, tie_break "upstream_half".  Returns the nearest E8 point of x: the
+// better of the nearest points of the two cosets D8 and D8 + 1/2 (lattice.py:18-34 gives
+// the D8 search: round every coordinate, and if the coordinate sum is odd move the first
+// coordinate with the largest |residual| to its second-nearest integer).
+//
+// Integer coset: the squared distance only needs the residuals x - rint(x) (exact); the
+// moved coordinate contributes (|residual| - 1)^2 = (max - 1)^2, one value per block.
+// Half coset: the reference measures x - (D8(x - 1/2) + 1/2), recomputed from x because
+// x - 1/2 may round; the same is done here.
 __device__ __forceinline__ void e8_nearest(const float (&x)[8], float (&out)[8]) {
-    float a[8], ea[8], xm[8], b[8], eb[8];
-    d8_nearest(x, a, ea);
-#pragma unroll
-    for (int j = 0; j < 8; j++) xm[j] = x[j] - 0.5f;
-    d8_nearest(xm, b, eb);
-    float da = 0.0f, db = 0.0f;
+    float a[8], ea[8], sum_a = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-        b[j] = b[j] + 0.5f;
-        const float t = x[j] - b[j];     // the reference recomputes x - point for both cosets
-        da = da + ea[j] * ea[j];         // ea[j] == x[j] - a[j]
-        db = db + t * t;
+        a[j] = __builtin_rintf(x[j]);
+        ea[j] = x[j] - a[j];                       // exact
+        sum_a = sum_a + a[j];
     }
-    const bool pick_a = da < db;         // ties go to the half-integer coset
+    const float max_a = max_abs8(ea);
+    const float moved_a = max_a - 1.0f;
+    const float alt_a = moved_a * moved_a;
+    bool done_a = !is_odd(sum_a);                  // an even sum needs no correction
+    float dist_a = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const bool top = fabsf(ea[j]) == max_a;
+        const bool hit = top && !done_a;           // first coordinate with the largest |residual|
+        done_a = done_a || top;
+        const float sq = ea[j] * ea[j];
+        dist_a = dist_a + (hit ? alt_a : sq);
+        // residual >= 0 moves up (a residual is never -0)
+        a[j] = hit ? a[j] + __builtin_copysignf(1.0f, ea[j]) : a[j];
+    }
+
+    float b[8], eb[8], sum_b = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float xm = x[j] - 0.5f;
+        b[j] = __builtin_rintf(xm);
+        eb[j] = xm - b[j];
+        sum_b = sum_b + b[j];
+    }
+    const float max_b = max_abs8(eb);
+    bool done_b = !is_odd(sum_b);
+    float dist_b = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const bool top = fabsf(eb[j]) == max_b;
+        const bool hit = top && !done_b;
+        done_b = done_b || top;
+        const float half_point = b[j] + 0.5f;
+        b[j] = hit ? half_point + __builtin_copysignf(1.0f, eb[j]) : half_point;
+        const float t = x[j] - b[j];
+        dist_b = dist_b + t * t;
+    }
+    const bool pick_a = dist_a < dist_b;           // ties go to the half-integer coset
 #pragma unroll
     for (int j = 0; j < 8; j++) out[j] = pick_a ? a[j] : b[j];
 }
@@ -116,12 +137,22 @@ __device__ __forceinline__ void encode_block(const float (&x)[8], float q, float
     for (int j = 0; j < 8; j++) code[j] = mod_q(c[j], q, inv_q);
 }
 
+// Correctly rounded p / 14 in three operations: q0 = RN(p * RN(1/14)), the exact remainder
+// r = fma(-14, q0, p), and q1 = fma(r, RN(1/14), q0).  Checked against IEEE division for
+// every finite float32 with 1e-30 <= |p| <= 1e30 (only the sign of a zero result differs).
+__device__ __forceinline__ float div_by_14(float p) {
+    const float c = 1.0f / 14.0f;
+    const float q0 = p * c;
+    const float r = __builtin_fmaf(-14.0f, q0, p);
+    return __builtin_fmaf(r, c, q0);
+}
+
 // codec.py:105-142 `decode_nested` for one block given its coset point (already minus
 // the dither when there is one): the minimum-energy representative p - q * Q(p / q).
 __device__ __forceinline__ void reduce_coset_point(const float (&p)[8], float q, float (&out)[8]) {
     float z[8], k[8];
 #pragma unroll
-    for (int j = 0; j < 8; j++) z[j] = p[j] / q;         // IEEE division
+    for (int j = 0; j < 8; j++) z[j] = (q == 14.0f) ? div_by_14(p[j]) : p[j] / q;   // IEEE division
     e8_nearest(z, k);
 #pragma unroll
     for (int j = 0; j < 8; j++) out[j] = p[j] - q * k[j]; // exact

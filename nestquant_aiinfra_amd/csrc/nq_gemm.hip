@@ -1,0 +1,228 @@
+// Packed W4A4 linear for prefill (M >= 9 tokens; any M) on the matrix cores.
+//
+// y[m, n] = sum_k a[m, k] * w[n, k]: a is the BF16 decode of the NQA4 activation [M, K]
+// (emitted by the encoder, or decoded once per call), w is decoded on the fly from the
+// NQRT4 stream, products accumulate in FP32 with v_mfma_f32_32x32x16_bf16.
+//
+// Tiling.  grid = (N / 32, split_k); a workgroup of eight wavefronts owns 32 output
+// channels and one K slab and walks it in steps of 128:
+//   * decode: lane t decodes one E8 block of the 32 x 128 weight tile (channel t / 16,
+//     block t % 16) -- one 32-bit word per lane, 64 contiguous bytes per channel -- and
+//     writes its eight BF16 values as one 16-byte LDS entry laid out as the MFMA B fragment
+//     (lane l of K-step s holds channel l % 32, k = 16 s + 8 (l / 32) .. + 8).  An E8 block
+//     is exactly one lane's fragment, so decoded weights never need a transpose.
+//   * multiply: wavefront w owns token tiles w, w + 8, ... of 32 rows; per K-step it reads
+//     the B fragment from LDS (one ds_read_b128) and its A fragments straight from the
+//     activation in global memory (L2-resident; 16 bytes per lane).
+//   * the weight tile is double-buffered in LDS: one barrier per 128-wide step.
+// Every weight block is decoded exactly once per call, whatever M is: the kernel is bound
+// by the decode's vector-ALU work, and the matrix cores run in its shadow.
+// M is padded up to a multiple of 32 with zero rows inside the kernel (masked loads and
+// stores), so ragged M needs no copy; M above 512 is processed in chunks of 512 rows.
+// Replaces: run_m16 / run_large_m_staged and the chunk-and-pad wrapper,
+// nestquant/runtime/nqrt4_w4a4_mma.cu:124-171, 606-667 and nestquant/runtime/cuda_w4a4_mma.py:450-474.
+#include "nq_linear_common.hip.h"
+
+#include <math.h>
+
+namespace nq {
+
+constexpr int kGemmThreads = 512;
+constexpr int kGemmWaves = kGemmThreads / 64;
+constexpr int kGemmBN = 32;
+constexpr int kGemmBK = 128;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+template <int TILES>   // token tiles (of 32 rows) per wavefront
+__global__ void __launch_bounds__(kGemmThreads)
+w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
+                 const uint32_t *__restrict__ w_codes, const uint8_t *__restrict__ w_beta_ids,
+                 const float *__restrict__ w_norms, const float *__restrict__ w_betas,
+                 int m_rows, int k_size, int n_size, int k_slab, uint32_t seed_plus_offset,
+                 float sqrt_k, float *__restrict__ out_f32, uint16_t *__restrict__ out_bf16) {
+    __shared__ uint4 b_tile[2][kGemmBK / 16][64];          // 2 x 8 K-steps x 64 lanes x 16 B = 16 KiB
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n0 = blockIdx.x * kGemmBN;
+    const int k_begin = blockIdx.y * k_slab;
+    const int blocks_per_row = k_size >> 3;
+
+    // decode role: channel n0 + tid / 16, block tid % 16 of the current 128-wide step
+    const int dec_n = n0 + (tid >> 4), dec_kb = tid & 15;
+    const bool dec_live = dec_n < n_size;
+    const float wscale = dec_live ? w_norms[dec_n] / sqrt_k : 0.0f;
+    const float wbeta[4] = {w_betas[0], w_betas[1], w_betas[2], w_betas[3]};
+    const int64_t dec_first = (int64_t)(dec_live ? dec_n : 0) * blocks_per_row + (k_begin >> 3) + dec_kb;
+    uint4 *dec_slot0 = &b_tile[0][dec_kb >> 1][(tid >> 4) + 32 * (dec_kb & 1)];
+    uint4 *dec_slot1 = &b_tile[1][dec_kb >> 1][(tid >> 4) + 32 * (dec_kb & 1)];
+
+    // multiply role: A fragment rows of this lane, one per owned tile
+    const uint16_t *a_row[TILES];
+    bool a_live[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; t++) {
+        const int m = (wave + t * kGemmWaves) * 32 + (lane & 31);
+        a_live[t] = m < m_rows;
+        a_row[t] = act + (int64_t)(a_live[t] ? m : 0) * k_size + k_begin + 8 * (lane >> 5);
+    }
+    floatx16 acc[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[t][i] = 0.0f;
+
+    const int steps = k_slab / kGemmBK;
+    for (int s = 0; s < steps; s++) {
+        {
+            const int64_t g = dec_first + (int64_t)s * (kGemmBK / 8);
+            uint4 packed = make_uint4(0, 0, 0, 0);
+            if (dec_live) {
+                float v[8];
+                decode_codeword<true>(w_codes[g], 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
+                const float scale = wbeta[(w_beta_ids[g >> 2] >> (2 * (g & 3))) & 3] * wscale;
+                const bf16x2 h0 = pack_bf16x2(v[0] * scale, v[1] * scale), h1 = pack_bf16x2(v[2] * scale, v[3] * scale);
+                const bf16x2 h2 = pack_bf16x2(v[4] * scale, v[5] * scale), h3 = pack_bf16x2(v[6] * scale, v[7] * scale);
+                packed = make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
+                                    __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
+            }
+            *((s & 1) ? dec_slot1 : dec_slot0) = packed;
+        }
+        __syncthreads();
+        if (wave * 32 < m_rows) {
+#pragma unroll
+            for (int kk = 0; kk < kGemmBK / 16; kk++) {
+                const bf16x8 b = __builtin_bit_cast(bf16x8, b_tile[s & 1][kk][lane]);
+#pragma unroll
+                for (int t = 0; t < TILES; t++) {
+                    uint4 raw = make_uint4(0, 0, 0, 0);
+                    if (a_live[t]) raw = *reinterpret_cast<const uint4 *>(a_row[t] + s * kGemmBK + kk * 16);
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), b, acc[t], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // accumulator register r of lane l holds token row (r % 4) + 8 * (r / 4) + 4 * (l / 32)
+    // of the tile and channel n0 + l % 32
+    const int n = n0 + (lane & 31);
+    if (n < n_size) {
+#pragma unroll
+        for (int t = 0; t < TILES; t++) {
+            const int m_base = (wave + t * kGemmWaves) * 32 + 4 * (lane >> 5);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m_base + (r & 3) + 8 * (r >> 2);
+                if (m < m_rows) {
+                    if (out_f32)
+                        out_f32[((int64_t)blockIdx.y * m_rows + m) * n_size + n] = acc[t][r];
+                    else
+                        out_bf16[(int64_t)m * n_size + n] = f32_to_bf16(acc[t][r]);
+                }
+            }
+        }
+    }
+}
+
+}  // namespace nq
+
+namespace {
+
+constexpr int kChunkRows = 512;    // 8 wavefronts x 2 tiles x 32 rows
+
+// enough workgroups for 256 CUs; slabs stay multiples of 128
+int pick_gemm_split(int k, int n, int requested) {
+    if (requested > 0) return requested;
+    const int groups = (n + nq::kGemmBN - 1) / nq::kGemmBN;
+    int split = 1;
+    while (split < 16 && groups * split < 256 && (k / (split * 2)) % nq::kGemmBK == 0) split *= 2;
+    return split;
+}
+
+}  // namespace
+
+extern "C" size_t nq_w4a4_gemm_workspace_bytes(int m, int k, int n, int split_k, int have_decoded_activation) {
+    if (m < 1 || n < 1 || k < 1) return 0;
+    const int split = pick_gemm_split(k, n, split_k);
+    size_t bytes = 0;
+    if (!have_decoded_activation) bytes += nq::align256((size_t)m * k * 2);
+    const int chunk = m < kChunkRows ? m : kChunkRows;
+    if (split > 1) bytes += (size_t)split * (size_t)chunk * (size_t)n * sizeof(float);
+    return bytes;
+}
+
+extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
+                            const float *act_norms_dev, const float *act_betas_dev,
+                            const void *act_decoded_dev, const uint8_t *w_codes_dev,
+                            const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
+                            const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
+                            int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
+                            void *workspace_dev, size_t workspace_bytes, void *stream) {
+    NQ_REQUIRE(m >= 1, NQ_ERR_SHAPE, "nq_w4a4_gemm: M must be positive");
+    NQ_REQUIRE(k >= nq::kGemmBK && k % nq::kGemmBK == 0, NQ_ERR_SHAPE,
+               "nq_w4a4_gemm: K = %d must be a positive multiple of 128", k);
+    NQ_REQUIRE(n >= 1, NQ_ERR_SHAPE, "nq_w4a4_gemm: N must be positive");
+    NQ_REQUIRE(split_k == 0 || split_k == 1 || split_k == 2 || split_k == 4 || split_k == 8 || split_k == 16,
+               NQ_ERR_ARGUMENT, "nq_w4a4_gemm: split_k must be 0, 1, 2, 4, 8 or 16");
+    NQ_REQUIRE(out_dtype == NQ_F32 || out_dtype == NQ_BF16, NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemm: output dtype tag %d is not F32 or BF16", out_dtype);
+    NQ_REQUIRE(w_codes_dev && w_beta_ids_dev && w_norms_dev && w_betas_dev && out_dev, NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemm: null pointer");
+    NQ_REQUIRE(act_decoded_dev || (act_codes_dev && act_beta_ids_dev && act_norms_dev && act_betas_dev),
+               NQ_ERR_ARGUMENT, "nq_w4a4_gemm: neither packed nor decoded activation given");
+    NQ_REQUIRE(nq::aligned(w_codes_dev, 4) && (!act_codes_dev || nq::aligned(act_codes_dev, 4)) &&
+                   (!act_decoded_dev || nq::aligned(act_decoded_dev, 16)),
+               NQ_ERR_ARGUMENT, "nq_w4a4_gemm: code streams need 4-byte, decoded activation 16-byte alignment");
+    NQ_REQUIRE(weight_seed >= 0 && weight_seed < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemm: seed must be in [0, 2**31)");
+    NQ_REQUIRE(weight_offset >= 0 && weight_offset + (int64_t)n * (k / 8) <= ((int64_t)1 << 28),
+               NQ_ERR_SHAPE, "nq_w4a4_gemm: block range exceeds the stateless dither counter space");
+    const int split = pick_gemm_split(k, n, split_k);
+    NQ_REQUIRE(k % split == 0 && (k / split) % nq::kGemmBK == 0, NQ_ERR_SHAPE,
+               "nq_w4a4_gemm: K / split_k = %d / %d must be a multiple of 128", k, split);
+    const int chunk_rows = m < kChunkRows ? m : kChunkRows;
+    const size_t decoded_bytes = act_decoded_dev ? 0 : nq::align256((size_t)m * k * 2);
+    const size_t need = decoded_bytes + (split > 1 ? (size_t)split * chunk_rows * n * sizeof(float) : 0);
+    NQ_REQUIRE(need == 0 || (workspace_dev && workspace_bytes >= need), NQ_ERR_WORKSPACE,
+               "nq_w4a4_gemm: needs a %zu-byte workspace, got %zu", need, workspace_bytes);
+    NQ_REQUIRE(need == 0 || nq::aligned(workspace_dev, 16), NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemm: workspace must be 16-byte aligned");
+
+    hipStream_t s = (hipStream_t)stream;
+    const uint16_t *act = reinterpret_cast<const uint16_t *>(act_decoded_dev);
+    if (!act) {
+        int status = nq::launch_decode_activation(act_codes_dev, act_beta_ids_dev, act_norms_dev, act_betas_dev,
+                                                  m, k, workspace_dev, s);
+        if (status != NQ_OK) return status;
+        act = reinterpret_cast<const uint16_t *>(workspace_dev);
+    }
+    float *partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace_dev) + decoded_bytes);
+    const uint32_t seed_plus_offset = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
+    const float sqrt_k = (float)sqrt((double)k);
+    const dim3 grid((unsigned)((n + nq::kGemmBN - 1) / nq::kGemmBN), (unsigned)split);
+    const uint32_t *wc = reinterpret_cast<const uint32_t *>(w_codes_dev);
+    const size_t out_row_bytes = (size_t)n * (out_dtype == NQ_F32 ? 4 : 2);
+
+    for (int m0 = 0; m0 < m; m0 += kChunkRows) {
+        const int rows = m - m0 < kChunkRows ? m - m0 : kChunkRows;
+        char *out_chunk = reinterpret_cast<char *>(out_dev) + (size_t)m0 * out_row_bytes;
+        float *target_f32 = split > 1 ? partials : (out_dtype == NQ_F32 ? (float *)out_chunk : nullptr);
+        uint16_t *target_bf16 = (split > 1 || out_dtype == NQ_F32) ? nullptr : (uint16_t *)out_chunk;
+        const uint16_t *act_chunk = act + (size_t)m0 * k;
+        if (rows <= 8 * 32)
+            hipLaunchKernelGGL(nq::w4a4_gemm_kernel<1>, grid, dim3(nq::kGemmThreads), 0, s, act_chunk, wc,
+                               w_beta_ids_dev, w_norms_dev, w_betas_dev, rows, k, n, k / split,
+                               seed_plus_offset, sqrt_k, target_f32, target_bf16);
+        else
+            hipLaunchKernelGGL(nq::w4a4_gemm_kernel<2>, grid, dim3(nq::kGemmThreads), 0, s, act_chunk, wc,
+                               w_beta_ids_dev, w_norms_dev, w_betas_dev, rows, k, n, k / split,
+                               seed_plus_offset, sqrt_k, target_f32, target_bf16);
+        int status = nq::check_launch("nq_w4a4_gemm");
+        if (status != NQ_OK) return status;
+        if (split > 1) {
+            status = nq::launch_splitk_reduce(partials, split, (int64_t)rows * n, out_chunk, out_dtype, s);
+            if (status != NQ_OK) return status;
+        }
+    }
+    return NQ_OK;
+}

@@ -1,0 +1,68 @@
+// Pieces shared by the packed W4A4 linear kernels (decode GEMV and prefill GEMM).
+#pragma once
+
+#include "nq_e8.hip.h"
+#include "nq_host.h"
+
+namespace nq {
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ bf16x2 pack_bf16x2(float lo, float hi) {
+    const floatx2 v = {lo, hi};
+    return __builtin_convertvector(v, bf16x2);          // v_cvt_pk_bf16_f32, round to nearest even
+}
+
+// NQA4 streams -> BF16 [M, K], exactly bf16((decode * beta) * (norm / sqrt(K)))
+static __global__ void __launch_bounds__(256)
+decode_activation_kernel(const uint32_t *__restrict__ codes, const uint8_t *__restrict__ beta_ids,
+                         const float *__restrict__ norms, const float *__restrict__ betas,
+                         int64_t blocks, int blocks_per_row, float sqrt_k, uint4 *__restrict__ out) {
+    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= blocks) return;
+    float v[8];
+    decode_codeword<false>(codes[g], 14.0f, 0u, v);
+    const float beta = betas[(beta_ids[g >> 2] >> (2 * (g & 3))) & 3];
+    const float scale = norms[g / blocks_per_row] / sqrt_k;
+    uint32_t h[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) h[j] = f32_to_bf16((v[j] * beta) * scale);
+    out[g] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+}
+
+
+// Decodes the NQA4 streams of [m, k] into BF16 at `out` (16-byte aligned, m * k * 2 bytes).
+inline int launch_decode_activation(const uint8_t *codes, const uint8_t *beta_ids, const float *norms,
+                                    const float *betas, int m, int k, void *out, hipStream_t stream) {
+    const int64_t blocks = (int64_t)m * (k / 8);
+    hipLaunchKernelGGL(decode_activation_kernel, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint32_t *>(codes), beta_ids, norms, betas, blocks, k / 8,
+                       (float)sqrt((double)k), reinterpret_cast<uint4 *>(out));
+    return check_launch("activation decode");
+}
+
+// partial [split][M][N] float32 -> out [M][N]; slices added in ascending order
+// (same rule as nestquant/runtime/nqrt4_w4a4_mma.cu:411-420).
+static __global__ void __launch_bounds__(256)
+splitk_reduce_kernel(const float *__restrict__ partial, int split, int64_t count,
+                     float *__restrict__ out_f32, uint16_t *__restrict__ out_bf16) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float total = 0.0f;
+    for (int s = 0; s < split; s++) total = total + partial[(int64_t)s * count + i];
+    if (out_f32) out_f32[i] = total;
+    else out_bf16[i] = f32_to_bf16(total);
+}
+
+inline int launch_splitk_reduce(const float *partials, int split, int64_t count, void *out, int out_dtype,
+                                hipStream_t stream) {
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, partials,
+                       split, count, out_dtype == NQ_F32 ? (float *)out : nullptr,
+                       out_dtype == NQ_F32 ? nullptr : (uint16_t *)out);
+    return check_launch("split-K reduce");
+}
+
+inline size_t align256(size_t bytes) { return (bytes + 255) & ~(size_t)255; }
+
+}  // namespace nq

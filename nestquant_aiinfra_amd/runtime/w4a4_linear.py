@@ -39,6 +39,10 @@ class PreparedNQA4Activation:
     code_width: int
     beta_width: int
     output_dtype: torch.dtype
+    # BF16 [tokens, features] decode of the payloads, emitted by the encoder as a side
+    # product so that the linear kernels need not decode the activation again; None for
+    # activations assembled from payloads alone (the kernels then decode them once per call).
+    decoded: torch.Tensor | None = None
 
     @property
     def token_count(self) -> int:
@@ -80,10 +84,12 @@ def _beta_values(betas: Sequence[float]) -> tuple[float, ...]:
 
 
 def quantize_rows_packed(rows: torch.Tensor, *, q: int, beta_table: torch.Tensor,
-                         dither_seed: int | None = None, block_offset: int = 0
+                         dither_seed: int | None = None, block_offset: int = 0,
+                         decoded: torch.Tensor | None = None
                          ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Encode ``rows`` [R, n] (float32 / bfloat16 / float16, on the GPU) into packed 4-bit
-    codes, packed 2-bit beta ids and float32 row norms with one kernel launch."""
+    codes, packed 2-bit beta ids and float32 row norms with one kernel launch.  ``decoded``
+    (optional BF16 [R, n]) receives the decode of the stored codes."""
     device = _native.require_cuda(rows, beta_table)
     if rows.ndim != 2:
         raise ValueError("rows must have shape [rows, features]")
@@ -94,7 +100,8 @@ def quantize_rows_packed(rows: torch.Tensor, *, q: int, beta_table: torch.Tensor
     _native.check(_native.library().nq_quantize_rows(
         rows.data_ptr(), _native.dtype_tag(rows.dtype), count, n, q, beta_table.data_ptr(),
         beta_table.numel(), int(dither_seed is not None), int(dither_seed or 0), block_offset,
-        codes.data_ptr(), beta_ids.data_ptr(), norms.data_ptr(), _native.stream_handle(device)))
+        codes.data_ptr(), beta_ids.data_ptr(), norms.data_ptr(),
+        None if decoded is None else decoded.data_ptr(), _native.stream_handle(device)))
     return codes, beta_ids, norms
 
 
@@ -124,11 +131,12 @@ def quantize_activation_cuda(inputs: torch.Tensor, *, q: int, betas: Sequence[fl
     rows = rows.contiguous()
     if beta_table is None:
         beta_table = torch.tensor(beta_values, device=inputs.device, dtype=torch.float32)
-    codes, beta_ids, norms = quantize_rows_packed(rows, q=q, beta_table=beta_table)
+    decoded = torch.empty(rows.shape, dtype=torch.bfloat16, device=rows.device) if q == 14 else None
+    codes, beta_ids, norms = quantize_rows_packed(rows, q=q, beta_table=beta_table, decoded=decoded)
     return PreparedNQA4Activation(
         code_payload=codes, beta_payload=beta_ids, row_norms=norms, beta_table=beta_table,
         original_shape=tuple(inputs.shape), q=q, code_width=code_width, beta_width=beta_width,
-        output_dtype=inputs.dtype,
+        output_dtype=inputs.dtype, decoded=decoded,
     )
 
 
@@ -255,22 +263,46 @@ def can_use_w4a4_mma_small_m(activation: PreparedNQA4Activation, weight: Prepare
     return activation.token_count in (2, 4, 8) and _common_ok(activation, weight, 32, 1)
 
 
+def can_use_w4a4_mma_m16(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear) -> bool:
+    return activation.token_count == 16 and _common_ok(activation, weight, 128, 1)
+
+
+def can_use_w4a4_mma_large_m_staged(activation: PreparedNQA4Activation,
+                                    weight: PreparedNQRTLinear) -> bool:
+    return activation.token_count in (32, 64, 128) and _common_ok(activation, weight, 128, 1)
+
+
+def can_use_w4a4_mma_m128_staged(activation: PreparedNQA4Activation,
+                                 weight: PreparedNQRTLinear) -> bool:
+    return activation.token_count == 128 and can_use_w4a4_mma_large_m_staged(activation, weight)
+
+
+def can_use_w4a4_mma_chunked_staged(activation: PreparedNQA4Activation,
+                                    weight: PreparedNQRTLinear) -> bool:
+    """Arbitrary M >= 1: the MFMA kernel pads ragged M inside the kernel."""
+    return activation.token_count >= 1 and _common_ok(activation, weight, 128, 1)
+
+
 # --------------------------------------------------------------------------------------
 # linear kernels, M = 1..8
 # --------------------------------------------------------------------------------------
 
 def _gemv(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *, split_k: int,
-          output_dtype: torch.dtype) -> torch.Tensor:
+          output_dtype: torch.dtype, kernel: str = "gemv") -> torch.Tensor:
     lib = _native.library()
+    launch = lib.nq_w4a4_gemv if kernel == "gemv" else lib.nq_w4a4_gemm
+    workspace_bytes = (lib.nq_w4a4_gemv_workspace_bytes if kernel == "gemv"
+                       else lib.nq_w4a4_gemm_workspace_bytes)
     device = activation.code_payload.device
     m, k, n = activation.token_count, activation.feature_count, weight.record.indices.shape[0]
     out = torch.empty((m, n), dtype=output_dtype, device=device)
-    need = lib.nq_w4a4_gemv_workspace_bytes(m, k, n, split_k)
+    decoded = activation.decoded
+    need = workspace_bytes(m, k, n, split_k, int(decoded is not None))
     workspace = torch.empty(need, dtype=torch.uint8, device=device) if need else None
-    _native.check(lib.nq_w4a4_gemv(
+    _native.check(launch(
         activation.code_payload.data_ptr(), activation.beta_payload.data_ptr(),
         activation.row_norms.data_ptr(), activation.beta_table.data_ptr(),
-        weight.code_payload.data_ptr(), weight.beta_payload.data_ptr(),
+        None if decoded is None else decoded.data_ptr(), weight.code_payload.data_ptr(), weight.beta_payload.data_ptr(),
         weight.row_norms.data_ptr(), weight.beta_table.data_ptr(), m, k, n, 0,
         int(weight.record.dither_seed), split_k, out.data_ptr(), _native.dtype_tag(output_dtype),
         None if workspace is None else workspace.data_ptr(), need, _native.stream_handle(device)))
@@ -340,3 +372,81 @@ def linear_packed_w4a4_mma_small_m_splitk_probe(activation: PreparedNQA4Activati
         raise ValueError("split_k must be 2, 4, or 8")
     return _gemv(activation, weight, split_k=split_k,
                  output_dtype=_kernel_dtype(activation)).to(activation.output_dtype)
+
+
+# --------------------------------------------------------------------------------------
+# linear kernels, prefill (matrix cores)
+# --------------------------------------------------------------------------------------
+
+def _gemm(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *,
+          output_dtype: torch.dtype | None = None, split_k: int = 0) -> torch.Tensor:
+    dtype = _kernel_dtype(activation) if output_dtype is None else output_dtype
+    return _gemv(activation, weight, split_k=split_k, output_dtype=dtype, kernel="gemm")
+
+
+def linear_packed_w4a4_mma_m16(activation: PreparedNQA4Activation,
+                               weight: PreparedNQRTLinear) -> torch.Tensor:
+    if not can_use_w4a4_mma_m16(activation, weight):
+        raise ValueError("activation or packed weight is unsupported by W4A4 M16")
+    return _gemm(activation, weight).to(activation.output_dtype)
+
+
+def linear_packed_w4a4_mma_large_m_staged(activation: PreparedNQA4Activation,
+                                          weight: PreparedNQRTLinear) -> torch.Tensor:
+    """M in {32, 64, 128}: decoded weight fragments staged once per workgroup in LDS."""
+    if not can_use_w4a4_mma_large_m_staged(activation, weight):
+        raise ValueError("activation or packed weight is unsupported by staged large-M")
+    return _gemm(activation, weight).to(activation.output_dtype)
+
+
+def linear_packed_w4a4_mma_m128_staged(activation: PreparedNQA4Activation,
+                                       weight: PreparedNQRTLinear) -> torch.Tensor:
+    if not can_use_w4a4_mma_m128_staged(activation, weight):
+        raise ValueError("activation or packed weight is unsupported by staged M128")
+    return _gemm(activation, weight).to(activation.output_dtype)
+
+
+def linear_packed_w4a4_mma_chunked_staged(activation: PreparedNQA4Activation,
+                                          weight: PreparedNQRTLinear) -> torch.Tensor:
+    """Arbitrary M.  The reference covers M with 128-row chunks plus a tail padded to the
+    next supported size (cuda_w4a4_mma.py:450-474); here one launch handles up to 512 rows
+    and pads the ragged tail to a multiple of 32 with zero rows inside the kernel, so every
+    weight block is decoded once per 512 rows instead of once per 128."""
+    if not can_use_w4a4_mma_chunked_staged(activation, weight):
+        raise ValueError("activation or packed weight is unsupported by chunked staged")
+    return _gemm(activation, weight).to(activation.output_dtype)
+
+
+linear_packed_w4a4_mma_chunked_staged_probe = linear_packed_w4a4_mma_chunked_staged
+
+
+def slice_pad_packed_activation_rows(activation: PreparedNQA4Activation, start: int, row_count: int,
+                                     padded_row_count: int) -> PreparedNQA4Activation:
+    """Slice row-aligned packed A4 payloads and append zero-norm padding rows
+    (nestquant/runtime/cuda_w4a4_mma.py:393-447).  Padding rows carry zero codes and a zero
+    norm, so they decode to exact zeros."""
+    if not 0 <= start < activation.token_count:
+        raise ValueError("packed activation slice start is out of range")
+    if row_count < 1 or start + row_count > activation.token_count:
+        raise ValueError("packed activation slice row count is out of range")
+    if padded_row_count < row_count:
+        raise ValueError("padded row count must cover the activation slice")
+    k = activation.feature_count
+    pad = padded_row_count - row_count
+
+    def cut(payload: torch.Tensor, per_row: int) -> torch.Tensor:
+        piece = payload[start * per_row:(start + row_count) * per_row]
+        if not pad:
+            return piece.contiguous()
+        return torch.cat((piece, torch.zeros(pad * per_row, dtype=payload.dtype, device=payload.device)))
+
+    decoded = None
+    if activation.decoded is not None:
+        decoded = cut(activation.decoded.reshape(-1), k).reshape(padded_row_count, k)
+    return PreparedNQA4Activation(
+        code_payload=cut(activation.code_payload, k * activation.code_width // 8),
+        beta_payload=cut(activation.beta_payload, (k // 8) * activation.beta_width // 8),
+        row_norms=cut(activation.row_norms, 1), beta_table=activation.beta_table,
+        original_shape=(padded_row_count, k), q=activation.q, code_width=activation.code_width,
+        beta_width=activation.beta_width, output_dtype=activation.output_dtype, decoded=decoded,
+    )

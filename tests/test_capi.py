@@ -1,0 +1,53 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/nqhip.h declares."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def _declared():
+    text = (ROOT / "include" / "nqhip.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_bindings_and_exports_agree():
+    from nestquant_aiinfra_amd import _native
+    declared = _declared()
+    assert declared, "no declarations found"
+    assert sorted(_native.SIGNATURES) == declared
+    if not _native.LIBRARY_PATH.exists():
+        from nestquant_aiinfra_amd import build
+        build.build()
+    lib = ctypes.CDLL(str(_native.LIBRARY_PATH))
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert _native.library().nq_abi_version() >= 1
+    assert _native.library().nq_last_error() is not None
+
+
+def test_host_side_validation_needs_no_gpu():
+    """Shape checks run before anything is launched and name the offending argument."""
+    from nestquant_aiinfra_amd import _native
+    lib = _native.library()
+    status = lib.nq_quantize_rows(None, 0, 1, 40, 14, None, 4, 0, 0, 0, None, None, None, None, None)
+    assert status == _native.NQ_ERR_SHAPE and b"multiple of 32" in lib.nq_last_error()
+    with pytest.raises(ValueError, match="multiple of 32"):
+        _native.check(status)
+    status = lib.nq_w4a4_gemv(*([None] * 9), 9, 2048, 2048, 0, 1, 0, None, 0, None, 0, None)
+    assert status == _native.NQ_ERR_SHAPE and b"outside [1, 8]" in lib.nq_last_error()
+    status = lib.nq_dequantize_rows(None, None, None, None, 1, 64, 14, 1, -5, 0, None, 0, None)
+    assert status == _native.NQ_ERR_ARGUMENT
+    assert lib.nq_w4a4_gemv_workspace_bytes(1, 8192, 2048, 8, 1) == 8 * 2048 * 4
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from nestquant_aiinfra_amd import _native
+    monkeypatch.setattr(_native, "_LIB", None)
+    monkeypatch.setattr(_native, "LIBRARY_PATH", tmp_path / "libnqhip.so")
+    with pytest.raises(_native.NativeLibraryMissing, match="no fallback"):
+        _native.library()

@@ -1,0 +1,103 @@
+"""GPU parity of the packed W4A4 prefill linear (MFMA), through the C ABI.
+
+Bar: max |y - y_ref| / max |y_ref| <= 1e-2 against the oracle's decode-then-FP32 matmul;
+<= 2e-3 against the same product on BF16-rounded operands (what the matrix cores multiply).
+"""
+
+import dataclasses
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ACTIVATION_BETAS, Q, WEIGHT_BETAS
+from gpu_util import bits, oracle_weight, outlier_rows, relative_error
+from test_gpu_gemv import BF16_TOLERANCE, TOLERANCE, _record, _references
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from nestquant_aiinfra_amd.runtime import w4a4_linear
+    return w4a4_linear
+
+
+def _activation(rt, oracle, m, k, seed):
+    x = torch.from_numpy(oracle.hadamard(outlier_rows(m, k, seed=seed).numpy())).to(torch.bfloat16).cuda()
+    return rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS)
+
+
+@pytest.mark.parametrize("m", [1, 9, 16, 33, 40, 64, 128, 300])
+@pytest.mark.parametrize("k,n_out", [(128, 32), (512, 72), (2048, 96)])
+def test_small_shapes_match_oracle(rt, oracle, m, k, n_out):
+    seed = 20261201 + m
+    _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=4000 + k + n_out, dither_seed=seed)
+    weight = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
+    activation = _activation(rt, oracle, m, k, seed=3001 + m)
+    ref32, ref16 = _references(oracle, activation, rt, wc, wb, wn, seed)
+    y = rt._gemm(activation, weight, output_dtype=torch.float32)
+    assert relative_error(bits(y), ref32) <= TOLERANCE
+    assert relative_error(bits(y), ref16) <= BF16_TOLERANCE
+    for split in (1, 2, 4):
+        if (k // split) % 128:
+            continue
+        ys = rt._gemm(activation, weight, output_dtype=torch.float32, split_k=split)
+        assert relative_error(bits(ys), ref16) <= BF16_TOLERANCE
+        assert torch.equal(ys, rt._gemm(activation, weight, output_dtype=torch.float32, split_k=split))
+    # the packed-only path (kernel decodes the activation itself) gives identical bits
+    packed_only = dataclasses.replace(activation, decoded=None)
+    assert torch.equal(rt._gemm(packed_only, weight, output_dtype=torch.float32), y)
+    y16 = rt.linear_packed_w4a4_mma_chunked_staged(activation, weight)
+    assert y16.dtype == torch.bfloat16 and relative_error(bits(y16.float()), ref32) <= TOLERANCE
+
+
+def test_gemm_agrees_with_gemv_rows(rt, oracle):
+    """Each prefill row equals the decode kernel's result for that row (same operands)."""
+    k, n_out, seed = 2048, 64, 20261301
+    _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=5, dither_seed=seed)
+    weight = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
+    activation = _activation(rt, oracle, 8, k, seed=6)
+    a = rt._gemm(activation, weight, output_dtype=torch.float32)
+    b = rt._gemv(activation, weight, split_k=1, output_dtype=torch.float32)
+    assert relative_error(bits(a), bits(b)) <= 1e-5
+
+
+@pytest.mark.parametrize("name,k,n_out,wseed,dseed", [("gate_proj", 2048, 8192, 1003, 20261103),
+                                                      ("down_proj", 8192, 2048, 1004, 20261104)])
+def test_llama_1b_prefill_shapes(rt, oracle, name, k, n_out, wseed, dseed):
+    """Full-size prefill shapes at ragged M; weights encoded on the GPU; the oracle checks a
+    random subset of 256 output channels (its decode of all channels takes too long here)."""
+    g = torch.Generator().manual_seed(wseed)
+    w = torch.from_numpy(oracle.hadamard((0.02 * torch.randn(n_out, k, generator=g)).numpy()))
+    record = rt.quantize_weight_nqrt4(w.cuda(), q=Q, betas=WEIGHT_BETAS, dither_seed=dseed, tensor_name=name)
+    weight = rt.prepare_fused_linear(record, device="cuda")
+    rows = np.sort(np.random.default_rng(1).choice(n_out, size=256, replace=False))
+    codes = oracle.unpack_unsigned(np.frombuffer(record.indices.code_payload, np.uint8), n_out * k, 4).reshape(n_out, k)
+    beta = oracle.unpack_unsigned(np.frombuffer(record.indices.beta_payload, np.uint8), n_out * k // 8, 2).reshape(n_out, k // 8)
+    norms = record.row_norms.numpy()
+    dither = oracle.dither_stateless(n_out * k // 8, dseed).reshape(n_out, k // 8, 8)[rows]
+    w_hat = oracle.dequantize_rows(codes[rows], beta[rows], norms[rows], WEIGHT_BETAS, Q, dither=dither)
+    for m in (16, 40, 64, 128, 384):
+        activation = _activation(rt, oracle, m, k, seed=3001)
+        a_codes = oracle.unpack_unsigned(bits(activation.code_payload), m * k, 4)
+        a_beta = oracle.unpack_unsigned(bits(activation.beta_payload), m * k // 8, 2)
+        a_hat = oracle.dequantize_rows(a_codes, a_beta, bits(activation.row_norms), ACTIVATION_BETAS, Q)
+        ref32 = oracle.matmul_nt(a_hat, w_hat)
+        y = rt.linear_packed_w4a4_mma_chunked_staged(activation, weight)
+        assert y.dtype == torch.bfloat16 and tuple(y.shape) == (m, n_out)
+        assert relative_error(bits(y.float())[:, rows], ref32) <= TOLERANCE, (name, m)
+
+
+def test_slice_and_pad_matches_reference_chunking(rt, oracle):
+    """Zero-norm padding rows decode to zeros; chunked results equal the one-launch result."""
+    k, n_out, seed = 512, 48, 20261302
+    _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=8, dither_seed=seed)
+    weight = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
+    activation = _activation(rt, oracle, 40, k, seed=9)
+    whole = rt._gemm(activation, weight, output_dtype=torch.float32)
+    chunk = rt.slice_pad_packed_activation_rows(activation, 32, 8, 16)
+    part = rt._gemm(chunk, weight, output_dtype=torch.float32)
+    assert torch.equal(part[:8], whole[32:40]) and not part[8:].any()
+    packed_only = dataclasses.replace(chunk, decoded=None)
+    assert torch.equal(rt._gemm(packed_only, weight, output_dtype=torch.float32), part)

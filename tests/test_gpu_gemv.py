@@ -106,7 +106,11 @@ def test_linearity_in_the_row_norm(rt, oracle):
     a = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS)
     y1 = rt._gemv(a, weight, split_k=1, output_dtype=torch.float32)
     import dataclasses
-    a2 = dataclasses.replace(a, row_norms=a.row_norms * 2.0)        # power of two: exact in BF16 and FP32
+    # without the encoder's BF16 side product the kernels decode the packed streams themselves
+    packed_only = dataclasses.replace(a, decoded=None)
+    assert torch.equal(rt._gemv(packed_only, weight, split_k=1, output_dtype=torch.float32), y1)
+    assert torch.equal(rt.decode_packed_a4(a, torch.bfloat16), a.decoded)
+    a2 = dataclasses.replace(packed_only, row_norms=a.row_norms * 2.0)   # power of two: exact in BF16 and FP32
     y2 = rt._gemv(a2, weight, split_k=1, output_dtype=torch.float32)
     assert torch.equal(y2, 2.0 * y1)
 
