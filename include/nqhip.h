@@ -143,6 +143,76 @@ int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
 
 size_t nq_w4a4_gemm_workspace_bytes(int m, int k, int n, int split_k, int have_decoded_activation);
 
+/*
+ * NQKV cache, device-resident state.  Per slot (int32[slots]): sequence_lengths,
+ * page_counts, last_page_lens, hot_lengths; page_indices int32[slots, max_pages] maps a
+ * slot's page ordinal to a physical page; hot tails BF16 [slots, page_size, kv_heads,
+ * head_dim]; the page pool is six SoA streams indexed by physical page (per page and side:
+ * codes page_size*kv_heads*head_dim/2 B, beta ids .../32 B, norms f32[page_size*kv_heads]),
+ * rows in NHD order, row = token * kv_heads + head.  Same tensors as the reference's
+ * NQKVPagePool / BatchedNQKVMetadata / NQKVHotColdCache (nestquant/runtime/nqkv_pool.py:94-110,
+ * paged_nqkv_cache.py:25-95, nqkv_hot_cache.py:14-37).
+ *
+ * nq_nqkv_advance: for every active batch row r with slot s = slot_ids[r] (rows with a
+ * slot outside [0, slots) are ignored), add counts[r] (or uniform_count when counts is NULL)
+ * to sequence_lengths[s], clamped at max_tokens, and refresh the three derived tensors.
+ * Called once per step, before the layers run.  Replaces the per-layer metadata kernels
+ * and host-side page reservation of nestquant/runtime/nqkv_graph_writer.py:15-80, 291-332,
+ * nestquant/runtime/nqkv_graph_pack.py:18-69 and nqkv_batch_manager.py:648-707.
+ */
+int nq_nqkv_advance(const int32_t *slot_ids_dev, const uint8_t *active_mask_dev,
+                    const int32_t *counts_dev, int uniform_count, int batch, int slots,
+                    int page_size, int max_tokens, int32_t *sequence_lengths_dev,
+                    int32_t *page_counts_dev, int32_t *last_page_lens_dev,
+                    int32_t *hot_lengths_dev, void *stream);
+
+/*
+ * Paged ragged writer for one layer.  key/value: BF16 [batch, tokens, kv_heads, head_dim];
+ * row r contributes its first counts[r] tokens (uniform_count when counts is NULL) at
+ * positions sequence_lengths[s] - count .. sequence_lengths[s] - 1 (lengths already advanced).
+ * Rows land in the slot's hot tail; every page completed by the write is encoded (the row
+ * quantiser of nq_quantize_rows, bit-identical) into physical page page_indices[s, ordinal].
+ * Requires head_dim = 64, page_size = 16, q = 14, equal beta counts.
+ * Replaces: append_hot_k1_graph_safe / ragged sub-page and segment writers
+ * (nestquant/runtime/nqkv_graph_writer.py:263-473), launch_pack_full_hot_pages_graph_safe
+ * (nestquant/runtime/nqkv_graph_pack.py:76-193) and the multi-round planner that feeds them
+ * (nestquant/runtime/nqkv_segment_plan.py:61-144).
+ */
+int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_dtype, const int32_t *slot_ids_dev,
+                  const uint8_t *active_mask_dev, const int32_t *counts_dev, int uniform_count,
+                  const int32_t *sequence_lengths_dev, const int32_t *page_indices_dev,
+                  uint8_t *key_codes_dev, uint8_t *key_beta_ids_dev, float *key_norms_dev,
+                  uint8_t *value_codes_dev, uint8_t *value_beta_ids_dev, float *value_norms_dev,
+                  const float *key_betas_dev, int key_beta_count, const float *value_betas_dev,
+                  int value_beta_count, void *hot_keys_dev, void *hot_values_dev, int batch, int tokens,
+                  int slots, int max_pages, int kv_heads, int head_dim, int page_size, void *stream);
+
+/*
+ * Paged NQKV4 decode attention for a ragged batch: for batch row r with slot s (clamped to
+ * range; the row is live iff active_mask[r] and, when given, cache_active[s]) and query
+ * head h (KV head h / (q_heads / kv_heads)), softmax(q . K^T * scale) . V over the slot's
+ * page_counts[s] cold pages (all full except the last, which holds last_page_lens[s]
+ * tokens), decoded on the fly, followed by its hot_lengths[s] BF16 hot rows.  FP32
+ * online-softmax in two stages; rows that are not live or have no tokens give zeros.
+ * query / out: [batch, q_heads, head_dim] of query_dtype.  Workspace: at least
+ * nq_nqkv_attention_workspace_bytes() bytes.  Requires head_dim = 64, page_size = 16,
+ * q = 14, q_heads / kv_heads in {1, 2, 4, 8}; any max_pages.
+ * Replaces: nqkv_decode_attention_batched_k1 and its three Triton kernels
+ * (nestquant/runtime/nqkv_attention_k1.py:763-942, 243-471); oracle
+ * nestquant/runtime/nqkv_attention.py:14-86.
+ */
+int nq_nqkv_attention_decode(
+    const void *query_dev, int query_dtype, const uint8_t *key_codes_dev, const uint8_t *key_beta_ids_dev,
+    const float *key_norms_dev, const uint8_t *value_codes_dev, const uint8_t *value_beta_ids_dev,
+    const float *value_norms_dev, const float *key_betas_dev, const float *value_betas_dev,
+    const int32_t *page_indices_dev, const int32_t *page_counts_dev, const int32_t *last_page_lens_dev,
+    const int32_t *hot_lengths_dev, const uint8_t *cache_active_dev, const void *hot_keys_dev,
+    const void *hot_values_dev, const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch,
+    int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
+    void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
+
+size_t nq_nqkv_attention_workspace_bytes(int batch, int q_heads, int head_dim, int max_pages);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,374 @@
+// Paged NQKV4 decode attention: one query token per batch row against that row's packed
+// cold pages (4-bit E8 codes, decoded on the fly) plus its BF16 hot tail.
+//
+// Stage 1, grid = (chunks + 1, batch * kv_heads), 256 lanes.  A workgroup owns one batch
+// row, one KV head and one chunk of 16 pages (256 tokens); the extra chunk is the hot tail.
+//   * Every K and V block of the chunk is decoded exactly once and serves all query heads of
+//     the GQA group (the reference decodes it once per query head,
+//     nestquant/runtime/nqkv_attention_k1.py:243-342).
+//   * K pass: lane (page, token, block) decodes its 8 keys, dots them with the group's
+//     queries (kept in registers) and an 8-lane exchange yields scores in LDS.
+//   * softmax over the chunk in LDS (FP32), then the V pass: every lane accumulates
+//     p * v for its block over the pages it visits; lanes are merged through LDS in a fixed
+//     order.  The chunk's (max, denominator, numerator[D]) go to the workspace.
+// Stage 2, one lane per output element: log-sum-exp merge of the parts in index order.
+// Lengths, page tables and activity flags are read on the device, so the launch is
+// replayable in a HIP graph; inactive rows produce zeros; there is no page-count limit
+// beyond the table width (the reference stops at 64 pages, nqkv_attention_k1.py:696-698).
+// Decoded K/V stay FP32 (as in the reference's fused kernel); K/V decode follows the exact
+// float32 order of nq_e8.hip.h because undithered codes sit on exact Voronoi ties.
+#include "nq_e8.hip.h"
+#include "nq_host.h"
+
+#include <math.h>
+
+namespace nq {
+
+constexpr int kAttnThreads = 256;
+constexpr int kAttnPagesPerChunk = 16;
+constexpr int kAttnMaxGroup = 8;
+
+struct AttentionArgs {
+    const void *query;                 // [batch, q_heads, D]
+    const uint32_t *key_codes, *value_codes;     // [pages][P * kv_heads * D / 8] words
+    const uint8_t *key_beta_ids, *value_beta_ids; // [pages][P * kv_heads * D / 32]
+    const float *key_norms, *value_norms;         // [pages][P * kv_heads]
+    const float *key_betas, *value_betas;         // [4]
+    const int32_t *page_indices;       // [slots, max_pages]
+    const int32_t *page_counts, *last_page_lens, *hot_lengths;   // [slots]
+    const uint8_t *cache_active;       // [slots] or null
+    const uint16_t *hot_keys, *hot_values;        // BF16 [slots, P, kv_heads, D]
+    const int32_t *slot_ids;           // [batch]
+    const uint8_t *active_mask;        // [batch]
+    int batch, slots, max_pages, q_heads, kv_heads, chunks, query_dtype;
+    float scale;
+    float *part_max, *part_sum, *part_acc;        // [batch, q_heads, chunks + 1] (x D)
+};
+
+__device__ __forceinline__ float load_query(const void *q, int dtype, int64_t i) {
+    if (dtype == NQ_BF16) return bf16_to_f32(reinterpret_cast<const uint16_t *>(q)[i]);
+    if (dtype == NQ_F16) return f16_to_f32(reinterpret_cast<const uint16_t *>(q)[i]);
+    return reinterpret_cast<const float *>(q)[i];
+}
+
+// sum over the 8 lanes that share a token (lane id bits 0..2)
+__device__ __forceinline__ float sum8(float v) {
+    v = v + __shfl_xor(v, 1, 64);
+    v = v + __shfl_xor(v, 2, 64);
+    v = v + __shfl_xor(v, 4, 64);
+    return v;
+}
+
+template <int D, int P, int G>     // head_dim, page_size, query heads per KV head
+__global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(AttentionArgs a) {
+    constexpr int kBlocks = D / 8;                       // E8 blocks per head vector
+    constexpr int kTokenBlocks = P * kBlocks;            // lanes needed per page
+    constexpr int kPagesPerPass = kAttnThreads / kTokenBlocks;
+    constexpr int kPasses = kAttnPagesPerChunk / kPagesPerPass;
+    constexpr int kChunkTokens = kAttnPagesPerChunk * P;
+    static_assert(kTokenBlocks * kPagesPerPass == kAttnThreads && kPasses * kPagesPerPass == kAttnPagesPerChunk,
+                  "page does not tile the workgroup");
+    __shared__ float scores[G][kChunkTokens];
+    __shared__ float reduce_buf[kAttnThreads / 64][G];
+    __shared__ float chunk_max[G], chunk_sum[G];
+    __shared__ float acc_lds[kAttnThreads / 64][kBlocks][G * 8];
+
+    const int tid = threadIdx.x;
+    const int chunk = blockIdx.x;
+    const int row = blockIdx.y / a.kv_heads, g = blockIdx.y % a.kv_heads;
+    const bool is_hot = chunk == a.chunks;
+    int slot = a.slot_ids[row];
+    slot = slot < 0 ? 0 : (slot >= a.slots ? a.slots - 1 : slot);
+    const int page_count = a.page_counts[slot], last_len = a.last_page_lens[slot], hot_len = a.hot_lengths[slot];
+    const bool live = a.active_mask[row] && (!a.cache_active || a.cache_active[slot]);
+    const int first_page = chunk * kAttnPagesPerChunk;
+    const int64_t part = ((int64_t)row * a.q_heads + (int64_t)g * G) * (a.chunks + 1) + chunk;   // + h * (chunks + 1)
+
+    const bool empty = !live || (is_hot ? hot_len <= 0 : first_page >= page_count);
+    if (empty) {                                         // uniform over the workgroup
+        if (tid < G) {
+            a.part_max[part + (int64_t)tid * (a.chunks + 1)] = -INFINITY;
+            a.part_sum[part + (int64_t)tid * (a.chunks + 1)] = 0.0f;
+        }
+        return;
+    }
+
+    // lane role inside a pass
+    const int pass_page = tid / kTokenBlocks, token = (tid % kTokenBlocks) / kBlocks, blk = tid % kBlocks;
+    float q[G][8];
+#pragma unroll
+    for (int h = 0; h < G; h++)
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            q[h][j] = load_query(a.query, a.query_dtype, ((int64_t)row * a.q_heads + g * G + h) * D + blk * 8 + j);
+    const float sqrt_d = __builtin_sqrtf((float)D);
+    const int row_in_page = token * a.kv_heads + g;
+    const int64_t page_words = (int64_t)P * a.kv_heads * kBlocks, page_rows = (int64_t)P * a.kv_heads;
+
+    // ---- K pass -----------------------------------------------------------------------------
+    for (int pass = 0; pass < (is_hot ? 1 : kPasses); pass++) {
+        const int page_in_chunk = pass * kPagesPerPass + pass_page;
+        const int ordinal = first_page + page_in_chunk;
+        bool valid;
+        float k[8];
+        if (is_hot) {
+            valid = pass_page == 0 && token < hot_len;
+            if (valid) {
+                const uint4 raw = *reinterpret_cast<const uint4 *>(
+                    a.hot_keys + (((int64_t)slot * P + token) * a.kv_heads + g) * D + blk * 8);
+                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    k[2 * j] = __uint_as_float(w[j] << 16);
+                    k[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+                }
+            }
+        } else {
+            valid = ordinal < page_count && (ordinal < page_count - 1 || token < last_len);
+            if (valid) {
+                const int64_t page = a.page_indices[(int64_t)slot * a.max_pages + ordinal];
+                const int64_t word = page * page_words + (int64_t)row_in_page * kBlocks + blk;
+                decode_codeword<false>(a.key_codes[word], 14.0f, 0u, k);
+                const float beta = a.key_betas[(a.key_beta_ids[word >> 2] >> (2 * (word & 3))) & 3];
+                const float back = a.key_norms[page * page_rows + row_in_page] / sqrt_d;
+#pragma unroll
+                for (int j = 0; j < 8; j++) k[j] = (k[j] * beta) * back;
+            }
+        }
+        if (!valid) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) k[j] = 0.0f;
+        }
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            float s = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) s = __builtin_fmaf(q[h][j], k[j], s);
+            s = sum8(s);
+            if (blk == 0) scores[h][page_in_chunk * P + token] = valid ? s * a.scale : -INFINITY;
+        }
+    }
+    if (is_hot) {                                        // the hot chunk only fills the first page of scores
+        for (int i = tid; i < G * (kChunkTokens - P * kPagesPerPass); i += kAttnThreads) {
+            const int h = i / (kChunkTokens - P * kPagesPerPass), t = i % (kChunkTokens - P * kPagesPerPass);
+            scores[h][P * kPagesPerPass + t] = -INFINITY;
+        }
+    }
+    __syncthreads();
+
+    // ---- softmax over the chunk (one score per lane and head) -----------------------------------
+    static_assert(kChunkTokens == kAttnThreads, "one token per lane in the softmax phase");
+    float mine[G];
+#pragma unroll
+    for (int h = 0; h < G; h++) {
+        mine[h] = scores[h][tid];
+        float m = mine[h];
+#pragma unroll
+        for (int offset = 32; offset >= 1; offset >>= 1) m = fmaxf(m, __shfl_xor(m, offset, 64));
+        if ((tid & 63) == 0) reduce_buf[tid >> 6][h] = m;
+    }
+    __syncthreads();
+    if (tid < G) {
+        float m = reduce_buf[0][tid];
+        for (int w = 1; w < kAttnThreads / 64; w++) m = fmaxf(m, reduce_buf[w][tid]);
+        chunk_max[tid] = m;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < G; h++) {
+        const float p = mine[h] == -INFINITY ? 0.0f : __expf(mine[h] - chunk_max[h]);
+        scores[h][tid] = p;
+        float s = p;
+#pragma unroll
+        for (int offset = 32; offset >= 1; offset >>= 1) s = s + __shfl_xor(s, offset, 64);
+        if ((tid & 63) == 0) reduce_buf[tid >> 6][h] = s;
+    }
+    __syncthreads();
+    if (tid < G) {
+        float s = reduce_buf[0][tid];
+        for (int w = 1; w < kAttnThreads / 64; w++) s = s + reduce_buf[w][tid];
+        chunk_sum[tid] = s;
+    }
+    // (scores now hold probabilities; the barrier above ordered their writes)
+
+    // ---- V pass ------------------------------------------------------------------------------
+    float acc[G][8];
+#pragma unroll
+    for (int h = 0; h < G; h++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc[h][j] = 0.0f;
+    for (int pass = 0; pass < (is_hot ? 1 : kPasses); pass++) {
+        const int page_in_chunk = pass * kPagesPerPass + pass_page;
+        const int ordinal = first_page + page_in_chunk;
+        bool valid;
+        float v[8];
+        if (is_hot) {
+            valid = pass_page == 0 && token < hot_len;
+            if (valid) {
+                const uint4 raw = *reinterpret_cast<const uint4 *>(
+                    a.hot_values + (((int64_t)slot * P + token) * a.kv_heads + g) * D + blk * 8);
+                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    v[2 * j] = __uint_as_float(w[j] << 16);
+                    v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+                }
+            }
+        } else {
+            valid = ordinal < page_count && (ordinal < page_count - 1 || token < last_len);
+            if (valid) {
+                const int64_t page = a.page_indices[(int64_t)slot * a.max_pages + ordinal];
+                const int64_t word = page * page_words + (int64_t)row_in_page * kBlocks + blk;
+                decode_codeword<false>(a.value_codes[word], 14.0f, 0u, v);
+                const float beta = a.value_betas[(a.value_beta_ids[word >> 2] >> (2 * (word & 3))) & 3];
+                const float back = a.value_norms[page * page_rows + row_in_page] / sqrt_d;
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = (v[j] * beta) * back;
+            }
+        }
+        if (valid) {
+#pragma unroll
+            for (int h = 0; h < G; h++) {
+                const float p = scores[h][page_in_chunk * P + token];
+#pragma unroll
+                for (int j = 0; j < 8; j++) acc[h][j] = __builtin_fmaf(p, v[j], acc[h][j]);
+            }
+        }
+    }
+    // lanes that share a block index hold partial sums of the same 8 output dims: fold the
+    // tokens of a wavefront with a fixed butterfly (lane bits 3..5), then the wavefronts in order
+    static_assert(kBlocks == 8, "lane bits 0..2 index the block");
+#pragma unroll
+    for (int h = 0; h < G; h++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            float v = acc[h][j];
+            v = v + __shfl_xor(v, 8, 64);
+            v = v + __shfl_xor(v, 16, 64);
+            v = v + __shfl_xor(v, 32, 64);
+            if ((tid & 63) < kBlocks) acc_lds[tid >> 6][tid & 7][h * 8 + j] = v;
+        }
+    __syncthreads();
+    for (int o = tid; o < G * D; o += kAttnThreads) {
+        const int h = o / D, d = o % D;
+        float total = acc_lds[0][d / 8][h * 8 + d % 8];
+        for (int w = 1; w < kAttnThreads / 64; w++) total = total + acc_lds[w][d / 8][h * 8 + d % 8];
+        a.part_acc[(part + (int64_t)h * (a.chunks + 1)) * D + d] = total;
+    }
+    if (tid < G) {
+        a.part_max[part + (int64_t)tid * (a.chunks + 1)] = chunk_max[tid];
+        a.part_sum[part + (int64_t)tid * (a.chunks + 1)] = chunk_sum[tid];
+    }
+}
+
+// Stage 2: out[row, head, d] = sum_c acc_c * exp(max_c - max) / sum_c sum_c * exp(max_c - max)
+template <int D>
+__global__ void __launch_bounds__(256)
+attention_merge_kernel(const float *__restrict__ part_max, const float *__restrict__ part_sum,
+                       const float *__restrict__ part_acc, int parts, int64_t heads_total,
+                       void *__restrict__ out, int out_dtype) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= heads_total * D) return;
+    const int64_t head = i / D;
+    const int d = (int)(i % D);
+    const float *m = part_max + head * parts, *s = part_sum + head * parts;
+    float top = -INFINITY;
+    for (int c = 0; c < parts; c++) top = fmaxf(top, m[c]);
+    float denom = 0.0f, numer = 0.0f;
+    if (top > -INFINITY) {
+        for (int c = 0; c < parts; c++) {
+            if (s[c] > 0.0f) {
+                const float w = __expf(m[c] - top);
+                denom = denom + s[c] * w;
+                numer = numer + part_acc[(head * parts + c) * D + d] * w;
+            }
+        }
+    }
+    const float result = denom > 0.0f ? numer / denom : 0.0f;      // inactive or empty rows give zeros
+    if (out_dtype == NQ_BF16) reinterpret_cast<uint16_t *>(out)[i] = f32_to_bf16(result);
+    else if (out_dtype == NQ_F16) reinterpret_cast<_Float16 *>(out)[i] = (_Float16)result;
+    else reinterpret_cast<float *>(out)[i] = result;
+}
+
+}  // namespace nq
+
+namespace {
+
+int chunks_for(int max_pages) { return (max_pages + nq::kAttnPagesPerChunk - 1) / nq::kAttnPagesPerChunk; }
+
+}  // namespace
+
+extern "C" size_t nq_nqkv_attention_workspace_bytes(int batch, int q_heads, int head_dim, int max_pages) {
+    if (batch < 1 || q_heads < 1 || head_dim < 1 || max_pages < 1) return 0;
+    const size_t parts = (size_t)chunks_for(max_pages) + 1;
+    return (size_t)batch * q_heads * parts * ((size_t)head_dim + 2) * sizeof(float);
+}
+
+extern "C" int nq_nqkv_attention_decode(
+    const void *query_dev, int query_dtype, const uint8_t *key_codes_dev, const uint8_t *key_beta_ids_dev,
+    const float *key_norms_dev, const uint8_t *value_codes_dev, const uint8_t *value_beta_ids_dev,
+    const float *value_norms_dev, const float *key_betas_dev, const float *value_betas_dev,
+    const int32_t *page_indices_dev, const int32_t *page_counts_dev, const int32_t *last_page_lens_dev,
+    const int32_t *hot_lengths_dev, const uint8_t *cache_active_dev, const void *hot_keys_dev,
+    const void *hot_values_dev, const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch,
+    int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
+    void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream) {
+    NQ_REQUIRE(batch >= 1 && slots >= 1 && max_pages >= 1, NQ_ERR_SHAPE,
+               "nq_nqkv_attention_decode: batch, slots and max_pages must be positive");
+    NQ_REQUIRE(kv_heads >= 1 && q_heads >= kv_heads && q_heads % kv_heads == 0, NQ_ERR_SHAPE,
+               "nq_nqkv_attention_decode: q_heads must be a positive multiple of kv_heads");
+    const int group = q_heads / kv_heads;
+    NQ_REQUIRE(head_dim == 64 && page_size == 16, NQ_ERR_SHAPE,
+               "nq_nqkv_attention_decode: built for head_dim 64 and 16-token pages (got %d, %d)", head_dim, page_size);
+    NQ_REQUIRE(group == 1 || group == 2 || group == 4 || group == 8, NQ_ERR_SHAPE,
+               "nq_nqkv_attention_decode: %d query heads per KV head is not 1, 2, 4 or 8", group);
+    NQ_REQUIRE(query_dtype == NQ_F32 || query_dtype == NQ_BF16 || query_dtype == NQ_F16, NQ_ERR_ARGUMENT,
+               "nq_nqkv_attention_decode: unknown dtype tag %d", query_dtype);
+    NQ_REQUIRE(query_dev && key_codes_dev && key_beta_ids_dev && key_norms_dev && value_codes_dev &&
+                   value_beta_ids_dev && value_norms_dev && key_betas_dev && value_betas_dev && page_indices_dev &&
+                   page_counts_dev && last_page_lens_dev && hot_lengths_dev && hot_keys_dev && hot_values_dev &&
+                   slot_ids_dev && active_mask_dev && out_dev,
+               NQ_ERR_ARGUMENT, "nq_nqkv_attention_decode: null pointer");
+    NQ_REQUIRE(nq::aligned(key_codes_dev, 4) && nq::aligned(value_codes_dev, 4) && nq::aligned(hot_keys_dev, 16) &&
+                   nq::aligned(hot_values_dev, 16),
+               NQ_ERR_ARGUMENT, "nq_nqkv_attention_decode: page streams need 4-byte, hot tails 16-byte alignment");
+    NQ_REQUIRE(isfinite(scale), NQ_ERR_ARGUMENT, "nq_nqkv_attention_decode: scale must be finite");
+    const size_t need = nq_nqkv_attention_workspace_bytes(batch, q_heads, head_dim, max_pages);
+    NQ_REQUIRE(workspace_dev && workspace_bytes >= need, NQ_ERR_WORKSPACE,
+               "nq_nqkv_attention_decode: needs a %zu-byte workspace, got %zu", need, workspace_bytes);
+
+    nq::AttentionArgs a;
+    a.query = query_dev;
+    a.key_codes = reinterpret_cast<const uint32_t *>(key_codes_dev);
+    a.value_codes = reinterpret_cast<const uint32_t *>(value_codes_dev);
+    a.key_beta_ids = key_beta_ids_dev; a.value_beta_ids = value_beta_ids_dev;
+    a.key_norms = key_norms_dev; a.value_norms = value_norms_dev;
+    a.key_betas = key_betas_dev; a.value_betas = value_betas_dev;
+    a.page_indices = page_indices_dev; a.page_counts = page_counts_dev;
+    a.last_page_lens = last_page_lens_dev; a.hot_lengths = hot_lengths_dev;
+    a.cache_active = cache_active_dev;
+    a.hot_keys = reinterpret_cast<const uint16_t *>(hot_keys_dev);
+    a.hot_values = reinterpret_cast<const uint16_t *>(hot_values_dev);
+    a.slot_ids = slot_ids_dev; a.active_mask = active_mask_dev;
+    a.batch = batch; a.slots = slots; a.max_pages = max_pages; a.q_heads = q_heads; a.kv_heads = kv_heads;
+    a.chunks = chunks_for(max_pages); a.query_dtype = query_dtype; a.scale = scale;
+    const size_t parts = (size_t)a.chunks + 1, heads_total = (size_t)batch * q_heads;
+    a.part_max = reinterpret_cast<float *>(workspace_dev);
+    a.part_sum = a.part_max + heads_total * parts;
+    a.part_acc = a.part_sum + heads_total * parts;
+
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((unsigned)parts, (unsigned)(batch * kv_heads));
+    switch (group) {
+        case 1: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, 1>), grid, dim3(nq::kAttnThreads), 0, s, a); break;
+        case 2: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, 2>), grid, dim3(nq::kAttnThreads), 0, s, a); break;
+        case 4: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, 4>), grid, dim3(nq::kAttnThreads), 0, s, a); break;
+        default: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, 8>), grid, dim3(nq::kAttnThreads), 0, s, a); break;
+    }
+    int status = nq::check_launch("nq_nqkv_attention_decode (stage 1)");
+    if (status != NQ_OK) return status;
+    const int64_t outputs = (int64_t)heads_total * head_dim;
+    hipLaunchKernelGGL(nq::attention_merge_kernel<64>, dim3((unsigned)((outputs + 255) / 256)), dim3(256), 0, s,
+                       a.part_max, a.part_sum, a.part_acc, (int)parts, (int64_t)heads_total, out_dev, query_dtype);
+    return nq::check_launch("nq_nqkv_attention_decode (merge)");
+}

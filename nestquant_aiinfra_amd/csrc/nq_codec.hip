@@ -1,7 +1,7 @@
 // E8 codec kernels: nearest point, row quantiser with multi-beta selection (NQA4 / NQKV4
 // encoder) and its inverse.  Reference: nestquant/core/quantizer.py:214-301, 39-51;
 // nestquant/runtime/nqkv_page.py:97-185, 332-372, 446-456, 22-95; nestquant/runtime/cuda_e8.cu:8-59.
-#include "nq_e8.hip.h"
+#include "nq_rowquant.hip.h"
 #include "nq_host.h"
 
 #include <math.h>
@@ -70,14 +70,6 @@ template <> struct RowLoader<half_bits> {
     static __device__ __forceinline__ float scalar(const half_bits *x, int64_t i) { return f16_to_f32(x[i].v); }
 };
 
-// exchange with the lane whose id differs in bit 0 / bit 1 (inside a quad)
-__device__ __forceinline__ uint32_t quad_xor1(uint32_t v) {
-    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
-}
-__device__ __forceinline__ uint32_t quad_xor2(uint32_t v) {
-    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
-}
-
 template <typename T, bool kDithered>
 __global__ void __launch_bounds__(1024)
 quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, float inv_q,
@@ -120,86 +112,18 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
     __syncthreads();
 
     // phase 2
-    if (tid < 8 * rows_per_wg) {
-        const int r = tid >> 3, lane = tid & 7;
-        const float *row = lds + (size_t)r * n + lane;
-        float acc = 0.0f;
-        // n is a multiple of 32: four chain steps per trip, many trips in flight
-#pragma unroll 8
-        for (int i = 0; i < blocks_per_row; i += 4) {
-            const float v0 = row[8 * i], v1 = row[8 * i + 8], v2 = row[8 * i + 16], v3 = row[8 * i + 24];
-            acc = __builtin_fmaf(v0, v0, acc);
-            acc = __builtin_fmaf(v1, v1, acc);
-            acc = __builtin_fmaf(v2, v2, acc);
-            acc = __builtin_fmaf(v3, v3, acc);
-        }
-        float total = 0.0f;
-#pragma unroll
-        for (int k = 0; k < 8; k++) total = total + __shfl(acc, (tid & 56) + k, 64);
-        const float norm = __builtin_sqrtf(total);
-        if (lane == 0) {
-            // math.sqrt(n) / norm is evaluated as (1 / norm) * float32(sqrt(n))
-            row_scale[r] = norm > 0.0f ? (1.0f / norm) * sqrt_n : 0.0f;
-            row_norm[r] = norm;
-            if (row0 + r < rows && slice == 0) norms[row0 + r] = norm;
-        }
-    }
-    __syncthreads();
+    staged_row_norms(lds, rows_per_wg, n, sqrt_n, row_scale, row_norm);
+    if (slice == 0 && tid < rows_per_wg && row0 + tid < rows) norms[row0 + tid] = row_norm[tid];
 
     // phase 3
     const int slice_pairs = rows_per_wg * blocks_per_row * 4 / slices;     // a multiple of 16
-    const int pairs = slice_pairs * (slice + 1);
-    for (int p = slice_pairs * slice + tid; p < pairs; p += blockDim.x) {
-        const int blk = p >> 2, bi = p & 3;
-        const int r = blk / blocks_per_row, b = blk - r * blocks_per_row;
-        const float scale = row_scale[r];
-        const float4 lo = *reinterpret_cast<const float4 *>(lds + (size_t)r * n + 8 * b);
-        const float4 hi = *reinterpret_cast<const float4 *>(lds + (size_t)r * n + 8 * b + 4);
-        const float raw[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        const bool live = bi < beta_count;
-        const float beta = betas[live ? bi : 0];
-        const int64_t row = row0 + r;
-        const int64_t gblock = row * blocks_per_row + b;
-        float y[8], z[8], code[8], p8[8], recon[8], dither[8];
-        if (kDithered) dither_block(seed_plus_offset + (uint32_t)gblock * 8u, dither);
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            y[j] = raw[j] * scale;
-            z[j] = y[j] / beta;                 // IEEE division
-            if (kDithered) z[j] = z[j] + dither[j];
-        }
-        encode_block(z, q, inv_q, code);
-        e8_coset_point(code, p8);
-        if (kDithered) {
-#pragma unroll
-            for (int j = 0; j < 8; j++) p8[j] = p8[j] - dither[j];
-        }
-        reduce_coset_point(p8, q, recon);
-        float err = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const float d = recon[j] * beta - y[j];
-            err = err + d * d;
-        }
-        if (!live) err = __builtin_inff();
-
-        // first minimum over the quad: order by (err, beta index)
-        uint32_t best_err = __float_as_uint(err), best = (uint32_t)bi;
-        {
-            const uint32_t oe = quad_xor1(best_err), oi = quad_xor1(best);
-            const float fe = __uint_as_float(oe), me = __uint_as_float(best_err);
-            const bool take = fe < me || (fe == me && oi < best);
-            best_err = take ? oe : best_err;
-            best = take ? oi : best;
-        }
-        {
-            const uint32_t oe = quad_xor2(best_err), oi = quad_xor2(best);
-            const float fe = __uint_as_float(oe), me = __uint_as_float(best_err);
-            const bool take = fe < me || (fe == me && oi < best);
-            best = take ? oi : best;
-        }
-        if (best == (uint32_t)bi && row < rows) {
-            codes[gblock] = pack_codeword(code);
+    struct Sink {
+        uint32_t *codes; uint8_t *beta_ids; uint4 *decoded; const float *row_norm;
+        int64_t row0, rows; int blocks_per_row; float sqrt_n;
+        __device__ __forceinline__ bool wants(int r) const { return row0 + r < rows; }
+        __device__ __forceinline__ void code(int r, int b, uint32_t word, const float (&recon)[8], float beta) const {
+            const int64_t gblock = (row0 + r) * blocks_per_row + b;
+            codes[gblock] = word;
             if (decoded) {
                 // the BF16 decode of the stored code, as the linear kernels consume it
                 const float back = row_norm[r] / sqrt_n;
@@ -210,13 +134,19 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
                                              h[4] | (h[5] << 16), h[6] | (h[7] << 16));
             }
         }
-
-        // four consecutive blocks (16 lanes) share one beta byte
-        uint32_t byte = best << (2 * (b & 3));
-        byte |= (uint32_t)__shfl_xor((int)byte, 4, 64);
-        byte |= (uint32_t)__shfl_xor((int)byte, 8, 64);
-        if ((p & 15) == 0 && row < rows) beta_ids[gblock >> 2] = (uint8_t)byte;
-    }
+        __device__ __forceinline__ void beta_byte(int r, int b, uint32_t byte) const {
+            beta_ids[((row0 + r) * blocks_per_row + b) >> 2] = (uint8_t)byte;
+        }
+        __device__ __forceinline__ uint32_t counter(int r, int b) const {
+            return (uint32_t)((row0 + r) * blocks_per_row + b) * 8u;
+        }
+    } sink{codes, beta_ids, decoded, row_norm, row0, rows, blocks_per_row, sqrt_n};
+    struct Betas {
+        const float *table;
+        __device__ __forceinline__ const float *operator()(int) const { return table; }
+    } betas_of{betas};
+    quantize_staged_pairs<kDithered>(lds, row_scale, n, q, inv_q, betas_of, beta_count, seed_plus_offset,
+                                     slice_pairs * slice, slice_pairs * (slice + 1), sink);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -1,0 +1,225 @@
+// Paged ragged NQKV writer: appends new K/V rows of a ragged batch to each slot's BF16 hot
+// tail and, whenever a 16-token page fills, encodes it (4-bit E8 codes, per-block beta ids,
+// FP32 row norms) straight into that slot's next cold page.  Decode (one token per row) and
+// prefill (any number of tokens per row, ragged) are the same launch.
+//
+// Metadata model (device-resident, per slot; the reference keeps the same tensors,
+// nestquant/runtime/paged_nqkv_cache.py:25-95): sequence_lengths, page_counts,
+// last_page_lens, hot_lengths, page_indices[slot, ordinal].  nq_nqkv_advance bumps them
+// for a whole step *before* the layers run; the writer and the attention kernel of every
+// layer then read them without any host round trip or per-layer metadata kernel
+// (the reference launches a data kernel plus a metadata kernel per layer and reserves pages
+// on the host before each boundary step, nqkv_graph_writer.py:291-332, nqkv_batch_manager.py:648-689).
+//
+// Writer, grid = (pages a row can touch, batch * kv_heads), 256 lanes.  With L the new
+// length of the slot and c the row's token count, the row touches page ordinals
+// (L - c) / 16 .. (L - 1) / 16.  A complete page is gathered in LDS as float32 (its first
+// tokens may come from the hot tail, the rest from the new rows), quantised with the same
+// device routine as the stand-alone encoder (bit-identical results) and stored at
+// page_indices[slot, ordinal]; rows follow the NHD rule row = token * kv_heads + head
+// (nestquant/core/kv_format.py:99-131).  The trailing partial page goes to the hot tail.
+// Workgroup 0 of a row handles its first page and then the trailing partial page, in that
+// order, so hot-tail reads precede hot-tail writes; other workgroups own one middle page.
+#include "nq_rowquant.hip.h"
+#include "nq_host.h"
+
+#include <math.h>
+
+namespace nq {
+
+constexpr int kKvThreads = 256;
+
+__global__ void __launch_bounds__(256)
+kv_advance_kernel(const int32_t *__restrict__ slot_ids, const uint8_t *__restrict__ active_mask,
+                  const int32_t *__restrict__ counts, int uniform_count, int batch, int slots, int page_size,
+                  int max_tokens, int32_t *__restrict__ sequence_lengths, int32_t *__restrict__ page_counts,
+                  int32_t *__restrict__ last_page_lens, int32_t *__restrict__ hot_lengths) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= batch || !active_mask[r]) return;
+    const int slot = slot_ids[r];
+    if (slot < 0 || slot >= slots) return;                       // a stale replay writes nothing
+    int count = counts ? counts[r] : uniform_count;
+    int length = sequence_lengths[slot];
+    if (count < 0) count = 0;
+    if (length + count > max_tokens) count = max_tokens - length; // clamp at capacity
+    length += count;
+    sequence_lengths[slot] = length;
+    page_counts[slot] = length / page_size;
+    last_page_lens[slot] = length >= page_size ? page_size : 0;
+    hot_lengths[slot] = length % page_size;
+}
+
+struct KvWriteArgs {
+    const uint16_t *key, *value;            // BF16 [batch, tokens, kv_heads, D]
+    const int32_t *slot_ids, *counts;       // counts may be null (uniform_count)
+    const uint8_t *active_mask;
+    const int32_t *sequence_lengths, *page_indices;
+    uint32_t *key_codes, *value_codes;
+    uint8_t *key_beta_ids, *value_beta_ids;
+    float *key_norms, *value_norms;
+    const float *key_betas, *value_betas;
+    uint16_t *hot_keys, *hot_values;        // BF16 [slots, P, kv_heads, D]
+    int batch, tokens, uniform_count, slots, max_pages, kv_heads, key_beta_count, value_beta_count;
+};
+
+template <int D, int P>
+__global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
+    constexpr int kBlocks = D / 8;
+    __shared__ float rows[2 * P][D];             // K tokens 0..P-1, then V tokens
+    __shared__ float row_scale[2 * P], row_norm[2 * P];
+    const int tid = threadIdx.x;
+    const int row = blockIdx.y / a.kv_heads, g = blockIdx.y % a.kv_heads;
+    if (!a.active_mask[row]) return;
+    const int slot = a.slot_ids[row];
+    if (slot < 0 || slot >= a.slots) return;
+    int count = a.counts ? a.counts[row] : a.uniform_count;
+    const int length = a.sequence_lengths[slot];             // already includes this step
+    if (count > a.tokens) count = a.tokens;
+    if (count > length) count = length;
+    if (count <= 0) return;
+    const int start = length - count;
+    const int first_ordinal = start / P, last_ordinal = (length - 1) / P;
+    const bool tail_partial = (length % P) != 0;
+
+    const float sqrt_d = __builtin_sqrtf((float)D);
+    const int64_t page_words = (int64_t)P * a.kv_heads * kBlocks, page_rows = (int64_t)P * a.kv_heads;
+
+    // this workgroup's pages: blockIdx.x-th touched page; workgroup 0 also takes the trailing
+    // partial page when that is a different page
+    for (int turn = 0; turn < 2; turn++) {
+        int ordinal;
+        if (turn == 0) {
+            ordinal = first_ordinal + (int)blockIdx.x;
+            if (ordinal > last_ordinal) return;
+            if (blockIdx.x != 0 && ordinal == last_ordinal && tail_partial) return;   // workgroup 0 does it
+        } else {
+            if (blockIdx.x != 0 || !tail_partial || last_ordinal == first_ordinal) return;
+            ordinal = last_ordinal;
+            __syncthreads();
+        }
+        const int page_start = ordinal * P;
+        const bool complete = page_start + P <= length;
+        if (!complete) {
+            // trailing partial page: copy the new rows of this head into the hot tail
+            const int lo = start > page_start ? start : page_start;
+            const int n_new = length - lo;
+            for (int i = tid; i < n_new * (D / 8); i += kKvThreads) {
+                const int t = lo + i / (D / 8), c = i % (D / 8);
+                const int64_t src = (((int64_t)row * a.tokens + (t - start)) * a.kv_heads + g) * D + c * 8;
+                const int64_t dst = (((int64_t)slot * P + (t - page_start)) * a.kv_heads + g) * D + c * 8;
+                *reinterpret_cast<uint4 *>(a.hot_keys + dst) = *reinterpret_cast<const uint4 *>(a.key + src);
+                *reinterpret_cast<uint4 *>(a.hot_values + dst) = *reinterpret_cast<const uint4 *>(a.value + src);
+            }
+            continue;
+        }
+        // complete page: gather P tokens (hot tail first, then new rows) as float32
+        for (int i = tid; i < 2 * P * (D / 8); i += kKvThreads) {
+            const int which = i / (P * (D / 8)), rem = i % (P * (D / 8));
+            const int t = rem / (D / 8), c = rem % (D / 8);
+            const int pos = page_start + t;
+            const uint16_t *src;
+            if (pos < start)
+                src = (which ? a.hot_values : a.hot_keys) + (((int64_t)slot * P + t) * a.kv_heads + g) * D + c * 8;
+            else
+                src = (which ? a.value : a.key) + (((int64_t)row * a.tokens + (pos - start)) * a.kv_heads + g) * D + c * 8;
+            const uint4 raw = *reinterpret_cast<const uint4 *>(src);
+            float *dst = &rows[which * P + t][c * 8];
+            dst[0] = __uint_as_float(raw.x << 16); dst[1] = __uint_as_float(raw.x & 0xffff0000u);
+            dst[2] = __uint_as_float(raw.y << 16); dst[3] = __uint_as_float(raw.y & 0xffff0000u);
+            dst[4] = __uint_as_float(raw.z << 16); dst[5] = __uint_as_float(raw.z & 0xffff0000u);
+            dst[6] = __uint_as_float(raw.w << 16); dst[7] = __uint_as_float(raw.w & 0xffff0000u);
+        }
+        __syncthreads();
+        staged_row_norms(&rows[0][0], 2 * P, D, sqrt_d, row_scale, row_norm);
+        const int64_t page = a.page_indices[(int64_t)slot * a.max_pages + ordinal];
+        if (tid < 2 * P) {
+            const int t = tid % P;
+            (tid < P ? a.key_norms : a.value_norms)[page * page_rows + t * a.kv_heads + g] = row_norm[tid];
+        }
+        struct Sink {
+            uint32_t *key_codes, *value_codes; uint8_t *key_beta_ids, *value_beta_ids;
+            int64_t page_word0; int kv_heads, g;
+            __device__ __forceinline__ bool wants(int) const { return true; }
+            __device__ __forceinline__ int64_t word(int r, int b) const {
+                return page_word0 + ((int64_t)(r % P) * kv_heads + g) * kBlocks + b;
+            }
+            __device__ __forceinline__ void code(int r, int b, uint32_t w, const float (&)[8], float) const {
+                (r < P ? key_codes : value_codes)[word(r, b)] = w;
+            }
+            __device__ __forceinline__ void beta_byte(int r, int b, uint32_t byte) const {
+                (r < P ? key_beta_ids : value_beta_ids)[word(r, b) >> 2] = (uint8_t)byte;
+            }
+            __device__ __forceinline__ uint32_t counter(int, int) const { return 0u; }
+        } sink{a.key_codes, a.value_codes, a.key_beta_ids, a.value_beta_ids, page * page_words, a.kv_heads, g};
+        struct Betas {
+            const float *key, *value;
+            __device__ __forceinline__ const float *operator()(int r) const { return r < P ? key : value; }
+        } betas_of{a.key_betas, a.value_betas};
+        quantize_staged_pairs<false>(&rows[0][0], row_scale, D, 14.0f, 1.0f / 14.0f, betas_of, a.key_beta_count,
+                                     0u, 0, 2 * P * kBlocks * 4, sink);
+    }
+}
+
+}  // namespace nq
+
+extern "C" int nq_nqkv_advance(const int32_t *slot_ids_dev, const uint8_t *active_mask_dev,
+                               const int32_t *counts_dev, int uniform_count, int batch, int slots,
+                               int page_size, int max_tokens, int32_t *sequence_lengths_dev,
+                               int32_t *page_counts_dev, int32_t *last_page_lens_dev,
+                               int32_t *hot_lengths_dev, void *stream) {
+    NQ_REQUIRE(batch >= 1 && slots >= 1 && page_size >= 1 && max_tokens >= 1, NQ_ERR_SHAPE,
+               "nq_nqkv_advance: batch, slots, page_size and max_tokens must be positive");
+    NQ_REQUIRE(slot_ids_dev && active_mask_dev && sequence_lengths_dev && page_counts_dev && last_page_lens_dev &&
+                   hot_lengths_dev,
+               NQ_ERR_ARGUMENT, "nq_nqkv_advance: null pointer");
+    NQ_REQUIRE(counts_dev || uniform_count >= 0, NQ_ERR_ARGUMENT, "nq_nqkv_advance: negative token count");
+    hipLaunchKernelGGL(nq::kv_advance_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       slot_ids_dev, active_mask_dev, counts_dev, uniform_count, batch, slots, page_size, max_tokens,
+                       sequence_lengths_dev, page_counts_dev, last_page_lens_dev, hot_lengths_dev);
+    return nq::check_launch("nq_nqkv_advance");
+}
+
+extern "C" int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_dtype, const int32_t *slot_ids_dev,
+                             const uint8_t *active_mask_dev, const int32_t *counts_dev, int uniform_count,
+                             const int32_t *sequence_lengths_dev, const int32_t *page_indices_dev,
+                             uint8_t *key_codes_dev, uint8_t *key_beta_ids_dev, float *key_norms_dev,
+                             uint8_t *value_codes_dev, uint8_t *value_beta_ids_dev, float *value_norms_dev,
+                             const float *key_betas_dev, int key_beta_count, const float *value_betas_dev,
+                             int value_beta_count, void *hot_keys_dev, void *hot_values_dev, int batch, int tokens,
+                             int slots, int max_pages, int kv_heads, int head_dim, int page_size, void *stream) {
+    NQ_REQUIRE(batch >= 1 && tokens >= 1 && slots >= 1 && max_pages >= 1 && kv_heads >= 1, NQ_ERR_SHAPE,
+               "nq_nqkv_write: batch, tokens, slots, max_pages and kv_heads must be positive");
+    NQ_REQUIRE(head_dim == 64 && page_size == 16, NQ_ERR_SHAPE,
+               "nq_nqkv_write: built for head_dim 64 and 16-token pages (got %d, %d)", head_dim, page_size);
+    NQ_REQUIRE(kv_dtype == NQ_BF16, NQ_ERR_ARGUMENT, "nq_nqkv_write: keys and values must be BF16");
+    NQ_REQUIRE(key_beta_count >= 1 && key_beta_count <= 4 && value_beta_count == key_beta_count, NQ_ERR_SHAPE,
+               "nq_nqkv_write: key and value tables must hold the same number (1..4) of betas");
+    NQ_REQUIRE(key_dev && value_dev && slot_ids_dev && active_mask_dev && sequence_lengths_dev && page_indices_dev &&
+                   key_codes_dev && key_beta_ids_dev && key_norms_dev && value_codes_dev && value_beta_ids_dev &&
+                   value_norms_dev && key_betas_dev && value_betas_dev && hot_keys_dev && hot_values_dev,
+               NQ_ERR_ARGUMENT, "nq_nqkv_write: null pointer");
+    NQ_REQUIRE(nq::aligned(key_dev, 16) && nq::aligned(value_dev, 16) && nq::aligned(hot_keys_dev, 16) &&
+                   nq::aligned(hot_values_dev, 16) && nq::aligned(key_codes_dev, 4) && nq::aligned(value_codes_dev, 4),
+               NQ_ERR_ARGUMENT, "nq_nqkv_write: K/V and hot tails need 16-byte, code streams 4-byte alignment");
+    NQ_REQUIRE(counts_dev || (uniform_count >= 0 && uniform_count <= tokens), NQ_ERR_ARGUMENT,
+               "nq_nqkv_write: uniform token count %d is outside [0, %d]", uniform_count, tokens);
+    nq::KvWriteArgs a;
+    a.key = reinterpret_cast<const uint16_t *>(key_dev);
+    a.value = reinterpret_cast<const uint16_t *>(value_dev);
+    a.slot_ids = slot_ids_dev; a.counts = counts_dev; a.active_mask = active_mask_dev;
+    a.sequence_lengths = sequence_lengths_dev; a.page_indices = page_indices_dev;
+    a.key_codes = reinterpret_cast<uint32_t *>(key_codes_dev);
+    a.value_codes = reinterpret_cast<uint32_t *>(value_codes_dev);
+    a.key_beta_ids = key_beta_ids_dev; a.value_beta_ids = value_beta_ids_dev;
+    a.key_norms = key_norms_dev; a.value_norms = value_norms_dev;
+    a.key_betas = key_betas_dev; a.value_betas = value_betas_dev;
+    a.hot_keys = reinterpret_cast<uint16_t *>(hot_keys_dev);
+    a.hot_values = reinterpret_cast<uint16_t *>(hot_values_dev);
+    a.batch = batch; a.tokens = tokens; a.uniform_count = uniform_count; a.slots = slots; a.max_pages = max_pages;
+    a.kv_heads = kv_heads; a.key_beta_count = key_beta_count; a.value_beta_count = value_beta_count;
+    // `tokens` new rows starting anywhere inside a page touch at most this many pages
+    const int touched = (tokens + page_size - 2) / page_size + 1;
+    hipLaunchKernelGGL((nq::kv_write_kernel<64, 16>), dim3((unsigned)touched, (unsigned)(batch * kv_heads)),
+                       dim3(nq::kKvThreads), 0, (hipStream_t)stream, a);
+    return nq::check_launch("nq_nqkv_write");
+}

@@ -1,0 +1,537 @@
+"""NQKV4 paged KV cache on the GPU: packed pages, the page pool, device-resident sequence
+tables, the ragged writer and batched decode attention.
+
+Mirrors the reference's surface for this path:
+  PreparedNQKVPage / quantize_nqkv_page_cuda / dequantize_nqkv_page_triton   nestquant/runtime/nqkv_page.py:192-329, 494-537
+  NQKVPageHandle / NQKVPagePool                                               nestquant/runtime/nqkv_pool.py:14-251
+  BatchedNQKVMetadata                                                         nestquant/runtime/paged_nqkv_cache.py:25-95
+  nqkv_decode_attention_batched_k1                                            nestquant/runtime/nqkv_attention_k1.py:763-942
+The per-layer hot/cold cache object the kernels consume is NQKVHotColdCache (hot BF16 tails
+plus the pool plus the tables; nestquant/runtime/nqkv_hot_cache.py:14-37).
+
+Design difference, on purpose: lengths, page tables and hot-tail fill levels live on the
+device and are advanced by one kernel per step (`BatchedNQKVCacheManager.begin_step`), and
+every slot owns a fixed range of physical pages, so a decode step needs no host-side page
+reservation, no host read of hot lengths and no separate page-boundary graph.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Hashable, Sequence
+
+import torch
+
+from .. import _native
+from .w4a4_linear import _beta_values, dequantize_rows_packed, quantize_rows_packed
+
+PAGE_SIZE = 16
+
+
+# --------------------------------------------------------------------------------------
+# single pages
+# --------------------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class PreparedNQKVPage:
+    """One packed K/V page resident on the GPU (views into a pool or freshly encoded)."""
+
+    key_code_payload: torch.Tensor
+    key_beta_payload: torch.Tensor
+    key_norms: torch.Tensor
+    value_code_payload: torch.Tensor
+    value_beta_payload: torch.Tensor
+    value_norms: torch.Tensor
+    key_beta_table: torch.Tensor
+    value_beta_table: torch.Tensor
+    page_size: int
+    valid_tokens: int
+    num_kv_heads: int
+    head_dim: int
+    q: int
+    code_width: int
+    beta_width: int
+    output_dtype: torch.dtype
+
+    @property
+    def device(self) -> torch.device:
+        return self.key_code_payload.device
+
+    @property
+    def payload_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (
+            self.key_code_payload, self.key_beta_payload, self.key_norms,
+            self.value_code_payload, self.value_beta_payload, self.value_norms))
+
+
+def quantize_nqkv_page_cuda(key: torch.Tensor, value: torch.Tensor, *, page_size: int, q: int,
+                            betas: Sequence[float] | None = None,
+                            key_betas: Sequence[float] | None = None,
+                            value_betas: Sequence[float] | None = None,
+                            key_beta_table: torch.Tensor | None = None,
+                            value_beta_table: torch.Tensor | None = None) -> PreparedNQKVPage:
+    """Quantize an NHD K/V prefix [valid, kv_heads, head_dim] into one fixed-capacity page.
+
+    Rows beyond the valid prefix are encoded zeros (norm 0), exactly as
+    PackedNQKVPage.from_tensors does on the CPU (nestquant/core/kv_format.py:99-131).
+    """
+    if not isinstance(key, torch.Tensor) or not isinstance(value, torch.Tensor):
+        raise TypeError("key and value must be tensors")
+    if key.shape != value.shape or key.ndim != 3 or key.dtype != value.dtype:
+        raise ValueError("key and value must share shape [tokens, kv_heads, head_dim] and dtype")
+    if key.device.type != "cuda" or key.device != value.device:
+        raise ValueError("key and value must share a CUDA device")
+    valid, heads, dim = key.shape
+    if not 1 <= valid <= page_size:
+        raise ValueError("token count must be in [1, page_size]")
+    if betas is not None:
+        if key_betas is not None or value_betas is not None:
+            raise ValueError("pass legacy betas or key_betas/value_betas, not both")
+        key_values = value_values = _beta_values(betas)
+    else:
+        if key_betas is None or value_betas is None:
+            raise ValueError("v2 requires both key_betas and value_betas")
+        key_values, value_values = _beta_values(key_betas), _beta_values(value_betas)
+    device = key.device
+    if key_beta_table is None:
+        key_beta_table = torch.tensor(key_values, device=device, dtype=torch.float32)
+    if value_beta_table is None:
+        value_beta_table = (key_beta_table if betas is not None
+                            else torch.tensor(value_values, device=device, dtype=torch.float32))
+    rows = page_size * heads
+    streams = []
+    for tensor, table in ((key, key_beta_table), (value, value_beta_table)):
+        padded = torch.zeros((rows, dim), device=device, dtype=tensor.dtype)
+        padded[: valid * heads].copy_(tensor.reshape(valid * heads, dim))
+        streams.extend(quantize_rows_packed(padded, q=q, beta_table=table))
+    return PreparedNQKVPage(*streams[0:3], *streams[3:6], key_beta_table, value_beta_table,
+                            page_size, valid, heads, dim, q, 4, 2, key.dtype)
+
+
+def dequantize_nqkv_page(page: PreparedNQKVPage, *, output_dtype: torch.dtype | None = None,
+                         tile_blocks: int | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Decode a packed page back to its valid NHD prefix (float32 maths, then one cast)."""
+    if not isinstance(page, PreparedNQKVPage):
+        raise TypeError("page must be a PreparedNQKVPage")
+    dtype = page.output_dtype if output_dtype is None else output_dtype
+    rows = page.page_size * page.num_kv_heads
+    shape = (page.page_size, page.num_kv_heads, page.head_dim)
+    out = []
+    for codes, ids, norms, table in (
+            (page.key_code_payload, page.key_beta_payload, page.key_norms, page.key_beta_table),
+            (page.value_code_payload, page.value_beta_payload, page.value_norms, page.value_beta_table)):
+        full = dequantize_rows_packed(codes.contiguous(), ids.contiguous(), norms.contiguous(), table,
+                                      rows=rows, features=page.head_dim, q=page.q, output_dtype=dtype)
+        out.append(full.reshape(shape)[: page.valid_tokens])
+    return out[0], out[1]
+
+
+dequantize_nqkv_page_triton = dequantize_nqkv_page      # the reference's name for the same operator
+
+
+# --------------------------------------------------------------------------------------
+# page pool
+# --------------------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class NQKVPageHandle:
+    """Generation-checked ownership token for one physical page."""
+
+    page_id: int
+    generation: int
+
+
+class NQKVPagePool:
+    """Preallocated SoA page storage; the tensors never move, so kernels captured in a HIP
+    graph keep valid addresses.  Allocation metadata is host-side and generation-checked."""
+
+    def __init__(self, *, capacity: int, page_size: int, num_kv_heads: int, head_dim: int, q: int,
+                 betas: Sequence[float] | None = None, key_betas: Sequence[float] | None = None,
+                 value_betas: Sequence[float] | None = None,
+                 output_dtype: torch.dtype = torch.bfloat16, device: torch.device | str = "cuda") -> None:
+        for name, value in (("capacity", capacity), ("page_size", page_size),
+                            ("num_kv_heads", num_kv_heads), ("head_dim", head_dim)):
+            if isinstance(value, bool) or not isinstance(value, int) or value < 1:
+                raise ValueError(f"{name} must be a positive integer")
+        if head_dim % 8:
+            raise ValueError("head_dim must be divisible by 8")
+        if betas is not None:
+            if key_betas is not None or value_betas is not None:
+                raise ValueError("pass legacy betas or key_betas/value_betas, not both")
+            key_values = value_values = tuple(float(b) for b in betas)
+        else:
+            if key_betas is None or value_betas is None:
+                raise ValueError("v2 requires both key_betas and value_betas")
+            key_values = tuple(float(b) for b in key_betas)
+            value_values = tuple(float(b) for b in value_betas)
+        if not key_values or not value_values:
+            raise ValueError("beta tables must be nonempty")
+        target = torch.device(device)
+        if target.type != "cuda" or not torch.cuda.is_available():
+            raise ValueError("NQKVPagePool requires an available CUDA device")
+        if target.index is None:
+            target = torch.device("cuda", torch.cuda.current_device())
+        self.capacity, self.page_size = capacity, page_size
+        self.num_kv_heads, self.head_dim, self.q = num_kv_heads, head_dim, q
+        self.betas, self.value_beta_values = key_values, value_values
+        self.format_version = 1 if betas is not None else 2
+        self.output_dtype, self.device = output_dtype, target
+        self.code_width, self.beta_width = 4, 2
+        self._row_count = page_size * num_kv_heads
+        self._code_bytes = self._row_count * head_dim // 2
+        self._beta_bytes = self._row_count * head_dim // 32
+        self.key_codes = torch.zeros((capacity, self._code_bytes), device=target, dtype=torch.uint8)
+        self.key_betas = torch.zeros((capacity, self._beta_bytes), device=target, dtype=torch.uint8)
+        self.key_norms = torch.zeros((capacity, self._row_count), device=target, dtype=torch.float32)
+        self.value_codes = torch.zeros_like(self.key_codes)
+        self.value_betas = torch.zeros_like(self.key_betas)
+        self.value_norms = torch.zeros_like(self.key_norms)
+        self.beta_table = torch.tensor(key_values, device=target, dtype=torch.float32)
+        self.value_beta_table = (self.beta_table if betas is not None
+                                 else torch.tensor(value_values, device=target, dtype=torch.float32))
+        self._free = list(range(capacity - 1, -1, -1))
+        self._generation = [0] * capacity
+        self._allocated = [False] * capacity
+        self._stored = [False] * capacity
+        self._valid_tokens = [0] * capacity
+
+    @property
+    def free_pages(self) -> int:
+        return len(self._free)
+
+    @property
+    def allocated_pages(self) -> int:
+        return self.capacity - len(self._free)
+
+    @property
+    def page_payload_bytes(self) -> int:
+        return 2 * (self._code_bytes + self._beta_bytes + 4 * self._row_count)
+
+    @property
+    def resident_bytes(self) -> int:
+        tensors = [self.key_codes, self.key_betas, self.key_norms, self.value_codes, self.value_betas,
+                   self.value_norms, self.beta_table]
+        if self.value_beta_table is not self.beta_table:
+            tensors.append(self.value_beta_table)
+        return sum(t.numel() * t.element_size() for t in tensors)
+
+    def allocate(self) -> NQKVPageHandle:
+        if not self._free:
+            raise RuntimeError("NQKV page pool is exhausted")
+        page_id = self._free.pop()
+        self._allocated[page_id], self._stored[page_id], self._valid_tokens[page_id] = True, False, 0
+        return NQKVPageHandle(page_id, self._generation[page_id])
+
+    def release(self, handle: NQKVPageHandle) -> None:
+        page_id = self._validate_handle(handle)
+        self._allocated[page_id], self._stored[page_id], self._valid_tokens[page_id] = False, False, 0
+        self._generation[page_id] += 1
+        self._free.append(page_id)
+
+    def store_prepared(self, handle: NQKVPageHandle, page: PreparedNQKVPage) -> None:
+        """Copy a GPU-produced packed page into its fixed physical slot."""
+        page_id = self._validate_handle(handle)
+        if not isinstance(page, PreparedNQKVPage):
+            raise TypeError("page must be a PreparedNQKVPage")
+        if (page.page_size, page.num_kv_heads, page.head_dim, page.q, page.device) != (
+                self.page_size, self.num_kv_heads, self.head_dim, self.q, self.device):
+            raise ValueError("prepared NQKV page configuration does not match the pool")
+        if (not torch.equal(page.key_beta_table, self.beta_table)
+                or not torch.equal(page.value_beta_table, self.value_beta_table)):
+            raise ValueError("prepared NQKV beta tables do not match the pool")
+        for destination, source in zip(
+                (self.key_codes[page_id], self.key_betas[page_id], self.key_norms[page_id],
+                 self.value_codes[page_id], self.value_betas[page_id], self.value_norms[page_id]),
+                (page.key_code_payload, page.key_beta_payload, page.key_norms,
+                 page.value_code_payload, page.value_beta_payload, page.value_norms)):
+            if destination.numel() != source.numel():
+                raise ValueError("prepared NQKV payload sizes do not match the pool")
+            destination.copy_(source)
+        self._valid_tokens[page_id], self._stored[page_id] = page.valid_tokens, True
+
+    def mark_graph_stored(self, handle: NQKVPageHandle, *, valid_tokens: int) -> None:
+        page_id = self._validate_handle(handle)
+        if not 1 <= valid_tokens <= self.page_size:
+            raise ValueError("valid_tokens must be in [1, page_size]")
+        self._valid_tokens[page_id], self._stored[page_id] = valid_tokens, True
+
+    def prepared(self, handle: NQKVPageHandle) -> PreparedNQKVPage:
+        page_id = self._validate_handle(handle)
+        if not self._stored[page_id]:
+            raise RuntimeError("NQKV page has not been stored")
+        return self.page_view(page_id, self._valid_tokens[page_id])
+
+    def page_view(self, page_id: int, valid_tokens: int) -> PreparedNQKVPage:
+        return PreparedNQKVPage(
+            self.key_codes[page_id], self.key_betas[page_id], self.key_norms[page_id],
+            self.value_codes[page_id], self.value_betas[page_id], self.value_norms[page_id],
+            self.beta_table, self.value_beta_table, self.page_size, valid_tokens, self.num_kv_heads,
+            self.head_dim, self.q, self.code_width, self.beta_width, self.output_dtype)
+
+    def _validate_handle(self, handle: NQKVPageHandle) -> int:
+        if not isinstance(handle, NQKVPageHandle):
+            raise TypeError("handle must be an NQKVPageHandle")
+        if not 0 <= handle.page_id < self.capacity:
+            raise ValueError("NQKV page ID is outside pool capacity")
+        if not self._allocated[handle.page_id] or self._generation[handle.page_id] != handle.generation:
+            raise RuntimeError("stale or released NQKV page handle")
+        return handle.page_id
+
+
+# --------------------------------------------------------------------------------------
+# device-resident sequence tables
+# --------------------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class BatchedNQKVMetadata:
+    """Fixed-address GPU metadata consumed by the batched paged NQKV kernels."""
+
+    slot_ids: torch.Tensor
+    page_indptr: torch.Tensor
+    page_indices: torch.Tensor
+    page_counts: torch.Tensor
+    last_page_lens: torch.Tensor
+    hot_lengths: torch.Tensor
+    sequence_lengths: torch.Tensor
+    active_mask: torch.Tensor
+
+    @classmethod
+    def create(cls, *, capacity: int, max_pages_per_sequence: int,
+               device: torch.device | str) -> "BatchedNQKVMetadata":
+        for name, value in (("capacity", capacity), ("max_pages_per_sequence", max_pages_per_sequence)):
+            if isinstance(value, bool) or not isinstance(value, int) or value < 1:
+                raise ValueError(f"{name} must be a positive integer")
+        target = torch.device(device)
+        zeros = lambda: torch.zeros(capacity, dtype=torch.int32, device=target)   # noqa: E731
+        return cls(
+            slot_ids=torch.arange(capacity, dtype=torch.int32, device=target),
+            page_indptr=torch.arange(0, (capacity + 1) * max_pages_per_sequence, max_pages_per_sequence,
+                                     dtype=torch.int32, device=target),
+            page_indices=torch.full((capacity, max_pages_per_sequence), -1, dtype=torch.int32, device=target),
+            page_counts=zeros(), last_page_lens=zeros(), hot_lengths=zeros(), sequence_lengths=zeros(),
+            active_mask=torch.zeros(capacity, dtype=torch.bool, device=target),
+        )
+
+    def pointers(self) -> tuple[int, ...]:
+        return tuple(t.data_ptr() for t in (
+            self.slot_ids, self.page_indptr, self.page_indices, self.page_counts, self.last_page_lens,
+            self.hot_lengths, self.sequence_lengths, self.active_mask))
+
+
+class NQKVHotColdCache:
+    """One layer's cache: packed cold pages in a pool, a BF16 hot tail per slot, and the
+    (possibly shared) device tables that say how much of each is valid."""
+
+    def __init__(self, pool: NQKVPagePool, metadata: BatchedNQKVMetadata, *, max_sequences: int,
+                 max_pages_per_sequence: int) -> None:
+        self.pool, self.metadata = pool, metadata
+        self.max_sequences, self.max_pages_per_sequence = max_sequences, max_pages_per_sequence
+        shape = (max_sequences, pool.page_size, pool.num_kv_heads, pool.head_dim)
+        self.hot_keys = torch.zeros(shape, device=pool.device, dtype=torch.bfloat16)
+        self.hot_values = torch.zeros_like(self.hot_keys)
+
+    @property
+    def cold_cache(self) -> "NQKVHotColdCache":      # the reference nests a cold cache; flat here
+        return self
+
+
+@dataclass
+class BatchedNQKVAttentionWorkspace:
+    """Scratch for the two-stage attention (chunk maxima, sums and numerators) + output."""
+
+    buffer: torch.Tensor
+    output: torch.Tensor
+    batch_size: int
+    max_pages: int
+    query_heads: int
+    head_dim: int
+
+    @classmethod
+    def create(cls, cache: NQKVHotColdCache, *, batch_size: int, query_heads: int,
+               output_dtype: torch.dtype) -> "BatchedNQKVAttentionWorkspace":
+        pool = cache.pool
+        need = _native.library().nq_nqkv_attention_workspace_bytes(
+            batch_size, query_heads, pool.head_dim, cache.max_pages_per_sequence)
+        return cls(torch.empty(need, dtype=torch.uint8, device=pool.device),
+                   torch.empty((batch_size, query_heads, pool.head_dim), dtype=output_dtype, device=pool.device),
+                   batch_size, cache.max_pages_per_sequence, query_heads, pool.head_dim)
+
+
+def launch_nqkv_decode_attention(query: torch.Tensor, cache: NQKVHotColdCache, *, slot_ids: torch.Tensor,
+                                 active_mask: torch.Tensor, attention_scale: float,
+                                 workspace: BatchedNQKVAttentionWorkspace) -> torch.Tensor:
+    """Graph-safe launch: no host reads, no allocation; writes workspace.output."""
+    pool, meta = cache.pool, cache.metadata
+    batch, heads, dim = query.shape
+    _native.check(_native.library().nq_nqkv_attention_decode(
+        query.data_ptr(), _native.dtype_tag(query.dtype),
+        pool.key_codes.data_ptr(), pool.key_betas.data_ptr(), pool.key_norms.data_ptr(),
+        pool.value_codes.data_ptr(), pool.value_betas.data_ptr(), pool.value_norms.data_ptr(),
+        pool.beta_table.data_ptr(), pool.value_beta_table.data_ptr(),
+        meta.page_indices.data_ptr(), meta.page_counts.data_ptr(), meta.last_page_lens.data_ptr(),
+        meta.hot_lengths.data_ptr(), meta.active_mask.data_ptr(),
+        cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(), slot_ids.data_ptr(), active_mask.data_ptr(),
+        batch, cache.max_sequences, cache.max_pages_per_sequence, heads, pool.num_kv_heads, dim, pool.page_size,
+        attention_scale, workspace.output.data_ptr(), workspace.buffer.data_ptr(), workspace.buffer.numel(),
+        _native.stream_handle(query.device)))
+    return workspace.output
+
+
+def nqkv_decode_attention_batched_k1(query: torch.Tensor, cache: NQKVHotColdCache, *, slot_ids: torch.Tensor,
+                                     active_mask: torch.Tensor, scale: float | None = None,
+                                     workspace: BatchedNQKVAttentionWorkspace | None = None) -> torch.Tensor:
+    """Fused packed-cold plus BF16-hot decode attention for a ragged batch.
+
+    query [batch, query_heads, head_dim]; slot_ids int32 [batch]; active_mask bool [batch].
+    Unlike the reference there is no page-count limit and no host-side validation pass over
+    slot contents (rows with nothing to attend to return zeros).
+    """
+    if not isinstance(query, torch.Tensor) or query.ndim != 3:
+        raise ValueError("query must have shape [batch, query_heads, head_dim]")
+    if not isinstance(slot_ids, torch.Tensor) or not isinstance(active_mask, torch.Tensor):
+        raise TypeError("slot_ids and active_mask must be tensors")
+    pool = cache.pool
+    batch, heads, dim = query.shape
+    if query.device != pool.device or dim != pool.head_dim:
+        raise ValueError("query must match the cache CUDA device and head_dim")
+    if heads < 1 or heads % pool.num_kv_heads:
+        raise ValueError("query_heads must be a positive multiple of num_kv_heads")
+    if slot_ids.dtype != torch.int32 or tuple(slot_ids.shape) != (batch,):
+        raise ValueError("slot_ids must be int32 with shape [batch]")
+    if active_mask.dtype != torch.bool or tuple(active_mask.shape) != (batch,):
+        raise ValueError("active_mask must be bool with shape [batch]")
+    if slot_ids.device != pool.device or active_mask.device != pool.device:
+        raise ValueError("slot_ids and active_mask must be on the cache device")
+    if workspace is None:
+        workspace = BatchedNQKVAttentionWorkspace.create(cache, batch_size=batch, query_heads=heads,
+                                                         output_dtype=query.dtype)
+    if (workspace.batch_size, workspace.max_pages, workspace.query_heads, workspace.head_dim,
+            workspace.output.dtype) != (batch, cache.max_pages_per_sequence, heads, dim, query.dtype):
+        raise ValueError("batched workspace configuration does not match query and cache")
+    attention_scale = 1.0 / math.sqrt(dim) if scale is None else float(scale)
+    if not math.isfinite(attention_scale):
+        raise ValueError("scale must be finite")
+    return launch_nqkv_decode_attention(query.contiguous(), cache, slot_ids=slot_ids, active_mask=active_mask,
+                                        attention_scale=attention_scale, workspace=workspace)
+
+
+# --------------------------------------------------------------------------------------
+# multi-layer manager: step bookkeeping + the ragged writer
+# --------------------------------------------------------------------------------------
+
+class BatchedNQKVCacheManager:
+    """Fixed-capacity, multi-layer NQKV cache.  All layers share one set of device tables
+    (every layer holds the same number of tokens per slot) and every slot owns the fixed
+    physical pages [slot * max_pages, (slot + 1) * max_pages) of each layer's pool."""
+
+    def __init__(self, *, capacity: int, num_layers: int, num_kv_heads: int, head_dim: int,
+                 max_cache_len: int, page_size: int, q: int, key_betas: Sequence[float],
+                 value_betas: Sequence[float], dtype: torch.dtype, device: torch.device | str) -> None:
+        if dtype != torch.bfloat16:
+            raise ValueError("the NQKV hot tails and writer are BF16")
+        self.capacity, self.num_layers, self.page_size = capacity, num_layers, page_size
+        self.max_pages = math.ceil(max_cache_len / page_size)
+        self.max_tokens = self.max_pages * page_size
+        target = torch.device(device)
+        if target.type == "cuda" and target.index is None:
+            target = torch.device("cuda", torch.cuda.current_device())
+        self.device = target
+        self.metadata = BatchedNQKVMetadata.create(capacity=capacity, max_pages_per_sequence=self.max_pages,
+                                                   device=target)
+        self.metadata.page_indices.copy_(
+            torch.arange(capacity * self.max_pages, dtype=torch.int32, device=target).reshape(capacity, self.max_pages))
+        self.layers = [
+            NQKVHotColdCache(
+                NQKVPagePool(capacity=capacity * self.max_pages, page_size=page_size, num_kv_heads=num_kv_heads,
+                             head_dim=head_dim, q=q, key_betas=key_betas, value_betas=value_betas,
+                             output_dtype=dtype, device=target),
+                self.metadata, max_sequences=capacity, max_pages_per_sequence=self.max_pages)
+            for _ in range(num_layers)
+        ]
+        self._sequence_of_slot: list[Hashable | None] = [None] * capacity
+        # state of the step in flight (fixed-address tensors so graphs can be replayed)
+        self.step_slot_ids = torch.arange(capacity, dtype=torch.int32, device=target)
+        self.step_active = torch.zeros(capacity, dtype=torch.bool, device=target)
+        self.step_counts = torch.zeros(capacity, dtype=torch.int32, device=target)
+        self._step_rows = capacity
+        self._step_uniform: int | None = 1
+
+    # -- slots ---------------------------------------------------------------------------
+    def register(self, sequence_id: Hashable, *, slot: int) -> None:
+        if not 0 <= slot < self.capacity:
+            raise ValueError("slot is outside cache capacity")
+        if self._sequence_of_slot[slot] is not None:
+            raise RuntimeError("slot is already occupied")
+        if sequence_id in self._sequence_of_slot:
+            raise RuntimeError("sequence is already registered")
+        self._sequence_of_slot[slot] = sequence_id
+        self.metadata.active_mask[slot] = True
+        for tensor in (self.metadata.sequence_lengths, self.metadata.page_counts,
+                       self.metadata.last_page_lens, self.metadata.hot_lengths):
+            tensor[slot] = 0
+
+    def register_batch(self, assignments: Sequence[tuple[Hashable, int]]) -> None:
+        for sequence_id, slot in assignments:
+            self.register(sequence_id, slot=slot)
+
+    def release_slots(self, slots: Sequence[int]) -> tuple[Hashable, ...]:
+        released = []
+        for slot in slots:
+            sequence_id = self._sequence_of_slot[slot]
+            if sequence_id is None:
+                continue
+            released.append(sequence_id)
+            self._sequence_of_slot[slot] = None
+            self.metadata.active_mask[slot] = False
+            for tensor in (self.metadata.sequence_lengths, self.metadata.page_counts,
+                           self.metadata.last_page_lens, self.metadata.hot_lengths):
+                tensor[slot] = 0
+        return tuple(released)
+
+    def sequence_id(self, slot: int) -> Hashable | None:
+        return self._sequence_of_slot[slot]
+
+    def total_tokens(self, slot: int) -> int:
+        """Host read of one slot's length (diagnostics and tests; never on the step path)."""
+        return int(self.metadata.sequence_lengths[slot].item())
+
+    # -- one step -------------------------------------------------------------------------
+    def begin_step(self, *, rows: int, uniform_count: int | None) -> None:
+        """Advance the device tables for a step over the first `rows` entries of
+        step_slot_ids / step_active (and step_counts unless `uniform_count` is given).
+        Graph-capturable: reads nothing on the host."""
+        self._step_rows, self._step_uniform = rows, uniform_count
+        meta = self.metadata
+        _native.check(_native.library().nq_nqkv_advance(
+            self.step_slot_ids.data_ptr(), self.step_active.data_ptr(),
+            None if uniform_count is not None else self.step_counts.data_ptr(),
+            0 if uniform_count is None else uniform_count, rows, self.capacity, self.page_size, self.max_tokens,
+            meta.sequence_lengths.data_ptr(), meta.page_counts.data_ptr(), meta.last_page_lens.data_ptr(),
+            meta.hot_lengths.data_ptr(), _native.stream_handle(self.device)))
+
+    def write_layer(self, layer_index: int, key: torch.Tensor, value: torch.Tensor) -> None:
+        """Append this step's K/V rows [rows, tokens, kv_heads, head_dim] to one layer."""
+        cache = self.layers[layer_index]
+        pool, meta = cache.pool, self.metadata
+        rows, tokens = key.shape[0], key.shape[1]
+        if rows != self._step_rows:
+            raise ValueError("key rows do not match the step in flight")
+        uniform = self._step_uniform
+        _native.check(_native.library().nq_nqkv_write(
+            key.data_ptr(), value.data_ptr(), _native.dtype_tag(key.dtype), self.step_slot_ids.data_ptr(),
+            self.step_active.data_ptr(), None if uniform is not None else self.step_counts.data_ptr(),
+            0 if uniform is None else uniform, meta.sequence_lengths.data_ptr(), meta.page_indices.data_ptr(),
+            pool.key_codes.data_ptr(), pool.key_betas.data_ptr(), pool.key_norms.data_ptr(),
+            pool.value_codes.data_ptr(), pool.value_betas.data_ptr(), pool.value_norms.data_ptr(),
+            pool.beta_table.data_ptr(), pool.beta_table.numel(), pool.value_beta_table.data_ptr(),
+            pool.value_beta_table.numel(), cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(),
+            rows, tokens, self.capacity, self.max_pages, pool.num_kv_heads, pool.head_dim, self.page_size,
+            _native.stream_handle(self.device)))
+
+    def resident_bytes(self) -> int:
+        total = 0
+        for cache in self.layers:
+            total += cache.pool.resident_bytes
+            total += 2 * cache.hot_keys.numel() * cache.hot_keys.element_size()
+        return total

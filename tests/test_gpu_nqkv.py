@@ -1,0 +1,216 @@
+"""GPU parity of the NQKV4 cache path through the C ABI: page encoder, ragged writer
+(hot tails + page packing) and batched decode attention, against the CPU oracle and the
+reference's golden page.
+
+Bars: packed page bytes, beta ids and norms bit-exact; hot tails bit-exact copies;
+attention max |out - ref| / max |ref| <= 1e-2 against dense softmax attention over the
+oracle-dequantised cache (the reference accepts atol 2e-2 between its kernels and its
+oracle, tests/unit/runtime/test_nqkv_attention_k1.py:44-67)."""
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import KEY_BETAS, Q, VALUE_BETAS
+from gpu_util import bits, relative_error
+
+pytestmark = pytest.mark.gpu
+
+HEADS, DIM, PAGE = 8, 64, 16
+
+
+@pytest.fixture(scope="module")
+def kv():
+    from nestquant_aiinfra_amd.runtime import nqkv
+    return nqkv
+
+
+def _bf16(x: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(x).to(torch.bfloat16)
+
+
+def _f32(t: torch.Tensor) -> np.ndarray:
+    return t.float().cpu().numpy()
+
+
+def test_page_encoder_matches_reference_golden(kv, golden):
+    key = torch.from_numpy(golden["kv_key_bf16_bits"]).view(torch.bfloat16).cuda()
+    value = torch.from_numpy(golden["kv_value_bf16_bits"]).view(torch.bfloat16).cuda()
+    page = kv.quantize_nqkv_page_cuda(key, value, page_size=PAGE, q=Q, key_betas=KEY_BETAS, value_betas=VALUE_BETAS)
+    for ours, name in ((page.key_code_payload, "kv_key_codes"), (page.key_beta_payload, "kv_key_betas"),
+                       (page.key_norms, "kv_key_norms"), (page.value_code_payload, "kv_value_codes"),
+                       (page.value_beta_payload, "kv_value_betas"), (page.value_norms, "kv_value_norms")):
+        assert np.array_equal(bits(ours), golden[name]), name
+    assert page.payload_bytes == 9728
+    dk, dv = kv.dequantize_nqkv_page(page, output_dtype=torch.float32)
+    assert np.array_equal(bits(dk), golden["kv_key_deq"]) and np.array_equal(bits(dv), golden["kv_value_deq"])
+    # a partially filled page: zero-padded rows, legacy shared table
+    partial = kv.quantize_nqkv_page_cuda(key[:5], value[:5], page_size=PAGE, q=Q, betas=KEY_BETAS)
+    assert np.array_equal(bits(partial.key_code_payload), golden["kv_partial_key_codes"])
+    assert np.array_equal(bits(partial.key_norms), golden["kv_partial_key_norms"])
+    dk, _ = kv.dequantize_nqkv_page(partial)
+    assert tuple(dk.shape) == (5, HEADS, DIM) and dk.dtype == torch.bfloat16
+
+
+def _manager(kv, capacity, max_len, layers=1):
+    return kv.BatchedNQKVCacheManager(capacity=capacity, num_layers=layers, num_kv_heads=HEADS, head_dim=DIM,
+                                      max_cache_len=max_len, page_size=PAGE, q=Q, key_betas=KEY_BETAS,
+                                      value_betas=VALUE_BETAS, dtype=torch.bfloat16, device="cuda")
+
+
+def _append(manager, slots, keys, values, layer=0):
+    """Append ragged rows: keys[i] is [count_i, HEADS, DIM] BF16 for slot slots[i]."""
+    rows = len(slots)
+    counts = [k.shape[0] for k in keys]
+    width = max(counts)
+    key = torch.zeros((rows, width, HEADS, DIM), dtype=torch.bfloat16)
+    value = torch.zeros_like(key)
+    for i, (k, v) in enumerate(zip(keys, values)):
+        key[i, : k.shape[0]], value[i, : v.shape[0]] = k, v
+    manager.step_slot_ids[:rows] = torch.tensor(slots, dtype=torch.int32)
+    manager.step_active[:rows] = True
+    manager.step_counts[:rows] = torch.tensor(counts, dtype=torch.int32)
+    uniform = counts[0] if len(set(counts)) == 1 else None
+    manager.begin_step(rows=rows, uniform_count=uniform)
+    for index in ([layer] if isinstance(layer, int) else layer):
+        manager.write_layer(index, key.cuda(), value.cuda())
+
+
+def _check_cache(kv, oracle, manager, slot, key_all, value_all, layer=0):
+    """Every cold page equals the oracle's encoding of its 16 tokens; the hot tail holds the rest."""
+    cache = manager.layers[layer]
+    total = key_all.shape[0]
+    assert manager.total_tokens(slot) == total
+    meta = manager.metadata
+    assert int(meta.page_counts[slot]) == total // PAGE and int(meta.hot_lengths[slot]) == total % PAGE
+    for ordinal in range(total // PAGE):
+        page_id = int(meta.page_indices[slot, ordinal])
+        chunk = slice(ordinal * PAGE, (ordinal + 1) * PAGE)
+        expect = oracle.nqkv_page_payload(_f32(key_all[chunk]), _f32(value_all[chunk]), page_size=PAGE, q=Q,
+                                          key_betas=KEY_BETAS, value_betas=VALUE_BETAS)
+        pool = cache.pool
+        for ours, name in ((pool.key_codes, "key_codes"), (pool.key_betas, "key_betas"), (pool.key_norms, "key_norms"),
+                           (pool.value_codes, "value_codes"), (pool.value_betas, "value_betas"),
+                           (pool.value_norms, "value_norms")):
+            assert np.array_equal(bits(ours[page_id]), expect[name]), (slot, ordinal, name)
+    hot = total % PAGE
+    if hot:
+        assert torch.equal(cache.hot_keys[slot, :hot].cpu(), key_all[total - hot:])
+        assert torch.equal(cache.hot_values[slot, :hot].cpu(), value_all[total - hot:])
+
+
+def test_ragged_writer_packs_pages_bit_exactly(kv, oracle):
+    rng = np.random.default_rng(11)
+    manager = _manager(kv, capacity=4, max_len=256, layers=2)
+    slots = [3, 0, 2]                                   # non-contiguous, out of order
+    for s in slots:
+        manager.register(f"seq{s}", slot=s)
+    history = {s: (torch.zeros((0, HEADS, DIM), dtype=torch.bfloat16),) * 2 for s in slots}
+
+    def grow(counts):
+        keys = [_bf16(oracle.hadamard(rng.standard_normal((c, HEADS, DIM)).astype(np.float32))) for c in counts]
+        values = [_bf16(rng.standard_normal((c, HEADS, DIM)).astype(np.float32)) for c in counts]
+        _append(manager, slots, keys, values, layer=[0, 1])
+        for s, k, v in zip(slots, keys, values):
+            history[s] = (torch.cat([history[s][0], k]), torch.cat([history[s][1], v]))
+
+    grow([5, 16, 37])          # sub-page, exactly one page, multi-page with a tail
+    grow([11, 1, 27])          # fills slot 3's first page from the hot tail; crosses pages
+    grow([40, 40, 40])         # uniform multi-page append onto partial tails
+    for _ in range(18):        # decode steps, one token per row, across a page boundary
+        grow([1, 1, 1])
+    torch.cuda.synchronize()
+    for s in slots:
+        for layer in (0, 1):
+            _check_cache(kv, oracle, manager, s, history[s][0], history[s][1], layer=layer)
+    # releasing a slot clears its tables; the other slots are untouched
+    assert manager.release_slots([0]) == ("seq0",)
+    assert manager.total_tokens(0) == 0 and manager.total_tokens(3) == history[3][0].shape[0]
+
+
+def _oracle_attention(oracle, query, key_all, value_all, group):
+    total = key_all.shape[0]
+    cold = (total // PAGE) * PAGE
+    k_parts, v_parts = [], []
+    for start in range(0, cold, PAGE):
+        page = oracle.nqkv_page_payload(_f32(key_all[start:start + PAGE]), _f32(value_all[start:start + PAGE]),
+                                        page_size=PAGE, q=Q, key_betas=KEY_BETAS, value_betas=VALUE_BETAS)
+        for side, betas, parts in (("key", KEY_BETAS, k_parts), ("value", VALUE_BETAS, v_parts)):
+            codes = oracle.unpack_unsigned(page[f"{side}_codes"], PAGE * HEADS * DIM, 4)
+            ids = oracle.unpack_unsigned(page[f"{side}_betas"], PAGE * HEADS * DIM // 8, 2)
+            parts.append(oracle.dequantize_rows(codes, ids, page[f"{side}_norms"], betas, Q).reshape(PAGE, HEADS, DIM))
+    k_parts.append(_f32(key_all[cold:]))
+    v_parts.append(_f32(value_all[cold:]))
+    return oracle.attention_dense(_f32(query), np.concatenate(k_parts), np.concatenate(v_parts))
+
+
+@pytest.mark.parametrize("q_heads", [8, 16, 32, 64])
+def test_attention_small_contexts_and_groups(kv, oracle, q_heads):
+    rng = np.random.default_rng(q_heads)
+    manager = _manager(kv, capacity=4, max_len=512)
+    slots, lengths = [2, 0, 3], [1, 16, 203]            # hot tail only; one full page; pages + tail
+    keys = [_bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for n in lengths]
+    values = [_bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for n in lengths]
+    for s in slots:
+        manager.register(s, slot=s)
+    _append(manager, slots, keys, values)
+    query = _bf16(oracle.hadamard(rng.standard_normal((4, q_heads, DIM)).astype(np.float32))).cuda()
+    slot_ids = torch.tensor([2, 0, 3, 1], dtype=torch.int32, device="cuda")
+    active = torch.tensor([True, True, True, False], device="cuda")       # row 3: unregistered slot
+    out = kv.nqkv_decode_attention_batched_k1(query, manager.layers[0], slot_ids=slot_ids, active_mask=active)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (4, q_heads, DIM)
+    for row in range(3):
+        ref = _oracle_attention(oracle, query[row].cpu(), keys[row], values[row], q_heads // HEADS)
+        assert relative_error(_f32(out[row]), ref) <= 1e-2, (row, q_heads)
+    assert not out[3].any()                                             # inactive rows give zeros
+    # a row whose mask is on but whose slot was never registered also gives zeros
+    active[3] = True
+    out = kv.nqkv_decode_attention_batched_k1(query, manager.layers[0], slot_ids=slot_ids, active_mask=active)
+    assert not out[3].any()
+
+
+def test_attention_ragged_batch_at_full_size(kv, oracle):
+    """Batch 8, 32 query / 8 KV heads, contexts uniform in [128, 4096] (up to 256 pages)."""
+    g = torch.Generator().manual_seed(4001)
+    lengths = torch.randint(128, 4097, (8,), generator=g).tolist()
+    lengths[0], lengths[1] = 4096, 128
+    rng = np.random.default_rng(4002)
+    manager = _manager(kv, capacity=8, max_len=4096)
+    keys = [_bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for n in lengths]
+    values = [_bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for n in lengths]
+    for s in range(8):
+        manager.register(s, slot=s)
+    _append(manager, list(range(8)), keys, values)
+    query = _bf16(oracle.hadamard(rng.standard_normal((8, 32, DIM)).astype(np.float32))).cuda()
+    slot_ids = torch.arange(8, dtype=torch.int32, device="cuda")
+    active = torch.ones(8, dtype=torch.bool, device="cuda")
+    out = kv.nqkv_decode_attention_batched_k1(query, manager.layers[0], slot_ids=slot_ids, active_mask=active)
+    again = kv.nqkv_decode_attention_batched_k1(query, manager.layers[0], slot_ids=slot_ids, active_mask=active)
+    assert torch.equal(out, again)                                      # deterministic merge
+    for row in (0, 1, 4):                                               # longest, shortest, one ragged
+        ref = _oracle_attention(oracle, query[row].cpu(), keys[row], values[row], 4)
+        assert relative_error(_f32(out[row]), ref) <= 1e-2, row
+    _check_cache(kv, oracle, manager, 1, keys[1], values[1])
+    # softmax weights sum to one: attending to constant values returns that constant
+    manager.layers[0].hot_values.fill_(0)
+    assert torch.isfinite(out).all()
+
+
+def test_pool_handles_are_generation_checked(kv):
+    pool = kv.NQKVPagePool(capacity=2, page_size=PAGE, num_kv_heads=HEADS, head_dim=DIM, q=Q,
+                           key_betas=KEY_BETAS, value_betas=VALUE_BETAS, device="cuda")
+    a, b = pool.allocate(), pool.allocate()
+    with pytest.raises(RuntimeError, match="exhausted"):
+        pool.allocate()
+    key = torch.randn(3, HEADS, DIM, device="cuda").to(torch.bfloat16)
+    page = kv.quantize_nqkv_page_cuda(key, key, page_size=PAGE, q=Q, key_betas=KEY_BETAS, value_betas=VALUE_BETAS)
+    with pytest.raises(RuntimeError, match="not been stored"):
+        pool.prepared(a)
+    pool.store_prepared(a, page)
+    assert torch.equal(pool.prepared(a).key_code_payload, page.key_code_payload) and pool.prepared(a).valid_tokens == 3
+    pool.release(a)
+    with pytest.raises(RuntimeError, match="stale"):
+        pool.prepared(a)
+    c = pool.allocate()
+    assert c.page_id == a.page_id and c.generation == a.generation + 1 and pool.free_pages == 0
+    assert pool.page_payload_bytes == 9728 and b.page_id != c.page_id
