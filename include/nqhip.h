@@ -63,6 +63,9 @@ int nq_e8_nearest(const float *x_dev, float *out_dev, int64_t count, void *strea
  * block_offset + r * n/8 + b and `seed` is added before the lattice search and removed
  * after it: this is the NQRT4 weight encoder (nestquant/core/quantizer.py:214-301 with
  * generate_e8_dither_stateless, nestquant/core/codec.py:176-224).
+ * hadamard != 0 first rotates every row with the normalized Hadamard transform (n a power
+ * of two), in the arithmetic of x_dtype as nq_hadamard does with stage_dtype = x_dtype, so
+ * a Linear input needs one launch for rotate + norm + encode + pack.
  * decoded_bf16_dev (optional, may be NULL): BF16 [rows, n] decode of the stored codes,
  * bf16((decode * beta) * (norm / sqrt(n))), which the linear kernels accept in place of
  * decoding the packed activation again.
@@ -74,8 +77,20 @@ int nq_e8_nearest(const float *x_dev, float *out_dev, int64_t count, void *strea
  */
 int nq_quantize_rows(const void *x_dev, int x_dtype, int64_t rows, int64_t n, int q,
                      const float *betas_dev, int beta_count, int has_dither, int64_t seed,
-                     int64_t block_offset, uint8_t *codes_dev, uint8_t *beta_ids_dev,
+                     int64_t block_offset, int hadamard, uint8_t *codes_dev, uint8_t *beta_ids_dev,
                      float *norms_dev, void *decoded_bf16_dev, void *stream);
+
+/*
+ * Normalized Sylvester-Hadamard transform of `rows` rows of power-of-two length n, with the
+ * reference's butterfly order (widths 1, 2, 4, ...), every sum and difference rounded to
+ * stage_dtype (NQ_F32 = no intermediate rounding) and a final multiplication by
+ * float32(1 / sqrt(n)); the result is written as out_dtype.
+ * Replaces: hadamard(), nestquant/core/rotation.py:12-27, as used on Linear inputs
+ * (nestquant/models/fused_linear.py:287-290, in the input dtype) and on post-RoPE queries
+ * and keys (nestquant/runtime/nqkv_batched_hf_backend.py:381, 549, in float32).
+ */
+int nq_hadamard(const void *x_dev, int x_dtype, int64_t rows, int64_t n, int stage_dtype,
+                void *out_dev, int out_dtype, void *stream);
 
 /*
  * Inverse of nq_quantize_rows: out[r, :] = (decode(codes) * beta[id]) * (norm[r] / sqrt(n)).
@@ -172,6 +187,9 @@ int nq_nqkv_advance(const int32_t *slot_ids_dev, const uint8_t *active_mask_dev,
  * positions sequence_lengths[s] - count .. sequence_lengths[s] - 1 (lengths already advanced).
  * Rows land in the slot's hot tail; every page completed by the write is encoded (the row
  * quantiser of nq_quantize_rows, bit-identical) into physical page page_indices[s, ordinal].
+ * rotate_keys != 0 first applies the normalized Hadamard transform over head_dim to the new
+ * key rows (float32 butterflies, result rounded to BF16), i.e. the caller passes post-RoPE
+ * keys and need not launch nq_hadamard.
  * Requires head_dim = 64, page_size = 16, q = 14, equal beta counts.
  * Replaces: append_hot_k1_graph_safe / ragged sub-page and segment writers
  * (nestquant/runtime/nqkv_graph_writer.py:263-473), launch_pack_full_hot_pages_graph_safe
@@ -185,7 +203,8 @@ int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_dtype, cons
                   uint8_t *value_codes_dev, uint8_t *value_beta_ids_dev, float *value_norms_dev,
                   const float *key_betas_dev, int key_beta_count, const float *value_betas_dev,
                   int value_beta_count, void *hot_keys_dev, void *hot_values_dev, int batch, int tokens,
-                  int slots, int max_pages, int kv_heads, int head_dim, int page_size, void *stream);
+                  int slots, int max_pages, int kv_heads, int head_dim, int page_size, int rotate_keys,
+                  void *stream);
 
 /*
  * Paged NQKV4 decode attention for a ragged batch: for batch row r with slot s (clamped to
@@ -194,7 +213,9 @@ int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_dtype, cons
  * page_counts[s] cold pages (all full except the last, which holds last_page_lens[s]
  * tokens), decoded on the fly, followed by its hot_lengths[s] BF16 hot rows.  FP32
  * online-softmax in two stages; rows that are not live or have no tokens give zeros.
- * query / out: [batch, q_heads, head_dim] of query_dtype.  Workspace: at least
+ * query / out: [batch, q_heads, head_dim] of query_dtype; rotate_query != 0 applies the
+ * normalized Hadamard transform over head_dim to the query first (float32, rounded to
+ * query_dtype), matching keys stored with rotate_keys.  Workspace: at least
  * nq_nqkv_attention_workspace_bytes() bytes.  Requires head_dim = 64, page_size = 16,
  * q = 14, q_heads / kv_heads in {1, 2, 4, 8}; any max_pages.
  * Replaces: nqkv_decode_attention_batched_k1 and its three Triton kernels
@@ -209,7 +230,7 @@ int nq_nqkv_attention_decode(
     const int32_t *hot_lengths_dev, const uint8_t *cache_active_dev, const void *hot_keys_dev,
     const void *hot_values_dev, const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch,
     int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
-    void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
+    int rotate_query, void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
 
 size_t nq_nqkv_attention_workspace_bytes(int batch, int q_heads, int head_dim, int max_pages);
 

@@ -30,8 +30,9 @@ SIGNATURES = {
     "nq_abi_version": (_i32, []),
     "nq_last_error": (_c.c_char_p, []),
     "nq_e8_nearest": (_i32, [_ptr, _ptr, _i64, _ptr]),
-    "nq_quantize_rows": (_i32, [_ptr, _i32, _i64, _i64, _i32, _ptr, _i32, _i32, _i64, _i64,
+    "nq_quantize_rows": (_i32, [_ptr, _i32, _i64, _i64, _i32, _ptr, _i32, _i32, _i64, _i64, _i32,
                                 _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "nq_hadamard": (_i32, [_ptr, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr]),
     "nq_dequantize_rows": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i64, _i64,
                                   _ptr, _i32, _ptr]),
     "nq_w4a4_gemv": (_i32, [_ptr] * 9 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
@@ -42,8 +43,8 @@ SIGNATURES = {
     "nq_w4a4_gemm_workspace_bytes": (_size, [_i32, _i32, _i32, _i32, _i32]),
     "nq_nqkv_advance": (_i32, [_ptr, _ptr, _ptr, _i32, _i32, _i32, _i32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "nq_nqkv_write": (_i32, [_ptr, _ptr, _i32, _ptr, _ptr, _ptr, _i32, _ptr, _ptr] + [_ptr] * 6
-                      + [_ptr, _i32, _ptr, _i32, _ptr, _ptr] + [_i32] * 7 + [_ptr]),
-    "nq_nqkv_attention_decode": (_i32, [_ptr, _i32] + [_ptr] * 17 + [_i32] * 7 + [_c.c_float, _ptr, _ptr,
+                      + [_ptr, _i32, _ptr, _i32, _ptr, _ptr] + [_i32] * 8 + [_ptr]),
+    "nq_nqkv_attention_decode": (_i32, [_ptr, _i32] + [_ptr] * 17 + [_i32] * 7 + [_c.c_float, _i32, _ptr, _ptr,
                                                                                 _size, _ptr]),
     "nq_nqkv_attention_workspace_bytes": (_size, [_i32, _i32, _i32, _i32]),
 }

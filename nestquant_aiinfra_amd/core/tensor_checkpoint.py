@@ -17,7 +17,6 @@ import json
 import struct
 from dataclasses import dataclass
 
-import numpy as np
 import torch
 
 from .codec import (CURRENT_CODEC_SEMANTICS, LEGACY_CODEC_SEMANTICS, STATELESS_DITHER_ALGORITHM,
@@ -30,20 +29,20 @@ _VERSION = 4
 _DTYPE_TO_NAME = {torch.float16: "float16", torch.bfloat16: "bfloat16",
                   torch.float32: "float32", torch.float64: "float64"}
 _NAME_TO_DTYPE = {name: dtype for dtype, name in _DTYPE_TO_NAME.items()}
-_NUMPY_VIEW = {torch.float16: np.float16, torch.float32: np.float32, torch.float64: np.float64}
 
 
 def _tensor_to_bytes(tensor: torch.Tensor) -> bytes:
-    tensor = tensor.detach().cpu().contiguous()
-    if tensor.dtype == torch.bfloat16:
-        return tensor.view(torch.int16).numpy().tobytes()
-    return tensor.numpy().tobytes()
+    """Raw little-endian bytes of a tensor of any dtype."""
+    flat = tensor.detach().cpu().contiguous().reshape(-1)
+    if flat.numel() == 0:
+        return b""
+    return flat.view(torch.uint8).numpy().tobytes()
 
 
 def _tensor_from_bytes(blob: bytes, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
-    if dtype == torch.bfloat16:
-        return torch.from_numpy(np.frombuffer(blob, dtype=np.int16).copy()).view(torch.bfloat16).reshape(shape)
-    return torch.from_numpy(np.frombuffer(blob, dtype=_NUMPY_VIEW[dtype]).copy()).reshape(shape)
+    if not blob:
+        return torch.empty(shape, dtype=dtype)
+    return torch.frombuffer(bytearray(blob), dtype=dtype).reshape(shape)
 
 
 def _validate_stateless(seed, algorithm) -> None:

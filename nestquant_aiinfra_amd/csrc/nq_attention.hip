@@ -40,7 +40,7 @@ struct AttentionArgs {
     const uint16_t *hot_keys, *hot_values;        // BF16 [slots, P, kv_heads, D]
     const int32_t *slot_ids;           // [batch]
     const uint8_t *active_mask;        // [batch]
-    int batch, slots, max_pages, q_heads, kv_heads, chunks, query_dtype;
+    int batch, slots, max_pages, q_heads, kv_heads, chunks, query_dtype, rotate_query;
     float scale;
     float *part_max, *part_sum, *part_acc;        // [batch, q_heads, chunks + 1] (x D)
 };
@@ -95,12 +95,39 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
 
     // lane role inside a pass
     const int pass_page = tid / kTokenBlocks, token = (tid % kTokenBlocks) / kBlocks, blk = tid % kBlocks;
+    // the group's queries, optionally Hadamard-rotated here (float32 butterflies over the head,
+    // scaled by 1 / sqrt(D), rounded to the query dtype: hadamard(query.float()).to(dtype),
+    // nestquant/runtime/nqkv_batched_hf_backend.py:549)
+    float *q_lds = &scores[0][0];
+    for (int i = tid; i < G * D; i += kAttnThreads)
+        q_lds[i] = load_query(a.query, a.query_dtype, ((int64_t)row * a.q_heads + g * G) * D + i);
+    __syncthreads();
+    if (a.rotate_query) {
+        for (int width = 1; width < D; width <<= 1) {
+            for (int i = tid; i < G * (D / 2); i += kAttnThreads) {
+                const int h = i / (D / 2), k = i % (D / 2);
+                const int x = h * D + (k / width) * 2 * width + (k % width), y = x + width;
+                const float left = q_lds[x], right = q_lds[y];
+                q_lds[x] = left + right;
+                q_lds[y] = left - right;
+            }
+            __syncthreads();
+        }
+    }
     float q[G][8];
 #pragma unroll
     for (int h = 0; h < G; h++)
 #pragma unroll
-        for (int j = 0; j < 8; j++)
-            q[h][j] = load_query(a.query, a.query_dtype, ((int64_t)row * a.q_heads + g * G + h) * D + blk * 8 + j);
+        for (int j = 0; j < 8; j++) {
+            float v = q_lds[h * D + blk * 8 + j];
+            if (a.rotate_query) {
+                v = v * (1.0f / __builtin_sqrtf((float)D));
+                v = a.query_dtype == NQ_BF16 ? bf16_to_f32(f32_to_bf16(v))
+                                             : (a.query_dtype == NQ_F16 ? (float)(_Float16)v : v);
+            }
+            q[h][j] = v;
+        }
+    __syncthreads();                                     // q_lds aliases the score buffer
     const float sqrt_d = __builtin_sqrtf((float)D);
     const int row_in_page = token * a.kv_heads + g;
     const int64_t page_words = (int64_t)P * a.kv_heads * kBlocks, page_rows = (int64_t)P * a.kv_heads;
@@ -312,7 +339,7 @@ extern "C" int nq_nqkv_attention_decode(
     const int32_t *hot_lengths_dev, const uint8_t *cache_active_dev, const void *hot_keys_dev,
     const void *hot_values_dev, const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch,
     int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
-    void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream) {
+    int rotate_query, void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream) {
     NQ_REQUIRE(batch >= 1 && slots >= 1 && max_pages >= 1, NQ_ERR_SHAPE,
                "nq_nqkv_attention_decode: batch, slots and max_pages must be positive");
     NQ_REQUIRE(kv_heads >= 1 && q_heads >= kv_heads && q_heads % kv_heads == 0, NQ_ERR_SHAPE,
@@ -352,6 +379,7 @@ extern "C" int nq_nqkv_attention_decode(
     a.slot_ids = slot_ids_dev; a.active_mask = active_mask_dev;
     a.batch = batch; a.slots = slots; a.max_pages = max_pages; a.q_heads = q_heads; a.kv_heads = kv_heads;
     a.chunks = chunks_for(max_pages); a.query_dtype = query_dtype; a.scale = scale;
+    a.rotate_query = rotate_query;
     const size_t parts = (size_t)a.chunks + 1, heads_total = (size_t)batch * q_heads;
     a.part_max = reinterpret_cast<float *>(workspace_dev);
     a.part_sum = a.part_max + heads_total * parts;

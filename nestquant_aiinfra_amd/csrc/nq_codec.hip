@@ -76,7 +76,8 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
                      const float *__restrict__ betas, int beta_count, float sqrt_n,
                      uint32_t seed_plus_offset, uint32_t *__restrict__ codes,
                      uint8_t *__restrict__ beta_ids, float *__restrict__ norms,
-                     uint4 *__restrict__ decoded, int rows_per_wg, int slices, int vector_loads) {
+                     uint4 *__restrict__ decoded, int rows_per_wg, int slices, int vector_loads,
+                     int hadamard_stage_dtype) {
     extern __shared__ float lds[];
     float *row_scale = lds + (size_t)rows_per_wg * n;
     float *row_norm = row_scale + rows_per_wg;
@@ -110,6 +111,9 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
         }
     }
     __syncthreads();
+
+    // optional input rotation, in the arithmetic of the caller's tensor dtype
+    if (hadamard_stage_dtype >= 0) staged_hadamard(lds, rows_per_wg, n, hadamard_stage_dtype);
 
     // phase 2
     staged_row_norms(lds, rows_per_wg, n, sqrt_n, row_scale, row_norm);
@@ -185,7 +189,62 @@ dequantize_rows_kernel(const uint32_t *__restrict__ codes, const uint8_t *__rest
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Stand-alone Hadamard rotation of rows (post-RoPE queries and keys, prefill inputs).
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+hadamard_rows_kernel(const T *__restrict__ x, int64_t rows, int n, int rows_per_wg, int stage_dtype,
+                     void *__restrict__ out, int out_dtype) {
+    extern __shared__ float lds[];
+    const int64_t row0 = (int64_t)blockIdx.x * rows_per_wg;
+    const int64_t first = row0 * n, limit = rows * (int64_t)n;
+    for (int idx = threadIdx.x; idx < rows_per_wg * n; idx += blockDim.x)
+        lds[idx] = first + idx < limit ? RowLoader<T>::scalar(x, first + idx) : 0.0f;
+    __syncthreads();
+    staged_hadamard(lds, rows_per_wg, n, stage_dtype);
+    for (int idx = threadIdx.x; idx < rows_per_wg * n; idx += blockDim.x) {
+        const int64_t g = first + idx;
+        if (g >= limit) continue;
+        if (out_dtype == NQ_BF16) reinterpret_cast<uint16_t *>(out)[g] = f32_to_bf16(lds[idx]);
+        else if (out_dtype == NQ_F16) reinterpret_cast<_Float16 *>(out)[g] = (_Float16)lds[idx];
+        else reinterpret_cast<float *>(out)[g] = lds[idx];
+    }
+}
+
 }  // namespace nq
+
+extern "C" int nq_hadamard(const void *x_dev, int x_dtype, int64_t rows, int64_t n, int stage_dtype,
+                           void *out_dev, int out_dtype, void *stream) {
+    NQ_REQUIRE(rows >= 1 && n >= 2 && (n & (n - 1)) == 0 && n <= 32768, NQ_ERR_SHAPE,
+               "nq_hadamard: feature count %lld must be a power of two in [2, 32768]", (long long)n);
+    NQ_REQUIRE(x_dev && out_dev, NQ_ERR_ARGUMENT, "nq_hadamard: null pointer");
+    for (int tag : {x_dtype, stage_dtype, out_dtype})
+        NQ_REQUIRE(tag == NQ_F32 || tag == NQ_BF16 || tag == NQ_F16, NQ_ERR_ARGUMENT,
+                   "nq_hadamard: unknown dtype tag %d", tag);
+    int rows_per_wg = (int)(2048 / n);
+    if (rows_per_wg < 1) rows_per_wg = 1;
+    if (rows_per_wg > rows) rows_per_wg = (int)rows;
+    const size_t lds_bytes = (size_t)rows_per_wg * n * sizeof(float);
+    const int64_t grid = (rows + rows_per_wg - 1) / rows_per_wg;
+    NQ_REQUIRE(grid <= 0x7fffffff, NQ_ERR_SHAPE, "nq_hadamard: too many rows");
+    hipStream_t s = (hipStream_t)stream;
+#define NQ_LAUNCH_HADAMARD(T)                                                                          \
+    do {                                                                                               \
+        auto kernel = nq::hadamard_rows_kernel<T>;                                                     \
+        if (lds_bytes > 48 * 1024)                                                                     \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),                          \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);     \
+        hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), lds_bytes, s,                      \
+                           reinterpret_cast<const T *>(x_dev), rows, (int)n, rows_per_wg, stage_dtype, \
+                           out_dev, out_dtype);                                                        \
+    } while (0)
+    if (x_dtype == NQ_F32) NQ_LAUNCH_HADAMARD(float);
+    else if (x_dtype == NQ_BF16) NQ_LAUNCH_HADAMARD(uint16_t);
+    else NQ_LAUNCH_HADAMARD(nq::half_bits);
+#undef NQ_LAUNCH_HADAMARD
+    return nq::check_launch("nq_hadamard");
+}
 
 extern "C" int nq_e8_nearest(const float *x_dev, float *out_dev, int64_t count, void *stream) {
     NQ_REQUIRE(count >= 0, NQ_ERR_SHAPE, "nq_e8_nearest: count must be non-negative");
@@ -207,7 +266,7 @@ namespace {
 template <typename T, bool kDithered>
 int launch_quantize(const void *x, int64_t rows, int n, int q, const float *betas, int beta_count,
                     uint32_t seed_plus_offset, uint8_t *codes, uint8_t *beta_ids, float *norms,
-                    void *decoded, hipStream_t stream) {
+                    void *decoded, int hadamard_stage_dtype, hipStream_t stream) {
     const int pairs_per_row = n / 2;
     const int target = pairs_per_row < 256 ? 256 : (pairs_per_row < 1024 ? pairs_per_row : 1024);
     int rows_per_wg = target / pairs_per_row;
@@ -243,7 +302,7 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
                        beta_count, (float)sqrt((double)n), seed_plus_offset,
                        reinterpret_cast<uint32_t *>(codes), beta_ids, norms,
                        reinterpret_cast<uint4 *>(decoded), rows_per_wg, slices,
-                       (int)nq::aligned(x, 16));
+                       (int)nq::aligned(x, 16), hadamard_stage_dtype);
     return nq::check_launch("nq_quantize_rows");
 }
 
@@ -251,8 +310,9 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
 
 extern "C" int nq_quantize_rows(const void *x_dev, int x_dtype, int64_t rows, int64_t n, int q,
                                 const float *betas_dev, int beta_count, int has_dither, int64_t seed,
-                                int64_t block_offset, uint8_t *codes_dev, uint8_t *beta_ids_dev,
-                                float *norms_dev, void *decoded_bf16_dev, void *stream) {
+                                int64_t block_offset, int hadamard, uint8_t *codes_dev,
+                                uint8_t *beta_ids_dev, float *norms_dev, void *decoded_bf16_dev,
+                                void *stream) {
     NQ_REQUIRE(rows >= 1 && n >= 1, NQ_ERR_SHAPE, "nq_quantize_rows: rows and n must be positive");
     NQ_REQUIRE(n % 32 == 0, NQ_ERR_SHAPE,
                "nq_quantize_rows: feature count %lld must be a multiple of 32", (long long)n);
@@ -266,6 +326,11 @@ extern "C" int nq_quantize_rows(const void *x_dev, int x_dtype, int64_t rows, in
     NQ_REQUIRE(nq::aligned(codes_dev, 4), NQ_ERR_ARGUMENT, "nq_quantize_rows: codes must be 4-byte aligned");
     NQ_REQUIRE(!decoded_bf16_dev || nq::aligned(decoded_bf16_dev, 16), NQ_ERR_ARGUMENT,
                "nq_quantize_rows: decoded output must be 16-byte aligned");
+    NQ_REQUIRE(!hadamard || (n & (n - 1)) == 0, NQ_ERR_SHAPE,
+               "nq_quantize_rows: the Hadamard rotation needs a power-of-two feature count, got %lld", (long long)n);
+    NQ_REQUIRE(x_dtype == NQ_F32 || x_dtype == NQ_BF16 || x_dtype == NQ_F16, NQ_ERR_ARGUMENT,
+               "nq_quantize_rows: unknown dtype tag %d", x_dtype);
+    const int stage_dtype = hadamard ? x_dtype : -1;
     uint32_t seed_plus_offset = 0;
     if (has_dither) {
         NQ_REQUIRE(seed >= 0 && seed < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
@@ -278,9 +343,9 @@ extern "C" int nq_quantize_rows(const void *x_dev, int x_dtype, int64_t rows, in
 #define NQ_DISPATCH_QUANTIZE(T)                                                                    \
     (has_dither ? launch_quantize<T, true>(x_dev, rows, (int)n, q, betas_dev, beta_count,           \
                                            seed_plus_offset, codes_dev, beta_ids_dev, norms_dev,  \
-                                           decoded_bf16_dev, s)                                     \
+                                           decoded_bf16_dev, stage_dtype, s)                        \
                 : launch_quantize<T, false>(x_dev, rows, (int)n, q, betas_dev, beta_count, 0u,      \
-                                            codes_dev, beta_ids_dev, norms_dev, decoded_bf16_dev, s))
+                                            codes_dev, beta_ids_dev, norms_dev, decoded_bf16_dev, stage_dtype, s))
     switch (x_dtype) {
         case NQ_F32: return NQ_DISPATCH_QUANTIZE(float);
         case NQ_BF16: return NQ_DISPATCH_QUANTIZE(uint16_t);

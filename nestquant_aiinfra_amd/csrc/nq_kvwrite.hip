@@ -59,7 +59,7 @@ struct KvWriteArgs {
     float *key_norms, *value_norms;
     const float *key_betas, *value_betas;
     uint16_t *hot_keys, *hot_values;        // BF16 [slots, P, kv_heads, D]
-    int batch, tokens, uniform_count, slots, max_pages, kv_heads, key_beta_count, value_beta_count;
+    int batch, tokens, uniform_count, slots, max_pages, kv_heads, key_beta_count, value_beta_count, rotate_keys;
 };
 
 template <int D, int P>
@@ -95,39 +95,71 @@ __global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
         } else {
             if (blockIdx.x != 0 || !tail_partial || last_ordinal == first_ordinal) return;
             ordinal = last_ordinal;
-            __syncthreads();
+            __syncthreads();                 // the first page's LDS rows are done with
         }
         const int page_start = ordinal * P;
         const bool complete = page_start + P <= length;
-        if (!complete) {
-            // trailing partial page: copy the new rows of this head into the hot tail
-            const int lo = start > page_start ? start : page_start;
-            const int n_new = length - lo;
-            for (int i = tid; i < n_new * (D / 8); i += kKvThreads) {
-                const int t = lo + i / (D / 8), c = i % (D / 8);
-                const int64_t src = (((int64_t)row * a.tokens + (t - start)) * a.kv_heads + g) * D + c * 8;
-                const int64_t dst = (((int64_t)slot * P + (t - page_start)) * a.kv_heads + g) * D + c * 8;
-                *reinterpret_cast<uint4 *>(a.hot_keys + dst) = *reinterpret_cast<const uint4 *>(a.key + src);
-                *reinterpret_cast<uint4 *>(a.hot_values + dst) = *reinterpret_cast<const uint4 *>(a.value + src);
-            }
-            continue;
-        }
-        // complete page: gather P tokens (hot tail first, then new rows) as float32
+        const int page_tokens = complete ? P : length - page_start;      // tokens of this page that exist
+        const int first_new = start > page_start ? start - page_start : 0;
+        // stage the page's tokens as float32: hot tail first, then the new rows
         for (int i = tid; i < 2 * P * (D / 8); i += kKvThreads) {
             const int which = i / (P * (D / 8)), rem = i % (P * (D / 8));
             const int t = rem / (D / 8), c = rem % (D / 8);
-            const int pos = page_start + t;
+            float *dst = &rows[which * P + t][c * 8];
+            if (t >= page_tokens) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) dst[j] = 0.0f;
+                continue;
+            }
             const uint16_t *src;
-            if (pos < start)
+            if (t < first_new)
                 src = (which ? a.hot_values : a.hot_keys) + (((int64_t)slot * P + t) * a.kv_heads + g) * D + c * 8;
             else
-                src = (which ? a.value : a.key) + (((int64_t)row * a.tokens + (pos - start)) * a.kv_heads + g) * D + c * 8;
+                src = (which ? a.value : a.key) +
+                      (((int64_t)row * a.tokens + (page_start + t - start)) * a.kv_heads + g) * D + c * 8;
             const uint4 raw = *reinterpret_cast<const uint4 *>(src);
-            float *dst = &rows[which * P + t][c * 8];
             dst[0] = __uint_as_float(raw.x << 16); dst[1] = __uint_as_float(raw.x & 0xffff0000u);
             dst[2] = __uint_as_float(raw.y << 16); dst[3] = __uint_as_float(raw.y & 0xffff0000u);
             dst[4] = __uint_as_float(raw.z << 16); dst[5] = __uint_as_float(raw.z & 0xffff0000u);
             dst[6] = __uint_as_float(raw.w << 16); dst[7] = __uint_as_float(raw.w & 0xffff0000u);
+        }
+        __syncthreads();
+        if (a.rotate_keys) {
+            // new key rows arrive unrotated: float32 Hadamard over the head, then BF16, as
+            // hadamard(key.float()).to(bfloat16) (nestquant/runtime/nqkv_batched_hf_backend.py:381)
+            const int new_rows = page_tokens - first_new;
+            for (int width = 1; width < D; width <<= 1) {
+                for (int i = tid; i < new_rows * (D / 2); i += kKvThreads) {
+                    const int r = first_new + i / (D / 2), k = i % (D / 2);
+                    const int x = (k / width) * 2 * width + (k % width), y = x + width;
+                    const float left = rows[r][x], right = rows[r][y];
+                    rows[r][x] = left + right;
+                    rows[r][y] = left - right;
+                }
+                __syncthreads();
+            }
+            const float inv = 1.0f / sqrt_d;
+            for (int i = tid; i < new_rows * D; i += kKvThreads) {
+                float &v = rows[first_new + i / D][i % D];
+                v = bf16_to_f32(f32_to_bf16(v * inv));
+            }
+            __syncthreads();
+        }
+        if (!complete) {
+            // trailing partial page: the new rows of this head go to the hot tail
+            for (int i = tid; i < 2 * (page_tokens - first_new) * (D / 8); i += kKvThreads) {
+                const int which = i / ((page_tokens - first_new) * (D / 8)), rem = i % ((page_tokens - first_new) * (D / 8));
+                const int t = first_new + rem / (D / 8), c = rem % (D / 8);
+                const float *src = &rows[which * P + t][c * 8];
+                uint4 packed;
+                packed.x = f32_to_bf16(src[0]) | ((uint32_t)f32_to_bf16(src[1]) << 16);
+                packed.y = f32_to_bf16(src[2]) | ((uint32_t)f32_to_bf16(src[3]) << 16);
+                packed.z = f32_to_bf16(src[4]) | ((uint32_t)f32_to_bf16(src[5]) << 16);
+                packed.w = f32_to_bf16(src[6]) | ((uint32_t)f32_to_bf16(src[7]) << 16);
+                *reinterpret_cast<uint4 *>((which ? a.hot_values : a.hot_keys) +
+                                           (((int64_t)slot * P + t) * a.kv_heads + g) * D + c * 8) = packed;
+            }
+            continue;
         }
         __syncthreads();
         staged_row_norms(&rows[0][0], 2 * P, D, sqrt_d, row_scale, row_norm);
@@ -186,7 +218,8 @@ extern "C" int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_
                              uint8_t *value_codes_dev, uint8_t *value_beta_ids_dev, float *value_norms_dev,
                              const float *key_betas_dev, int key_beta_count, const float *value_betas_dev,
                              int value_beta_count, void *hot_keys_dev, void *hot_values_dev, int batch, int tokens,
-                             int slots, int max_pages, int kv_heads, int head_dim, int page_size, void *stream) {
+                             int slots, int max_pages, int kv_heads, int head_dim, int page_size, int rotate_keys,
+                             void *stream) {
     NQ_REQUIRE(batch >= 1 && tokens >= 1 && slots >= 1 && max_pages >= 1 && kv_heads >= 1, NQ_ERR_SHAPE,
                "nq_nqkv_write: batch, tokens, slots, max_pages and kv_heads must be positive");
     NQ_REQUIRE(head_dim == 64 && page_size == 16, NQ_ERR_SHAPE,
@@ -217,6 +250,7 @@ extern "C" int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_
     a.hot_values = reinterpret_cast<uint16_t *>(hot_values_dev);
     a.batch = batch; a.tokens = tokens; a.uniform_count = uniform_count; a.slots = slots; a.max_pages = max_pages;
     a.kv_heads = kv_heads; a.key_beta_count = key_beta_count; a.value_beta_count = value_beta_count;
+    a.rotate_keys = rotate_keys;
     // `tokens` new rows starting anywhere inside a page touch at most this many pages
     const int touched = (tokens + page_size - 2) / page_size + 1;
     hipLaunchKernelGGL((nq::kv_write_kernel<64, 16>), dim3((unsigned)touched, (unsigned)(batch * kv_heads)),

@@ -23,6 +23,35 @@ __device__ __forceinline__ uint32_t quad_xor2(uint32_t v) {
 }
 
 
+// Round a float32 to the value the given storage dtype would hold (tags as in nqhip.h:
+// 0 = float32, 1 = bfloat16, 2 = float16), keeping it as float32.
+__device__ __forceinline__ float round_to_dtype(float x, int dtype) {
+    if (dtype == 1) return bf16_to_f32(f32_to_bf16(x));
+    if (dtype == 2) return (float)(_Float16)x;
+    return x;
+}
+
+// Normalized Sylvester-Hadamard transform of rows staged in LDS (nestquant/core/rotation.py:12-27):
+// butterflies of growing width, each sum and difference rounded to `stage_dtype` (the dtype
+// the reference's tensor ops would run in), then one multiplication by float32(1 / sqrt(n))
+// -- the form a tensor / python-scalar division takes on the GPU.  Ends with a barrier.
+__device__ __forceinline__ void staged_hadamard(float *rows, int row_count, int n, int stage_dtype) {
+    const int half = n >> 1;
+    for (int width = 1; width < n; width <<= 1) {
+        for (int i = threadIdx.x; i < row_count * half; i += blockDim.x) {
+            const int r = i / half, k = i - r * half;
+            const int a = r * n + (k / width) * 2 * width + (k % width), b = a + width;
+            const float left = rows[a], right = rows[b];
+            rows[a] = round_to_dtype(left + right, stage_dtype);
+            rows[b] = round_to_dtype(left - right, stage_dtype);
+        }
+        __syncthreads();
+    }
+    const float inv = 1.0f / __builtin_sqrtf((float)n);
+    for (int i = threadIdx.x; i < row_count * n; i += blockDim.x) rows[i] = round_to_dtype(rows[i] * inv, stage_dtype);
+    __syncthreads();
+}
+
 // rows: [row_count][n] float32 in LDS, n a multiple of 32.  Writes row_scale[r] =
 // (1 / norm) * sqrt(n) (0 for a zero row) and row_norm[r]; ends with a barrier.
 __device__ __forceinline__ void staged_row_norms(const float *rows, int row_count, int n, float sqrt_n,

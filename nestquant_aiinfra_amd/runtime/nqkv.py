@@ -360,7 +360,8 @@ class BatchedNQKVAttentionWorkspace:
 
 def launch_nqkv_decode_attention(query: torch.Tensor, cache: NQKVHotColdCache, *, slot_ids: torch.Tensor,
                                  active_mask: torch.Tensor, attention_scale: float,
-                                 workspace: BatchedNQKVAttentionWorkspace) -> torch.Tensor:
+                                 workspace: BatchedNQKVAttentionWorkspace,
+                                 rotate_query: bool = False) -> torch.Tensor:
     """Graph-safe launch: no host reads, no allocation; writes workspace.output."""
     pool, meta = cache.pool, cache.metadata
     batch, heads, dim = query.shape
@@ -373,14 +374,16 @@ def launch_nqkv_decode_attention(query: torch.Tensor, cache: NQKVHotColdCache, *
         meta.hot_lengths.data_ptr(), meta.active_mask.data_ptr(),
         cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(), slot_ids.data_ptr(), active_mask.data_ptr(),
         batch, cache.max_sequences, cache.max_pages_per_sequence, heads, pool.num_kv_heads, dim, pool.page_size,
-        attention_scale, workspace.output.data_ptr(), workspace.buffer.data_ptr(), workspace.buffer.numel(),
+        attention_scale, int(rotate_query), workspace.output.data_ptr(), workspace.buffer.data_ptr(),
+        workspace.buffer.numel(),
         _native.stream_handle(query.device)))
     return workspace.output
 
 
 def nqkv_decode_attention_batched_k1(query: torch.Tensor, cache: NQKVHotColdCache, *, slot_ids: torch.Tensor,
                                      active_mask: torch.Tensor, scale: float | None = None,
-                                     workspace: BatchedNQKVAttentionWorkspace | None = None) -> torch.Tensor:
+                                     workspace: BatchedNQKVAttentionWorkspace | None = None,
+                                     rotate_query: bool = False) -> torch.Tensor:
     """Fused packed-cold plus BF16-hot decode attention for a ragged batch.
 
     query [batch, query_heads, head_dim]; slot_ids int32 [batch]; active_mask bool [batch].
@@ -413,7 +416,8 @@ def nqkv_decode_attention_batched_k1(query: torch.Tensor, cache: NQKVHotColdCach
     if not math.isfinite(attention_scale):
         raise ValueError("scale must be finite")
     return launch_nqkv_decode_attention(query.contiguous(), cache, slot_ids=slot_ids, active_mask=active_mask,
-                                        attention_scale=attention_scale, workspace=workspace)
+                                        attention_scale=attention_scale, workspace=workspace,
+                                        rotate_query=rotate_query)
 
 
 # --------------------------------------------------------------------------------------
@@ -510,8 +514,10 @@ class BatchedNQKVCacheManager:
             meta.sequence_lengths.data_ptr(), meta.page_counts.data_ptr(), meta.last_page_lens.data_ptr(),
             meta.hot_lengths.data_ptr(), _native.stream_handle(self.device)))
 
-    def write_layer(self, layer_index: int, key: torch.Tensor, value: torch.Tensor) -> None:
-        """Append this step's K/V rows [rows, tokens, kv_heads, head_dim] to one layer."""
+    def write_layer(self, layer_index: int, key: torch.Tensor, value: torch.Tensor, *,
+                    rotate_keys: bool = False) -> None:
+        """Append this step's K/V rows [rows, tokens, kv_heads, head_dim] to one layer;
+        `rotate_keys` Hadamard-rotates the new keys inside the kernel."""
         cache = self.layers[layer_index]
         pool, meta = cache.pool, self.metadata
         rows, tokens = key.shape[0], key.shape[1]
@@ -527,7 +533,7 @@ class BatchedNQKVCacheManager:
             pool.beta_table.data_ptr(), pool.beta_table.numel(), pool.value_beta_table.data_ptr(),
             pool.value_beta_table.numel(), cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(),
             rows, tokens, self.capacity, self.max_pages, pool.num_kv_heads, pool.head_dim, self.page_size,
-            _native.stream_handle(self.device)))
+            int(rotate_keys), _native.stream_handle(self.device)))
 
     def resident_bytes(self) -> int:
         total = 0

@@ -1,0 +1,354 @@
+"""Hugging Face integration of the batched NQKV4 cache: a `transformers` Cache, the
+AttentionInterface function, and a fixed-capacity runner with a captured decode step.
+
+Mirrors BatchedNQKVLlamaCache / install_batched_nqkv_llama_backend
+(nestquant/runtime/nqkv_batched_hf_backend.py:26-680) and BatchedNQKVLlamaRunner
+(nestquant/runtime/nqkv_batched_runner.py:10-378).  What differs, and why:
+  * one decode graph per batch width instead of a normal and a page-boundary graph, and no
+    host read of hot lengths before a step: the writer kernel packs a page whenever one
+    fills, from device-resident lengths;
+  * post-RoPE key and query rotations run inside the writer and attention kernels;
+  * the prefill attention output is returned as [batch, tokens, heads, dim], which is what
+    `LlamaAttention.forward` reshapes (the reference returns the raw SDPA layout).
+"""
+
+from __future__ import annotations
+
+from collections.abc import Hashable, Sequence
+
+import torch
+import torch.nn.functional as F
+from transformers.cache_utils import Cache
+from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+
+from .nqkv import BatchedNQKVAttentionWorkspace, BatchedNQKVCacheManager, launch_nqkv_decode_attention
+from .w4a4_linear import hadamard_cuda
+
+BATCHED_NQKV_ATTENTION_NAME = "nestquant_batched_nqkv_k1"
+
+
+class BatchedNQKVLlamaCache(Cache):
+    """Multi-layer fixed-capacity NQKV cache driven by scheduler slot state."""
+
+    def __init__(self, *, capacity: int, num_layers: int, num_query_heads: int, num_kv_heads: int,
+                 head_dim: int, max_cache_len: int, page_size: int, q: int, key_betas: Sequence[float],
+                 value_betas: Sequence[float], dtype: torch.dtype, device: torch.device | str) -> None:
+        super().__init__(layers=[])
+        for name, value in (("capacity", capacity), ("num_layers", num_layers),
+                            ("num_query_heads", num_query_heads), ("num_kv_heads", num_kv_heads),
+                            ("head_dim", head_dim), ("max_cache_len", max_cache_len), ("page_size", page_size)):
+            if isinstance(value, bool) or not isinstance(value, int) or value < 1:
+                raise ValueError(f"{name} must be a positive integer")
+        if num_query_heads % num_kv_heads:
+            raise ValueError("num_query_heads must be divisible by num_kv_heads")
+        self.manager = BatchedNQKVCacheManager(
+            capacity=capacity, num_layers=num_layers, num_kv_heads=num_kv_heads, head_dim=head_dim,
+            max_cache_len=max_cache_len, page_size=page_size, q=q, key_betas=key_betas,
+            value_betas=value_betas, dtype=dtype, device=device)
+        self.capacity, self.num_layers = capacity, num_layers
+        self.num_query_heads, self.num_kv_heads, self.head_dim = num_query_heads, num_kv_heads, head_dim
+        self._max_cache_len = max_cache_len
+        self.page_size, self.dtype, self.device = page_size, dtype, self.manager.device
+        self.slot_ids = torch.arange(capacity, device=self.device, dtype=torch.int32)
+        self.active_mask = torch.zeros(capacity, device=self.device, dtype=torch.bool)
+        self._rows = capacity
+        self._tokens: int | None = None
+        self._workspaces: dict[int, BatchedNQKVAttentionWorkspace] = {}
+        self._host_lengths = [0] * capacity      # host mirror of sequence lengths (admission checks)
+
+    # -- slots ---------------------------------------------------------------------------
+    def register(self, sequence_id: Hashable, *, slot: int) -> None:
+        self.manager.register(sequence_id, slot=slot)
+        self._host_lengths[slot] = 0
+
+    def register_batch(self, assignments: Sequence[tuple[Hashable, int]]) -> None:
+        for sequence_id, slot in assignments:
+            self.register(sequence_id, slot=slot)
+
+    def release_slots(self, slots: Sequence[int]) -> tuple[Hashable, ...]:
+        for slot in slots:
+            self._host_lengths[slot] = 0
+        return self.manager.release_slots(slots)
+
+    # -- step state ------------------------------------------------------------------------
+    def set_batch_state(self, *, slot_ids: Sequence[int], counts: Sequence[int]) -> None:
+        """Eager (prefill) step: row i writes its first counts[i] tokens into slot_ids[i].
+        Copies the row state to the fixed step tensors and advances the device tables."""
+        rows = len(slot_ids)
+        if rows < 1 or rows > self.capacity or len(counts) != rows:
+            raise ValueError("slot_ids and counts must describe 1..capacity rows")
+        for slot, count in zip(slot_ids, counts):
+            if self._host_lengths[slot] + count > self.manager.max_tokens:
+                raise RuntimeError("sequence would exceed max_cache_len")
+        m = self.manager
+        m.step_slot_ids[:rows].copy_(torch.tensor(list(slot_ids), dtype=torch.int32))
+        m.step_counts[:rows].copy_(torch.tensor(list(counts), dtype=torch.int32))
+        m.step_active[:rows].copy_(torch.tensor([c > 0 for c in counts]))
+        for slot, count in zip(slot_ids, counts):
+            self._host_lengths[slot] += count
+        self._rows, self._tokens = rows, max(counts)
+        m.begin_step(rows=rows, uniform_count=None)
+
+    def set_decode_execution_state(self, *, slot_ids: torch.Tensor, active_mask: torch.Tensor) -> None:
+        """Decode rows for the steps that follow (device tensors of equal length <= capacity);
+        copied into the fixed step tensors so that a captured graph sees new values."""
+        rows = slot_ids.numel()
+        if rows < 1 or rows > self.capacity or active_mask.numel() != rows:
+            raise ValueError("decode state must describe 1..capacity rows")
+        self.manager.step_slot_ids[:rows].copy_(slot_ids)
+        self.manager.step_active[:rows].copy_(active_mask)
+        self._rows, self._tokens = rows, 1
+
+    def begin_decode_step(self) -> None:
+        """Advance every active decode row by one token (graph-capturable)."""
+        self.manager.begin_step(rows=self._rows, uniform_count=1)
+
+    def note_decode_step(self, slots: Sequence[int]) -> None:
+        """Host mirror of a (possibly graph-replayed) decode step."""
+        for slot in slots:
+            self._host_lengths[slot] += 1
+
+    # -- Cache protocol -------------------------------------------------------------------------
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int, *args, **kwargs):
+        del args, kwargs
+        self._validate_layer(layer_idx)
+        if self._tokens is None:
+            raise RuntimeError("set_batch_state must run before model forward")
+        if key_states.ndim != 4 or key_states.shape != value_states.shape:
+            raise ValueError("batched NQKV update requires matching BHTD Key/Value")
+        if tuple(key_states.shape) != (self._rows, self.num_kv_heads, key_states.shape[2], self.head_dim):
+            raise ValueError("Key/Value shape disagrees with batched NQKV state")
+        if key_states.device != self.device or key_states.dtype != self.dtype:
+            raise ValueError("Key/Value must match the NQKV cache device and dtype")
+        value_rows = value_states.transpose(1, 2).contiguous()
+        if key_states.shape[2] == 1:
+            # decode: rotation fused into the writer; attention reads the cache, not the return value
+            self.manager.write_layer(layer_idx, key_states.transpose(1, 2).contiguous(), value_rows, rotate_keys=True)
+            return key_states, value_states
+        rotated_key = hadamard_cuda(key_states.contiguous(), compute_dtype=torch.float32)
+        self.manager.write_layer(layer_idx, rotated_key.transpose(1, 2).contiguous(), value_rows)
+        return rotated_key, value_states
+
+    def _workspace(self, rows: int, dtype: torch.dtype) -> BatchedNQKVAttentionWorkspace:
+        workspace = self._workspaces.get(rows)
+        if workspace is None or workspace.output.dtype != dtype:
+            workspace = BatchedNQKVAttentionWorkspace.create(
+                self.manager.layers[0], batch_size=rows, query_heads=self.num_query_heads, output_dtype=dtype)
+            self._workspaces[rows] = workspace
+        return workspace
+
+    def attend(self, layer_idx: int, query_states: torch.Tensor, *, scale: float) -> torch.Tensor:
+        self._validate_layer(layer_idx)
+        if tuple(query_states.shape) != (self._rows, self.num_query_heads, 1, self.head_dim):
+            raise ValueError("batched NQKV decode requires [rows, heads, 1, dim]")
+        query = query_states[:, :, 0].contiguous()
+        m = self.manager
+        output = launch_nqkv_decode_attention(
+            query, m.layers[layer_idx], slot_ids=m.step_slot_ids, active_mask=m.step_active,
+            attention_scale=scale, workspace=self._workspace(self._rows, query.dtype), rotate_query=True)
+        return output.unsqueeze(1)                        # [rows, 1, heads, dim]
+
+    def prefill(self, query_states: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor,
+                attention_mask: torch.Tensor | None, *, scale: float) -> torch.Tensor:
+        """Prefill attends to the current BF16 K/V (keys already rotated by `update`)."""
+        rotated_query = hadamard_cuda(query_states.contiguous(), compute_dtype=torch.float32)
+        output = F.scaled_dot_product_attention(
+            rotated_query, key_states, value_states, attn_mask=attention_mask, dropout_p=0.0,
+            is_causal=attention_mask is None, scale=scale,
+            enable_gqa=self.num_query_heads != self.num_kv_heads)
+        return output.transpose(1, 2).contiguous()         # [rows, tokens, heads, dim]
+
+    def get_seq_length(self, layer_idx: int = 0) -> int:
+        self._validate_layer(layer_idx)
+        return max(self._host_lengths, default=0)
+
+    def get_max_length(self, layer_idx: int | None = None) -> int:
+        if layer_idx is not None:
+            self._validate_layer(layer_idx)
+        return self._max_cache_len
+
+    get_max_cache_shape = get_max_length
+
+    @property
+    def max_cache_len(self) -> int:
+        return self._max_cache_len
+
+    def get_mask_sizes(self, query_length, layer_idx: int) -> tuple[int, int]:
+        self._validate_layer(layer_idx)
+        length = query_length if isinstance(query_length, int) else int(query_length.shape[0])
+        return self.get_seq_length(layer_idx) + length, 0
+
+    @property
+    def batch_size(self) -> int:
+        return self.capacity
+
+    @property
+    def is_compileable(self) -> bool:
+        return False
+
+    def reorder_cache(self, beam_idx: torch.LongTensor) -> None:
+        del beam_idx
+        raise NotImplementedError("batched NQKV backend does not support beam search")
+
+    def _validate_layer(self, layer_idx: int) -> None:
+        if isinstance(layer_idx, bool) or not isinstance(layer_idx, int):
+            raise TypeError("layer_idx must be an integer")
+        if not 0 <= layer_idx < self.num_layers:
+            raise ValueError("layer_idx is outside the batched NQKV layer range")
+
+
+def _batched_nqkv_attention_interface(module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                                      attention_mask: torch.Tensor | None, **kwargs):
+    cache = getattr(module, "_nestquant_batched_nqkv_cache", None)
+    if not isinstance(cache, BatchedNQKVLlamaCache):
+        raise RuntimeError("Llama attention module has no batched NQKV cache")
+    if kwargs.get("dropout", 0.0) != 0.0:
+        raise ValueError("batched NQKV backend supports inference dropout=0 only")
+    scale = float(kwargs.get("scaling", module.scaling))
+    if query.shape[2] == 1:
+        return cache.attend(module.layer_idx, query, scale=scale), None
+    return cache.prefill(query, key, value, attention_mask, scale=scale), None
+
+
+def install_batched_nqkv_llama_backend(model: torch.nn.Module, cache: BatchedNQKVLlamaCache) -> str:
+    """Attach fixed-capacity batched NQKV attention to every Llama layer."""
+    if not isinstance(model, torch.nn.Module):
+        raise TypeError("model must be a torch module")
+    if not isinstance(cache, BatchedNQKVLlamaCache):
+        raise TypeError("cache must be a BatchedNQKVLlamaCache")
+    ALL_ATTENTION_FUNCTIONS.register(BATCHED_NQKV_ATTENTION_NAME, _batched_nqkv_attention_interface)
+    attached = 0
+    for module in model.modules():
+        if module.__class__.__name__ == "LlamaAttention":
+            if not 0 <= module.layer_idx < cache.num_layers:
+                raise ValueError("Llama layer index disagrees with batched NQKV cache")
+            module._nestquant_batched_nqkv_cache = cache
+            module.config._attn_implementation = BATCHED_NQKV_ATTENTION_NAME
+            attached += 1
+    if attached != cache.num_layers:
+        raise ValueError(f"expected {cache.num_layers} LlamaAttention modules, found {attached}")
+    if hasattr(model, "config"):
+        model.config._attn_implementation = BATCHED_NQKV_ATTENTION_NAME
+    return BATCHED_NQKV_ATTENTION_NAME
+
+
+class BatchedNQKVLlamaRunner:
+    """Fixed-capacity prefill / decode driver over a causal Llama model and an NQKV cache.
+
+    Decode steps of width w in {1, 2, 4, ..., capacity} are captured once as HIP graphs
+    (`capture`); active rows are compacted to the smallest width that holds them.  A step
+    reads nothing from the device: token ids, positions, slot ids and masks are copied into
+    the graph's fixed input tensors, the graph is replayed, logits are returned.
+    """
+
+    def __init__(self, model: torch.nn.Module, cache: BatchedNQKVLlamaCache) -> None:
+        if not isinstance(model, torch.nn.Module):
+            raise TypeError("model must be a torch module")
+        if not isinstance(cache, BatchedNQKVLlamaCache):
+            raise TypeError("cache must be a BatchedNQKVLlamaCache")
+        if model.training:
+            raise ValueError("model must be in eval mode")
+        device = next(model.parameters()).device
+        if device.type != "cuda" or device != cache.device:
+            raise ValueError("model and NQKV cache must share one CUDA device")
+        self.model, self.cache, self.device = model, cache, device
+        self.batch_size, self.max_cache_len = cache.capacity, cache.max_cache_len
+        self._generation = [0] * self.batch_size
+        self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor, torch.Tensor]] = {}
+        self.graph_replay_counts: dict[int, int] = {}
+
+    @property
+    def graph_captured(self) -> bool:
+        return bool(self._graphs)
+
+    # -- prefill -------------------------------------------------------------------------------
+    @torch.inference_mode()
+    def prefill_slots(self, input_ids: torch.Tensor, *, slots: Sequence[int], lengths: Sequence[int],
+                      positions: torch.Tensor | None = None) -> torch.Tensor:
+        """Prefill `slots[i]` with the first `lengths[i]` tokens of row i of input_ids
+        [rows, width] (right padded).  New slots are registered.  Returns logits [rows, width, vocab]."""
+        rows, width = input_ids.shape
+        if len(slots) != rows or len(lengths) != rows:
+            raise ValueError("slots and lengths must have one entry per row")
+        for slot in slots:
+            if self.cache.manager.sequence_id(slot) is None:
+                self._generation[slot] += 1
+                self.cache.register(f"slot-{slot}-generation-{self._generation[slot]}", slot=slot)
+        if positions is None:
+            starts = torch.tensor([self.cache._host_lengths[s] for s in slots], device=self.device)
+            positions = starts[:, None] + torch.arange(width, device=self.device)[None, :]
+        self.cache.set_batch_state(slot_ids=slots, counts=lengths)
+        output = self.model(input_ids=input_ids, position_ids=positions, past_key_values=self.cache, use_cache=True)
+        return output.logits
+
+    def release_slots(self, slots: Sequence[int]) -> None:
+        self.cache.release_slots(slots)
+
+    # -- decode --------------------------------------------------------------------------------
+    def _step(self, tokens: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        self.cache.begin_decode_step()
+        return self.model(input_ids=tokens, position_ids=positions, past_key_values=self.cache,
+                          use_cache=True).logits
+
+    @torch.inference_mode()
+    def decode_eager(self, tokens: torch.Tensor, *, slots: Sequence[int], positions: torch.Tensor) -> torch.Tensor:
+        """One un-captured decode step for `slots` (tokens, positions: [rows, 1])."""
+        rows = len(slots)
+        self.cache.set_decode_execution_state(
+            slot_ids=torch.tensor(list(slots), dtype=torch.int32, device=self.device),
+            active_mask=torch.ones(rows, dtype=torch.bool, device=self.device))
+        logits = self._step(tokens, positions)
+        self.cache.note_decode_step(slots)
+        return logits
+
+    @torch.inference_mode()
+    def capture(self, widths: Sequence[int] | None = None) -> None:
+        """Capture one decode graph per batch width.  Captured on slots that hold at least one
+        token; the tables are restored afterwards, so capture leaves the cache unchanged."""
+        if widths is None:
+            widths, width = [], 1
+            while width < self.batch_size:
+                widths.append(width)
+                width *= 2
+            widths.append(self.batch_size)
+        meta = self.cache.manager.metadata
+        saved = [t.clone() for t in (meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths)]
+        stream = torch.cuda.Stream(device=self.device)
+        for width in widths:
+            tokens = torch.zeros((width, 1), dtype=torch.long, device=self.device)
+            positions = torch.zeros((width, 1), dtype=torch.long, device=self.device)
+            self.cache.set_decode_execution_state(
+                slot_ids=torch.arange(width, dtype=torch.int32, device=self.device),
+                active_mask=torch.zeros(width, dtype=torch.bool, device=self.device))   # inactive: writes nothing
+            stream.wait_stream(torch.cuda.current_stream(self.device))
+            with torch.cuda.stream(stream):
+                for _ in range(2):
+                    self._step(tokens, positions)
+                stream.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=stream):
+                    logits = self._step(tokens, positions)
+            torch.cuda.current_stream(self.device).wait_stream(stream)
+            self._graphs[width] = (graph, tokens, positions, logits)
+            self.graph_replay_counts[width] = 0
+        for tensor, value in zip((meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths), saved):
+            tensor.copy_(value)
+
+    @torch.inference_mode()
+    def decode(self, tokens: torch.Tensor, *, slots: Sequence[int], positions: torch.Tensor) -> torch.Tensor:
+        """One captured decode step: tokens / positions [rows, 1] for `slots`; logits [rows, 1, vocab]."""
+        rows = len(slots)
+        width = next((w for w in sorted(self._graphs) if w >= rows), None)
+        if width is None:
+            return self.decode_eager(tokens, slots=slots, positions=positions)
+        graph, graph_tokens, graph_positions, logits = self._graphs[width]
+        graph_tokens[:rows].copy_(tokens)
+        graph_positions[:rows].copy_(positions)
+        padded_slots = list(slots) + [0] * (width - rows)
+        self.cache.set_decode_execution_state(
+            slot_ids=torch.tensor(padded_slots, dtype=torch.int32, device=self.device),
+            active_mask=torch.tensor([True] * rows + [False] * (width - rows), device=self.device))
+        graph.replay()
+        self.graph_replay_counts[width] += 1
+        self.cache.note_decode_step(slots)
+        return logits[:rows]

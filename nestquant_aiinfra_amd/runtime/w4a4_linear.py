@@ -85,7 +85,7 @@ def _beta_values(betas: Sequence[float]) -> tuple[float, ...]:
 
 def quantize_rows_packed(rows: torch.Tensor, *, q: int, beta_table: torch.Tensor,
                          dither_seed: int | None = None, block_offset: int = 0,
-                         decoded: torch.Tensor | None = None
+                         decoded: torch.Tensor | None = None, hadamard: bool = False
                          ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Encode ``rows`` [R, n] (float32 / bfloat16 / float16, on the GPU) into packed 4-bit
     codes, packed 2-bit beta ids and float32 row norms with one kernel launch.  ``decoded``
@@ -100,14 +100,35 @@ def quantize_rows_packed(rows: torch.Tensor, *, q: int, beta_table: torch.Tensor
     _native.check(_native.library().nq_quantize_rows(
         rows.data_ptr(), _native.dtype_tag(rows.dtype), count, n, q, beta_table.data_ptr(),
         beta_table.numel(), int(dither_seed is not None), int(dither_seed or 0), block_offset,
-        codes.data_ptr(), beta_ids.data_ptr(), norms.data_ptr(),
+        int(hadamard), codes.data_ptr(), beta_ids.data_ptr(), norms.data_ptr(),
         None if decoded is None else decoded.data_ptr(), _native.stream_handle(device)))
     return codes, beta_ids, norms
 
 
+def hadamard_cuda(inputs: torch.Tensor, *, compute_dtype: torch.dtype | None = None,
+                  output_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """Normalized Hadamard transform along the last axis in one kernel.  `compute_dtype` is the
+    dtype whose arithmetic the butterflies follow (default: the input's; float32 = no
+    intermediate rounding); `output_dtype` defaults to the input's."""
+    if not isinstance(inputs, torch.Tensor) or not inputs.is_floating_point() or inputs.ndim == 0:
+        raise ValueError("expected a floating-point tensor with a feature axis")
+    device = _native.require_cuda(inputs)
+    n = inputs.shape[-1]
+    out = torch.empty(inputs.shape, dtype=output_dtype or inputs.dtype, device=device)
+    _native.check(_native.library().nq_hadamard(
+        inputs.data_ptr(), _native.dtype_tag(inputs.dtype), inputs.numel() // n, n,
+        _native.dtype_tag(compute_dtype or inputs.dtype), out.data_ptr(), _native.dtype_tag(out.dtype),
+        _native.stream_handle(device)))
+    return out
+
+
 def quantize_activation_cuda(inputs: torch.Tensor, *, q: int, betas: Sequence[float],
-                             beta_table: torch.Tensor | None = None) -> PreparedNQA4Activation:
+                             beta_table: torch.Tensor | None = None,
+                             hadamard: bool = False) -> PreparedNQA4Activation:
     """Encode floating activations into packed NQA4 payloads on the GPU.
+
+    `hadamard=True` (an extension) rotates the rows inside the same kernel, equivalent to
+    encoding ``hadamard(inputs)``.
 
     BF16 / FP16 inputs are promoted to float32 inside the kernel (the reference promotes
     with ``.float()`` first, triton_w4a4_linear.py:599); results are identical.
@@ -132,7 +153,8 @@ def quantize_activation_cuda(inputs: torch.Tensor, *, q: int, betas: Sequence[fl
     if beta_table is None:
         beta_table = torch.tensor(beta_values, device=inputs.device, dtype=torch.float32)
     decoded = torch.empty(rows.shape, dtype=torch.bfloat16, device=rows.device) if q == 14 else None
-    codes, beta_ids, norms = quantize_rows_packed(rows, q=q, beta_table=beta_table, decoded=decoded)
+    codes, beta_ids, norms = quantize_rows_packed(rows, q=q, beta_table=beta_table, decoded=decoded,
+                                                  hadamard=hadamard)
     return PreparedNQA4Activation(
         code_payload=codes, beta_payload=beta_ids, row_norms=norms, beta_table=beta_table,
         original_shape=tuple(inputs.shape), q=q, code_width=code_width, beta_width=beta_width,

@@ -34,7 +34,7 @@ def test_host_side_validation_needs_no_gpu():
     """Shape checks run before anything is launched and name the offending argument."""
     from nestquant_aiinfra_amd import _native
     lib = _native.library()
-    status = lib.nq_quantize_rows(None, 0, 1, 40, 14, None, 4, 0, 0, 0, None, None, None, None, None)
+    status = lib.nq_quantize_rows(None, 0, 1, 40, 14, None, 4, 0, 0, 0, 0, None, None, None, None, None)
     assert status == _native.NQ_ERR_SHAPE and b"multiple of 32" in lib.nq_last_error()
     with pytest.raises(ValueError, match="multiple of 32"):
         _native.check(status)
