@@ -50,6 +50,11 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--steps", type=int, default=200)
     parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--skip-cpu-baseline", action="store_true")
+    parser.add_argument("--profile-copy", action="store_true",
+                        help="also run three 256 MiB device-to-device copies (a kernel of known traffic, "
+                             "to calibrate FETCH_SIZE / WRITE_SIZE counters under rocprofv3)")
+    parser.add_argument("--skip-extras", action="store_true",
+                        help="only the headline GEMV workload (no prefill GEMM, attention, TPOT)")
     return parser.parse_args()
 
 
@@ -188,6 +193,158 @@ def cpu_baseline(cases, budget_s: float = 20.0):
     }
 
 
+def time_graph(fn, launches: int, repeats: int = 5) -> float:
+    """Seconds per call of `fn`, from events around replays of a graph holding `launches` calls."""
+    import torch
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        fn(0)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            keep = [fn(i) for i in range(launches)]
+        graph.replay()
+        stream.synchronize()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record(stream)
+        for _ in range(repeats):
+            graph.replay()
+        end.record(stream)
+        end.synchronize()
+    del keep
+    return begin.elapsed_time(end) * 1e-3 / (repeats * launches)
+
+
+def prefill_gemm_extra(rt, device):
+    """W4A4 prefill linear (MFMA) at gate/up and down shapes, ragged M, outlier-channel inputs."""
+    import numpy as np
+    import torch
+    results = {}
+    for name, k, n, wseed, dseed in (("gate_proj", 2048, 8192, 1003, 20261103), ("down_proj", 8192, 2048, 1004, 20261104)):
+        g = torch.Generator().manual_seed(wseed)
+        w = hadamard_gpu((0.02 * torch.randn(n, k, generator=g)).to(device))
+        record = rt.quantize_weight_nqrt4(w, q=Q, betas=WEIGHT_BETAS, dither_seed=dseed, tensor_name=name)
+        base = rt.prepare_fused_linear(record, device=device)
+        copies = 32
+        weights = [base] + [rt.PreparedNQRTLinear(record, base.code_payload.clone(), base.beta_payload.clone(),
+                                                  base.row_norms, base.beta_table) for _ in range(copies - 1)]
+        table = torch.tensor(ACTIVATION_BETAS, dtype=torch.float32, device=device)
+        for m in (16, 40, 64, 128, 384):
+            rng = np.random.default_rng(3001)
+            x = rng.standard_normal((m, k)).astype(np.float32)
+            x[:, rng.choice(k, size=k // 100, replace=False)] *= 20.0
+            x = torch.from_numpy(x).to(device).to(torch.bfloat16)
+            activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS, beta_table=table, hadamard=True)
+            seconds = time_graph(lambda i: rt.linear_packed_w4a4_mma_chunked_staged(activation, weights[i % copies]), copies)
+            encode = time_graph(lambda i: rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS, beta_table=table,
+                                                                      hadamard=True), 16)
+            flops = 2.0 * m * k * n
+            results[f"{name}_m{m}"] = {"us": seconds * 1e6, "TFLOPs": flops / seconds / 1e12,
+                                       "mfma_frac": flops / seconds / 2.5e15, "encode_us": encode * 1e6}
+    return results
+
+
+def attention_extra(device):
+    """Paged NQKV4 decode attention: 32 / 8 heads, D 64, batch 8, contexts uniform in [128, 4096]."""
+    import torch
+    from nestquant_aiinfra_amd.runtime import nqkv
+    key_betas = tuple(v / 14 for v in (3.50, 4.58, 6.47, 17.06))
+    value_betas = tuple(v / 14 for v in (3.53, 5.59, 9.62, 29.03))
+    g = torch.Generator().manual_seed(4001)
+    lengths = torch.randint(128, 4097, (8,), generator=g).tolist()
+    manager = nqkv.BatchedNQKVCacheManager(capacity=8, num_layers=4, num_kv_heads=8, head_dim=64, max_cache_len=4096,
+                                           page_size=16, q=Q, key_betas=key_betas, value_betas=value_betas,
+                                           dtype=torch.bfloat16, device=device)
+    width = max(lengths)
+    for slot in range(8):
+        manager.register(slot, slot=slot)
+    manager.step_counts.copy_(torch.tensor(lengths, dtype=torch.int32))
+    manager.step_active.fill_(True)
+    manager.begin_step(rows=8, uniform_count=None)
+    for layer in range(4):                       # distinct layers = distinct (cold) pages per launch
+        key = hadamard_gpu(torch.randn(8, width, 8, 64, generator=g).to(device)).to(torch.bfloat16)
+        value = torch.randn(8, width, 8, 64, generator=g).to(device).to(torch.bfloat16)
+        manager.write_layer(layer, key, value)
+    query = hadamard_gpu(torch.randn(8, 32, 64, generator=g).to(device)).to(torch.bfloat16)
+    slot_ids = torch.arange(8, dtype=torch.int32, device=device)
+    active = torch.ones(8, dtype=torch.bool, device=device)
+    workspace = nqkv.BatchedNQKVAttentionWorkspace.create(manager.layers[0], batch_size=8, query_heads=32,
+                                                          output_dtype=torch.bfloat16)
+    seconds = time_graph(lambda i: nqkv.launch_nqkv_decode_attention(
+        query, manager.layers[i % 4], slot_ids=slot_ids, active_mask=active, attention_scale=0.125,
+        workspace=workspace).clone(), 8)
+    bytes_moved = sum(608 * 16 * (n // 16) + (n % 16) * 8 * 64 * 2 * 2 + 2 * 32 * 64 * 2 for n in lengths)
+    step_key = torch.randn(8, 1, 8, 64, device=device).to(torch.bfloat16)
+    manager.step_active.fill_(False)             # time the writer's launch without growing the cache
+    write = time_graph(lambda i: manager.write_layer(i % 4, step_key, step_key, rotate_keys=True), 8)
+    return {"contexts": lengths, "us": seconds * 1e6, "algorithmic_bytes": bytes_moved,
+            "GBps": bytes_moved / seconds / 1e9, "hbm_frac": bytes_moved / seconds / 1e9 / HBM_PEAK_GBPS,
+            "append_launch_us": write * 1e6}
+
+
+def tpot_extra(device, batches=(1, 8), prompt=128, generate=128):
+    """Random-init Llama-3.2-1B architecture, all 112 projections W4A4, KV4 cache, captured decode
+    step.  Per batch size: mean decode-step wall time (host argmax included) and GPU graph time."""
+    import tempfile
+
+    import torch
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
+
+    torch.manual_seed(5001)
+    config = LlamaConfig(hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, num_attention_heads=32,
+                         num_key_value_heads=8, head_dim=64, vocab_size=128256, max_position_embeddings=4096,
+                         rope_theta=500000.0, tie_word_embeddings=True)
+    with torch.device(device):
+        model = LlamaForCausalLM(config).to(torch.bfloat16).eval()
+    results = {}
+    with tempfile.TemporaryDirectory() as folder:
+        path = os.path.join(folder, "llama1b_random.nqmc")
+        asm.write_w4_checkpoint(model, path)
+        packed_bytes = os.path.getsize(path)
+        runner = asm.build_w4a4kv4_runner(model, path, capacity=max(batches), max_cache_len=prompt + generate + 16,
+                                          enable_m1_down_splitk=False)
+        g = torch.Generator().manual_seed(5002)
+        for batch in batches:
+            slots = list(range(batch))
+            ids = torch.randint(0, config.vocab_size, (batch, prompt), generator=g).to(device)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            logits = runner.prefill_slots(ids, slots=slots, lengths=[prompt] * batch)
+            token = logits[:, -1].argmax(-1).reshape(batch, 1)
+            torch.cuda.synchronize()
+            prefill_s = time.perf_counter() - t0
+            if not runner.graph_captured:
+                runner.capture()
+            position = torch.full((batch, 1), prompt, dtype=torch.long, device=device)
+            step_times = []
+            for _ in range(generate):
+                t0 = time.perf_counter()
+                out = runner.decode(token, slots=slots, positions=position)
+                token = out[:, 0].argmax(-1).reshape(batch, 1)
+                token.tolist()                                   # host sampler read, as the reference's engine does
+                step_times.append(time.perf_counter() - t0)
+                position = position + 1
+            width = next(w for w in sorted(runner._graphs) if w >= batch)
+            graph = runner._graphs[width][0]
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            runner.cache.manager.step_active.fill_(False)        # replay without growing the cache
+            begin.record()
+            for _ in range(20):
+                graph.replay()
+            end.record()
+            end.synchronize()
+            runner.release_slots(slots)
+            steps = sorted(step_times[1:])
+            results[f"batch{batch}"] = {
+                "tpot_ms_mean": 1e3 * sum(steps) / len(steps), "tpot_ms_p50": 1e3 * steps[len(steps) // 2],
+                "tpot_ms_p95": 1e3 * steps[int(0.95 * len(steps))], "graph_replay_ms": begin.elapsed_time(end) / 20,
+                "prefill_ms": prefill_s * 1e3, "tokens_per_s": batch / (sum(steps) / len(steps)),
+            }
+        results["checkpoint_bytes"] = packed_bytes
+    return results
+
+
 def main() -> None:
     args = parse_args()
     if args.gpus != 1:
@@ -202,6 +359,14 @@ def main() -> None:
         sys.exit("bench.py: no GPU visible")
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+
+    if args.profile_copy:
+        source = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=device).fill_(1)
+        target = torch.empty_like(source)
+        for _ in range(3):
+            target.copy_(source)                 # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del source, target
 
     cases, copies = build_workload(device)
     graphs, keep, stream = capture_steps(rt, cases, copies)
@@ -246,6 +411,14 @@ def main() -> None:
         "cpu_baseline": None if args.skip_cpu_baseline else cpu_baseline(cases),
         "extra": {"linear_kernel_alone": per_case},
     }
+    if not args.skip_extras:
+        del graphs, keep
+        for case in cases:
+            case["weights"] = case["weights"][:1]
+        torch.cuda.empty_cache()
+        result["extra"]["prefill_gemm"] = prefill_gemm_extra(rt, device)
+        result["extra"]["nqkv_attention"] = attention_extra(device)
+        result["extra"]["llama_1b_w4a4kv4"] = tpot_extra(device)
     print(json.dumps(result))
 
 

@@ -230,6 +230,13 @@ def nqkv_page_payload(key, value, *, page_size: int, q: int, key_betas, value_be
     return result
 
 
+def count_div14_mismatches() -> int:
+    """Exhaustive float32 check of the kernels' fused three-operation division by 14."""
+    fn = lib().nqo_count_div14_mismatches
+    fn.restype = ctypes.c_longlong
+    return int(fn())
+
+
 def num_threads() -> int:
     return int(lib().nqo_num_threads())
 

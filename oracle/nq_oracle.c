@@ -408,6 +408,34 @@ NQO_EXPORT void nqo_attention_dense(const float *query, const float *k, const fl
     }
 }
 
+/* ------------------------------------------------------------------ */
+/* Exhaustive check of the GPU kernels' three-operation division by 14 */
+/* ------------------------------------------------------------------ */
+
+/* For every finite float32 p with 1e-30 <= |p| <= 1e30 (and +-0) compares
+ *   q0 = p * c;  r = fma(-14, q0, p);  q1 = fma(r, c, q0),  c = float(1/14)
+ * with the IEEE quotient p / 14.  Returns the number of inputs whose results
+ * differ as numbers (a differing sign of zero is not counted). */
+NQO_EXPORT long long nqo_count_div14_mismatches(void) {
+    const float c = 1.0f / 14.0f;
+    long long bad = 0;
+#pragma omp parallel for reduction(+ : bad) schedule(static)
+    for (long long b = 0; b < (1LL << 32); b++) {
+        uint32_t bits = (uint32_t)b;
+        float p;
+        memcpy(&p, &bits, 4);
+        if (!isfinite(p)) continue;
+        float ap = fabsf(p);
+        if (ap != 0.0f && (ap < 1e-30f || ap > 1e30f)) continue;
+        float q0 = p * c;
+        float r = fmaf(-14.0f, q0, p);
+        float q1 = fmaf(r, c, q0);
+        float t = p / 14.0f;
+        if (q1 != t) bad++;
+    }
+    return bad;
+}
+
 NQO_EXPORT int nqo_num_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

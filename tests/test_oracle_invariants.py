@@ -215,3 +215,9 @@ def test_attention_dense_matches_numpy_softmax(oracle):
         s = (k[:, g] @ q[h]) / 8.0
         p = np.exp(s - s.max()); p /= p.sum()
         assert np.allclose(out[h], p @ v[:, g], atol=1e-5)
+
+
+def test_three_operation_division_by_14_is_ieee_exact(oracle):
+    """The HIP kernels divide by 14 with q0 = p*c, r = fma(-14, q0, p), q = fma(r, c, q0);
+    checked against IEEE division for every finite float32 in [1e-30, 1e30]."""
+    assert oracle.count_div14_mismatches() == 0
