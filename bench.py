@@ -86,7 +86,8 @@ def build_workload(device):
         base = rt.prepare_fused_linear(record, device=device)
         weights = [base] + [
             rt.PreparedNQRTLinear(record, base.code_payload.clone(), base.beta_payload.clone(),
-                                  base.row_norms.clone(), base.beta_table.clone())
+                                  base.row_norms.clone(), base.beta_table.clone(),
+                                  None if base.decode_hints is None else base.decode_hints.clone())
             for _ in range(copies - 1)
         ]
         for m in TOKEN_COUNTS:
@@ -227,7 +228,9 @@ def prefill_gemm_extra(rt, device):
         base = rt.prepare_fused_linear(record, device=device)
         copies = 32
         weights = [base] + [rt.PreparedNQRTLinear(record, base.code_payload.clone(), base.beta_payload.clone(),
-                                                  base.row_norms, base.beta_table) for _ in range(copies - 1)]
+                                                  base.row_norms, base.beta_table,
+                                                  None if base.decode_hints is None else base.decode_hints.clone())
+                            for _ in range(copies - 1)]
         table = torch.tensor(ACTIVATION_BETAS, dtype=torch.float32, device=device)
         for m in (16, 40, 64, 128, 384):
             rng = np.random.default_rng(3001)

@@ -108,6 +108,20 @@ int nq_dequantize_rows(const uint8_t *codes_dev, const uint8_t *beta_ids_dev,
                        void *out_dev, int out_dtype, void *stream);
 
 /*
+ * Decode hints for one NQRT4 weight [rows, K]: for every 8-weight block, the outcomes of the
+ * two exact E8 searches its decode performs (which coset won, which coordinate was moved and
+ * in which direction; 6 bits each, packed in a uint16).  They depend only on the stored code
+ * words, the seed and the block index, so they are computed once when a weight is prepared;
+ * the linear kernels then rebuild the same lattice points without searching (bit-identical
+ * results, about half the vector instructions per block).  hints_dev: uint16[rows * K / 8].
+ * No counterpart in the reference (its kernels repeat both searches on every call,
+ * nestquant/runtime/nqrt4_cooperative_device.cuh:150-171).
+ */
+int nq_w4a4_make_decode_hints(const uint8_t *w_codes_dev, int64_t rows, int64_t k,
+                              int64_t weight_offset, int64_t weight_seed, uint16_t *hints_dev,
+                              void *stream);
+
+/*
  * Packed W4A4 linear for decode, M = 1..8 tokens: y[m, n] = sum_k bf16(a[m, k]) * bf16(w[n, k]),
  * FP32 accumulation; the weight is decoded in registers from its packed stream (dither
  * regenerated; counter = weight_offset * 8 + n * K + k).
@@ -116,6 +130,7 @@ int nq_dequantize_rows(const uint8_t *codes_dev, const uint8_t *beta_ids_dev,
  *                    when NULL the packed streams are decoded once into the workspace,
  *                    when given the packed streams may be NULL
  *   w_*              NQRT4 streams of [N, K] (codes N*K/2 B, beta ids N*K/32 B, norms f32[N], betas f32[4])
+ *   w_hints_dev      optional uint16[N * K / 8] from nq_w4a4_make_decode_hints (NULL: search)
  *   out_dev          [M, N] of out_dtype (NQ_F32 or NQ_BF16)
  *   split_k          1, 2, 4 or 8 slices of K reduced in ascending order (deterministic); 0 lets
  *                    the library choose
@@ -129,7 +144,7 @@ int nq_dequantize_rows(const uint8_t *codes_dev, const uint8_t *beta_ids_dev,
 int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
                  const float *act_norms_dev, const float *act_betas_dev,
                  const void *act_decoded_dev, const uint8_t *w_codes_dev,
-                 const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
+                 const uint16_t *w_hints_dev, const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
                  const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
                  int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
                  void *workspace_dev, size_t workspace_bytes, void *stream);
@@ -151,7 +166,7 @@ size_t nq_w4a4_gemv_workspace_bytes(int m, int k, int n, int split_k, int have_d
 int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
                  const float *act_norms_dev, const float *act_betas_dev,
                  const void *act_decoded_dev, const uint8_t *w_codes_dev,
-                 const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
+                 const uint16_t *w_hints_dev, const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
                  const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
                  int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
                  void *workspace_dev, size_t workspace_bytes, void *stream);

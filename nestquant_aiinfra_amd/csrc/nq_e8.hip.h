@@ -37,7 +37,12 @@ __device__ __forceinline__ bool is_odd(float sum) { return __builtin_amdgcn_frac
 // moved coordinate contributes (|residual| - 1)^2 = (max - 1)^2, one value per block.
 // Half coset: the reference measures x - (D8(x - 1/2) + 1/2), recomputed from x because
 // x - 1/2 may round; the same is done here.
-__device__ __forceinline__ void e8_nearest(const float (&x)[8], float (&out)[8]) {
+//
+// `hint` (optional) receives six bits that let e8_nearest_hinted() rebuild the same point
+// without searching: bit 0 = the integer coset won, bit 1 = a coordinate was moved,
+// bits 2..4 = which one, bit 5 = it moved down (-1).
+template <bool kWantHint>
+__device__ __forceinline__ void e8_nearest_impl(const float (&x)[8], float (&out)[8], uint32_t *hint) {
     float a[8], ea[8], sum_a = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
@@ -50,6 +55,7 @@ __device__ __forceinline__ void e8_nearest(const float (&x)[8], float (&out)[8])
     const float alt_a = moved_a * moved_a;
     bool done_a = !is_odd(sum_a);                  // an even sum needs no correction
     float dist_a = 0.0f;
+    uint32_t hint_a = 0u;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const bool top = fabsf(ea[j]) == max_a;
@@ -59,6 +65,7 @@ __device__ __forceinline__ void e8_nearest(const float (&x)[8], float (&out)[8])
         dist_a = dist_a + (hit ? alt_a : sq);
         // residual >= 0 moves up (a residual is never -0)
         a[j] = hit ? a[j] + __builtin_copysignf(1.0f, ea[j]) : a[j];
+        if (kWantHint) hint_a = hit ? (2u | ((uint32_t)j << 2) | (ea[j] < 0.0f ? 32u : 0u)) : hint_a;
     }
 
     float b[8], eb[8], sum_b = 0.0f;
@@ -72,6 +79,7 @@ __device__ __forceinline__ void e8_nearest(const float (&x)[8], float (&out)[8])
     const float max_b = max_abs8(eb);
     bool done_b = !is_odd(sum_b);
     float dist_b = 0.0f;
+    uint32_t hint_b = 0u;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const bool top = fabsf(eb[j]) == max_b;
@@ -81,10 +89,32 @@ __device__ __forceinline__ void e8_nearest(const float (&x)[8], float (&out)[8])
         b[j] = hit ? half_point + __builtin_copysignf(1.0f, eb[j]) : half_point;
         const float t = x[j] - b[j];
         dist_b = dist_b + t * t;
+        if (kWantHint) hint_b = hit ? (2u | ((uint32_t)j << 2) | (eb[j] < 0.0f ? 32u : 0u)) : hint_b;
     }
     const bool pick_a = dist_a < dist_b;           // ties go to the half-integer coset
 #pragma unroll
     for (int j = 0; j < 8; j++) out[j] = pick_a ? a[j] : b[j];
+    if (kWantHint) *hint = pick_a ? (hint_a | 1u) : hint_b;
+}
+
+__device__ __forceinline__ void e8_nearest(const float (&x)[8], float (&out)[8]) {
+    e8_nearest_impl<false>(x, out, nullptr);
+}
+
+// The point e8_nearest() returns for x, rebuilt from the six hint bits it emitted for the
+// same x: round in the chosen coset, move the recorded coordinate.  Same float operations
+// as the search performs on the winning coset, so the result is bit-identical.
+__device__ __forceinline__ void e8_nearest_hinted(const float (&x)[8], uint32_t hint, float (&out)[8]) {
+    // x - (+0) and r + (-0) leave every float, signed zeros included, unchanged
+    const float shift = (hint & 1u) ? 0.0f : 0.5f;
+    const float back = (hint & 1u) ? -0.0f : 0.5f;
+    const float step = (hint & 2u) ? ((hint & 32u) ? -1.0f : 1.0f) : 0.0f;
+    const uint32_t moved = (hint >> 2) & 7u;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float point = __builtin_rintf(x[j] - shift) + back;
+        out[j] = moved == (uint32_t)j ? point + step : point;
+    }
 }
 
 // Integer generator coordinates of a lattice point (closed form of codec.py:89-96,
@@ -149,11 +179,16 @@ __device__ __forceinline__ float div_by_14(float p) {
 
 // codec.py:105-142 `decode_nested` for one block given its coset point (already minus
 // the dither when there is one): the minimum-energy representative p - q * Q(p / q).
-__device__ __forceinline__ void reduce_coset_point(const float (&p)[8], float q, float (&out)[8]) {
+// kHint: 0 = search, 1 = rebuild from `hint`, 2 = search and emit `hint`.
+template <int kHint = 0>
+__device__ __forceinline__ void reduce_coset_point(const float (&p)[8], float q, float (&out)[8],
+                                                   uint32_t *hint = nullptr) {
     float z[8], k[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) z[j] = (q == 14.0f) ? div_by_14(p[j]) : p[j] / q;   // IEEE division
-    e8_nearest(z, k);
+    if (kHint == 1) e8_nearest_hinted(z, *hint, k);
+    else if (kHint == 2) e8_nearest_impl<true>(z, k, hint);
+    else e8_nearest(z, k);
 #pragma unroll
     for (int j = 0; j < 8; j++) out[j] = p[j] - q * k[j]; // exact
 }
@@ -171,12 +206,16 @@ __device__ __forceinline__ uint32_t lcg31_mix(uint32_t counter_plus_seed) {
 }
 
 // codec.py:222-224: u = float32(v) * 2^-30 in [0, 2], then d = u - Q_E8(u).
-__device__ __forceinline__ void dither_block(uint32_t first_counter_plus_seed, float (&d)[8]) {
+template <int kHint = 0>
+__device__ __forceinline__ void dither_block(uint32_t first_counter_plus_seed, float (&d)[8],
+                                             uint32_t *hint = nullptr) {
     float u[8], n[8];
 #pragma unroll
     for (int j = 0; j < 8; j++)
         u[j] = (float)lcg31_mix(first_counter_plus_seed + (uint32_t)j) * (2.0f / 2147483648.0f);
-    e8_nearest(u, n);
+    if (kHint == 1) e8_nearest_hinted(u, *hint, n);
+    else if (kHint == 2) e8_nearest_impl<true>(u, n, hint);
+    else e8_nearest(u, n);
 #pragma unroll
     for (int j = 0; j < 8; j++) d[j] = u[j] - n[j];
 }
@@ -184,19 +223,29 @@ __device__ __forceinline__ void dither_block(uint32_t first_counter_plus_seed, f
 // Decode one packed block to lattice units (no beta / norm scale yet).
 // counter_plus_seed is the low 32 bits of (global_block * 8 + seed); dithered == false
 // skips the dither (activations and KV pages).
-template <bool kDithered>
+//
+// Decode hints (dithered weights only).  Both lattice searches of a weight block depend only
+// on the stored code, the seed and the block index, so their outcomes can be computed once
+// when a weight is prepared and kept as 12 bits per block (bits 0..5: dither search,
+// bits 6..11: coarse search; layout in e8_nearest_impl).  kHint = 1 rebuilds both points
+// from `*hints` instead of searching -- the same values, about half the instructions;
+// kHint = 2 searches and writes `*hints`.
+template <bool kDithered, int kHint = 0>
 __device__ __forceinline__ void decode_codeword(uint32_t word, float q, uint32_t counter_plus_seed,
-                                                float (&out)[8]) {
+                                                float (&out)[8], uint32_t *hints = nullptr) {
     float c[8], p[8];
     unpack_codeword(word, c);
     e8_coset_point(c, p);
+    uint32_t hint_dither = 0u, hint_coarse = 0u;
+    if (kHint == 1) { hint_dither = *hints & 63u; hint_coarse = (*hints >> 6) & 63u; }
     if (kDithered) {
         float d[8];
-        dither_block(counter_plus_seed, d);
+        dither_block<kHint>(counter_plus_seed, d, &hint_dither);
 #pragma unroll
         for (int j = 0; j < 8; j++) p[j] = p[j] - d[j];
     }
-    reduce_coset_point(p, q, out);
+    reduce_coset_point<kHint>(p, q, out, &hint_coarse);
+    if (kHint == 2) *hints = hint_dither | (hint_coarse << 6);
 }
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t bits) {

@@ -35,10 +35,11 @@ constexpr int kGemmBK = 128;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-template <int TILES>   // token tiles (of 32 rows) per wavefront
+template <int TILES, bool kHinted>   // token tiles (of 32 rows) per wavefront; decode hints present
 __global__ void __launch_bounds__(kGemmThreads)
 w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
-                 const uint32_t *__restrict__ w_codes, const uint8_t *__restrict__ w_beta_ids,
+                 const uint32_t *__restrict__ w_codes, const uint16_t *__restrict__ w_hints,
+                 const uint8_t *__restrict__ w_beta_ids,
                  const float *__restrict__ w_norms, const float *__restrict__ w_betas,
                  int m_rows, int k_size, int n_size, int k_slab, uint32_t seed_plus_offset,
                  float sqrt_k, float *__restrict__ out_f32, uint16_t *__restrict__ out_bf16) {
@@ -79,7 +80,12 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
             uint4 packed = make_uint4(0, 0, 0, 0);
             if (dec_live) {
                 float v[8];
-                decode_codeword<true>(w_codes[g], 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
+                if (kHinted) {
+                    uint32_t hints = w_hints[g];
+                    decode_codeword<true, 1>(w_codes[g], 14.0f, seed_plus_offset + (uint32_t)g * 8u, v, &hints);
+                } else {
+                    decode_codeword<true>(w_codes[g], 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
+                }
                 const float scale = wbeta[(w_beta_ids[g >> 2] >> (2 * (g & 3))) & 3] * wscale;
                 const bf16x2 h0 = pack_bf16x2(v[0] * scale, v[1] * scale), h1 = pack_bf16x2(v[2] * scale, v[3] * scale);
                 const bf16x2 h2 = pack_bf16x2(v[4] * scale, v[5] * scale), h3 = pack_bf16x2(v[6] * scale, v[7] * scale);
@@ -154,7 +160,7 @@ extern "C" size_t nq_w4a4_gemm_workspace_bytes(int m, int k, int n, int split_k,
 extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
                             const float *act_norms_dev, const float *act_betas_dev,
                             const void *act_decoded_dev, const uint8_t *w_codes_dev,
-                            const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
+                            const uint16_t *w_hints_dev, const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
                             const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
                             int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
                             void *workspace_dev, size_t workspace_bytes, void *stream) {
@@ -209,14 +215,18 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
         float *target_f32 = split > 1 ? partials : (out_dtype == NQ_F32 ? (float *)out_chunk : nullptr);
         uint16_t *target_bf16 = (split > 1 || out_dtype == NQ_F32) ? nullptr : (uint16_t *)out_chunk;
         const uint16_t *act_chunk = act + (size_t)m0 * k;
-        if (rows <= 8 * 32)
-            hipLaunchKernelGGL(nq::w4a4_gemm_kernel<1>, grid, dim3(nq::kGemmThreads), 0, s, act_chunk, wc,
-                               w_beta_ids_dev, w_norms_dev, w_betas_dev, rows, k, n, k / split,
-                               seed_plus_offset, sqrt_k, target_f32, target_bf16);
-        else
-            hipLaunchKernelGGL(nq::w4a4_gemm_kernel<2>, grid, dim3(nq::kGemmThreads), 0, s, act_chunk, wc,
-                               w_beta_ids_dev, w_norms_dev, w_betas_dev, rows, k, n, k / split,
-                               seed_plus_offset, sqrt_k, target_f32, target_bf16);
+#define NQ_LAUNCH_GEMM(TILES, HINTED)                                                                  \
+    hipLaunchKernelGGL((nq::w4a4_gemm_kernel<TILES, HINTED>), grid, dim3(nq::kGemmThreads), 0, s, act_chunk, \
+                       wc, w_hints_dev, w_beta_ids_dev, w_norms_dev, w_betas_dev, rows, k, n, k / split,      \
+                       seed_plus_offset, sqrt_k, target_f32, target_bf16)
+        if (rows <= 8 * 32) {
+            if (w_hints_dev) NQ_LAUNCH_GEMM(1, true);
+            else NQ_LAUNCH_GEMM(1, false);
+        } else {
+            if (w_hints_dev) NQ_LAUNCH_GEMM(2, true);
+            else NQ_LAUNCH_GEMM(2, false);
+        }
+#undef NQ_LAUNCH_GEMM
         int status = nq::check_launch("nq_w4a4_gemm");
         if (status != NQ_OK) return status;
         if (split > 1) {

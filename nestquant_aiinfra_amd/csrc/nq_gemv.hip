@@ -28,10 +28,11 @@ constexpr int kGemvThreads = 256;
 constexpr int kGemvWaves = kGemvThreads / 64;
 constexpr int kGemvMaxRows = 8;
 
-template <int M>
+template <int M, bool kHinted>
 __global__ void __launch_bounds__(kGemvThreads)
 w4a4_gemv_kernel(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8] blocks
-                 const uint32_t *__restrict__ w_codes, const uint8_t *__restrict__ w_beta_ids,
+                 const uint32_t *__restrict__ w_codes, const uint16_t *__restrict__ w_hints,
+                 const uint8_t *__restrict__ w_beta_ids,
                  const float *__restrict__ w_norms, const float *__restrict__ w_betas,
                  int m_rows, int k_size, int n_size, int k_slice, int rows_per_wg,
                  uint32_t seed_plus_offset, float sqrt_k, float *__restrict__ out_f32,
@@ -55,21 +56,28 @@ w4a4_gemv_kernel(const uint4 *__restrict__ act,          // decoded BF16 [m_rows
                 const int64_t g = row_first_block + b;
                 const uint32_t word = w_codes[g];
                 const uint32_t ids = w_beta_ids[g >> 2];
+                // the activation blocks do not depend on the decode: request them first
+                uint4 a[M];
+#pragma unroll
+                for (int m = 0; m < M; m++)
+                    a[m] = m < m_rows ? act[(int64_t)m * blocks_per_row + slice_first_block + b] : make_uint4(0, 0, 0, 0);
                 float v[8];
-                decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
+                if (kHinted) {
+                    uint32_t hints = w_hints[g];
+                    decode_codeword<true, 1>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v, &hints);
+                } else {
+                    decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
+                }
                 const float scale = wbeta[(ids >> (2 * (g & 3))) & 3] * wscale;
                 bf16x2 w[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) w[j] = pack_bf16x2(v[2 * j] * scale, v[2 * j + 1] * scale);
 #pragma unroll
                 for (int m = 0; m < M; m++) {
-                    if (m < m_rows) {
-                        const uint4 a = act[(int64_t)m * blocks_per_row + slice_first_block + b];
-                        acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.x), w[0], acc[m], false);
-                        acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.y), w[1], acc[m], false);
-                        acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.z), w[2], acc[m], false);
-                        acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.w), w[3], acc[m], false);
-                    }
+                    acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].x), w[0], acc[m], false);
+                    acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].y), w[1], acc[m], false);
+                    acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].z), w[2], acc[m], false);
+                    acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].w), w[3], acc[m], false);
                 }
             }
         }
@@ -99,7 +107,38 @@ w4a4_gemv_kernel(const uint4 *__restrict__ act,          // decoded BF16 [m_rows
     }
 }
 
+// One lane per weight block: run both exact lattice searches once and keep their outcomes.
+__global__ void __launch_bounds__(256)
+make_decode_hints_kernel(const uint32_t *__restrict__ w_codes, int64_t blocks, uint32_t seed_plus_offset,
+                         uint16_t *__restrict__ hints) {
+    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= blocks) return;
+    float v[8];
+    uint32_t h = 0u;
+    decode_codeword<true, 2>(w_codes[g], 14.0f, seed_plus_offset + (uint32_t)g * 8u, v, &h);
+    hints[g] = (uint16_t)h;
+}
+
 }  // namespace nq
+
+extern "C" int nq_w4a4_make_decode_hints(const uint8_t *w_codes_dev, int64_t rows, int64_t k,
+                                         int64_t weight_offset, int64_t weight_seed, uint16_t *hints_dev,
+                                         void *stream) {
+    NQ_REQUIRE(rows >= 1 && k >= 8 && k % 8 == 0, NQ_ERR_SHAPE,
+               "nq_w4a4_make_decode_hints: rows must be positive and K a positive multiple of 8");
+    NQ_REQUIRE(w_codes_dev && hints_dev && nq::aligned(w_codes_dev, 4) && nq::aligned(hints_dev, 2),
+               NQ_ERR_ARGUMENT, "nq_w4a4_make_decode_hints: null or misaligned pointer");
+    NQ_REQUIRE(weight_seed >= 0 && weight_seed < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
+               "nq_w4a4_make_decode_hints: seed must be in [0, 2**31)");
+    const int64_t blocks = rows * (k / 8);
+    NQ_REQUIRE(weight_offset >= 0 && weight_offset + blocks <= ((int64_t)1 << 28), NQ_ERR_SHAPE,
+               "nq_w4a4_make_decode_hints: block range exceeds the stateless dither counter space");
+    const uint32_t seed_plus_offset = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
+    hipLaunchKernelGGL(nq::make_decode_hints_kernel, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, reinterpret_cast<const uint32_t *>(w_codes_dev), blocks,
+                       seed_plus_offset, hints_dev);
+    return nq::check_launch("nq_w4a4_make_decode_hints");
+}
 
 namespace {
 
@@ -129,7 +168,7 @@ extern "C" size_t nq_w4a4_gemv_workspace_bytes(int m, int k, int n, int split_k,
 extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
                             const float *act_norms_dev, const float *act_betas_dev,
                             const void *act_decoded_dev, const uint8_t *w_codes_dev,
-                            const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
+                            const uint16_t *w_hints_dev, const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
                             const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
                             int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
                             void *workspace_dev, size_t workspace_bytes, void *stream) {
@@ -145,7 +184,7 @@ extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_bet
     NQ_REQUIRE(act_decoded_dev || (act_codes_dev && act_beta_ids_dev && act_norms_dev && act_betas_dev),
                NQ_ERR_ARGUMENT, "nq_w4a4_gemv: neither packed nor decoded activation given");
     NQ_REQUIRE(nq::aligned(w_codes_dev, 4) && (!act_codes_dev || nq::aligned(act_codes_dev, 4)) &&
-                   (!act_decoded_dev || nq::aligned(act_decoded_dev, 16)),
+                   (!act_decoded_dev || nq::aligned(act_decoded_dev, 16)) && nq::aligned(w_hints_dev, 2),
                NQ_ERR_ARGUMENT, "nq_w4a4_gemv: code streams need 4-byte, decoded activation 16-byte alignment");
     NQ_REQUIRE(weight_seed >= 0 && weight_seed < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
                "nq_w4a4_gemv: seed must be in [0, 2**31)");
@@ -180,10 +219,15 @@ extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_bet
     float *target_f32 = split > 1 ? partials : (out_dtype == NQ_F32 ? (float *)out_dev : nullptr);
     uint16_t *target_bf16 = (split > 1 || out_dtype == NQ_F32) ? nullptr : (uint16_t *)out_dev;
     const uint32_t *wc = reinterpret_cast<const uint32_t *>(w_codes_dev);
+#define NQ_LAUNCH_GEMV_AS(MT, HINTED)                                                               \
+    hipLaunchKernelGGL((nq::w4a4_gemv_kernel<MT, HINTED>), grid, dim3(nq::kGemvThreads), 0, s, act, \
+                       wc, w_hints_dev, w_beta_ids_dev, w_norms_dev, w_betas_dev, m, k, n, k_slice, \
+                       rows_per_wg, seed_plus_offset, sqrt_k, target_f32, target_bf16)
 #define NQ_LAUNCH_GEMV(MT)                                                                          \
-    hipLaunchKernelGGL(nq::w4a4_gemv_kernel<MT>, grid, dim3(nq::kGemvThreads), 0, s, act, wc,       \
-                       w_beta_ids_dev, w_norms_dev, w_betas_dev, m, k, n, k_slice, rows_per_wg,     \
-                       seed_plus_offset, sqrt_k, target_f32, target_bf16)
+    do {                                                                                            \
+        if (w_hints_dev) NQ_LAUNCH_GEMV_AS(MT, true);                                               \
+        else NQ_LAUNCH_GEMV_AS(MT, false);                                                          \
+    } while (0)
     switch (m_tile_of(m)) {
         case 1: NQ_LAUNCH_GEMV(1); break;
         case 2: NQ_LAUNCH_GEMV(2); break;
@@ -191,6 +235,7 @@ extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_bet
         default: NQ_LAUNCH_GEMV(8); break;
     }
 #undef NQ_LAUNCH_GEMV
+#undef NQ_LAUNCH_GEMV_AS
     int status = nq::check_launch("nq_w4a4_gemv");
     if (status != NQ_OK || split == 1) return status;
     return nq::launch_splitk_reduce(partials, split, (int64_t)m * n, out_dev, out_dtype, s);

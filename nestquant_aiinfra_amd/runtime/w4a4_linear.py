@@ -67,6 +67,9 @@ class PreparedNQRTLinear:
     beta_payload: torch.Tensor
     row_norms: torch.Tensor
     beta_table: torch.Tensor
+    # Optional uint16 per 8-weight block: the outcomes of the two lattice searches of the
+    # block's decode, computed once here so the linear kernels need not search (same results).
+    decode_hints: torch.Tensor | None = None
 
 
 # --------------------------------------------------------------------------------------
@@ -189,8 +192,20 @@ def _payload_tensor(payload: bytes, device: torch.device) -> torch.Tensor:
     return torch.frombuffer(bytearray(payload), dtype=torch.uint8).to(device)
 
 
-def prepare_fused_linear(record: Any, *, device: torch.device | str = "cuda") -> PreparedNQRTLinear:
-    """Copy only the packed NQRT streams and compact metadata to the target GPU."""
+def make_decode_hints(code_payload: torch.Tensor, *, rows: int, features: int, dither_seed: int,
+                      block_offset: int = 0) -> torch.Tensor:
+    device = _native.require_cuda(code_payload)
+    hints = torch.empty(rows * features // 8, dtype=torch.int16, device=device)
+    _native.check(_native.library().nq_w4a4_make_decode_hints(
+        code_payload.data_ptr(), rows, features, block_offset, int(dither_seed), hints.data_ptr(),
+        _native.stream_handle(device)))
+    return hints
+
+
+def prepare_fused_linear(record: Any, *, device: torch.device | str = "cuda",
+                         decode_hints: bool = True) -> PreparedNQRTLinear:
+    """Copy only the packed NQRT streams and compact metadata to the target GPU, and (unless
+    `decode_hints=False`) derive the 2-byte-per-block decode hints from them."""
     for attribute in ("indices", "row_norms", "betas", "feature_count", "dither_seed",
                       "dither_algorithm", "codec_semantics"):
         if not hasattr(record, attribute):
@@ -202,12 +217,18 @@ def prepare_fused_linear(record: Any, *, device: torch.device | str = "cuda") ->
         raise ValueError("fused Linear requires NQRT v4 stateless dither")
     if record.codec_semantics != UPSTREAM_CODEC_SEMANTICS:
         raise ValueError("fused Linear requires upstream E8 semantics")
+    codes = _payload_tensor(record.indices.code_payload, target)
+    hints = None
+    if decode_hints and record.indices.q == 14 and record.indices.code_bit_width == 4:
+        hints = make_decode_hints(codes, rows=record.indices.shape[0], features=record.feature_count,
+                                  dither_seed=record.dither_seed)
     return PreparedNQRTLinear(
         record=record,
-        code_payload=_payload_tensor(record.indices.code_payload, target),
+        code_payload=codes,
         beta_payload=_payload_tensor(record.indices.beta_payload, target),
         row_norms=record.row_norms.to(device=target, dtype=torch.float32),
         beta_table=torch.tensor(record.betas, device=target, dtype=torch.float32),
+        decode_hints=hints,
     )
 
 
@@ -324,7 +345,8 @@ def _gemv(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *, spl
     _native.check(launch(
         activation.code_payload.data_ptr(), activation.beta_payload.data_ptr(),
         activation.row_norms.data_ptr(), activation.beta_table.data_ptr(),
-        None if decoded is None else decoded.data_ptr(), weight.code_payload.data_ptr(), weight.beta_payload.data_ptr(),
+        None if decoded is None else decoded.data_ptr(), weight.code_payload.data_ptr(),
+        None if weight.decode_hints is None else weight.decode_hints.data_ptr(), weight.beta_payload.data_ptr(),
         weight.row_norms.data_ptr(), weight.beta_table.data_ptr(), m, k, n, 0,
         int(weight.record.dither_seed), split_k, out.data_ptr(), _native.dtype_tag(output_dtype),
         None if workspace is None else workspace.data_ptr(), need, _native.stream_handle(device)))

@@ -129,3 +129,31 @@ def test_predicates_and_errors(rt, oracle):
         rt.linear_packed_w4a4_gemv_m1_splitk_probe(a1, weight, split_k=3)
     other = rt.quantize_activation_cuda(torch.randn(1, 512, device="cuda"), q=Q, betas=ACTIVATION_BETAS)
     assert not rt.can_use_w4a4_gemv_m1(other, weight)
+
+
+@pytest.mark.parametrize("k,n_out,seed", [(256, 64, 0), (2048, 2048, 20261101), (8192, 256, 2**31 - 1)])
+def test_decode_hints_change_no_bit(rt, oracle, k, n_out, seed):
+    """The hint stream is a pure function of (codes, seed, block index); kernels that rebuild the
+    lattice points from it must return exactly what the searching kernels return."""
+    import dataclasses
+    _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=77 + k, dither_seed=seed)
+    hinted = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
+    assert hinted.decode_hints is not None and hinted.decode_hints.numel() == n_out * k // 8
+    searching = dataclasses.replace(hinted, decode_hints=None)
+    assert rt.prepare_fused_linear(hinted.record, device="cuda", decode_hints=False).decode_hints is None
+    # every hint carries a legal coset/move encoding and both searches are represented
+    h = hinted.decode_hints.cpu().numpy().view(np.uint16)
+    assert int(h.max()) < 4096
+    for m in (1, 4, 8, 48, 160):
+        x = torch.from_numpy(oracle.hadamard(student_t_rows(m, k, seed=5 + m).numpy())).to(torch.bfloat16).cuda()
+        activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS)
+        for out_dtype in (torch.float32, torch.bfloat16):
+            if m <= 8:
+                a = rt._gemv(activation, hinted, split_k=0, output_dtype=out_dtype)
+                b = rt._gemv(activation, searching, split_k=0, output_dtype=out_dtype)
+                assert torch.equal(a.view(torch.int32 if out_dtype == torch.float32 else torch.int16),
+                                   b.view(torch.int32 if out_dtype == torch.float32 else torch.int16))
+            a = rt._gemm(activation, hinted, split_k=0, output_dtype=out_dtype)
+            b = rt._gemm(activation, searching, split_k=0, output_dtype=out_dtype)
+            assert torch.equal(a.view(torch.int32 if out_dtype == torch.float32 else torch.int16),
+                               b.view(torch.int32 if out_dtype == torch.float32 else torch.int16))
