@@ -87,7 +87,8 @@ def build_workload(device):
         weights = [base] + [
             rt.PreparedNQRTLinear(record, base.code_payload.clone(), base.beta_payload.clone(),
                                   base.row_norms.clone(), base.beta_table.clone(),
-                                  None if base.decode_hints is None else base.decode_hints.clone())
+                                  None if base.resolved_words is None else base.resolved_words.clone(),
+                                  None if base.resolved_tails is None else base.resolved_tails.clone())
             for _ in range(copies - 1)
         ]
         for m in TOKEN_COUNTS:
@@ -229,7 +230,8 @@ def prefill_gemm_extra(rt, device):
         copies = 32
         weights = [base] + [rt.PreparedNQRTLinear(record, base.code_payload.clone(), base.beta_payload.clone(),
                                                   base.row_norms, base.beta_table,
-                                                  None if base.decode_hints is None else base.decode_hints.clone())
+                                                  None if base.resolved_words is None else base.resolved_words.clone(),
+                                                  None if base.resolved_tails is None else base.resolved_tails.clone())
                             for _ in range(copies - 1)]
         table = torch.tensor(ACTIVATION_BETAS, dtype=torch.float32, device=device)
         for m in (16, 40, 64, 128, 384):

@@ -108,18 +108,27 @@ int nq_dequantize_rows(const uint8_t *codes_dev, const uint8_t *beta_ids_dev,
                        void *out_dev, int out_dtype, void *stream);
 
 /*
- * Decode hints for one NQRT4 weight [rows, K]: for every 8-weight block, the outcomes of the
- * two exact E8 searches its decode performs (which coset won, which coordinate was moved and
- * in which direction; 6 bits each, packed in a uint16).  They depend only on the stored code
- * words, the seed and the block index, so they are computed once when a weight is prepared;
- * the linear kernels then rebuild the same lattice points without searching (bit-identical
- * results, about half the vector instructions per block).  hints_dev: uint16[rows * K / 8].
+ * Resolved form of one NQRT4 weight [rows, K], made once when the weight is prepared.
+ * A dithered block decodes to w = (G c - d) - 14 Q_E8((G c - d) / 14), d = u - Q_E8(u) with u
+ * the hashed uniforms of the block; both lattice searches depend only on the stored code, the
+ * seed and the block index.  This entry runs the exact decode and stores the lattice point
+ * s = G c + Q_E8(u) - 14 Q_E8(...) of every block, so that the linear kernels compute w = s - u
+ * with the hash alone (no search, no division; about a third of the vector instructions).
+ *   words_dev  uint32[rows * K / 8]: floor(s_j) + 15 for j = 0..5 in 5-bit fields from bit 0,
+ *              the block's beta id in bits 30..31
+ *   tails_dev  uint16[rows * K / 8]: fields 6 and 7 in bits 0..9, bit 10 set when s lies in
+ *              the half-integer coset
+ *   out_of_range_dev  int32 counter (caller zeroes it): blocks whose s does not fit the
+ *              fields; geometry bounds s_j to [-14, 16], so any count other than 0 means the
+ *              streams are not a valid NQRT4 record and the resolved form must not be used
+ * 6 bytes per block (6 bits per weight) against the 4.25 bits of the NQRT4 streams.
  * No counterpart in the reference (its kernels repeat both searches on every call,
  * nestquant/runtime/nqrt4_cooperative_device.cuh:150-171).
  */
-int nq_w4a4_make_decode_hints(const uint8_t *w_codes_dev, int64_t rows, int64_t k,
-                              int64_t weight_offset, int64_t weight_seed, uint16_t *hints_dev,
-                              void *stream);
+int nq_w4a4_resolve_weight(const uint8_t *w_codes_dev, const uint8_t *w_beta_ids_dev, int64_t rows,
+                           int64_t k, int64_t weight_offset, int64_t weight_seed,
+                           uint32_t *words_dev, uint16_t *tails_dev, int32_t *out_of_range_dev,
+                           void *stream);
 
 /*
  * Packed W4A4 linear for decode, M = 1..8 tokens: y[m, n] = sum_k bf16(a[m, k]) * bf16(w[n, k]),
@@ -130,7 +139,11 @@ int nq_w4a4_make_decode_hints(const uint8_t *w_codes_dev, int64_t rows, int64_t 
  *                    when NULL the packed streams are decoded once into the workspace,
  *                    when given the packed streams may be NULL
  *   w_*              NQRT4 streams of [N, K] (codes N*K/2 B, beta ids N*K/32 B, norms f32[N], betas f32[4])
- *   w_hints_dev      optional uint16[N * K / 8] from nq_w4a4_make_decode_hints (NULL: search)
+ *   w_resolved_words_dev, w_resolved_tails_dev
+ *                    optional resolved form from nq_w4a4_resolve_weight; when given it is used
+ *                    instead of w_codes_dev / w_beta_ids_dev, which may then be NULL.  Results
+ *                    agree with the NQRT4 path to FP32 rounding (before the BF16 rounding of
+ *                    the weight), not bit for bit
  *   out_dev          [M, N] of out_dtype (NQ_F32 or NQ_BF16)
  *   split_k          1, 2, 4 or 8 slices of K reduced in ascending order (deterministic); 0 lets
  *                    the library choose
@@ -144,7 +157,8 @@ int nq_w4a4_make_decode_hints(const uint8_t *w_codes_dev, int64_t rows, int64_t 
 int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
                  const float *act_norms_dev, const float *act_betas_dev,
                  const void *act_decoded_dev, const uint8_t *w_codes_dev,
-                 const uint16_t *w_hints_dev, const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
+                 const uint8_t *w_beta_ids_dev, const uint32_t *w_resolved_words_dev,
+                 const uint16_t *w_resolved_tails_dev, const float *w_norms_dev,
                  const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
                  int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
                  void *workspace_dev, size_t workspace_bytes, void *stream);
@@ -166,7 +180,8 @@ size_t nq_w4a4_gemv_workspace_bytes(int m, int k, int n, int split_k, int have_d
 int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
                  const float *act_norms_dev, const float *act_betas_dev,
                  const void *act_decoded_dev, const uint8_t *w_codes_dev,
-                 const uint16_t *w_hints_dev, const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
+                 const uint8_t *w_beta_ids_dev, const uint32_t *w_resolved_words_dev,
+                 const uint16_t *w_resolved_tails_dev, const float *w_norms_dev,
                  const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
                  int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
                  void *workspace_dev, size_t workspace_bytes, void *stream);

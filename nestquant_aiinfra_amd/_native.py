@@ -35,11 +35,11 @@ SIGNATURES = {
     "nq_hadamard": (_i32, [_ptr, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr]),
     "nq_dequantize_rows": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i64, _i64,
                                   _ptr, _i32, _ptr]),
-    "nq_w4a4_make_decode_hints": (_i32, [_ptr, _i64, _i64, _i64, _i64, _ptr, _ptr]),
-    "nq_w4a4_gemv": (_i32, [_ptr] * 10 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
+    "nq_w4a4_resolve_weight": (_i32, [_ptr, _ptr, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "nq_w4a4_gemv": (_i32, [_ptr] * 11 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
                                           _size, _ptr]),
     "nq_w4a4_gemv_workspace_bytes": (_size, [_i32, _i32, _i32, _i32, _i32]),
-    "nq_w4a4_gemm": (_i32, [_ptr] * 10 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
+    "nq_w4a4_gemm": (_i32, [_ptr] * 11 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
                                           _size, _ptr]),
     "nq_w4a4_gemm_workspace_bytes": (_size, [_i32, _i32, _i32, _i32, _i32]),
     "nq_nqkv_advance": (_i32, [_ptr, _ptr, _ptr, _i32, _i32, _i32, _i32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),

@@ -37,12 +37,7 @@ __device__ __forceinline__ bool is_odd(float sum) { return __builtin_amdgcn_frac
 // moved coordinate contributes (|residual| - 1)^2 = (max - 1)^2, one value per block.
 // Half coset: the reference measures x - (D8(x - 1/2) + 1/2), recomputed from x because
 // x - 1/2 may round; the same is done here.
-//
-// `hint` (optional) receives six bits that let e8_nearest_hinted() rebuild the same point
-// without searching: bit 0 = the integer coset won, bit 1 = a coordinate was moved,
-// bits 2..4 = which one, bit 5 = it moved down (-1).
-template <bool kWantHint>
-__device__ __forceinline__ void e8_nearest_impl(const float (&x)[8], float (&out)[8], uint32_t *hint) {
+__device__ __forceinline__ void e8_nearest(const float (&x)[8], float (&out)[8]) {
     float a[8], ea[8], sum_a = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
@@ -55,7 +50,6 @@ __device__ __forceinline__ void e8_nearest_impl(const float (&x)[8], float (&out
     const float alt_a = moved_a * moved_a;
     bool done_a = !is_odd(sum_a);                  // an even sum needs no correction
     float dist_a = 0.0f;
-    uint32_t hint_a = 0u;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const bool top = fabsf(ea[j]) == max_a;
@@ -65,7 +59,6 @@ __device__ __forceinline__ void e8_nearest_impl(const float (&x)[8], float (&out
         dist_a = dist_a + (hit ? alt_a : sq);
         // residual >= 0 moves up (a residual is never -0)
         a[j] = hit ? a[j] + __builtin_copysignf(1.0f, ea[j]) : a[j];
-        if (kWantHint) hint_a = hit ? (2u | ((uint32_t)j << 2) | (ea[j] < 0.0f ? 32u : 0u)) : hint_a;
     }
 
     float b[8], eb[8], sum_b = 0.0f;
@@ -79,7 +72,6 @@ __device__ __forceinline__ void e8_nearest_impl(const float (&x)[8], float (&out
     const float max_b = max_abs8(eb);
     bool done_b = !is_odd(sum_b);
     float dist_b = 0.0f;
-    uint32_t hint_b = 0u;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const bool top = fabsf(eb[j]) == max_b;
@@ -89,32 +81,10 @@ __device__ __forceinline__ void e8_nearest_impl(const float (&x)[8], float (&out
         b[j] = hit ? half_point + __builtin_copysignf(1.0f, eb[j]) : half_point;
         const float t = x[j] - b[j];
         dist_b = dist_b + t * t;
-        if (kWantHint) hint_b = hit ? (2u | ((uint32_t)j << 2) | (eb[j] < 0.0f ? 32u : 0u)) : hint_b;
     }
     const bool pick_a = dist_a < dist_b;           // ties go to the half-integer coset
 #pragma unroll
     for (int j = 0; j < 8; j++) out[j] = pick_a ? a[j] : b[j];
-    if (kWantHint) *hint = pick_a ? (hint_a | 1u) : hint_b;
-}
-
-__device__ __forceinline__ void e8_nearest(const float (&x)[8], float (&out)[8]) {
-    e8_nearest_impl<false>(x, out, nullptr);
-}
-
-// The point e8_nearest() returns for x, rebuilt from the six hint bits it emitted for the
-// same x: round in the chosen coset, move the recorded coordinate.  Same float operations
-// as the search performs on the winning coset, so the result is bit-identical.
-__device__ __forceinline__ void e8_nearest_hinted(const float (&x)[8], uint32_t hint, float (&out)[8]) {
-    // x - (+0) and r + (-0) leave every float, signed zeros included, unchanged
-    const float shift = (hint & 1u) ? 0.0f : 0.5f;
-    const float back = (hint & 1u) ? -0.0f : 0.5f;
-    const float step = (hint & 2u) ? ((hint & 32u) ? -1.0f : 1.0f) : 0.0f;
-    const uint32_t moved = (hint >> 2) & 7u;
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const float point = __builtin_rintf(x[j] - shift) + back;
-        out[j] = moved == (uint32_t)j ? point + step : point;
-    }
 }
 
 // Integer generator coordinates of a lattice point (closed form of codec.py:89-96,
@@ -179,43 +149,51 @@ __device__ __forceinline__ float div_by_14(float p) {
 
 // codec.py:105-142 `decode_nested` for one block given its coset point (already minus
 // the dither when there is one): the minimum-energy representative p - q * Q(p / q).
-// kHint: 0 = search, 1 = rebuild from `hint`, 2 = search and emit `hint`.
-template <int kHint = 0>
-__device__ __forceinline__ void reduce_coset_point(const float (&p)[8], float q, float (&out)[8],
-                                                   uint32_t *hint = nullptr) {
+__device__ __forceinline__ void reduce_coset_point(const float (&p)[8], float q, float (&out)[8]) {
     float z[8], k[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) z[j] = (q == 14.0f) ? div_by_14(p[j]) : p[j] / q;   // IEEE division
-    if (kHint == 1) e8_nearest_hinted(z, *hint, k);
-    else if (kHint == 2) e8_nearest_impl<true>(z, k, hint);
-    else e8_nearest(z, k);
+    e8_nearest(z, k);
 #pragma unroll
     for (int j = 0; j < 8; j++) out[j] = p[j] - q * k[j]; // exact
 }
 
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+// x * c + a modulo 2^32 from two 16-bit dot products and a shift-add (three full-rate
+// instructions; a 32-bit integer multiply issues at a quarter of that rate).
+// With x = xl + 2^16 xh and c = cl + 2^16 ch:  x c = xl cl + 2^16 (xl ch + xh cl)  (mod 2^32).
+__device__ __forceinline__ uint32_t mul_add_u32(uint32_t x, uint32_t c, uint32_t a) {
+    const u16x2 xv = __builtin_bit_cast(u16x2, x);
+    const uint32_t cross = __builtin_amdgcn_udot2(xv, __builtin_bit_cast(u16x2, (c << 16) | (c >> 16)), 0u, false);
+    const uint32_t low = __builtin_amdgcn_udot2(xv, __builtin_bit_cast(u16x2, c & 0xffffu), a, false);
+    return (cross << 16) + low;
+}
+
 // codec.py:213-222 / nestquant/runtime/nqrt4_device.cuh:7-17: lcg31_mix_v1.  Only the
-// low 31 bits of every stage matter, so masks are folded into bit-field extracts.
-__device__ __forceinline__ uint32_t lcg31_mix(uint32_t counter_plus_seed) {
+// low 31 bits of every stage matter, so masks are folded into bit-field extracts; bit 31 of
+// the value returned here is not meaningful.
+__device__ __forceinline__ uint32_t lcg31_mix_bits(uint32_t counter_plus_seed) {
     uint32_t v = counter_plus_seed;
     v ^= (v >> 16) & 0x7fffu;                 // bits 16..30 of the masked value
-    v = v * 1103515245u + 12345u;
+    v = mul_add_u32(v, 1103515245u, 12345u);
     v ^= (v >> 13) & 0x3ffffu;                // bits 13..30
-    v = v * 134775813u + 1u;
+    v = mul_add_u32(v, 134775813u, 1u);
     v ^= (v >> 16) & 0x7fffu;
-    return v & 0x7fffffffu;
+    return v;
+}
+
+__device__ __forceinline__ uint32_t lcg31_mix(uint32_t counter_plus_seed) {
+    return lcg31_mix_bits(counter_plus_seed) & 0x7fffffffu;
 }
 
 // codec.py:222-224: u = float32(v) * 2^-30 in [0, 2], then d = u - Q_E8(u).
-template <int kHint = 0>
-__device__ __forceinline__ void dither_block(uint32_t first_counter_plus_seed, float (&d)[8],
-                                             uint32_t *hint = nullptr) {
+__device__ __forceinline__ void dither_block(uint32_t first_counter_plus_seed, float (&d)[8]) {
     float u[8], n[8];
 #pragma unroll
     for (int j = 0; j < 8; j++)
         u[j] = (float)lcg31_mix(first_counter_plus_seed + (uint32_t)j) * (2.0f / 2147483648.0f);
-    if (kHint == 1) e8_nearest_hinted(u, *hint, n);
-    else if (kHint == 2) e8_nearest_impl<true>(u, n, hint);
-    else e8_nearest(u, n);
+    e8_nearest(u, n);
 #pragma unroll
     for (int j = 0; j < 8; j++) d[j] = u[j] - n[j];
 }
@@ -223,29 +201,78 @@ __device__ __forceinline__ void dither_block(uint32_t first_counter_plus_seed, f
 // Decode one packed block to lattice units (no beta / norm scale yet).
 // counter_plus_seed is the low 32 bits of (global_block * 8 + seed); dithered == false
 // skips the dither (activations and KV pages).
-//
-// Decode hints (dithered weights only).  Both lattice searches of a weight block depend only
-// on the stored code, the seed and the block index, so their outcomes can be computed once
-// when a weight is prepared and kept as 12 bits per block (bits 0..5: dither search,
-// bits 6..11: coarse search; layout in e8_nearest_impl).  kHint = 1 rebuilds both points
-// from `*hints` instead of searching -- the same values, about half the instructions;
-// kHint = 2 searches and writes `*hints`.
-template <bool kDithered, int kHint = 0>
+template <bool kDithered>
 __device__ __forceinline__ void decode_codeword(uint32_t word, float q, uint32_t counter_plus_seed,
-                                                float (&out)[8], uint32_t *hints = nullptr) {
+                                                float (&out)[8]) {
     float c[8], p[8];
     unpack_codeword(word, c);
     e8_coset_point(c, p);
-    uint32_t hint_dither = 0u, hint_coarse = 0u;
-    if (kHint == 1) { hint_dither = *hints & 63u; hint_coarse = (*hints >> 6) & 63u; }
     if (kDithered) {
         float d[8];
-        dither_block<kHint>(counter_plus_seed, d, &hint_dither);
+        dither_block(counter_plus_seed, d);
 #pragma unroll
         for (int j = 0; j < 8; j++) p[j] = p[j] - d[j];
     }
-    reduce_coset_point<kHint>(p, q, out, &hint_coarse);
-    if (kHint == 2) *hints = hint_dither | (hint_coarse << 6);
+    reduce_coset_point(p, q, out);
+}
+
+// ---------------------------------------------------------------------------------------
+// Resolved weight blocks.
+//
+// A dithered block decodes to  w = (p - d) - 14 k  with p = G c the coset point of its code,
+// d = u - n the dither (u the hashed uniforms, n = Q_E8(u)) and k = Q_E8((p - d) / 14).  Both
+// lattice searches depend only on the stored code, the seed and the block index, so they can
+// be done once when a weight is prepared: s = p + n - 14 k is a point of E8 and  w = s - u.
+// resolve_codeword() runs the exact decode and stores s in 43 bits: the eight floors
+// floor(s_j) + 15 as 5-bit fields (w and u bound s_j to [-14, 16]), one bit saying that
+// the point lies in the half-integer coset, and the block's 2-bit beta id, as a 32-bit word
+// (fields 0..5, beta id in bits 30..31) and a 16-bit word (fields 6..7, half flag in bit 10).
+// decode_resolved() then needs the hash and six instructions per weight, no search and no
+// division.  It returns (s - u) * 2^26 computed in integers from the hash value with its
+// four lowest bits dropped: a 2^-26 absolute deviation from the float decode, far below the
+// BF16 rounding that follows, and the lattice points themselves are the exact ones.
+constexpr float kResolvedUnit = 1.0f / 67108864.0f;   // 2^-26
+
+__device__ __forceinline__ bool resolve_codeword(uint32_t word, uint32_t counter_plus_seed, uint32_t beta_id,
+                                                 uint32_t &lo, uint32_t &hi) {
+    float c[8], p[8], u[8], n[8], t[8], k[8];
+    unpack_codeword(word, c);
+    e8_coset_point(c, p);
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+        u[j] = (float)lcg31_mix(counter_plus_seed + (uint32_t)j) * (2.0f / 2147483648.0f);
+    e8_nearest(u, n);
+#pragma unroll
+    for (int j = 0; j < 8; j++) t[j] = div_by_14(p[j] - (u[j] - n[j]));
+    e8_nearest(t, k);
+    bool in_range = true;
+    uint32_t field[8];
+    float first_floor = 0.0f, first = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float s = (p[j] + n[j]) - 14.0f * k[j];     // half-integers of small magnitude: exact
+        const float biased = __builtin_floorf(s) + 15.0f;
+        in_range = in_range && biased >= 0.0f && biased <= 31.0f;
+        field[j] = (uint32_t)(int)biased & 31u;
+        if (j == 0) { first = s; first_floor = __builtin_floorf(s); }
+    }
+    lo = field[0] | (field[1] << 5) | (field[2] << 10) | (field[3] << 15) | (field[4] << 20) |
+         (field[5] << 25) | (beta_id << 30);
+    hi = field[6] | (field[7] << 5) | (first != first_floor ? 1024u : 0u);
+    return in_range;
+}
+
+__device__ __forceinline__ void decode_resolved(uint32_t lo, uint32_t hi, uint32_t counter_plus_seed,
+                                                float (&out)[8]) {
+    // (half ? 2^25 : 0) - 15 * 2^26, wrapping like the sums below
+    const uint32_t base = ((hi << 15) & (1u << 25)) - (15u << 26);
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t field = j < 6 ? (lo >> (5 * j)) & 31u : (hi >> (5 * (j - 6))) & 31u;
+        const uint32_t point = (field << 26) + base;                                    // s_j * 2^26
+        const uint32_t uniform = (lcg31_mix_bits(counter_plus_seed + (uint32_t)j) >> 4) & 0x7ffffffu;
+        out[j] = (float)(int32_t)(point - uniform);
+    }
 }
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t bits) {

@@ -35,10 +35,12 @@ constexpr int kGemmBK = 128;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-template <int TILES, bool kHinted>   // token tiles (of 32 rows) per wavefront; decode hints present
+// TILES: token tiles (of 32 rows) per wavefront.  kResolved: the weight comes as resolved
+// blocks (w_words / w_tails, see nq_e8.hip.h) instead of NQRT4 code words and beta bytes.
+template <int TILES, bool kResolved>
 __global__ void __launch_bounds__(kGemmThreads)
 w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
-                 const uint32_t *__restrict__ w_codes, const uint16_t *__restrict__ w_hints,
+                 const uint32_t *__restrict__ w_words, const uint16_t *__restrict__ w_tails,
                  const uint8_t *__restrict__ w_beta_ids,
                  const float *__restrict__ w_norms, const float *__restrict__ w_betas,
                  int m_rows, int k_size, int n_size, int k_slab, uint32_t seed_plus_offset,
@@ -52,7 +54,7 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
     // decode role: channel n0 + tid / 16, block tid % 16 of the current 128-wide step
     const int dec_n = n0 + (tid >> 4), dec_kb = tid & 15;
     const bool dec_live = dec_n < n_size;
-    const float wscale = dec_live ? w_norms[dec_n] / sqrt_k : 0.0f;
+    const float wscale = dec_live ? (kResolved ? (w_norms[dec_n] / sqrt_k) * kResolvedUnit : w_norms[dec_n] / sqrt_k) : 0.0f;
     const float wbeta[4] = {w_betas[0], w_betas[1], w_betas[2], w_betas[3]};
     const int64_t dec_first = (int64_t)(dec_live ? dec_n : 0) * blocks_per_row + (k_begin >> 3) + dec_kb;
     uint4 *dec_slot0 = &b_tile[0][dec_kb >> 1][(tid >> 4) + 32 * (dec_kb & 1)];
@@ -80,13 +82,15 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
             uint4 packed = make_uint4(0, 0, 0, 0);
             if (dec_live) {
                 float v[8];
-                if (kHinted) {
-                    uint32_t hints = w_hints[g];
-                    decode_codeword<true, 1>(w_codes[g], 14.0f, seed_plus_offset + (uint32_t)g * 8u, v, &hints);
+                float scale;
+                const uint32_t word = w_words[g];
+                if (kResolved) {
+                    decode_resolved(word, w_tails[g], seed_plus_offset + (uint32_t)g * 8u, v);
+                    scale = wbeta[word >> 30] * wscale;
                 } else {
-                    decode_codeword<true>(w_codes[g], 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
+                    decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
+                    scale = wbeta[(w_beta_ids[g >> 2] >> (2 * (g & 3))) & 3] * wscale;
                 }
-                const float scale = wbeta[(w_beta_ids[g >> 2] >> (2 * (g & 3))) & 3] * wscale;
                 const bf16x2 h0 = pack_bf16x2(v[0] * scale, v[1] * scale), h1 = pack_bf16x2(v[2] * scale, v[3] * scale);
                 const bf16x2 h2 = pack_bf16x2(v[4] * scale, v[5] * scale), h3 = pack_bf16x2(v[6] * scale, v[7] * scale);
                 packed = make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
@@ -160,7 +164,8 @@ extern "C" size_t nq_w4a4_gemm_workspace_bytes(int m, int k, int n, int split_k,
 extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
                             const float *act_norms_dev, const float *act_betas_dev,
                             const void *act_decoded_dev, const uint8_t *w_codes_dev,
-                            const uint16_t *w_hints_dev, const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
+                            const uint8_t *w_beta_ids_dev, const uint32_t *w_resolved_words_dev,
+                            const uint16_t *w_resolved_tails_dev, const float *w_norms_dev,
                             const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
                             int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
                             void *workspace_dev, size_t workspace_bytes, void *stream) {
@@ -172,12 +177,15 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
                NQ_ERR_ARGUMENT, "nq_w4a4_gemm: split_k must be 0, 1, 2, 4, 8 or 16");
     NQ_REQUIRE(out_dtype == NQ_F32 || out_dtype == NQ_BF16, NQ_ERR_ARGUMENT,
                "nq_w4a4_gemm: output dtype tag %d is not F32 or BF16", out_dtype);
-    NQ_REQUIRE(w_codes_dev && w_beta_ids_dev && w_norms_dev && w_betas_dev && out_dev, NQ_ERR_ARGUMENT,
-               "nq_w4a4_gemm: null pointer");
+    const bool resolved = w_resolved_words_dev != nullptr;
+    NQ_REQUIRE(w_norms_dev && w_betas_dev && out_dev, NQ_ERR_ARGUMENT, "nq_w4a4_gemm: null pointer");
+    NQ_REQUIRE(resolved ? w_resolved_tails_dev != nullptr : (w_codes_dev && w_beta_ids_dev), NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemm: neither packed nor resolved weight streams given");
     NQ_REQUIRE(act_decoded_dev || (act_codes_dev && act_beta_ids_dev && act_norms_dev && act_betas_dev),
                NQ_ERR_ARGUMENT, "nq_w4a4_gemm: neither packed nor decoded activation given");
     NQ_REQUIRE(nq::aligned(w_codes_dev, 4) && (!act_codes_dev || nq::aligned(act_codes_dev, 4)) &&
-                   (!act_decoded_dev || nq::aligned(act_decoded_dev, 16)),
+                   (!act_decoded_dev || nq::aligned(act_decoded_dev, 16)) &&
+                   nq::aligned(w_resolved_words_dev, 4) && nq::aligned(w_resolved_tails_dev, 2),
                NQ_ERR_ARGUMENT, "nq_w4a4_gemm: code streams need 4-byte, decoded activation 16-byte alignment");
     NQ_REQUIRE(weight_seed >= 0 && weight_seed < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
                "nq_w4a4_gemm: seed must be in [0, 2**31)");
@@ -206,7 +214,7 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
     const uint32_t seed_plus_offset = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
     const float sqrt_k = (float)sqrt((double)k);
     const dim3 grid((unsigned)((n + nq::kGemmBN - 1) / nq::kGemmBN), (unsigned)split);
-    const uint32_t *wc = reinterpret_cast<const uint32_t *>(w_codes_dev);
+    const uint32_t *wc = resolved ? w_resolved_words_dev : reinterpret_cast<const uint32_t *>(w_codes_dev);
     const size_t out_row_bytes = (size_t)n * (out_dtype == NQ_F32 ? 4 : 2);
 
     for (int m0 = 0; m0 < m; m0 += kChunkRows) {
@@ -215,15 +223,15 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
         float *target_f32 = split > 1 ? partials : (out_dtype == NQ_F32 ? (float *)out_chunk : nullptr);
         uint16_t *target_bf16 = (split > 1 || out_dtype == NQ_F32) ? nullptr : (uint16_t *)out_chunk;
         const uint16_t *act_chunk = act + (size_t)m0 * k;
-#define NQ_LAUNCH_GEMM(TILES, HINTED)                                                                  \
-    hipLaunchKernelGGL((nq::w4a4_gemm_kernel<TILES, HINTED>), grid, dim3(nq::kGemmThreads), 0, s, act_chunk, \
-                       wc, w_hints_dev, w_beta_ids_dev, w_norms_dev, w_betas_dev, rows, k, n, k / split,      \
-                       seed_plus_offset, sqrt_k, target_f32, target_bf16)
+#define NQ_LAUNCH_GEMM(TILES, RESOLVED)                                                                       \
+    hipLaunchKernelGGL((nq::w4a4_gemm_kernel<TILES, RESOLVED>), grid, dim3(nq::kGemmThreads), 0, s, act_chunk, \
+                       wc, w_resolved_tails_dev, w_beta_ids_dev, w_norms_dev, w_betas_dev, rows, k, n,          \
+                       k / split, seed_plus_offset, sqrt_k, target_f32, target_bf16)
         if (rows <= 8 * 32) {
-            if (w_hints_dev) NQ_LAUNCH_GEMM(1, true);
+            if (resolved) NQ_LAUNCH_GEMM(1, true);
             else NQ_LAUNCH_GEMM(1, false);
         } else {
-            if (w_hints_dev) NQ_LAUNCH_GEMM(2, true);
+            if (resolved) NQ_LAUNCH_GEMM(2, true);
             else NQ_LAUNCH_GEMM(2, false);
         }
 #undef NQ_LAUNCH_GEMM

@@ -14,10 +14,12 @@
 //   * The activation is consumed as decoded BF16 [M, K]: the encoder emits it as a side
 //     product, otherwise a small kernel decodes the NQA4 streams once per call (the
 //     reference re-decodes it in every warp, nestquant/runtime/nqrt4_w4a4_mma.cu:914-925).
-//   * Lanes are combined with a fixed butterfly, wavefronts through LDS in index order, and
-//     K slices by a second kernel in ascending slice order: results are deterministic.
-// The kernel is bound by vector-ALU work (about 600 instructions per 8-weight block, most
-// of it the 31-bit hash and two exact E8 searches), not by the 4.25 bits per weight it reads.
+//   * Lanes are combined in rows of 16 with fixed register exchanges, rows and wavefronts
+//     through LDS in index order, and K slices by a second kernel in ascending slice order:
+//     results are deterministic.
+// The kernel is bound by vector-ALU work, not by the bits it reads: about 600 instructions
+// per 8-weight block from the NQRT4 stream (the 31-bit hash and two exact E8 searches), about
+// 200 from resolved blocks (the hash and little else).
 #include "nq_linear_common.hip.h"
 
 #include <math.h>
@@ -28,77 +30,103 @@ constexpr int kGemvThreads = 256;
 constexpr int kGemvWaves = kGemvThreads / 64;
 constexpr int kGemvMaxRows = 8;
 
-template <int M, bool kHinted>
+// Sum over the 16 lanes of a DPP row, left in every lane of the row: exchanges inside quads,
+// then the mirrored half row, then the mirrored row.
+__device__ __forceinline__ float row16_sum(float v) {
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
+    return v;
+}
+
+// kResolved: the weight comes as resolved blocks (w_words = 32-bit words, w_tails = 16-bit
+// words, see nq_e8.hip.h) instead of NQRT4 code words and beta bytes.
+// R: output channels per workgroup.  A lane decodes block b of all R channels against one
+// load of the M activation blocks, and the R weight loads of a step are issued together.
+template <int M, int R, bool kResolved>
 __global__ void __launch_bounds__(kGemvThreads)
 w4a4_gemv_kernel(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8] blocks
-                 const uint32_t *__restrict__ w_codes, const uint16_t *__restrict__ w_hints,
+                 const uint32_t *__restrict__ w_words, const uint16_t *__restrict__ w_tails,
                  const uint8_t *__restrict__ w_beta_ids,
                  const float *__restrict__ w_norms, const float *__restrict__ w_betas,
-                 int m_rows, int k_size, int n_size, int k_slice, int rows_per_wg,
+                 int m_rows, int k_size, int n_size, int k_slice,
                  uint32_t seed_plus_offset, float sqrt_k, float *__restrict__ out_f32,
                  uint16_t *__restrict__ out_bf16) {
-    __shared__ float partial[kGemvWaves][kGemvMaxRows][M];
+    __shared__ float partial[kGemvWaves * 4][R][M];        // one entry per 16-lane row of every wavefront
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int blocks_per_row = k_size >> 3;
     const int slice_blocks = k_slice >> 3;
     const int slice_first_block = blockIdx.y * slice_blocks;
     const float wbeta[4] = {w_betas[0], w_betas[1], w_betas[2], w_betas[3]};
+    const int n0 = blockIdx.x * R;
 
-    for (int r = 0; r < rows_per_wg; r++) {
-        const int n = blockIdx.x * rows_per_wg + r;
-        float acc[M];
+    float acc[R][M], wscale[R];
+    int64_t row_first_block[R];
 #pragma unroll
-        for (int m = 0; m < M; m++) acc[m] = 0.0f;
-        if (n < n_size) {
-            const float wscale = w_norms[n] / sqrt_k;
-            const int64_t row_first_block = (int64_t)n * blocks_per_row + slice_first_block;
-            for (int b = tid; b < slice_blocks; b += kGemvThreads) {
-                const int64_t g = row_first_block + b;
-                const uint32_t word = w_codes[g];
-                const uint32_t ids = w_beta_ids[g >> 2];
-                // the activation blocks do not depend on the decode: request them first
-                uint4 a[M];
+    for (int r = 0; r < R; r++) {
+        const int n = n0 + r < n_size ? n0 + r : n_size - 1;       // channels past the end repeat the last one
+        const float unit = w_norms[n] / sqrt_k;
+        wscale[r] = kResolved ? unit * kResolvedUnit : unit;
+        row_first_block[r] = (int64_t)n * blocks_per_row + slice_first_block;
 #pragma unroll
-                for (int m = 0; m < M; m++)
-                    a[m] = m < m_rows ? act[(int64_t)m * blocks_per_row + slice_first_block + b] : make_uint4(0, 0, 0, 0);
-                float v[8];
-                if (kHinted) {
-                    uint32_t hints = w_hints[g];
-                    decode_codeword<true, 1>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v, &hints);
-                } else {
-                    decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
-                }
-                const float scale = wbeta[(ids >> (2 * (g & 3))) & 3] * wscale;
-                bf16x2 w[4];
+        for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
+    }
+
+    for (int b = tid; b < slice_blocks; b += kGemvThreads) {
+        uint32_t word[R], side[R];
 #pragma unroll
-                for (int j = 0; j < 4; j++) w[j] = pack_bf16x2(v[2 * j] * scale, v[2 * j + 1] * scale);
+        for (int r = 0; r < R; r++) {
+            const int64_t g = row_first_block[r] + b;
+            word[r] = w_words[g];
+            side[r] = kResolved ? (uint32_t)w_tails[g] : (uint32_t)w_beta_ids[g >> 2];
+        }
+        uint4 a[M];
 #pragma unroll
-                for (int m = 0; m < M; m++) {
-                    acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].x), w[0], acc[m], false);
-                    acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].y), w[1], acc[m], false);
-                    acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].z), w[2], acc[m], false);
-                    acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].w), w[3], acc[m], false);
-                }
+        for (int m = 0; m < M; m++)
+            a[m] = m < m_rows ? act[(int64_t)m * blocks_per_row + slice_first_block + b] : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int64_t g = row_first_block[r] + b;
+            float v[8];
+            float scale;
+            if (kResolved) {
+                decode_resolved(word[r], side[r], seed_plus_offset + (uint32_t)g * 8u, v);
+                scale = wbeta[word[r] >> 30] * wscale[r];
+            } else {
+                decode_codeword<true>(word[r], 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
+                scale = wbeta[(side[r] >> (2 * (g & 3))) & 3] * wscale[r];
+            }
+            bf16x2 w[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) w[j] = pack_bf16x2(v[2 * j] * scale, v[2 * j + 1] * scale);
+#pragma unroll
+            for (int m = 0; m < M; m++) {
+                acc[r][m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].x), w[0], acc[r][m], false);
+                acc[r][m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].y), w[1], acc[r][m], false);
+                acc[r][m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].z), w[2], acc[r][m], false);
+                acc[r][m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].w), w[3], acc[r][m], false);
             }
         }
-        // fixed butterfly over the 64 lanes
+    }
+    // sums over the 16 lanes of every row with register-only lane exchanges (fixed order)
+#pragma unroll
+    for (int r = 0; r < R; r++) {
 #pragma unroll
         for (int m = 0; m < M; m++) {
-            float v = acc[m];
-#pragma unroll
-            for (int offset = 32; offset >= 1; offset >>= 1) v = v + __shfl_xor(v, offset, 64);
-            if (lane == 0) partial[wave][r][m] = v;
+            const float v = row16_sum(acc[r][m]);
+            if ((lane & 15) == 0) partial[tid >> 4][r][m] = v;
         }
     }
     __syncthreads();
-    // wavefront partials in index order
-    if (tid < rows_per_wg * M) {
+    // row partials in index order
+    if (tid < R * M) {
         const int r = tid / M, m = tid - r * M;
-        const int n = blockIdx.x * rows_per_wg + r;
+        const int n = n0 + r;
         if (n < n_size && m < m_rows) {
             float total = partial[0][r][m];
 #pragma unroll
-            for (int w = 1; w < kGemvWaves; w++) total = total + partial[w][r][m];
+            for (int w = 1; w < kGemvWaves * 4; w++) total = total + partial[w][r][m];
             if (out_f32)
                 out_f32[((int64_t)blockIdx.y * m_rows + m) * n_size + n] = total;
             else
@@ -107,52 +135,60 @@ w4a4_gemv_kernel(const uint4 *__restrict__ act,          // decoded BF16 [m_rows
     }
 }
 
-// One lane per weight block: run both exact lattice searches once and keep their outcomes.
+// One lane per weight block: run the exact decode once and keep the lattice point it implies.
 __global__ void __launch_bounds__(256)
-make_decode_hints_kernel(const uint32_t *__restrict__ w_codes, int64_t blocks, uint32_t seed_plus_offset,
-                         uint16_t *__restrict__ hints) {
+resolve_weight_kernel(const uint32_t *__restrict__ w_codes, const uint8_t *__restrict__ w_beta_ids,
+                      int64_t blocks, uint32_t seed_plus_offset, uint32_t *__restrict__ words,
+                      uint16_t *__restrict__ tails, int32_t *__restrict__ out_of_range) {
     const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (g >= blocks) return;
-    float v[8];
-    uint32_t h = 0u;
-    decode_codeword<true, 2>(w_codes[g], 14.0f, seed_plus_offset + (uint32_t)g * 8u, v, &h);
-    hints[g] = (uint16_t)h;
+    const uint32_t beta_id = ((uint32_t)w_beta_ids[g >> 2] >> (2 * (g & 3))) & 3u;
+    uint32_t lo, hi;
+    const bool ok = resolve_codeword(w_codes[g], seed_plus_offset + (uint32_t)g * 8u, beta_id, lo, hi);
+    words[g] = lo;
+    tails[g] = (uint16_t)hi;
+    if (!ok) atomicAdd(out_of_range, 1);
 }
 
 }  // namespace nq
 
-extern "C" int nq_w4a4_make_decode_hints(const uint8_t *w_codes_dev, int64_t rows, int64_t k,
-                                         int64_t weight_offset, int64_t weight_seed, uint16_t *hints_dev,
-                                         void *stream) {
-    NQ_REQUIRE(rows >= 1 && k >= 8 && k % 8 == 0, NQ_ERR_SHAPE,
-               "nq_w4a4_make_decode_hints: rows must be positive and K a positive multiple of 8");
-    NQ_REQUIRE(w_codes_dev && hints_dev && nq::aligned(w_codes_dev, 4) && nq::aligned(hints_dev, 2),
-               NQ_ERR_ARGUMENT, "nq_w4a4_make_decode_hints: null or misaligned pointer");
+extern "C" int nq_w4a4_resolve_weight(const uint8_t *w_codes_dev, const uint8_t *w_beta_ids_dev, int64_t rows,
+                                      int64_t k, int64_t weight_offset, int64_t weight_seed,
+                                      uint32_t *words_dev, uint16_t *tails_dev, int32_t *out_of_range_dev,
+                                      void *stream) {
+    NQ_REQUIRE(rows >= 1 && k >= 32 && k % 32 == 0, NQ_ERR_SHAPE,
+               "nq_w4a4_resolve_weight: rows must be positive and K a positive multiple of 32");
+    NQ_REQUIRE(w_codes_dev && w_beta_ids_dev && words_dev && tails_dev && out_of_range_dev, NQ_ERR_ARGUMENT,
+               "nq_w4a4_resolve_weight: null pointer");
+    NQ_REQUIRE(nq::aligned(w_codes_dev, 4) && nq::aligned(words_dev, 4) && nq::aligned(tails_dev, 2) &&
+                   nq::aligned(out_of_range_dev, 4),
+               NQ_ERR_ARGUMENT, "nq_w4a4_resolve_weight: misaligned pointer");
     NQ_REQUIRE(weight_seed >= 0 && weight_seed < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
-               "nq_w4a4_make_decode_hints: seed must be in [0, 2**31)");
+               "nq_w4a4_resolve_weight: seed must be in [0, 2**31)");
     const int64_t blocks = rows * (k / 8);
     NQ_REQUIRE(weight_offset >= 0 && weight_offset + blocks <= ((int64_t)1 << 28), NQ_ERR_SHAPE,
-               "nq_w4a4_make_decode_hints: block range exceeds the stateless dither counter space");
+               "nq_w4a4_resolve_weight: block range exceeds the stateless dither counter space");
     const uint32_t seed_plus_offset = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
-    hipLaunchKernelGGL(nq::make_decode_hints_kernel, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, reinterpret_cast<const uint32_t *>(w_codes_dev), blocks,
-                       seed_plus_offset, hints_dev);
-    return nq::check_launch("nq_w4a4_make_decode_hints");
+    hipLaunchKernelGGL(nq::resolve_weight_kernel, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, reinterpret_cast<const uint32_t *>(w_codes_dev), w_beta_ids_dev,
+                       blocks, seed_plus_offset, words_dev, tails_dev, out_of_range_dev);
+    return nq::check_launch("nq_w4a4_resolve_weight");
 }
 
 namespace {
 
 int m_tile_of(int m) { return m == 1 ? 1 : (m == 2 ? 2 : (m <= 4 ? 4 : 8)); }
 
-// A workgroup consumes 2048 K-elements per step.  Long-K, narrow-N shapes (down_proj) are
-// split until every SIMD of the 256 CUs has several wavefronts to interleave.
+// A workgroup consumes 2048 K-elements per step.  Only long-K shapes too narrow to give
+// every CU a workgroup are split; the others finish in one kernel.
 int pick_split(int k, int n, int requested) {
     if (requested > 0) return requested;
     int split = 1;
-    while (split < 8 && (k / (split * 2)) % 32 == 0 && (int64_t)n * split < 4096 && k / (split * 2) >= 2048)
+    while (split < 8 && (k / (split * 2)) % 32 == 0 && (int64_t)n * split < 1024 && k / (split * 2) >= 2048)
         split *= 2;
     return split;
 }
+
 
 }  // namespace
 
@@ -168,7 +204,8 @@ extern "C" size_t nq_w4a4_gemv_workspace_bytes(int m, int k, int n, int split_k,
 extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
                             const float *act_norms_dev, const float *act_betas_dev,
                             const void *act_decoded_dev, const uint8_t *w_codes_dev,
-                            const uint16_t *w_hints_dev, const uint8_t *w_beta_ids_dev, const float *w_norms_dev,
+                            const uint8_t *w_beta_ids_dev, const uint32_t *w_resolved_words_dev,
+                            const uint16_t *w_resolved_tails_dev, const float *w_norms_dev,
                             const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
                             int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
                             void *workspace_dev, size_t workspace_bytes, void *stream) {
@@ -179,12 +216,15 @@ extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_bet
                NQ_ERR_ARGUMENT, "nq_w4a4_gemv: split_k must be 0, 1, 2, 4 or 8");
     NQ_REQUIRE(out_dtype == NQ_F32 || out_dtype == NQ_BF16, NQ_ERR_ARGUMENT,
                "nq_w4a4_gemv: output dtype tag %d is not F32 or BF16", out_dtype);
-    NQ_REQUIRE(w_codes_dev && w_beta_ids_dev && w_norms_dev && w_betas_dev && out_dev, NQ_ERR_ARGUMENT,
-               "nq_w4a4_gemv: null pointer");
+    const bool resolved = w_resolved_words_dev != nullptr;
+    NQ_REQUIRE(w_norms_dev && w_betas_dev && out_dev, NQ_ERR_ARGUMENT, "nq_w4a4_gemv: null pointer");
+    NQ_REQUIRE(resolved ? w_resolved_tails_dev != nullptr : (w_codes_dev && w_beta_ids_dev), NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemv: neither packed nor resolved weight streams given");
     NQ_REQUIRE(act_decoded_dev || (act_codes_dev && act_beta_ids_dev && act_norms_dev && act_betas_dev),
                NQ_ERR_ARGUMENT, "nq_w4a4_gemv: neither packed nor decoded activation given");
     NQ_REQUIRE(nq::aligned(w_codes_dev, 4) && (!act_codes_dev || nq::aligned(act_codes_dev, 4)) &&
-                   (!act_decoded_dev || nq::aligned(act_decoded_dev, 16)) && nq::aligned(w_hints_dev, 2),
+                   (!act_decoded_dev || nq::aligned(act_decoded_dev, 16)) &&
+                   nq::aligned(w_resolved_words_dev, 4) && nq::aligned(w_resolved_tails_dev, 2),
                NQ_ERR_ARGUMENT, "nq_w4a4_gemv: code streams need 4-byte, decoded activation 16-byte alignment");
     NQ_REQUIRE(weight_seed >= 0 && weight_seed < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
                "nq_w4a4_gemv: seed must be in [0, 2**31)");
@@ -213,20 +253,21 @@ extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_bet
 
     const int k_slice = k / split;
     // few rows per workgroup keeps many short wavefronts in flight on every SIMD
-    const int rows_per_wg = (int64_t)n * split >= 8192 ? 4 : 2;
+    const int rows_per_wg = (resolved && (int64_t)n * split >= 8192) ? 4 : 2;
     const dim3 grid((unsigned)((n + rows_per_wg - 1) / rows_per_wg), (unsigned)split);
     const uint32_t seed_plus_offset = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
     float *target_f32 = split > 1 ? partials : (out_dtype == NQ_F32 ? (float *)out_dev : nullptr);
     uint16_t *target_bf16 = (split > 1 || out_dtype == NQ_F32) ? nullptr : (uint16_t *)out_dev;
-    const uint32_t *wc = reinterpret_cast<const uint32_t *>(w_codes_dev);
-#define NQ_LAUNCH_GEMV_AS(MT, HINTED)                                                               \
-    hipLaunchKernelGGL((nq::w4a4_gemv_kernel<MT, HINTED>), grid, dim3(nq::kGemvThreads), 0, s, act, \
-                       wc, w_hints_dev, w_beta_ids_dev, w_norms_dev, w_betas_dev, m, k, n, k_slice, \
-                       rows_per_wg, seed_plus_offset, sqrt_k, target_f32, target_bf16)
+    const uint32_t *wc = resolved ? w_resolved_words_dev : reinterpret_cast<const uint32_t *>(w_codes_dev);
+#define NQ_LAUNCH_GEMV_AS(MT, ROWS, RESOLVED)                                                       \
+    hipLaunchKernelGGL((nq::w4a4_gemv_kernel<MT, ROWS, RESOLVED>), grid, dim3(nq::kGemvThreads), 0, \
+                       s, act, wc, w_resolved_tails_dev, w_beta_ids_dev, w_norms_dev, w_betas_dev,  \
+                       m, k, n, k_slice, seed_plus_offset, sqrt_k, target_f32, target_bf16)
 #define NQ_LAUNCH_GEMV(MT)                                                                          \
     do {                                                                                            \
-        if (w_hints_dev) NQ_LAUNCH_GEMV_AS(MT, true);                                               \
-        else NQ_LAUNCH_GEMV_AS(MT, false);                                                          \
+        if (!resolved) NQ_LAUNCH_GEMV_AS(MT, 2, false);                                             \
+        else if (rows_per_wg == 4) NQ_LAUNCH_GEMV_AS(MT, 4, true);                                  \
+        else NQ_LAUNCH_GEMV_AS(MT, 2, true);                                                        \
     } while (0)
     switch (m_tile_of(m)) {
         case 1: NQ_LAUNCH_GEMV(1); break;

@@ -67,9 +67,11 @@ class PreparedNQRTLinear:
     beta_payload: torch.Tensor
     row_norms: torch.Tensor
     beta_table: torch.Tensor
-    # Optional uint16 per 8-weight block: the outcomes of the two lattice searches of the
-    # block's decode, computed once here so the linear kernels need not search (same results).
-    decode_hints: torch.Tensor | None = None
+    # Optional resolved form (int32 word + int16 tail per 8-weight block): the lattice point
+    # each block's decode lands on, found once here so that the linear kernels need neither
+    # lattice search.  6 bits per weight on top of (or instead of) the 4.25-bit streams.
+    resolved_words: torch.Tensor | None = None
+    resolved_tails: torch.Tensor | None = None
 
 
 # --------------------------------------------------------------------------------------
@@ -192,20 +194,27 @@ def _payload_tensor(payload: bytes, device: torch.device) -> torch.Tensor:
     return torch.frombuffer(bytearray(payload), dtype=torch.uint8).to(device)
 
 
-def make_decode_hints(code_payload: torch.Tensor, *, rows: int, features: int, dither_seed: int,
-                      block_offset: int = 0) -> torch.Tensor:
+def resolve_weight(code_payload: torch.Tensor, beta_payload: torch.Tensor, *, rows: int, features: int,
+                   dither_seed: int, block_offset: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
+    """Resolved form of an NQRT4 weight: (int32 words, int16 tails), one of each per E8 block."""
     device = _native.require_cuda(code_payload)
-    hints = torch.empty(rows * features // 8, dtype=torch.int16, device=device)
-    _native.check(_native.library().nq_w4a4_make_decode_hints(
-        code_payload.data_ptr(), rows, features, block_offset, int(dither_seed), hints.data_ptr(),
-        _native.stream_handle(device)))
-    return hints
+    blocks = rows * features // 8
+    words = torch.empty(blocks, dtype=torch.int32, device=device)
+    tails = torch.empty(blocks, dtype=torch.int16, device=device)
+    out_of_range = torch.zeros(1, dtype=torch.int32, device=device)
+    _native.check(_native.library().nq_w4a4_resolve_weight(
+        code_payload.data_ptr(), beta_payload.data_ptr(), rows, features, block_offset, int(dither_seed),
+        words.data_ptr(), tails.data_ptr(), out_of_range.data_ptr(), _native.stream_handle(device)))
+    bad = int(out_of_range.item())
+    if bad:
+        raise ValueError(f"{bad} weight blocks decode outside the range of the resolved form")
+    return words, tails
 
 
 def prepare_fused_linear(record: Any, *, device: torch.device | str = "cuda",
-                         decode_hints: bool = True) -> PreparedNQRTLinear:
+                         resolve: bool = True) -> PreparedNQRTLinear:
     """Copy only the packed NQRT streams and compact metadata to the target GPU, and (unless
-    `decode_hints=False`) derive the 2-byte-per-block decode hints from them."""
+    `resolve=False`) derive the resolved form of the weight from them."""
     for attribute in ("indices", "row_norms", "betas", "feature_count", "dither_seed",
                       "dither_algorithm", "codec_semantics"):
         if not hasattr(record, attribute):
@@ -218,17 +227,20 @@ def prepare_fused_linear(record: Any, *, device: torch.device | str = "cuda",
     if record.codec_semantics != UPSTREAM_CODEC_SEMANTICS:
         raise ValueError("fused Linear requires upstream E8 semantics")
     codes = _payload_tensor(record.indices.code_payload, target)
-    hints = None
-    if decode_hints and record.indices.q == 14 and record.indices.code_bit_width == 4:
-        hints = make_decode_hints(codes, rows=record.indices.shape[0], features=record.feature_count,
-                                  dither_seed=record.dither_seed)
+    beta_ids = _payload_tensor(record.indices.beta_payload, target)
+    words = tails = None
+    if (resolve and record.indices.q == 14 and record.indices.code_bit_width == 4
+            and record.feature_count % 32 == 0 and len(record.betas) == 4):
+        words, tails = resolve_weight(codes, beta_ids, rows=record.indices.shape[0],
+                                      features=record.feature_count, dither_seed=record.dither_seed)
     return PreparedNQRTLinear(
         record=record,
         code_payload=codes,
-        beta_payload=_payload_tensor(record.indices.beta_payload, target),
+        beta_payload=beta_ids,
         row_norms=record.row_norms.to(device=target, dtype=torch.float32),
         beta_table=torch.tensor(record.betas, device=target, dtype=torch.float32),
-        decode_hints=hints,
+        resolved_words=words,
+        resolved_tails=tails,
     )
 
 
@@ -346,7 +358,9 @@ def _gemv(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *, spl
         activation.code_payload.data_ptr(), activation.beta_payload.data_ptr(),
         activation.row_norms.data_ptr(), activation.beta_table.data_ptr(),
         None if decoded is None else decoded.data_ptr(), weight.code_payload.data_ptr(),
-        None if weight.decode_hints is None else weight.decode_hints.data_ptr(), weight.beta_payload.data_ptr(),
+        weight.beta_payload.data_ptr(),
+        None if weight.resolved_words is None else weight.resolved_words.data_ptr(),
+        None if weight.resolved_tails is None else weight.resolved_tails.data_ptr(),
         weight.row_norms.data_ptr(), weight.beta_table.data_ptr(), m, k, n, 0,
         int(weight.record.dither_seed), split_k, out.data_ptr(), _native.dtype_tag(output_dtype),
         None if workspace is None else workspace.data_ptr(), need, _native.stream_handle(device)))

@@ -38,7 +38,7 @@ def test_host_side_validation_needs_no_gpu():
     assert status == _native.NQ_ERR_SHAPE and b"multiple of 32" in lib.nq_last_error()
     with pytest.raises(ValueError, match="multiple of 32"):
         _native.check(status)
-    status = lib.nq_w4a4_gemv(*([None] * 10), 9, 2048, 2048, 0, 1, 0, None, 0, None, 0, None)
+    status = lib.nq_w4a4_gemv(*([None] * 11), 9, 2048, 2048, 0, 1, 0, None, 0, None, 0, None)
     assert status == _native.NQ_ERR_SHAPE and b"outside [1, 8]" in lib.nq_last_error()
     status = lib.nq_dequantize_rows(None, None, None, None, 1, 64, 14, 1, -5, 0, None, 0, None)
     assert status == _native.NQ_ERR_ARGUMENT
