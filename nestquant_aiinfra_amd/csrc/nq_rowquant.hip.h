@@ -31,24 +31,47 @@ __device__ __forceinline__ float round_to_dtype(float x, int dtype) {
     return x;
 }
 
+// S butterfly stages (pair distances 2^log_w .. 2^(log_w + S - 1)) on 2^S values held in
+// registers: one LDS round trip per pass instead of one per stage.  `total` counts all staged
+// values; groups never straddle rows because n is a power of two.
+template <int S>
+__device__ __forceinline__ void hadamard_pass(float *rows, int total, int log_w, int stage_dtype) {
+    constexpr int kValues = 1 << S;
+    const int groups = total >> S;
+    for (int t = threadIdx.x; t < groups; t += blockDim.x) {
+        const int base = ((t >> log_w) << (log_w + S)) + (t & ((1 << log_w) - 1));
+        float v[kValues];
+#pragma unroll
+        for (int j = 0; j < kValues; j++) v[j] = rows[base + (j << log_w)];
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+#pragma unroll
+            for (int j = 0; j < kValues; j++) {
+                if (j & (1 << s)) continue;
+                const float left = v[j], right = v[j + (1 << s)];
+                v[j] = round_to_dtype(left + right, stage_dtype);
+                v[j + (1 << s)] = round_to_dtype(left - right, stage_dtype);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kValues; j++) rows[base + (j << log_w)] = v[j];
+    }
+    __syncthreads();
+}
+
 // Normalized Sylvester-Hadamard transform of rows staged in LDS (nestquant/core/rotation.py:12-27):
 // butterflies of growing width, each sum and difference rounded to `stage_dtype` (the dtype
 // the reference's tensor ops would run in), then one multiplication by float32(1 / sqrt(n))
 // -- the form a tensor / python-scalar division takes on the GPU.  Ends with a barrier.
 __device__ __forceinline__ void staged_hadamard(float *rows, int row_count, int n, int stage_dtype) {
-    const int half = n >> 1;
-    for (int width = 1; width < n; width <<= 1) {
-        for (int i = threadIdx.x; i < row_count * half; i += blockDim.x) {
-            const int r = i / half, k = i - r * half;
-            const int a = r * n + (k / width) * 2 * width + (k % width), b = a + width;
-            const float left = rows[a], right = rows[b];
-            rows[a] = round_to_dtype(left + right, stage_dtype);
-            rows[b] = round_to_dtype(left - right, stage_dtype);
-        }
-        __syncthreads();
-    }
+    const int log_n = 31 - __builtin_clz(n);
+    const int total = row_count * n;
+    int log_w = 0;
+    for (; log_n - log_w >= 3; log_w += 3) hadamard_pass<3>(rows, total, log_w, stage_dtype);
+    if (log_n - log_w == 2) hadamard_pass<2>(rows, total, log_w, stage_dtype);
+    if (log_n - log_w == 1) hadamard_pass<1>(rows, total, log_w, stage_dtype);
     const float inv = 1.0f / __builtin_sqrtf((float)n);
-    for (int i = threadIdx.x; i < row_count * n; i += blockDim.x) rows[i] = round_to_dtype(rows[i] * inv, stage_dtype);
+    for (int i = threadIdx.x; i < total; i += blockDim.x) rows[i] = round_to_dtype(rows[i] * inv, stage_dtype);
     __syncthreads();
 }
 
