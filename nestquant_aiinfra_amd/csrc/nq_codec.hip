@@ -278,11 +278,14 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
     // lanes so that the whole chip encodes it; beta bytes need 16-pair alignment
     int slices = 1;
     if (rows_per_wg == 1 && pairs_per_row > 256) {
-        const int64_t wanted = 1024 / rows;                 // about four workgroups per CU in total
+        // long rows keep 1024 lanes for staging, rotation and the norm; about two such
+        // workgroups (or four of 256 lanes) per CU in total
+        const int sliced_threads = n >= 4096 ? 1024 : 256;
+        const int64_t wanted = (sliced_threads == 1024 ? 512 : 1024) / rows;
         while (slices * 2 <= wanted && pairs_per_row / (slices * 2) >= 256 &&
                pairs_per_row % (slices * 2 * 16) == 0)
             slices *= 2;
-        if (slices > 1) threads = 256;
+        if (slices > 1) threads = sliced_threads;
     }
     if (threads < 64) threads = 64;
     const size_t lds_bytes = ((size_t)rows_per_wg * n + 2 * rows_per_wg) * sizeof(float);

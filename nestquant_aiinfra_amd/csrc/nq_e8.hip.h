@@ -286,6 +286,14 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float x) {
     return (uint16_t)(bits >> 16);
 }
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ bf16x2 pack_bf16x2(float lo, float hi) {
+    const floatx2 v = {lo, hi};
+    return __builtin_convertvector(v, bf16x2);          // v_cvt_pk_bf16_f32, round to nearest even
+}
+
 __device__ __forceinline__ float f16_to_f32(uint16_t bits) {
     return (float)__builtin_bit_cast(_Float16, bits);
 }

@@ -6,13 +6,6 @@
 
 namespace nq {
 
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float floatx2 __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ bf16x2 pack_bf16x2(float lo, float hi) {
-    const floatx2 v = {lo, hi};
-    return __builtin_convertvector(v, bf16x2);          // v_cvt_pk_bf16_f32, round to nearest even
-}
 
 // NQA4 streams -> BF16 [M, K], exactly bf16((decode * beta) * (norm / sqrt(K)))
 static __global__ void __launch_bounds__(256)

@@ -34,8 +34,21 @@ __device__ __forceinline__ float round_to_dtype(float x, int dtype) {
 // S butterfly stages (pair distances 2^log_w .. 2^(log_w + S - 1)) on 2^S values held in
 // registers: one LDS round trip per pass instead of one per stage.  `total` counts all staged
 // values; groups never straddle rows because n is a power of two.
-template <int S>
-__device__ __forceinline__ void hadamard_pass(float *rows, int total, int log_w, int stage_dtype) {
+// Both values rounded to the storage dtype kDtype (tags as above), kept as float32.
+template <int kDtype>
+__device__ __forceinline__ void round_pair(float &a, float &b) {
+    if (kDtype == 1) {
+        const uint32_t packed = __builtin_bit_cast(uint32_t, pack_bf16x2(a, b));
+        a = __uint_as_float(packed << 16);
+        b = __uint_as_float(packed & 0xffff0000u);
+    } else if (kDtype == 2) {
+        a = (float)(_Float16)a;
+        b = (float)(_Float16)b;
+    }
+}
+
+template <int S, int kDtype>
+__device__ __forceinline__ void hadamard_pass(float *rows, int total, int log_w) {
     constexpr int kValues = 1 << S;
     const int groups = total >> S;
     for (int t = threadIdx.x; t < groups; t += blockDim.x) {
@@ -49,8 +62,9 @@ __device__ __forceinline__ void hadamard_pass(float *rows, int total, int log_w,
             for (int j = 0; j < kValues; j++) {
                 if (j & (1 << s)) continue;
                 const float left = v[j], right = v[j + (1 << s)];
-                v[j] = round_to_dtype(left + right, stage_dtype);
-                v[j + (1 << s)] = round_to_dtype(left - right, stage_dtype);
+                v[j] = left + right;
+                v[j + (1 << s)] = left - right;
+                round_pair<kDtype>(v[j], v[j + (1 << s)]);
             }
         }
 #pragma unroll
@@ -63,16 +77,28 @@ __device__ __forceinline__ void hadamard_pass(float *rows, int total, int log_w,
 // butterflies of growing width, each sum and difference rounded to `stage_dtype` (the dtype
 // the reference's tensor ops would run in), then one multiplication by float32(1 / sqrt(n))
 // -- the form a tensor / python-scalar division takes on the GPU.  Ends with a barrier.
-__device__ __forceinline__ void staged_hadamard(float *rows, int row_count, int n, int stage_dtype) {
+template <int kDtype>
+__device__ __forceinline__ void staged_hadamard_as(float *rows, int row_count, int n) {
     const int log_n = 31 - __builtin_clz(n);
     const int total = row_count * n;
     int log_w = 0;
-    for (; log_n - log_w >= 3; log_w += 3) hadamard_pass<3>(rows, total, log_w, stage_dtype);
-    if (log_n - log_w == 2) hadamard_pass<2>(rows, total, log_w, stage_dtype);
-    if (log_n - log_w == 1) hadamard_pass<1>(rows, total, log_w, stage_dtype);
+    for (; log_n - log_w >= 3; log_w += 3) hadamard_pass<3, kDtype>(rows, total, log_w);
+    if (log_n - log_w == 2) hadamard_pass<2, kDtype>(rows, total, log_w);
+    if (log_n - log_w == 1) hadamard_pass<1, kDtype>(rows, total, log_w);
     const float inv = 1.0f / __builtin_sqrtf((float)n);
-    for (int i = threadIdx.x; i < total; i += blockDim.x) rows[i] = round_to_dtype(rows[i] * inv, stage_dtype);
+    for (int i = 2 * threadIdx.x; i < total; i += 2 * blockDim.x) {
+        float a = rows[i] * inv, b = rows[i + 1] * inv;
+        round_pair<kDtype>(a, b);
+        rows[i] = a;
+        rows[i + 1] = b;
+    }
     __syncthreads();
+}
+
+__device__ __forceinline__ void staged_hadamard(float *rows, int row_count, int n, int stage_dtype) {
+    if (stage_dtype == 1) staged_hadamard_as<1>(rows, row_count, n);
+    else if (stage_dtype == 2) staged_hadamard_as<2>(rows, row_count, n);
+    else staged_hadamard_as<0>(rows, row_count, n);
 }
 
 // rows: [row_count][n] float32 in LDS, n a multiple of 32.  Writes row_scale[r] =
