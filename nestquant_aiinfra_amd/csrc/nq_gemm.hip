@@ -12,9 +12,10 @@
 //     (lane l of K-step s holds channel l % 32, k = 16 s + 8 (l / 32) .. + 8).  An E8 block
 //     is exactly one lane's fragment, so decoded weights never need a transpose.
 //   * multiply: wavefront w owns token tiles w, w + 8, ... of 32 rows; per K-step it reads
-//     the B fragment from LDS (one ds_read_b128) and its A fragments straight from the
-//     activation in global memory (L2-resident; 16 bytes per lane).
-//   * the weight tile is double-buffered in LDS: one barrier per 128-wide step.
+//     the B fragment from LDS (one ds_read_b128) and takes its A fragments from registers
+//     filled one trip earlier straight from the activation in global memory (L2-resident).
+//   * the weight tile is double-buffered in LDS and the loop is software-pipelined: a trip
+//     multiplies the previous step while it decodes the current one, with one barrier.
 // Every weight block is decoded exactly once per call, whatever M is: the kernel is bound
 // by the decode's vector-ALU work, and the matrix cores run in its shadow.
 // M is padded up to a multiple of 32 with zero rows inside the kernel (masked loads and
@@ -51,66 +52,92 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
     const int k_begin = blockIdx.y * k_slab;
     const int blocks_per_row = k_size >> 3;
 
-    // decode role: channel n0 + tid / 16, block tid % 16 of the current 128-wide step
-    const int dec_n = n0 + (tid >> 4), dec_kb = tid & 15;
-    const bool dec_live = dec_n < n_size;
-    const float wscale = dec_live ? (kResolved ? (w_norms[dec_n] / sqrt_k) * kResolvedUnit : w_norms[dec_n] / sqrt_k) : 0.0f;
+    // decode role: channel n0 + tid / 16, block tid % 16 of the current 128-wide step.
+    // Channels past the end repeat the last one; their results are never stored.
+    const int dec_n = n0 + (tid >> 4) < n_size ? n0 + (tid >> 4) : n_size - 1, dec_kb = tid & 15;
+    const float unit = w_norms[dec_n] / sqrt_k;
+    const float wscale = kResolved ? unit * kResolvedUnit : unit;
     const float wbeta[4] = {w_betas[0], w_betas[1], w_betas[2], w_betas[3]};
-    const int64_t dec_first = (int64_t)(dec_live ? dec_n : 0) * blocks_per_row + (k_begin >> 3) + dec_kb;
-    uint4 *dec_slot0 = &b_tile[0][dec_kb >> 1][(tid >> 4) + 32 * (dec_kb & 1)];
-    uint4 *dec_slot1 = &b_tile[1][dec_kb >> 1][(tid >> 4) + 32 * (dec_kb & 1)];
+    const int64_t dec_first = (int64_t)dec_n * blocks_per_row + (k_begin >> 3) + dec_kb;
+    // LDS entry of (K-step kk, fragment lane f): [kk][f ^ (4 kk)] -- the rotation spreads the
+    // 16 blocks a channel's lanes write over the banks, and is a permutation for the readers
+    const int dec_kk = dec_kb >> 1;
+    const int dec_entry = (((tid >> 4) ^ (dec_kk << 2)) & 31) + 32 * (dec_kb & 1);
+    uint4 *dec_slot0 = &b_tile[0][dec_kk][dec_entry];
+    uint4 *dec_slot1 = &b_tile[1][dec_kk][dec_entry];
 
-    // multiply role: A fragment rows of this lane, one per owned tile
+    // multiply role: A fragment rows of this lane, one per owned tile (rows past the end
+    // repeat the last one; their results are never stored)
     const uint16_t *a_row[TILES];
-    bool a_live[TILES];
 #pragma unroll
     for (int t = 0; t < TILES; t++) {
         const int m = (wave + t * kGemmWaves) * 32 + (lane & 31);
-        a_live[t] = m < m_rows;
-        a_row[t] = act + (int64_t)(a_live[t] ? m : 0) * k_size + k_begin + 8 * (lane >> 5);
+        a_row[t] = act + (int64_t)(m < m_rows ? m : m_rows - 1) * k_size + k_begin + 8 * (lane >> 5);
     }
+    const bool multiplies = wave * 32 < m_rows;
     floatx16 acc[TILES];
 #pragma unroll
     for (int t = 0; t < TILES; t++)
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[t][i] = 0.0f;
 
+    // Software pipeline, one barrier per trip: trip s multiplies step s - 1 (weights from
+    // LDS, activation fragments requested one trip earlier) while it decodes step s, and
+    // requests the code words of step s + 1 and the fragments of step s.
     const int steps = k_slab / kGemmBK;
-    for (int s = 0; s < steps; s++) {
-        {
-            const int64_t g = dec_first + (int64_t)s * (kGemmBK / 8);
-            uint4 packed = make_uint4(0, 0, 0, 0);
-            if (dec_live) {
-                float v[8];
-                float scale;
-                const uint32_t word = w_words[g];
-                if (kResolved) {
-                    decode_resolved(word, w_tails[g], seed_plus_offset + (uint32_t)g * 8u, v);
-                    scale = wbeta[word >> 30] * wscale;
-                } else {
-                    decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
-                    scale = wbeta[(w_beta_ids[g >> 2] >> (2 * (g & 3))) & 3] * wscale;
-                }
-                const bf16x2 h0 = pack_bf16x2(v[0] * scale, v[1] * scale), h1 = pack_bf16x2(v[2] * scale, v[3] * scale);
-                const bf16x2 h2 = pack_bf16x2(v[4] * scale, v[5] * scale), h3 = pack_bf16x2(v[6] * scale, v[7] * scale);
-                packed = make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
-                                    __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
-            }
-            *((s & 1) ? dec_slot1 : dec_slot0) = packed;
+    uint32_t word_next = w_words[dec_first];
+    uint32_t side_next = kResolved ? (uint32_t)w_tails[dec_first] : (uint32_t)w_beta_ids[dec_first >> 2];
+    uint4 a_next[TILES][kGemmBK / 16];
+#pragma unroll
+    for (int t = 0; t < TILES; t++)
+#pragma unroll
+        for (int kk = 0; kk < kGemmBK / 16; kk++) a_next[t][kk] = make_uint4(0, 0, 0, 0);
+
+    for (int s = 0; s <= steps; s++) {
+        const uint32_t word = word_next, side = side_next;
+        uint4 a_now[TILES][kGemmBK / 16];
+#pragma unroll
+        for (int t = 0; t < TILES; t++)
+#pragma unroll
+            for (int kk = 0; kk < kGemmBK / 16; kk++) a_now[t][kk] = a_next[t][kk];
+        const int64_t g = dec_first + (int64_t)s * (kGemmBK / 8);
+        if (s + 1 < steps) {
+            word_next = w_words[g + kGemmBK / 8];
+            side_next = kResolved ? (uint32_t)w_tails[g + kGemmBK / 8] : (uint32_t)w_beta_ids[(g + kGemmBK / 8) >> 2];
         }
-        __syncthreads();
-        if (wave * 32 < m_rows) {
+        if (s < steps && multiplies) {
+#pragma unroll
+            for (int t = 0; t < TILES; t++)
+#pragma unroll
+                for (int kk = 0; kk < kGemmBK / 16; kk++)
+                    a_next[t][kk] = *reinterpret_cast<const uint4 *>(a_row[t] + s * kGemmBK + kk * 16);
+        }
+        if (s > 0 && multiplies) {
 #pragma unroll
             for (int kk = 0; kk < kGemmBK / 16; kk++) {
-                const bf16x8 b = __builtin_bit_cast(bf16x8, b_tile[s & 1][kk][lane]);
+                const bf16x8 b = __builtin_bit_cast(bf16x8, b_tile[(s - 1) & 1][kk][lane ^ (kk << 2)]);
 #pragma unroll
-                for (int t = 0; t < TILES; t++) {
-                    uint4 raw = make_uint4(0, 0, 0, 0);
-                    if (a_live[t]) raw = *reinterpret_cast<const uint4 *>(a_row[t] + s * kGemmBK + kk * 16);
-                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), b, acc[t], 0, 0, 0);
-                }
+                for (int t = 0; t < TILES; t++)
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[t][kk]), b, acc[t], 0, 0, 0);
             }
         }
+        if (s < steps) {
+            float v[8];
+            float scale;
+            if (kResolved) {
+                decode_resolved(word, side, seed_plus_offset + (uint32_t)g * 8u, v);
+                scale = wbeta[word >> 30] * wscale;
+            } else {
+                decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
+                scale = wbeta[(side >> (2 * (g & 3))) & 3] * wscale;
+            }
+            const bf16x2 h0 = pack_bf16x2(v[0] * scale, v[1] * scale), h1 = pack_bf16x2(v[2] * scale, v[3] * scale);
+            const bf16x2 h2 = pack_bf16x2(v[4] * scale, v[5] * scale), h3 = pack_bf16x2(v[6] * scale, v[7] * scale);
+            *((s & 1) ? dec_slot1 : dec_slot0) =
+                make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
+                           __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
+        }
+        __syncthreads();
     }
 
     // accumulator register r of lane l holds token row (r % 4) + 8 * (r / 4) + 4 * (l / 32)
