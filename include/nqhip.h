@@ -81,6 +81,28 @@ int nq_quantize_rows(const void *x_dev, int x_dtype, int64_t rows, int64_t n, in
                      float *norms_dev, void *decoded_bf16_dev, void *stream);
 
 /*
+ * One launch for everything between two Linear layers of a Llama block and the packed
+ * activation the next Linear consumes: an element-wise stage on BF16 rows [rows, n], then
+ * (when codes_dev is given) the rotate + norm + encode + pack of nq_quantize_rows.
+ *   mode 1  h = x + residual (residual_dev may be NULL: h = x); residual_out_dev (optional)
+ *           receives h; y = norm_weight * bf16(h * rsqrt(mean(h^2) + eps))  -- the residual
+ *           add and LlamaRMSNorm in front of q/k/v_proj and gate/up_proj
+ *   mode 2  y = bf16(silu(gate)) * x  -- the SwiGLU product in front of down_proj
+ * Every tensor-level result is rounded to BF16 as the BF16 tensor operations it replaces do.
+ * staged_out_dev (optional) receives y as BF16 [rows, n].  With codes_dev == NULL only the
+ * element-wise stage runs (the final norm in front of the LM head).
+ * Replaces (decode step): the residual adds, LlamaRMSNorm / SiLU-and-multiply tensor
+ * operations of the model code and the input stage of FusedNQRTLinear.forward,
+ * nestquant/models/fused_linear.py:287-306.
+ */
+int nq_fused_input_stage(const void *x_dev, int64_t rows, int64_t n, int mode,
+                         const void *residual_dev, void *residual_out_dev,
+                         const void *norm_weight_dev, float eps, const void *gate_dev,
+                         void *staged_out_dev, int q, const float *betas_dev, int beta_count,
+                         int hadamard, uint8_t *codes_dev, uint8_t *beta_ids_dev, float *norms_dev,
+                         void *decoded_bf16_dev, void *stream);
+
+/*
  * Normalized Sylvester-Hadamard transform of `rows` rows of power-of-two length n, with the
  * reference's butterfly order (widths 1, 2, 4, ...), every sum and difference rounded to
  * stage_dtype (NQ_F32 = no intermediate rounding) and a final multiplication by
@@ -166,6 +188,21 @@ int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
 size_t nq_w4a4_gemv_workspace_bytes(int m, int k, int n, int split_k, int have_decoded_activation);
 
 /*
+ * nq_w4a4_gemv for `count` (1..4) weights that share one activation (q/k/v_proj, gate/up_proj)
+ * in a single launch.  Every array argument is a host array of `count` entries; weights are
+ * given in resolved form (nq_w4a4_resolve_weight) and the activation as its decoded BF16
+ * [M, K] rows; out_dev[i] receives [M, n[i]] of out_dtype.  No split-K, no workspace.
+ * Results equal those of `count` nq_w4a4_gemv calls with split_k = 1 bit for bit.
+ * No counterpart in the reference, which launches once per projection
+ * (nestquant/models/fused_linear.py:316-407).
+ */
+int nq_w4a4_gemv_grouped(const void *act_decoded_dev, int count, const uint32_t *const *w_resolved_words_dev,
+                         const uint16_t *const *w_resolved_tails_dev, const float *const *w_norms_dev,
+                         const float *const *w_betas_dev, const int *n, const int64_t *weight_offsets,
+                         const int64_t *weight_seeds, void *const *out_dev, int m, int k, int out_dtype,
+                         void *stream);
+
+/*
  * Packed W4A4 linear for prefill, any M >= 1 (meant for M >= 9): same product and same
  * arguments as nq_w4a4_gemv, computed on the matrix cores (v_mfma_f32_32x32x16_bf16).  The
  * weight tile is decoded once per call into double-buffered LDS as MFMA B fragments; ragged
@@ -220,6 +257,9 @@ int nq_nqkv_advance(const int32_t *slot_ids_dev, const uint8_t *active_mask_dev,
  * rotate_keys != 0 first applies the normalized Hadamard transform over head_dim to the new
  * key rows (float32 butterflies, result rounded to BF16), i.e. the caller passes post-RoPE
  * keys and need not launch nq_hadamard.
+ * rope_cos_dev / rope_sin_dev (optional, both or neither): BF16 [batch, tokens, head_dim]
+ * rotary tables; the new key rows then arrive pre-RoPE and (k * cos) + (rotate_half(k) * sin)
+ * is applied first, in BF16 tensor arithmetic (every product and the sum rounded to BF16).
  * Requires head_dim = 64, page_size = 16, q = 14, equal beta counts.
  * Replaces: append_hot_k1_graph_safe / ragged sub-page and segment writers
  * (nestquant/runtime/nqkv_graph_writer.py:263-473), launch_pack_full_hot_pages_graph_safe
@@ -234,7 +274,7 @@ int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_dtype, cons
                   const float *key_betas_dev, int key_beta_count, const float *value_betas_dev,
                   int value_beta_count, void *hot_keys_dev, void *hot_values_dev, int batch, int tokens,
                   int slots, int max_pages, int kv_heads, int head_dim, int page_size, int rotate_keys,
-                  void *stream);
+                  const void *rope_cos_dev, const void *rope_sin_dev, void *stream);
 
 /*
  * Paged NQKV4 decode attention for a ragged batch: for batch row r with slot s (clamped to
@@ -245,7 +285,9 @@ int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_dtype, cons
  * online-softmax in two stages; rows that are not live or have no tokens give zeros.
  * query / out: [batch, q_heads, head_dim] of query_dtype; rotate_query != 0 applies the
  * normalized Hadamard transform over head_dim to the query first (float32, rounded to
- * query_dtype), matching keys stored with rotate_keys.  Workspace: at least
+ * query_dtype), matching keys stored with rotate_keys.  rope_cos_dev / rope_sin_dev (optional,
+ * both or neither): BF16 [batch, head_dim] rotary tables applied to the (BF16) query before
+ * that, as nq_nqkv_write applies them to keys.  Workspace: at least
  * nq_nqkv_attention_workspace_bytes() bytes.  Requires head_dim = 64, page_size = 16,
  * q = 14, q_heads / kv_heads in {1, 2, 4, 8}; any max_pages.
  * Replaces: nqkv_decode_attention_batched_k1 and its three Triton kernels
@@ -260,7 +302,8 @@ int nq_nqkv_attention_decode(
     const int32_t *hot_lengths_dev, const uint8_t *cache_active_dev, const void *hot_keys_dev,
     const void *hot_values_dev, const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch,
     int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
-    int rotate_query, void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
+    int rotate_query, const void *rope_cos_dev, const void *rope_sin_dev, void *out_dev, void *workspace_dev,
+    size_t workspace_bytes, void *stream);
 
 size_t nq_nqkv_attention_workspace_bytes(int batch, int q_heads, int head_dim, int max_pages);
 

@@ -35,6 +35,9 @@ SIGNATURES = {
     "nq_hadamard": (_i32, [_ptr, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr]),
     "nq_dequantize_rows": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i64, _i64,
                                   _ptr, _i32, _ptr]),
+    "nq_fused_input_stage": (_i32, [_ptr, _i64, _i64, _i32, _ptr, _ptr, _ptr, _c.c_float, _ptr, _ptr, _i32, _ptr, _i32,
+                                    _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "nq_w4a4_gemv_grouped": (_i32, [_ptr, _i32] + [_ptr] * 8 + [_i32, _i32, _i32, _ptr]),
     "nq_w4a4_resolve_weight": (_i32, [_ptr, _ptr, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "nq_w4a4_gemv": (_i32, [_ptr] * 11 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
                                           _size, _ptr]),
@@ -44,9 +47,9 @@ SIGNATURES = {
     "nq_w4a4_gemm_workspace_bytes": (_size, [_i32, _i32, _i32, _i32, _i32]),
     "nq_nqkv_advance": (_i32, [_ptr, _ptr, _ptr, _i32, _i32, _i32, _i32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "nq_nqkv_write": (_i32, [_ptr, _ptr, _i32, _ptr, _ptr, _ptr, _i32, _ptr, _ptr] + [_ptr] * 6
-                      + [_ptr, _i32, _ptr, _i32, _ptr, _ptr] + [_i32] * 8 + [_ptr]),
+                      + [_ptr, _i32, _ptr, _i32, _ptr, _ptr] + [_i32] * 8 + [_ptr, _ptr, _ptr]),
     "nq_nqkv_attention_decode": (_i32, [_ptr, _i32] + [_ptr] * 17 + [_i32] * 7 + [_c.c_float, _i32, _ptr, _ptr,
-                                                                                _size, _ptr]),
+                                                                                _ptr, _ptr, _size, _ptr]),
     "nq_nqkv_attention_workspace_bytes": (_size, [_i32, _i32, _i32, _i32]),
 }
 

@@ -30,6 +30,7 @@ constexpr int kAttnMaxGroup = 8;
 
 struct AttentionArgs {
     const void *query;                 // [batch, q_heads, D]
+    const uint16_t *rope_cos, *rope_sin;   // optional BF16 [batch, D]: rotary embedding of the queries
     const uint32_t *key_codes, *value_codes;     // [pages][P * kv_heads * D / 8] words
     const uint8_t *key_beta_ids, *value_beta_ids; // [pages][P * kv_heads * D / 32]
     const float *key_norms, *value_norms;         // [pages][P * kv_heads]
@@ -102,6 +103,19 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     for (int i = tid; i < G * D; i += kAttnThreads)
         q_lds[i] = load_query(a.query, a.query_dtype, ((int64_t)row * a.q_heads + g * G) * D + i);
     __syncthreads();
+    if (a.rope_cos) {
+        // (q * cos) + (rotate_half(q) * sin) in BF16 tensor arithmetic, before the rotation
+        for (int i = tid; i < G * (D / 2); i += kAttnThreads) {
+            const int h = i / (D / 2), k = i % (D / 2);
+            const int64_t at = (int64_t)row * D;
+            const float c_lo = bf16_to_f32(a.rope_cos[at + k]), c_hi = bf16_to_f32(a.rope_cos[at + k + D / 2]);
+            const float s_lo = bf16_to_f32(a.rope_sin[at + k]), s_hi = bf16_to_f32(a.rope_sin[at + k + D / 2]);
+            const float x1 = q_lds[h * D + k], x2 = q_lds[h * D + k + D / 2];
+            q_lds[h * D + k] = bf16_to_f32(f32_to_bf16(bf16_to_f32(f32_to_bf16(x1 * c_lo)) - bf16_to_f32(f32_to_bf16(x2 * s_lo))));
+            q_lds[h * D + k + D / 2] = bf16_to_f32(f32_to_bf16(bf16_to_f32(f32_to_bf16(x2 * c_hi)) + bf16_to_f32(f32_to_bf16(x1 * s_hi))));
+        }
+        __syncthreads();
+    }
     if (a.rotate_query) {
         for (int width = 1; width < D; width <<= 1) {
             for (int i = tid; i < G * (D / 2); i += kAttnThreads) {
@@ -339,7 +353,8 @@ extern "C" int nq_nqkv_attention_decode(
     const int32_t *hot_lengths_dev, const uint8_t *cache_active_dev, const void *hot_keys_dev,
     const void *hot_values_dev, const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch,
     int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
-    int rotate_query, void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream) {
+    int rotate_query, const void *rope_cos_dev, const void *rope_sin_dev, void *out_dev, void *workspace_dev,
+    size_t workspace_bytes, void *stream) {
     NQ_REQUIRE(batch >= 1 && slots >= 1 && max_pages >= 1, NQ_ERR_SHAPE,
                "nq_nqkv_attention_decode: batch, slots and max_pages must be positive");
     NQ_REQUIRE(kv_heads >= 1 && q_heads >= kv_heads && q_heads % kv_heads == 0, NQ_ERR_SHAPE,
@@ -380,6 +395,12 @@ extern "C" int nq_nqkv_attention_decode(
     a.batch = batch; a.slots = slots; a.max_pages = max_pages; a.q_heads = q_heads; a.kv_heads = kv_heads;
     a.chunks = chunks_for(max_pages); a.query_dtype = query_dtype; a.scale = scale;
     a.rotate_query = rotate_query;
+    NQ_REQUIRE((rope_cos_dev == nullptr) == (rope_sin_dev == nullptr), NQ_ERR_ARGUMENT,
+               "nq_nqkv_attention_decode: rotary cos and sin tables come together");
+    NQ_REQUIRE(!rope_cos_dev || query_dtype == NQ_BF16, NQ_ERR_ARGUMENT,
+               "nq_nqkv_attention_decode: the fused rotary embedding takes BF16 queries");
+    a.rope_cos = reinterpret_cast<const uint16_t *>(rope_cos_dev);
+    a.rope_sin = reinterpret_cast<const uint16_t *>(rope_sin_dev);
     const size_t parts = (size_t)a.chunks + 1, heads_total = (size_t)batch * q_heads;
     a.part_max = reinterpret_cast<float *>(workspace_dev);
     a.part_sum = a.part_max + heads_total * parts;

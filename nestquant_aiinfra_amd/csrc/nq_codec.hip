@@ -70,14 +70,28 @@ template <> struct RowLoader<half_bits> {
     static __device__ __forceinline__ float scalar(const half_bits *x, int64_t i) { return f16_to_f32(x[i].v); }
 };
 
-template <typename T, bool kDithered>
+// Optional element-wise stage in front of the quantiser (BF16 rows only), in the arithmetic
+// of BF16 tensor operations: every tensor-level result is rounded to BF16.
+//   mode 1  h = x + residual (residual may be null); residual_out = h;
+//           y = weight * bf16(h * rsqrt(mean(h^2) + eps))      (LlamaRMSNorm)
+//   mode 2  y = bf16(silu(gate)) * x                            (the SwiGLU product)
+// normed_out (optional) receives y; rows are then rotated / quantised as usual.
+struct InputPrologue {
+    const uint16_t *residual, *weight, *gate;
+    uint16_t *residual_out, *normed_out;
+    float eps;
+};
+
+__device__ __forceinline__ float bf16_round(float x) { return bf16_to_f32(f32_to_bf16(x)); }
+
+template <typename T, bool kDithered, int kPrologue>
 __global__ void __launch_bounds__(1024)
 quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, float inv_q,
                      const float *__restrict__ betas, int beta_count, float sqrt_n,
                      uint32_t seed_plus_offset, uint32_t *__restrict__ codes,
                      uint8_t *__restrict__ beta_ids, float *__restrict__ norms,
                      uint4 *__restrict__ decoded, int rows_per_wg, int slices, int vector_loads,
-                     int hadamard_stage_dtype) {
+                     int hadamard_stage_dtype, InputPrologue pro) {
     extern __shared__ float lds[];
     float *row_scale = lds + (size_t)rows_per_wg * n;
     float *row_norm = row_scale + rows_per_wg;
@@ -111,6 +125,54 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
         }
     }
     __syncthreads();
+
+    if (kPrologue == 1) {
+        __shared__ float wave_sums[16];
+        const int count = rows_per_wg * n;
+        for (int idx = tid; idx < count; idx += blockDim.x) {
+            const int64_t g = first + idx;
+            if (g >= limit) continue;
+            float h = lds[idx];
+            if (pro.residual) h = bf16_round(h + bf16_to_f32(pro.residual[g]));
+            lds[idx] = h;
+            if (pro.residual_out && slice == 0) pro.residual_out[g] = f32_to_bf16(h);
+        }
+        __syncthreads();
+        for (int r = 0; r < rows_per_wg; r++) {
+            float sum = 0.0f;
+            for (int i = tid; i < n; i += blockDim.x) sum = __builtin_fmaf(lds[r * n + i], lds[r * n + i], sum);
+#pragma unroll
+            for (int offset = 32; offset >= 1; offset >>= 1) sum = sum + __shfl_xor(sum, offset, 64);
+            if ((tid & 63) == 0) wave_sums[tid >> 6] = sum;
+            __syncthreads();
+            if (tid == 0) {
+                float total = 0.0f;
+                for (int w = 0; w < (int)(blockDim.x + 63) / 64; w++) total = total + wave_sums[w];
+                row_scale[r] = 1.0f / __builtin_sqrtf(total / (float)n + pro.eps);
+            }
+            __syncthreads();
+        }
+        for (int idx = tid; idx < count; idx += blockDim.x) {
+            const int64_t g = first + idx;
+            if (g >= limit) continue;
+            const int r = idx / n, i = idx - r * n;
+            const float y = bf16_round(bf16_to_f32(pro.weight[i]) * bf16_round(lds[idx] * row_scale[r]));
+            lds[idx] = y;
+            if (pro.normed_out && slice == 0) pro.normed_out[g] = f32_to_bf16(y);
+        }
+        __syncthreads();
+    } else if (kPrologue == 2) {
+        for (int idx = tid; idx < rows_per_wg * n; idx += blockDim.x) {
+            const int64_t g = first + idx;
+            if (g >= limit) continue;
+            const float gate = bf16_to_f32(pro.gate[g]);
+            const float y = bf16_round(bf16_round(gate / (1.0f + __expf(-gate))) * lds[idx]);
+            lds[idx] = y;
+            if (pro.normed_out && slice == 0) pro.normed_out[g] = f32_to_bf16(y);
+        }
+        __syncthreads();
+    }
+    if (kPrologue != 0 && codes == nullptr) return;        // element-wise stage only
 
     // optional input rotation, in the arithmetic of the caller's tensor dtype
     if (hadamard_stage_dtype >= 0) staged_hadamard(lds, rows_per_wg, n, hadamard_stage_dtype);
@@ -263,10 +325,11 @@ extern "C" int nq_e8_nearest(const float *x_dev, float *out_dev, int64_t count, 
 
 namespace {
 
-template <typename T, bool kDithered>
+template <typename T, bool kDithered, int kPrologue = 0>
 int launch_quantize(const void *x, int64_t rows, int n, int q, const float *betas, int beta_count,
                     uint32_t seed_plus_offset, uint8_t *codes, uint8_t *beta_ids, float *norms,
-                    void *decoded, int hadamard_stage_dtype, hipStream_t stream) {
+                    void *decoded, int hadamard_stage_dtype, hipStream_t stream,
+                    nq::InputPrologue prologue = nq::InputPrologue{}) {
     const int pairs_per_row = n / 2;
     const int target = pairs_per_row < 256 ? 256 : (pairs_per_row < 1024 ? pairs_per_row : 1024);
     int rows_per_wg = target / pairs_per_row;
@@ -289,7 +352,7 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
     }
     if (threads < 64) threads = 64;
     const size_t lds_bytes = ((size_t)rows_per_wg * n + 2 * rows_per_wg) * sizeof(float);
-    auto kernel = nq::quantize_rows_kernel<T, kDithered>;
+    auto kernel = nq::quantize_rows_kernel<T, kDithered, kPrologue>;
     if (lds_bytes > 48 * 1024) {
         hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -305,7 +368,7 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
                        beta_count, (float)sqrt((double)n), seed_plus_offset,
                        reinterpret_cast<uint32_t *>(codes), beta_ids, norms,
                        reinterpret_cast<uint4 *>(decoded), rows_per_wg, slices,
-                       (int)nq::aligned(x, 16), hadamard_stage_dtype);
+                       (int)nq::aligned(x, 16), hadamard_stage_dtype, prologue);
     return nq::check_launch("nq_quantize_rows");
 }
 
@@ -356,6 +419,50 @@ extern "C" int nq_quantize_rows(const void *x_dev, int x_dtype, int64_t rows, in
         default: return nq::fail(NQ_ERR_ARGUMENT, "nq_quantize_rows: unknown dtype tag %d", x_dtype);
     }
 #undef NQ_DISPATCH_QUANTIZE
+}
+
+extern "C" int nq_fused_input_stage(const void *x_dev, int64_t rows, int64_t n, int mode,
+                                    const void *residual_dev, void *residual_out_dev,
+                                    const void *norm_weight_dev, float eps, const void *gate_dev,
+                                    void *staged_out_dev, int q, const float *betas_dev, int beta_count,
+                                    int hadamard, uint8_t *codes_dev, uint8_t *beta_ids_dev,
+                                    float *norms_dev, void *decoded_bf16_dev, void *stream) {
+    NQ_REQUIRE(rows >= 1 && n >= 32 && n % 32 == 0 && n <= 32768, NQ_ERR_SHAPE,
+               "nq_fused_input_stage: rows must be positive and n a multiple of 32 up to 32768");
+    NQ_REQUIRE(mode == 1 || mode == 2, NQ_ERR_ARGUMENT,
+               "nq_fused_input_stage: mode must be 1 (residual + RMSNorm) or 2 (SiLU(gate) * x)");
+    NQ_REQUIRE(x_dev, NQ_ERR_ARGUMENT, "nq_fused_input_stage: null input");
+    NQ_REQUIRE(mode != 1 || norm_weight_dev, NQ_ERR_ARGUMENT, "nq_fused_input_stage: mode 1 needs the norm weight");
+    NQ_REQUIRE(mode != 2 || gate_dev, NQ_ERR_ARGUMENT, "nq_fused_input_stage: mode 2 needs the gate rows");
+    NQ_REQUIRE(mode != 1 || (eps >= 0.0f && eps < 1.0f), NQ_ERR_ARGUMENT, "nq_fused_input_stage: eps out of range");
+    const bool encodes = codes_dev != nullptr;
+    NQ_REQUIRE(encodes || staged_out_dev || residual_out_dev, NQ_ERR_ARGUMENT,
+               "nq_fused_input_stage: nothing to produce");
+    if (encodes) {
+        NQ_REQUIRE(betas_dev && beta_ids_dev && norms_dev, NQ_ERR_ARGUMENT, "nq_fused_input_stage: null pointer");
+        NQ_REQUIRE(q >= 2 && q <= 16 && beta_count >= 1 && beta_count <= 4, NQ_ERR_SHAPE,
+                   "nq_fused_input_stage: q must be in [2, 16] and beta_count in [1, 4]");
+        NQ_REQUIRE(nq::aligned(codes_dev, 4) && nq::aligned(decoded_bf16_dev, 16), NQ_ERR_ARGUMENT,
+                   "nq_fused_input_stage: codes need 4-byte, the decoded output 16-byte alignment");
+        NQ_REQUIRE(!hadamard || (n & (n - 1)) == 0, NQ_ERR_SHAPE,
+                   "nq_fused_input_stage: the Hadamard rotation needs a power-of-two feature count");
+    }
+    nq::InputPrologue prologue{};
+    prologue.residual = reinterpret_cast<const uint16_t *>(residual_dev);
+    prologue.weight = reinterpret_cast<const uint16_t *>(norm_weight_dev);
+    prologue.gate = reinterpret_cast<const uint16_t *>(gate_dev);
+    prologue.residual_out = reinterpret_cast<uint16_t *>(residual_out_dev);
+    prologue.normed_out = reinterpret_cast<uint16_t *>(staged_out_dev);
+    prologue.eps = eps;
+    const int stage_dtype = (encodes && hadamard) ? NQ_BF16 : -1;
+    hipStream_t s = (hipStream_t)stream;
+    if (mode == 1)
+        return launch_quantize<uint16_t, false, 1>(x_dev, rows, (int)n, encodes ? q : 14, betas_dev, beta_count, 0u,
+                                                   codes_dev, beta_ids_dev, norms_dev, decoded_bf16_dev,
+                                                   stage_dtype, s, prologue);
+    return launch_quantize<uint16_t, false, 2>(x_dev, rows, (int)n, encodes ? q : 14, betas_dev, beta_count, 0u,
+                                               codes_dev, beta_ids_dev, norms_dev, decoded_bf16_dev, stage_dtype,
+                                               s, prologue);
 }
 
 extern "C" int nq_dequantize_rows(const uint8_t *codes_dev, const uint8_t *beta_ids_dev,

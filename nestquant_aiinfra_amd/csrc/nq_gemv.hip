@@ -44,22 +44,23 @@ __device__ __forceinline__ float row16_sum(float v) {
 // words, see nq_e8.hip.h) instead of NQRT4 code words and beta bytes.
 // R: output channels per workgroup.  A lane decodes block b of all R channels against one
 // load of the M activation blocks, and the R weight loads of a step are issued together.
+// The work of one workgroup: channels group * R .. + R of one weight, K slice `slice`.
 template <int M, int R, bool kResolved>
-__global__ void __launch_bounds__(kGemvThreads)
-w4a4_gemv_kernel(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8] blocks
-                 const uint32_t *__restrict__ w_words, const uint16_t *__restrict__ w_tails,
-                 const uint8_t *__restrict__ w_beta_ids,
-                 const float *__restrict__ w_norms, const float *__restrict__ w_betas,
-                 int m_rows, int k_size, int n_size, int k_slice,
-                 uint32_t seed_plus_offset, float sqrt_k, float *__restrict__ out_f32,
-                 uint16_t *__restrict__ out_bf16) {
+__device__ __forceinline__ void
+gemv_rows(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8] blocks
+          const uint32_t *__restrict__ w_words, const uint16_t *__restrict__ w_tails,
+          const uint8_t *__restrict__ w_beta_ids,
+          const float *__restrict__ w_norms, const float *__restrict__ w_betas,
+          int m_rows, int k_size, int n_size, int k_slice, int group, int slice,
+          uint32_t seed_plus_offset, float sqrt_k, float *__restrict__ out_f32,
+          uint16_t *__restrict__ out_bf16) {
     __shared__ float partial[kGemvWaves * 4][R][M];        // one entry per 16-lane row of every wavefront
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
     const int blocks_per_row = k_size >> 3;
     const int slice_blocks = k_slice >> 3;
-    const int slice_first_block = blockIdx.y * slice_blocks;
+    const int slice_first_block = slice * slice_blocks;
     const float wbeta[4] = {w_betas[0], w_betas[1], w_betas[2], w_betas[3]};
-    const int n0 = blockIdx.x * R;
+    const int n0 = group * R;
 
     float acc[R][M], wscale[R];
     int64_t row_first_block[R];
@@ -128,11 +129,49 @@ w4a4_gemv_kernel(const uint4 *__restrict__ act,          // decoded BF16 [m_rows
 #pragma unroll
             for (int w = 1; w < kGemvWaves * 4; w++) total = total + partial[w][r][m];
             if (out_f32)
-                out_f32[((int64_t)blockIdx.y * m_rows + m) * n_size + n] = total;
+                out_f32[((int64_t)slice * m_rows + m) * n_size + n] = total;
             else
                 out_bf16[(int64_t)m * n_size + n] = f32_to_bf16(total);
         }
     }
+}
+
+template <int M, int R, bool kResolved>
+__global__ void __launch_bounds__(kGemvThreads)
+w4a4_gemv_kernel(const uint4 *__restrict__ act, const uint32_t *__restrict__ w_words,
+                 const uint16_t *__restrict__ w_tails, const uint8_t *__restrict__ w_beta_ids,
+                 const float *__restrict__ w_norms, const float *__restrict__ w_betas,
+                 int m_rows, int k_size, int n_size, int k_slice, uint32_t seed_plus_offset, float sqrt_k,
+                 float *__restrict__ out_f32, uint16_t *__restrict__ out_bf16) {
+    gemv_rows<M, R, kResolved>(act, w_words, w_tails, w_beta_ids, w_norms, w_betas, m_rows, k_size, n_size,
+                               k_slice, blockIdx.x, blockIdx.y, seed_plus_offset, sqrt_k, out_f32, out_bf16);
+}
+
+// Several weights that share one activation (q/k/v or gate/up) in one launch: the grid is the
+// concatenation of their channel groups.
+constexpr int kGemvMaxGroup = 4;
+struct GemvWeights {
+    const uint32_t *words[kGemvMaxGroup];
+    const uint16_t *tails[kGemvMaxGroup];
+    const float *norms[kGemvMaxGroup], *betas[kGemvMaxGroup];
+    void *out[kGemvMaxGroup];
+    int n[kGemvMaxGroup], first_group[kGemvMaxGroup];
+    uint32_t seed_plus_offset[kGemvMaxGroup];
+    int count;
+};
+
+template <int M, int R>
+__global__ void __launch_bounds__(kGemvThreads)
+w4a4_gemv_grouped_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, int k_size, float sqrt_k,
+                         int out_is_f32) {
+    int which = 0;
+#pragma unroll
+    for (int i = 1; i < kGemvMaxGroup; i++)
+        if (i < w.count && (int)blockIdx.x >= w.first_group[i]) which = i;
+    gemv_rows<M, R, true>(act, w.words[which], w.tails[which], nullptr, w.norms[which], w.betas[which], m_rows,
+                          k_size, w.n[which], k_size, (int)blockIdx.x - w.first_group[which], 0,
+                          w.seed_plus_offset[which], sqrt_k, out_is_f32 ? (float *)w.out[which] : nullptr,
+                          out_is_f32 ? nullptr : (uint16_t *)w.out[which]);
 }
 
 // One lane per weight block: run the exact decode once and keep the lattice point it implies.
@@ -280,4 +319,68 @@ extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_bet
     int status = nq::check_launch("nq_w4a4_gemv");
     if (status != NQ_OK || split == 1) return status;
     return nq::launch_splitk_reduce(partials, split, (int64_t)m * n, out_dev, out_dtype, s);
+}
+
+extern "C" int nq_w4a4_gemv_grouped(const void *act_decoded_dev, int count, const uint32_t *const *w_resolved_words_dev,
+                                    const uint16_t *const *w_resolved_tails_dev, const float *const *w_norms_dev,
+                                    const float *const *w_betas_dev, const int *n, const int64_t *weight_offsets,
+                                    const int64_t *weight_seeds, void *const *out_dev, int m, int k, int out_dtype,
+                                    void *stream) {
+    NQ_REQUIRE(count >= 1 && count <= nq::kGemvMaxGroup, NQ_ERR_SHAPE,
+               "nq_w4a4_gemv_grouped: between 1 and %d weights per launch", nq::kGemvMaxGroup);
+    NQ_REQUIRE(m >= 1 && m <= 8, NQ_ERR_SHAPE, "nq_w4a4_gemv_grouped: M = %d is outside [1, 8]", m);
+    NQ_REQUIRE(k >= 32 && k % 32 == 0, NQ_ERR_SHAPE, "nq_w4a4_gemv_grouped: K = %d must be a positive multiple of 32", k);
+    NQ_REQUIRE(out_dtype == NQ_F32 || out_dtype == NQ_BF16, NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemv_grouped: output dtype tag %d is not F32 or BF16", out_dtype);
+    NQ_REQUIRE(act_decoded_dev && nq::aligned(act_decoded_dev, 16), NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemv_grouped: needs the decoded BF16 activation, 16-byte aligned");
+    NQ_REQUIRE(w_resolved_words_dev && w_resolved_tails_dev && w_norms_dev && w_betas_dev && n && weight_offsets &&
+                   weight_seeds && out_dev, NQ_ERR_ARGUMENT, "nq_w4a4_gemv_grouped: null argument array");
+    nq::GemvWeights w{};
+    w.count = count;
+    int64_t total_n = 0;
+    for (int i = 0; i < count; i++) total_n += n[i];
+    const int rows_per_wg = total_n >= 8192 ? 4 : 2;
+    int groups = 0;
+    for (int i = 0; i < count; i++) {
+        NQ_REQUIRE(n[i] >= 1, NQ_ERR_SHAPE, "nq_w4a4_gemv_grouped: N must be positive");
+        NQ_REQUIRE(w_resolved_words_dev[i] && w_resolved_tails_dev[i] && w_norms_dev[i] && w_betas_dev[i] && out_dev[i],
+                   NQ_ERR_ARGUMENT, "nq_w4a4_gemv_grouped: null pointer in weight %d", i);
+        NQ_REQUIRE(nq::aligned(w_resolved_words_dev[i], 4) && nq::aligned(w_resolved_tails_dev[i], 2), NQ_ERR_ARGUMENT,
+                   "nq_w4a4_gemv_grouped: misaligned resolved streams in weight %d", i);
+        NQ_REQUIRE(weight_seeds[i] >= 0 && weight_seeds[i] < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
+                   "nq_w4a4_gemv_grouped: seed must be in [0, 2**31)");
+        NQ_REQUIRE(weight_offsets[i] >= 0 && weight_offsets[i] + (int64_t)n[i] * (k / 8) <= ((int64_t)1 << 28),
+                   NQ_ERR_SHAPE, "nq_w4a4_gemv_grouped: block range exceeds the stateless dither counter space");
+        w.words[i] = w_resolved_words_dev[i];
+        w.tails[i] = w_resolved_tails_dev[i];
+        w.norms[i] = w_norms_dev[i];
+        w.betas[i] = w_betas_dev[i];
+        w.out[i] = out_dev[i];
+        w.n[i] = n[i];
+        w.first_group[i] = groups;
+        w.seed_plus_offset[i] = (uint32_t)((uint64_t)weight_seeds[i] + (uint64_t)weight_offsets[i] * 8u);
+        groups += (n[i] + rows_per_wg - 1) / rows_per_wg;
+    }
+    const float sqrt_k = (float)sqrt((double)k);
+    const uint4 *act = reinterpret_cast<const uint4 *>(act_decoded_dev);
+    const int out_is_f32 = out_dtype == NQ_F32;
+    hipStream_t s = (hipStream_t)stream;
+#define NQ_LAUNCH_GROUPED(MT)                                                                        \
+    do {                                                                                             \
+        if (rows_per_wg == 4)                                                                        \
+            hipLaunchKernelGGL((nq::w4a4_gemv_grouped_kernel<MT, 4>), dim3((unsigned)groups),        \
+                               dim3(nq::kGemvThreads), 0, s, act, w, m, k, sqrt_k, out_is_f32);      \
+        else                                                                                         \
+            hipLaunchKernelGGL((nq::w4a4_gemv_grouped_kernel<MT, 2>), dim3((unsigned)groups),        \
+                               dim3(nq::kGemvThreads), 0, s, act, w, m, k, sqrt_k, out_is_f32);      \
+    } while (0)
+    switch (m_tile_of(m)) {
+        case 1: NQ_LAUNCH_GROUPED(1); break;
+        case 2: NQ_LAUNCH_GROUPED(2); break;
+        case 4: NQ_LAUNCH_GROUPED(4); break;
+        default: NQ_LAUNCH_GROUPED(8); break;
+    }
+#undef NQ_LAUNCH_GROUPED
+    return nq::check_launch("nq_w4a4_gemv_grouped");
 }

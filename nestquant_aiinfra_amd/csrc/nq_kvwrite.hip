@@ -59,6 +59,7 @@ struct KvWriteArgs {
     float *key_norms, *value_norms;
     const float *key_betas, *value_betas;
     uint16_t *hot_keys, *hot_values;        // BF16 [slots, P, kv_heads, D]
+    const uint16_t *rope_cos, *rope_sin;    // optional BF16 [batch, tokens, D]: rotary embedding of the new keys
     int batch, tokens, uniform_count, slots, max_pages, kv_heads, key_beta_count, value_beta_count, rotate_keys;
 };
 
@@ -124,6 +125,21 @@ __global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
             dst[6] = __uint_as_float(raw.w << 16); dst[7] = __uint_as_float(raw.w & 0xffff0000u);
         }
         __syncthreads();
+        if (a.rope_cos) {
+            // rotary position embedding of the new key rows in BF16 tensor arithmetic:
+            // (k * cos) + (rotate_half(k) * sin), every product and the sum rounded to BF16
+            const int new_rows = page_tokens - first_new;
+            for (int i = tid; i < new_rows * (D / 2); i += kKvThreads) {
+                const int r = first_new + i / (D / 2), k = i % (D / 2);
+                const int64_t at = ((int64_t)row * a.tokens + (page_start + r - start)) * D;
+                const float c_lo = bf16_to_f32(a.rope_cos[at + k]), c_hi = bf16_to_f32(a.rope_cos[at + k + D / 2]);
+                const float s_lo = bf16_to_f32(a.rope_sin[at + k]), s_hi = bf16_to_f32(a.rope_sin[at + k + D / 2]);
+                const float x1 = rows[r][k], x2 = rows[r][k + D / 2];
+                rows[r][k] = bf16_to_f32(f32_to_bf16(bf16_to_f32(f32_to_bf16(x1 * c_lo)) - bf16_to_f32(f32_to_bf16(x2 * s_lo))));
+                rows[r][k + D / 2] = bf16_to_f32(f32_to_bf16(bf16_to_f32(f32_to_bf16(x2 * c_hi)) + bf16_to_f32(f32_to_bf16(x1 * s_hi))));
+            }
+            __syncthreads();
+        }
         if (a.rotate_keys) {
             // new key rows arrive unrotated: float32 Hadamard over the head, then BF16, as
             // hadamard(key.float()).to(bfloat16) (nestquant/runtime/nqkv_batched_hf_backend.py:381)
@@ -219,7 +235,7 @@ extern "C" int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_
                              const float *key_betas_dev, int key_beta_count, const float *value_betas_dev,
                              int value_beta_count, void *hot_keys_dev, void *hot_values_dev, int batch, int tokens,
                              int slots, int max_pages, int kv_heads, int head_dim, int page_size, int rotate_keys,
-                             void *stream) {
+                             const void *rope_cos_dev, const void *rope_sin_dev, void *stream) {
     NQ_REQUIRE(batch >= 1 && tokens >= 1 && slots >= 1 && max_pages >= 1 && kv_heads >= 1, NQ_ERR_SHAPE,
                "nq_nqkv_write: batch, tokens, slots, max_pages and kv_heads must be positive");
     NQ_REQUIRE(head_dim == 64 && page_size == 16, NQ_ERR_SHAPE,
@@ -251,6 +267,10 @@ extern "C" int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_
     a.batch = batch; a.tokens = tokens; a.uniform_count = uniform_count; a.slots = slots; a.max_pages = max_pages;
     a.kv_heads = kv_heads; a.key_beta_count = key_beta_count; a.value_beta_count = value_beta_count;
     a.rotate_keys = rotate_keys;
+    NQ_REQUIRE((rope_cos_dev == nullptr) == (rope_sin_dev == nullptr), NQ_ERR_ARGUMENT,
+               "nq_nqkv_write: rotary cos and sin tables come together");
+    a.rope_cos = reinterpret_cast<const uint16_t *>(rope_cos_dev);
+    a.rope_sin = reinterpret_cast<const uint16_t *>(rope_sin_dev);
     // `tokens` new rows starting anywhere inside a page touch at most this many pages
     const int touched = (tokens + page_size - 2) / page_size + 1;
     hipLaunchKernelGGL((nq::kv_write_kernel<64, 16>), dim3((unsigned)touched, (unsigned)(batch * kv_heads)),

@@ -1,0 +1,137 @@
+"""One decode step of a W4A4KV4 Llama with the glue between its packed kernels fused away.
+
+The reference runs the Hugging Face module graph for a decode step: per layer about thirty
+small tensor kernels (residual adds, LlamaRMSNorm, rotary embedding, SiLU and multiply,
+Hadamard passes) surround the packed linears and the NQKV attention
+(nestquant/models/fused_linear.py:276-421, nestquant/runtime/nqkv_batched_hf_backend.py:357-631).
+Here the same arithmetic, in the same BF16 tensor-operation rounding, runs in eleven launches
+per layer:
+
+    residual add + RMSNorm + Hadamard + A4 encode      nq_fused_input_stage (mode 1)
+    q_proj, k_proj, v_proj                             nq_w4a4_gemv_grouped
+    RoPE(k) + Hadamard(k) + KV append / page pack      nq_nqkv_write
+    RoPE(q) + Hadamard(q) + paged attention            nq_nqkv_attention_decode (two kernels)
+    Hadamard + A4 encode, o_proj                       nq_quantize_rows, nq_w4a4_gemv
+    residual add + RMSNorm + Hadamard + A4 encode      nq_fused_input_stage (mode 1)
+    gate_proj, up_proj                                 nq_w4a4_gemv_grouped
+    SiLU(gate) * up + Hadamard + A4 encode             nq_fused_input_stage (mode 2)
+    down_proj                                          nq_w4a4_gemv
+
+The module graph stays the path for prefill and for models this step does not recognise.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .nqkv import launch_nqkv_decode_attention
+from .w4a4_linear import (PreparedNQRTLinear, _gemm, _gemv, fused_input_stage, linear_packed_w4a4_gemv_grouped,
+                          quantize_activation_cuda)
+
+
+class UnsupportedForFusedDecode(ValueError):
+    pass
+
+
+def _require(condition: bool, reason: str) -> None:
+    if not condition:
+        raise UnsupportedForFusedDecode(reason)
+
+
+class FusedLlamaDecodeStep:
+    """Callable `(tokens [rows, 1], positions [rows, 1]) -> logits [rows, 1, vocab]` over a
+    LlamaForCausalLM whose projections are FusedNQRTLinear modules and a BatchedNQKVLlamaCache.
+    Raises UnsupportedForFusedDecode at construction for anything else."""
+
+    def __init__(self, model: torch.nn.Module, cache) -> None:
+        from ..models.fused_linear import FusedNQRTLinear
+
+        inner = getattr(model, "model", None)
+        _require(inner is not None and hasattr(inner, "layers") and hasattr(model, "lm_head"),
+                 "not a causal Llama model")
+        _require(all(hasattr(inner, name) for name in ("embed_tokens", "rotary_emb", "norm")), "not a Llama body")
+        self.model, self.inner, self.cache = model, inner, cache
+        self.layers = []
+        betas = None
+        for layer in inner.layers:
+            attention, mlp = getattr(layer, "self_attn", None), getattr(layer, "mlp", None)
+            _require(attention is not None and mlp is not None, "layer without self_attn / mlp")
+            _require(getattr(getattr(mlp, "act_fn", None), "__class__", type(None)).__name__ in {"SiLUActivation", "SiLU"},
+                     "MLP activation is not SiLU")
+            linears = [getattr(attention, n, None) for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
+            linears += [getattr(mlp, n, None) for n in ("gate_proj", "up_proj", "down_proj")]
+            for linear in linears:
+                _require(isinstance(linear, FusedNQRTLinear), "projection is not a FusedNQRTLinear")
+                _require(linear.bias is None and linear.input_hadamard and linear.activation_q == 14
+                         and not linear.force_w4a4_tiled_fallback and len(linear.activation_betas) == 4,
+                         "projection configuration outside the fused step")
+                _require(betas is None or linear.activation_betas == betas, "projections disagree on activation betas")
+                betas = linear.activation_betas
+            for norm in (layer.input_layernorm, layer.post_attention_layernorm):
+                _require(hasattr(norm, "weight") and hasattr(norm, "variance_epsilon"), "norm is not an RMSNorm")
+            self.layers.append((layer, attention, mlp, linears))
+        _require(len(self.layers) == cache.num_layers, "layer count disagrees with the cache")
+        hidden = inner.embed_tokens.weight.shape[1]
+        _require(hidden & (hidden - 1) == 0 and hidden % 32 == 0, "hidden size is not a power of two")
+        self.hidden = hidden
+
+    @staticmethod
+    def _prepared(linear, device) -> PreparedNQRTLinear:
+        prepared = linear._prepared_for(device)
+        _require(prepared.resolved_words is not None, "weight has no resolved form")
+        return prepared
+
+    @staticmethod
+    def _linear(activation, prepared: PreparedNQRTLinear) -> torch.Tensor:
+        if activation.token_count <= 8:
+            return _gemv(activation, prepared, split_k=0, output_dtype=torch.bfloat16)
+        return _gemm(activation, prepared, output_dtype=torch.bfloat16)
+
+    def _linears(self, activation, prepared: list[PreparedNQRTLinear]) -> list[torch.Tensor]:
+        if activation.token_count <= 8:
+            return linear_packed_w4a4_gemv_grouped(activation, prepared, output_dtype=torch.bfloat16)
+        return [self._linear(activation, weight) for weight in prepared]
+
+    @torch.inference_mode()
+    def __call__(self, tokens: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        cache, inner = self.cache, self.inner
+        manager = cache.manager
+        rows = tokens.shape[0]
+        if tokens.shape != (rows, 1) or positions.shape != (rows, 1) or rows != cache._rows:
+            raise ValueError("the fused decode step takes [rows, 1] tokens and positions for the rows in flight")
+        device = tokens.device
+        embedded = inner.embed_tokens(tokens)                               # [rows, 1, hidden]
+        if embedded.dtype != torch.bfloat16:
+            raise TypeError("the fused decode step runs BF16 models")
+        cos, sin = inner.rotary_emb(embedded, positions)                    # [rows, 1, head_dim]
+        cos, sin = cos.to(torch.bfloat16).contiguous(), sin.to(torch.bfloat16).contiguous()
+        query_rope = (cos.view(rows, -1), sin.view(rows, -1))
+        heads, kv_heads, dim = cache.num_query_heads, cache.num_kv_heads, cache.head_dim
+        workspace = cache._workspace(rows, torch.bfloat16)
+
+        delta, residual = embedded.view(rows, self.hidden), None
+        for index, (layer, attention, mlp, linears) in enumerate(self.layers):
+            q_w, k_w, v_w, o_w, gate_w, up_w, down_w = (self._prepared(linear, device) for linear in linears)
+            table = linears[0].activation_beta_table
+            activation, residual, _ = fused_input_stage(
+                delta, mode="rmsnorm", residual=residual, norm_weight=layer.input_layernorm.weight,
+                eps=layer.input_layernorm.variance_epsilon, beta_table=table, want_residual=True)
+            query, key, value = self._linears(activation, [q_w, k_w, v_w])
+            manager.write_layer(index, key.view(rows, 1, kv_heads, dim), value.view(rows, 1, kv_heads, dim),
+                                rotate_keys=True, rope=(cos, sin))
+            attended = launch_nqkv_decode_attention(
+                query.view(rows, heads, dim), manager.layers[index], slot_ids=manager.step_slot_ids,
+                active_mask=manager.step_active, attention_scale=float(attention.scaling), workspace=workspace,
+                rotate_query=True, rope=query_rope)
+            o_input = quantize_activation_cuda(attended.view(rows, heads * dim), q=14,
+                                               betas=linears[3].activation_betas, beta_table=table, hadamard=True)
+            delta = self._linear(o_input, o_w)
+            activation, residual, _ = fused_input_stage(
+                delta, mode="rmsnorm", residual=residual, norm_weight=layer.post_attention_layernorm.weight,
+                eps=layer.post_attention_layernorm.variance_epsilon, beta_table=table, want_residual=True)
+            gate, up = self._linears(activation, [gate_w, up_w])
+            activation, _, _ = fused_input_stage(up, mode="swiglu", gate=gate, beta_table=table)
+            delta = self._linear(activation, down_w)
+        _, _, normed = fused_input_stage(delta, mode="rmsnorm", residual=residual, norm_weight=inner.norm.weight,
+                                         eps=inner.norm.variance_epsilon, encode=False, want_staged=True)
+        return self.model.lm_head(normed.view(rows, 1, self.hidden))

@@ -361,8 +361,10 @@ class BatchedNQKVAttentionWorkspace:
 def launch_nqkv_decode_attention(query: torch.Tensor, cache: NQKVHotColdCache, *, slot_ids: torch.Tensor,
                                  active_mask: torch.Tensor, attention_scale: float,
                                  workspace: BatchedNQKVAttentionWorkspace,
-                                 rotate_query: bool = False) -> torch.Tensor:
-    """Graph-safe launch: no host reads, no allocation; writes workspace.output."""
+                                 rotate_query: bool = False,
+                                 rope: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
+    """Graph-safe launch: no host reads, no allocation; writes workspace.output.  `rope`:
+    BF16 (cos, sin) [batch, head_dim] applied to the query inside the kernel."""
     pool, meta = cache.pool, cache.metadata
     batch, heads, dim = query.shape
     _native.check(_native.library().nq_nqkv_attention_decode(
@@ -374,7 +376,8 @@ def launch_nqkv_decode_attention(query: torch.Tensor, cache: NQKVHotColdCache, *
         meta.hot_lengths.data_ptr(), meta.active_mask.data_ptr(),
         cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(), slot_ids.data_ptr(), active_mask.data_ptr(),
         batch, cache.max_sequences, cache.max_pages_per_sequence, heads, pool.num_kv_heads, dim, pool.page_size,
-        attention_scale, int(rotate_query), workspace.output.data_ptr(), workspace.buffer.data_ptr(),
+        attention_scale, int(rotate_query), None if rope is None else rope[0].data_ptr(),
+        None if rope is None else rope[1].data_ptr(), workspace.output.data_ptr(), workspace.buffer.data_ptr(),
         workspace.buffer.numel(),
         _native.stream_handle(query.device)))
     return workspace.output
@@ -515,9 +518,11 @@ class BatchedNQKVCacheManager:
             meta.hot_lengths.data_ptr(), _native.stream_handle(self.device)))
 
     def write_layer(self, layer_index: int, key: torch.Tensor, value: torch.Tensor, *,
-                    rotate_keys: bool = False) -> None:
+                    rotate_keys: bool = False,
+                    rope: tuple[torch.Tensor, torch.Tensor] | None = None) -> None:
         """Append this step's K/V rows [rows, tokens, kv_heads, head_dim] to one layer;
-        `rotate_keys` Hadamard-rotates the new keys inside the kernel."""
+        `rotate_keys` Hadamard-rotates the new keys inside the kernel, `rope` (BF16 cos, sin
+        [rows, tokens, head_dim]) applies the rotary embedding to them before that."""
         cache = self.layers[layer_index]
         pool, meta = cache.pool, self.metadata
         rows, tokens = key.shape[0], key.shape[1]
@@ -533,7 +538,8 @@ class BatchedNQKVCacheManager:
             pool.beta_table.data_ptr(), pool.beta_table.numel(), pool.value_beta_table.data_ptr(),
             pool.value_beta_table.numel(), cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(),
             rows, tokens, self.capacity, self.max_pages, pool.num_kv_heads, pool.head_dim, self.page_size,
-            int(rotate_keys), _native.stream_handle(self.device)))
+            int(rotate_keys), None if rope is None else rope[0].data_ptr(),
+            None if rope is None else rope[1].data_ptr(), _native.stream_handle(self.device)))
 
     def resident_bytes(self) -> int:
         total = 0

@@ -241,7 +241,10 @@ class BatchedNQKVLlamaRunner:
     the graph's fixed input tensors, the graph is replayed, logits are returned.
     """
 
-    def __init__(self, model: torch.nn.Module, cache: BatchedNQKVLlamaCache) -> None:
+    def __init__(self, model: torch.nn.Module, cache: BatchedNQKVLlamaCache, *,
+                 fused_decode: bool | None = None) -> None:
+        """`fused_decode`: run decode steps through FusedLlamaDecodeStep (eleven launches per
+        layer) instead of the module graph; None = whenever the model qualifies."""
         if not isinstance(model, torch.nn.Module):
             raise TypeError("model must be a torch module")
         if not isinstance(cache, BatchedNQKVLlamaCache):
@@ -256,6 +259,14 @@ class BatchedNQKVLlamaRunner:
         self._generation = [0] * self.batch_size
         self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor, torch.Tensor]] = {}
         self.graph_replay_counts: dict[int, int] = {}
+        self.fused_step = None
+        if fused_decode is None or fused_decode:
+            from .llama_decode_step import FusedLlamaDecodeStep, UnsupportedForFusedDecode
+            try:
+                self.fused_step = FusedLlamaDecodeStep(model, cache)
+            except UnsupportedForFusedDecode:
+                if fused_decode:
+                    raise
 
     @property
     def graph_captured(self) -> bool:
@@ -287,6 +298,8 @@ class BatchedNQKVLlamaRunner:
     # -- decode --------------------------------------------------------------------------------
     def _step(self, tokens: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
         self.cache.begin_decode_step()
+        if self.fused_step is not None:
+            return self.fused_step(tokens, positions)
         return self.model(input_ids=tokens, position_ids=positions, past_key_values=self.cache,
                           use_cache=True).logits
 

@@ -167,6 +167,63 @@ def quantize_activation_cuda(inputs: torch.Tensor, *, q: int, betas: Sequence[fl
     )
 
 
+def fused_input_stage(inputs: torch.Tensor, *, mode: str, q: int = 14, beta_table: torch.Tensor | None = None,
+                      residual: torch.Tensor | None = None, norm_weight: torch.Tensor | None = None,
+                      eps: float = 0.0, gate: torch.Tensor | None = None, hadamard: bool = True,
+                      encode: bool = True, want_residual: bool = False, want_staged: bool = False
+                      ) -> tuple[PreparedNQA4Activation | None, torch.Tensor | None, torch.Tensor | None]:
+    """Element-wise stage + rotate + encode of BF16 rows in one launch.
+
+    mode "rmsnorm": h = inputs + residual (residual optional), y = norm_weight * rmsnorm(h);
+    mode "swiglu": y = silu(gate) * inputs.  Returns (packed activation of y or None when
+    `encode` is false, h when `want_residual`, y when `want_staged`), each BF16 tensor shaped
+    like `inputs`.
+    """
+    if mode not in ("rmsnorm", "swiglu"):
+        raise ValueError("mode must be 'rmsnorm' or 'swiglu'")
+    device = _native.require_cuda(inputs)
+    others = [t for t in (residual, norm_weight, gate) if t is not None]
+    if inputs.dtype != torch.bfloat16 or any(t.dtype != torch.bfloat16 for t in others):
+        raise TypeError("the fused input stage takes BF16 tensors")
+    if not inputs.is_contiguous() or any(not t.is_contiguous() for t in others):
+        raise RuntimeError("fused input stage tensors must be contiguous")
+    n = inputs.shape[-1]
+    count = inputs.numel() // n
+    for name, tensor in (("residual", residual), ("gate", gate)):
+        if tensor is not None and tensor.shape != inputs.shape:
+            raise ValueError(f"{name} must have the shape of inputs")
+    if mode == "rmsnorm" and (norm_weight is None or norm_weight.numel() != n):
+        raise ValueError("mode 'rmsnorm' needs a norm weight of the feature size")
+    if mode == "swiglu" and gate is None:
+        raise ValueError("mode 'swiglu' needs the gate rows")
+    residual_out = torch.empty_like(inputs) if want_residual else None
+    staged = torch.empty_like(inputs) if want_staged else None
+    codes = beta_ids = norms = decoded = None
+    if encode:
+        if beta_table is None or q != 14 or beta_table.numel() != 4:
+            raise ValueError("encoding needs q = 14 and a table of four betas")
+        codes = torch.empty(count * n // 2, dtype=torch.uint8, device=device)
+        beta_ids = torch.empty(count * n // 32, dtype=torch.uint8, device=device)
+        norms = torch.empty(count, dtype=torch.float32, device=device)
+        decoded = torch.empty((count, n), dtype=torch.bfloat16, device=device)
+
+    def ptr(tensor):
+        return None if tensor is None else tensor.data_ptr()
+
+    _native.check(_native.library().nq_fused_input_stage(
+        inputs.data_ptr(), count, n, 1 if mode == "rmsnorm" else 2, ptr(residual), ptr(residual_out),
+        ptr(norm_weight), float(eps), ptr(gate), ptr(staged), q, ptr(beta_table),
+        0 if beta_table is None else beta_table.numel(), int(hadamard), ptr(codes), ptr(beta_ids), ptr(norms),
+        ptr(decoded), _native.stream_handle(device)))
+    activation = None
+    if encode:
+        activation = PreparedNQA4Activation(
+            code_payload=codes, beta_payload=beta_ids, row_norms=norms, beta_table=beta_table,
+            original_shape=tuple(inputs.shape), q=q, code_width=4, beta_width=2,
+            output_dtype=inputs.dtype, decoded=decoded)
+    return activation, residual_out, staged
+
+
 def quantize_weight_nqrt4(weight: torch.Tensor, *, q: int = 14, betas: Sequence[float],
                           dither_seed: int, tensor_name: str = "weight") -> PackedNestQuantTensor:
     """Quantize an (already rotated) weight [N, K] on the GPU into an NQRT v4 record with
@@ -365,6 +422,35 @@ def _gemv(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *, spl
         int(weight.record.dither_seed), split_k, out.data_ptr(), _native.dtype_tag(output_dtype),
         None if workspace is None else workspace.data_ptr(), need, _native.stream_handle(device)))
     return out.reshape(*activation.original_shape[:-1], n)
+
+
+def linear_packed_w4a4_gemv_grouped(activation: PreparedNQA4Activation, weights: Sequence[PreparedNQRTLinear], *,
+                                    output_dtype: torch.dtype | None = None) -> list[torch.Tensor]:
+    """One launch for up to four projections of the same M <= 8 activation (q/k/v, gate/up)."""
+    import ctypes
+    if not 1 <= len(weights) <= 4:
+        raise ValueError("between one and four weights per grouped launch")
+    if activation.decoded is None or any(w.resolved_words is None for w in weights):
+        raise ValueError("the grouped GEMV takes a decoded activation and resolved weights")
+    m, k = activation.token_count, activation.feature_count
+    if not 1 <= m <= 8 or any(w.record.feature_count != k for w in weights):
+        raise ValueError("activation or packed weights are unsupported by the grouped W4A4 GEMV")
+    dtype = output_dtype or _kernel_dtype(activation)
+    device = activation.decoded.device
+    count = len(weights)
+    sizes = [w.record.indices.shape[0] for w in weights]
+    outs = [torch.empty((m, n), dtype=dtype, device=device) for n in sizes]
+    pointers = ctypes.c_void_p * count
+    _native.check(_native.library().nq_w4a4_gemv_grouped(
+        activation.decoded.data_ptr(), count,
+        pointers(*[w.resolved_words.data_ptr() for w in weights]),
+        pointers(*[w.resolved_tails.data_ptr() for w in weights]),
+        pointers(*[w.row_norms.data_ptr() for w in weights]),
+        pointers(*[w.beta_table.data_ptr() for w in weights]),
+        (ctypes.c_int * count)(*sizes), (ctypes.c_int64 * count)(*([0] * count)),
+        (ctypes.c_int64 * count)(*[int(w.record.dither_seed) for w in weights]),
+        pointers(*[o.data_ptr() for o in outs]), m, k, _native.dtype_tag(dtype), _native.stream_handle(device)))
+    return [o.reshape(*activation.original_shape[:-1], n) for o, n in zip(outs, sizes)]
 
 
 def _kernel_dtype(activation: PreparedNQA4Activation) -> torch.dtype:

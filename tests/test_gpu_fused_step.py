@@ -1,0 +1,219 @@
+"""GPU checks of the fused decode-step pieces, through the C ABI:
+  * nq_fused_input_stage against the BF16 tensor operations it replaces (LlamaRMSNorm with a
+    residual add, SiLU-and-multiply) followed by the plain encoder;
+  * nq_w4a4_gemv_grouped against one nq_w4a4_gemv call per weight (bit for bit);
+  * the rotary embedding inside nq_nqkv_write / nq_nqkv_attention_decode against the same
+    BF16 tensor arithmetic done beforehand (bit for bit);
+  * FusedLlamaDecodeStep against the module graph of the same tiny model (tolerance: the
+    row reductions of the norm run in a different order).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ACTIVATION_BETAS, Q, WEIGHT_BETAS
+from gpu_util import bits, oracle_weight, relative_error
+
+pytestmark = pytest.mark.gpu
+
+KEY_BETAS = tuple(v / 14 for v in (3.50, 4.58, 6.47, 17.06))
+VALUE_BETAS = tuple(v / 14 for v in (3.53, 5.59, 9.62, 29.03))
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from nestquant_aiinfra_amd.runtime import w4a4_linear
+    return w4a4_linear
+
+
+def _table():
+    return torch.tensor(ACTIVATION_BETAS, dtype=torch.float32, device="cuda")
+
+
+def _same_activation(a, b):
+    return (torch.equal(a.code_payload, b.code_payload) and torch.equal(a.beta_payload, b.beta_payload)
+            and torch.equal(a.row_norms, b.row_norms) and torch.equal(a.decoded, b.decoded))
+
+
+def _rms_norm(h, weight, eps):
+    x = h.float()
+    x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    return weight * x.to(h.dtype)
+
+
+@pytest.mark.parametrize("rows,n", [(1, 2048), (8, 2048), (3, 256), (5, 8192), (40, 512)])
+@pytest.mark.parametrize("with_residual", [False, True])
+def test_residual_rmsnorm_stage(rt, rows, n, with_residual):
+    g = torch.Generator().manual_seed(rows * n + with_residual)
+    x = torch.randn(rows, n, generator=g).to(torch.bfloat16).cuda()
+    residual = (3 * torch.randn(rows, n, generator=g)).to(torch.bfloat16).cuda() if with_residual else None
+    weight = (1 + 0.1 * torch.randn(n, generator=g)).to(torch.bfloat16).cuda()
+    eps = 1e-5
+    activation, h, staged = rt.fused_input_stage(x, mode="rmsnorm", residual=residual, norm_weight=weight, eps=eps,
+                                                 beta_table=_table(), want_residual=True, want_staged=True)
+    expect_h = x + residual if with_residual else x
+    assert torch.equal(h, expect_h)
+    expect = _rms_norm(expect_h, weight, eps)
+    # one BF16 step at most, and only where the differently ordered mean moved a rounding
+    difference = (staged.float() - expect.float()).abs()
+    assert bool((difference <= expect.float().abs() * 2.0 ** -7 + 1e-30).all())
+    assert int((staged != expect).sum()) <= max(2, rows * n // 200)
+    # the encode that follows is the plain encoder on the staged rows
+    plain = rt.quantize_activation_cuda(staged, q=Q, betas=ACTIVATION_BETAS, hadamard=True)
+    assert _same_activation(activation, plain)
+    # element-wise stage alone
+    none, _, staged_only = rt.fused_input_stage(x, mode="rmsnorm", residual=residual, norm_weight=weight, eps=eps,
+                                                encode=False, want_staged=True)
+    assert none is None and torch.equal(staged_only, staged)
+
+
+@pytest.mark.parametrize("rows,n", [(1, 8192), (8, 8192), (2, 512)])
+def test_swiglu_stage(rt, rows, n):
+    g = torch.Generator().manual_seed(rows + n)
+    gate = (2 * torch.randn(rows, n, generator=g)).to(torch.bfloat16).cuda()
+    up = torch.randn(rows, n, generator=g).to(torch.bfloat16).cuda()
+    activation, _, staged = rt.fused_input_stage(up, mode="swiglu", gate=gate, beta_table=_table(), want_staged=True)
+    expect = torch.nn.functional.silu(gate) * up
+    difference = (staged.float() - expect.float()).abs()
+    assert bool((difference <= expect.float().abs() * 2.0 ** -6 + 1e-30).all())      # exp differs in the last place
+    assert int((staged != expect).sum()) <= max(2, rows * n // 100)
+    plain = rt.quantize_activation_cuda(staged, q=Q, betas=ACTIVATION_BETAS, hadamard=True)
+    assert _same_activation(activation, plain)
+
+
+def test_fused_stage_argument_checks(rt):
+    x = torch.zeros(2, 256, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        rt.fused_input_stage(x, mode="layernorm", beta_table=_table())
+    with pytest.raises(ValueError):
+        rt.fused_input_stage(x, mode="rmsnorm", beta_table=_table())                 # no norm weight
+    with pytest.raises(ValueError):
+        rt.fused_input_stage(x, mode="swiglu", beta_table=_table())                  # no gate
+    with pytest.raises(TypeError):
+        rt.fused_input_stage(x.float(), mode="swiglu", gate=x.float(), beta_table=_table())
+
+
+@pytest.mark.parametrize("m", [1, 3, 8])
+def test_grouped_gemv_equals_single_launches(rt, oracle, m):
+    from test_gpu_gemv import _record
+    from gpu_util import student_t_rows
+    k = 2048
+    weights = []
+    for index, n_out in enumerate((512, 136, 2050)):
+        seed = 20261101 + index
+        _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=900 + index, dither_seed=seed)
+        weights.append(rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda"))
+    x = torch.from_numpy(oracle.hadamard(student_t_rows(m, k, seed=31 + m).numpy())).to(torch.bfloat16).cuda()
+    activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS)
+    for dtype, view in ((torch.float32, torch.int32), (torch.bfloat16, torch.int16)):
+        grouped = rt.linear_packed_w4a4_gemv_grouped(activation, weights, output_dtype=dtype)
+        for out, weight in zip(grouped, weights):
+            single = rt._gemv(activation, weight, split_k=1, output_dtype=dtype)
+            assert torch.equal(out.view(view), single.view(view))
+    with pytest.raises(ValueError):
+        rt.linear_packed_w4a4_gemv_grouped(activation, weights * 2)
+
+
+def _rope_tables(rows, tokens, dim, seed):
+    g = torch.Generator().manual_seed(seed)
+    angle = 6.0 * torch.rand(rows, tokens, dim // 2, generator=g)
+    angle = torch.cat([angle, angle], dim=-1)
+    return angle.cos().to(torch.bfloat16).cuda(), angle.sin().to(torch.bfloat16).cuda()
+
+
+def _apply_rope(x, cos, sin):
+    half = x.shape[-1] // 2
+    rotated = torch.cat([-x[..., half:], x[..., :half]], dim=-1)
+    return (x * cos) + (rotated * sin)
+
+
+def test_rotary_embedding_inside_writer_and_attention():
+    from nestquant_aiinfra_amd.runtime import nqkv as kv
+    heads, q_heads, dim, page = 2, 8, 64, 16
+    def manager():
+        return kv.BatchedNQKVCacheManager(capacity=2, num_layers=1, num_kv_heads=heads, head_dim=dim,
+                                          max_cache_len=96, page_size=page, q=Q, key_betas=KEY_BETAS,
+                                          value_betas=VALUE_BETAS, dtype=torch.bfloat16, device="cuda")
+    fused, plain = manager(), manager()
+    for m in (fused, plain):
+        m.register("a", slot=0)
+        m.register("b", slot=1)
+    g = torch.Generator().manual_seed(77)
+    for step, tokens in enumerate((21, 1, 1, 11, 1)):                       # crosses pages in both slots
+        key = torch.randn(2, tokens, heads, dim, generator=g).to(torch.bfloat16).cuda()
+        value = torch.randn(2, tokens, heads, dim, generator=g).to(torch.bfloat16).cuda()
+        cos, sin = _rope_tables(2, tokens, dim, seed=100 + step)
+        for m in (fused, plain):
+            m.step_slot_ids[:2] = torch.tensor([1, 0], dtype=torch.int32)
+            m.step_active[:2] = True
+            m.begin_step(rows=2, uniform_count=tokens)
+        fused.write_layer(0, key, value, rotate_keys=True, rope=(cos, sin))
+        plain.write_layer(0, _apply_rope(key, cos[:, :, None, :], sin[:, :, None, :]).contiguous(), value,
+                          rotate_keys=True)
+    a, b = fused.layers[0], plain.layers[0]
+    for name in ("key_codes", "key_betas", "key_norms", "value_codes", "value_betas", "value_norms"):
+        assert torch.equal(getattr(a.pool, name), getattr(b.pool, name)), name
+    assert torch.equal(a.hot_keys, b.hot_keys) and torch.equal(a.hot_values, b.hot_values)
+
+    query = torch.randn(2, q_heads, dim, generator=g).to(torch.bfloat16).cuda()
+    cos, sin = _rope_tables(2, 1, dim, seed=999)
+    workspace = kv.BatchedNQKVAttentionWorkspace.create(a, batch_size=2, query_heads=q_heads,
+                                                        output_dtype=torch.bfloat16)
+    common = dict(slot_ids=fused.step_slot_ids[:2], active_mask=fused.step_active[:2], attention_scale=0.125,
+                  workspace=workspace, rotate_query=True)
+    inside = kv.launch_nqkv_decode_attention(query, a, rope=(cos.view(2, dim), sin.view(2, dim)), **common).clone()
+    before = kv.launch_nqkv_decode_attention(_apply_rope(query, cos, sin).contiguous(), a, **common).clone()
+    assert torch.equal(inside, before) and bool(inside.float().abs().sum() > 0)
+
+
+def test_fused_decode_step_tracks_the_module_graph(tmp_path):
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
+    from nestquant_aiinfra_amd.runtime.nqkv_hf_backend import BatchedNQKVLlamaRunner
+
+    torch.manual_seed(5001)
+    config = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                         num_key_value_heads=2, head_dim=64, vocab_size=128, max_position_embeddings=512,
+                         rope_theta=500000.0, tie_word_embeddings=True)
+    model = LlamaForCausalLM(config).to(torch.bfloat16).cuda().eval()
+    path = tmp_path / "tiny.nqmc"
+    asm.write_w4_checkpoint(model, path)
+    runner = asm.build_w4a4kv4_runner(model, path, capacity=2, max_cache_len=96)
+    assert runner.fused_step is not None
+    modular = BatchedNQKVLlamaRunner(model, runner.cache, fused_decode=False)
+    assert modular.fused_step is None
+
+    g = torch.Generator().manual_seed(5002)
+    ids = torch.randint(0, 128, (2, 20), generator=g).cuda()
+    logits = runner.prefill_slots(ids, slots=[0, 1], lengths=[20, 9])
+    cache = runner.cache
+    meta = cache.manager.metadata
+    tensors = [meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths]
+    for layer in cache.manager.layers:
+        pool = layer.pool
+        tensors += [layer.hot_keys, layer.hot_values, pool.key_codes, pool.key_betas, pool.key_norms,
+                    pool.value_codes, pool.value_betas, pool.value_norms]
+    saved, host = [t.clone() for t in tensors], list(cache._host_lengths)
+
+    token = torch.stack([logits[0, 19].argmax(), logits[1, 8].argmax()]).reshape(2, 1)
+    position = torch.tensor([[20], [9]], device="cuda")
+    def run(which, steps=12):
+        outs, tok, pos = [], token, position
+        for _ in range(steps):
+            out = which.decode_eager(tok, slots=[0, 1], positions=pos).float().clone()
+            outs.append(out)
+            tok = token                                   # same inputs for both paths at every step
+            pos = pos + 1
+        return torch.stack(outs)
+    fused = run(runner)
+    for tensor, value in zip(tensors, saved):
+        tensor.copy_(value)
+    cache._host_lengths[:] = host
+    reference = run(modular)
+    assert torch.isfinite(fused).all()
+    cosine = torch.nn.functional.cosine_similarity(fused.flatten(1), reference.flatten(1), dim=1)
+    assert float(cosine.min()) > 0.995
+    assert relative_error(bits(fused), bits(reference)) < 0.08
+    # the first step starts from identical state: only reduction order separates the two
+    assert relative_error(bits(fused[0]), bits(reference[0])) < 0.03
