@@ -82,7 +82,122 @@ struct InputPrologue {
     float eps;
 };
 
-__device__ __forceinline__ float bf16_round(float x) { return bf16_to_f32(f32_to_bf16(x)); }
+
+__device__ __forceinline__ void unpack_bf16x8(const uint4 raw, float (&v)[8]) {
+    v[0] = __uint_as_float(raw.x << 16); v[1] = __uint_as_float(raw.x & 0xffff0000u);
+    v[2] = __uint_as_float(raw.y << 16); v[3] = __uint_as_float(raw.y & 0xffff0000u);
+    v[4] = __uint_as_float(raw.z << 16); v[5] = __uint_as_float(raw.z & 0xffff0000u);
+    v[6] = __uint_as_float(raw.w << 16); v[7] = __uint_as_float(raw.w & 0xffff0000u);
+}
+
+// eight float32 values that are exact BF16 numbers -> packed BF16
+__device__ __forceinline__ uint4 pack_bf16x8_exact(const float (&v)[8]) {
+    return make_uint4((__float_as_uint(v[0]) >> 16) | (__float_as_uint(v[1]) & 0xffff0000u),
+                      (__float_as_uint(v[2]) >> 16) | (__float_as_uint(v[3]) & 0xffff0000u),
+                      (__float_as_uint(v[4]) >> 16) | (__float_as_uint(v[5]) & 0xffff0000u),
+                      (__float_as_uint(v[6]) >> 16) | (__float_as_uint(v[7]) & 0xffff0000u));
+}
+
+// Stages rows [first, first + rows_per_wg * n) into `staged` through the element-wise stage
+// of `pro` (see InputPrologue).  Every global operand of a 16-byte vector is requested before
+// any is used, so the kernel pays one memory round trip, not one per operand.  `weights`
+// (n floats of LDS) holds the norm weight in mode 1.  Ends with a barrier.
+template <int kPrologue>
+__device__ __forceinline__ void stage_with_prologue(const uint16_t *__restrict__ x, const InputPrologue &pro,
+                                                    float *staged, float *row_scale, float *weights,
+                                                    int64_t first, int64_t limit, int rows_per_wg, int n,
+                                                    bool writes_outputs) {
+    __shared__ float row_sums[64];
+    const int tid = threadIdx.x;
+    const int row_vectors = n >> 3, vectors = rows_per_wg * row_vectors;
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    for (int v = tid; v < vectors; v += blockDim.x) {
+        const int64_t g = first + (int64_t)v * 8;
+        const bool live = g < limit;
+        const uint4 raw_x = live ? reinterpret_cast<const uint4 *>(x)[g >> 3] : zero;
+        uint4 raw_a = zero, raw_w = zero;
+        if (kPrologue == 1) {
+            if (live && pro.residual) raw_a = reinterpret_cast<const uint4 *>(pro.residual)[g >> 3];
+            if (v < row_vectors) raw_w = reinterpret_cast<const uint4 *>(pro.weight)[v];
+        } else {
+            if (live) raw_a = reinterpret_cast<const uint4 *>(pro.gate)[g >> 3];
+        }
+        float h[8], a[8];
+        unpack_bf16x8(raw_x, h);
+        unpack_bf16x8(raw_a, a);
+        if (kPrologue == 1) {
+            if (pro.residual) {
+#pragma unroll
+                for (int j = 0; j < 8; j += 2) {
+                    h[j] = h[j] + a[j];
+                    h[j + 1] = h[j + 1] + a[j + 1];
+                    round_pair<1>(h[j], h[j + 1]);
+                }
+            }
+            if (live && writes_outputs && pro.residual_out)
+                reinterpret_cast<uint4 *>(pro.residual_out)[g >> 3] = pack_bf16x8_exact(h);
+            if (v < row_vectors) {
+                float w[8];
+                unpack_bf16x8(raw_w, w);
+#pragma unroll
+                for (int j = 0; j < 8; j++) weights[v * 8 + j] = w[j];
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) {
+                float s0 = a[j] / (1.0f + __expf(-a[j])), s1 = a[j + 1] / (1.0f + __expf(-a[j + 1]));
+                round_pair<1>(s0, s1);
+                h[j] = s0 * h[j];
+                h[j + 1] = s1 * h[j + 1];
+                round_pair<1>(h[j], h[j + 1]);
+            }
+            if (live && writes_outputs && pro.normed_out)
+                reinterpret_cast<uint4 *>(pro.normed_out)[g >> 3] = pack_bf16x8_exact(h);
+        }
+        *reinterpret_cast<float4 *>(staged + v * 8) = make_float4(h[0], h[1], h[2], h[3]);
+        *reinterpret_cast<float4 *>(staged + v * 8 + 4) = make_float4(h[4], h[5], h[6], h[7]);
+    }
+    __syncthreads();
+    if (kPrologue != 1) return;
+
+    // LlamaRMSNorm: bf16(weight * bf16(h * rsqrt(mean(h^2) + eps))), one row at a time
+    const int rows16 = (int)(blockDim.x >> 4);
+    for (int r = 0; r < rows_per_wg; r++) {
+        float sum = 0.0f;
+        for (int i = tid; i < n; i += blockDim.x) sum = __builtin_fmaf(staged[r * n + i], staged[r * n + i], sum);
+        sum = sum + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, sum), 0xB1, 0xF, 0xF, true));
+        sum = sum + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, sum), 0x4E, 0xF, 0xF, true));
+        sum = sum + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, sum), 0x141, 0xF, 0xF, true));
+        sum = sum + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, sum), 0x140, 0xF, 0xF, true));
+        if ((tid & 15) == 0) row_sums[tid >> 4] = sum;
+        __syncthreads();
+        float total = 0.0f;
+        for (int w = 0; w < rows16; w++) total = total + row_sums[w];
+        if (tid == 0) row_scale[r] = 1.0f / __builtin_sqrtf(total / (float)n + pro.eps);
+        __syncthreads();
+    }
+    for (int v = tid; v < vectors; v += blockDim.x) {
+        const int64_t g = first + (int64_t)v * 8;
+        const int r = rows_per_wg == 1 ? 0 : v / row_vectors;
+        const int column = (v - r * row_vectors) * 8;
+        const float scale = row_scale[r];
+        float y[8];
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            y[j] = staged[v * 8 + j] * scale;
+            y[j + 1] = staged[v * 8 + j + 1] * scale;
+            round_pair<1>(y[j], y[j + 1]);
+            y[j] = weights[column + j] * y[j];
+            y[j + 1] = weights[column + j + 1] * y[j + 1];
+            round_pair<1>(y[j], y[j + 1]);
+        }
+        *reinterpret_cast<float4 *>(staged + v * 8) = make_float4(y[0], y[1], y[2], y[3]);
+        *reinterpret_cast<float4 *>(staged + v * 8 + 4) = make_float4(y[4], y[5], y[6], y[7]);
+        if (g < limit && writes_outputs && pro.normed_out)
+            reinterpret_cast<uint4 *>(pro.normed_out)[g >> 3] = pack_bf16x8_exact(y);
+    }
+    __syncthreads();
+}
 
 template <typename T, bool kDithered, int kPrologue>
 __global__ void __launch_bounds__(1024)
@@ -104,7 +219,11 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
 
     // phase 1
     const int64_t first = row0 * n, limit = rows * (int64_t)n;
-    if (vector_loads) {
+    if (kPrologue != 0) {
+        stage_with_prologue<kPrologue>(reinterpret_cast<const uint16_t *>(x), pro, lds, row_scale, row_norm + rows_per_wg,
+                                       first, limit, rows_per_wg, n, slice == 0);
+        if (codes == nullptr) return;                      // element-wise stage only
+    } else if (vector_loads) {
         // n is a multiple of 32, so every row is a whole number of 16-byte vectors
         constexpr int kPer = RowLoader<T>::kPerVector;
         const int vectors = rows_per_wg * n / kPer;
@@ -125,54 +244,6 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
         }
     }
     __syncthreads();
-
-    if (kPrologue == 1) {
-        __shared__ float wave_sums[16];
-        const int count = rows_per_wg * n;
-        for (int idx = tid; idx < count; idx += blockDim.x) {
-            const int64_t g = first + idx;
-            if (g >= limit) continue;
-            float h = lds[idx];
-            if (pro.residual) h = bf16_round(h + bf16_to_f32(pro.residual[g]));
-            lds[idx] = h;
-            if (pro.residual_out && slice == 0) pro.residual_out[g] = f32_to_bf16(h);
-        }
-        __syncthreads();
-        for (int r = 0; r < rows_per_wg; r++) {
-            float sum = 0.0f;
-            for (int i = tid; i < n; i += blockDim.x) sum = __builtin_fmaf(lds[r * n + i], lds[r * n + i], sum);
-#pragma unroll
-            for (int offset = 32; offset >= 1; offset >>= 1) sum = sum + __shfl_xor(sum, offset, 64);
-            if ((tid & 63) == 0) wave_sums[tid >> 6] = sum;
-            __syncthreads();
-            if (tid == 0) {
-                float total = 0.0f;
-                for (int w = 0; w < (int)(blockDim.x + 63) / 64; w++) total = total + wave_sums[w];
-                row_scale[r] = 1.0f / __builtin_sqrtf(total / (float)n + pro.eps);
-            }
-            __syncthreads();
-        }
-        for (int idx = tid; idx < count; idx += blockDim.x) {
-            const int64_t g = first + idx;
-            if (g >= limit) continue;
-            const int r = idx / n, i = idx - r * n;
-            const float y = bf16_round(bf16_to_f32(pro.weight[i]) * bf16_round(lds[idx] * row_scale[r]));
-            lds[idx] = y;
-            if (pro.normed_out && slice == 0) pro.normed_out[g] = f32_to_bf16(y);
-        }
-        __syncthreads();
-    } else if (kPrologue == 2) {
-        for (int idx = tid; idx < rows_per_wg * n; idx += blockDim.x) {
-            const int64_t g = first + idx;
-            if (g >= limit) continue;
-            const float gate = bf16_to_f32(pro.gate[g]);
-            const float y = bf16_round(bf16_round(gate / (1.0f + __expf(-gate))) * lds[idx]);
-            lds[idx] = y;
-            if (pro.normed_out && slice == 0) pro.normed_out[g] = f32_to_bf16(y);
-        }
-        __syncthreads();
-    }
-    if (kPrologue != 0 && codes == nullptr) return;        // element-wise stage only
 
     // optional input rotation, in the arithmetic of the caller's tensor dtype
     if (hadamard_stage_dtype >= 0) staged_hadamard(lds, rows_per_wg, n, hadamard_stage_dtype);
@@ -351,7 +422,7 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
         if (slices > 1) threads = sliced_threads;
     }
     if (threads < 64) threads = 64;
-    const size_t lds_bytes = ((size_t)rows_per_wg * n + 2 * rows_per_wg) * sizeof(float);
+    const size_t lds_bytes = ((size_t)rows_per_wg * n + 2 * rows_per_wg + (kPrologue == 1 ? n : 0)) * sizeof(float);
     auto kernel = nq::quantize_rows_kernel<T, kDithered, kPrologue>;
     if (lds_bytes > 48 * 1024) {
         hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -435,6 +506,9 @@ extern "C" int nq_fused_input_stage(const void *x_dev, int64_t rows, int64_t n, 
     NQ_REQUIRE(mode != 1 || norm_weight_dev, NQ_ERR_ARGUMENT, "nq_fused_input_stage: mode 1 needs the norm weight");
     NQ_REQUIRE(mode != 2 || gate_dev, NQ_ERR_ARGUMENT, "nq_fused_input_stage: mode 2 needs the gate rows");
     NQ_REQUIRE(mode != 1 || (eps >= 0.0f && eps < 1.0f), NQ_ERR_ARGUMENT, "nq_fused_input_stage: eps out of range");
+    NQ_REQUIRE(nq::aligned(x_dev, 16) && nq::aligned(residual_dev, 16) && nq::aligned(residual_out_dev, 16) &&
+                   nq::aligned(norm_weight_dev, 16) && nq::aligned(gate_dev, 16) && nq::aligned(staged_out_dev, 16),
+               NQ_ERR_ARGUMENT, "nq_fused_input_stage: BF16 rows must be 16-byte aligned");
     const bool encodes = codes_dev != nullptr;
     NQ_REQUIRE(encodes || staged_out_dev || residual_out_dev, NQ_ERR_ARGUMENT,
                "nq_fused_input_stage: nothing to produce");
