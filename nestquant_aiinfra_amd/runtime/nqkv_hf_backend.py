@@ -259,6 +259,7 @@ class BatchedNQKVLlamaRunner:
         self._generation = [0] * self.batch_size
         self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor, torch.Tensor]] = {}
         self.graph_replay_counts: dict[int, int] = {}
+        self._decode_state: tuple | None = None      # (width, slots) the step tensors were last set for
         self.fused_step = None
         if fused_decode is None or fused_decode:
             from .llama_decode_step import FusedLlamaDecodeStep, UnsupportedForFusedDecode
@@ -288,6 +289,7 @@ class BatchedNQKVLlamaRunner:
         if positions is None:
             starts = torch.tensor([self.cache._host_lengths[s] for s in slots], device=self.device)
             positions = starts[:, None] + torch.arange(width, device=self.device)[None, :]
+        self._decode_state = None
         self.cache.set_batch_state(slot_ids=slots, counts=lengths)
         output = self.model(input_ids=input_ids, position_ids=positions, past_key_values=self.cache, use_cache=True)
         return output.logits
@@ -307,6 +309,7 @@ class BatchedNQKVLlamaRunner:
     def decode_eager(self, tokens: torch.Tensor, *, slots: Sequence[int], positions: torch.Tensor) -> torch.Tensor:
         """One un-captured decode step for `slots` (tokens, positions: [rows, 1])."""
         rows = len(slots)
+        self._decode_state = None
         self.cache.set_decode_execution_state(
             slot_ids=torch.tensor(list(slots), dtype=torch.int32, device=self.device),
             active_mask=torch.ones(rows, dtype=torch.bool, device=self.device))
@@ -324,6 +327,7 @@ class BatchedNQKVLlamaRunner:
                 widths.append(width)
                 width *= 2
             widths.append(self.batch_size)
+        self._decode_state = None
         meta = self.cache.manager.metadata
         saved = [t.clone() for t in (meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths)]
         stream = torch.cuda.Stream(device=self.device)
@@ -357,10 +361,14 @@ class BatchedNQKVLlamaRunner:
         graph, graph_tokens, graph_positions, logits = self._graphs[width]
         graph_tokens[:rows].copy_(tokens)
         graph_positions[:rows].copy_(positions)
-        padded_slots = list(slots) + [0] * (width - rows)
-        self.cache.set_decode_execution_state(
-            slot_ids=torch.tensor(padded_slots, dtype=torch.int32, device=self.device),
-            active_mask=torch.tensor([True] * rows + [False] * (width - rows), device=self.device))
+        state = (width, tuple(slots))
+        if state != self._decode_state:
+            # the step tensors still hold this row layout when consecutive steps decode the same slots
+            padded_slots = list(slots) + [0] * (width - rows)
+            self.cache.set_decode_execution_state(
+                slot_ids=torch.tensor(padded_slots, dtype=torch.int32, device=self.device),
+                active_mask=torch.tensor([True] * rows + [False] * (width - rows), device=self.device))
+            self._decode_state = state
         graph.replay()
         self.graph_replay_counts[width] += 1
         self.cache.note_decode_step(slots)
