@@ -44,6 +44,13 @@ def linear_bytes(m: int, k: int, n: int) -> int:
     return n * k // 2 + n * k // 32 + 4 * n + 16 + m * (k // 2 + k // 32 + 4) + 16 + 2 * m * n
 
 
+# HBM bytes per launch of the linear kernel (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by
+# what the same counters read for a 256 MiB copy; runs and factors in
+# profiles/w4a4_gemv_decode_rocprofv3.md).  Counters cannot be read from inside this process.
+MEASURED_TRAFFIC_BYTES = {"q_proj_m1": 3_416_000, "q_proj_m8": 3_894_000, "down_proj_m1": 12_950_000,
+                          "down_proj_m8": 14_116_000}
+
+
 def parse_args() -> argparse.Namespace:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -53,6 +60,8 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--profile-copy", action="store_true",
                         help="also run three 256 MiB device-to-device copies (a kernel of known traffic, "
                              "to calibrate FETCH_SIZE / WRITE_SIZE counters under rocprofv3)")
+    parser.add_argument("--only", choices=("tpot", "gemm", "attention"), default=None,
+                        help="run one of the extra measurements alone (for profiling) and print its JSON")
     parser.add_argument("--skip-extras", action="store_true",
                         help="only the headline GEMV workload (no prefill GEMM, attention, TPOT)")
     return parser.parse_args()
@@ -307,7 +316,7 @@ def tpot_extra(device, batches=(1, 8), prompt=128, generate=128):
         path = os.path.join(folder, "llama1b_random.nqmc")
         asm.write_w4_checkpoint(model, path)
         packed_bytes = os.path.getsize(path)
-        runner = asm.build_w4a4kv4_runner(model, path, capacity=max(batches), max_cache_len=prompt + generate + 16,
+        runner = asm.build_w4a4kv4_runner(model, path, capacity=max(batches), max_cache_len=prompt + generate + 48,
                                           enable_m1_down_splitk=False)
         g = torch.Generator().manual_seed(5002)
         for batch in batches:
@@ -333,8 +342,7 @@ def tpot_extra(device, batches=(1, 8), prompt=128, generate=128):
             width = next(w for w in sorted(runner._graphs) if w >= batch)
             graph = runner._graphs[width][0]
             begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            runner.cache.manager.step_active.fill_(False)        # replay without growing the cache
-            begin.record()
+            begin.record()                                       # rows stay active: 20 more tokens per slot
             for _ in range(20):
                 graph.replay()
             end.record()
@@ -364,6 +372,12 @@ def main() -> None:
         sys.exit("bench.py: no GPU visible")
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+
+    if args.only:
+        extra = {"tpot": lambda: tpot_extra(device), "gemm": lambda: prefill_gemm_extra(rt, device),
+                 "attention": lambda: attention_extra(device)}[args.only]()
+        print(json.dumps({args.only: extra}))
+        return
 
     if args.profile_copy:
         source = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=device).fill_(1)
@@ -398,7 +412,7 @@ def main() -> None:
     roofline = {
         "bound": "hbm", "kernel": f"w4a4_gemv_kernel ({dominant})",
         "achieved": per_case[dominant]["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": per_case[dominant]["GBps"] / HBM_PEAK_GBPS, "traffic": None,
+        "frac": per_case[dominant]["GBps"] / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
         "launch_us": per_case[dominant]["us"], "algorithmic_bytes": per_case[dominant]["bytes"],
     }
 

@@ -2,7 +2,9 @@
 // cold pages (4-bit E8 codes, decoded on the fly) plus its BF16 hot tail.
 //
 // Stage 1, grid = (chunks + 1, batch * kv_heads), 256 lanes.  A workgroup owns one batch
-// row, one KV head and one chunk of 16 pages (256 tokens); the extra chunk is the hot tail.
+// row, one KV head and one chunk of 2, 4, 8 or 16 pages (the fewer rows and pages a launch
+// covers, the smaller the chunks, so that short contexts still spread over the chip); the
+// extra chunk is the hot tail.
 //   * Every K and V block of the chunk is decoded exactly once and serves all query heads of
 //     the GQA group (the reference decodes it once per query head,
 //     nestquant/runtime/nqkv_attention_k1.py:243-342).
@@ -25,7 +27,7 @@
 namespace nq {
 
 constexpr int kAttnThreads = 256;
-constexpr int kAttnPagesPerChunk = 16;
+constexpr int kAttnMaxPagesPerChunk = 16;
 constexpr int kAttnMaxGroup = 8;
 
 struct AttentionArgs {
@@ -60,7 +62,7 @@ __device__ __forceinline__ float sum8(float v) {
     return v;
 }
 
-template <int D, int P, int G>     // head_dim, page_size, query heads per KV head
+template <int D, int P, int G, int kAttnPagesPerChunk>     // head_dim, page_size, query heads per KV head, pages per chunk
 __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(AttentionArgs a) {
     constexpr int kBlocks = D / 8;                       // E8 blocks per head vector
     constexpr int kTokenBlocks = P * kBlocks;            // lanes needed per page
@@ -96,6 +98,32 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
 
     // lane role inside a pass
     const int pass_page = tid / kTokenBlocks, token = (tid % kTokenBlocks) / kBlocks, blk = tid % kBlocks;
+    const int row_in_page = token * a.kv_heads + g;
+    const int64_t page_words = (int64_t)P * a.kv_heads * kBlocks, page_rows = (int64_t)P * a.kv_heads;
+
+    // Which (page, token) this lane serves in every pass, and the packed key operands of all
+    // passes, requested together so that a chunk pays one memory round trip, not one per pass.
+    bool pass_valid[kPasses];
+    int64_t pass_word[kPasses], pass_norm[kPasses];
+    uint32_t k_code[kPasses], k_ids[kPasses];
+    float k_norm[kPasses];
+#pragma unroll
+    for (int pass = 0; pass < kPasses; pass++) {
+        const int ordinal = first_page + pass * kPagesPerPass + pass_page;
+        pass_valid[pass] = is_hot ? (pass == 0 && pass_page == 0 && token < hot_len)
+                                  : (ordinal < page_count && (ordinal < page_count - 1 || token < last_len));
+        pass_word[pass] = 0;
+        pass_norm[pass] = 0;
+        k_code[pass] = 0u; k_ids[pass] = 0u; k_norm[pass] = 0.0f;
+        if (!is_hot && pass_valid[pass]) {
+            const int64_t page = a.page_indices[(int64_t)slot * a.max_pages + ordinal];
+            pass_word[pass] = page * page_words + (int64_t)row_in_page * kBlocks + blk;
+            pass_norm[pass] = page * page_rows + row_in_page;
+            k_code[pass] = a.key_codes[pass_word[pass]];
+            k_ids[pass] = a.key_beta_ids[pass_word[pass] >> 2];
+            k_norm[pass] = a.key_norms[pass_norm[pass]];
+        }
+    }
     // the group's queries, optionally Hadamard-rotated here (float32 butterflies over the head,
     // scaled by 1 / sqrt(D), rounded to the query dtype: hadamard(query.float()).to(dtype),
     // nestquant/runtime/nqkv_batched_hf_backend.py:549)
@@ -143,17 +171,16 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
         }
     __syncthreads();                                     // q_lds aliases the score buffer
     const float sqrt_d = __builtin_sqrtf((float)D);
-    const int row_in_page = token * a.kv_heads + g;
-    const int64_t page_words = (int64_t)P * a.kv_heads * kBlocks, page_rows = (int64_t)P * a.kv_heads;
 
     // ---- K pass -----------------------------------------------------------------------------
-    for (int pass = 0; pass < (is_hot ? 1 : kPasses); pass++) {
+#pragma unroll
+    for (int pass = 0; pass < kPasses; pass++) {
         const int page_in_chunk = pass * kPagesPerPass + pass_page;
-        const int ordinal = first_page + page_in_chunk;
-        bool valid;
+        const bool valid = pass_valid[pass];
         float k[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) k[j] = 0.0f;
         if (is_hot) {
-            valid = pass_page == 0 && token < hot_len;
             if (valid) {
                 const uint4 raw = *reinterpret_cast<const uint4 *>(
                     a.hot_keys + (((int64_t)slot * P + token) * a.kv_heads + g) * D + blk * 8);
@@ -164,22 +191,14 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
                     k[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
                 }
             }
-        } else {
-            valid = ordinal < page_count && (ordinal < page_count - 1 || token < last_len);
-            if (valid) {
-                const int64_t page = a.page_indices[(int64_t)slot * a.max_pages + ordinal];
-                const int64_t word = page * page_words + (int64_t)row_in_page * kBlocks + blk;
-                decode_codeword<false>(a.key_codes[word], 14.0f, 0u, k);
-                const float beta = a.key_betas[(a.key_beta_ids[word >> 2] >> (2 * (word & 3))) & 3];
-                const float back = a.key_norms[page * page_rows + row_in_page] / sqrt_d;
+        } else if (valid) {
+            decode_codeword<false>(k_code[pass], 14.0f, 0u, k);
+            const float beta = a.key_betas[(k_ids[pass] >> (2 * (blk & 3))) & 3];     // word index % 4 == blk % 4
+            const float back = k_norm[pass] / sqrt_d;
 #pragma unroll
-                for (int j = 0; j < 8; j++) k[j] = (k[j] * beta) * back;
-            }
+            for (int j = 0; j < 8; j++) k[j] = (k[j] * beta) * back;
         }
-        if (!valid) {
-#pragma unroll
-            for (int j = 0; j < 8; j++) k[j] = 0.0f;
-        }
+        // every pass writes its scores, so a hot or ragged chunk leaves no stale entry
 #pragma unroll
         for (int h = 0; h < G; h++) {
             float s = 0.0f;
@@ -189,20 +208,26 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
             if (blk == 0) scores[h][page_in_chunk * P + token] = valid ? s * a.scale : -INFINITY;
         }
     }
-    if (is_hot) {                                        // the hot chunk only fills the first page of scores
-        for (int i = tid; i < G * (kChunkTokens - P * kPagesPerPass); i += kAttnThreads) {
-            const int h = i / (kChunkTokens - P * kPagesPerPass), t = i % (kChunkTokens - P * kPagesPerPass);
-            scores[h][P * kPagesPerPass + t] = -INFINITY;
+    // the packed value operands of all passes, in flight during the softmax
+    uint32_t v_code[kPasses], v_ids[kPasses];
+    float v_norm[kPasses];
+#pragma unroll
+    for (int pass = 0; pass < kPasses; pass++) {
+        v_code[pass] = 0u; v_ids[pass] = 0u; v_norm[pass] = 0.0f;
+        if (!is_hot && pass_valid[pass]) {
+            v_code[pass] = a.value_codes[pass_word[pass]];
+            v_ids[pass] = a.value_beta_ids[pass_word[pass] >> 2];
+            v_norm[pass] = a.value_norms[pass_norm[pass]];
         }
     }
     __syncthreads();
 
     // ---- softmax over the chunk (one score per lane and head) -----------------------------------
-    static_assert(kChunkTokens == kAttnThreads, "one token per lane in the softmax phase");
+    static_assert(kChunkTokens <= kAttnThreads, "at most one token per lane in the softmax phase");
     float mine[G];
 #pragma unroll
     for (int h = 0; h < G; h++) {
-        mine[h] = scores[h][tid];
+        mine[h] = tid < kChunkTokens ? scores[h][tid] : -INFINITY;
         float m = mine[h];
 #pragma unroll
         for (int offset = 32; offset >= 1; offset >>= 1) m = fmaxf(m, __shfl_xor(m, offset, 64));
@@ -218,7 +243,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
 #pragma unroll
     for (int h = 0; h < G; h++) {
         const float p = mine[h] == -INFINITY ? 0.0f : __expf(mine[h] - chunk_max[h]);
-        scores[h][tid] = p;
+        if (tid < kChunkTokens) scores[h][tid] = p;
         float s = p;
 #pragma unroll
         for (int offset = 32; offset >= 1; offset >>= 1) s = s + __shfl_xor(s, offset, 64);
@@ -238,13 +263,12 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     for (int h = 0; h < G; h++)
 #pragma unroll
         for (int j = 0; j < 8; j++) acc[h][j] = 0.0f;
-    for (int pass = 0; pass < (is_hot ? 1 : kPasses); pass++) {
+#pragma unroll
+    for (int pass = 0; pass < kPasses; pass++) {
         const int page_in_chunk = pass * kPagesPerPass + pass_page;
-        const int ordinal = first_page + page_in_chunk;
-        bool valid;
+        const bool valid = pass_valid[pass];
         float v[8];
         if (is_hot) {
-            valid = pass_page == 0 && token < hot_len;
             if (valid) {
                 const uint4 raw = *reinterpret_cast<const uint4 *>(
                     a.hot_values + (((int64_t)slot * P + token) * a.kv_heads + g) * D + blk * 8);
@@ -255,17 +279,12 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
                     v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
                 }
             }
-        } else {
-            valid = ordinal < page_count && (ordinal < page_count - 1 || token < last_len);
-            if (valid) {
-                const int64_t page = a.page_indices[(int64_t)slot * a.max_pages + ordinal];
-                const int64_t word = page * page_words + (int64_t)row_in_page * kBlocks + blk;
-                decode_codeword<false>(a.value_codes[word], 14.0f, 0u, v);
-                const float beta = a.value_betas[(a.value_beta_ids[word >> 2] >> (2 * (word & 3))) & 3];
-                const float back = a.value_norms[page * page_rows + row_in_page] / sqrt_d;
+        } else if (valid) {
+            decode_codeword<false>(v_code[pass], 14.0f, 0u, v);
+            const float beta = a.value_betas[(v_ids[pass] >> (2 * (blk & 3))) & 3];
+            const float back = v_norm[pass] / sqrt_d;
 #pragma unroll
-                for (int j = 0; j < 8; j++) v[j] = (v[j] * beta) * back;
-            }
+            for (int j = 0; j < 8; j++) v[j] = (v[j] * beta) * back;
         }
         if (valid) {
 #pragma unroll
@@ -317,12 +336,14 @@ attention_merge_kernel(const float *__restrict__ part_max, const float *__restri
     for (int c = 0; c < parts; c++) top = fmaxf(top, m[c]);
     float denom = 0.0f, numer = 0.0f;
     if (top > -INFINITY) {
+        // empty parts hold no numerator: their (unwritten) entry is read but never used
+#pragma unroll 4
         for (int c = 0; c < parts; c++) {
-            if (s[c] > 0.0f) {
-                const float w = __expf(m[c] - top);
-                denom = denom + s[c] * w;
-                numer = numer + part_acc[(head * parts + c) * D + d] * w;
-            }
+            const float sc = s[c], value = part_acc[(head * parts + c) * D + d];
+            const bool used = sc > 0.0f;
+            const float w = used ? __expf(m[c] - top) : 0.0f;
+            denom = denom + sc * w;
+            numer = numer + (used ? value * w : 0.0f);
         }
     }
     const float result = denom > 0.0f ? numer / denom : 0.0f;      // inactive or empty rows give zeros
@@ -335,13 +356,24 @@ attention_merge_kernel(const float *__restrict__ part_max, const float *__restri
 
 namespace {
 
-int chunks_for(int max_pages) { return (max_pages + nq::kAttnPagesPerChunk - 1) / nq::kAttnPagesPerChunk; }
+// Pages per chunk: halved from 16 while the launch would have fewer than 64 (row, chunk)
+// pairs, so that a few short contexts still occupy many compute units.
+int pages_per_chunk_for(int batch, int max_pages) {
+    int pages = nq::kAttnMaxPagesPerChunk;
+    while (pages > 2 && (int64_t)batch * ((max_pages + pages - 1) / pages) < 64) pages /= 2;
+    return pages;
+}
+
+int chunks_for(int batch, int max_pages) {
+    const int pages = pages_per_chunk_for(batch, max_pages);
+    return (max_pages + pages - 1) / pages;
+}
 
 }  // namespace
 
 extern "C" size_t nq_nqkv_attention_workspace_bytes(int batch, int q_heads, int head_dim, int max_pages) {
     if (batch < 1 || q_heads < 1 || head_dim < 1 || max_pages < 1) return 0;
-    const size_t parts = (size_t)chunks_for(max_pages) + 1;
+    const size_t parts = (size_t)chunks_for(batch, max_pages) + 1;
     return (size_t)batch * q_heads * parts * ((size_t)head_dim + 2) * sizeof(float);
 }
 
@@ -393,7 +425,7 @@ extern "C" int nq_nqkv_attention_decode(
     a.hot_values = reinterpret_cast<const uint16_t *>(hot_values_dev);
     a.slot_ids = slot_ids_dev; a.active_mask = active_mask_dev;
     a.batch = batch; a.slots = slots; a.max_pages = max_pages; a.q_heads = q_heads; a.kv_heads = kv_heads;
-    a.chunks = chunks_for(max_pages); a.query_dtype = query_dtype; a.scale = scale;
+    a.chunks = chunks_for(batch, max_pages); a.query_dtype = query_dtype; a.scale = scale;
     a.rotate_query = rotate_query;
     NQ_REQUIRE((rope_cos_dev == nullptr) == (rope_sin_dev == nullptr), NQ_ERR_ARGUMENT,
                "nq_nqkv_attention_decode: rotary cos and sin tables come together");
@@ -408,12 +440,20 @@ extern "C" int nq_nqkv_attention_decode(
 
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((unsigned)parts, (unsigned)(batch * kv_heads));
-    switch (group) {
-        case 1: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, 1>), grid, dim3(nq::kAttnThreads), 0, s, a); break;
-        case 2: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, 2>), grid, dim3(nq::kAttnThreads), 0, s, a); break;
-        case 4: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, 4>), grid, dim3(nq::kAttnThreads), 0, s, a); break;
-        default: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, 8>), grid, dim3(nq::kAttnThreads), 0, s, a); break;
+#define NQ_LAUNCH_STAGE1(GROUP)                                                                                   \
+    switch (pages_per_chunk_for(batch, max_pages)) {                                                              \
+        case 2: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 2>), grid, dim3(nq::kAttnThreads), 0, s, a); break;  \
+        case 4: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 4>), grid, dim3(nq::kAttnThreads), 0, s, a); break;  \
+        case 8: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 8>), grid, dim3(nq::kAttnThreads), 0, s, a); break;  \
+        default: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 16>), grid, dim3(nq::kAttnThreads), 0, s, a); break; \
     }
+    switch (group) {
+        case 1: NQ_LAUNCH_STAGE1(1); break;
+        case 2: NQ_LAUNCH_STAGE1(2); break;
+        case 4: NQ_LAUNCH_STAGE1(4); break;
+        default: NQ_LAUNCH_STAGE1(8); break;
+    }
+#undef NQ_LAUNCH_STAGE1
     int status = nq::check_launch("nq_nqkv_attention_decode (stage 1)");
     if (status != NQ_OK) return status;
     const int64_t outputs = (int64_t)heads_total * head_dim;
