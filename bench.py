@@ -164,7 +164,7 @@ def time_kernel_alone(rt, case, copies, launches_per_graph=None):
     return begin.elapsed_time(end) * 1e-3 / (repeats * count)
 
 
-def cpu_baseline(cases, budget_s: float = 20.0):
+def cpu_baseline(cases, budget_s: float = 12.0):
     """The CPU oracle on the same workload: NQA4-encode the activation, dequantise the
     NQRT4 weight (dither regenerated), FP32 matvec.  Bounded to about `budget_s` seconds."""
     import numpy as np
@@ -193,7 +193,7 @@ def cpu_baseline(cases, budget_s: float = 20.0):
         one_step()
         steps += 1
         elapsed = time.perf_counter() - begin
-        if elapsed >= budget_s or steps >= 50:
+        if elapsed >= budget_s or steps >= 1000:
             break
     step_bytes = sum(case["bytes"] for case in cases)
     return {
