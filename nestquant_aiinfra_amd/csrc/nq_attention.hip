@@ -13,7 +13,7 @@
 //   * softmax over the chunk in LDS (FP32), then the V pass: every lane accumulates
 //     p * v for its block over the pages it visits; lanes are merged through LDS in a fixed
 //     order.  The chunk's (max, denominator, numerator[D]) go to the workspace.
-// Stage 2, one lane per output element: log-sum-exp merge of the parts in index order.
+// Stage 2, one wavefront per (row, head): log-sum-exp merge of the parts.
 // Lengths, page tables and activity flags are read on the device, so the launch is
 // replayable in a HIP graph; inactive rows produce zeros; there is no page-count limit
 // beyond the table width (the reference stops at 64 pages, nqkv_attention_k1.py:696-698).
@@ -54,11 +54,24 @@ __device__ __forceinline__ float load_query(const void *q, int dtype, int64_t i)
     return reinterpret_cast<const float *>(q)[i];
 }
 
-// sum over the 8 lanes that share a token (lane id bits 0..2)
+__device__ __forceinline__ float dpp_quad_xor1(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_quad_xor2(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_half_mirror(float v) {      // lane i <- lane 7 - i inside groups of 8
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_rotate8(float v) {          // lane i <- lane i ^ 8 inside rows of 16
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xF, 0xF, true));
+}
+
+// sum over the 8 lanes that share a token (lane id bits 0..2), register exchanges only
 __device__ __forceinline__ float sum8(float v) {
-    v = v + __shfl_xor(v, 1, 64);
-    v = v + __shfl_xor(v, 2, 64);
-    v = v + __shfl_xor(v, 4, 64);
+    v = v + dpp_quad_xor1(v);
+    v = v + dpp_quad_xor2(v);
+    v = v + dpp_half_mirror(v);
     return v;
 }
 
@@ -74,7 +87,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     __shared__ float scores[G][kChunkTokens];
     __shared__ float reduce_buf[kAttnThreads / 64][G];
     __shared__ float chunk_max[G], chunk_sum[G];
-    __shared__ float acc_lds[kAttnThreads / 64][kBlocks][G * 8];
+    __shared__ float acc_lds[kAttnThreads / 16][kBlocks][G * 8];   // one entry per 16-lane row
 
     const int tid = threadIdx.x;
     const int chunk = blockIdx.x;
@@ -127,7 +140,8 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     // the group's queries, optionally Hadamard-rotated here (float32 butterflies over the head,
     // scaled by 1 / sqrt(D), rounded to the query dtype: hadamard(query.float()).to(dtype),
     // nestquant/runtime/nqkv_batched_hf_backend.py:549)
-    float *q_lds = &scores[0][0];
+    static_assert(sizeof(acc_lds) >= sizeof(float) * G * D, "the query staging fits the accumulator buffer");
+    float *q_lds = &acc_lds[0][0][0];                    // free until the V pass ends
     for (int i = tid; i < G * D; i += kAttnThreads)
         q_lds[i] = load_query(a.query, a.query_dtype, ((int64_t)row * a.q_heads + g * G) * D + i);
     __syncthreads();
@@ -169,7 +183,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
             }
             q[h][j] = v;
         }
-    __syncthreads();                                     // q_lds aliases the score buffer
+    __syncthreads();
     const float sqrt_d = __builtin_sqrtf((float)D);
 
     // ---- K pass -----------------------------------------------------------------------------
@@ -295,24 +309,22 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
             }
         }
     }
-    // lanes that share a block index hold partial sums of the same 8 output dims: fold the
-    // tokens of a wavefront with a fixed butterfly (lane bits 3..5), then the wavefronts in order
+    // lanes that share a block index hold partial sums of the same 8 output dims: the two
+    // tokens of a 16-lane row are folded with a register exchange, rows through LDS in order
     static_assert(kBlocks == 8, "lane bits 0..2 index the block");
 #pragma unroll
     for (int h = 0; h < G; h++)
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            float v = acc[h][j];
-            v = v + __shfl_xor(v, 8, 64);
-            v = v + __shfl_xor(v, 16, 64);
-            v = v + __shfl_xor(v, 32, 64);
-            if ((tid & 63) < kBlocks) acc_lds[tid >> 6][tid & 7][h * 8 + j] = v;
+            const float v = acc[h][j] + dpp_rotate8(acc[h][j]);
+            if ((tid & 8) == 0) acc_lds[tid >> 4][tid & 7][h * 8 + j] = v;
         }
     __syncthreads();
     for (int o = tid; o < G * D; o += kAttnThreads) {
         const int h = o / D, d = o % D;
         float total = acc_lds[0][d / 8][h * 8 + d % 8];
-        for (int w = 1; w < kAttnThreads / 64; w++) total = total + acc_lds[w][d / 8][h * 8 + d % 8];
+#pragma unroll
+        for (int w = 1; w < kAttnThreads / 16; w++) total = total + acc_lds[w][d / 8][h * 8 + d % 8];
         a.part_acc[(part + (int64_t)h * (a.chunks + 1)) * D + d] = total;
     }
     if (tid < G) {
@@ -321,32 +333,44 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     }
 }
 
-// Stage 2: out[row, head, d] = sum_c acc_c * exp(max_c - max) / sum_c sum_c * exp(max_c - max)
+// Stage 2, one wavefront per (row, head): out[d] = sum_c acc_c[d] w_c / sum_c sum_c w_c with
+// w_c = exp(max_c - max).  Lanes first take one part each (max, weights), then one output
+// dimension each; every load of a phase is independent of the others.
 template <int D>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64)
 attention_merge_kernel(const float *__restrict__ part_max, const float *__restrict__ part_sum,
                        const float *__restrict__ part_acc, int parts, int64_t heads_total,
                        void *__restrict__ out, int out_dtype) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= heads_total * D) return;
-    const int64_t head = i / D;
-    const int d = (int)(i % D);
+    static_assert(D == 64, "one output dimension per lane");
+    constexpr int kMaxParts = 512;
+    __shared__ float weight[kMaxParts];
+    const int64_t head = blockIdx.x;
+    const int lane = threadIdx.x;
     const float *m = part_max + head * parts, *s = part_sum + head * parts;
     float top = -INFINITY;
-    for (int c = 0; c < parts; c++) top = fmaxf(top, m[c]);
-    float denom = 0.0f, numer = 0.0f;
-    if (top > -INFINITY) {
-        // empty parts hold no numerator: their (unwritten) entry is read but never used
-#pragma unroll 4
-        for (int c = 0; c < parts; c++) {
-            const float sc = s[c], value = part_acc[(head * parts + c) * D + d];
-            const bool used = sc > 0.0f;
-            const float w = used ? __expf(m[c] - top) : 0.0f;
-            denom = denom + sc * w;
-            numer = numer + (used ? value * w : 0.0f);
-        }
+    for (int c = lane; c < parts; c += 64) top = fmaxf(top, m[c]);
+#pragma unroll
+    for (int offset = 32; offset >= 1; offset >>= 1) top = fmaxf(top, __shfl_xor(top, offset, 64));
+    float denom = 0.0f;
+    for (int c = lane; c < parts; c += 64) {
+        const float sc = s[c];
+        const float w = (sc > 0.0f && top > -INFINITY) ? __expf(m[c] - top) : 0.0f;
+        weight[c] = w;
+        denom = denom + sc * w;
+    }
+#pragma unroll
+    for (int offset = 32; offset >= 1; offset >>= 1) denom = denom + __shfl_xor(denom, offset, 64);
+    __syncthreads();
+    // empty parts hold no numerator: their (unwritten) entry is read but never used
+    float numer = 0.0f;
+    const float *acc = part_acc + head * parts * D + lane;
+#pragma unroll 8
+    for (int c = 0; c < parts; c++) {
+        const float value = acc[(int64_t)c * D], w = weight[c];
+        numer = numer + (w > 0.0f ? value * w : 0.0f);
     }
     const float result = denom > 0.0f ? numer / denom : 0.0f;      // inactive or empty rows give zeros
+    const int64_t i = head * D + lane;
     if (out_dtype == NQ_BF16) reinterpret_cast<uint16_t *>(out)[i] = f32_to_bf16(result);
     else if (out_dtype == NQ_F16) reinterpret_cast<_Float16 *>(out)[i] = (_Float16)result;
     else reinterpret_cast<float *>(out)[i] = result;
@@ -407,6 +431,8 @@ extern "C" int nq_nqkv_attention_decode(
                    nq::aligned(hot_values_dev, 16),
                NQ_ERR_ARGUMENT, "nq_nqkv_attention_decode: page streams need 4-byte, hot tails 16-byte alignment");
     NQ_REQUIRE(isfinite(scale), NQ_ERR_ARGUMENT, "nq_nqkv_attention_decode: scale must be finite");
+    NQ_REQUIRE(chunks_for(batch, max_pages) + 1 <= 512, NQ_ERR_SHAPE,
+               "nq_nqkv_attention_decode: a page table of %d pages needs more than 512 context chunks", max_pages);
     const size_t need = nq_nqkv_attention_workspace_bytes(batch, q_heads, head_dim, max_pages);
     NQ_REQUIRE(workspace_dev && workspace_bytes >= need, NQ_ERR_WORKSPACE,
                "nq_nqkv_attention_decode: needs a %zu-byte workspace, got %zu", need, workspace_bytes);
@@ -456,8 +482,7 @@ extern "C" int nq_nqkv_attention_decode(
 #undef NQ_LAUNCH_STAGE1
     int status = nq::check_launch("nq_nqkv_attention_decode (stage 1)");
     if (status != NQ_OK) return status;
-    const int64_t outputs = (int64_t)heads_total * head_dim;
-    hipLaunchKernelGGL(nq::attention_merge_kernel<64>, dim3((unsigned)((outputs + 255) / 256)), dim3(256), 0, s,
+    hipLaunchKernelGGL(nq::attention_merge_kernel<64>, dim3((unsigned)heads_total), dim3(64), 0, s,
                        a.part_max, a.part_sum, a.part_acc, (int)parts, (int64_t)heads_total, out_dev, query_dtype);
     return nq::check_launch("nq_nqkv_attention_decode (merge)");
 }

@@ -196,6 +196,27 @@ def test_attention_ragged_batch_at_full_size(kv, oracle):
     assert torch.isfinite(out).all()
 
 
+@pytest.mark.parametrize("capacity,max_len,q_heads", [(4, 1024, 64), (8, 1024, 16), (1, 4096, 32), (2, 64, 8)])
+def test_attention_chunk_sizes(kv, oracle, capacity, max_len, q_heads):
+    """The context is cut into chunks of 2 to 16 pages depending on batch and table width:
+    every chunk size, with contexts that end inside a chunk, on a page edge and in the hot tail."""
+    rng = np.random.default_rng(capacity * max_len + q_heads)
+    manager = _manager(kv, capacity=capacity, max_len=max_len)
+    lengths = [max_len, max_len // 2 + 5, 33, 16, max_len - 16, 7, 1, max_len // 4][:capacity]
+    keys = [_bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for n in lengths]
+    values = [_bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for n in lengths]
+    for s in range(capacity):
+        manager.register(s, slot=s)
+    _append(manager, list(range(capacity)), keys, values)
+    query = _bf16(oracle.hadamard(rng.standard_normal((capacity, q_heads, DIM)).astype(np.float32))).cuda()
+    slot_ids = torch.arange(capacity, dtype=torch.int32, device="cuda")
+    active = torch.ones(capacity, dtype=torch.bool, device="cuda")
+    out = kv.nqkv_decode_attention_batched_k1(query, manager.layers[0], slot_ids=slot_ids, active_mask=active)
+    for row in range(capacity):
+        ref = _oracle_attention(oracle, query[row].cpu(), keys[row], values[row], q_heads // HEADS)
+        assert relative_error(_f32(out[row]), ref) <= 1e-2, (row, lengths[row])
+
+
 def test_pool_handles_are_generation_checked(kv):
     pool = kv.NQKVPagePool(capacity=2, page_size=PAGE, num_kv_heads=HEADS, head_dim=DIM, q=Q,
                            key_betas=KEY_BETAS, value_betas=VALUE_BETAS, device="cuda")
