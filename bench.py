@@ -291,9 +291,18 @@ def attention_extra(device):
     step_key = torch.randn(8, 1, 8, 64, device=device).to(torch.bfloat16)
     manager.step_active.fill_(False)             # time the writer's launch without growing the cache
     write = time_graph(lambda i: manager.write_layer(i % 4, step_key, step_key, rotate_keys=True), 8)
+    # chunked prefill: the last 128 tokens of every sequence attend causally to the packed cache
+    chunk = 128
+    chunk_query = hadamard_gpu(torch.randn(8, chunk, 32, 64, generator=g).to(device)).to(torch.bfloat16)
+    manager.step_active.fill_(True)
+    prefill = time_graph(lambda i: nqkv.nqkv_prefill_attention(
+        chunk_query, manager.layers[i % 4], slot_ids=slot_ids, active_mask=active, uniform_count=chunk, scale=0.125), 8)
+    prefill_flops = sum(4 * 32 * 64 * sum(n - chunk + t + 1 for t in range(chunk)) for n in lengths)
     return {"contexts": lengths, "us": seconds * 1e6, "algorithmic_bytes": bytes_moved,
             "GBps": bytes_moved / seconds / 1e9, "hbm_frac": bytes_moved / seconds / 1e9 / HBM_PEAK_GBPS,
-            "append_launch_us": write * 1e6}
+            "append_launch_us": write * 1e6,
+            "prefill_chunk128": {"us": prefill * 1e6, "flops": prefill_flops,
+                                 "TFLOPs": prefill_flops / prefill / 1e12}}
 
 
 def tpot_extra(device, batches=(1, 8), prompt=128, generate=128):

@@ -307,6 +307,31 @@ int nq_nqkv_attention_decode(
 
 size_t nq_nqkv_attention_workspace_bytes(int batch, int q_heads, int head_dim, int max_pages);
 
+/*
+ * Causal attention of a chunk of new tokens over the packed cache (prefill, chunked prefill,
+ * continuation).  Call after nq_nqkv_advance + nq_nqkv_write of the same chunk: query token t
+ * of batch row r (t < counts[r], or uniform_count when counts is NULL) sits at absolute
+ * position sequence_lengths[s] - count + t and attends to cache tokens 0 .. that position of
+ * its slot s: cold pages decoded on the fly, then the BF16 hot tail.  Tokens past counts[r]
+ * and rows that are not active give zeros.
+ *   query_dev / out_dev: BF16 [batch, tokens, q_heads, head_dim]; queries already rotated the
+ *   way the stored keys are.  FP32 online softmax; no workspace.
+ * Requires head_dim = 64, page_size = 16, q = 14, q_heads / kv_heads in {1, 2, 4, 8}.
+ * Replaces, for prompts that should not be held in BF16: the SDPA prefill over the current
+ * keys and values, nestquant/runtime/nqkv_batched_hf_backend.py:569-589 (which cannot see
+ * tokens already in the cache); semantics of the oracle nestquant/runtime/nqkv_attention.py:14-86
+ * applied per query token with a causal prefix.
+ */
+int nq_nqkv_attention_prefill(
+    const void *query_dev, const uint8_t *key_codes_dev, const uint8_t *key_beta_ids_dev, const float *key_norms_dev,
+    const uint8_t *value_codes_dev, const uint8_t *value_beta_ids_dev, const float *value_norms_dev,
+    const float *key_betas_dev, const float *value_betas_dev, const int32_t *page_indices_dev,
+    const int32_t *page_counts_dev, const int32_t *last_page_lens_dev, const int32_t *hot_lengths_dev,
+    const int32_t *sequence_lengths_dev, const void *hot_keys_dev, const void *hot_values_dev,
+    const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, const int32_t *counts_dev, int uniform_count,
+    int batch, int tokens, int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size,
+    float scale, void *out_dev, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -423,6 +423,43 @@ def nqkv_decode_attention_batched_k1(query: torch.Tensor, cache: NQKVHotColdCach
                                         rotate_query=rotate_query)
 
 
+def nqkv_prefill_attention(query: torch.Tensor, cache: NQKVHotColdCache, *, slot_ids: torch.Tensor,
+                           active_mask: torch.Tensor, counts: torch.Tensor | None = None, uniform_count: int | None = None,
+                           scale: float | None = None) -> torch.Tensor:
+    """Causal attention of a chunk of new tokens over the packed cache, after the chunk was
+    written: query BF16 [batch, tokens, query_heads, head_dim] (rotated like the stored keys);
+    row r holds counts[r] (or uniform_count) new tokens that end at the slot's sequence length.
+    Returns BF16 [batch, tokens, query_heads, head_dim]; padding tokens give zeros."""
+    if not isinstance(query, torch.Tensor) or query.ndim != 4 or query.dtype != torch.bfloat16:
+        raise ValueError("query must be BF16 [batch, tokens, query_heads, head_dim]")
+    pool, meta = cache.pool, cache.metadata
+    batch, tokens, heads, dim = query.shape
+    if query.device != pool.device or dim != pool.head_dim:
+        raise ValueError("query must match the cache CUDA device and head_dim")
+    if heads < 1 or heads % pool.num_kv_heads:
+        raise ValueError("query_heads must be a positive multiple of num_kv_heads")
+    if (counts is None) == (uniform_count is None):
+        raise ValueError("give either counts or uniform_count")
+    if slot_ids.dtype != torch.int32 or slot_ids.numel() < batch or active_mask.dtype != torch.bool:
+        raise ValueError("slot_ids must be int32 and active_mask bool, one entry per row")
+    if counts is not None and (counts.dtype != torch.int32 or counts.numel() < batch):
+        raise ValueError("counts must be int32 with one entry per row")
+    attention_scale = 1.0 / math.sqrt(dim) if scale is None else float(scale)
+    query = query.contiguous()
+    out = torch.empty_like(query)
+    _native.check(_native.library().nq_nqkv_attention_prefill(
+        query.data_ptr(), pool.key_codes.data_ptr(), pool.key_betas.data_ptr(), pool.key_norms.data_ptr(),
+        pool.value_codes.data_ptr(), pool.value_betas.data_ptr(), pool.value_norms.data_ptr(),
+        pool.beta_table.data_ptr(), pool.value_beta_table.data_ptr(), meta.page_indices.data_ptr(),
+        meta.page_counts.data_ptr(), meta.last_page_lens.data_ptr(), meta.hot_lengths.data_ptr(),
+        meta.sequence_lengths.data_ptr(), cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(),
+        slot_ids.data_ptr(), active_mask.data_ptr(), None if counts is None else counts.data_ptr(),
+        0 if uniform_count is None else int(uniform_count), batch, tokens, cache.max_sequences,
+        cache.max_pages_per_sequence, heads, pool.num_kv_heads, dim, pool.page_size, attention_scale,
+        out.data_ptr(), _native.stream_handle(query.device)))
+    return out
+
+
 # --------------------------------------------------------------------------------------
 # multi-layer manager: step bookkeeping + the ragged writer
 # --------------------------------------------------------------------------------------

@@ -21,7 +21,8 @@ import torch.nn.functional as F
 from transformers.cache_utils import Cache
 from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
 
-from .nqkv import BatchedNQKVAttentionWorkspace, BatchedNQKVCacheManager, launch_nqkv_decode_attention
+from .nqkv import (BatchedNQKVAttentionWorkspace, BatchedNQKVCacheManager, launch_nqkv_decode_attention,
+                   nqkv_prefill_attention)
 from .w4a4_linear import hadamard_cuda
 
 BATCHED_NQKV_ATTENTION_NAME = "nestquant_batched_nqkv_k1"
@@ -32,7 +33,11 @@ class BatchedNQKVLlamaCache(Cache):
 
     def __init__(self, *, capacity: int, num_layers: int, num_query_heads: int, num_kv_heads: int,
                  head_dim: int, max_cache_len: int, page_size: int, q: int, key_betas: Sequence[float],
-                 value_betas: Sequence[float], dtype: torch.dtype, device: torch.device | str) -> None:
+                 value_betas: Sequence[float], dtype: torch.dtype, device: torch.device | str,
+                 packed_prefill: bool = False) -> None:
+        """`packed_prefill` (an extension): prefill chunks attend to the packed cache instead of
+        the BF16 keys and values of the chunk, so long prompts can be fed in pieces.  A chunk
+        written into a slot that already holds tokens always takes that route."""
         super().__init__(layers=[])
         for name, value in (("capacity", capacity), ("num_layers", num_layers),
                             ("num_query_heads", num_query_heads), ("num_kv_heads", num_kv_heads),
@@ -51,6 +56,8 @@ class BatchedNQKVLlamaCache(Cache):
         self.page_size, self.dtype, self.device = page_size, dtype, self.manager.device
         self.slot_ids = torch.arange(capacity, device=self.device, dtype=torch.int32)
         self.active_mask = torch.zeros(capacity, device=self.device, dtype=torch.bool)
+        self.packed_prefill = bool(packed_prefill)
+        self._continuation = False
         self._rows = capacity
         self._tokens: int | None = None
         self._workspaces: dict[int, BatchedNQKVAttentionWorkspace] = {}
@@ -80,6 +87,7 @@ class BatchedNQKVLlamaCache(Cache):
         for slot, count in zip(slot_ids, counts):
             if self._host_lengths[slot] + count > self.manager.max_tokens:
                 raise RuntimeError("sequence would exceed max_cache_len")
+        self._continuation = any(self._host_lengths[slot] > 0 and count > 0 for slot, count in zip(slot_ids, counts))
         m = self.manager
         m.step_slot_ids[:rows].copy_(torch.tensor(list(slot_ids), dtype=torch.int32))
         m.step_counts[:rows].copy_(torch.tensor(list(counts), dtype=torch.int32))
@@ -149,9 +157,19 @@ class BatchedNQKVLlamaCache(Cache):
         return output.unsqueeze(1)                        # [rows, 1, heads, dim]
 
     def prefill(self, query_states: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor,
-                attention_mask: torch.Tensor | None, *, scale: float) -> torch.Tensor:
-        """Prefill attends to the current BF16 K/V (keys already rotated by `update`)."""
+                attention_mask: torch.Tensor | None, *, scale: float, layer_idx: int | None = None) -> torch.Tensor:
+        """Prefill attends to the current BF16 K/V (keys already rotated by `update`), or, for a
+        continuation chunk or with `packed_prefill`, causally to the packed cache that `update`
+        has just extended."""
         rotated_query = hadamard_cuda(query_states.contiguous(), compute_dtype=torch.float32)
+        if self.packed_prefill or self._continuation:
+            if layer_idx is None:
+                raise ValueError("attention over the packed cache needs the layer index")
+            self._validate_layer(layer_idx)
+            m = self.manager
+            return nqkv_prefill_attention(
+                rotated_query.transpose(1, 2).contiguous(), m.layers[layer_idx], slot_ids=m.step_slot_ids,
+                active_mask=m.step_active, counts=m.step_counts, scale=scale)
         output = F.scaled_dot_product_attention(
             rotated_query, key_states, value_states, attn_mask=attention_mask, dropout_p=0.0,
             is_causal=attention_mask is None, scale=scale,
@@ -207,7 +225,7 @@ def _batched_nqkv_attention_interface(module, query: torch.Tensor, key: torch.Te
     scale = float(kwargs.get("scaling", module.scaling))
     if query.shape[2] == 1:
         return cache.attend(module.layer_idx, query, scale=scale), None
-    return cache.prefill(query, key, value, attention_mask, scale=scale), None
+    return cache.prefill(query, key, value, attention_mask, scale=scale, layer_idx=module.layer_idx), None
 
 
 def install_batched_nqkv_llama_backend(model: torch.nn.Module, cache: BatchedNQKVLlamaCache) -> str:

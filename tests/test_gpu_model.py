@@ -122,6 +122,35 @@ def test_decode_logits_track_a_full_prefill(tiny):
     assert float(cosine) > 0.97
 
 
+def test_chunked_prefill_attends_to_the_packed_cache(tiny):
+    """A prompt fed in pieces: later pieces attend to what the cache already holds (packed pages
+    and hot tail).  Logits stay close to the one-shot prefill (which attends to BF16 K/V), and
+    decoding continues from either state."""
+    model, runner, *_ = tiny
+    ids = _prompt(1, 50, 5005)
+    whole = runner.prefill_slots(ids, slots=[3], lengths=[50])[0, 49].float()
+    runner.release_slots([3])
+    first = runner.prefill_slots(ids[:, :21], slots=[3], lengths=[21])
+    assert not runner.cache._continuation
+    second = runner.prefill_slots(ids[:, 21:44], slots=[3], lengths=[23])
+    assert runner.cache._continuation and runner.cache.manager.total_tokens(3) == 44
+    third = runner.prefill_slots(ids[:, 44:], slots=[3], lengths=[6])[0, 5].float()
+    assert torch.isfinite(first).all() and torch.isfinite(second).all()
+    cosine = torch.nn.functional.cosine_similarity(whole, third, dim=0)
+    assert float(cosine) > 0.97
+    step = runner.decode(third.argmax().reshape(1, 1), slots=[3], positions=torch.tensor([[50]], device="cuda"))
+    assert torch.isfinite(step).all() and runner.cache.manager.total_tokens(3) == 51
+    runner.release_slots([3])
+    # the same route for a whole prompt, on request
+    runner.cache.packed_prefill = True
+    try:
+        packed = runner.prefill_slots(ids, slots=[3], lengths=[50])[0, 49].float()
+    finally:
+        runner.cache.packed_prefill = False
+        runner.release_slots([3])
+    assert float(torch.nn.functional.cosine_similarity(whole, packed, dim=0)) > 0.97
+
+
 def test_dispatch_counters_and_m_routes(tiny):
     from nestquant_aiinfra_amd.models.fused_linear import FusedNQRTLinear
     model, runner, *_ = tiny

@@ -128,7 +128,8 @@ def test_ragged_writer_packs_pages_bit_exactly(kv, oracle):
     assert manager.total_tokens(0) == 0 and manager.total_tokens(3) == history[3][0].shape[0]
 
 
-def _oracle_attention(oracle, query, key_all, value_all, group):
+def _cache_view(oracle, key_all, value_all):
+    """What the cache holds for a sequence: full pages through the codec, the remainder in BF16."""
     total = key_all.shape[0]
     cold = (total // PAGE) * PAGE
     k_parts, v_parts = [], []
@@ -141,7 +142,12 @@ def _oracle_attention(oracle, query, key_all, value_all, group):
             parts.append(oracle.dequantize_rows(codes, ids, page[f"{side}_norms"], betas, Q).reshape(PAGE, HEADS, DIM))
     k_parts.append(_f32(key_all[cold:]))
     v_parts.append(_f32(value_all[cold:]))
-    return oracle.attention_dense(_f32(query), np.concatenate(k_parts), np.concatenate(v_parts))
+    return np.concatenate(k_parts), np.concatenate(v_parts)
+
+
+def _oracle_attention(oracle, query, key_all, value_all, group):
+    k_view, v_view = _cache_view(oracle, key_all, value_all)
+    return oracle.attention_dense(_f32(query), k_view, v_view)
 
 
 @pytest.mark.parametrize("q_heads", [8, 16, 32, 64])
@@ -215,6 +221,59 @@ def test_attention_chunk_sizes(kv, oracle, capacity, max_len, q_heads):
     for row in range(capacity):
         ref = _oracle_attention(oracle, query[row].cpu(), keys[row], values[row], q_heads // HEADS)
         assert relative_error(_f32(out[row]), ref) <= 1e-2, (row, lengths[row])
+
+
+@pytest.mark.parametrize("q_heads", [8, 32, 64])
+def test_prefill_attention_over_the_packed_cache(kv, oracle, q_heads):
+    """Chunks of new tokens attend causally to everything their slot holds: a fresh prompt that
+    crosses pages, a continuation of a sequence with cold pages, a one-token chunk, a padded row."""
+    rng = np.random.default_rng(100 + q_heads)
+    group = q_heads // HEADS
+    manager = _manager(kv, capacity=4, max_len=256)
+    for s in range(4):
+        manager.register(s, slot=s)
+    history = {0: 0, 1: 37, 2: 16, 3: 5}                       # tokens already in the cache per slot
+    keys = {s: _bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for s, n in history.items()}
+    values = {s: _bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for s, n in history.items()}
+    old = [s for s in history if history[s]]
+    _append(manager, old, [keys[s] for s in old], [values[s] for s in old])
+
+    slots, counts = [1, 0, 3, 2], [40, 23, 1, 0]               # the last row is padding only
+    new_k = [_bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for n in counts]
+    new_v = [_bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for n in counts]
+    live = [i for i, n in enumerate(counts) if n]
+    width = max(counts)
+    key = torch.zeros((4, width, HEADS, DIM), dtype=torch.bfloat16)
+    value = torch.zeros_like(key)
+    for i in live:
+        key[i, : counts[i]], value[i, : counts[i]] = new_k[i], new_v[i]
+    manager.step_slot_ids[:4] = torch.tensor(slots, dtype=torch.int32)
+    manager.step_active[:4] = torch.tensor([n > 0 for n in counts])
+    manager.step_counts[:4] = torch.tensor(counts, dtype=torch.int32)
+    manager.begin_step(rows=4, uniform_count=None)
+    manager.write_layer(0, key.cuda(), value.cuda())
+
+    query = _bf16(oracle.hadamard(rng.standard_normal((4, width, q_heads, DIM)).astype(np.float32))).cuda()
+    out = kv.nqkv_prefill_attention(query, manager.layers[0], slot_ids=manager.step_slot_ids, active_mask=manager.step_active,
+                                    counts=manager.step_counts)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (4, width, q_heads, DIM)
+    for i in live:
+        slot = slots[i]
+        all_k = torch.cat([keys[slot], new_k[i]]) if history[slot] else new_k[i]
+        all_v = torch.cat([values[slot], new_v[i]]) if history[slot] else new_v[i]
+        k_view, v_view = _cache_view(oracle, all_k, all_v)      # pages complete after the chunk are already packed
+        for t in sorted({0, counts[i] // 2, counts[i] - 1}):
+            visible = history[slot] + t + 1
+            ref = oracle.attention_dense(_f32(query[i, t].cpu()), k_view[:visible], v_view[:visible])
+            assert relative_error(_f32(out[i, t]), ref) <= 1e-2, (i, t)
+        assert not out[i, counts[i]:].any()                     # padding tokens give zeros
+    assert not out[3].any()
+    # the last token of a chunk sees exactly what a decode step at that position sees
+    i = 0
+    decode = kv.nqkv_decode_attention_batched_k1(
+        query[:, counts[i] - 1].contiguous(), manager.layers[0], slot_ids=manager.step_slot_ids[:4].clone(),
+        active_mask=torch.tensor([True, False, False, False], device="cuda"))
+    assert relative_error(_f32(out[i, counts[i] - 1]), _f32(decode[0])) <= 2e-2
 
 
 def test_pool_handles_are_generation_checked(kv):
