@@ -7,21 +7,28 @@
 // copy of the context is ever materialised (the reference's prefill runs SDPA on the BF16
 // keys and values of the current prompt only, nestquant/runtime/nqkv_batched_hf_backend.py:569-589).
 //
-// grid = (query tiles, batch * kv_heads), 256 lanes.  A workgroup owns 64 query vectors: the
-// G query heads of one KV head for 64 / G consecutive tokens.  Lane (v, part) = (tid / 4,
-// tid % 4) holds query vector v's dims 16 part .. + 16, its running max / denominator and
-// 16 output dims.  Per page of 16 tokens:
+// grid = (query tiles, batch * kv_heads), 256 lanes.  A workgroup owns 64 query vectors (the
+// G query heads of one KV head for 64 / G consecutive tokens), 16 per wavefront.  Pages are
+// taken two at a time; per page of 16 tokens:
 //   * every lane decodes one E8 block of the page (lanes 0..127 keys, 128..255 values; the
-//     exact float order of nq_e8.hip.h, as in the decode kernel) into LDS as float32: a page
-//     is decoded once per workgroup and serves all 64 query vectors;
-//   * scores: 16 partial dot products per lane, summed over the 4 lanes of a vector with two
-//     register exchanges; causal and length masks; online softmax in FP32;
-//   * output: 16 x 16 multiply-adds per lane from the value page in LDS.
-// Pages past the last position of the tile are never visited.
+//     exact float order of nq_e8.hip.h, as in the decode kernel) and stores it to LDS as BF16:
+//     keys row-major, values transposed.  A page is decoded once per workgroup and serves
+//     all 64 query vectors; its packed operands are requested one trip ahead.
+//   * scores on the matrix cores, transposed: S^T[token, vector] = K . Q^T with two
+//     v_mfma_f32_16x16x32_bf16 per wavefront (Q^T fragments live in registers for the whole
+//     kernel).  A lane then holds 4 tokens of one query vector: causal and length masks, the
+//     online softmax in FP32 (two cross-row exchanges per statistic), and its four
+//     probabilities are already laid out as the B operand of the next product;
+//   * output, transposed: O^T[dim, vector] += V^T . P^T over the pair's 32 tokens, four
+//     v_mfma_f32_16x16x32_bf16.
+// LDS tiles are double-buffered (one barrier per pair of pages).  Pages past the last position of the
+// tile are never visited.
 #include "nq_e8.hip.h"
 #include "nq_host.h"
 
 #include <math.h>
+
+#include <type_traits>
 
 namespace nq {
 
@@ -41,25 +48,29 @@ struct PrefillAttentionArgs {
     float scale;
 };
 
-__device__ __forceinline__ float quad_sum(float v) {
-    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
-    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
-    return v;
-}
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// the value held by the lane whose id differs in bit 4 / bit 5
+__device__ __forceinline__ float lane_xor16(float v) { return __shfl_xor(v, 16, 64); }
+__device__ __forceinline__ float lane_xor32(float v) { return __shfl_xor(v, 32, 64); }
 
 template <int D, int P, int G>
 __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(PrefillAttentionArgs a) {
     static_assert(D == 64 && P == 16, "lane roles assume 64-dim heads and 16-token pages");
     constexpr int kBlocks = D / 8;
     constexpr int kTileTokens = 64 / G;                  // query tokens per workgroup
-    __shared__ float k_page[P][D + 4], v_page[P][D + 4];  // padded rows: the 4 parts of a vector hit distinct banks
+    constexpr int kKeyRow = D + 8;                       // BF16 elements per key row: 144 bytes, conflict-free 16-byte reads
+    __shared__ __attribute__((aligned(16))) uint16_t k_page[2][2][P][kKeyRow];   // [buffer][page of the pair][token][dim]
+    __shared__ __attribute__((aligned(16))) uint16_t v_page[2][2][D][P];         // transposed: [dim][token]
 
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = blockIdx.y / a.kv_heads, g = blockIdx.y % a.kv_heads;
-    const int vec = tid >> 2, part = tid & 3;
-    const int t = blockIdx.x * kTileTokens + vec / G;    // token of this lane's query vector inside the chunk
+    const int vec = 16 * wave + (lane & 15);             // this lane's query vector (column of S^T and O^T)
+    const int quarter = lane >> 4;                       // which 4 tokens / 4 dims of a 16-row tile the lane holds
+    const int t = blockIdx.x * kTileTokens + vec / G;    // token of the query vector inside the chunk
     const int head = g * G + vec % G;
-    const int64_t q_at = (((int64_t)row * a.tokens + t) * a.q_heads + head) * D + 16 * part;
+    const int64_t q_at = (((int64_t)row * a.tokens + t) * a.q_heads + head) * D;
 
     int slot = a.slot_ids[row];
     const bool live = a.active_mask[row] && slot >= 0 && slot < a.slots;
@@ -70,7 +81,7 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     if (count > length) count = length;
     if (!live) count = 0;
     const int start = length - count;
-    const bool has_query = t < count && t < a.tokens;
+    const bool has_query = t < count;
     const int position = start + t;                      // attends to cache tokens 0 .. position
     const int page_count = a.page_counts[slot], last_len = a.last_page_lens[slot], hot_len = a.hot_lengths[slot];
 
@@ -79,119 +90,170 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     const int tile_last_token = (tile_first + kTileTokens < count ? tile_first + kTileTokens : count) - 1;
     const int pages_needed = tile_last_token >= tile_first ? (start + tile_last_token) / P + 1 : 0;
 
-    float q[16], o[16];
+    // Q^T fragments of the two 32-dim steps: lane (vector, quarter) holds dims 32 step + 8 quarter .. + 8
+    bf16x8 q_frag[2];
 #pragma unroll
-    for (int j = 0; j < 16; j++) { q[j] = 0.0f; o[j] = 0.0f; }
-    if (has_query) {
-        const uint4 lo = *reinterpret_cast<const uint4 *>(a.query + q_at), hi = *reinterpret_cast<const uint4 *>(a.query + q_at + 8);
-        const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            q[2 * j] = __uint_as_float(w[j] << 16) * a.scale;
-            q[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u) * a.scale;
-        }
+    for (int step = 0; step < 2; step++) {
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (has_query) raw = *reinterpret_cast<const uint4 *>(a.query + q_at + 32 * step + 8 * quarter);
+        q_frag[step] = __builtin_bit_cast(bf16x8, raw);
     }
+    floatx4 o[4];                                        // O^T tiles: dims 16 tile + 4 quarter + r of this lane's vector
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     float running_max = -INFINITY, denom = 0.0f;
 
     // decode role: lanes 0..127 keys, 128..255 values; (token, block) of the page
     const bool decodes_values = tid >= 128;
     const int dec_token = (tid & 127) >> 3, dec_blk = tid & 7;
     const int row_in_page = dec_token * a.kv_heads + g;
-    const int64_t page_words = (int64_t)P * a.kv_heads * kBlocks, page_rows = (int64_t)P * a.kv_heads;
+    const uint32_t page_words = (uint32_t)(P * a.kv_heads * kBlocks), page_rows = (uint32_t)(P * a.kv_heads);
+    const uint32_t lane_word = (uint32_t)(row_in_page * kBlocks + dec_blk);
+    const uint32_t *side_codes = decodes_values ? a.value_codes : a.key_codes;
+    const uint8_t *side_ids = decodes_values ? a.value_beta_ids : a.key_beta_ids;
+    const float *side_norms = decodes_values ? a.value_norms : a.key_norms;
+    const float *side_betas = decodes_values ? a.value_betas : a.key_betas;
+    const uint16_t *side_hot = (decodes_values ? a.hot_values : a.hot_keys) +
+                               (((int64_t)slot * P + dec_token) * a.kv_heads + g) * D + dec_blk * 8;
+    const float beta_table[4] = {side_betas[0], side_betas[1], side_betas[2], side_betas[3]};
     const float sqrt_d = __builtin_sqrtf((float)D);
+    const int32_t *slot_pages = a.page_indices + (int64_t)slot * a.max_pages;
 
-    for (int ordinal = 0; ordinal < pages_needed; ordinal++) {
-        // ---- stage the page ---------------------------------------------------------------------
-        float staged[8];
+    struct ColdOperands { uint32_t code, ids; float norm; };
+    auto request_cold = [&](int ordinal) {               // operands of this lane's block of a full cold page
+        const uint32_t page = (uint32_t)slot_pages[ordinal];
+        const uint32_t word = page * page_words + lane_word;
+        return ColdOperands{side_codes[word], (uint32_t)side_ids[word >> 2], side_norms[page * page_rows + (uint32_t)row_in_page]};
+    };
+    auto decode_cold = [&](const ColdOperands &operands) {
+        float v[8];
+        decode_codeword<false>(operands.code, 14.0f, 0u, v);
+        const float beta = beta_table[(operands.ids >> (2 * (dec_blk & 3))) & 3];
+        const float back = operands.norm / sqrt_d;
+        const bf16x2 h0 = pack_bf16x2((v[0] * beta) * back, (v[1] * beta) * back);
+        const bf16x2 h1 = pack_bf16x2((v[2] * beta) * back, (v[3] * beta) * back);
+        const bf16x2 h2 = pack_bf16x2((v[4] * beta) * back, (v[5] * beta) * back);
+        const bf16x2 h3 = pack_bf16x2((v[6] * beta) * back, (v[7] * beta) * back);
+        return make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
+                          __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
+    };
+    auto write_page = [&](int buf, int half, const uint4 packed) {
+        if (decodes_values) {
+            const uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
 #pragma unroll
-        for (int j = 0; j < 8; j++) staged[j] = 0.0f;
-        const bool cold = ordinal < page_count;
-        const int tokens_here = cold ? (ordinal < page_count - 1 ? P : last_len) : (ordinal == page_count ? hot_len : 0);
-        if (dec_token < tokens_here) {
-            if (cold) {
-                const int64_t page = a.page_indices[(int64_t)slot * a.max_pages + ordinal];
-                const int64_t word = page * page_words + (int64_t)row_in_page * kBlocks + dec_blk;
-                const uint32_t code = decodes_values ? a.value_codes[word] : a.key_codes[word];
-                const uint32_t ids = decodes_values ? a.value_beta_ids[word >> 2] : a.key_beta_ids[word >> 2];
-                const float norm = decodes_values ? a.value_norms[page * page_rows + row_in_page]
-                                                  : a.key_norms[page * page_rows + row_in_page];
-                decode_codeword<false>(code, 14.0f, 0u, staged);
-                const float beta = (decodes_values ? a.value_betas : a.key_betas)[(ids >> (2 * (dec_blk & 3))) & 3];
-                const float back = norm / sqrt_d;
+            for (int j = 0; j < 4; j++) {
+                v_page[buf][half][dec_blk * 8 + 2 * j][dec_token] = (uint16_t)(w[j] & 0xffffu);
+                v_page[buf][half][dec_blk * 8 + 2 * j + 1][dec_token] = (uint16_t)(w[j] >> 16);
+            }
+        } else {
+            *reinterpret_cast<uint4 *>(&k_page[buf][half][dec_token][dec_blk * 8]) = packed;
+        }
+    };
+    auto tokens_of = [&](int ordinal) {
+        if (ordinal >= pages_needed) return 0;
+        if (ordinal < page_count) return ordinal < page_count - 1 ? P : last_len;
+        return ordinal == page_count ? hot_len : 0;
+    };
+    // scores, online softmax and output update for the two staged pages of buffer `buf`;
+    // kMasked = false when all 32 tokens exist and are visible to every vector of the tile
+    auto attend = [&](auto masked, int buf, int first) {
+        constexpr bool kMasked = decltype(masked)::value;
+        float s[8], trip_max = -INFINITY;
 #pragma unroll
-                for (int j = 0; j < 8; j++) staged[j] = (staged[j] * beta) * back;
-            } else {
-                const uint16_t *hot = decodes_values ? a.hot_values : a.hot_keys;
-                const uint4 raw = *reinterpret_cast<const uint4 *>(
-                    hot + (((int64_t)slot * P + dec_token) * a.kv_heads + g) * D + dec_blk * 8);
-                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+        for (int half = 0; half < 2; half++) {
+            floatx4 st = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    staged[2 * j] = __uint_as_float(w[j] << 16);
-                    staged[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
-                }
+            for (int step = 0; step < 2; step++) {
+                const bf16x8 k_frag = __builtin_bit_cast(
+                    bf16x8, *reinterpret_cast<const uint4 *>(&k_page[buf][half][lane & 15][32 * step + 8 * quarter]));
+                st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag, q_frag[step], st, 0, 0, 0);
+            }
+            const int tokens_here = kMasked ? tokens_of(first + half) : P;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int tok = 4 * quarter + r;
+                const bool visible = !kMasked || (has_query && tok < tokens_here && (first + half) * P + tok <= position);
+                s[4 * half + r] = visible ? st[r] * a.scale : -INFINITY;
+                trip_max = fmaxf(trip_max, s[4 * half + r]);
             }
         }
-        __syncthreads();                                 // the previous page has been consumed
-        {
-            float *dst = decodes_values ? &v_page[dec_token][dec_blk * 8] : &k_page[dec_token][dec_blk * 8];
-            *reinterpret_cast<float4 *>(dst) = make_float4(staged[0], staged[1], staged[2], staged[3]);
-            *reinterpret_cast<float4 *>(dst + 4) = make_float4(staged[4], staged[5], staged[6], staged[7]);
+        trip_max = fmaxf(trip_max, lane_xor16(trip_max));
+        trip_max = fmaxf(trip_max, lane_xor32(trip_max));
+        const float new_max = fmaxf(running_max, trip_max);
+        // a vector that has seen nothing yet keeps max = -inf: exponents are forced to zero weight
+        const float keep = (kMasked && new_max == -INFINITY) ? 1.0f : __expf(running_max - new_max);
+        float p[8], trip_sum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+            p[r] = (kMasked && s[r] == -INFINITY) ? 0.0f : __expf(s[r] - new_max);
+            trip_sum = trip_sum + p[r];
         }
-        __syncthreads();
+        trip_sum = trip_sum + lane_xor16(trip_sum);
+        trip_sum = trip_sum + lane_xor32(trip_sum);
+        denom = denom * keep + trip_sum;
+        running_max = new_max;
+        // B operand of the 32-deep product: slots 0..3 = this lane's tokens of the first page, 4..7 of the second
+        const uint4 p_bits = make_uint4(__builtin_bit_cast(uint32_t, pack_bf16x2(p[0], p[1])),
+                                        __builtin_bit_cast(uint32_t, pack_bf16x2(p[2], p[3])),
+                                        __builtin_bit_cast(uint32_t, pack_bf16x2(p[4], p[5])),
+                                        __builtin_bit_cast(uint32_t, pack_bf16x2(p[6], p[7])));
+        const bf16x8 p_frag = __builtin_bit_cast(bf16x8, p_bits);
+#pragma unroll
+        for (int tile = 0; tile < 4; tile++) {
+            const uint2 v0 = *reinterpret_cast<const uint2 *>(&v_page[buf][0][16 * tile + (lane & 15)][4 * quarter]);
+            const uint2 v1 = *reinterpret_cast<const uint2 *>(&v_page[buf][1][16 * tile + (lane & 15)][4 * quarter]);
+#pragma unroll
+            for (int r = 0; r < 4; r++) o[tile][r] = o[tile][r] * keep;
+            o[tile] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, make_uint4(v0.x, v0.y, v1.x, v1.y)),
+                                                             p_frag, o[tile], 0, 0, 0);
+        }
+    };
 
-        // ---- scores of this vector against the 16 tokens ------------------------------------------
-        float s[P];
-        float page_max = -INFINITY;
-#pragma unroll
-        for (int tok = 0; tok < P; tok++) {
-            const float *k = &k_page[tok][16 * part];
-            float partial = 0.0f;
-#pragma unroll
-            for (int j = 0; j < 16; j += 4) {
-                const float4 kv = *reinterpret_cast<const float4 *>(k + j);
-                partial = __builtin_fmaf(q[j], kv.x, partial);
-                partial = __builtin_fmaf(q[j + 1], kv.y, partial);
-                partial = __builtin_fmaf(q[j + 2], kv.z, partial);
-                partial = __builtin_fmaf(q[j + 3], kv.w, partial);
+    // Leading trips whose 32 tokens are full cold pages visible to the whole tile: no masks, operands
+    // requested one trip ahead.  The rest (causal edge, partial page, hot tail) takes the masked path.
+    const int visible_pages = (start + tile_first + 1) / P;
+    const int full_cold_pages = page_count > 0 ? page_count - (last_len == P ? 0 : 1) : 0;
+    int fast_pages = visible_pages < full_cold_pages ? visible_pages : full_cold_pages;
+    if (fast_pages > pages_needed) fast_pages = pages_needed;
+    if (tile_first >= count || fast_pages < 0) fast_pages = 0;
+    fast_pages &= ~1;
+    int trip = 0;
+    if (fast_pages > 0) {
+        ColdOperands next[2] = {request_cold(0), request_cold(1)};
+        for (int first = 0; first < fast_pages; first += 2, trip++) {
+            const ColdOperands now[2] = {next[0], next[1]};
+            if (first + 2 < fast_pages) {
+                next[0] = request_cold(first + 2);
+                next[1] = request_cold(first + 3);
             }
-            const float total = quad_sum(partial);
-            const int index = ordinal * P + tok;
-            const bool visible = has_query && tok < tokens_here && index <= position;
-            s[tok] = visible ? total : -INFINITY;
-            page_max = fmaxf(page_max, s[tok]);
-        }
-        if (page_max > -INFINITY) {                      // divergent per vector, no barrier inside
-            const float new_max = fmaxf(running_max, page_max);
-            const float keep = __expf(running_max - new_max);        // exp(-inf) = 0 on the first visible page
-            denom = denom * keep;
-#pragma unroll
-            for (int j = 0; j < 16; j++) o[j] = o[j] * keep;
-#pragma unroll
-            for (int tok = 0; tok < P; tok++) {
-                const float p = s[tok] == -INFINITY ? 0.0f : __expf(s[tok] - new_max);
-                denom = denom + p;
-                const float *v = &v_page[tok][16 * part];
-#pragma unroll
-                for (int j = 0; j < 16; j += 4) {
-                    const float4 vv = *reinterpret_cast<const float4 *>(v + j);
-                    o[j] = __builtin_fmaf(p, vv.x, o[j]);
-                    o[j + 1] = __builtin_fmaf(p, vv.y, o[j + 1]);
-                    o[j + 2] = __builtin_fmaf(p, vv.z, o[j + 2]);
-                    o[j + 3] = __builtin_fmaf(p, vv.w, o[j + 3]);
-                }
-            }
-            running_max = new_max;
+            write_page(trip & 1, 0, decode_cold(now[0]));
+            write_page(trip & 1, 1, decode_cold(now[1]));
+            __syncthreads();     // pages staged; also orders the reads of this buffer two trips ago before these writes
+            attend(std::false_type{}, trip & 1, first);
         }
     }
-    if (t < a.tokens) {
-        const float inv = denom > 0.0f ? 1.0f / denom : 0.0f;          // padding tokens and inactive rows give zeros
-        uint32_t packed[8];
+    for (int first = fast_pages; first < pages_needed; first += 2, trip++) {
 #pragma unroll
-        for (int j = 0; j < 8; j++)
-            packed[j] = (uint32_t)f32_to_bf16(o[2 * j] * inv) | ((uint32_t)f32_to_bf16(o[2 * j + 1] * inv) << 16);
-        *reinterpret_cast<uint4 *>(a.out + q_at) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
-        *reinterpret_cast<uint4 *>(a.out + q_at + 8) = make_uint4(packed[4], packed[5], packed[6], packed[7]);
+        for (int half = 0; half < 2; half++) {
+            const int ordinal = first + half;
+            uint4 packed = make_uint4(0, 0, 0, 0);
+            if (dec_token < tokens_of(ordinal)) {
+                if (ordinal < page_count) packed = decode_cold(request_cold(ordinal));
+                else packed = *reinterpret_cast<const uint4 *>(side_hot);
+            }
+            write_page(trip & 1, half, packed);
+        }
+        __syncthreads();
+        attend(std::true_type{}, trip & 1, first);
+    }
+    if (t < a.tokens) {
+        const float inv = (has_query && denom > 0.0f) ? 1.0f / denom : 0.0f;   // padding tokens and inactive rows give zeros
+#pragma unroll
+        for (int tile = 0; tile < 4; tile++) {
+            const uint32_t lo = (uint32_t)f32_to_bf16(o[tile][0] * inv) | ((uint32_t)f32_to_bf16(o[tile][1] * inv) << 16);
+            const uint32_t hi = (uint32_t)f32_to_bf16(o[tile][2] * inv) | ((uint32_t)f32_to_bf16(o[tile][3] * inv) << 16);
+            *reinterpret_cast<uint2 *>(a.out + q_at + 16 * tile + 4 * quarter) = make_uint2(lo, hi);
+        }
     }
 }
 
@@ -220,7 +282,7 @@ extern "C" int nq_nqkv_attention_prefill(
                    page_counts_dev && last_page_lens_dev && hot_lengths_dev && sequence_lengths_dev && hot_keys_dev &&
                    hot_values_dev && slot_ids_dev && active_mask_dev && out_dev,
                NQ_ERR_ARGUMENT, "nq_nqkv_attention_prefill: null pointer");
-    NQ_REQUIRE(nq::aligned(query_dev, 16) && nq::aligned(out_dev, 16) && nq::aligned(key_codes_dev, 4) &&
+    NQ_REQUIRE(nq::aligned(query_dev, 16) && nq::aligned(out_dev, 8) && nq::aligned(key_codes_dev, 4) &&
                    nq::aligned(value_codes_dev, 4) && nq::aligned(hot_keys_dev, 16) && nq::aligned(hot_values_dev, 16),
                NQ_ERR_ARGUMENT, "nq_nqkv_attention_prefill: queries, output and hot tails need 16-byte, page streams 4-byte alignment");
     NQ_REQUIRE(isfinite(scale), NQ_ERR_ARGUMENT, "nq_nqkv_attention_prefill: scale must be finite");
