@@ -7,13 +7,13 @@
 // copy of the context is ever materialised (the reference's prefill runs SDPA on the BF16
 // keys and values of the current prompt only, nestquant/runtime/nqkv_batched_hf_backend.py:569-589).
 //
-// grid = (query tiles, batch * kv_heads), 256 lanes.  A workgroup owns 64 query vectors (the
-// G query heads of one KV head for 64 / G consecutive tokens), 16 per wavefront.  Pages are
-// taken two at a time; per page of 16 tokens:
-//   * every lane decodes one E8 block of the page (lanes 0..127 keys, 128..255 values; the
+// grid = (query tiles, batch * kv_heads), 512 lanes.  A workgroup owns 128 query vectors (the
+// G query heads of one KV head for 128 / G consecutive tokens), 16 per wavefront.  Pages are
+// taken two at a time, one per half of the workgroup; per page of 16 tokens:
+//   * every lane decodes one E8 block of the page (128 lanes keys, 128 lanes values; the
 //     exact float order of nq_e8.hip.h, as in the decode kernel) and stores it to LDS as BF16:
 //     keys row-major, values transposed.  A page is decoded once per workgroup and serves
-//     all 64 query vectors; its packed operands are requested one trip ahead.
+//     all 128 query vectors; its packed operands are requested one trip ahead.
 //   * scores on the matrix cores, transposed: S^T[token, vector] = K . Q^T with two
 //     v_mfma_f32_16x16x32_bf16 per wavefront (Q^T fragments live in registers for the whole
 //     kernel).  A lane then holds 4 tokens of one query vector: causal and length masks, the
@@ -32,7 +32,7 @@
 
 namespace nq {
 
-constexpr int kPrefillThreads = 256;
+constexpr int kPrefillThreads = 512;
 
 struct PrefillAttentionArgs {
     const uint16_t *query;             // BF16 [batch, tokens, q_heads, D], already rotated like the stored keys
@@ -59,7 +59,7 @@ template <int D, int P, int G>
 __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(PrefillAttentionArgs a) {
     static_assert(D == 64 && P == 16, "lane roles assume 64-dim heads and 16-token pages");
     constexpr int kBlocks = D / 8;
-    constexpr int kTileTokens = 64 / G;                  // query tokens per workgroup
+    constexpr int kTileTokens = 128 / G;                 // query tokens per workgroup
     constexpr int kKeyRow = D + 8;                       // BF16 elements per key row: 144 bytes, conflict-free 16-byte reads
     __shared__ __attribute__((aligned(16))) uint16_t k_page[2][2][P][kKeyRow];   // [buffer][page of the pair][token][dim]
     __shared__ __attribute__((aligned(16))) uint16_t v_page[2][2][D][P];         // transposed: [dim][token]
@@ -103,8 +103,10 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     for (int i = 0; i < 4; i++) o[i] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     float running_max = -INFINITY, denom = 0.0f;
 
-    // decode role: lanes 0..127 keys, 128..255 values; (token, block) of the page
-    const bool decodes_values = tid >= 128;
+    // decode role: lanes 0..255 stage the first page of a pair, 256..511 the second; of each
+    // half, 128 lanes take keys and 128 values; (token, block) of the page
+    const int dec_half = tid >> 8;
+    const bool decodes_values = (tid & 255) >= 128;
     const int dec_token = (tid & 127) >> 3, dec_blk = tid & 7;
     const int row_in_page = dec_token * a.kv_heads + g;
     const uint32_t page_words = (uint32_t)(P * a.kv_heads * kBlocks), page_rows = (uint32_t)(P * a.kv_heads);
@@ -219,29 +221,24 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     fast_pages &= ~1;
     int trip = 0;
     if (fast_pages > 0) {
-        ColdOperands next[2] = {request_cold(0), request_cold(1)};
+        ColdOperands next = request_cold(dec_half);
         for (int first = 0; first < fast_pages; first += 2, trip++) {
-            const ColdOperands now[2] = {next[0], next[1]};
-            if (first + 2 < fast_pages) {
-                next[0] = request_cold(first + 2);
-                next[1] = request_cold(first + 3);
-            }
-            write_page(trip & 1, 0, decode_cold(now[0]));
-            write_page(trip & 1, 1, decode_cold(now[1]));
+            const ColdOperands now = next;
+            if (first + 2 < fast_pages) next = request_cold(first + 2 + dec_half);
+            write_page(trip & 1, dec_half, decode_cold(now));
             __syncthreads();     // pages staged; also orders the reads of this buffer two trips ago before these writes
             attend(std::false_type{}, trip & 1, first);
         }
     }
     for (int first = fast_pages; first < pages_needed; first += 2, trip++) {
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
-            const int ordinal = first + half;
+        {
+            const int ordinal = first + dec_half;
             uint4 packed = make_uint4(0, 0, 0, 0);
             if (dec_token < tokens_of(ordinal)) {
                 if (ordinal < page_count) packed = decode_cold(request_cold(ordinal));
                 else packed = *reinterpret_cast<const uint4 *>(side_hot);
             }
-            write_page(trip & 1, half, packed);
+            write_page(trip & 1, dec_half, packed);
         }
         __syncthreads();
         attend(std::true_type{}, trip & 1, first);
@@ -303,7 +300,7 @@ extern "C" int nq_nqkv_attention_prefill(
     a.slot_ids = slot_ids_dev; a.counts = counts_dev; a.active_mask = active_mask_dev;
     a.batch = batch; a.tokens = tokens; a.uniform_count = uniform_count; a.slots = slots; a.max_pages = max_pages;
     a.q_heads = q_heads; a.kv_heads = kv_heads; a.scale = scale;
-    const int tile_tokens = 64 / group;
+    const int tile_tokens = 128 / group;
     const dim3 grid((unsigned)((tokens + tile_tokens - 1) / tile_tokens), (unsigned)(batch * kv_heads));
     hipStream_t s = (hipStream_t)stream;
     switch (group) {
