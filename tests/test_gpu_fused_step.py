@@ -217,3 +217,47 @@ def test_fused_decode_step_tracks_the_module_graph(tmp_path):
     assert relative_error(bits(fused), bits(reference)) < 0.08
     # the first step starts from identical state: only reduction order separates the two
     assert relative_error(bits(fused[0]), bits(reference[0])) < 0.03
+
+
+def test_fused_decode_step_with_more_than_eight_rows(tmp_path):
+    """Above eight rows the step's linears run on the MFMA kernel instead of the grouped GEMV."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
+    from nestquant_aiinfra_amd.runtime.nqkv_hf_backend import BatchedNQKVLlamaRunner
+
+    torch.manual_seed(5003)
+    config = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                         num_key_value_heads=2, head_dim=64, vocab_size=128, max_position_embeddings=512,
+                         rope_theta=500000.0, tie_word_embeddings=True)
+    model = LlamaForCausalLM(config).to(torch.bfloat16).cuda().eval()
+    path = tmp_path / "tiny.nqmc"
+    asm.write_w4_checkpoint(model, path)
+    rows = 12
+    runner = asm.build_w4a4kv4_runner(model, path, capacity=rows, max_cache_len=64)
+    modular = BatchedNQKVLlamaRunner(model, runner.cache, fused_decode=False)
+    g = torch.Generator().manual_seed(5004)
+    ids = torch.randint(0, 128, (rows, 18), generator=g).cuda()
+    lengths = [18 - (i % 5) for i in range(rows)]
+    logits = runner.prefill_slots(ids, slots=list(range(rows)), lengths=lengths)
+    token = torch.stack([logits[i, n - 1].argmax() for i, n in enumerate(lengths)]).reshape(rows, 1)
+    position = torch.tensor(lengths, device="cuda").reshape(rows, 1)
+    cache = runner.cache
+    meta = cache.manager.metadata
+    tensors = [meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths]
+    for layer in cache.manager.layers:
+        tensors += [layer.hot_keys, layer.hot_values]
+    saved, host = [t.clone() for t in tensors], list(cache._host_lengths)
+    fused = runner.decode_eager(token, slots=list(range(rows)), positions=position).float().clone()
+    for tensor, value in zip(tensors, saved):
+        tensor.copy_(value)
+    cache._host_lengths[:] = host
+    reference = modular.decode_eager(token, slots=list(range(rows)), positions=position).float()
+    assert torch.isfinite(fused).all() and tuple(fused.shape) == (rows, 1, 128)
+    assert relative_error(bits(fused), bits(reference)) < 0.03
+    # and through the captured graph of that width
+    for tensor, value in zip(tensors, saved):
+        tensor.copy_(value)
+    cache._host_lengths[:] = host
+    runner.capture(widths=[rows])
+    replayed = runner.decode(token, slots=list(range(rows)), positions=position).float()
+    assert torch.equal(replayed, fused)
