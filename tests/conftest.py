@@ -34,6 +34,14 @@ def golden():
 
 
 @pytest.fixture(scope="session")
+def golden_long_rows():
+    """Rows of 8192 and 4096 features through the reference's quantize_rows
+    (tests/golden/make_golden_long_rows.py); inputs are BF16 bit patterns."""
+    with np.load(GOLDEN_DIR / "reference_long_rows.npz") as data:
+        return {name: data[name] for name in data.files}
+
+
+@pytest.fixture(scope="session")
 def golden_meta():
     return json.loads((GOLDEN_DIR / "reference_vectors.json").read_text())
 

@@ -70,6 +70,18 @@ def _pack_ids(beta):
     return (b[:, 0] | (b[:, 1] << 2) | (b[:, 2] << 4) | (b[:, 3] << 6)).astype(np.uint8)
 
 
+def test_quantize_rows_long_rows_match_reference_golden(rt, golden_long_rows):
+    """BF16 rows of 8192 and 4096 features (the sliced, 1024-lane encoder path): codes, beta ids
+    and norms of the reference's CPU quantiser, bit for bit."""
+    for name in ("qr8192", "qr4096"):
+        x = torch.from_numpy(golden_long_rows[f"{name}_x_bf16"].copy()).view(torch.bfloat16).cuda()
+        codes, beta_ids, norms = rt.quantize_rows_packed(x, q=Q, beta_table=_table(ACTIVATION_BETAS))
+        assert np.array_equal(bits(norms), golden_long_rows[f"{name}_norms"]), name
+        assert np.array_equal(bits(codes).reshape(-1, 4).view(np.uint32).reshape(-1),
+                              _pack_words(golden_long_rows[f"{name}_codes"].reshape(-1, 8))), name
+        assert np.array_equal(bits(beta_ids), _pack_ids(golden_long_rows[f"{name}_beta"].reshape(-1))), name
+
+
 @pytest.mark.parametrize("rows,n,kind,dtype", [
     (1, 2048, "student", torch.bfloat16),
     (8, 8192, "student", torch.bfloat16),

@@ -44,6 +44,16 @@ def test_quantize_rows_undithered(oracle, golden):
     assert not golden["qr64_deq"][5].any()          # the zero row stays zero
 
 
+def test_quantize_rows_long_rows(oracle, golden_long_rows):
+    """The eight-chain row norm and the scaling hold at the down_proj activation width."""
+    for name in ("qr8192", "qr4096"):
+        x = (golden_long_rows[f"{name}_x_bf16"].view(np.uint16).astype(np.uint32) << 16).view(np.float32)
+        codes, beta, norms = oracle.quantize_rows(x, Q, ACTIVATION_BETAS)
+        assert np.array_equal(norms, golden_long_rows[f"{name}_norms"]), name
+        assert np.array_equal(codes.reshape(golden_long_rows[f"{name}_codes"].shape), golden_long_rows[f"{name}_codes"]), name
+        assert np.array_equal(beta.reshape(golden_long_rows[f"{name}_beta"].shape), golden_long_rows[f"{name}_beta"]), name
+
+
 def test_nqrt4_record_payloads_and_dequantize(oracle, golden, golden_meta):
     seed = golden_meta["nqrt_seed"]
     w = golden["nqrt_w"]
