@@ -109,6 +109,10 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
         return;
     }
 
+    // beta tables in registers: a table lookup from memory would sit behind every decode
+    const float key_beta[4] = {a.key_betas[0], a.key_betas[1], a.key_betas[2], a.key_betas[3]};
+    const float value_beta[4] = {a.value_betas[0], a.value_betas[1], a.value_betas[2], a.value_betas[3]};
+
     // lane role inside a pass
     const int pass_page = tid / kTokenBlocks, token = (tid % kTokenBlocks) / kBlocks, blk = tid % kBlocks;
     const int row_in_page = token * a.kv_heads + g;
@@ -207,7 +211,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
             }
         } else if (valid) {
             decode_codeword<false>(k_code[pass], 14.0f, 0u, k);
-            const float beta = a.key_betas[(k_ids[pass] >> (2 * (blk & 3))) & 3];     // word index % 4 == blk % 4
+            const float beta = key_beta[(k_ids[pass] >> (2 * (blk & 3))) & 3];     // word index % 4 == blk % 4
             const float back = k_norm[pass] / sqrt_d;
 #pragma unroll
             for (int j = 0; j < 8; j++) k[j] = (k[j] * beta) * back;
@@ -295,7 +299,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
             }
         } else if (valid) {
             decode_codeword<false>(v_code[pass], 14.0f, 0u, v);
-            const float beta = a.value_betas[(v_ids[pass] >> (2 * (blk & 3))) & 3];
+            const float beta = value_beta[(v_ids[pass] >> (2 * (blk & 3))) & 3];
             const float back = v_norm[pass] / sqrt_d;
 #pragma unroll
             for (int j = 0; j < 8; j++) v[j] = (v[j] * beta) * back;
