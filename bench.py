@@ -243,7 +243,7 @@ def prefill_gemm_extra(rt, device):
                                                   None if base.resolved_tails is None else base.resolved_tails.clone())
                             for _ in range(copies - 1)]
         table = torch.tensor(ACTIVATION_BETAS, dtype=torch.float32, device=device)
-        for m in (16, 40, 64, 128, 384):
+        for m in (16, 40, 64, 128, 384, 1024, 4096):         # the last two: long prefill, beyond the reference's list
             rng = np.random.default_rng(3001)
             x = rng.standard_normal((m, k)).astype(np.float32)
             x[:, rng.choice(k, size=k // 100, replace=False)] *= 20.0

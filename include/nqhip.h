@@ -226,6 +226,21 @@ int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
 size_t nq_w4a4_gemm_workspace_bytes(int m, int k, int n, int split_k, int have_decoded_activation);
 
 /*
+ * The BF16 weight [N, K] that nq_w4a4_gemv / nq_w4a4_gemm multiply by, written out:
+ * bf16(decode * beta * (norm / sqrt(K))) per element, from the resolved form when given, else
+ * from the NQRT4 streams.  For prefills long enough that decoding the weight once and running
+ * a plain BF16 GEMM (a library's) beats decoding it inside the multiply; the scratch is the
+ * caller's and lives only for that call.
+ * Replaces: PackedNestQuantTensor.dequantize_chunked(output_dtype=bfloat16),
+ * nestquant/core/tensor_checkpoint.py:285-330 (up to the scale's rounding order, which follows
+ * the linear kernels here).
+ */
+int nq_w4a4_decode_weight(const uint8_t *w_codes_dev, const uint8_t *w_beta_ids_dev,
+                          const uint32_t *w_resolved_words_dev, const uint16_t *w_resolved_tails_dev,
+                          const float *w_norms_dev, const float *w_betas_dev, int64_t n, int64_t k,
+                          int64_t weight_offset, int64_t weight_seed, void *out_bf16_dev, void *stream);
+
+/*
  * NQKV cache, device-resident state.  Per slot (int32[slots]): sequence_lengths,
  * page_counts, last_page_lens, hot_lengths; page_indices int32[slots, max_pages] maps a
  * slot's page ordinal to a physical page; hot tails BF16 [slots, page_size, kv_heads,

@@ -38,6 +38,7 @@ SIGNATURES = {
     "nq_fused_input_stage": (_i32, [_ptr, _i64, _i64, _i32, _ptr, _ptr, _ptr, _c.c_float, _ptr, _ptr, _i32, _ptr, _i32,
                                     _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "nq_w4a4_gemv_grouped": (_i32, [_ptr, _i32] + [_ptr] * 8 + [_i32, _i32, _i32, _ptr]),
+    "nq_w4a4_decode_weight": (_i32, [_ptr] * 6 + [_i64, _i64, _i64, _i64, _ptr, _ptr]),
     "nq_w4a4_resolve_weight": (_i32, [_ptr, _ptr, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "nq_w4a4_gemv": (_i32, [_ptr] * 11 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
                                           _size, _ptr]),

@@ -161,6 +161,35 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
     }
 }
 
+
+// The BF16 weight [N][K] the linear kernels multiply by, written out: one lane per E8 block,
+// the same decode, scale and rounding as the decode role of the kernel above.  Long prefills
+// decode the weight once with the whole chip and hand the plain GEMM to a library.
+template <bool kResolved>
+__global__ void __launch_bounds__(256)
+decode_weight_kernel(const uint32_t *__restrict__ w_words, const uint16_t *__restrict__ w_tails,
+                     const uint8_t *__restrict__ w_beta_ids, const float *__restrict__ w_norms,
+                     const float *__restrict__ w_betas, int64_t blocks, int blocks_per_row,
+                     uint32_t seed_plus_offset, float sqrt_k, uint4 *__restrict__ out) {
+    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= blocks) return;
+    const int64_t row = g / blocks_per_row;
+    const uint32_t word = w_words[g];
+    const float unit = w_norms[row] / sqrt_k;
+    float v[8], scale;
+    if (kResolved) {
+        decode_resolved(word, w_tails[g], seed_plus_offset + (uint32_t)g * 8u, v);
+        scale = w_betas[word >> 30] * (unit * kResolvedUnit);
+    } else {
+        decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
+        scale = w_betas[(w_beta_ids[g >> 2] >> (2 * (g & 3))) & 3] * unit;
+    }
+    const bf16x2 h0 = pack_bf16x2(v[0] * scale, v[1] * scale), h1 = pack_bf16x2(v[2] * scale, v[3] * scale);
+    const bf16x2 h2 = pack_bf16x2(v[4] * scale, v[5] * scale), h3 = pack_bf16x2(v[6] * scale, v[7] * scale);
+    out[g] = make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
+                        __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
+}
+
 }  // namespace nq
 
 namespace {
@@ -270,4 +299,37 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
         }
     }
     return NQ_OK;
+}
+
+extern "C" int nq_w4a4_decode_weight(const uint8_t *w_codes_dev, const uint8_t *w_beta_ids_dev,
+                                     const uint32_t *w_resolved_words_dev, const uint16_t *w_resolved_tails_dev,
+                                     const float *w_norms_dev, const float *w_betas_dev, int64_t n, int64_t k,
+                                     int64_t weight_offset, int64_t weight_seed, void *out_bf16_dev, void *stream) {
+    NQ_REQUIRE(n >= 1 && k >= 32 && k % 32 == 0, NQ_ERR_SHAPE,
+               "nq_w4a4_decode_weight: N must be positive and K a positive multiple of 32");
+    const bool resolved = w_resolved_words_dev != nullptr;
+    NQ_REQUIRE(w_norms_dev && w_betas_dev && out_bf16_dev, NQ_ERR_ARGUMENT, "nq_w4a4_decode_weight: null pointer");
+    NQ_REQUIRE(resolved ? w_resolved_tails_dev != nullptr : (w_codes_dev && w_beta_ids_dev), NQ_ERR_ARGUMENT,
+               "nq_w4a4_decode_weight: neither packed nor resolved weight streams given");
+    NQ_REQUIRE(nq::aligned(w_codes_dev, 4) && nq::aligned(w_resolved_words_dev, 4) &&
+                   nq::aligned(w_resolved_tails_dev, 2) && nq::aligned(out_bf16_dev, 16),
+               NQ_ERR_ARGUMENT, "nq_w4a4_decode_weight: code streams need 4-byte, the output 16-byte alignment");
+    NQ_REQUIRE(weight_seed >= 0 && weight_seed < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
+               "nq_w4a4_decode_weight: seed must be in [0, 2**31)");
+    const int64_t blocks = n * (k / 8);
+    NQ_REQUIRE(weight_offset >= 0 && weight_offset + blocks <= ((int64_t)1 << 28), NQ_ERR_SHAPE,
+               "nq_w4a4_decode_weight: block range exceeds the stateless dither counter space");
+    const uint32_t seed_plus_offset = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
+    const float sqrt_k = (float)sqrt((double)k);
+    const dim3 grid((unsigned)((blocks + 255) / 256));
+    const uint32_t *words = resolved ? w_resolved_words_dev : reinterpret_cast<const uint32_t *>(w_codes_dev);
+    if (resolved)
+        hipLaunchKernelGGL(nq::decode_weight_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, words,
+                           w_resolved_tails_dev, w_beta_ids_dev, w_norms_dev, w_betas_dev, blocks, (int)(k / 8),
+                           seed_plus_offset, sqrt_k, reinterpret_cast<uint4 *>(out_bf16_dev));
+    else
+        hipLaunchKernelGGL(nq::decode_weight_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, words,
+                           w_resolved_tails_dev, w_beta_ids_dev, w_norms_dev, w_betas_dev, blocks, (int)(k / 8),
+                           seed_plus_offset, sqrt_k, reinterpret_cast<uint4 *>(out_bf16_dev));
+    return nq::check_launch("nq_w4a4_decode_weight");
 }

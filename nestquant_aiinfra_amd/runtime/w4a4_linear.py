@@ -522,9 +522,39 @@ def linear_packed_w4a4_mma_small_m_splitk_probe(activation: PreparedNQA4Activati
 # linear kernels, prefill (matrix cores)
 # --------------------------------------------------------------------------------------
 
+# From this many rows on (BF16 output, automatic split) a packed linear decodes its weight once
+# into a BF16 scratch (nq_w4a4_decode_weight) and hands the plain BF16 GEMM to the BLAS library
+# behind torch.matmul.  The fused kernel decodes a block once per 512 rows but re-reads the
+# activation once per 32 channels, which is what it waits for beyond a few hundred rows;
+# measured crossover on MI355X at the 1B shapes: between 256 and 384 rows.
+LIBRARY_GEMM_ROWS = 288
+
+
+def decode_weight_bf16(weight: PreparedNQRTLinear) -> torch.Tensor:
+    """The BF16 weight [N, K] the packed linear kernels multiply by (transient scratch)."""
+    device = weight.row_norms.device
+    n, k = weight.record.indices.shape[0], weight.record.feature_count
+    out = torch.empty((n, k), dtype=torch.bfloat16, device=device)
+    resolved = weight.resolved_words is not None
+    _native.check(_native.library().nq_w4a4_decode_weight(
+        weight.code_payload.data_ptr(), weight.beta_payload.data_ptr(),
+        weight.resolved_words.data_ptr() if resolved else None,
+        weight.resolved_tails.data_ptr() if resolved else None,
+        weight.row_norms.data_ptr(), weight.beta_table.data_ptr(), n, k, 0, int(weight.record.dither_seed),
+        out.data_ptr(), _native.stream_handle(device)))
+    return out
+
+
 def _gemm(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *,
           output_dtype: torch.dtype | None = None, split_k: int = 0) -> torch.Tensor:
     dtype = _kernel_dtype(activation) if output_dtype is None else output_dtype
+    if (dtype == torch.bfloat16 and split_k == 0 and activation.token_count >= LIBRARY_GEMM_ROWS
+            and activation.feature_count % 32 == 0):
+        rows = activation.decoded
+        if rows is None:
+            rows = decode_packed_a4(activation, output_dtype=torch.bfloat16).reshape(-1, activation.feature_count)
+        out = torch.matmul(rows, decode_weight_bf16(weight).t())
+        return out.reshape(*activation.original_shape[:-1], out.shape[-1])
     return _gemv(activation, weight, split_k=split_k, output_dtype=dtype, kernel="gemm")
 
 

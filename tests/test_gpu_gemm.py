@@ -101,3 +101,41 @@ def test_slice_and_pad_matches_reference_chunking(rt, oracle):
     assert torch.equal(part[:8], whole[32:40]) and not part[8:].any()
     packed_only = dataclasses.replace(chunk, decoded=None)
     assert torch.equal(rt._gemm(packed_only, weight, output_dtype=torch.float32), part)
+
+
+@pytest.mark.parametrize("k,n_out", [(2048, 2048), (512, 200)])
+def test_long_prefill_decodes_the_weight_once(rt, oracle, k, n_out):
+    """From LIBRARY_GEMM_ROWS rows on, BF16 outputs come from nq_w4a4_decode_weight + a library
+    GEMM: the decoded weight equals the oracle's BF16-rounded weight (resolved form: but for
+    rare one-step roundings) and the product stays within the bar; below the threshold and for
+    FP32 outputs the fused kernel runs."""
+    from test_gpu_gemv import _record
+    seed = 20261150
+    _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=4000 + k, dither_seed=seed)
+    record = _record(rt, wc, wb, wn, k, seed)
+    weight = rt.prepare_fused_linear(record, device="cuda")
+    streams_only = rt.prepare_fused_linear(record, device="cuda", resolve=False)
+    w_hat = oracle.bf16_round(oracle.dequantize_rows(wc, wb, wn, WEIGHT_BETAS, Q, seed=seed))
+    # the kernels form beta * (norm / sqrt(K)) first (the oracle multiplies by beta, then by the
+    # row scale): same lattice points, FP32 products that differ in the last place, hence rare
+    # one-step differences after the BF16 rounding.  The resolved form adds at most 2^-26 lattice
+    # units before the scale, which only shows on weights that are themselves almost zero.
+    row_peak = np.abs(w_hat).max(axis=1, keepdims=True)
+    for form in (streams_only, weight):
+        decoded = bits(rt.decode_weight_bf16(form).float())
+        assert np.all(np.abs(decoded - w_hat) <= np.maximum(np.abs(w_hat) * 2.0 ** -7, row_peak * 2.0 ** -22))
+        assert np.count_nonzero(decoded != w_hat) <= decoded.size // 500 + 1
+    from_streams, from_resolved = (bits(rt.decode_weight_bf16(form).float()) for form in (streams_only, weight))
+    assert np.count_nonzero(from_streams != from_resolved) <= from_streams.size // 500 + 1
+
+    m = rt.LIBRARY_GEMM_ROWS + 37
+    activation = _activation(rt, oracle, m, k, seed=77)
+    a_codes = oracle.unpack_unsigned(bits(activation.code_payload), m * k, 4)
+    a_beta = oracle.unpack_unsigned(bits(activation.beta_payload), m * k // 8, 2)
+    a_hat = oracle.dequantize_rows(a_codes, a_beta, bits(activation.row_norms), ACTIVATION_BETAS, Q)
+    ref = oracle.matmul_nt(a_hat, oracle.dequantize_rows(wc, wb, wn, WEIGHT_BETAS, Q, seed=seed))
+    y = rt.linear_packed_w4a4_mma_chunked_staged(activation, weight)
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (m, n_out)
+    assert relative_error(bits(y.float()), ref) <= TOLERANCE
+    fused = rt._gemm(activation, weight, output_dtype=torch.bfloat16, split_k=1)      # explicit split: fused kernel
+    assert relative_error(bits(y.float()), bits(fused.float())) <= 5e-3
