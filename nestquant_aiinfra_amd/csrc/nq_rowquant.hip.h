@@ -31,9 +31,6 @@ __device__ __forceinline__ float round_to_dtype(float x, int dtype) {
     return x;
 }
 
-// S butterfly stages (pair distances 2^log_w .. 2^(log_w + S - 1)) on 2^S values held in
-// registers: one LDS round trip per pass instead of one per stage.  `total` counts all staged
-// values; groups never straddle rows because n is a power of two.
 // Both values rounded to the storage dtype kDtype (tags as above), kept as float32.
 template <int kDtype>
 __device__ __forceinline__ void round_pair(float &a, float &b) {
@@ -47,8 +44,11 @@ __device__ __forceinline__ void round_pair(float &a, float &b) {
     }
 }
 
-template <int S, int kDtype>
-__device__ __forceinline__ void hadamard_pass(float *rows, int total, int log_w) {
+// S butterfly stages (pair distances 2^log_w .. 2^(log_w + S - 1)) on 2^S values held in
+// registers: one LDS round trip per pass instead of one per stage.  `total` counts all staged
+// values; groups never straddle rows because n is a power of two.  With kScale the results are multiplied by `inv` and rounded once more on the way out.
+template <int S, int kDtype, bool kScale>
+__device__ __forceinline__ void hadamard_pass(float *rows, int total, int log_w, float inv) {
     constexpr int kValues = 1 << S;
     const int groups = total >> S;
     for (int t = threadIdx.x; t < groups; t += blockDim.x) {
@@ -67,32 +67,123 @@ __device__ __forceinline__ void hadamard_pass(float *rows, int total, int log_w)
                 round_pair<kDtype>(v[j], v[j + (1 << s)]);
             }
         }
+        if (kScale) {
+#pragma unroll
+            for (int j = 0; j < kValues; j += 2) {
+                v[j] = v[j] * inv;
+                v[j + 1] = v[j + 1] * inv;
+                round_pair<kDtype>(v[j], v[j + 1]);
+            }
+        }
 #pragma unroll
         for (int j = 0; j < kValues; j++) rows[base + (j << log_w)] = v[j];
     }
     __syncthreads();
 }
 
+// The value the lane whose id differs by kXor holds (all lanes of the exchange active).
+template <int kXor>
+__device__ __forceinline__ float lane_xor(float v) {
+    const int x = __builtin_bit_cast(int, v);
+    if (kXor == 1) return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(x, 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    if (kXor == 2) return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(x, 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    if (kXor == 4) {
+        int r = __builtin_amdgcn_update_dpp(0, x, 0x104, 0xF, 0x5, false);       // row_shl:4 into lanes 0-3, 8-11
+        r = __builtin_amdgcn_update_dpp(r, x, 0x114, 0xF, 0xA, false);           // row_shr:4 into lanes 4-7, 12-15
+        return __builtin_bit_cast(float, r);
+    }
+    if (kXor == 8) return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(x, 0x128, 0xF, 0xF, true));  // row_ror:8
+    return __shfl_xor(v, kXor, 64);
+}
+
+// One butterfly stage between lanes: the lane with the lower id holds the left operands.
+template <int kXor, int kDtype>
+__device__ __forceinline__ void lane_stage(float (&v)[8], int lane) {
+    const bool upper = (lane & kXor) != 0;
+    float other[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) other[j] = lane_xor<kXor>(v[j]);
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = other[j] + (upper ? -v[j] : v[j]);       // left + right | left - right
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) round_pair<kDtype>(v[j], v[j + 1]);
+}
+
 // Normalized Sylvester-Hadamard transform of rows staged in LDS (nestquant/core/rotation.py:12-27):
 // butterflies of growing width, each sum and difference rounded to `stage_dtype` (the dtype
 // the reference's tensor ops would run in), then one multiplication by float32(1 / sqrt(n))
 // -- the form a tensor / python-scalar division takes on the GPU.  Ends with a barrier.
+//
+// Every lane takes eight neighbouring values: distances 1, 2, 4 are butterflies in registers,
+// distances 8 .. 256 exchanges between the lanes of a wavefront, and only the distances from
+// 512 up (rows of 1024 values and more) make further trips through LDS.
 template <int kDtype>
 __device__ __forceinline__ void staged_hadamard_as(float *rows, int row_count, int n) {
     const int log_n = 31 - __builtin_clz(n);
     const int total = row_count * n;
-    int log_w = 0;
-    for (; log_n - log_w >= 3; log_w += 3) hadamard_pass<3, kDtype>(rows, total, log_w);
-    if (log_n - log_w == 2) hadamard_pass<2, kDtype>(rows, total, log_w);
-    if (log_n - log_w == 1) hadamard_pass<1, kDtype>(rows, total, log_w);
     const float inv = 1.0f / __builtin_sqrtf((float)n);
-    for (int i = 2 * threadIdx.x; i < total; i += 2 * blockDim.x) {
-        float a = rows[i] * inv, b = rows[i + 1] * inv;
-        round_pair<kDtype>(a, b);
-        rows[i] = a;
-        rows[i + 1] = b;
+    if (n < 8 || (blockDim.x & 63)) {
+        // short rows or ragged wavefronts: every stage through LDS
+        int log_w = 0;
+        for (; log_n - log_w >= 3; log_w += 3) hadamard_pass<3, kDtype, false>(rows, total, log_w, inv);
+        if (log_n - log_w == 2) hadamard_pass<2, kDtype, false>(rows, total, log_w, inv);
+        if (log_n - log_w == 1) hadamard_pass<1, kDtype, false>(rows, total, log_w, inv);
+        for (int i = 2 * threadIdx.x; i < total; i += 2 * blockDim.x) {
+            float a = rows[i] * inv, b = rows[i + 1] * inv;
+            round_pair<kDtype>(a, b);
+            rows[i] = a;
+            rows[i + 1] = b;
+        }
+        __syncthreads();
+        return;
+    }
+    const int lane = threadIdx.x & 63;
+    const int lane_stages = log_n - 3 < 6 ? log_n - 3 : 6;
+    const bool scale_here = log_n <= 9;
+    for (int chunk = threadIdx.x; chunk < (total >> 3); chunk += blockDim.x) {
+        float4 *slot = reinterpret_cast<float4 *>(rows + 8 * chunk);
+        const float4 lo = slot[0], hi = slot[1];
+        float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+        for (int s = 0; s < 3; s++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                if (j & (1 << s)) continue;
+                const float left = v[j], right = v[j + (1 << s)];
+                v[j] = left + right;
+                v[j + (1 << s)] = left - right;
+                round_pair<kDtype>(v[j], v[j + (1 << s)]);
+            }
+        }
+        // a row's chunks sit in neighbouring lanes (n / 8 of them, a power of two), so the
+        // stage count is the same for the whole wavefront
+        if (lane_stages > 0) lane_stage<1, kDtype>(v, lane);
+        if (lane_stages > 1) lane_stage<2, kDtype>(v, lane);
+        if (lane_stages > 2) lane_stage<4, kDtype>(v, lane);
+        if (lane_stages > 3) lane_stage<8, kDtype>(v, lane);
+        if (lane_stages > 4) lane_stage<16, kDtype>(v, lane);
+        if (lane_stages > 5) lane_stage<32, kDtype>(v, lane);
+        if (scale_here) {
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) {
+                v[j] = v[j] * inv;
+                v[j + 1] = v[j + 1] * inv;
+                round_pair<kDtype>(v[j], v[j + 1]);
+            }
+        }
+        slot[0] = make_float4(v[0], v[1], v[2], v[3]);
+        slot[1] = make_float4(v[4], v[5], v[6], v[7]);
     }
     __syncthreads();
+    int log_w = 9;
+    for (; log_n - log_w > 4; log_w += 3) hadamard_pass<3, kDtype, false>(rows, total, log_w, inv);
+    switch (log_n - log_w) {
+        case 4: hadamard_pass<4, kDtype, true>(rows, total, log_w, inv); break;
+        case 3: hadamard_pass<3, kDtype, true>(rows, total, log_w, inv); break;
+        case 2: hadamard_pass<2, kDtype, true>(rows, total, log_w, inv); break;
+        case 1: hadamard_pass<1, kDtype, true>(rows, total, log_w, inv); break;
+        default: break;
+    }
 }
 
 __device__ __forceinline__ void staged_hadamard(float *rows, int row_count, int n, int stage_dtype) {
@@ -112,10 +203,41 @@ __device__ __forceinline__ void staged_row_norms(const float *rows, int row_coun
             const int r = t >> 3, lane = t & 7;
             const float *row = rows + (size_t)r * n + lane;
             float acc = 0.0f;
-            // n is a multiple of 32: four chain steps per trip, many trips in flight
-#pragma unroll 8
-            for (int i = 0; i < (n >> 3); i += 4) {
-                const float v0 = row[8 * i], v1 = row[8 * i + 8], v2 = row[8 * i + 16], v3 = row[8 * i + 24];
+            // n is a multiple of 32.  Batches of 32 chain steps, double-buffered by hand: the
+            // next batch is requested from LDS before the chain runs over the current one, so
+            // that the LDS latency stays off the serial path (a request past the end is clamped
+            // to the last batch and not used).
+            const int groups = n >> 5, batches = groups >> 3;
+            if (batches > 0) {
+                float a[32], b[32];
+#pragma unroll
+                for (int k = 0; k < 32; k++) a[k] = row[8 * k];
+                int batch = 0;
+                for (; batch + 2 <= batches; batch += 2) {
+                    const float *next = row + 256 * (batch + 1);
+#pragma unroll
+                    for (int k = 0; k < 32; k++) b[k] = next[8 * k];
+                    __builtin_amdgcn_sched_barrier(0);      // keep the requests ahead of the chain
+#pragma unroll
+                    for (int k = 0; k < 32; k++) acc = __builtin_fmaf(a[k], a[k], acc);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const int after = batch + 2 < batches ? batch + 2 : batches - 1;
+                    next = row + 256 * after;
+#pragma unroll
+                    for (int k = 0; k < 32; k++) a[k] = next[8 * k];
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int k = 0; k < 32; k++) acc = __builtin_fmaf(b[k], b[k], acc);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (batch < batches) {
+#pragma unroll
+                    for (int k = 0; k < 32; k++) acc = __builtin_fmaf(a[k], a[k], acc);
+                }
+            }
+#pragma unroll 1
+            for (int g = batches << 3; g < groups; g++) {
+                const float v0 = row[32 * g], v1 = row[32 * g + 8], v2 = row[32 * g + 16], v3 = row[32 * g + 24];
                 acc = __builtin_fmaf(v0, v0, acc);
                 acc = __builtin_fmaf(v1, v1, acc);
                 acc = __builtin_fmaf(v2, v2, acc);

@@ -183,6 +183,11 @@ def test_fused_rotation_matches_separate_rotation(oracle):
         plain = rt.quantize_activation_cuda(rotated, q=Q, betas=ACTIVATION_BETAS)
         assert torch.equal(fused.code_payload, plain.code_payload) and torch.equal(fused.row_norms, plain.row_norms)
         assert torch.equal(fused.beta_payload, plain.beta_payload) and torch.equal(fused.decoded, plain.decoded)
+    # every row length takes its own mix of register, lane and LDS stages
+    for n in (2, 4, 8, 16, 32, 64, 128, 256, 512, 1024, 4096, 8192, 16384, 32768):
+        for dtype in (torch.bfloat16, torch.float16, torch.float32):
+            x = torch.randn(3, n, device="cuda").to(dtype)
+            assert torch.equal(rt.hadamard_cuda(x), hadamard(x)), (n, dtype)
     # float32 butterflies over a 64-wide head, rounded to BF16 once (the key / query rotation)
     k = torch.randn(3, 2, 7, 64, device="cuda").to(torch.bfloat16)
     assert torch.equal(rt.hadamard_cuda(k, compute_dtype=torch.float32), hadamard(k.float()).to(torch.bfloat16))
