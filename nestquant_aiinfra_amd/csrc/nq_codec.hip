@@ -199,6 +199,38 @@ __device__ __forceinline__ void stage_with_prologue(const uint16_t *__restrict__
     __syncthreads();
 }
 
+// Where the encoder kernels put a block's results: the packed streams, and optionally the
+// BF16 decode of the stored code as the linear kernels consume it.
+struct RowSink {
+    uint32_t *codes; uint8_t *beta_ids; uint4 *decoded; const float *row_norm;
+    int64_t row0, rows; int blocks_per_row; float sqrt_n;
+    __device__ __forceinline__ bool wants(int r) const { return row0 + r < rows; }
+    __device__ __forceinline__ void code(int r, int b, uint32_t word, const float (&recon)[8], float beta) const {
+        const int64_t gblock = (row0 + r) * blocks_per_row + b;
+        codes[gblock] = word;
+        if (decoded) {
+            // the BF16 decode of the stored code, as the linear kernels consume it
+            const float back = row_norm[r] / sqrt_n;
+            uint32_t h[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) h[j] = f32_to_bf16((recon[j] * beta) * back);
+            decoded[gblock] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16),
+                                         h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+        }
+    }
+    __device__ __forceinline__ void beta_byte(int r, int b, uint32_t byte) const {
+        beta_ids[((row0 + r) * blocks_per_row + b) >> 2] = (uint8_t)byte;
+    }
+    __device__ __forceinline__ uint32_t counter(int r, int b) const {
+        return (uint32_t)((row0 + r) * blocks_per_row + b) * 8u;
+    }
+};
+
+struct SharedBetas {
+    const float *table;
+    __device__ __forceinline__ const float *operator()(int) const { return table; }
+};
+
 template <typename T, bool kDithered, int kPrologue>
 __global__ void __launch_bounds__(1024)
 quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, float inv_q,
@@ -254,36 +286,54 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
 
     // phase 3
     const int slice_pairs = rows_per_wg * blocks_per_row * 4 / slices;     // a multiple of 16
-    struct Sink {
-        uint32_t *codes; uint8_t *beta_ids; uint4 *decoded; const float *row_norm;
-        int64_t row0, rows; int blocks_per_row; float sqrt_n;
-        __device__ __forceinline__ bool wants(int r) const { return row0 + r < rows; }
-        __device__ __forceinline__ void code(int r, int b, uint32_t word, const float (&recon)[8], float beta) const {
-            const int64_t gblock = (row0 + r) * blocks_per_row + b;
-            codes[gblock] = word;
-            if (decoded) {
-                // the BF16 decode of the stored code, as the linear kernels consume it
-                const float back = row_norm[r] / sqrt_n;
-                uint32_t h[8];
-#pragma unroll
-                for (int j = 0; j < 8; j++) h[j] = f32_to_bf16((recon[j] * beta) * back);
-                decoded[gblock] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16),
-                                             h[4] | (h[5] << 16), h[6] | (h[7] << 16));
-            }
-        }
-        __device__ __forceinline__ void beta_byte(int r, int b, uint32_t byte) const {
-            beta_ids[((row0 + r) * blocks_per_row + b) >> 2] = (uint8_t)byte;
-        }
-        __device__ __forceinline__ uint32_t counter(int r, int b) const {
-            return (uint32_t)((row0 + r) * blocks_per_row + b) * 8u;
-        }
-    } sink{codes, beta_ids, decoded, row_norm, row0, rows, blocks_per_row, sqrt_n};
-    struct Betas {
-        const float *table;
-        __device__ __forceinline__ const float *operator()(int) const { return table; }
-    } betas_of{betas};
+    const RowSink sink{codes, beta_ids, decoded, row_norm, row0, rows, blocks_per_row, sqrt_n};
+    const SharedBetas betas_of{betas};
     quantize_staged_pairs<kDithered>(lds, row_scale, n, q, inv_q, betas_of, beta_count, seed_plus_offset,
                                      slice_pairs * slice, slice_pairs * (slice + 1), sink);
+}
+
+// Many rows: 256 lanes per workgroup, `rows_per_wg` rows of together at least 2048 values, one
+// lane per block in the encode phase (several such workgroups share a compute unit and fill
+// each other's serial stretches: the norm chain, the barriers of the rotation).
+template <typename T>
+__global__ void __launch_bounds__(256)
+quantize_rows_bulk_kernel(const T *__restrict__ x, int64_t rows, int n, float q, float inv_q,
+                          const float *__restrict__ betas, int beta_count, float sqrt_n,
+                          uint32_t *__restrict__ codes, uint8_t *__restrict__ beta_ids,
+                          float *__restrict__ norms, uint4 *__restrict__ decoded, int rows_per_wg,
+                          int vector_loads, int hadamard_stage_dtype) {
+    extern __shared__ float lds[];
+    float *row_scale = lds + (size_t)rows_per_wg * n;
+    float *row_norm = row_scale + rows_per_wg;
+    const int tid = threadIdx.x;
+    const int64_t row0 = (int64_t)blockIdx.x * rows_per_wg;
+    const int64_t first = row0 * n, limit = rows * (int64_t)n;
+    if (vector_loads) {
+        constexpr int kPer = RowLoader<T>::kPerVector;
+        const int vectors = rows_per_wg * n / kPer;
+#pragma unroll 4
+        for (int v = tid; v < vectors; v += blockDim.x) {
+            const int64_t g = first + (int64_t)v * kPer;
+            if (g < limit) {
+                RowLoader<T>::load(x, g / kPer, lds + v * kPer);
+            } else {
+#pragma unroll
+                for (int j = 0; j < kPer; j++) lds[v * kPer + j] = 0.0f;
+            }
+        }
+    } else {
+        for (int idx = tid; idx < rows_per_wg * n; idx += blockDim.x) {
+            const int64_t g = first + idx;
+            lds[idx] = g < limit ? RowLoader<T>::scalar(x, g) : 0.0f;
+        }
+    }
+    __syncthreads();
+    if (hadamard_stage_dtype >= 0) staged_hadamard(lds, rows_per_wg, n, hadamard_stage_dtype);
+    staged_row_norms(lds, rows_per_wg, n, sqrt_n, row_scale, row_norm);
+    if (tid < rows_per_wg && row0 + tid < rows) norms[row0 + tid] = row_norm[tid];
+    const RowSink sink{codes, beta_ids, decoded, row_norm, row0, rows, n >> 3, sqrt_n};
+    quantize_staged_blocks(lds, row_scale, n, q, inv_q, SharedBetas{betas}, beta_count, 0,
+                           rows_per_wg * (n >> 3), sink);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -396,11 +446,34 @@ extern "C" int nq_e8_nearest(const float *x_dev, float *out_dev, int64_t count, 
 
 namespace {
 
+// from this many values on, undithered rows go to the kernel built for throughput
+constexpr int64_t kBulkElements = 1 << 21;
+
 template <typename T, bool kDithered, int kPrologue = 0>
 int launch_quantize(const void *x, int64_t rows, int n, int q, const float *betas, int beta_count,
                     uint32_t seed_plus_offset, uint8_t *codes, uint8_t *beta_ids, float *norms,
                     void *decoded, int hadamard_stage_dtype, hipStream_t stream,
                     nq::InputPrologue prologue = nq::InputPrologue{}) {
+    if (!kDithered && kPrologue == 0 && rows * (int64_t)n >= kBulkElements) {
+        int rows_per_wg = n >= 2048 ? 1 : 2048 / n;
+        const size_t lds_bytes = ((size_t)rows_per_wg * n + 2 * rows_per_wg) * sizeof(float);
+        auto kernel = nq::quantize_rows_bulk_kernel<T>;
+        if (lds_bytes > 48 * 1024) {
+            hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (status != hipSuccess)
+                return nq::fail(NQ_ERR_LAUNCH, "nq_quantize_rows: cannot reserve %zu bytes of LDS: %s",
+                                lds_bytes, hipGetErrorString(status));
+        }
+        const int64_t grid = (rows + rows_per_wg - 1) / rows_per_wg;
+        if (grid > 0x7fffffff) return nq::fail(NQ_ERR_SHAPE, "nq_quantize_rows: too many rows");
+        hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), lds_bytes, stream,
+                           reinterpret_cast<const T *>(x), rows, n, (float)q, 1.0f / (float)q, betas, beta_count,
+                           (float)sqrt((double)n), reinterpret_cast<uint32_t *>(codes), beta_ids, norms,
+                           reinterpret_cast<uint4 *>(decoded), rows_per_wg, (int)nq::aligned(x, 16),
+                           hadamard_stage_dtype);
+        return nq::check_launch("nq_quantize_rows");
+    }
     const int pairs_per_row = n / 2;
     const int target = pairs_per_row < 256 ? 256 : (pairs_per_row < 1024 ? pairs_per_row : 1024);
     int rows_per_wg = target / pairs_per_row;

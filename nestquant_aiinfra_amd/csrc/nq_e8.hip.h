@@ -147,6 +147,31 @@ __device__ __forceinline__ float div_by_14(float p) {
     return __builtin_fmaf(r, c, q0);
 }
 
+// Correctly rounded a / b from the correctly rounded reciprocal `rcp` = 1 / b: a first quotient,
+// then two rounds of exact remainder (one fused multiply-add) and correction.  The first round
+// leaves a faithful quotient, and a faithful quotient corrected with a correctly rounded
+// reciprocal is the correctly rounded one (Markstein).  Needs the remainders to be exact:
+// callers keep |a| >= 2^-61 (or a == 0) and 2^-40 <= b <= 2^40.  Only the sign of a zero
+// quotient can differ from the IEEE division.
+__device__ __forceinline__ float divide_by_reciprocal(float a, float b, float rcp) {
+    float quotient = a * rcp;
+    float remainder = __builtin_fmaf(-b, quotient, a);
+    quotient = __builtin_fmaf(remainder, rcp, quotient);
+    remainder = __builtin_fmaf(-b, quotient, a);
+    return __builtin_fmaf(remainder, rcp, quotient);
+}
+
+// True when some value is nonzero and below 2^-61 in magnitude.
+__device__ __forceinline__ bool has_tiny_nonzero(const float (&v)[8]) {
+    uint32_t least = 0xffffffffu;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t key = (__float_as_uint(v[j]) << 1) - 1u;      // zero wraps to the largest key
+        least = key < least ? key : least;
+    }
+    return least < ((66u << 24) - 1u);                                // exponent field below 66
+}
+
 // codec.py:105-142 `decode_nested` for one block given its coset point (already minus
 // the dither when there is one): the minimum-energy representative p - q * Q(p / q).
 __device__ __forceinline__ void reduce_coset_point(const float (&p)[8], float q, float (&out)[8]) {

@@ -105,6 +105,36 @@ def test_quantize_rows_matches_oracle(rt, oracle, rows, n, kind, dtype):
     _check_rows(rt, oracle, x, ACTIVATION_BETAS, dtype=dtype)
 
 
+@pytest.mark.parametrize("rows,n,dtype", [
+    (1100, 2048, torch.bfloat16),
+    (300, 8192, torch.bfloat16),
+    (2100, 1024, torch.float32),
+    (9000, 256, torch.float16),
+    (70, 32768, torch.float32),
+])
+def test_many_rows_take_the_throughput_kernel_and_match_oracle(rt, oracle, rows, n, dtype):
+    """From two million values on the encoder runs one lane per block (betas in turn, coset
+    reduction skipped where the lattice point lies inside the Voronoi cell, division through the
+    reciprocal): same bits as the oracle, also for zero rows, signed zeros, values far below
+    the rest of their row (which take the IEEE division) and rows in overload."""
+    x = torch.from_numpy(oracle.hadamard(student_t_rows(rows, n, seed=rows + n).numpy()))
+    x[1] = 0.0
+    x[2, ::3] = -0.0
+    x[3, 5::7] = 1e-25                      # quotients whose remainders would underflow
+    x[4, 1::2] = 3e-17                      # small, but above that limit
+    x[5] *= torch.linspace(0.0, 40.0, n)    # most blocks overloaded for the small betas
+    x[6, :8] = torch.tensor([1e4, -1e4, 0, 0, 0, 0, 0, 0])
+    codes, beta_ids, norms, _ = _check_rows(rt, oracle, x, ACTIVATION_BETAS, dtype=dtype)
+    # the row-at-a-time kernel (below the size limit) writes the same streams and BF16 decode
+    xd = x.to(dtype).cuda()
+    whole = rt.quantize_activation_cuda(xd, q=Q, betas=ACTIVATION_BETAS)
+    part = rt.quantize_activation_cuda(xd[:16], q=Q, betas=ACTIVATION_BETAS)
+    assert torch.equal(whole.code_payload, codes) and torch.equal(whole.beta_payload, beta_ids)
+    assert torch.equal(whole.decoded[:16], part.decoded)
+    assert torch.equal(whole.code_payload[: part.code_payload.numel()], part.code_payload)
+    _check_rows(rt, oracle, x[:, : n // 2].contiguous() if n >= 8192 else x, (0.25, 0.5, 1.0), dtype=dtype)
+
+
 def test_quantize_rows_key_value_tables_and_three_betas(rt, oracle):
     x = torch.from_numpy(np.random.default_rng(77).standard_normal((128, 64)).astype(np.float32))
     _check_rows(rt, oracle, x, KEY_BETAS, dtype=torch.bfloat16)
