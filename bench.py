@@ -60,7 +60,7 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--profile-copy", action="store_true",
                         help="also run three 256 MiB device-to-device copies (a kernel of known traffic, "
                              "to calibrate FETCH_SIZE / WRITE_SIZE counters under rocprofv3)")
-    parser.add_argument("--only", choices=("tpot", "gemm", "attention"), default=None,
+    parser.add_argument("--only", choices=("tpot", "gemm", "attention", "encode"), default=None,
                         help="run one of the extra measurements alone (for profiling) and print its JSON")
     parser.add_argument("--skip-extras", action="store_true",
                         help="only the headline GEMV workload (no prefill GEMM, attention, TPOT)")
@@ -258,6 +258,33 @@ def prefill_gemm_extra(rt, device):
     return results
 
 
+def encode_extra(rt, device):
+    """E8 row encoder alone: the 2048 x 2048 float32 plumbing case (undithered A4 and dithered
+    NQRT4 weight rows) and BF16 activations from one decode row to a long prefill, rotation fused.
+    Algorithmic bytes: rows * n * input size + rows * (n / 2 + n / 32 + 4)."""
+    import torch
+    results = {}
+    g = torch.Generator().manual_seed(58)
+    cases = [("config1_a4_f32", torch.randn(2048, 2048, generator=g), None, False),
+             ("config1_nqrt4_f32", torch.randn(2048, 2048, generator=g), 20261025, False)]
+    for m, n in ((1, 2048), (8, 2048), (1, 8192), (8, 8192), (128, 2048), (1024, 2048), (4096, 2048), (4096, 8192)):
+        cases.append((f"a4_bf16_m{m}_n{n}", torch.randn(m, n, generator=g).to(torch.bfloat16), None, True))
+    act = torch.tensor(ACTIVATION_BETAS, dtype=torch.float32, device=device)
+    wgt = torch.tensor(WEIGHT_BETAS, dtype=torch.float32, device=device)
+    for name, x, seed, rotate in cases:
+        x = x.to(device)
+        rows, n = x.shape
+        if seed is None:
+            fn = lambda i: rt.quantize_rows_packed(x, q=Q, beta_table=act, hadamard=rotate)
+        else:
+            fn = lambda i: rt.quantize_rows_packed(x, q=Q, beta_table=wgt, dither_seed=seed)
+        seconds = time_graph(fn, 16)
+        nbytes = rows * n * x.element_size() + rows * (n // 2 + n // 32 + 4)
+        results[name] = {"us": seconds * 1e6, "bytes": nbytes, "GBps": nbytes / seconds / 1e9,
+                         "hbm_frac": nbytes / seconds / 1e9 / HBM_PEAK_GBPS, "values_per_us": rows * n / seconds / 1e6}
+    return results
+
+
 def attention_extra(device):
     """Paged NQKV4 decode attention: 32 / 8 heads, D 64, batch 8, contexts uniform in [128, 4096]."""
     import torch
@@ -382,12 +409,6 @@ def main() -> None:
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
-    if args.only:
-        extra = {"tpot": lambda: tpot_extra(device), "gemm": lambda: prefill_gemm_extra(rt, device),
-                 "attention": lambda: attention_extra(device)}[args.only]()
-        print(json.dumps({args.only: extra}))
-        return
-
     if args.profile_copy:
         source = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=device).fill_(1)
         target = torch.empty_like(source)
@@ -395,6 +416,12 @@ def main() -> None:
             target.copy_(source)                 # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del source, target
+
+    if args.only:
+        extra = {"tpot": lambda: tpot_extra(device), "gemm": lambda: prefill_gemm_extra(rt, device),
+                 "attention": lambda: attention_extra(device), "encode": lambda: encode_extra(rt, device)}[args.only]()
+        print(json.dumps({args.only: extra}))
+        return
 
     cases, copies = build_workload(device)
     graphs, keep, stream = capture_steps(rt, cases, copies)
@@ -444,6 +471,7 @@ def main() -> None:
         for case in cases:
             case["weights"] = case["weights"][:1]
         torch.cuda.empty_cache()
+        result["extra"]["e8_encode"] = encode_extra(rt, device)
         result["extra"]["prefill_gemm"] = prefill_gemm_extra(rt, device)
         result["extra"]["nqkv_attention"] = attention_extra(device)
         result["extra"]["llama_1b_w4a4kv4"] = tpot_extra(device)
