@@ -115,6 +115,19 @@ int nq_hadamard(const void *x_dev, int x_dtype, int64_t rows, int64_t n, int sta
                 void *out_dev, int out_dtype, void *stream);
 
 /*
+ * Rotary position embedding and Hadamard rotation of BF16 head vectors x [rows, heads, head_dim]
+ * in one launch (prefill queries and keys).  rope_cos_dev / rope_sin_dev (optional, both or
+ * neither): BF16 [rows, head_dim]; (x * cos) + (rotate_half(x) * sin) in BF16 tensor arithmetic
+ * (every product and the sum rounded to BF16), as nq_nqkv_write applies it.  hadamard != 0 then
+ * applies the normalized Hadamard transform over head_dim with float32 butterflies, rounded to
+ * BF16 once.  head_dim is 64 or 128.
+ * Replaces: apply_rotary_pos_emb (transformers' Llama) followed by
+ * hadamard(x.float()).to(bfloat16), nestquant/runtime/nqkv_batched_hf_backend.py:381, 549.
+ */
+int nq_rope_hadamard(const void *x_dev, int64_t rows, int heads, int head_dim, const void *rope_cos_dev,
+                     const void *rope_sin_dev, int hadamard, void *out_dev, void *stream);
+
+/*
  * Inverse of nq_quantize_rows: out[r, :] = (decode(codes) * beta[id]) * (norm[r] / sqrt(n)).
  * With has_dither != 0 the stateless dither lcg31_mix_v1 of global block
  * block_offset + r * n/8 + b and `seed` is regenerated and subtracted (NQRT4 weights).

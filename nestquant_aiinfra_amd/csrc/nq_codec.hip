@@ -90,6 +90,12 @@ __device__ __forceinline__ void unpack_bf16x8(const uint4 raw, float (&v)[8]) {
     v[6] = __uint_as_float(raw.w << 16); v[7] = __uint_as_float(raw.w & 0xffff0000u);
 }
 
+// eight float32 values -> packed BF16, round to nearest even
+__device__ __forceinline__ uint4 pack_bf16x8(const float (&v)[8]) {
+    return make_uint4(__builtin_bit_cast(uint32_t, pack_bf16x2(v[0], v[1])), __builtin_bit_cast(uint32_t, pack_bf16x2(v[2], v[3])),
+                      __builtin_bit_cast(uint32_t, pack_bf16x2(v[4], v[5])), __builtin_bit_cast(uint32_t, pack_bf16x2(v[6], v[7])));
+}
+
 // eight float32 values that are exact BF16 numbers -> packed BF16
 __device__ __forceinline__ uint4 pack_bf16x8_exact(const float (&v)[8]) {
     return make_uint4((__float_as_uint(v[0]) >> 16) | (__float_as_uint(v[1]) & 0xffff0000u),
@@ -295,20 +301,24 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
 // Many rows: 256 lanes per workgroup, `rows_per_wg` rows of together at least 2048 values, one
 // lane per block in the encode phase (several such workgroups share a compute unit and fill
 // each other's serial stretches: the norm chain, the barriers of the rotation).
-template <typename T>
+template <typename T, int kPrologue>
 __global__ void __launch_bounds__(256)
 quantize_rows_bulk_kernel(const T *__restrict__ x, int64_t rows, int n, float q, float inv_q,
                           const float *__restrict__ betas, int beta_count, float sqrt_n,
                           uint32_t *__restrict__ codes, uint8_t *__restrict__ beta_ids,
                           float *__restrict__ norms, uint4 *__restrict__ decoded, int rows_per_wg,
-                          int vector_loads, int hadamard_stage_dtype) {
+                          int vector_loads, int hadamard_stage_dtype, InputPrologue pro) {
     extern __shared__ float lds[];
     float *row_scale = lds + (size_t)rows_per_wg * n;
     float *row_norm = row_scale + rows_per_wg;
     const int tid = threadIdx.x;
     const int64_t row0 = (int64_t)blockIdx.x * rows_per_wg;
     const int64_t first = row0 * n, limit = rows * (int64_t)n;
-    if (vector_loads) {
+    if (kPrologue != 0) {
+        stage_with_prologue<kPrologue>(reinterpret_cast<const uint16_t *>(x), pro, lds, row_scale, row_norm + rows_per_wg,
+                                       first, limit, rows_per_wg, n, true);
+        if (codes == nullptr) return;                      // element-wise stage only
+    } else if (vector_loads) {
         constexpr int kPer = RowLoader<T>::kPerVector;
         const int vectors = rows_per_wg * n / kPer;
 #pragma unroll 4
@@ -327,7 +337,7 @@ quantize_rows_bulk_kernel(const T *__restrict__ x, int64_t rows, int n, float q,
             lds[idx] = g < limit ? RowLoader<T>::scalar(x, g) : 0.0f;
         }
     }
-    __syncthreads();
+    if (kPrologue == 0) __syncthreads();
     if (hadamard_stage_dtype >= 0) staged_hadamard(lds, rows_per_wg, n, hadamard_stage_dtype);
     staged_row_norms(lds, rows_per_wg, n, sqrt_n, row_scale, row_norm);
     if (tid < rows_per_wg && row0 + tid < rows) norms[row0 + tid] = row_norm[tid];
@@ -395,6 +405,61 @@ hadamard_rows_kernel(const T *__restrict__ x, int64_t rows, int n, int rows_per_
     }
 }
 
+// Rotary position embedding and / or Hadamard rotation of BF16 head vectors [rows, heads, D]
+// (prefill queries and keys): eight values per lane, D / 8 neighbouring lanes per vector, no
+// LDS.  The embedding is (x * cos) + (rotate_half(x) * sin) in BF16 tensor arithmetic (every
+// product and the sum rounded to BF16); the rotation runs float32 butterflies and rounds once.
+template <int D>
+__global__ void __launch_bounds__(256)
+rope_hadamard_kernel(const uint16_t *__restrict__ x, int64_t vectors, int heads,
+                     const uint16_t *__restrict__ rope_cos, const uint16_t *__restrict__ rope_sin,
+                     int rotate, uint16_t *__restrict__ out) {
+    constexpr int kLanes = D / 8;
+    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;        // one 8-value chunk each
+    if (g >= vectors * kLanes) return;                                        // whole vectors leave together
+    const int lane = threadIdx.x & 63, part = (int)(g % kLanes);
+    float v[8];
+    unpack_bf16x8(reinterpret_cast<const uint4 *>(x)[g], v);
+    if (rope_cos) {
+        const int64_t at = (g / kLanes / heads) * kLanes + part;
+        float c[8], s[8];
+        unpack_bf16x8(reinterpret_cast<const uint4 *>(rope_cos)[at], c);
+        unpack_bf16x8(reinterpret_cast<const uint4 *>(rope_sin)[at], s);
+        const bool upper = part >= kLanes / 2;
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            float o0 = lane_xor<kLanes / 2>(v[j]), o1 = lane_xor<kLanes / 2>(v[j + 1]);
+            float a0 = v[j] * c[j], a1 = v[j + 1] * c[j + 1];
+            round_pair<1>(a0, a1);
+            float b0 = o0 * s[j], b1 = o1 * s[j + 1];
+            round_pair<1>(b0, b1);
+            v[j] = upper ? a0 + b0 : a0 - b0;
+            v[j + 1] = upper ? a1 + b1 : a1 - b1;
+            round_pair<1>(v[j], v[j + 1]);
+        }
+    }
+    if (rotate) {
+#pragma unroll
+        for (int s = 0; s < 3; s++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                if (j & (1 << s)) continue;
+                const float left = v[j], right = v[j + (1 << s)];
+                v[j] = left + right;
+                v[j + (1 << s)] = left - right;
+            }
+        }
+        lane_stage<1, 0>(v, lane);
+        lane_stage<2, 0>(v, lane);
+        lane_stage<4, 0>(v, lane);
+        if (kLanes > 8) lane_stage<8, 0>(v, lane);
+        const float inv = 1.0f / __builtin_sqrtf((float)D);
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = v[j] * inv;
+    }
+    reinterpret_cast<uint4 *>(out)[g] = pack_bf16x8(v);
+}
+
 }  // namespace nq
 
 extern "C" int nq_hadamard(const void *x_dev, int x_dtype, int64_t rows, int64_t n, int stage_dtype,
@@ -429,6 +494,34 @@ extern "C" int nq_hadamard(const void *x_dev, int x_dtype, int64_t rows, int64_t
     return nq::check_launch("nq_hadamard");
 }
 
+extern "C" int nq_rope_hadamard(const void *x_dev, int64_t rows, int heads, int head_dim, const void *rope_cos_dev,
+                                const void *rope_sin_dev, int hadamard, void *out_dev, void *stream) {
+    NQ_REQUIRE(rows >= 1 && heads >= 1, NQ_ERR_SHAPE, "nq_rope_hadamard: rows and heads must be positive");
+    NQ_REQUIRE(head_dim == 64 || head_dim == 128, NQ_ERR_SHAPE, "nq_rope_hadamard: head_dim %d is not 64 or 128", head_dim);
+    NQ_REQUIRE(x_dev && out_dev, NQ_ERR_ARGUMENT, "nq_rope_hadamard: null pointer");
+    NQ_REQUIRE((rope_cos_dev == nullptr) == (rope_sin_dev == nullptr), NQ_ERR_ARGUMENT,
+               "nq_rope_hadamard: rotary tables come as a pair");
+    NQ_REQUIRE(nq::aligned(x_dev, 16) && nq::aligned(out_dev, 16) && nq::aligned(rope_cos_dev, 16) &&
+                   nq::aligned(rope_sin_dev, 16), NQ_ERR_ARGUMENT, "nq_rope_hadamard: pointers must be 16-byte aligned");
+    const int64_t vectors = rows * heads, chunks = vectors * (head_dim / 8);
+    const int64_t grid = (chunks + 255) / 256;
+    NQ_REQUIRE(grid <= 0x7fffffff, NQ_ERR_SHAPE, "nq_rope_hadamard: too many vectors");
+    hipStream_t s = (hipStream_t)stream;
+    if (head_dim == 64)
+        hipLaunchKernelGGL(nq::rope_hadamard_kernel<64>, dim3((unsigned)grid), dim3(256), 0, s,
+                           reinterpret_cast<const uint16_t *>(x_dev), vectors, heads,
+                           reinterpret_cast<const uint16_t *>(rope_cos_dev),
+                           reinterpret_cast<const uint16_t *>(rope_sin_dev), hadamard,
+                           reinterpret_cast<uint16_t *>(out_dev));
+    else
+        hipLaunchKernelGGL(nq::rope_hadamard_kernel<128>, dim3((unsigned)grid), dim3(256), 0, s,
+                           reinterpret_cast<const uint16_t *>(x_dev), vectors, heads,
+                           reinterpret_cast<const uint16_t *>(rope_cos_dev),
+                           reinterpret_cast<const uint16_t *>(rope_sin_dev), hadamard,
+                           reinterpret_cast<uint16_t *>(out_dev));
+    return nq::check_launch("nq_rope_hadamard");
+}
+
 extern "C" int nq_e8_nearest(const float *x_dev, float *out_dev, int64_t count, void *stream) {
     NQ_REQUIRE(count >= 0, NQ_ERR_SHAPE, "nq_e8_nearest: count must be non-negative");
     if (count == 0) return NQ_OK;
@@ -454,10 +547,10 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
                     uint32_t seed_plus_offset, uint8_t *codes, uint8_t *beta_ids, float *norms,
                     void *decoded, int hadamard_stage_dtype, hipStream_t stream,
                     nq::InputPrologue prologue = nq::InputPrologue{}) {
-    if (!kDithered && kPrologue == 0 && rows * (int64_t)n >= kBulkElements) {
+    if (!kDithered && rows * (int64_t)n >= kBulkElements) {
         int rows_per_wg = n >= 2048 ? 1 : 2048 / n;
-        const size_t lds_bytes = ((size_t)rows_per_wg * n + 2 * rows_per_wg) * sizeof(float);
-        auto kernel = nq::quantize_rows_bulk_kernel<T>;
+        const size_t lds_bytes = ((size_t)rows_per_wg * n + 2 * rows_per_wg + (kPrologue == 1 ? n : 0)) * sizeof(float);
+        auto kernel = nq::quantize_rows_bulk_kernel<T, kPrologue>;
         if (lds_bytes > 48 * 1024) {
             hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -471,7 +564,7 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
                            reinterpret_cast<const T *>(x), rows, n, (float)q, 1.0f / (float)q, betas, beta_count,
                            (float)sqrt((double)n), reinterpret_cast<uint32_t *>(codes), beta_ids, norms,
                            reinterpret_cast<uint4 *>(decoded), rows_per_wg, (int)nq::aligned(x, 16),
-                           hadamard_stage_dtype);
+                           hadamard_stage_dtype, prologue);
         return nq::check_launch("nq_quantize_rows");
     }
     const int pairs_per_row = n / 2;

@@ -17,16 +17,23 @@ per layer:
     SiLU(gate) * up + Hadamard + A4 encode             nq_fused_input_stage (mode 2)
     down_proj                                          nq_w4a4_gemv
 
-The module graph stays the path for prefill and for models this step does not recognise.
+FusedLlamaPrefillStep runs a prompt (or a chunk of one) the same way over [rows * tokens]
+activation rows: the input stages and linears as above (the linears on the matrix cores), RoPE
+and Hadamard of queries and keys in one launch each, the KV writer, and the attention the
+module graph would use (PyTorch's SDPA over the rotated BF16 keys and values of the chunk, or
+the packed-cache kernel for a continuation).  The module graph stays the path for models these
+steps do not recognise.
 """
 
 from __future__ import annotations
 
 import torch
 
-from .nqkv import launch_nqkv_decode_attention
+import torch.nn.functional as F
+
+from .nqkv import launch_nqkv_decode_attention, nqkv_prefill_attention
 from .w4a4_linear import (PreparedNQRTLinear, _gemm, _gemv, fused_input_stage, linear_packed_w4a4_gemv_grouped,
-                          quantize_activation_cuda)
+                          quantize_activation_cuda, rope_hadamard_cuda)
 
 
 class UnsupportedForFusedDecode(ValueError):
@@ -135,3 +142,59 @@ class FusedLlamaDecodeStep:
         _, _, normed = fused_input_stage(delta, mode="rmsnorm", residual=residual, norm_weight=inner.norm.weight,
                                          eps=inner.norm.variance_epsilon, encode=False, want_staged=True)
         return self.model.lm_head(normed.view(rows, 1, self.hidden))
+
+
+class FusedLlamaPrefillStep(FusedLlamaDecodeStep):
+    """Callable `(tokens [rows, width], positions [rows, width]) -> logits [rows, width, vocab]`
+    for the rows `BatchedNQKVLlamaCache.set_batch_state` has announced; same model requirements
+    as FusedLlamaDecodeStep."""
+
+    @torch.inference_mode()
+    def __call__(self, tokens: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        cache, inner = self.cache, self.inner
+        manager = cache.manager
+        rows, width = tokens.shape
+        if positions.shape != (rows, width) or rows != cache._rows:
+            raise ValueError("the fused prefill step takes [rows, width] tokens and positions for the rows in flight")
+        device = tokens.device
+        embedded = inner.embed_tokens(tokens)                               # [rows, width, hidden]
+        if embedded.dtype != torch.bfloat16:
+            raise TypeError("the fused prefill step runs BF16 models")
+        count = rows * width
+        cos, sin = inner.rotary_emb(embedded, positions)                    # [rows, width, head_dim]
+        heads, kv_heads, dim = cache.num_query_heads, cache.num_kv_heads, cache.head_dim
+        rope = (cos.to(torch.bfloat16).reshape(count, dim).contiguous(), sin.to(torch.bfloat16).reshape(count, dim).contiguous())
+        over_cache = cache.packed_prefill or cache._continuation
+
+        delta, residual = embedded.reshape(count, self.hidden), None
+        for index, (layer, attention, mlp, linears) in enumerate(self.layers):
+            q_w, k_w, v_w, o_w, gate_w, up_w, down_w = (self._prepared(linear, device) for linear in linears)
+            table = linears[0].activation_beta_table
+            activation, residual, _ = fused_input_stage(
+                delta, mode="rmsnorm", residual=residual, norm_weight=layer.input_layernorm.weight,
+                eps=layer.input_layernorm.variance_epsilon, beta_table=table, want_residual=True)
+            query, key, value = self._linears(activation, [q_w, k_w, v_w])
+            query = rope_hadamard_cuda(query.view(count, heads, dim), rope=rope).view(rows, width, heads, dim)
+            key = rope_hadamard_cuda(key.view(count, kv_heads, dim), rope=rope).view(rows, width, kv_heads, dim)
+            value = value.view(rows, width, kv_heads, dim)
+            manager.write_layer(index, key, value)
+            scale = float(attention.scaling)
+            if over_cache:
+                attended = nqkv_prefill_attention(query, manager.layers[index], slot_ids=manager.step_slot_ids,
+                                                  active_mask=manager.step_active, counts=manager.step_counts, scale=scale)
+            else:
+                attended = F.scaled_dot_product_attention(
+                    query.transpose(1, 2), key.transpose(1, 2), value.transpose(1, 2), dropout_p=0.0, is_causal=True,
+                    scale=scale, enable_gqa=heads != kv_heads).transpose(1, 2)
+            o_input = quantize_activation_cuda(attended.reshape(count, heads * dim), q=14,
+                                               betas=linears[3].activation_betas, beta_table=table, hadamard=True)
+            delta = self._linear(o_input, o_w)
+            activation, residual, _ = fused_input_stage(
+                delta, mode="rmsnorm", residual=residual, norm_weight=layer.post_attention_layernorm.weight,
+                eps=layer.post_attention_layernorm.variance_epsilon, beta_table=table, want_residual=True)
+            gate, up = self._linears(activation, [gate_w, up_w])
+            activation, _, _ = fused_input_stage(up, mode="swiglu", gate=gate, beta_table=table)
+            delta = self._linear(activation, down_w)
+        _, _, normed = fused_input_stage(delta, mode="rmsnorm", residual=residual, norm_weight=inner.norm.weight,
+                                         eps=inner.norm.variance_epsilon, encode=False, want_staged=True)
+        return self.model.lm_head(normed.view(rows, width, self.hidden))

@@ -260,9 +260,10 @@ class BatchedNQKVLlamaRunner:
     """
 
     def __init__(self, model: torch.nn.Module, cache: BatchedNQKVLlamaCache, *,
-                 fused_decode: bool | None = None) -> None:
-        """`fused_decode`: run decode steps through FusedLlamaDecodeStep (eleven launches per
-        layer) instead of the module graph; None = whenever the model qualifies."""
+                 fused_decode: bool | None = None, fused_prefill: bool | None = None) -> None:
+        """`fused_decode` / `fused_prefill`: run decode steps through FusedLlamaDecodeStep (eleven
+        launches per layer) and prompts through FusedLlamaPrefillStep instead of the module
+        graph; None = whenever the model qualifies."""
         if not isinstance(model, torch.nn.Module):
             raise TypeError("model must be a torch module")
         if not isinstance(cache, BatchedNQKVLlamaCache):
@@ -285,6 +286,14 @@ class BatchedNQKVLlamaRunner:
                 self.fused_step = FusedLlamaDecodeStep(model, cache)
             except UnsupportedForFusedDecode:
                 if fused_decode:
+                    raise
+        self.fused_prefill = None
+        if fused_prefill is None or fused_prefill:
+            from .llama_decode_step import FusedLlamaPrefillStep, UnsupportedForFusedDecode
+            try:
+                self.fused_prefill = FusedLlamaPrefillStep(model, cache)
+            except UnsupportedForFusedDecode:
+                if fused_prefill:
                     raise
 
     @property
@@ -309,6 +318,8 @@ class BatchedNQKVLlamaRunner:
             positions = starts[:, None] + torch.arange(width, device=self.device)[None, :]
         self._decode_state = None
         self.cache.set_batch_state(slot_ids=slots, counts=lengths)
+        if self.fused_prefill is not None:
+            return self.fused_prefill(input_ids, positions)
         output = self.model(input_ids=input_ids, position_ids=positions, past_key_values=self.cache, use_cache=True)
         return output.logits
 

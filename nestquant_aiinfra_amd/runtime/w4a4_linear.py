@@ -127,6 +127,26 @@ def hadamard_cuda(inputs: torch.Tensor, *, compute_dtype: torch.dtype | None = N
     return out
 
 
+def rope_hadamard_cuda(vectors: torch.Tensor, *, rope: tuple[torch.Tensor, torch.Tensor] | None = None,
+                       hadamard: bool = True) -> torch.Tensor:
+    """Rotary embedding and / or Hadamard rotation of BF16 head vectors [rows, heads, head_dim]
+    in one kernel: `rope` = BF16 (cos, sin) [rows, head_dim] applied as transformers'
+    apply_rotary_pos_emb does in BF16, then ``hadamard(x.float()).to(bfloat16)``."""
+    device = _native.require_cuda(vectors)
+    if vectors.dtype != torch.bfloat16 or vectors.ndim != 3 or not vectors.is_contiguous():
+        raise ValueError("expected a contiguous BF16 tensor [rows, heads, head_dim]")
+    rows, heads, dim = vectors.shape
+    if rope is not None:
+        for table in rope:
+            if table.dtype != torch.bfloat16 or tuple(table.shape) != (rows, dim) or not table.is_contiguous():
+                raise ValueError("rotary tables must be contiguous BF16 [rows, head_dim]")
+    out = torch.empty_like(vectors)
+    _native.check(_native.library().nq_rope_hadamard(
+        vectors.data_ptr(), rows, heads, dim, None if rope is None else rope[0].data_ptr(),
+        None if rope is None else rope[1].data_ptr(), int(hadamard), out.data_ptr(), _native.stream_handle(device)))
+    return out
+
+
 def quantize_activation_cuda(inputs: torch.Tensor, *, q: int, betas: Sequence[float],
                              beta_table: torch.Tensor | None = None,
                              hadamard: bool = False) -> PreparedNQA4Activation:

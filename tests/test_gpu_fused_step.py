@@ -4,8 +4,9 @@
   * nq_w4a4_gemv_grouped against one nq_w4a4_gemv call per weight (bit for bit);
   * the rotary embedding inside nq_nqkv_write / nq_nqkv_attention_decode against the same
     BF16 tensor arithmetic done beforehand (bit for bit);
-  * FusedLlamaDecodeStep against the module graph of the same tiny model (tolerance: the
-    row reductions of the norm run in a different order).
+  * nq_rope_hadamard against the BF16 rotary embedding and float32 Hadamard it replaces;
+  * FusedLlamaDecodeStep and FusedLlamaPrefillStep against the module graph of the same tiny
+    model (tolerance: the row reductions of the norm run in a different order).
 """
 
 import numpy as np
@@ -42,7 +43,7 @@ def _rms_norm(h, weight, eps):
     return weight * x.to(h.dtype)
 
 
-@pytest.mark.parametrize("rows,n", [(1, 2048), (8, 2048), (3, 256), (5, 8192), (40, 512)])
+@pytest.mark.parametrize("rows,n", [(1, 2048), (8, 2048), (3, 256), (5, 8192), (40, 512), (1100, 2048), (4200, 512)])
 @pytest.mark.parametrize("with_residual", [False, True])
 def test_residual_rmsnorm_stage(rt, rows, n, with_residual):
     g = torch.Generator().manual_seed(rows * n + with_residual)
@@ -55,9 +56,11 @@ def test_residual_rmsnorm_stage(rt, rows, n, with_residual):
     expect_h = x + residual if with_residual else x
     assert torch.equal(h, expect_h)
     expect = _rms_norm(expect_h, weight, eps)
-    # one BF16 step at most, and only where the differently ordered mean moved a rounding
+    # only where the differently ordered mean moved a rounding: one BF16 step, or (a few values per
+    # million) two when the step of the normalised value is stretched by a weight above one
     difference = (staged.float() - expect.float()).abs()
-    assert bool((difference <= expect.float().abs() * 2.0 ** -7 + 1e-30).all())
+    assert bool((difference <= expect.float().abs() * 2.0 ** -6 + 1e-30).all())
+    assert int((difference > expect.float().abs() * 2.0 ** -7 + 1e-30).sum()) <= rows * n // 100000
     assert int((staged != expect).sum()) <= max(2, rows * n // 200)
     # the encode that follows is the plain encoder on the staged rows
     plain = rt.quantize_activation_cuda(staged, q=Q, betas=ACTIVATION_BETAS, hadamard=True)
@@ -68,7 +71,7 @@ def test_residual_rmsnorm_stage(rt, rows, n, with_residual):
     assert none is None and torch.equal(staged_only, staged)
 
 
-@pytest.mark.parametrize("rows,n", [(1, 8192), (8, 8192), (2, 512)])
+@pytest.mark.parametrize("rows,n", [(1, 8192), (8, 8192), (2, 512), (300, 8192)])
 def test_swiglu_stage(rt, rows, n):
     g = torch.Generator().manual_seed(rows + n)
     gate = (2 * torch.randn(rows, n, generator=g)).to(torch.bfloat16).cuda()
@@ -165,6 +168,76 @@ def test_rotary_embedding_inside_writer_and_attention():
     inside = kv.launch_nqkv_decode_attention(query, a, rope=(cos.view(2, dim), sin.view(2, dim)), **common).clone()
     before = kv.launch_nqkv_decode_attention(_apply_rope(query, cos, sin).contiguous(), a, **common).clone()
     assert torch.equal(inside, before) and bool(inside.float().abs().sum() > 0)
+
+
+@pytest.mark.parametrize("heads,dim", [(8, 64), (3, 128)])
+def test_rope_and_rotation_of_head_vectors_in_one_launch(rt, heads, dim):
+    from nestquant_aiinfra_amd.core.rotation import hadamard
+    rows = 37
+    g = torch.Generator().manual_seed(heads * dim)
+    x = torch.randn(rows, heads, dim, generator=g).to(torch.bfloat16).cuda()
+    cos, sin = _rope_tables(rows, 1, dim, seed=5)
+    cos, sin = cos.view(rows, dim), sin.view(rows, dim)
+    embedded = _apply_rope(x, cos[:, None, :], sin[:, None, :])
+    assert torch.equal(rt.rope_hadamard_cuda(x, rope=(cos, sin), hadamard=False), embedded)
+    assert torch.equal(rt.rope_hadamard_cuda(x, hadamard=True), hadamard(x.float()).to(torch.bfloat16))
+    assert torch.equal(rt.rope_hadamard_cuda(x, rope=(cos, sin)), hadamard(embedded.float()).to(torch.bfloat16))
+    with pytest.raises(ValueError):
+        rt.rope_hadamard_cuda(x, rope=(cos[:5], sin[:5]))
+    with pytest.raises(ValueError):
+        rt.rope_hadamard_cuda(torch.zeros(2, 2, 32, dtype=torch.bfloat16, device="cuda"))
+
+
+def _tiny_runners(tmp_path, seed, capacity, max_cache_len):
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
+
+    runners = []
+    for fused in (True, False):
+        torch.manual_seed(seed)
+        config = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                             num_key_value_heads=2, head_dim=64, vocab_size=128, max_position_embeddings=512,
+                             rope_theta=500000.0, tie_word_embeddings=True)
+        model = LlamaForCausalLM(config).to(torch.bfloat16).cuda().eval()
+        path = tmp_path / f"tiny{int(fused)}.nqmc"
+        asm.write_w4_checkpoint(model, path)
+        runners.append(asm.build_w4a4kv4_runner(model, path, capacity=capacity, max_cache_len=max_cache_len,
+                                                fused_prefill=fused, fused_decode=fused))
+    return runners
+
+
+def test_fused_prefill_step_tracks_the_module_graph(tmp_path):
+    """A ragged prompt batch, then a continuation chunk over the packed cache, then decode steps:
+    the fused prefill step against the module graph of an identical model (tolerance: the
+    row reductions of the norm run in a different order, so activations differ in the last place
+    and a few codes with them)."""
+    fused, modular = _tiny_runners(tmp_path, 5005, capacity=3, max_cache_len=160)
+    assert fused.fused_prefill is not None and modular.fused_prefill is None
+    g = torch.Generator().manual_seed(5006)
+    ids = torch.randint(0, 128, (3, 70), generator=g).cuda()
+    lengths = [70, 33, 1]
+    more = torch.randint(0, 128, (3, 40), generator=g).cuda()
+    more_lengths = [40, 17, 5]
+
+    def run(runner):
+        first = runner.prefill_slots(ids, slots=[0, 1, 2], lengths=lengths).float()
+        second = runner.prefill_slots(more, slots=[0, 1, 2], lengths=more_lengths).float()     # continuation
+        token = torch.stack([second[i, n - 1].argmax() for i, n in enumerate(more_lengths)]).reshape(3, 1)
+        position = torch.tensor([[a + b] for a, b in zip(lengths, more_lengths)], device="cuda")
+        step = runner.decode_eager(token * 0 + 7, slots=[0, 1, 2], positions=position).float()
+        return first, second, step
+    a, b = run(fused), run(modular)
+    for i, (n, m) in enumerate(zip(lengths, more_lengths)):
+        for got, want, count in ((a[0][i], b[0][i], n), (a[1][i], b[1][i], m)):
+            got, want = got[:count], want[:count]
+            assert torch.isfinite(got).all()
+            cosine = torch.nn.functional.cosine_similarity(got, want, dim=-1)
+            assert float(cosine.min()) > 0.99, (i, float(cosine.min()))
+            assert relative_error(bits(got), bits(want)) < 0.08
+    cosine = torch.nn.functional.cosine_similarity(a[2].flatten(1), b[2].flatten(1), dim=1)
+    assert float(cosine.min()) > 0.99
+    lengths_a = fused.cache.manager.metadata.sequence_lengths[:3].tolist()
+    assert lengths_a == modular.cache.manager.metadata.sequence_lengths[:3].tolist() == [111, 51, 7]
 
 
 def test_fused_decode_step_tracks_the_module_graph(tmp_path):
