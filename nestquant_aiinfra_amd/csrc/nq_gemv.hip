@@ -174,6 +174,100 @@ w4a4_gemv_grouped_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_row
                           out_is_f32 ? nullptr : (uint16_t *)w.out[which]);
 }
 
+// Five to sixteen tokens: the dot products move to the matrix cores.  A decoded E8 block is
+// exactly one lane's A fragment of v_mfma_f32_16x16x32_bf16 (lane l: channel l % 16, eight
+// consecutive k), so a wavefront that decodes 16 channels x 4 blocks multiplies them by the
+// matching activation fragment (lane l: token l % 16, the same eight k) with no exchange, no
+// LDS and no per-token work on the vector units.  A workgroup owns 16 channels; its wavefronts
+// (up to 16) take super-steps of 128 k in turn and each lane reads 16 contiguous bytes of words,
+// 8 of tails and 64 of activation per super-step, requested one super-step ahead.  Partial
+// tiles meet in LDS and are added in wavefront order.  (The 4 x 4 x 4 block instruction would
+// allow four channels per workgroup, but issues at a quarter of this one's rate.)
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+constexpr int kMfmaGemvMaxWaves = 16;
+
+__global__ void __launch_bounds__(kMfmaGemvMaxWaves * 64)
+w4a4_gemv_mfma_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, int k_size, float sqrt_k,
+                      int out_is_f32) {
+    __shared__ float part[kMfmaGemvMaxWaves][256];
+    int which = 0;
+#pragma unroll
+    for (int i = 1; i < kGemvMaxGroup; i++)
+        if (i < w.count && (int)blockIdx.x >= w.first_group[i]) which = i;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
+    const int n_size = w.n[which], n0 = ((int)blockIdx.x - w.first_group[which]) * 16;
+    const int column = lane & 15, quarter = lane >> 4;
+    const int blocks_per_row = k_size >> 3, super_steps = k_size >> 7;
+    const int n = n0 + column < n_size ? n0 + column : n_size - 1;          // channels past the end repeat the last one
+    const float wscale = (w.norms[which][n] / sqrt_k) * kResolvedUnit;
+    const float *betas = w.betas[which];
+    const float wbeta[4] = {betas[0], betas[1], betas[2], betas[3]};
+    const uint32_t seed_plus_offset = w.seed_plus_offset[which];
+    const int64_t row_first = (int64_t)n * blocks_per_row + 4 * quarter;
+    const uint32_t *words = w.words[which];
+    const uint16_t *tails = w.tails[which];
+    const bool has_token = column < m_rows;
+    const uint4 *act_row = act + (int64_t)(has_token ? column : 0) * blocks_per_row + 4 * quarter;
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+
+    floatx4 acc = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    uint4 word_next = zero, b_next[4] = {zero, zero, zero, zero};
+    uint2 tail_next = make_uint2(0, 0);
+    if (wave < super_steps) {
+        word_next = *reinterpret_cast<const uint4 *>(words + row_first + 16 * wave);
+        tail_next = *reinterpret_cast<const uint2 *>(tails + row_first + 16 * wave);
+        if (has_token) {
+#pragma unroll
+            for (int t = 0; t < 4; t++) b_next[t] = act_row[16 * wave + t];
+        }
+    }
+    for (int ss = wave; ss < super_steps; ss += waves) {
+        const uint4 word4 = word_next;
+        const uint2 tail2 = tail_next;
+        uint4 b[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) b[t] = b_next[t];
+        if (ss + waves < super_steps) {
+            word_next = *reinterpret_cast<const uint4 *>(words + row_first + 16 * (ss + waves));
+            tail_next = *reinterpret_cast<const uint2 *>(tails + row_first + 16 * (ss + waves));
+            if (has_token) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) b_next[t] = act_row[16 * (ss + waves) + t];
+            }
+        }
+        const uint32_t word[4] = {word4.x, word4.y, word4.z, word4.w};
+        const uint32_t tail[4] = {tail2.x & 0xffffu, tail2.x >> 16, tail2.y & 0xffffu, tail2.y >> 16};
+        const int64_t g = row_first + 16 * ss;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            float v[8];
+            decode_resolved(word[t], tail[t], seed_plus_offset + (uint32_t)(g + t) * 8u, v);
+            const float scale = wbeta[word[t] >> 30] * wscale;
+            const bf16x2 h0 = pack_bf16x2(v[0] * scale, v[1] * scale), h1 = pack_bf16x2(v[2] * scale, v[3] * scale);
+            const bf16x2 h2 = pack_bf16x2(v[4] * scale, v[5] * scale), h3 = pack_bf16x2(v[6] * scale, v[7] * scale);
+            const uint4 a = make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
+                                       __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b[t]),
+                                                          acc, 0, 0, 0);
+        }
+    }
+    // accumulator r of lane l: channel 4 (l / 16) + r, token l % 16
+#pragma unroll
+    for (int r = 0; r < 4; r++) part[wave][(4 * quarter + r) * 16 + column] = acc[r];
+    __syncthreads();
+    if (tid < 256) {
+        const int channel = tid >> 4, token = tid & 15;
+        if (n0 + channel < n_size && token < m_rows) {
+            float total = part[0][tid];
+            for (int i = 1; i < waves; i++) total = total + part[i][tid];
+            const int64_t at = (int64_t)token * n_size + n0 + channel;
+            if (out_is_f32) reinterpret_cast<float *>(w.out[which])[at] = total;
+            else reinterpret_cast<uint16_t *>(w.out[which])[at] = f32_to_bf16(total);
+        }
+    }
+}
+
 // One lane per weight block: run the exact decode once and keep the lattice point it implies.
 __global__ void __launch_bounds__(256)
 resolve_weight_kernel(const uint32_t *__restrict__ w_codes, const uint8_t *__restrict__ w_beta_ids,
@@ -216,6 +310,28 @@ extern "C" int nq_w4a4_resolve_weight(const uint8_t *w_codes_dev, const uint8_t 
 
 namespace {
 
+// The matrix-core kernel (resolved weights, K a multiple of 128, 16-byte aligned streams) works
+// in tiles of 16 channels: above eight rows it is the only decode kernel, from five rows on it
+// is taken when there are enough tiles for most of the chip (192: q/k/v or gate/up together).
+constexpr int kMfmaGemvMinRows = 5;
+constexpr int kMfmaGemvMaxRows = 16;
+constexpr int kMfmaGemvMinTiles = 192;
+
+bool takes_mfma_gemv(int m, int k, int64_t total_n, bool resolved) {
+    if (!resolved || k % 128 != 0 || m > kMfmaGemvMaxRows) return false;
+    return m > 8 || (m >= kMfmaGemvMinRows && (total_n + 15) / 16 >= kMfmaGemvMinTiles);
+}
+
+int launch_mfma_gemv(const void *act, const nq::GemvWeights &w, int groups, int m, int k, int out_is_f32,
+                     hipStream_t stream) {
+    const int super_steps = k / 128;
+    int waves = super_steps < nq::kMfmaGemvMaxWaves ? super_steps : nq::kMfmaGemvMaxWaves;
+    if (waves < 4) waves = 4;                    // the last stage wants 256 lanes
+    hipLaunchKernelGGL(nq::w4a4_gemv_mfma_kernel, dim3((unsigned)groups), dim3(64 * waves), 0, stream,
+                       reinterpret_cast<const uint4 *>(act), w, m, k, (float)sqrt((double)k), out_is_f32);
+    return nq::check_launch("nq_w4a4_gemv (matrix cores)");
+}
+
 int m_tile_of(int m) { return m == 1 ? 1 : (m == 2 ? 2 : (m <= 4 ? 4 : 8)); }
 
 // A workgroup consumes 2048 K-elements per step.  Only long-K shapes too narrow to give
@@ -248,7 +364,10 @@ extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_bet
                             const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
                             int64_t weight_seed, int split_k, void *out_dev, int out_dtype,
                             void *workspace_dev, size_t workspace_bytes, void *stream) {
-    NQ_REQUIRE(m >= 1 && m <= 8, NQ_ERR_SHAPE, "nq_w4a4_gemv: M = %d is outside [1, 8]", m);
+    const bool mfma = takes_mfma_gemv(m, k, n, w_resolved_words_dev != nullptr) && split_k <= 1 &&
+                      nq::aligned(w_resolved_words_dev, 16) && nq::aligned(w_resolved_tails_dev, 8);
+    NQ_REQUIRE(m >= 1 && (m <= 8 || mfma), NQ_ERR_SHAPE,
+               "nq_w4a4_gemv: M = %d is outside [1, 8] (up to 16 with resolved weights and K a multiple of 128)", m);
     NQ_REQUIRE(k >= 32 && k % 32 == 0, NQ_ERR_SHAPE, "nq_w4a4_gemv: K = %d must be a positive multiple of 32", k);
     NQ_REQUIRE(n >= 1, NQ_ERR_SHAPE, "nq_w4a4_gemv: N must be positive");
     NQ_REQUIRE(split_k == 0 || split_k == 1 || split_k == 2 || split_k == 4 || split_k == 8,
@@ -269,7 +388,7 @@ extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_bet
                "nq_w4a4_gemv: seed must be in [0, 2**31)");
     NQ_REQUIRE(weight_offset >= 0 && weight_offset + (int64_t)n * (k / 8) <= ((int64_t)1 << 28),
                NQ_ERR_SHAPE, "nq_w4a4_gemv: block range exceeds the stateless dither counter space");
-    const int split = pick_split(k, n, split_k);
+    const int split = mfma ? 1 : pick_split(k, n, split_k);
     NQ_REQUIRE(k % split == 0 && (k / split) % 32 == 0, NQ_ERR_SHAPE,
                "nq_w4a4_gemv: K / split_k = %d / %d must be a multiple of 32", k, split);
     const size_t decoded_bytes = act_decoded_dev ? 0 : nq::align256((size_t)m * k * 2);
@@ -289,6 +408,19 @@ extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_bet
         act = reinterpret_cast<const uint4 *>(workspace_dev);
     }
     float *partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace_dev) + decoded_bytes);
+    if (mfma) {
+        nq::GemvWeights one{};
+        one.count = 1;
+        one.words[0] = w_resolved_words_dev;
+        one.tails[0] = w_resolved_tails_dev;
+        one.norms[0] = w_norms_dev;
+        one.betas[0] = w_betas_dev;
+        one.out[0] = out_dev;
+        one.n[0] = n;
+        one.first_group[0] = 0;
+        one.seed_plus_offset[0] = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
+        return launch_mfma_gemv(act, one, (n + 15) / 16, m, k, out_dtype == NQ_F32, s);
+    }
 
     const int k_slice = k / split;
     // few rows per workgroup keeps many short wavefronts in flight on every SIMD
@@ -328,7 +460,14 @@ extern "C" int nq_w4a4_gemv_grouped(const void *act_decoded_dev, int count, cons
                                     void *stream) {
     NQ_REQUIRE(count >= 1 && count <= nq::kGemvMaxGroup, NQ_ERR_SHAPE,
                "nq_w4a4_gemv_grouped: between 1 and %d weights per launch", nq::kGemvMaxGroup);
-    NQ_REQUIRE(m >= 1 && m <= 8, NQ_ERR_SHAPE, "nq_w4a4_gemv_grouped: M = %d is outside [1, 8]", m);
+    int64_t total_n = 0;
+    for (int i = 0; n && i < count; i++) total_n += n[i];
+    bool mfma = takes_mfma_gemv(m, k, total_n, true);
+    for (int i = 0; mfma && i < count; i++)
+        mfma = w_resolved_words_dev && w_resolved_tails_dev && nq::aligned(w_resolved_words_dev[i], 16) &&
+               nq::aligned(w_resolved_tails_dev[i], 8);
+    NQ_REQUIRE(m >= 1 && (m <= 8 || mfma), NQ_ERR_SHAPE,
+               "nq_w4a4_gemv_grouped: M = %d is outside [1, 8] (up to 16 with K a multiple of 128)", m);
     NQ_REQUIRE(k >= 32 && k % 32 == 0, NQ_ERR_SHAPE, "nq_w4a4_gemv_grouped: K = %d must be a positive multiple of 32", k);
     NQ_REQUIRE(out_dtype == NQ_F32 || out_dtype == NQ_BF16, NQ_ERR_ARGUMENT,
                "nq_w4a4_gemv_grouped: output dtype tag %d is not F32 or BF16", out_dtype);
@@ -338,9 +477,7 @@ extern "C" int nq_w4a4_gemv_grouped(const void *act_decoded_dev, int count, cons
                    weight_seeds && out_dev, NQ_ERR_ARGUMENT, "nq_w4a4_gemv_grouped: null argument array");
     nq::GemvWeights w{};
     w.count = count;
-    int64_t total_n = 0;
-    for (int i = 0; i < count; i++) total_n += n[i];
-    const int rows_per_wg = total_n >= 8192 ? 4 : 2;
+    const int rows_per_wg = mfma ? 16 : (total_n >= 8192 ? 4 : 2);
     int groups = 0;
     for (int i = 0; i < count; i++) {
         NQ_REQUIRE(n[i] >= 1, NQ_ERR_SHAPE, "nq_w4a4_gemv_grouped: N must be positive");
@@ -366,6 +503,7 @@ extern "C" int nq_w4a4_gemv_grouped(const void *act_decoded_dev, int count, cons
     const uint4 *act = reinterpret_cast<const uint4 *>(act_decoded_dev);
     const int out_is_f32 = out_dtype == NQ_F32;
     hipStream_t s = (hipStream_t)stream;
+    if (mfma) return launch_mfma_gemv(act_decoded_dev, w, groups, m, k, out_is_f32, s);
 #define NQ_LAUNCH_GROUPED(MT)                                                                        \
     do {                                                                                             \
         if (rows_per_wg == 4)                                                                        \

@@ -446,14 +446,15 @@ def _gemv(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *, spl
 
 def linear_packed_w4a4_gemv_grouped(activation: PreparedNQA4Activation, weights: Sequence[PreparedNQRTLinear], *,
                                     output_dtype: torch.dtype | None = None) -> list[torch.Tensor]:
-    """One launch for up to four projections of the same M <= 8 activation (q/k/v, gate/up)."""
+    """One launch for up to four projections of the same activation of at most 8 rows (16 when K
+    is a multiple of 128): q/k/v, gate/up."""
     import ctypes
     if not 1 <= len(weights) <= 4:
         raise ValueError("between one and four weights per grouped launch")
     if activation.decoded is None or any(w.resolved_words is None for w in weights):
         raise ValueError("the grouped GEMV takes a decoded activation and resolved weights")
     m, k = activation.token_count, activation.feature_count
-    if not 1 <= m <= 8 or any(w.record.feature_count != k for w in weights):
+    if not 1 <= m <= (MATRIX_CORE_GEMV_ROWS if k % 128 == 0 else 8) or any(w.record.feature_count != k for w in weights):
         raise ValueError("activation or packed weights are unsupported by the grouped W4A4 GEMV")
     dtype = output_dtype or _kernel_dtype(activation)
     device = activation.decoded.device
@@ -548,6 +549,9 @@ def linear_packed_w4a4_mma_small_m_splitk_probe(activation: PreparedNQA4Activati
 # activation once per 32 channels, which is what it waits for beyond a few hundred rows;
 # measured crossover on MI355X at the 1B shapes: between 256 and 384 rows.
 LIBRARY_GEMM_ROWS = 288
+# up to this many rows a linear over resolved weights (K a multiple of 128) takes the decode GEMV,
+# which from five rows on multiplies on the matrix cores
+MATRIX_CORE_GEMV_ROWS = 16
 
 
 def decode_weight_bf16(weight: PreparedNQRTLinear) -> torch.Tensor:
@@ -575,6 +579,10 @@ def _gemm(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *,
             rows = decode_packed_a4(activation, output_dtype=torch.bfloat16).reshape(-1, activation.feature_count)
         out = torch.matmul(rows, decode_weight_bf16(weight).t())
         return out.reshape(*activation.original_shape[:-1], out.shape[-1])
+    if (split_k == 0 and activation.token_count <= MATRIX_CORE_GEMV_ROWS and weight.resolved_words is not None
+            and activation.feature_count % 128 == 0):
+        # up to sixteen rows the decode-in-register kernel feeds the matrix cores directly
+        return _gemv(activation, weight, split_k=0, output_dtype=dtype)
     return _gemv(activation, weight, split_k=split_k, output_dtype=dtype, kernel="gemm")
 
 

@@ -118,6 +118,37 @@ def test_grouped_gemv_equals_single_launches(rt, oracle, m):
         rt.linear_packed_w4a4_gemv_grouped(activation, weights * 2)
 
 
+@pytest.mark.parametrize("m", [5, 8, 11, 16])
+def test_grouped_gemv_on_the_matrix_cores(rt, oracle, m):
+    """From five rows on, weights that together fill the chip in tiles of 16 channels (here
+    3568 channels, one tile ragged) multiply on the matrix cores; above eight rows every
+    weight does.  Same decoded operands as the vector-unit kernel, another summation order."""
+    from test_gpu_gemv import _record, _references, TOLERANCE, BF16_TOLERANCE
+    from gpu_util import student_t_rows
+    k = 2048
+    weights, streams = [], []
+    for index, n_out in enumerate((2048, 520, 1000)):
+        seed = 20261201 + index
+        _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=700 + index, dither_seed=seed)
+        weights.append(rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda"))
+        streams.append((wc, wb, wn, seed))
+    x = torch.from_numpy(oracle.hadamard(student_t_rows(m, k, seed=41 + m).numpy())).to(torch.bfloat16).cuda()
+    activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS)
+    grouped = rt.linear_packed_w4a4_gemv_grouped(activation, weights, output_dtype=torch.float32)
+    again = rt.linear_packed_w4a4_gemv_grouped(activation, weights, output_dtype=torch.float32)
+    for out, twin, weight, (wc, wb, wn, seed) in zip(grouped, again, weights, streams):
+        assert torch.equal(out, twin)                                            # deterministic
+        ref32, ref16 = _references(oracle, activation, rt, wc, wb, wn, seed)
+        assert relative_error(bits(out), ref32) <= TOLERANCE
+        assert relative_error(bits(out), ref16) <= BF16_TOLERANCE
+        single = rt._gemv(activation, weight, split_k=0, output_dtype=torch.float32)
+        assert relative_error(bits(single), bits(out)) < 1e-5
+        if m > 8:
+            assert torch.equal(single, out)                                      # the same kernel either way
+    half = rt.linear_packed_w4a4_gemv_grouped(activation, weights[:1], output_dtype=torch.bfloat16)[0]
+    assert relative_error(bits(half.float()), bits(grouped[0])) < 1e-2
+
+
 def _rope_tables(rows, tokens, dim, seed):
     g = torch.Generator().manual_seed(seed)
     angle = 6.0 * torch.rand(rows, tokens, dim // 2, generator=g)

@@ -96,9 +96,12 @@ def test_slice_and_pad_matches_reference_chunking(rt, oracle):
     weight = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
     activation = _activation(rt, oracle, 40, k, seed=9)
     whole = rt._gemm(activation, weight, output_dtype=torch.float32)
-    chunk = rt.slice_pad_packed_activation_rows(activation, 32, 8, 16)
+    chunk = rt.slice_pad_packed_activation_rows(activation, 32, 8, 32)
     part = rt._gemm(chunk, weight, output_dtype=torch.float32)
     assert torch.equal(part[:8], whole[32:40]) and not part[8:].any()
+    # a 16-row chunk takes the decode-in-register kernel: same products, another summation order
+    small = rt._gemm(rt.slice_pad_packed_activation_rows(activation, 32, 8, 16), weight, output_dtype=torch.float32)
+    assert relative_error(bits(small[:8]), bits(whole[32:40])) < 1e-5 and not small[8:].any()
     packed_only = dataclasses.replace(chunk, decoded=None)
     assert torch.equal(rt._gemm(packed_only, weight, output_dtype=torch.float32), part)
 

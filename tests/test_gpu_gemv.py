@@ -47,9 +47,12 @@ def _references(oracle, activation, rt, wc, wb, wn, seed):
     return oracle.matmul_nt(a_hat, w_hat), oracle.matmul_nt(oracle.bf16_round(a_hat), oracle.bf16_round(w_hat))
 
 
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8])
-@pytest.mark.parametrize("k,n_out", [(256, 64), (2048, 136), (4096, 40)])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 8, 9, 13, 16])
+@pytest.mark.parametrize("k,n_out", [(256, 64), (2048, 136), (4096, 40), (128, 16), (1024, 23)])
 def test_small_shapes_match_oracle(rt, oracle, m, k, n_out):
+    # from five rows on (K a multiple of 128) the products run on the matrix cores
+    if m > 8 and k % 128:
+        pytest.skip("more than eight rows need K to be a multiple of 128")
     seed = 20261101 + m
     _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=1000 + k + n_out, dither_seed=seed)
     weight = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
@@ -61,7 +64,7 @@ def test_small_shapes_match_oracle(rt, oracle, m, k, n_out):
     assert relative_error(bits(y), ref16) <= BF16_TOLERANCE
     y16 = rt._gemv(activation, weight, split_k=0, output_dtype=torch.bfloat16)
     assert relative_error(bits(y16.float()), ref32) <= TOLERANCE
-    if k >= 512:
+    if k >= 512 and m <= 8:                                   # explicit K splits belong to the vector-unit kernel
         for split in (2, 4, 8):
             if (k // split) % 32:
                 continue
