@@ -311,21 +311,23 @@ extern "C" int nq_w4a4_resolve_weight(const uint8_t *w_codes_dev, const uint8_t 
 namespace {
 
 // The matrix-core kernel (resolved weights, K a multiple of 128, 16-byte aligned streams) works
-// in tiles of 16 channels: above eight rows it is the only decode kernel, from five rows on it
-// is taken when there are enough tiles for most of the chip (192: q/k/v or gate/up together).
-constexpr int kMfmaGemvMinRows = 5;
+// in tiles of 16 channels.  Above eight rows it is the only decode kernel; below, it is taken
+// when the weights of a launch give the chip enough tiles: 192 (q/k/v together) from five rows
+// on, where it saves the per-token vector work, and 512 (gate/up) for any row count, where it
+// also beats the vector-unit kernel's reductions (measured: 25.0 against 26.2 us at one row).
 constexpr int kMfmaGemvMaxRows = 16;
-constexpr int kMfmaGemvMinTiles = 192;
 
 bool takes_mfma_gemv(int m, int k, int64_t total_n, bool resolved) {
     if (!resolved || k % 128 != 0 || m > kMfmaGemvMaxRows) return false;
-    return m > 8 || (m >= kMfmaGemvMinRows && (total_n + 15) / 16 >= kMfmaGemvMinTiles);
+    const int64_t tiles = (total_n + 15) / 16;
+    return m > 8 || tiles >= 512 || (m >= 5 && tiles >= 192);
 }
 
 int launch_mfma_gemv(const void *act, const nq::GemvWeights &w, int groups, int m, int k, int out_is_f32,
                      hipStream_t stream) {
     const int super_steps = k / 128;
-    int waves = super_steps < nq::kMfmaGemvMaxWaves ? super_steps : nq::kMfmaGemvMaxWaves;
+    // two or more super-steps per wavefront, so that the requests of the next one hide behind a decode
+    int waves = super_steps / 2 < nq::kMfmaGemvMaxWaves ? super_steps / 2 : nq::kMfmaGemvMaxWaves;
     if (waves < 4) waves = 4;                    // the last stage wants 256 lanes
     hipLaunchKernelGGL(nq::w4a4_gemv_mfma_kernel, dim3((unsigned)groups), dim3(64 * waves), 0, stream,
                        reinterpret_cast<const uint4 *>(act), w, m, k, (float)sqrt((double)k), out_is_f32);
