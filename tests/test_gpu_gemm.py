@@ -78,7 +78,7 @@ def test_llama_1b_prefill_shapes(rt, oracle, name, k, n_out, wseed, dseed):
     norms = record.row_norms.numpy()
     dither = oracle.dither_stateless(n_out * k // 8, dseed).reshape(n_out, k // 8, 8)[rows]
     w_hat = oracle.dequantize_rows(codes[rows], beta[rows], norms[rows], WEIGHT_BETAS, Q, dither=dither)
-    for m in (16, 40, 64, 128, 384):
+    for m in (9, 16, 40, 64, 128, 384):                  # up to 16 rows gate_proj decodes in registers
         activation = _activation(rt, oracle, m, k, seed=3001)
         a_codes = oracle.unpack_unsigned(bits(activation.code_payload), m * k, 4)
         a_beta = oracle.unpack_unsigned(bits(activation.beta_payload), m * k // 8, 2)
