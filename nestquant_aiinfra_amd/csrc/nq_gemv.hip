@@ -187,24 +187,34 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int kMfmaGemvMaxWaves = 16;
 
+// R: K ranges per tile.  With R = 1 the 16 rows of the A operand are 16 channels.  Narrow
+// weights would then leave part of the chip without a tile, so with R = 2 the rows are 8
+// channels times two interleaved ranges of 128 k: a super-step spans 128 R k, a lane still decodes
+// four consecutive blocks of its (channel, range), and every decoded block goes through R
+// instructions, the r-th with the activation fragment of range r and with the rows of the other
+// ranges zeroed, so that row (range, channel) only ever meets its own k.  The rows of a channel
+// are added at the end.
+template <int R>
 __global__ void __launch_bounds__(kMfmaGemvMaxWaves * 64)
 w4a4_gemv_mfma_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, int k_size, float sqrt_k,
                       int out_is_f32) {
+    constexpr int kChannels = 16 / R;
     __shared__ float part[kMfmaGemvMaxWaves][256];
     int which = 0;
 #pragma unroll
     for (int i = 1; i < kGemvMaxGroup; i++)
         if (i < w.count && (int)blockIdx.x >= w.first_group[i]) which = i;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
-    const int n_size = w.n[which], n0 = ((int)blockIdx.x - w.first_group[which]) * 16;
+    const int n_size = w.n[which], n0 = ((int)blockIdx.x - w.first_group[which]) * kChannels;
     const int column = lane & 15, quarter = lane >> 4;
-    const int blocks_per_row = k_size >> 3, super_steps = k_size >> 7;
-    const int n = n0 + column < n_size ? n0 + column : n_size - 1;          // channels past the end repeat the last one
+    const int range = column / kChannels;                                   // of this lane's A rows
+    const int blocks_per_row = k_size >> 3, super_steps = k_size / (128 * R);
+    const int n = n0 + column % kChannels < n_size ? n0 + column % kChannels : n_size - 1;   // channels past the end repeat the last one
     const float wscale = (w.norms[which][n] / sqrt_k) * kResolvedUnit;
     const float *betas = w.betas[which];
     const float wbeta[4] = {betas[0], betas[1], betas[2], betas[3]};
     const uint32_t seed_plus_offset = w.seed_plus_offset[which];
-    const int64_t row_first = (int64_t)n * blocks_per_row + 4 * quarter;
+    const int64_t row_first = (int64_t)n * blocks_per_row + 16 * range + 4 * quarter;
     const uint32_t *words = w.words[which];
     const uint16_t *tails = w.tails[which];
     const bool has_token = column < m_rows;
@@ -212,33 +222,43 @@ w4a4_gemv_mfma_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, 
     const uint4 zero = make_uint4(0, 0, 0, 0);
 
     floatx4 acc = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-    uint4 word_next = zero, b_next[4] = {zero, zero, zero, zero};
+    uint4 word_next = zero, b_next[R][4];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int t = 0; t < 4; t++) b_next[r][t] = zero;
     uint2 tail_next = make_uint2(0, 0);
     if (wave < super_steps) {
-        word_next = *reinterpret_cast<const uint4 *>(words + row_first + 16 * wave);
-        tail_next = *reinterpret_cast<const uint2 *>(tails + row_first + 16 * wave);
+        word_next = *reinterpret_cast<const uint4 *>(words + row_first + 16 * R * wave);
+        tail_next = *reinterpret_cast<const uint2 *>(tails + row_first + 16 * R * wave);
         if (has_token) {
 #pragma unroll
-            for (int t = 0; t < 4; t++) b_next[t] = act_row[16 * wave + t];
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int t = 0; t < 4; t++) b_next[r][t] = act_row[16 * (R * wave + r) + t];
         }
     }
     for (int ss = wave; ss < super_steps; ss += waves) {
         const uint4 word4 = word_next;
         const uint2 tail2 = tail_next;
-        uint4 b[4];
+        uint4 b[R][4];
 #pragma unroll
-        for (int t = 0; t < 4; t++) b[t] = b_next[t];
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) b[r][t] = b_next[r][t];
         if (ss + waves < super_steps) {
-            word_next = *reinterpret_cast<const uint4 *>(words + row_first + 16 * (ss + waves));
-            tail_next = *reinterpret_cast<const uint2 *>(tails + row_first + 16 * (ss + waves));
+            word_next = *reinterpret_cast<const uint4 *>(words + row_first + 16 * R * (ss + waves));
+            tail_next = *reinterpret_cast<const uint2 *>(tails + row_first + 16 * R * (ss + waves));
             if (has_token) {
 #pragma unroll
-                for (int t = 0; t < 4; t++) b_next[t] = act_row[16 * (ss + waves) + t];
+                for (int r = 0; r < R; r++)
+#pragma unroll
+                    for (int t = 0; t < 4; t++) b_next[r][t] = act_row[16 * (R * (ss + waves) + r) + t];
             }
         }
         const uint32_t word[4] = {word4.x, word4.y, word4.z, word4.w};
         const uint32_t tail[4] = {tail2.x & 0xffffu, tail2.x >> 16, tail2.y & 0xffffu, tail2.y >> 16};
-        const int64_t g = row_first + 16 * ss;
+        const int64_t g = row_first + 16 * R * ss;
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             float v[8];
@@ -248,19 +268,25 @@ w4a4_gemv_mfma_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, 
             const bf16x2 h2 = pack_bf16x2(v[4] * scale, v[5] * scale), h3 = pack_bf16x2(v[6] * scale, v[7] * scale);
             const uint4 a = make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
                                        __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b[t]),
-                                                          acc, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const uint4 rows = (R == 1 || range == r) ? a : zero;
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rows),
+                                                              __builtin_bit_cast(bf16x8, b[r][t]), acc, 0, 0, 0);
+            }
         }
     }
-    // accumulator r of lane l: channel 4 (l / 16) + r, token l % 16
+    // accumulator i of lane l: A row 4 (l / 16) + i = (range, channel), token l % 16
 #pragma unroll
-    for (int r = 0; r < 4; r++) part[wave][(4 * quarter + r) * 16 + column] = acc[r];
+    for (int i = 0; i < 4; i++) part[wave][(4 * quarter + i) * 16 + column] = acc[i];
     __syncthreads();
-    if (tid < 256) {
+    if (tid < kChannels * 16) {
         const int channel = tid >> 4, token = tid & 15;
         if (n0 + channel < n_size && token < m_rows) {
-            float total = part[0][tid];
-            for (int i = 1; i < waves; i++) total = total + part[i][tid];
+            float total = 0.0f;
+            for (int p = 0; p < waves; p++)
+#pragma unroll
+                for (int r = 0; r < R; r++) total = total + part[p][(r * kChannels + channel) * 16 + token];
             const int64_t at = (int64_t)token * n_size + n0 + channel;
             if (out_is_f32) reinterpret_cast<float *>(w.out[which])[at] = total;
             else reinterpret_cast<uint16_t *>(w.out[which])[at] = f32_to_bf16(total);
@@ -310,27 +336,34 @@ extern "C" int nq_w4a4_resolve_weight(const uint8_t *w_codes_dev, const uint8_t 
 
 namespace {
 
-// The matrix-core kernel (resolved weights, K a multiple of 128, 16-byte aligned streams) works
-// in tiles of 16 channels.  Above eight rows it is the only decode kernel; below, it is taken
-// when the weights of a launch give the chip enough tiles: 192 (q/k/v together) from five rows
-// on, where it saves the per-token vector work, and 512 (gate/up) for any row count, where it
-// also beats the vector-unit kernel's reductions (measured: 25.0 against 26.2 us at one row).
+// The matrix-core kernel (resolved weights, 16-byte aligned streams) works in tiles of 16 / R
+// channels: R = 2 interleaved K ranges (K a multiple of 256) when 16-channel tiles would number
+// fewer than 192, else R = 1.  (R = 4 was measured at more than twice the time of R = 2.)  Above eight rows it is the only decode kernel; below, it is taken
+// from five rows on, where it saves the per-token vector work, and for any row count when even
+// R = 1 gives 512 tiles (gate/up), where it also beats the vector-unit kernel's reductions
+// (measured: 25.0 against 26.2 us at one row).
 constexpr int kMfmaGemvMaxRows = 16;
+
+int mfma_gemv_ranges(int k, int64_t total_n) {
+    return (total_n < 16 * 192 && k % 256 == 0) ? 2 : 1;
+}
 
 bool takes_mfma_gemv(int m, int k, int64_t total_n, bool resolved) {
     if (!resolved || k % 128 != 0 || m > kMfmaGemvMaxRows) return false;
-    const int64_t tiles = (total_n + 15) / 16;
-    return m > 8 || tiles >= 512 || (m >= 5 && tiles >= 192);
+    return m > 8 || m >= 5 || total_n >= 16 * 512;
 }
 
-int launch_mfma_gemv(const void *act, const nq::GemvWeights &w, int groups, int m, int k, int out_is_f32,
-                     hipStream_t stream) {
-    const int super_steps = k / 128;
+int launch_mfma_gemv(const void *act, const nq::GemvWeights &w, int ranges, int groups, int m, int k,
+                     int out_is_f32, hipStream_t stream) {
+    const int super_steps = k / (128 * ranges);
     // two or more super-steps per wavefront, so that the requests of the next one hide behind a decode
     int waves = super_steps / 2 < nq::kMfmaGemvMaxWaves ? super_steps / 2 : nq::kMfmaGemvMaxWaves;
     if (waves < 4) waves = 4;                    // the last stage wants 256 lanes
-    hipLaunchKernelGGL(nq::w4a4_gemv_mfma_kernel, dim3((unsigned)groups), dim3(64 * waves), 0, stream,
-                       reinterpret_cast<const uint4 *>(act), w, m, k, (float)sqrt((double)k), out_is_f32);
+    const uint4 *a = reinterpret_cast<const uint4 *>(act);
+    const float sqrt_k = (float)sqrt((double)k);
+    const dim3 grid((unsigned)groups), block(64 * waves);
+    if (ranges == 1) hipLaunchKernelGGL(nq::w4a4_gemv_mfma_kernel<1>, grid, block, 0, stream, a, w, m, k, sqrt_k, out_is_f32);
+    else hipLaunchKernelGGL(nq::w4a4_gemv_mfma_kernel<2>, grid, block, 0, stream, a, w, m, k, sqrt_k, out_is_f32);
     return nq::check_launch("nq_w4a4_gemv (matrix cores)");
 }
 
@@ -421,7 +454,8 @@ extern "C" int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_bet
         one.n[0] = n;
         one.first_group[0] = 0;
         one.seed_plus_offset[0] = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
-        return launch_mfma_gemv(act, one, (n + 15) / 16, m, k, out_dtype == NQ_F32, s);
+        const int ranges = mfma_gemv_ranges(k, n), channels = 16 / ranges;
+        return launch_mfma_gemv(act, one, ranges, (n + channels - 1) / channels, m, k, out_dtype == NQ_F32, s);
     }
 
     const int k_slice = k / split;
@@ -479,7 +513,8 @@ extern "C" int nq_w4a4_gemv_grouped(const void *act_decoded_dev, int count, cons
                    weight_seeds && out_dev, NQ_ERR_ARGUMENT, "nq_w4a4_gemv_grouped: null argument array");
     nq::GemvWeights w{};
     w.count = count;
-    const int rows_per_wg = mfma ? 16 : (total_n >= 8192 ? 4 : 2);
+    const int ranges = mfma ? mfma_gemv_ranges(k, total_n) : 1;
+    const int rows_per_wg = mfma ? 16 / ranges : (total_n >= 8192 ? 4 : 2);
     int groups = 0;
     for (int i = 0; i < count; i++) {
         NQ_REQUIRE(n[i] >= 1, NQ_ERR_SHAPE, "nq_w4a4_gemv_grouped: N must be positive");
@@ -505,7 +540,7 @@ extern "C" int nq_w4a4_gemv_grouped(const void *act_decoded_dev, int count, cons
     const uint4 *act = reinterpret_cast<const uint4 *>(act_decoded_dev);
     const int out_is_f32 = out_dtype == NQ_F32;
     hipStream_t s = (hipStream_t)stream;
-    if (mfma) return launch_mfma_gemv(act_decoded_dev, w, groups, m, k, out_is_f32, s);
+    if (mfma) return launch_mfma_gemv(act_decoded_dev, w, ranges, groups, m, k, out_is_f32, s);
 #define NQ_LAUNCH_GROUPED(MT)                                                                        \
     do {                                                                                             \
         if (rows_per_wg == 4)                                                                        \

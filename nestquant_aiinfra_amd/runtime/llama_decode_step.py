@@ -32,7 +32,7 @@ import torch
 import torch.nn.functional as F
 
 from .nqkv import launch_nqkv_decode_attention, nqkv_prefill_attention
-from .w4a4_linear import (MATRIX_CORE_GEMV_CHANNELS, MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, _gemm, _gemv, fused_input_stage,
+from .w4a4_linear import (MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, _gemm, _gemv, fused_input_stage,
                           linear_packed_w4a4_gemv_grouped, quantize_activation_cuda, rope_hadamard_cuda)
 
 
@@ -93,14 +93,12 @@ class FusedLlamaDecodeStep:
         return MATRIX_CORE_GEMV_ROWS if activation.feature_count % 128 == 0 else 8
 
     def _linear(self, activation, prepared: PreparedNQRTLinear) -> torch.Tensor:
-        if activation.token_count <= 8:
+        if activation.token_count <= self._gemv_rows(activation):
             return _gemv(activation, prepared, split_k=0, output_dtype=torch.bfloat16)
-        return _gemm(activation, prepared, output_dtype=torch.bfloat16)     # picks the kernel by rows and channels
+        return _gemm(activation, prepared, output_dtype=torch.bfloat16)
 
     def _linears(self, activation, prepared: list[PreparedNQRTLinear]) -> list[torch.Tensor]:
-        channels = sum(weight.record.indices.shape[0] for weight in prepared)
-        if activation.token_count <= 8 or (activation.token_count <= self._gemv_rows(activation)
-                                           and channels >= MATRIX_CORE_GEMV_CHANNELS):
+        if activation.token_count <= self._gemv_rows(activation):
             return linear_packed_w4a4_gemv_grouped(activation, prepared, output_dtype=torch.bfloat16)
         return [self._linear(activation, weight) for weight in prepared]
 

@@ -552,9 +552,6 @@ LIBRARY_GEMM_ROWS = 288
 # up to this many rows a linear over resolved weights (K a multiple of 128) takes the decode GEMV,
 # which from five rows on multiplies on the matrix cores
 MATRIX_CORE_GEMV_ROWS = 16
-# ... when the weight has enough channels to give most of the chip a 16-channel tile (measured at 9 to
-# 16 rows: 16.2 against 20.2 us for 8192 channels, 26.0 against 23.4 us for 2048)
-MATRIX_CORE_GEMV_CHANNELS = 3072
 
 
 def decode_weight_bf16(weight: PreparedNQRTLinear) -> torch.Tensor:
@@ -583,7 +580,7 @@ def _gemm(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *,
         out = torch.matmul(rows, decode_weight_bf16(weight).t())
         return out.reshape(*activation.original_shape[:-1], out.shape[-1])
     if (split_k == 0 and activation.token_count <= MATRIX_CORE_GEMV_ROWS and weight.resolved_words is not None
-            and activation.feature_count % 128 == 0 and weight.record.indices.shape[0] >= MATRIX_CORE_GEMV_CHANNELS):
+            and activation.feature_count % 128 == 0):
         # up to sixteen rows the decode-in-register kernel feeds the matrix cores directly
         return _gemv(activation, weight, split_k=0, output_dtype=dtype)
     return _gemv(activation, weight, split_k=split_k, output_dtype=dtype, kernel="gemm")
