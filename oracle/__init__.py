@@ -237,6 +237,14 @@ def count_div14_mismatches() -> int:
     return int(fn())
 
 
+def count_reciprocal_division_mismatches(divisor: float) -> int:
+    """Exhaustive float32 check (2^-61 <= |a| < 2^40) of the many-row encoder's division through the reciprocal."""
+    fn = lib().nqo_count_reciprocal_division_mismatches
+    fn.restype = ctypes.c_longlong
+    fn.argtypes = [ctypes.c_float]
+    return int(fn(ctypes.c_float(divisor)))
+
+
 def num_threads() -> int:
     return int(lib().nqo_num_threads())
 

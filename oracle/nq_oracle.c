@@ -436,6 +436,37 @@ NQO_EXPORT long long nqo_count_div14_mismatches(void) {
     return bad;
 }
 
+/* The many-row encoder divides by a beta through its correctly rounded reciprocal:
+ *   q0 = a * r;  q1 = fma(fma(-b, q0, a), r, q0);  q2 = fma(fma(-b, q1, a), r, q1),  r = 1 / b
+ * Compared with the IEEE quotient a / b for every float32 a with 2^-61 <= |a| < 2^40 (the
+ * kernel takes the IEEE division below that magnitude) and for a = 0.  Returns the number of
+ * inputs whose results differ as numbers. */
+NQO_EXPORT long long nqo_count_reciprocal_division_mismatches(float b) {
+    volatile float one = 1.0f;
+    const float r = one / b;
+    long long bad = 0;
+#pragma omp parallel for reduction(+ : bad) schedule(static)
+    for (long long e = 66; e < 168; e++) {
+        for (uint32_t m = 0; m < (1u << 23); m++) {
+            for (int sign = 0; sign < 2; sign++) {
+                uint32_t bits = ((uint32_t)sign << 31) | ((uint32_t)e << 23) | m;
+                float a;
+                memcpy(&a, &bits, 4);
+                float q = a * r;
+                q = fmaf(fmaf(-b, q, a), r, q);
+                q = fmaf(fmaf(-b, q, a), r, q);
+                if (q != a / b) bad++;
+            }
+        }
+    }
+    const float zero = 0.0f;
+    float q = zero * r;
+    q = fmaf(fmaf(-b, q, zero), r, q);
+    q = fmaf(fmaf(-b, q, zero), r, q);
+    if (q != 0.0f) bad++;
+    return bad;
+}
+
 NQO_EXPORT int nqo_num_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

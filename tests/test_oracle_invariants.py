@@ -221,3 +221,14 @@ def test_three_operation_division_by_14_is_ieee_exact(oracle):
     """The HIP kernels divide by 14 with q0 = p*c, r = fma(-14, q0, p), q = fma(r, c, q0);
     checked against IEEE division for every finite float32 in [1e-30, 1e30]."""
     assert oracle.count_div14_mismatches() == 0
+
+
+def test_division_through_the_reciprocal_is_ieee_exact(oracle):
+    """The many-row encoder forms y / beta as two exact-remainder corrections of y * (1 / beta);
+    checked against IEEE division over every float32 of the range the kernel uses it on, for
+    the activation, key and value betas and a few awkward divisors."""
+    import numpy as np
+    betas = [v / 14 for v in (3.47, 4.74, 6.90, 18.11, 3.50, 4.58, 6.47, 17.06, 3.53, 5.59, 9.62, 29.03)]
+    betas += [1.0 / 3.0, 0.7, 1.9999999, 1.0000001, 3.1415927]
+    for beta in betas:
+        assert oracle.count_reciprocal_division_mismatches(float(np.float32(beta))) == 0, beta
