@@ -19,7 +19,7 @@
 // beyond the table width (the reference stops at 64 pages, nqkv_attention_k1.py:696-698).
 // Decoded K/V stay FP32 (as in the reference's fused kernel); K/V decode follows the exact
 // float32 order of nq_e8.hip.h because undithered codes sit on exact Voronoi ties.
-#include "nq_e8.hip.h"
+#include "nq_rowquant.hip.h"
 #include "nq_host.h"
 
 #include <math.h>
@@ -145,48 +145,63 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     // scaled by 1 / sqrt(D), rounded to the query dtype: hadamard(query.float()).to(dtype),
     // nestquant/runtime/nqkv_batched_hf_backend.py:549)
     static_assert(sizeof(acc_lds) >= sizeof(float) * G * D, "the query staging fits the accumulator buffer");
+    static_assert(D == 64 && G * 8 <= 64, "eight lanes of the first wavefront prepare one head's query");
     float *q_lds = &acc_lds[0][0][0];                    // free until the V pass ends
-    for (int i = tid; i < G * D; i += kAttnThreads)
-        q_lds[i] = load_query(a.query, a.query_dtype, ((int64_t)row * a.q_heads + g * G) * D + i);
-    __syncthreads();
-    if (a.rope_cos) {
-        // (q * cos) + (rotate_half(q) * sin) in BF16 tensor arithmetic, before the rotation
-        for (int i = tid; i < G * (D / 2); i += kAttnThreads) {
-            const int h = i / (D / 2), k = i % (D / 2);
-            const int64_t at = (int64_t)row * D;
-            const float c_lo = bf16_to_f32(a.rope_cos[at + k]), c_hi = bf16_to_f32(a.rope_cos[at + k + D / 2]);
-            const float s_lo = bf16_to_f32(a.rope_sin[at + k]), s_hi = bf16_to_f32(a.rope_sin[at + k + D / 2]);
-            const float x1 = q_lds[h * D + k], x2 = q_lds[h * D + k + D / 2];
-            q_lds[h * D + k] = bf16_to_f32(f32_to_bf16(bf16_to_f32(f32_to_bf16(x1 * c_lo)) - bf16_to_f32(f32_to_bf16(x2 * s_lo))));
-            q_lds[h * D + k + D / 2] = bf16_to_f32(f32_to_bf16(bf16_to_f32(f32_to_bf16(x2 * c_hi)) + bf16_to_f32(f32_to_bf16(x1 * s_hi))));
-        }
-        __syncthreads();
-    }
-    if (a.rotate_query) {
-        for (int width = 1; width < D; width <<= 1) {
-            for (int i = tid; i < G * (D / 2); i += kAttnThreads) {
-                const int h = i / (D / 2), k = i % (D / 2);
-                const int x = h * D + (k / width) * 2 * width + (k % width), y = x + width;
-                const float left = q_lds[x], right = q_lds[y];
-                q_lds[x] = left + right;
-                q_lds[y] = left - right;
+    if (tid < G * 8) {
+        // lane 8 h + part holds elements 8 part .. 8 part + 7 of head h: the embedding pairs it with
+        // the lane four further on, the rotation runs in registers and between the eight lanes
+        const int h = tid >> 3, part = tid & 7;
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            v[j] = load_query(a.query, a.query_dtype, ((int64_t)row * a.q_heads + g * G + h) * D + part * 8 + j);
+        if (a.rope_cos) {
+            // (q * cos) + (rotate_half(q) * sin) in BF16 tensor arithmetic, before the rotation
+            const int64_t at = (int64_t)row * D + part * 8;
+            const bool upper = part >= 4;
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) {
+                const float o0 = lane_xor<4>(v[j]), o1 = lane_xor<4>(v[j + 1]);
+                float a0 = v[j] * bf16_to_f32(a.rope_cos[at + j]), a1 = v[j + 1] * bf16_to_f32(a.rope_cos[at + j + 1]);
+                round_pair<1>(a0, a1);
+                float b0 = o0 * bf16_to_f32(a.rope_sin[at + j]), b1 = o1 * bf16_to_f32(a.rope_sin[at + j + 1]);
+                round_pair<1>(b0, b1);
+                v[j] = upper ? a0 + b0 : a0 - b0;
+                v[j + 1] = upper ? a1 + b1 : a1 - b1;
+                round_pair<1>(v[j], v[j + 1]);
             }
-            __syncthreads();
         }
+        if (a.rotate_query) {
+#pragma unroll
+            for (int s = 0; s < 3; s++) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    if (j & (1 << s)) continue;
+                    const float left = v[j], right = v[j + (1 << s)];
+                    v[j] = left + right;
+                    v[j + (1 << s)] = left - right;
+                }
+            }
+            lane_stage<1, 0>(v, tid);
+            lane_stage<2, 0>(v, tid);
+            lane_stage<4, 0>(v, tid);
+            const float inv = 1.0f / __builtin_sqrtf((float)D);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float scaled = v[j] * inv;
+                v[j] = a.query_dtype == NQ_BF16 ? bf16_to_f32(f32_to_bf16(scaled))
+                                                : (a.query_dtype == NQ_F16 ? (float)(_Float16)scaled : scaled);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) q_lds[h * D + part * 8 + j] = v[j];
     }
+    __syncthreads();
     float q[G][8];
 #pragma unroll
     for (int h = 0; h < G; h++)
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            float v = q_lds[h * D + blk * 8 + j];
-            if (a.rotate_query) {
-                v = v * (1.0f / __builtin_sqrtf((float)D));
-                v = a.query_dtype == NQ_BF16 ? bf16_to_f32(f32_to_bf16(v))
-                                             : (a.query_dtype == NQ_F16 ? (float)(_Float16)v : v);
-            }
-            q[h][j] = v;
-        }
+        for (int j = 0; j < 8; j++) q[h][j] = q_lds[h * D + blk * 8 + j];
     __syncthreads();
     const float sqrt_d = __builtin_sqrtf((float)D);
 
