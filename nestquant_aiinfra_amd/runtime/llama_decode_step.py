@@ -81,6 +81,27 @@ class FusedLlamaDecodeStep:
         hidden = inner.embed_tokens.weight.shape[1]
         _require(hidden & (hidden - 1) == 0 and hidden % 32 == 0, "hidden size is not a power of two")
         self.hidden = hidden
+        self._rope_tables: tuple[torch.Tensor, torch.Tensor] | None = None
+
+    def _rope(self, embedded: torch.Tensor, positions: torch.Tensor, *, padded: bool = False
+              ) -> tuple[torch.Tensor, torch.Tensor]:
+        """BF16 (cos, sin) [positions.numel(), head_dim] of the model's rotary embedding.  For
+        embeddings that depend on the position alone the module is evaluated once, over every
+        position the cache can hold, and a step gathers its rows (two launches instead of the
+        module's dozen)."""
+        rotary = self.inner.rotary_emb
+        if getattr(rotary, "rope_type", "default") not in ("default", "llama3", "linear"):
+            cos, sin = rotary(embedded, positions)
+            dim = cos.shape[-1]
+            return cos.to(torch.bfloat16).reshape(-1, dim).contiguous(), sin.to(torch.bfloat16).reshape(-1, dim).contiguous()
+        if self._rope_tables is None:
+            every = torch.arange(self.cache.max_cache_len, device=embedded.device)[None, :]
+            cos, sin = rotary(embedded[:1, :1], every)
+            self._rope_tables = (cos[0].to(torch.bfloat16).contiguous(), sin[0].to(torch.bfloat16).contiguous())
+        index = positions.reshape(-1)
+        if padded:                      # positions of padding tokens may lie past the cache's last one
+            index = index.clamp(max=self._rope_tables[0].shape[0] - 1)
+        return self._rope_tables[0].index_select(0, index), self._rope_tables[1].index_select(0, index)
 
     @staticmethod
     def _prepared(linear, device) -> PreparedNQRTLinear:
@@ -113,9 +134,8 @@ class FusedLlamaDecodeStep:
         embedded = inner.embed_tokens(tokens)                               # [rows, 1, hidden]
         if embedded.dtype != torch.bfloat16:
             raise TypeError("the fused decode step runs BF16 models")
-        cos, sin = inner.rotary_emb(embedded, positions)                    # [rows, 1, head_dim]
-        cos, sin = cos.to(torch.bfloat16).contiguous(), sin.to(torch.bfloat16).contiguous()
-        query_rope = (cos.view(rows, -1), sin.view(rows, -1))
+        query_rope = self._rope(embedded, positions)                        # 2 x [rows, head_dim]
+        cos, sin = query_rope[0].view(rows, 1, -1), query_rope[1].view(rows, 1, -1)
         heads, kv_heads, dim = cache.num_query_heads, cache.num_kv_heads, cache.head_dim
         workspace = cache._workspace(rows, torch.bfloat16)
 
@@ -164,9 +184,8 @@ class FusedLlamaPrefillStep(FusedLlamaDecodeStep):
         if embedded.dtype != torch.bfloat16:
             raise TypeError("the fused prefill step runs BF16 models")
         count = rows * width
-        cos, sin = inner.rotary_emb(embedded, positions)                    # [rows, width, head_dim]
         heads, kv_heads, dim = cache.num_query_heads, cache.num_kv_heads, cache.head_dim
-        rope = (cos.to(torch.bfloat16).reshape(count, dim).contiguous(), sin.to(torch.bfloat16).reshape(count, dim).contiguous())
+        rope = self._rope(embedded, positions, padded=True)                 # 2 x [rows * width, head_dim]
         over_cache = cache.packed_prefill or cache._continuation
 
         delta, residual = embedded.reshape(count, self.hidden), None
