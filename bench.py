@@ -47,8 +47,11 @@ def linear_bytes(m: int, k: int, n: int) -> int:
 # HBM bytes per launch of the linear kernel (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by
 # what the same counters read for a 256 MiB copy; runs and factors in
 # profiles/w4a4_gemv_decode_rocprofv3.md).  Counters cannot be read from inside this process.
-MEASURED_TRAFFIC_BYTES = {"q_proj_m1": 3_416_000, "q_proj_m8": 3_894_000, "down_proj_m1": 12_950_000,
-                          "down_proj_m8": 14_116_000}
+MEASURED_TRAFFIC_BYTES = {"q_proj_m1": 3_417_000, "q_proj_m8": 3_634_000, "down_proj_m1": 12_951_000,
+                          "down_proj_m8": 13_856_000}
+# the kernel each case launches (one row: vector units; eight rows: matrix cores, two K ranges per tile)
+CASE_KERNEL = {"q_proj_m1": "w4a4_gemv_kernel<1, 2, true>", "down_proj_m1": "w4a4_gemv_kernel<1, 2, true>",
+               "q_proj_m8": "w4a4_gemv_mfma_kernel<2>", "down_proj_m8": "w4a4_gemv_mfma_kernel<2>"}
 
 
 def parse_args() -> argparse.Namespace:
@@ -446,7 +449,7 @@ def main() -> None:
         }
     dominant = max(per_case, key=lambda name: per_case[name]["us"])
     roofline = {
-        "bound": "hbm", "kernel": f"w4a4_gemv_kernel ({dominant})",
+        "bound": "hbm", "kernel": f"{CASE_KERNEL.get(dominant, 'w4a4_gemv_kernel')} ({dominant})",
         "achieved": per_case[dominant]["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": per_case[dominant]["GBps"] / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
         "launch_us": per_case[dominant]["us"], "algorithmic_bytes": per_case[dominant]["bytes"],
