@@ -1,8 +1,9 @@
-// Packed W4A4 linear for decode (M = 1..8 tokens): the NQRT4 weight stream is decoded in
+// Packed W4A4 linear for decode (M = 1..16 tokens): the NQRT4 weight stream is decoded in
 // registers; nothing but packed words, norms, the BF16 activation and the output touches
-// memory.
+// memory.  Two kernels share the decode: the vector-unit kernel described next (any weight
+// form, up to eight tokens), and a matrix-core kernel for resolved weights (further down).
 //
-// Layout of the work.  grid = (ceil(N / rows_per_wg), split_k); a workgroup of four
+// Layout of the work (vector-unit kernel).  grid = (ceil(N / rows_per_wg), split_k); a workgroup of four
 // wavefronts owns `rows_per_wg` output channels and one K slice, and its wavefronts
 // interleave over the slice: in every step lane l of wavefront w decodes block
 // 256 * step + 64 * w + l, so a wavefront reads 256 contiguous bytes of code words (one

@@ -222,7 +222,9 @@ __device__ __forceinline__ void staged_row_norms(const float *rows, int row_coun
                     for (int k = 0; k < 32; k++) acc = __builtin_fmaf(a[k], a[k], acc);
                     __builtin_amdgcn_sched_barrier(0);
                     const int after = batch + 2 < batches ? batch + 2 : batches - 1;
-                    next = row + 256 * after;
+                    // the address waits for the chain (adding zero unless the sum is NaN): the request
+                    // then reuses the registers the chain has just released, with no copies in the loop
+                    next = row + 256 * after + (acc != acc ? 1 : 0);
 #pragma unroll
                     for (int k = 0; k < 32; k++) a[k] = next[8 * k];
                     __builtin_amdgcn_sched_barrier(0);
