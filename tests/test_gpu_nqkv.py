@@ -175,6 +175,37 @@ def test_attention_small_contexts_and_groups(kv, oracle, q_heads):
     assert not out[3].any()
 
 
+@pytest.mark.parametrize("batch", [1, 2, 4, 8])
+def test_batched_attention_equals_rows_taken_alone(kv, oracle, batch):
+    """A row's result does not depend on the rows next to it, their order or the slot it sits in
+    (non-contiguous slots).  The reference asserts equality between its batched and
+    single-sequence kernels (tests/unit/runtime/test_nqkv_attention_batched_k1.py:116-143); here
+    the chunk a workgroup takes depends on the batch width, so the same row taken alone may sum
+    in another order: equal to within the rounding of the BF16 result."""
+    rng = np.random.default_rng(100 + batch)
+    manager = _manager(kv, capacity=8, max_len=1024)
+    slots = [6, 1, 7, 0, 3, 5, 2, 4][:batch]
+    lengths = [901, 17, 256, 3, 640, 33, 128, 1000][:batch]
+    keys = [_bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for n in lengths]
+    values = [_bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for n in lengths]
+    for s in slots:
+        manager.register(s, slot=s)
+    _append(manager, slots, keys, values)
+    query = _bf16(oracle.hadamard(rng.standard_normal((batch, 32, DIM)).astype(np.float32))).cuda()
+    slot_ids = torch.tensor(slots, dtype=torch.int32, device="cuda")
+    active = torch.ones(batch, dtype=torch.bool, device="cuda")
+    together = kv.nqkv_decode_attention_batched_k1(query, manager.layers[0], slot_ids=slot_ids, active_mask=active).clone()
+    for row in range(batch):
+        alone = kv.nqkv_decode_attention_batched_k1(query[row:row + 1], manager.layers[0], slot_ids=slot_ids[row:row + 1],
+                                                    active_mask=active[:1])
+        assert relative_error(_f32(alone[0]), _f32(together[row])) <= 2.0 ** -7, (batch, row)
+    # reversing the rows reverses the results, bit for bit (same batch width, same chunks)
+    order = list(range(batch))[::-1]
+    flipped = kv.nqkv_decode_attention_batched_k1(query[order].contiguous(), manager.layers[0],
+                                                  slot_ids=slot_ids[order].contiguous(), active_mask=active)
+    assert torch.equal(flipped, together[order])
+
+
 def test_attention_ragged_batch_at_full_size(kv, oracle):
     """Batch 8, 32 query / 8 KV heads, contexts uniform in [128, 4096] (up to 256 pages)."""
     g = torch.Generator().manual_seed(4001)
