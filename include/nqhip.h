@@ -317,7 +317,8 @@ int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_dtype, cons
  * online-softmax in two stages; rows that are not live or have no tokens give zeros.
  * query / out: [batch, q_heads, head_dim] of query_dtype; rotate_query != 0 applies the
  * normalized Hadamard transform over head_dim to the query first (float32, rounded to
- * query_dtype), matching keys stored with rotate_keys.  rope_cos_dev / rope_sin_dev (optional,
+ * query_dtype), matching keys stored with rotate_keys.  out_dev may be NULL: then only the first
+ * stage runs (see nq_attention_output_stage).  rope_cos_dev / rope_sin_dev (optional,
  * both or neither): BF16 [batch, head_dim] rotary tables applied to the (BF16) query before
  * that, as nq_nqkv_write applies them to keys.  Workspace: at least
  * nq_nqkv_attention_workspace_bytes() bytes.  Requires head_dim = 64, page_size = 16,
@@ -338,6 +339,25 @@ int nq_nqkv_attention_decode(
     size_t workspace_bytes, void *stream);
 
 size_t nq_nqkv_attention_workspace_bytes(int batch, int q_heads, int head_dim, int max_pages);
+
+/*
+ * The second stage of the decode attention done where its result is consumed.  With
+ * out_dev == NULL nq_nqkv_attention_decode leaves the per-chunk partial results (maxima, sums
+ * and numerators of nq_nqkv_attention_parts(batch, max_pages) chunks per head) in its workspace;
+ * this call merges them into the BF16 attention output [rows = batch, q_heads * head_dim]
+ * (staged_out_dev, optional) and, when codes_dev is given, rotates, norms, encodes and packs
+ * those rows as nq_quantize_rows does for the o_proj input.  Same stream, same batch, q_heads
+ * and max_pages as the attention call.  The merged rows equal nq_nqkv_attention_decode's BF16
+ * output but for the summation order of the softmax denominator (at most one BF16 step).
+ * Replaces: the stage-2 kernel of nqkv_decode_attention_batched_k1
+ * (nestquant/runtime/nqkv_attention_k1.py:400-471) together with the input stage of
+ * FusedNQRTLinear.forward (nestquant/models/fused_linear.py:287-306) of o_proj.
+ */
+int nq_nqkv_attention_parts(int batch, int max_pages);
+int nq_attention_output_stage(const void *workspace_dev, int64_t rows, int q_heads, int head_dim, int parts,
+                              void *staged_out_dev, int q, const float *betas_dev, int beta_count,
+                              int hadamard, uint8_t *codes_dev, uint8_t *beta_ids_dev, float *norms_dev,
+                              void *decoded_bf16_dev, void *stream);
 
 /*
  * Causal attention of a chunk of new tokens over the packed cache (prefill, chunked prefill,

@@ -414,6 +414,11 @@ int chunks_for(int batch, int max_pages) {
 
 }  // namespace
 
+extern "C" int nq_nqkv_attention_parts(int batch, int max_pages) {
+    if (batch < 1 || max_pages < 1) return 0;
+    return chunks_for(batch, max_pages) + 1;
+}
+
 extern "C" size_t nq_nqkv_attention_workspace_bytes(int batch, int q_heads, int head_dim, int max_pages) {
     if (batch < 1 || q_heads < 1 || head_dim < 1 || max_pages < 1) return 0;
     const size_t parts = (size_t)chunks_for(batch, max_pages) + 1;
@@ -444,7 +449,7 @@ extern "C" int nq_nqkv_attention_decode(
     NQ_REQUIRE(query_dev && key_codes_dev && key_beta_ids_dev && key_norms_dev && value_codes_dev &&
                    value_beta_ids_dev && value_norms_dev && key_betas_dev && value_betas_dev && page_indices_dev &&
                    page_counts_dev && last_page_lens_dev && hot_lengths_dev && hot_keys_dev && hot_values_dev &&
-                   slot_ids_dev && active_mask_dev && out_dev,
+                   slot_ids_dev && active_mask_dev,
                NQ_ERR_ARGUMENT, "nq_nqkv_attention_decode: null pointer");
     NQ_REQUIRE(nq::aligned(key_codes_dev, 4) && nq::aligned(value_codes_dev, 4) && nq::aligned(hot_keys_dev, 16) &&
                    nq::aligned(hot_values_dev, 16),
@@ -500,7 +505,8 @@ extern "C" int nq_nqkv_attention_decode(
     }
 #undef NQ_LAUNCH_STAGE1
     int status = nq::check_launch("nq_nqkv_attention_decode (stage 1)");
-    if (status != NQ_OK) return status;
+    // without an output the partial results stay in the workspace for nq_attention_output_stage
+    if (status != NQ_OK || out_dev == nullptr) return status;
     hipLaunchKernelGGL(nq::attention_merge_kernel<64>, dim3((unsigned)heads_total), dim3(64), 0, s,
                        a.part_max, a.part_sum, a.part_acc, (int)parts, (int64_t)heads_total, out_dev, query_dtype);
     return nq::check_launch("nq_nqkv_attention_decode (merge)");

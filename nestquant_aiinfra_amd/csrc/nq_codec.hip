@@ -75,11 +75,16 @@ template <> struct RowLoader<half_bits> {
 //   mode 1  h = x + residual (residual may be null); residual_out = h;
 //           y = weight * bf16(h * rsqrt(mean(h^2) + eps))      (LlamaRMSNorm)
 //   mode 2  y = bf16(silu(gate)) * x                            (the SwiGLU product)
+//   mode 3  y = the attention output [rows, heads * 64] merged from the per-chunk partial results
+//           of the decode attention (online-softmax maxima, sums and numerators of `parts` chunks
+//           per head), rounded to BF16: stage 2 of the attention, done where its result is consumed
 // normed_out (optional) receives y; rows are then rotated / quantised as usual.
 struct InputPrologue {
     const uint16_t *residual, *weight, *gate;
     uint16_t *residual_out, *normed_out;
     float eps;
+    const float *part_max, *part_sum, *part_acc;       // mode 3: [rows * heads][parts] (x 64 for part_acc)
+    int parts, heads;
 };
 
 
@@ -117,6 +122,74 @@ __device__ __forceinline__ void stage_with_prologue(const uint16_t *__restrict__
     const int tid = threadIdx.x;
     const int row_vectors = n >> 3, vectors = rows_per_wg * row_vectors;
     const uint4 zero = make_uint4(0, 0, 0, 0);
+    if (kPrologue == 3) {
+        // one lane per eight output dimensions of one head: out = sum_c acc_c w_c / sum_c sum_c w_c with
+        // w_c = exp(max_c - max).  Online over batches of eight chunks whose maxima, sums and numerators
+        // are all requested before the first is used (one memory latency per batch, not per chunk);
+        // chunks without tokens carry no numerator (their entry is read, never used) and weigh nothing.
+        constexpr int kBatch = 8;
+        const float kNone = -__builtin_inff();
+        for (int v = tid; v < vectors; v += blockDim.x) {
+            const int64_t g = first + (int64_t)v * 8;
+            float y[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) y[j] = 0.0f;
+            if (g < limit) {
+                const int64_t head = (g / n) * pro.heads + (g % n) / 64;
+                const float *m = pro.part_max + head * pro.parts, *sum = pro.part_sum + head * pro.parts;
+                const float *acc = pro.part_acc + head * pro.parts * 64 + (g % 64);
+                float top = kNone, denom = 0.0f;
+                for (int c0 = 0; c0 < pro.parts; c0 += kBatch) {
+                    float mc[kBatch], sc[kBatch];
+                    float4 lo[kBatch], hi[kBatch];
+#pragma unroll
+                    for (int j = 0; j < kBatch; j++) {
+                        const int c = min(c0 + j, pro.parts - 1);
+                        mc[j] = m[c];
+                        sc[j] = sum[c];
+                        lo[j] = *reinterpret_cast<const float4 *>(acc + (int64_t)c * 64);
+                        hi[j] = *reinterpret_cast<const float4 *>(acc + (int64_t)c * 64 + 4);
+                    }
+                    float batch_top = kNone;
+#pragma unroll
+                    for (int j = 0; j < kBatch; j++) {
+                        if (c0 + j >= pro.parts) sc[j] = 0.0f;
+                        batch_top = fmaxf(batch_top, mc[j]);
+                    }
+                    const float next_top = fmaxf(top, batch_top);
+                    if (next_top > kNone) {
+                        const float keep = top > kNone ? __expf(top - next_top) : 0.0f;
+                        denom = denom * keep;
+#pragma unroll
+                        for (int i = 0; i < 8; i++) y[i] = y[i] * keep;
+#pragma unroll
+                        for (int j = 0; j < kBatch; j++) {
+                            const float w = sc[j] > 0.0f ? __expf(mc[j] - next_top) : 0.0f;
+                            denom = denom + sc[j] * w;
+                            const bool used = w > 0.0f;
+                            y[0] += used ? lo[j].x * w : 0.0f; y[1] += used ? lo[j].y * w : 0.0f;
+                            y[2] += used ? lo[j].z * w : 0.0f; y[3] += used ? lo[j].w * w : 0.0f;
+                            y[4] += used ? hi[j].x * w : 0.0f; y[5] += used ? hi[j].y * w : 0.0f;
+                            y[6] += used ? hi[j].z * w : 0.0f; y[7] += used ? hi[j].w * w : 0.0f;
+                        }
+                        top = next_top;
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j += 2) {
+                    y[j] = denom > 0.0f ? y[j] / denom : 0.0f;               // inactive or empty rows give zeros
+                    y[j + 1] = denom > 0.0f ? y[j + 1] / denom : 0.0f;
+                    round_pair<1>(y[j], y[j + 1]);
+                }
+                if (writes_outputs && pro.normed_out)
+                    reinterpret_cast<uint4 *>(pro.normed_out)[g >> 3] = pack_bf16x8_exact(y);
+            }
+            *reinterpret_cast<float4 *>(staged + v * 8) = make_float4(y[0], y[1], y[2], y[3]);
+            *reinterpret_cast<float4 *>(staged + v * 8 + 4) = make_float4(y[4], y[5], y[6], y[7]);
+        }
+        __syncthreads();
+        return;
+    }
     for (int v = tid; v < vectors; v += blockDim.x) {
         const int64_t g = first + (int64_t)v * 8;
         const bool live = g < limit;
@@ -547,7 +620,7 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
                     uint32_t seed_plus_offset, uint8_t *codes, uint8_t *beta_ids, float *norms,
                     void *decoded, int hadamard_stage_dtype, hipStream_t stream,
                     nq::InputPrologue prologue = nq::InputPrologue{}) {
-    if (!kDithered && rows * (int64_t)n >= kBulkElements) {
+    if (!kDithered && kPrologue != 3 && rows * (int64_t)n >= kBulkElements) {
         int rows_per_wg = n >= 2048 ? 1 : 2048 / n;
         const size_t lds_bytes = ((size_t)rows_per_wg * n + 2 * rows_per_wg + (kPrologue == 1 ? n : 0)) * sizeof(float);
         auto kernel = nq::quantize_rows_bulk_kernel<T, kPrologue>;
@@ -703,6 +776,43 @@ extern "C" int nq_fused_input_stage(const void *x_dev, int64_t rows, int64_t n, 
     return launch_quantize<uint16_t, false, 2>(x_dev, rows, (int)n, encodes ? q : 14, betas_dev, beta_count, 0u,
                                                codes_dev, beta_ids_dev, norms_dev, decoded_bf16_dev, stage_dtype,
                                                s, prologue);
+}
+
+extern "C" int nq_attention_output_stage(const void *workspace_dev, int64_t rows, int q_heads, int head_dim,
+                                         int parts, void *staged_out_dev, int q, const float *betas_dev,
+                                         int beta_count, int hadamard, uint8_t *codes_dev, uint8_t *beta_ids_dev,
+                                         float *norms_dev, void *decoded_bf16_dev, void *stream) {
+    NQ_REQUIRE(rows >= 1 && q_heads >= 1 && parts >= 1 && parts <= 512, NQ_ERR_SHAPE,
+               "nq_attention_output_stage: rows, heads and parts (at most 512) must be positive");
+    NQ_REQUIRE(head_dim == 64, NQ_ERR_SHAPE, "nq_attention_output_stage: head_dim %d is not 64", head_dim);
+    const int64_t n = (int64_t)q_heads * head_dim;
+    NQ_REQUIRE(n % 32 == 0 && n <= 32768, NQ_ERR_SHAPE, "nq_attention_output_stage: heads * head_dim exceeds 32768");
+    NQ_REQUIRE(workspace_dev && nq::aligned(workspace_dev, 16), NQ_ERR_ARGUMENT,
+               "nq_attention_output_stage: the attention workspace must be given, 16-byte aligned");
+    const bool encodes = codes_dev != nullptr;
+    NQ_REQUIRE(encodes || staged_out_dev, NQ_ERR_ARGUMENT, "nq_attention_output_stage: nothing to produce");
+    if (encodes) {
+        NQ_REQUIRE(betas_dev && beta_ids_dev && norms_dev, NQ_ERR_ARGUMENT, "nq_attention_output_stage: null pointer");
+        NQ_REQUIRE(q >= 2 && q <= 16 && beta_count >= 1 && beta_count <= 4, NQ_ERR_SHAPE,
+                   "nq_attention_output_stage: q must be in [2, 16] and beta_count in [1, 4]");
+        NQ_REQUIRE(nq::aligned(codes_dev, 4) && nq::aligned(decoded_bf16_dev, 16) && nq::aligned(staged_out_dev, 16),
+                   NQ_ERR_ARGUMENT, "nq_attention_output_stage: codes need 4-byte, BF16 outputs 16-byte alignment");
+        NQ_REQUIRE(!hadamard || (n & (n - 1)) == 0, NQ_ERR_SHAPE,
+                   "nq_attention_output_stage: the Hadamard rotation needs a power-of-two feature count");
+    }
+    // the layout nq_nqkv_attention_decode leaves in its workspace
+    const size_t heads_total = (size_t)rows * q_heads;
+    nq::InputPrologue prologue{};
+    prologue.part_max = reinterpret_cast<const float *>(workspace_dev);
+    prologue.part_sum = prologue.part_max + heads_total * parts;
+    prologue.part_acc = prologue.part_sum + heads_total * parts;
+    prologue.parts = parts;
+    prologue.heads = q_heads;
+    prologue.normed_out = reinterpret_cast<uint16_t *>(staged_out_dev);
+    const int stage_dtype = (encodes && hadamard) ? NQ_BF16 : -1;
+    return launch_quantize<uint16_t, false, 3>(workspace_dev, rows, (int)n, encodes ? q : 14, betas_dev, beta_count, 0u,
+                                               codes_dev, beta_ids_dev, norms_dev, decoded_bf16_dev, stage_dtype,
+                                               (hipStream_t)stream, prologue);
 }
 
 extern "C" int nq_dequantize_rows(const uint8_t *codes_dev, const uint8_t *beta_ids_dev,

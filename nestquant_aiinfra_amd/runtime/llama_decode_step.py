@@ -31,7 +31,7 @@ import torch
 
 import torch.nn.functional as F
 
-from .nqkv import launch_nqkv_decode_attention, nqkv_prefill_attention
+from .nqkv import attention_output_stage, launch_nqkv_decode_attention, nqkv_prefill_attention
 from .w4a4_linear import (MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, _gemm, _gemv, fused_input_stage,
                           linear_packed_w4a4_gemv_grouped, quantize_activation_cuda, rope_hadamard_cuda)
 
@@ -149,12 +149,12 @@ class FusedLlamaDecodeStep:
             query, key, value = self._linears(activation, [q_w, k_w, v_w])
             manager.write_layer(index, key.view(rows, 1, kv_heads, dim), value.view(rows, 1, kv_heads, dim),
                                 rotate_keys=True, rope=(cos, sin))
-            attended = launch_nqkv_decode_attention(
+            # the attention leaves per-chunk results; o_proj's input stage merges them as it loads its rows
+            launch_nqkv_decode_attention(
                 query.view(rows, heads, dim), manager.layers[index], slot_ids=manager.step_slot_ids,
                 active_mask=manager.step_active, attention_scale=float(attention.scaling), workspace=workspace,
-                rotate_query=True, rope=query_rope)
-            o_input = quantize_activation_cuda(attended.view(rows, heads * dim), q=14,
-                                               betas=linears[3].activation_betas, beta_table=table, hadamard=True)
+                rotate_query=True, rope=query_rope, merge=False)
+            o_input, _ = attention_output_stage(workspace, q=14, beta_table=table, hadamard=True)
             delta = self._linear(o_input, o_w)
             activation, residual, _ = fused_input_stage(
                 delta, mode="rmsnorm", residual=residual, norm_weight=layer.post_attention_layernorm.weight,

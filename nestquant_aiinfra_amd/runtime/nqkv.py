@@ -24,7 +24,7 @@ from typing import Hashable, Sequence
 import torch
 
 from .. import _native
-from .w4a4_linear import _beta_values, dequantize_rows_packed, quantize_rows_packed
+from .w4a4_linear import PreparedNQA4Activation, _beta_values, dequantize_rows_packed, quantize_rows_packed
 
 PAGE_SIZE = 16
 
@@ -362,9 +362,12 @@ def launch_nqkv_decode_attention(query: torch.Tensor, cache: NQKVHotColdCache, *
                                  active_mask: torch.Tensor, attention_scale: float,
                                  workspace: BatchedNQKVAttentionWorkspace,
                                  rotate_query: bool = False,
-                                 rope: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
+                                 rope: tuple[torch.Tensor, torch.Tensor] | None = None,
+                                 merge: bool = True) -> torch.Tensor | None:
     """Graph-safe launch: no host reads, no allocation; writes workspace.output.  `rope`:
-    BF16 (cos, sin) [batch, head_dim] applied to the query inside the kernel."""
+    BF16 (cos, sin) [batch, head_dim] applied to the query inside the kernel.  With `merge`
+    false only the first stage runs and the per-chunk results stay in workspace.buffer for
+    attention_output_stage (returns None)."""
     pool, meta = cache.pool, cache.metadata
     batch, heads, dim = query.shape
     _native.check(_native.library().nq_nqkv_attention_decode(
@@ -377,10 +380,49 @@ def launch_nqkv_decode_attention(query: torch.Tensor, cache: NQKVHotColdCache, *
         cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(), slot_ids.data_ptr(), active_mask.data_ptr(),
         batch, cache.max_sequences, cache.max_pages_per_sequence, heads, pool.num_kv_heads, dim, pool.page_size,
         attention_scale, int(rotate_query), None if rope is None else rope[0].data_ptr(),
-        None if rope is None else rope[1].data_ptr(), workspace.output.data_ptr(), workspace.buffer.data_ptr(),
-        workspace.buffer.numel(),
+        None if rope is None else rope[1].data_ptr(), workspace.output.data_ptr() if merge else None,
+        workspace.buffer.data_ptr(), workspace.buffer.numel(),
         _native.stream_handle(query.device)))
-    return workspace.output
+    return workspace.output if merge else None
+
+
+def attention_output_stage(workspace: BatchedNQKVAttentionWorkspace, *, q: int = 14,
+                           beta_table: torch.Tensor | None = None, hadamard: bool = True, encode: bool = True,
+                           want_staged: bool = False):
+    """Second stage of launch_nqkv_decode_attention(..., merge=False) fused with the input stage
+    of the Linear that consumes the attention output: merges the per-chunk results into BF16 rows
+    [batch, query_heads * head_dim] and (with `encode`) rotates, encodes and packs them in the
+    same launch.  Returns (packed activation or None, merged rows when `want_staged`)."""
+    device = workspace.buffer.device
+    batch, n = workspace.batch_size, workspace.query_heads * workspace.head_dim
+    staged = torch.empty((batch, n), dtype=torch.bfloat16, device=device) if want_staged else None
+    codes = beta_ids = norms = decoded = None
+    if encode:
+        if beta_table is None or q != 14 or beta_table.numel() != 4:
+            raise ValueError("encoding needs q = 14 and a table of four betas")
+        codes = torch.empty(batch * n // 2, dtype=torch.uint8, device=device)
+        beta_ids = torch.empty(batch * n // 32, dtype=torch.uint8, device=device)
+        norms = torch.empty(batch, dtype=torch.float32, device=device)
+        decoded = torch.empty((batch, n), dtype=torch.bfloat16, device=device)
+    elif not want_staged:
+        raise ValueError("nothing to produce")
+
+    def ptr(tensor):
+        return None if tensor is None else tensor.data_ptr()
+
+    lib = _native.library()
+    parts = lib.nq_nqkv_attention_parts(batch, workspace.max_pages)
+    _native.check(lib.nq_attention_output_stage(
+        workspace.buffer.data_ptr(), batch, workspace.query_heads, workspace.head_dim, parts, ptr(staged), q,
+        ptr(beta_table), 0 if beta_table is None else beta_table.numel(), int(hadamard), ptr(codes), ptr(beta_ids),
+        ptr(norms), ptr(decoded), _native.stream_handle(device)))
+    activation = None
+    if encode:
+        activation = PreparedNQA4Activation(
+            code_payload=codes, beta_payload=beta_ids, row_norms=norms, beta_table=beta_table,
+            original_shape=(batch, n), q=q, code_width=4, beta_width=2, output_dtype=torch.bfloat16,
+            decoded=decoded)
+    return activation, staged
 
 
 def nqkv_decode_attention_batched_k1(query: torch.Tensor, cache: NQKVHotColdCache, *, slot_ids: torch.Tensor,

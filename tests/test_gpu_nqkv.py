@@ -206,6 +206,54 @@ def test_batched_attention_equals_rows_taken_alone(kv, oracle, batch):
     assert torch.equal(flipped, together[order])
 
 
+@pytest.mark.parametrize("batch,max_len,q_heads", [(8, 1024, 32), (3, 4096, 32), (1, 256, 8), (5, 64, 64)])
+def test_attention_merged_inside_the_output_encoder(kv, oracle, batch, max_len, q_heads):
+    """Stage 2 of the attention done by the encoder of the o_proj input: the merged rows equal the
+    two-launch attention to within one BF16 step (the softmax denominator is summed in another
+    order), an inactive row gives zeros, and codes, beta ids, norms and the decoded rows are bit for
+    bit what the plain encoder makes of those merged rows."""
+    from conftest import ACTIVATION_BETAS, Q
+    from nestquant_aiinfra_amd.runtime import w4a4_linear as rt
+    rng = np.random.default_rng(300 + batch)
+    manager = _manager(kv, capacity=batch, max_len=max_len)
+    lengths = [int(n) for n in rng.integers(1, max_len + 1, batch)]
+    lengths[0] = max_len
+    keys = [_bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for n in lengths]
+    values = [_bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for n in lengths]
+    for s in range(batch):
+        manager.register(s, slot=s)
+    _append(manager, list(range(batch)), keys, values)
+    cache = manager.layers[0]
+    query = _bf16(oracle.hadamard(rng.standard_normal((batch, q_heads, DIM)).astype(np.float32))).cuda()
+    slot_ids = torch.arange(batch, dtype=torch.int32, device="cuda")
+    active = torch.ones(batch, dtype=torch.bool, device="cuda")
+    if batch > 1:
+        active[batch - 1] = False
+    workspace = kv.BatchedNQKVAttentionWorkspace.create(cache, batch_size=batch, query_heads=q_heads,
+                                                        output_dtype=torch.bfloat16)
+    two_launches = kv.launch_nqkv_decode_attention(query, cache, slot_ids=slot_ids, active_mask=active,
+                                                   attention_scale=0.125, workspace=workspace).clone()
+    workspace.output.fill_(7.0)
+    assert kv.launch_nqkv_decode_attention(query, cache, slot_ids=slot_ids, active_mask=active, attention_scale=0.125,
+                                           workspace=workspace, merge=False) is None
+    assert (workspace.output == 7.0).all()                                 # no merge launch ran
+    table = torch.tensor(ACTIVATION_BETAS, dtype=torch.float32, device="cuda")
+    _, merged = kv.attention_output_stage(workspace, encode=False, want_staged=True)
+    n = q_heads * DIM
+    a, b = _f32(merged), _f32(two_launches.view(batch, n))
+    assert np.all(np.abs(a - b) <= np.abs(b) * 2.0 ** -7)
+    assert np.count_nonzero(a != b) <= a.size // 50
+    if batch > 1:
+        assert not merged[batch - 1].any()
+    power_of_two = n & (n - 1) == 0
+    activation, again = kv.attention_output_stage(workspace, q=Q, beta_table=table, hadamard=power_of_two,
+                                                  want_staged=True)
+    assert torch.equal(again, merged)
+    plain = rt.quantize_activation_cuda(merged, q=Q, betas=ACTIVATION_BETAS, beta_table=table, hadamard=power_of_two)
+    for name in ("code_payload", "beta_payload", "row_norms", "decoded"):
+        assert torch.equal(getattr(activation, name), getattr(plain, name)), name
+
+
 def test_attention_ragged_batch_at_full_size(kv, oracle):
     """Batch 8, 32 query / 8 KV heads, contexts uniform in [128, 4096] (up to 256 pages)."""
     g = torch.Generator().manual_seed(4001)
