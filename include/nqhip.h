@@ -384,6 +384,27 @@ int nq_nqkv_attention_prefill(
     int batch, int tokens, int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size,
     float scale, void *out_dev, void *stream);
 
+/*
+ * Greedy sampling inside the decode step: for every row r (all rows when active_mask_dev is NULL,
+ * else those with active_mask[r] != 0) the first index of the largest of logits[r, 0..vocab)
+ * (rows row_stride elements apart; NaN counts as the largest) is written to tokens_dev[r];
+ * positions_dev[r] (optional) is advanced by one and, when history_dev is given, the token is
+ * stored at history[cursors[r] % history_steps][r] (int64 [history_steps, rows]) and cursors[r]
+ * advanced by one.  Pointing tokens_dev / positions_dev at the captured step's own input
+ * tensors lets a graph be replayed many times without the host reading a token in between.
+ * Workspace: nq_greedy_sample_workspace_bytes(rows) bytes, 16-byte aligned, zeroed once by the
+ * caller before the first call (every call leaves it ready for the next); calls that share a
+ * workspace must not overlap.
+ * Replaces: GreedyHostSampler (nestquant/runtime/inference_engine.py:63-69) and the per-step
+ * host read of the sampled tokens (nestquant/runtime/cuda_graph_decode.py:166-182).
+ */
+int nq_greedy_sample(const void *logits_dev, int logits_dtype, int rows, int64_t vocab, int64_t row_stride,
+                     const uint8_t *active_mask_dev, int64_t *tokens_dev, int64_t *positions_dev,
+                     int64_t *history_dev, int history_steps, int32_t *cursors_dev, void *workspace_dev,
+                     size_t workspace_bytes, void *stream);
+
+size_t nq_greedy_sample_workspace_bytes(int rows);
+
 #ifdef __cplusplus
 }
 #endif

@@ -4,14 +4,15 @@ The reference runs the Hugging Face module graph for a decode step: per layer ab
 small tensor kernels (residual adds, LlamaRMSNorm, rotary embedding, SiLU and multiply,
 Hadamard passes) surround the packed linears and the NQKV attention
 (nestquant/models/fused_linear.py:276-421, nestquant/runtime/nqkv_batched_hf_backend.py:357-631).
-Here the same arithmetic, in the same BF16 tensor-operation rounding, runs in eleven launches
+Here the same arithmetic, in the same BF16 tensor-operation rounding, runs in ten launches
 per layer:
 
     residual add + RMSNorm + Hadamard + A4 encode      nq_fused_input_stage (mode 1)
     q_proj, k_proj, v_proj                             nq_w4a4_gemv_grouped
     RoPE(k) + Hadamard(k) + KV append / page pack      nq_nqkv_write
-    RoPE(q) + Hadamard(q) + paged attention            nq_nqkv_attention_decode (two kernels)
-    Hadamard + A4 encode, o_proj                       nq_quantize_rows, nq_w4a4_gemv
+    RoPE(q) + Hadamard(q) + paged attention, stage 1   nq_nqkv_attention_decode (no output given)
+    attention stage 2 + Hadamard + A4 encode           nq_attention_output_stage
+    o_proj                                             nq_w4a4_gemv
     residual add + RMSNorm + Hadamard + A4 encode      nq_fused_input_stage (mode 1)
     gate_proj, up_proj                                 nq_w4a4_gemv_grouped
     SiLU(gate) * up + Hadamard + A4 encode             nq_fused_input_stage (mode 2)

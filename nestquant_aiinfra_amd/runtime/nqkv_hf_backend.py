@@ -21,6 +21,7 @@ import torch.nn.functional as F
 from transformers.cache_utils import Cache
 from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
 
+from .. import _native
 from .nqkv import (BatchedNQKVAttentionWorkspace, BatchedNQKVCacheManager, launch_nqkv_decode_attention,
                    nqkv_prefill_attention)
 from .w4a4_linear import hadamard_cuda
@@ -250,18 +251,73 @@ def install_batched_nqkv_llama_backend(model: torch.nn.Module, cache: BatchedNQK
     return BATCHED_NQKV_ATTENTION_NAME
 
 
+def greedy_sample_(logits: torch.Tensor, tokens: torch.Tensor, *, positions: torch.Tensor | None = None,
+                   active_mask: torch.Tensor | None = None, history: torch.Tensor | None = None,
+                   cursors: torch.Tensor | None = None, workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """Device-side GreedyHostSampler (nestquant/runtime/inference_engine.py:63-69): writes the
+    argmax of logits [rows, vocab] (ties: lowest index) into tokens (int64, `rows` entries), in
+    place, for the rows of `active_mask` (bool [rows]; all when None); advances `positions`
+    (int64, `rows` entries) by one and appends to `history` (int64 [steps, rows]) at
+    `cursors` (int32 [rows]), which it advances.  One launch; graph-safe when `workspace`
+    (`greedy_sample_workspace(rows, device)`, reusable by calls that do not overlap) is given."""
+    if logits.ndim != 2 or logits.stride(1) != 1:
+        raise ValueError("sampler logits must have shape [requests, vocabulary] with contiguous rows")
+    rows, vocab = logits.shape
+    device = logits.device
+    if device.type != "cuda":
+        raise ValueError("tensors must live on the GPU (device type 'cuda' under ROCm)")
+    for name, tensor, dtype in (("tokens", tokens, torch.int64), ("positions", positions, torch.int64),
+                                ("history", history, torch.int64), ("cursors", cursors, torch.int32),
+                                ("active_mask", active_mask, torch.bool)):
+        if tensor is None:
+            continue
+        if tensor.dtype != dtype or tensor.device != device or not tensor.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous {dtype} tensor on the logits' device")
+    if tokens.numel() != rows or (positions is not None and positions.numel() != rows) or (
+            active_mask is not None and active_mask.numel() != rows):
+        raise ValueError("tokens, positions and active_mask hold one entry per row of logits")
+    steps = 0
+    if history is not None:
+        if cursors is None or cursors.numel() != rows or history.ndim != 2 or history.shape[1] != rows:
+            raise ValueError("history must be [steps, rows] with one cursor per row")
+        steps = history.shape[0]
+
+    if workspace is None:
+        workspace = greedy_sample_workspace(rows, device)
+    elif workspace.dtype != torch.uint8 or workspace.device != device or not workspace.is_contiguous():
+        raise ValueError("workspace must come from greedy_sample_workspace on the logits' device")
+
+    def ptr(tensor):
+        return None if tensor is None else tensor.data_ptr()
+
+    _native.check(_native.library().nq_greedy_sample(
+        logits.data_ptr(), _native.dtype_tag(logits.dtype), rows, vocab, logits.stride(0), ptr(active_mask),
+        tokens.data_ptr(), ptr(positions), ptr(history), steps, ptr(cursors), workspace.data_ptr(),
+        workspace.numel(), _native.stream_handle(device)))
+    return tokens
+
+
+def greedy_sample_workspace(rows: int, device: torch.device) -> torch.Tensor:
+    """Zeroed scratch of greedy_sample_ for up to `rows` rows."""
+    return torch.zeros(_native.library().nq_greedy_sample_workspace_bytes(rows), dtype=torch.uint8, device=device)
+
+
 class BatchedNQKVLlamaRunner:
     """Fixed-capacity prefill / decode driver over a causal Llama model and an NQKV cache.
 
     Decode steps of width w in {1, 2, 4, ..., capacity} are captured once as HIP graphs
     (`capture`); active rows are compacted to the smallest width that holds them.  A step
     reads nothing from the device: token ids, positions, slot ids and masks are copied into
-    the graph's fixed input tensors, the graph is replayed, logits are returned.
+    the graph's fixed input tensors, the graph is replayed, logits are returned.  The captured
+    step ends with the greedy sampler writing each active row's next token and position back
+    into those input tensors, so `decode_greedy` replays it many times between host reads.
     """
+
+    GREEDY_HISTORY_STEPS = 256
 
     def __init__(self, model: torch.nn.Module, cache: BatchedNQKVLlamaCache, *,
                  fused_decode: bool | None = None, fused_prefill: bool | None = None) -> None:
-        """`fused_decode` / `fused_prefill`: run decode steps through FusedLlamaDecodeStep (eleven
+        """`fused_decode` / `fused_prefill`: run decode steps through FusedLlamaDecodeStep (ten
         launches per layer) and prompts through FusedLlamaPrefillStep instead of the module
         graph; None = whenever the model qualifies."""
         if not isinstance(model, torch.nn.Module):
@@ -277,6 +333,7 @@ class BatchedNQKVLlamaRunner:
         self.batch_size, self.max_cache_len = cache.capacity, cache.max_cache_len
         self._generation = [0] * self.batch_size
         self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor, torch.Tensor]] = {}
+        self._greedy: dict[int, tuple[torch.Tensor, ...]] = {}       # width -> (history, cursors, sampler scratch)
         self.graph_replay_counts: dict[int, int] = {}
         self._decode_state: tuple | None = None      # (width, slots) the step tensors were last set for
         self.fused_step = None
@@ -371,11 +428,18 @@ class BatchedNQKVLlamaRunner:
                 for _ in range(2):
                     self._step(tokens, positions)
                 stream.synchronize()
+                history = torch.zeros((self.GREEDY_HISTORY_STEPS, width), dtype=torch.long, device=self.device)
+                cursors = torch.zeros(width, dtype=torch.int32, device=self.device)
+                scratch = greedy_sample_workspace(width, self.device)
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph, stream=stream):
                     logits = self._step(tokens, positions)
+                    greedy_sample_(logits.view(width, -1), tokens, positions=positions,
+                                   active_mask=self.cache.manager.step_active[:width], history=history,
+                                   cursors=cursors, workspace=scratch)
             torch.cuda.current_stream(self.device).wait_stream(stream)
             self._graphs[width] = (graph, tokens, positions, logits)
+            self._greedy[width] = (history, cursors, scratch)
             self.graph_replay_counts[width] = 0
         for tensor, value in zip((meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths), saved):
             tensor.copy_(value)
@@ -402,3 +466,37 @@ class BatchedNQKVLlamaRunner:
         self.graph_replay_counts[width] += 1
         self.cache.note_decode_step(slots)
         return logits[:rows]
+
+    @torch.inference_mode()
+    def decode_greedy(self, tokens: torch.Tensor, *, slots: Sequence[int], positions: torch.Tensor,
+                      steps: int) -> torch.Tensor:
+        """`steps` captured decode steps with the greedy sampler on the device and no host read in
+        between: step i feeds the token step i - 1 chose.  tokens / positions [rows, 1] as for
+        `decode`; returns the chosen tokens, int64 [steps, rows] (the same tokens `decode` followed
+        by an argmax of its logits gives, step by step)."""
+        rows = len(slots)
+        if isinstance(steps, bool) or not isinstance(steps, int) or not 1 <= steps <= self.GREEDY_HISTORY_STEPS:
+            raise ValueError(f"steps must be an integer in [1, {self.GREEDY_HISTORY_STEPS}]")
+        width = next((w for w in sorted(self._graphs) if w >= rows), None)
+        if width is None:
+            raise RuntimeError("decode_greedy needs a captured graph of this width: call capture() first")
+        for slot in slots:
+            if self.cache._host_lengths[slot] + steps > self.max_cache_len:
+                raise ValueError("the generated tokens exceed max_cache_len")
+        graph, graph_tokens, graph_positions, _ = self._graphs[width]
+        history, cursors, _ = self._greedy[width]
+        graph_tokens[:rows].copy_(tokens)
+        graph_positions[:rows].copy_(positions)
+        cursors.zero_()
+        state = (width, tuple(slots))
+        if state != self._decode_state:
+            padded_slots = list(slots) + [0] * (width - rows)
+            self.cache.set_decode_execution_state(
+                slot_ids=torch.tensor(padded_slots, dtype=torch.int32, device=self.device),
+                active_mask=torch.tensor([True] * rows + [False] * (width - rows), device=self.device))
+            self._decode_state = state
+        for _ in range(steps):
+            graph.replay()
+            self.cache.note_decode_step(slots)
+        self.graph_replay_counts[width] += steps
+        return history[:steps, :rows].clone()

@@ -366,3 +366,77 @@ def test_fused_decode_step_with_more_than_eight_rows(tmp_path):
     runner.capture(widths=[rows])
     replayed = runner.decode(token, slots=list(range(rows)), positions=position).float()
     assert torch.equal(replayed, fused)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_greedy_sampler_is_the_first_argmax(dtype):
+    """The device sampler against torch.argmax: ties (BF16 logits repeat values) go to the lowest
+    index, NaN counts as the largest value, rows may be strided slices, a vocabulary that is not a
+    whole number of 16-byte vectors takes the element loop; inactive rows keep token and position."""
+    from nestquant_aiinfra_amd.runtime.nqkv_hf_backend import greedy_sample_
+    g = torch.Generator().manual_seed(77)
+    for rows, vocab, stride in ((8, 128256, 128256), (3, 1000, 1024), (5, 777, 777), (1, 5, 8), (2, 70001, 70001)):
+        storage = torch.randn((rows, stride), generator=g).to(dtype).cuda()
+        storage[0, :vocab] = storage[0, :vocab].round()                    # many equal maxima
+        if rows > 1:
+            storage[1, vocab // 2] = float("nan")
+            storage[1, vocab - 1] = float("nan")
+        if stride > vocab:
+            storage[:, vocab:] = 1e4                                      # beyond the vocabulary: never chosen
+        logits = storage[:, :vocab]
+        want = logits.float().argmax(-1)
+        if rows > 1:
+            want[1] = vocab // 2                                          # the first NaN
+        tokens = torch.full((rows, 1), -1, dtype=torch.long, device="cuda")
+        positions = torch.arange(rows, dtype=torch.long, device="cuda").reshape(rows, 1) * 10
+        active = torch.ones(rows, dtype=torch.bool, device="cuda")
+        if rows > 2:
+            active[2] = False
+        history = torch.full((4, rows), -1, dtype=torch.long, device="cuda")
+        cursors = torch.zeros(rows, dtype=torch.int32, device="cuda")
+        for step in range(6):                                             # the history is a ring of four steps
+            greedy_sample_(logits, tokens, positions=positions, active_mask=active, history=history, cursors=cursors)
+        live = active.cpu()
+        assert torch.equal(tokens.view(-1).cpu()[live], want.cpu()[live]), (rows, vocab)
+        assert (tokens.view(-1).cpu()[~live] == -1).all()
+        assert torch.equal(positions.view(-1).cpu(), torch.arange(rows) * 10 + 6 * live.long())
+        assert torch.equal(cursors.cpu(), 6 * live.int())
+        assert (history.cpu()[:, live] == want.cpu()[live]).all() and (history.cpu()[:, ~live] == -1).all()
+        plain = torch.zeros(rows, dtype=torch.long, device="cuda")
+        assert torch.equal(greedy_sample_(logits, plain), want)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_many_greedy_steps_without_a_host_read(tmp_path, fused):
+    """decode_greedy replays the captured step with the sampler's token fed back on the device:
+    the same tokens as decode + argmax on the host, step by step, and the same cache state."""
+    runner = _tiny_runners(tmp_path, 5010, capacity=4, max_cache_len=200)[0 if fused else 1]
+    g = torch.Generator().manual_seed(5011)
+    ids = torch.randint(0, 128, (3, 40), generator=g).cuda()
+    lengths, slots, steps = [40, 21, 5], [2, 0, 3], 37
+
+    def start():
+        logits = runner.prefill_slots(ids, slots=slots, lengths=lengths)
+        token = torch.stack([logits[i, n - 1].argmax() for i, n in enumerate(lengths)]).reshape(3, 1)
+        return token, torch.tensor(lengths, device="cuda").reshape(3, 1)
+
+    token, position = start()
+    runner.capture()
+    by_host = []
+    for _ in range(steps):
+        token = runner.decode(token, slots=slots, positions=position)[:, 0].argmax(-1).reshape(3, 1)
+        by_host.append(token.view(-1).clone())
+        position = position + 1
+    lengths_by_host = runner.cache.manager.metadata.sequence_lengths.clone()
+    runner.release_slots(slots)
+
+    token, position = start()
+    on_device = runner.decode_greedy(token, slots=slots, positions=position, steps=steps)
+    assert torch.equal(on_device, torch.stack(by_host))
+    assert torch.equal(runner.cache.manager.metadata.sequence_lengths, lengths_by_host)
+    assert [runner.cache._host_lengths[s] for s in slots] == [n + steps for n in lengths]
+    # a second run continues from the device's own tokens
+    more = runner.decode_greedy(on_device[-1].reshape(3, 1), slots=slots, positions=position + steps, steps=5)
+    assert more.shape == (5, 3)
+    with pytest.raises(ValueError):
+        runner.decode_greedy(token, slots=slots, positions=position, steps=500)
