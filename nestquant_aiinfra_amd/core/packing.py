@@ -137,6 +137,40 @@ class PackedNestQuantIndices:
                 torch.from_numpy(betas.astype(np.int64)).reshape(self.shape[:-1]).to(device))
 
 
+    def unpack_rows(self, start: int, end: int, *, device: torch.device | str = "cpu"
+                    ) -> tuple[torch.Tensor, torch.Tensor]:
+        """Rows [start, end) of the leading dimension (nestquant/core/packing.py:108-135): only the
+        bytes of those rows are read, also when a row's beta ids begin inside a byte."""
+        if any(isinstance(v, bool) or not isinstance(v, int) for v in (start, end)):
+            raise TypeError("row bounds must be integers")
+        if start < 0 or end < start or end > self.shape[0]:
+            raise ValueError("row range is outside packed tensor bounds")
+        per_row_codes, per_row_betas = math.prod(self.shape[1:]), math.prod(self.shape[1:-1])
+        codes = _unpack_window(self.code_payload, start * per_row_codes, end * per_row_codes, self.code_bit_width)
+        betas = _unpack_window(self.beta_payload, start * per_row_betas, end * per_row_betas,
+                               self.beta_index_bit_width)
+        if codes.size and int(codes.max()) >= self.q:
+            raise ValueError("decoded residue is outside [0, q)")
+        if betas.size and int(betas.max()) >= self.beta_count:
+            raise ValueError("decoded beta index is outside [0, beta_count)")
+        rows = end - start
+        return (torch.from_numpy(codes.astype(np.int64)).reshape((rows, *self.shape[1:])).to(device),
+                torch.from_numpy(betas.astype(np.int64)).reshape((rows, *self.shape[1:-1])).to(device))
+
+
+def _unpack_window(payload: bytes, first: int, last: int, width: int) -> np.ndarray:
+    """Values [first, last) of a fixed-width stream, touching only the bytes that hold them."""
+    if first == last:
+        return np.empty(0, dtype=np.uint8)
+    per_byte = 8 // width
+    byte0, byte1 = first // per_byte, -(-last // per_byte)
+    window = np.frombuffer(payload, dtype=np.uint8, count=byte1 - byte0, offset=byte0)
+    shifts = (np.arange(per_byte, dtype=np.uint8) * width)[None, :]
+    values = ((window[:, None] >> shifts) & ((1 << width) - 1)).reshape(-1)
+    skip = first - byte0 * per_byte
+    return values[skip:skip + (last - first)].copy()
+
+
 def pack_nestquant_indices(codes: torch.Tensor, beta_indices: torch.Tensor, *, q: int,
                            beta_count: int) -> PackedNestQuantIndices:
     """Pack integer code / beta-id tensors (nestquant/core/packing.py:137-171)."""

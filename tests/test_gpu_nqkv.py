@@ -373,3 +373,55 @@ def test_pool_handles_are_generation_checked(kv):
     c = pool.allocate()
     assert c.page_id == a.page_id and c.generation == a.generation + 1 and pool.free_pages == 0
     assert pool.page_payload_bytes == 9728 and b.page_id != c.page_id
+
+
+def test_page_container_from_the_gpu_encoder_equals_the_reference_file(kv, golden, golden_meta):
+    """PackedNQKVPage.from_tensors (HIP encoder) serialises to the bytes the reference's CPU path
+    wrote for the same page (SHA-256 in the golden metadata), decodes to the reference's values, and
+    survives the trip through bytes and back onto the device."""
+    import hashlib
+    from nestquant_aiinfra_amd.core.kv_format import PackedNQKVPage
+    key = torch.from_numpy(golden["kv_key_bf16_bits"]).view(torch.bfloat16).cuda()
+    value = torch.from_numpy(golden["kv_value_bf16_bits"]).view(torch.bfloat16).cuda()
+    page = PackedNQKVPage.from_tensors(key, value, page_size=PAGE, q=Q, key_betas=KEY_BETAS, value_betas=VALUE_BETAS)
+    blob = page.to_bytes()
+    assert hashlib.sha256(blob).hexdigest() == golden_meta["kv_container_v2_sha256"]
+    restored = PackedNQKVPage.from_bytes(blob)
+    dk, dv = restored.dequantize(output_dtype=torch.float32)
+    assert np.array_equal(_f32(dk), golden["kv_key_deq"]) and np.array_equal(_f32(dv), golden["kv_value_deq"])
+    # back into a pool page
+    pool = kv.NQKVPagePool(capacity=2, page_size=PAGE, num_kv_heads=HEADS, head_dim=DIM, q=Q, key_betas=KEY_BETAS,
+                           value_betas=VALUE_BETAS, device="cuda")
+    handle = pool.allocate()
+    pool.store_prepared(handle, restored.to_prepared("cuda"))
+    stored = pool.prepared(handle)
+    assert np.array_equal(bits(stored.key_code_payload), golden["kv_key_codes"])
+    assert np.array_equal(bits(stored.value_norms), golden["kv_value_norms"])
+
+
+@pytest.mark.parametrize("valid", [1, 5, 15, 16])
+def test_page_container_fill_levels(kv, oracle, golden, valid):
+    """Boundary fill levels (tests/unit/core/test_kv_format.py:59-78): padding rows are encoded
+    zeros, never leak into the valid prefix, and both container versions round-trip."""
+    from nestquant_aiinfra_amd.core.kv_format import PackedNQKVPage
+    key = torch.from_numpy(golden["kv_key_bf16_bits"]).view(torch.bfloat16).cuda()[:valid]
+    value = torch.from_numpy(golden["kv_value_bf16_bits"]).view(torch.bfloat16).cuda()[:valid]
+    for tables in ({"betas": KEY_BETAS}, {"key_betas": KEY_BETAS, "value_betas": VALUE_BETAS}):
+        page = PackedNQKVPage.from_tensors(key, value, page_size=PAGE, q=Q, **tables)
+        assert page.valid_tokens == valid and page.payload_bytes == 9728
+        assert not page.key_norms[valid * HEADS:].any() and not page.value_norms[valid * HEADS:].any()
+        again = PackedNQKVPage.from_bytes(page.to_bytes())
+        assert again.format_version == (1 if "betas" in tables else 2)
+        dk, dv = again.dequantize(output_dtype=torch.float32)
+        assert tuple(dk.shape) == tuple(dv.shape) == (valid, HEADS, DIM)
+        assert np.array_equal(_f32(dk), golden["kv_key_deq"][:valid])
+        if "betas" not in tables:
+            assert np.array_equal(_f32(dv), golden["kv_value_deq"][:valid])
+    if valid == 5:
+        legacy = PackedNQKVPage.from_tensors(key, value, page_size=PAGE, q=Q, betas=KEY_BETAS)
+        assert np.array_equal(np.frombuffer(legacy.key_indices.code_payload, np.uint8), golden["kv_partial_key_codes"])
+        assert np.array_equal(legacy.key_norms.numpy(), golden["kv_partial_key_norms"])
+    with pytest.raises(ValueError):
+        PackedNQKVPage.from_tensors(key, value, page_size=PAGE, q=Q, betas=KEY_BETAS, key_betas=KEY_BETAS)
+    with pytest.raises(ValueError):
+        PackedNQKVPage.from_tensors(key, value, page_size=PAGE, q=Q, key_betas=KEY_BETAS)
