@@ -117,6 +117,13 @@ class BatchedNQKVLlamaCache(Cache):
         for slot in slots:
             self._host_lengths[slot] += 1
 
+    def require_room(self, slots: Sequence[int], tokens: int = 1) -> None:
+        """Raises before a step that would take a slot past the cache length (the device tables
+        clamp there, so the step itself would overwrite the newest tokens instead)."""
+        for slot in slots:
+            if self._host_lengths[slot] + tokens > self.manager.max_tokens:
+                raise RuntimeError("sequence would exceed max_cache_len")
+
     # -- Cache protocol -------------------------------------------------------------------------
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int, *args, **kwargs):
         del args, kwargs
@@ -395,6 +402,7 @@ class BatchedNQKVLlamaRunner:
     def decode_eager(self, tokens: torch.Tensor, *, slots: Sequence[int], positions: torch.Tensor) -> torch.Tensor:
         """One un-captured decode step for `slots` (tokens, positions: [rows, 1])."""
         rows = len(slots)
+        self.cache.require_room(slots)
         self._decode_state = None
         self.cache.set_decode_execution_state(
             slot_ids=torch.tensor(list(slots), dtype=torch.int32, device=self.device),
@@ -451,6 +459,7 @@ class BatchedNQKVLlamaRunner:
         width = next((w for w in sorted(self._graphs) if w >= rows), None)
         if width is None:
             return self.decode_eager(tokens, slots=slots, positions=positions)
+        self.cache.require_room(slots)
         graph, graph_tokens, graph_positions, logits = self._graphs[width]
         graph_tokens[:rows].copy_(tokens)
         graph_positions[:rows].copy_(positions)
@@ -480,9 +489,7 @@ class BatchedNQKVLlamaRunner:
         width = next((w for w in sorted(self._graphs) if w >= rows), None)
         if width is None:
             raise RuntimeError("decode_greedy needs a captured graph of this width: call capture() first")
-        for slot in slots:
-            if self.cache._host_lengths[slot] + steps > self.max_cache_len:
-                raise ValueError("the generated tokens exceed max_cache_len")
+        self.cache.require_room(slots, steps)
         graph, graph_tokens, graph_positions, _ = self._graphs[width]
         history, cursors, _ = self._greedy[width]
         graph_tokens[:rows].copy_(tokens)

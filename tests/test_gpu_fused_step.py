@@ -440,3 +440,24 @@ def test_many_greedy_steps_without_a_host_read(tmp_path, fused):
     assert more.shape == (5, 3)
     with pytest.raises(ValueError):
         runner.decode_greedy(token, slots=slots, positions=position, steps=500)
+
+
+def test_decode_refuses_to_run_past_the_cache_length(tmp_path):
+    """The host mirror of the lengths stops a step that would not fit (the device tables clamp at
+    capacity, they never write out of bounds): decode, decode_eager, decode_greedy and prefill."""
+    runner = _tiny_runners(tmp_path, 5020, capacity=2, max_cache_len=48)[0]
+    ids = torch.randint(0, 128, (1, 40), generator=torch.Generator().manual_seed(1)).cuda()
+    logits = runner.prefill_slots(ids, slots=[1], lengths=[40])
+    token = logits[:, -1].argmax(-1).reshape(1, 1)
+    position = torch.tensor([[40]], device="cuda")
+    runner.capture()
+    with pytest.raises(RuntimeError, match="max_cache_len"):
+        runner.decode_greedy(token, slots=[1], positions=position, steps=9)
+    tokens = runner.decode_greedy(token, slots=[1], positions=position, steps=8)          # fills the cache exactly
+    assert runner.cache.manager.total_tokens(1) == 48
+    for step in (runner.decode, runner.decode_eager):
+        with pytest.raises(RuntimeError, match="max_cache_len"):
+            step(tokens[-1].reshape(1, 1), slots=[1], positions=position + 8)
+    with pytest.raises(RuntimeError, match="max_cache_len"):
+        runner.prefill_slots(ids[:, :1], slots=[1], lengths=[1])
+    assert runner.cache.manager.total_tokens(1) == 48
