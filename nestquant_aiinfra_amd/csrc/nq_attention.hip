@@ -399,12 +399,15 @@ attention_merge_kernel(const float *__restrict__ part_max, const float *__restri
 
 namespace {
 
-// Pages per chunk: halved from 16 while the launch would have fewer than 64 (row, chunk)
-// pairs, so that a few short contexts still occupy many compute units.
+// Pages per chunk, from measurements over batches of 1 to 8 and tables of 23 to 512 pages: a
+// workgroup's time is mostly the latency of its first loads up to 4 pages and grows from there,
+// while every further chunk adds workgroups (a second round on the chip beyond about 768) and a
+// part to merge.  Tables of up to 64 pages: 4; longer ones: 8; 16 only when even that would
+// launch more than 384 (row, chunk) pairs.
 int pages_per_chunk_for(int batch, int max_pages) {
-    int pages = nq::kAttnMaxPagesPerChunk;
-    while (pages > 2 && (int64_t)batch * ((max_pages + pages - 1) / pages) < 64) pages /= 2;
-    return pages;
+    if (max_pages <= 64) return 4;
+    if ((int64_t)batch * ((max_pages + 7) / 8) > 384) return nq::kAttnMaxPagesPerChunk;
+    return 8;
 }
 
 int chunks_for(int batch, int max_pages) {
@@ -492,7 +495,6 @@ extern "C" int nq_nqkv_attention_decode(
     const dim3 grid((unsigned)parts, (unsigned)(batch * kv_heads));
 #define NQ_LAUNCH_STAGE1(GROUP)                                                                                   \
     switch (pages_per_chunk_for(batch, max_pages)) {                                                              \
-        case 2: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 2>), grid, dim3(nq::kAttnThreads), 0, s, a); break;  \
         case 4: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 4>), grid, dim3(nq::kAttnThreads), 0, s, a); break;  \
         case 8: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 8>), grid, dim3(nq::kAttnThreads), 0, s, a); break;  \
         default: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 16>), grid, dim3(nq::kAttnThreads), 0, s, a); break; \

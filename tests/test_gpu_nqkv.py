@@ -281,10 +281,12 @@ def test_attention_ragged_batch_at_full_size(kv, oracle):
     assert torch.isfinite(out).all()
 
 
-@pytest.mark.parametrize("capacity,max_len,q_heads", [(4, 1024, 64), (8, 1024, 16), (1, 4096, 32), (2, 64, 8)])
+@pytest.mark.parametrize("capacity,max_len,q_heads", [(4, 1024, 64), (8, 1024, 16), (1, 4096, 32), (2, 64, 8),
+                                                      (8, 6400, 32)])
 def test_attention_chunk_sizes(kv, oracle, capacity, max_len, q_heads):
-    """The context is cut into chunks of 2 to 16 pages depending on batch and table width:
-    every chunk size, with contexts that end inside a chunk, on a page edge and in the hot tail."""
+    """The context is cut into chunks of 4, 8 or 16 pages depending on batch and table width
+    (4 up to 64 pages, 16 from 8 x 400 pages): every chunk size, with contexts that end inside a
+    chunk, on a page edge and in the hot tail."""
     rng = np.random.default_rng(capacity * max_len + q_heads)
     manager = _manager(kv, capacity=capacity, max_len=max_len)
     lengths = [max_len, max_len // 2 + 5, 33, 16, max_len - 16, 7, 1, max_len // 4][:capacity]
