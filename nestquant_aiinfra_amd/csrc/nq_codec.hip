@@ -459,17 +459,47 @@ dequantize_rows_kernel(const uint32_t *__restrict__ codes, const uint8_t *__rest
 // Stand-alone Hadamard rotation of rows (post-RoPE queries and keys, prefill inputs).
 // ---------------------------------------------------------------------------------------
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 hadamard_rows_kernel(const T *__restrict__ x, int64_t rows, int n, int rows_per_wg, int stage_dtype,
-                     void *__restrict__ out, int out_dtype) {
+                     void *__restrict__ out, int out_dtype, int vector_io) {
     extern __shared__ float lds[];
     const int64_t row0 = (int64_t)blockIdx.x * rows_per_wg;
     const int64_t first = row0 * n, limit = rows * (int64_t)n;
-    for (int idx = threadIdx.x; idx < rows_per_wg * n; idx += blockDim.x)
-        lds[idx] = first + idx < limit ? RowLoader<T>::scalar(x, first + idx) : 0.0f;
+    const int staged = rows_per_wg * n;
+    if (vector_io) {
+        // rows are whole numbers of 16-byte vectors, input and output 16-byte aligned
+        constexpr int kPer = RowLoader<T>::kPerVector;
+        for (int v = threadIdx.x; v < staged / kPer; v += blockDim.x) {
+            const int64_t g = first + (int64_t)v * kPer;
+            if (g < limit) {
+                RowLoader<T>::load(x, g / kPer, lds + v * kPer);
+            } else {
+#pragma unroll
+                for (int j = 0; j < kPer; j++) lds[v * kPer + j] = 0.0f;
+            }
+        }
+    } else {
+        for (int idx = threadIdx.x; idx < staged; idx += blockDim.x)
+            lds[idx] = first + idx < limit ? RowLoader<T>::scalar(x, first + idx) : 0.0f;
+    }
     __syncthreads();
     staged_hadamard(lds, rows_per_wg, n, stage_dtype);
-    for (int idx = threadIdx.x; idx < rows_per_wg * n; idx += blockDim.x) {
+    if (vector_io && out_dtype != NQ_F16) {
+        for (int v = threadIdx.x; v < staged / 8; v += blockDim.x) {
+            const int64_t g = first + (int64_t)v * 8;
+            if (g >= limit) continue;
+            const float4 lo = *reinterpret_cast<const float4 *>(lds + v * 8), hi = *reinterpret_cast<const float4 *>(lds + v * 8 + 4);
+            if (out_dtype == NQ_BF16) {
+                const float y[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                reinterpret_cast<uint4 *>(out)[g >> 3] = pack_bf16x8(y);
+            } else {
+                reinterpret_cast<float4 *>(out)[g >> 2] = lo;
+                reinterpret_cast<float4 *>(out)[(g >> 2) + 1] = hi;
+            }
+        }
+        return;
+    }
+    for (int idx = threadIdx.x; idx < staged; idx += blockDim.x) {
         const int64_t g = first + idx;
         if (g >= limit) continue;
         if (out_dtype == NQ_BF16) reinterpret_cast<uint16_t *>(out)[g] = f32_to_bf16(lds[idx]);
@@ -549,6 +579,10 @@ extern "C" int nq_hadamard(const void *x_dev, int x_dtype, int64_t rows, int64_t
     const size_t lds_bytes = (size_t)rows_per_wg * n * sizeof(float);
     const int64_t grid = (rows + rows_per_wg - 1) / rows_per_wg;
     NQ_REQUIRE(grid <= 0x7fffffff, NQ_ERR_SHAPE, "nq_hadamard: too many rows");
+    // eight values per lane: long rows get up to 1024 lanes
+    int threads = (int)((int64_t)rows_per_wg * n / 8);
+    threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : (threads + 63) / 64 * 64);
+    const int vector_io = n % 8 == 0 && nq::aligned(x_dev, 16) && nq::aligned(out_dev, 16);
     hipStream_t s = (hipStream_t)stream;
 #define NQ_LAUNCH_HADAMARD(T)                                                                          \
     do {                                                                                               \
@@ -556,9 +590,9 @@ extern "C" int nq_hadamard(const void *x_dev, int x_dtype, int64_t rows, int64_t
         if (lds_bytes > 48 * 1024)                                                                     \
             (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),                          \
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);     \
-        hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), lds_bytes, s,                      \
+        hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(threads), lds_bytes, s,                  \
                            reinterpret_cast<const T *>(x_dev), rows, (int)n, rows_per_wg, stage_dtype, \
-                           out_dev, out_dtype);                                                        \
+                           out_dev, out_dtype, vector_io);                                             \
     } while (0)
     if (x_dtype == NQ_F32) NQ_LAUNCH_HADAMARD(float);
     else if (x_dtype == NQ_BF16) NQ_LAUNCH_HADAMARD(uint16_t);
