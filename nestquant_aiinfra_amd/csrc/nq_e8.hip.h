@@ -183,16 +183,12 @@ __device__ __forceinline__ void reduce_coset_point(const float (&p)[8], float q,
     for (int j = 0; j < 8; j++) out[j] = p[j] - q * k[j]; // exact
 }
 
-typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-
-// x * c + a modulo 2^32 from two 16-bit dot products and a shift-add (three full-rate
-// instructions; a 32-bit integer multiply issues at a quarter of that rate).
-// With x = xl + 2^16 xh and c = cl + 2^16 ch:  x c = xl cl + 2^16 (xl ch + xh cl)  (mod 2^32).
+// x * c + a modulo 2^32.  On gfx950 the 32-bit multiply issues at the rate of the other
+// three-operand integer instructions (measured: v_mul_lo_u32 2.0 ns per wavefront instruction and
+// SIMD, v_dot2_u32_u16 1.9, v_lshl_add_u32 1.8, v_add_u32 1.1), so one multiply and one add beat
+// the two 16-bit dot products and the shift-add a quarter-rate multiplier would call for.
 __device__ __forceinline__ uint32_t mul_add_u32(uint32_t x, uint32_t c, uint32_t a) {
-    const u16x2 xv = __builtin_bit_cast(u16x2, x);
-    const uint32_t cross = __builtin_amdgcn_udot2(xv, __builtin_bit_cast(u16x2, (c << 16) | (c >> 16)), 0u, false);
-    const uint32_t low = __builtin_amdgcn_udot2(xv, __builtin_bit_cast(u16x2, c & 0xffffu), a, false);
-    return (cross << 16) + low;
+    return x * c + a;
 }
 
 // codec.py:213-222 / nestquant/runtime/nqrt4_device.cuh:7-17: lcg31_mix_v1.  Only the
