@@ -75,18 +75,44 @@ gemv_rows(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8
         for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
     }
 
-    for (int b = tid; b < slice_blocks; b += kGemvThreads) {
-        uint32_t word[R], side[R];
+    // the operands of a step are requested one step ahead: a long row (down_proj: four steps)
+    // waits for memory once, not once per step
+    uint32_t word_next[R], side_next[R];
+    uint4 a_next[M];
+#pragma unroll
+    for (int r = 0; r < R; r++) { word_next[r] = 0u; side_next[r] = 0u; }
+#pragma unroll
+    for (int m = 0; m < M; m++) a_next[m] = make_uint4(0, 0, 0, 0);
+    if (tid < slice_blocks) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const int64_t g = row_first_block[r] + b;
-            word[r] = w_words[g];
-            side[r] = kResolved ? (uint32_t)w_tails[g] : (uint32_t)w_beta_ids[g >> 2];
+            const int64_t g = row_first_block[r] + tid;
+            word_next[r] = w_words[g];
+            side_next[r] = kResolved ? (uint32_t)w_tails[g] : (uint32_t)w_beta_ids[g >> 2];
         }
-        uint4 a[M];
 #pragma unroll
         for (int m = 0; m < M; m++)
-            a[m] = m < m_rows ? act[(int64_t)m * blocks_per_row + slice_first_block + b] : make_uint4(0, 0, 0, 0);
+            if (m < m_rows) a_next[m] = act[(int64_t)m * blocks_per_row + slice_first_block + tid];
+    }
+    for (int b = tid; b < slice_blocks; b += kGemvThreads) {
+        uint32_t word[R], side[R];
+        uint4 a[M];
+#pragma unroll
+        for (int r = 0; r < R; r++) { word[r] = word_next[r]; side[r] = side_next[r]; }
+#pragma unroll
+        for (int m = 0; m < M; m++) a[m] = a_next[m];
+        const int ahead = b + kGemvThreads;
+        if (ahead < slice_blocks) {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const int64_t g = row_first_block[r] + ahead;
+                word_next[r] = w_words[g];
+                side_next[r] = kResolved ? (uint32_t)w_tails[g] : (uint32_t)w_beta_ids[g >> 2];
+            }
+#pragma unroll
+            for (int m = 0; m < M; m++)
+                if (m < m_rows) a_next[m] = act[(int64_t)m * blocks_per_row + slice_first_block + ahead];
+        }
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const int64_t g = row_first_block[r] + b;
