@@ -47,7 +47,7 @@ def linear_bytes(m: int, k: int, n: int) -> int:
 # HBM bytes per launch of the linear kernel (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by
 # what the same counters read for a 256 MiB copy; runs and factors in
 # profiles/w4a4_gemv_decode_rocprofv3.md).  Counters cannot be read from inside this process.
-MEASURED_TRAFFIC_BYTES = {"q_proj_m1": 3_411_000, "q_proj_m8": 3_613_000, "down_proj_m1": 12_945_000,
+MEASURED_TRAFFIC_BYTES = {"q_proj_m1": 3_414_000, "q_proj_m8": 3_613_000, "down_proj_m1": 12_948_000,
                           "down_proj_m8": 13_836_000}
 # the kernel each case launches (one row: vector units; eight rows: matrix cores, two K ranges per tile)
 CASE_KERNEL = {"q_proj_m1": "w4a4_gemv_kernel<1, 2, true>", "down_proj_m1": "w4a4_gemv_kernel<1, 2, true>",
