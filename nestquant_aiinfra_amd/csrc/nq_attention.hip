@@ -90,8 +90,14 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     __shared__ float acc_lds[kAttnThreads / 16][kBlocks][G * 8];   // one entry per 16-lane row
 
     const int tid = threadIdx.x;
-    const int chunk = blockIdx.x;
-    const int row = blockIdx.y / a.kv_heads, g = blockIdx.y % a.kv_heads;
+    // Workgroups go to the eight XCDs in turn by their linear index, and every XCD has its own L2.
+    // A page stores the blocks of all KV heads of a token side by side, so the workgroups of one
+    // (row, chunk) -- one per KV head -- fetch the same cache lines: they are numbered so that they
+    // share an XCD and follow each other there (index = 8 * (kv_heads * (pair / 8) + head) + pair % 8).
+    const int place = blockIdx.x >> 3, pair = (place / a.kv_heads) * 8 + (blockIdx.x & 7);
+    const int g = place % a.kv_heads;
+    const int chunk = pair % (a.chunks + 1), row = pair / (a.chunks + 1);
+    if (row >= a.batch) return;                          // padding of the last group of eight pairs
     const bool is_hot = chunk == a.chunks;
     int slot = a.slot_ids[row];
     slot = slot < 0 ? 0 : (slot >= a.slots ? a.slots - 1 : slot);
@@ -492,7 +498,8 @@ extern "C" int nq_nqkv_attention_decode(
     a.part_acc = a.part_sum + heads_total * parts;
 
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid((unsigned)parts, (unsigned)(batch * kv_heads));
+    const size_t pairs = parts * (size_t)batch;                    // (row, chunk) pairs, padded to whole groups of eight
+    const dim3 grid((unsigned)((pairs + 7) / 8 * 8 * kv_heads));
 #define NQ_LAUNCH_STAGE1(GROUP)                                                                                   \
     switch (pages_per_chunk_for(batch, max_pages)) {                                                              \
         case 4: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 4>), grid, dim3(nq::kAttnThreads), 0, s, a); break;  \

@@ -65,10 +65,17 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     __shared__ __attribute__((aligned(16))) uint16_t v_page[2][2][D][P];         // transposed: [dim][token]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int row = blockIdx.y / a.kv_heads, g = blockIdx.y % a.kv_heads;
+    // The workgroups of one (row, token tile) -- one per KV head -- read the same cache lines of every
+    // page (a page keeps the blocks of all KV heads of a token side by side): they are numbered so
+    // that they share an XCD, hence an L2 (index = 8 * (kv_heads * (pair / 8) + head) + pair % 8;
+    // workgroups go to the eight XCDs in turn).
+    const int tiles = (a.tokens + kTileTokens - 1) / kTileTokens;
+    const int place = blockIdx.x >> 3, pair = (place / a.kv_heads) * 8 + (blockIdx.x & 7);
+    const int g = place % a.kv_heads, tile = pair % tiles, row = pair / tiles;
+    if (row >= a.batch) return;                          // padding of the last group of eight pairs
     const int vec = 16 * wave + (lane & 15);             // this lane's query vector (column of S^T and O^T)
     const int quarter = lane >> 4;                       // which 4 tokens / 4 dims of a 16-row tile the lane holds
-    const int t = blockIdx.x * kTileTokens + vec / G;    // token of the query vector inside the chunk
+    const int t = tile * kTileTokens + vec / G;          // token of the query vector inside the chunk
     const int head = g * G + vec % G;
     const int64_t q_at = (((int64_t)row * a.tokens + t) * a.q_heads + head) * D;
 
@@ -86,7 +93,7 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     const int page_count = a.page_counts[slot], last_len = a.last_page_lens[slot], hot_len = a.hot_lengths[slot];
 
     // last position any vector of this tile looks at (uniform over the workgroup)
-    const int tile_first = blockIdx.x * kTileTokens;
+    const int tile_first = tile * kTileTokens;
     const int tile_last_token = (tile_first + kTileTokens < count ? tile_first + kTileTokens : count) - 1;
     const int pages_needed = tile_last_token >= tile_first ? (start + tile_last_token) / P + 1 : 0;
 
@@ -301,7 +308,8 @@ extern "C" int nq_nqkv_attention_prefill(
     a.batch = batch; a.tokens = tokens; a.uniform_count = uniform_count; a.slots = slots; a.max_pages = max_pages;
     a.q_heads = q_heads; a.kv_heads = kv_heads; a.scale = scale;
     const int tile_tokens = 128 / group;
-    const dim3 grid((unsigned)((tokens + tile_tokens - 1) / tile_tokens), (unsigned)(batch * kv_heads));
+    const int64_t pairs = (int64_t)((tokens + tile_tokens - 1) / tile_tokens) * batch;     // (row, token tile), padded to eights
+    const dim3 grid((unsigned)((pairs + 7) / 8 * 8 * kv_heads));
     hipStream_t s = (hipStream_t)stream;
     switch (group) {
         case 1: hipLaunchKernelGGL((nq::attention_prefill_kernel<64, 16, 1>), grid, dim3(nq::kPrefillThreads), 0, s, a); break;
