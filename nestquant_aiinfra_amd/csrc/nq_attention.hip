@@ -89,6 +89,10 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     __shared__ float chunk_max[G], chunk_sum[G];
     __shared__ float acc_lds[kAttnThreads / 16][kBlocks][G * 8];   // one entry per 16-lane row
 
+    // The part of (block, row) that does not reach the bank index through the address, as an XOR mask
+    // for the G * 8 columns of acc_lds: the block bits that overflow 32 banks, and two row bits.
+    constexpr int kOverflowShift = G >= 4 ? 0 : (G == 2 ? 1 : 2);
+    auto acc_swizzle = [](int block, int row16) { return 4 * (block >> kOverflowShift) + (row16 & 3); };
     const int tid = threadIdx.x;
     // Workgroups go to the eight XCDs in turn by their linear index, and every XCD has its own L2.
     // A page stores the blocks of all KV heads of a token side by side, so the workgroups of one
@@ -342,14 +346,16 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const float v = acc[h][j] + dpp_rotate8(acc[h][j]);
-            if ((tid & 8) == 0) acc_lds[tid >> 4][tid & 7][h * 8 + j] = v;
+            // column swizzled by (block, row): the 32 lanes of a wavefront that store one (h, j) hit 32
+            // banks (unswizzled they all met in one: blocks lie G * 32 bytes apart, rows G * 256)
+            if ((tid & 8) == 0) acc_lds[tid >> 4][tid & 7][(h * 8 + j) ^ acc_swizzle(tid & 7, tid >> 4)] = v;
         }
     __syncthreads();
     for (int o = tid; o < G * D; o += kAttnThreads) {
         const int h = o / D, d = o % D;
-        float total = acc_lds[0][d / 8][h * 8 + d % 8];
+        float total = acc_lds[0][d / 8][(h * 8 + d % 8) ^ acc_swizzle(d / 8, 0)];
 #pragma unroll
-        for (int w = 1; w < kAttnThreads / 16; w++) total = total + acc_lds[w][d / 8][h * 8 + d % 8];
+        for (int w = 1; w < kAttnThreads / 16; w++) total = total + acc_lds[w][d / 8][(h * 8 + d % 8) ^ acc_swizzle(d / 8, w)];
         a.part_acc[(part + (int64_t)h * (a.chunks + 1)) * D + d] = total;
     }
     if (tid < G) {
