@@ -59,10 +59,13 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
     const float wscale = kResolved ? unit * kResolvedUnit : unit;
     const float wbeta[4] = {w_betas[0], w_betas[1], w_betas[2], w_betas[3]};
     const int64_t dec_first = (int64_t)dec_n * blocks_per_row + (k_begin >> 3) + dec_kb;
-    // LDS entry of (K-step kk, fragment lane f): [kk][f ^ (4 kk)] -- the rotation spreads the
-    // 16 blocks a channel's lanes write over the banks, and is a permutation for the readers
+    // LDS entry of (K-step kk, fragment lane f): [kk][f ^ (2 (kk % 4) + f / 32)].  Eight neighbouring
+    // decode lanes (one channel, blocks 8 i .. 8 i + 7, i.e. four K-steps x the two halves of the
+    // fragment) then write eight different 16-byte bank groups, and for the readers the mask is a
+    // permutation of the 64 fragment lanes of a K-step (it leaves f / 32 alone).
     const int dec_kk = dec_kb >> 1;
-    const int dec_entry = (((tid >> 4) ^ (dec_kk << 2)) & 31) + 32 * (dec_kb & 1);
+    const int dec_f = (tid >> 4) + 32 * (dec_kb & 1);
+    const int dec_entry = dec_f ^ (2 * (dec_kk & 3) + (dec_kb & 1));
     uint4 *dec_slot0 = &b_tile[0][dec_kk][dec_entry];
     uint4 *dec_slot1 = &b_tile[1][dec_kk][dec_entry];
 
@@ -115,7 +118,7 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
         if (s > 0 && multiplies) {
 #pragma unroll
             for (int kk = 0; kk < kGemmBK / 16; kk++) {
-                const bf16x8 b = __builtin_bit_cast(bf16x8, b_tile[(s - 1) & 1][kk][lane ^ (kk << 2)]);
+                const bf16x8 b = __builtin_bit_cast(bf16x8, b_tile[(s - 1) & 1][kk][lane ^ (2 * (kk & 3) + (lane >> 5))]);
 #pragma unroll
                 for (int t = 0; t < TILES; t++)
                     acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[t][kk]), b, acc[t], 0, 0, 0);
