@@ -100,6 +100,29 @@ __device__ __forceinline__ float lane_xor(float v) {
 template <int kXor, int kDtype>
 __device__ __forceinline__ void lane_stage(float (&v)[8], int lane) {
     const bool upper = (lane & kXor) != 0;
+    if (kXor == 16 || kXor == 32) {
+        // v_permlane{16,32}_swap exchanges the odd rows (of 16 / 32 lanes) of its first operand with
+        // the even rows of its second: given the value twice, the first result holds the left
+        // operand of the lane's butterfly and the second the right one, in both partner lanes
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int bits = __builtin_bit_cast(int, v[j]);
+            float left, right;
+            if (kXor == 16) {
+                const auto pair = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+                left = __builtin_bit_cast(float, (int)pair[0]);
+                right = __builtin_bit_cast(float, (int)pair[1]);
+            } else {
+                const auto pair = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+                left = __builtin_bit_cast(float, (int)pair[0]);
+                right = __builtin_bit_cast(float, (int)pair[1]);
+            }
+            v[j] = upper ? left - right : left + right;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) round_pair<kDtype>(v[j], v[j + 1]);
+        return;
+    }
     float other[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) other[j] = lane_xor<kXor>(v[j]);
