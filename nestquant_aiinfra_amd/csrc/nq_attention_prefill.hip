@@ -62,7 +62,11 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     constexpr int kTileTokens = 128 / G;                 // query tokens per workgroup
     constexpr int kKeyRow = D + 8;                       // BF16 elements per key row: 144 bytes, conflict-free 16-byte reads
     __shared__ __attribute__((aligned(16))) uint16_t k_page[2][2][P][kKeyRow];   // [buffer][page of the pair][token][dim]
-    __shared__ __attribute__((aligned(16))) uint16_t v_page[2][2][D][P];         // transposed: [dim][token]
+    // transposed: [dim][token], rows of 40 bytes, and the rows of dims 32..63 keep their two halves of
+    // eight tokens swapped: the 64 lanes of a decode wavefront (8 tokens x 8 blocks) that store one
+    // value each then hit 16 banks instead of 4, and the 8-byte fragment reads stay aligned
+    constexpr int kValueRow = P + 4;
+    __shared__ __attribute__((aligned(16))) uint16_t v_page[2][2][D][kValueRow];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // The workgroups of one (row, token tile) -- one per KV head -- read the same cache lines of every
@@ -151,8 +155,8 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
             const uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                v_page[buf][half][dec_blk * 8 + 2 * j][dec_token] = (uint16_t)(w[j] & 0xffffu);
-                v_page[buf][half][dec_blk * 8 + 2 * j + 1][dec_token] = (uint16_t)(w[j] >> 16);
+                v_page[buf][half][dec_blk * 8 + 2 * j][dec_token ^ (8 * (dec_blk >> 2))] = (uint16_t)(w[j] & 0xffffu);
+                v_page[buf][half][dec_blk * 8 + 2 * j + 1][dec_token ^ (8 * (dec_blk >> 2))] = (uint16_t)(w[j] >> 16);
             }
         } else {
             *reinterpret_cast<uint4 *>(&k_page[buf][half][dec_token][dec_blk * 8]) = packed;
@@ -209,8 +213,9 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
         const bf16x8 p_frag = __builtin_bit_cast(bf16x8, p_bits);
 #pragma unroll
         for (int tile = 0; tile < 4; tile++) {
-            const uint2 v0 = *reinterpret_cast<const uint2 *>(&v_page[buf][0][16 * tile + (lane & 15)][4 * quarter]);
-            const uint2 v1 = *reinterpret_cast<const uint2 *>(&v_page[buf][1][16 * tile + (lane & 15)][4 * quarter]);
+            const int column = (4 * quarter) ^ (8 * (tile >> 1));
+            const uint2 v0 = *reinterpret_cast<const uint2 *>(&v_page[buf][0][16 * tile + (lane & 15)][column]);
+            const uint2 v1 = *reinterpret_cast<const uint2 *>(&v_page[buf][1][16 * tile + (lane & 15)][column]);
 #pragma unroll
             for (int r = 0; r < 4; r++) o[tile][r] = o[tile][r] * keep;
             o[tile] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, make_uint4(v0.x, v0.y, v1.x, v1.y)),
