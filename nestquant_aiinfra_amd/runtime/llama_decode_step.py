@@ -82,13 +82,13 @@ class FusedLlamaDecodeStep:
         hidden = inner.embed_tokens.weight.shape[1]
         _require(hidden & (hidden - 1) == 0 and hidden % 32 == 0, "hidden size is not a power of two")
         self.hidden = hidden
-        self._rope_tables: tuple[torch.Tensor, torch.Tensor] | None = None
+        self._rope_tables: torch.Tensor | None = None
 
     def _rope(self, embedded: torch.Tensor, positions: torch.Tensor, *, padded: bool = False
               ) -> tuple[torch.Tensor, torch.Tensor]:
         """BF16 (cos, sin) [positions.numel(), head_dim] of the model's rotary embedding.  For
         embeddings that depend on the position alone the module is evaluated once, over every
-        position the cache can hold, and a step gathers its rows (two launches instead of the
+        position the cache can hold, and a step gathers its rows (one launch instead of the
         module's dozen)."""
         rotary = self.inner.rotary_emb
         if getattr(rotary, "rope_type", "default") not in ("default", "llama3", "linear"):
@@ -98,11 +98,12 @@ class FusedLlamaDecodeStep:
         if self._rope_tables is None:
             every = torch.arange(self.cache.max_cache_len, device=embedded.device)[None, :]
             cos, sin = rotary(embedded[:1, :1], every)
-            self._rope_tables = (cos[0].to(torch.bfloat16).contiguous(), sin[0].to(torch.bfloat16).contiguous())
+            self._rope_tables = torch.stack((cos[0], sin[0])).to(torch.bfloat16).contiguous()     # [2, positions, dim]
         index = positions.reshape(-1)
         if padded:                      # positions of padding tokens may lie past the cache's last one
-            index = index.clamp(max=self._rope_tables[0].shape[0] - 1)
-        return self._rope_tables[0].index_select(0, index), self._rope_tables[1].index_select(0, index)
+            index = index.clamp(max=self._rope_tables.shape[1] - 1)
+        both = self._rope_tables.index_select(1, index)
+        return both[0], both[1]
 
     @staticmethod
     def _prepared(linear, device) -> PreparedNQRTLinear:
