@@ -405,6 +405,18 @@ int nq_greedy_sample(const void *logits_dev, int logits_dtype, int rows, int64_t
 
 size_t nq_greedy_sample_workspace_bytes(int rows);
 
+/*
+ * out[r, j] = sum_k act[r, k] weight[j, k] for a few rows (rows in [1, 16], K 2048 or 4096) of a
+ * BF16 activation [rows, K] against a BF16 weight [N, K], both dense row-major and 16-byte
+ * aligned; FP32 accumulation, BF16 out [rows, N].  One stream over the weight on the matrix
+ * cores, for the LM head of a decode step where a library GEMM of this shape leaves a third of
+ * the memory rate unused.  No bias.
+ * Replaces: the lm_head call inside the model forward of a decode step
+ * (nestquant/runtime/nqkv_batched_runner.py:162-169).
+ */
+int nq_bf16_rows_linear(const void *act_bf16_dev, const void *weight_bf16_dev, int rows, int64_t k, int64_t n,
+                        void *out_bf16_dev, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

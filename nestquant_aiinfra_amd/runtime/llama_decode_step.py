@@ -18,6 +18,8 @@ per layer:
     SiLU(gate) * up + Hadamard + A4 encode             nq_fused_input_stage (mode 2)
     down_proj                                          nq_w4a4_gemv
 
+and the LM head of up to 16 rows as one stream over its BF16 weight (nq_bf16_rows_linear).
+
 FusedLlamaPrefillStep runs a prompt (or a chunk of one) the same way over [rows * tokens]
 activation rows: the input stages and linears as above (the linears on the matrix cores), RoPE
 and Hadamard of queries and keys in one launch each, the KV writer, and the attention the
@@ -33,7 +35,8 @@ import torch
 import torch.nn.functional as F
 
 from .nqkv import attention_output_stage, launch_nqkv_decode_attention, nqkv_prefill_attention
-from .w4a4_linear import (MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, _gemm, _gemv, fused_input_stage,
+from .w4a4_linear import (MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, _gemm, _gemv, bf16_rows_linear,
+                          can_use_bf16_rows_linear, fused_input_stage,
                           linear_packed_w4a4_gemv_grouped, quantize_activation_cuda, rope_hadamard_cuda)
 
 
@@ -166,7 +169,15 @@ class FusedLlamaDecodeStep:
             delta = self._linear(activation, down_w)
         _, _, normed = fused_input_stage(delta, mode="rmsnorm", residual=residual, norm_weight=inner.norm.weight,
                                          eps=inner.norm.variance_epsilon, encode=False, want_staged=True)
-        return self.model.lm_head(normed.view(rows, 1, self.hidden))
+        return self._lm_head(normed.view(rows, self.hidden)).view(rows, 1, -1)
+
+    def _lm_head(self, normed: torch.Tensor) -> torch.Tensor:
+        """Logits of a few rows: one stream over the BF16 head weight when it has the shape the
+        stream kernel takes, the module's own linear otherwise."""
+        head = self.model.lm_head
+        if getattr(head, "bias", None) is None and can_use_bf16_rows_linear(normed, head.weight):
+            return bf16_rows_linear(normed, head.weight)
+        return head(normed)
 
 
 class FusedLlamaPrefillStep(FusedLlamaDecodeStep):

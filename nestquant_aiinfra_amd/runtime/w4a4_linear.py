@@ -552,6 +552,7 @@ LIBRARY_GEMM_ROWS = 288
 # up to this many rows a linear over resolved weights (K a multiple of 128) takes the decode GEMV,
 # which from five rows on multiplies on the matrix cores
 MATRIX_CORE_GEMV_ROWS = 16
+BF16_ROWS_LINEAR_MAX_ROWS = 16
 
 
 def decode_weight_bf16(weight: PreparedNQRTLinear) -> torch.Tensor:
@@ -566,6 +567,29 @@ def decode_weight_bf16(weight: PreparedNQRTLinear) -> torch.Tensor:
         weight.resolved_tails.data_ptr() if resolved else None,
         weight.row_norms.data_ptr(), weight.beta_table.data_ptr(), n, k, 0, int(weight.record.dither_seed),
         out.data_ptr(), _native.stream_handle(device)))
+    return out
+
+
+def can_use_bf16_rows_linear(rows: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether `bf16_rows_linear` takes this activation and weight."""
+    return (rows.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and rows.device.type == "cuda"
+            and weight.device == rows.device and rows.ndim == 2 and weight.ndim == 2
+            and 1 <= rows.shape[0] <= BF16_ROWS_LINEAR_MAX_ROWS and rows.shape[1] == weight.shape[1]
+            and weight.shape[1] in (2048, 4096) and rows.is_contiguous() and weight.is_contiguous()
+            and rows.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def bf16_rows_linear(rows: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """`rows @ weight.T` for at most 16 BF16 rows against a BF16 [N, K] weight (K 2048 or 4096),
+    FP32 accumulation, BF16 out: the LM head of a decode step
+    (nestquant/runtime/nqkv_batched_runner.py:162-169) as one stream over the weight."""
+    if not can_use_bf16_rows_linear(rows, weight):
+        raise ValueError("bf16_rows_linear takes contiguous BF16 [rows <= 16, K] and [N, K] on one GPU, K 2048 or 4096")
+    device = _native.require_cuda(rows)
+    out = torch.empty((rows.shape[0], weight.shape[0]), dtype=torch.bfloat16, device=device)
+    _native.check(_native.library().nq_bf16_rows_linear(
+        rows.data_ptr(), weight.data_ptr(), rows.shape[0], rows.shape[1], weight.shape[0], out.data_ptr(),
+        _native.stream_handle(device)))
     return out
 
 

@@ -60,6 +60,13 @@ def test_host_side_validation_needs_no_gpu():
     assert status == _native.NQ_ERR_SHAPE and b"row_stride" in lib.nq_last_error()
     status = lib.nq_greedy_sample(None, 1, 8, 100, 100, None, None, None, None, 0, None, None, 0, None)
     assert status == _native.NQ_ERR_ARGUMENT and b"null pointer" in lib.nq_last_error()
+    # the LM-head stream: row count, K, then pointers
+    status = lib.nq_bf16_rows_linear(None, None, 17, 2048, 128256, None, None)
+    assert status == _native.NQ_ERR_SHAPE and b"outside [1, 16]" in lib.nq_last_error()
+    status = lib.nq_bf16_rows_linear(None, None, 8, 1024, 128256, None, None)
+    assert status == _native.NQ_ERR_SHAPE and b"not 2048 or 4096" in lib.nq_last_error()
+    status = lib.nq_bf16_rows_linear(None, None, 8, 2048, 128256, None, None)
+    assert status == _native.NQ_ERR_ARGUMENT and b"null pointer" in lib.nq_last_error()
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -461,3 +461,29 @@ def test_decode_refuses_to_run_past_the_cache_length(tmp_path):
     with pytest.raises(RuntimeError, match="max_cache_len"):
         runner.prefill_slots(ids[:, :1], slots=[1], lengths=[1])
     assert runner.cache.manager.total_tokens(1) == 48
+
+
+def test_bf16_rows_linear_against_float64():
+    """The LM-head stream kernel: small-integer operands make every sum exact, so the result must
+    equal the float64 product bit for bit whatever the order of accumulation (a wrong row, token
+    or k pairing cannot pass); Gaussian operands must agree with the float64 product to one BF16
+    rounding (2**-8 relative) plus the FP32 accumulation error.  Ragged N, every row count class,
+    both K."""
+    from nestquant_aiinfra_amd.runtime.w4a4_linear import bf16_rows_linear, can_use_bf16_rows_linear
+    g = torch.Generator().manual_seed(4242)
+    for rows, n, k in ((1, 128256, 2048), (8, 4099, 2048), (16, 1000, 4096), (5, 77, 2048), (13, 16, 4096), (3, 1, 2048)):
+        act = torch.randint(-3, 4, (rows, k), generator=g).to(torch.bfloat16).cuda()
+        weight = torch.randint(-3, 4, (n, k), generator=g).to(torch.bfloat16).cuda()
+        assert can_use_bf16_rows_linear(act, weight)
+        want = (act.double() @ weight.double().T).to(torch.bfloat16)
+        assert torch.equal(bf16_rows_linear(act, weight), want), (rows, n, k)
+        act = torch.randn((rows, k), generator=g).to(torch.bfloat16).cuda()
+        weight = (0.05 * torch.randn((n, k), generator=g)).to(torch.bfloat16).cuda()
+        exact = act.double() @ weight.double().T
+        got = bf16_rows_linear(act, weight).double()
+        bound = exact.abs() * 2.0 ** -8 + (act.double().abs() @ weight.double().abs().T) * k * 2.0 ** -24
+        assert bool(((got - exact).abs() <= bound).all()), (rows, n, k, float(((got - exact).abs() / bound).max()))
+    for bad_rows, bad_weight in ((torch.zeros((17, 2048)), torch.zeros((32, 2048))), (torch.zeros((4, 1024)), torch.zeros((32, 1024)))):
+        assert not can_use_bf16_rows_linear(bad_rows.to(torch.bfloat16).cuda(), bad_weight.to(torch.bfloat16).cuda())
+        with pytest.raises(ValueError):
+            bf16_rows_linear(bad_rows.to(torch.bfloat16).cuda(), bad_weight.to(torch.bfloat16).cuda())
