@@ -186,12 +186,18 @@ class FusedLlamaPrefillStep(FusedLlamaDecodeStep):
     as FusedLlamaDecodeStep."""
 
     @torch.inference_mode()
-    def __call__(self, tokens: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+    def __call__(self, tokens: torch.Tensor, positions: torch.Tensor, *,
+                 keep: torch.Tensor | None = None) -> torch.Tensor:
+        """`keep` (int64 [rows], optional): the one token of every row whose logits are wanted;
+        the final norm and the LM head then run on those rows only and the result is
+        [rows, 1, vocab]."""
         cache, inner = self.cache, self.inner
         manager = cache.manager
         rows, width = tokens.shape
         if positions.shape != (rows, width) or rows != cache._rows:
             raise ValueError("the fused prefill step takes [rows, width] tokens and positions for the rows in flight")
+        if keep is not None and (keep.shape != (rows,) or keep.dtype != torch.int64 or keep.device != tokens.device):
+            raise ValueError("keep holds one int64 token index per row, on the tokens' device")
         device = tokens.device
         embedded = inner.embed_tokens(tokens)                               # [rows, width, hidden]
         if embedded.dtype != torch.bfloat16:
@@ -230,6 +236,11 @@ class FusedLlamaPrefillStep(FusedLlamaDecodeStep):
             gate, up = self._linears(activation, [gate_w, up_w])
             activation, _, _ = fused_input_stage(up, mode="swiglu", gate=gate, beta_table=table)
             delta = self._linear(activation, down_w)
+        if keep is not None:
+            flat = torch.arange(rows, device=device) * width + keep
+            delta, residual = delta.index_select(0, flat), residual.index_select(0, flat)
         _, _, normed = fused_input_stage(delta, mode="rmsnorm", residual=residual, norm_weight=inner.norm.weight,
                                          eps=inner.norm.variance_epsilon, encode=False, want_staged=True)
+        if keep is not None:
+            return self._lm_head(normed.view(rows, self.hidden)).view(rows, 1, -1)
         return self.model.lm_head(normed.view(rows, width, self.hidden))

@@ -367,12 +367,16 @@ class BatchedNQKVLlamaRunner:
     # -- prefill -------------------------------------------------------------------------------
     @torch.inference_mode()
     def prefill_slots(self, input_ids: torch.Tensor, *, slots: Sequence[int], lengths: Sequence[int],
-                      positions: torch.Tensor | None = None) -> torch.Tensor:
+                      positions: torch.Tensor | None = None, last_token_logits: bool = False) -> torch.Tensor:
         """Prefill `slots[i]` with the first `lengths[i]` tokens of row i of input_ids
-        [rows, width] (right padded).  New slots are registered.  Returns logits [rows, width, vocab]."""
+        [rows, width] (right padded).  New slots are registered.  Returns logits [rows, width, vocab],
+        or, with `last_token_logits`, only those of every row's last token, [rows, 1, vocab]
+        (what sampling the first new token needs: the LM head then runs on `rows` vectors)."""
         rows, width = input_ids.shape
         if len(slots) != rows or len(lengths) != rows:
             raise ValueError("slots and lengths must have one entry per row")
+        if last_token_logits and not all(1 <= int(length) <= width for length in lengths):
+            raise ValueError("last_token_logits needs at least one token in every row")
         for slot in slots:
             if self.cache.manager.sequence_id(slot) is None:
                 self._generation[slot] += 1
@@ -382,9 +386,14 @@ class BatchedNQKVLlamaRunner:
             positions = starts[:, None] + torch.arange(width, device=self.device)[None, :]
         self._decode_state = None
         self.cache.set_batch_state(slot_ids=slots, counts=lengths)
+        keep = None
+        if last_token_logits:
+            keep = torch.tensor([int(length) - 1 for length in lengths], dtype=torch.long, device=self.device)
         if self.fused_prefill is not None:
-            return self.fused_prefill(input_ids, positions)
+            return self.fused_prefill(input_ids, positions, keep=keep)
         output = self.model(input_ids=input_ids, position_ids=positions, past_key_values=self.cache, use_cache=True)
+        if keep is not None:
+            return output.logits[torch.arange(rows, device=self.device), keep].unsqueeze(1)
         return output.logits
 
     def release_slots(self, slots: Sequence[int]) -> None:

@@ -487,3 +487,53 @@ def test_bf16_rows_linear_against_float64():
         assert not can_use_bf16_rows_linear(bad_rows.to(torch.bfloat16).cuda(), bad_weight.to(torch.bfloat16).cuda())
         with pytest.raises(ValueError):
             bf16_rows_linear(bad_rows.to(torch.bfloat16).cuda(), bad_weight.to(torch.bfloat16).cuda())
+
+
+def test_last_token_logits_and_the_lm_head_stream(tmp_path, monkeypatch):
+    """A model as wide as the stream kernel's K (2048): `last_token_logits` returns the logits of
+    every row's last prompt token (against the full prefill of the same prompt: the same hidden
+    state, the head through the library there and through the stream kernel here, so equal to a
+    BF16 rounding), and a decode step's logits are the same through either head."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
+    from nestquant_aiinfra_amd.runtime import llama_decode_step
+
+    torch.manual_seed(6001)
+    config = LlamaConfig(hidden_size=2048, intermediate_size=1024, num_hidden_layers=1, num_attention_heads=32,
+                         num_key_value_heads=8, head_dim=64, vocab_size=1000, max_position_embeddings=256,
+                         rope_theta=500000.0, tie_word_embeddings=True)
+    model = LlamaForCausalLM(config).to(torch.bfloat16).cuda().eval()
+    path = tmp_path / "wide.nqmc"
+    asm.write_w4_checkpoint(model, path)
+    runner = asm.build_w4a4kv4_runner(model, path, capacity=2, max_cache_len=96)
+    assert runner.fused_step is not None and runner.fused_prefill is not None
+    calls = []
+    stream_kernel = llama_decode_step.bf16_rows_linear
+    monkeypatch.setattr(llama_decode_step, "bf16_rows_linear", lambda *a: calls.append(1) or stream_kernel(*a))
+
+    ids = torch.randint(0, 1000, (2, 20), generator=torch.Generator().manual_seed(6002)).cuda()
+    lengths = [20, 9]
+    full = runner.prefill_slots(ids, slots=[0, 1], lengths=lengths).float()
+    assert not calls                                   # all positions: the library's GEMM
+    runner.release_slots([0, 1])
+    last = runner.prefill_slots(ids, slots=[0, 1], lengths=lengths, last_token_logits=True).float()
+    assert len(calls) == 1 and last.shape == (2, 1, 1000)
+    for row, length in enumerate(lengths):
+        want = full[row, length - 1]
+        assert float((last[row, 0] - want).abs().max()) <= 2.0 ** -7 * float(want.abs().max())
+    with pytest.raises(ValueError, match="at least one token"):
+        runner.prefill_slots(ids, slots=[0, 1], lengths=[0, 3], last_token_logits=True)
+
+    # the same prompt in both slots: slot 0 decodes through the stream kernel, slot 1 through the library
+    runner.release_slots([0, 1])
+    same = ids[:1].repeat(2, 1)
+    runner.prefill_slots(same, slots=[0, 1], lengths=[20, 20], last_token_logits=True)
+    token, position = torch.tensor([[7]], device="cuda"), torch.tensor([[20]], device="cuda")
+    calls.clear()
+    streamed = runner.decode_eager(token, slots=[0], positions=position).float()
+    assert len(calls) == 1
+    monkeypatch.setattr(llama_decode_step, "can_use_bf16_rows_linear", lambda *a: False)
+    library = runner.decode_eager(token, slots=[1], positions=position).float()
+    assert len(calls) == 1
+    assert float((streamed - library).abs().max()) <= 2.0 ** -7 * float(library.abs().max())
+    assert int(streamed.argmax()) == int(library.argmax())
