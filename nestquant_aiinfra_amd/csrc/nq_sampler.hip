@@ -29,7 +29,7 @@ __device__ __forceinline__ float logit_as_float<uint16_t>(uint16_t raw) { return
 template <>
 __device__ __forceinline__ float logit_as_float<_Float16>(_Float16 raw) { return (float)raw; }
 
-// Scratch of one call: per row a ticket counter and kSamplerSplits partial results.
+// Scratch of one call: per row a ticket counter and up to kSamplerSplits partial results.
 constexpr int kSamplerSplits = 32;
 
 struct SamplerScratch {
@@ -40,7 +40,7 @@ struct SamplerScratch {
 
 __host__ __device__ inline size_t sampler_ticket_bytes(int rows) { return ((size_t)rows * 4 + 15) / 16 * 16; }
 
-// grid (kSamplerSplits, rows) x 256 lanes: every workgroup scans one stretch of a row (one
+// grid (stretches <= kSamplerSplits, rows) x 256 lanes: every workgroup scans one stretch of a row (one
 // compute unit alone reads a 256 KB row far too slowly), publishes its best and takes a ticket;
 // the workgroup that draws the last ticket of a row folds the row's partial results and writes
 // the outputs.  Nothing waits for anything: the ticket counter returns to zero for the next call.
@@ -52,14 +52,14 @@ greedy_sample_kernel(const T *__restrict__ logits, int64_t vocab, int64_t row_st
                      int rows, int32_t *__restrict__ cursors, int vector_loads, SamplerScratch scratch) {
     constexpr int kPer = 16 / sizeof(T);
     __shared__ Best wave_best[4];
-    const int split = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
+    const int split = blockIdx.x, splits = gridDim.x, row = blockIdx.y, tid = threadIdx.x;
     const T *line = logits + (int64_t)row * row_stride;
     Best best{-__builtin_inff(), vocab};
     if (vector_loads) {
         // a stretch of whole 16-byte vectors, up to four loads in flight per lane
         constexpr int kDepth = 4;
         const int64_t vectors = vocab / kPer;
-        const int64_t stretch = (vectors + kSamplerSplits - 1) / kSamplerSplits;
+        const int64_t stretch = (vectors + splits - 1) / splits;
         const int64_t begin = split * stretch, end = begin + stretch < vectors ? begin + stretch : vectors;
         for (int64_t v0 = begin + tid; v0 < end; v0 += (int64_t)kDepth * blockDim.x) {
             uint4 raw[kDepth];
@@ -87,14 +87,14 @@ greedy_sample_kernel(const T *__restrict__ logits, int64_t vocab, int64_t row_st
                 if (beats(top, v * kPer + at, best)) best = Best{top, v * kPer + at};
             }
         }
-        if (split == kSamplerSplits - 1) {
+        if (split == splits - 1) {
             for (int64_t i = vectors * kPer + tid; i < vocab; i += blockDim.x) {
                 const float value = logit_as_float<T>(line[i]);
                 if (beats(value, i, best)) best = Best{value, i};
             }
         }
     } else {
-        const int64_t stretch = (vocab + kSamplerSplits - 1) / kSamplerSplits;
+        const int64_t stretch = (vocab + splits - 1) / splits;
         const int64_t begin = split * stretch, end = begin + stretch < vocab ? begin + stretch : vocab;
         for (int64_t i = begin + tid; i < end; i += blockDim.x) {
             const float value = logit_as_float<T>(line[i]);
@@ -118,14 +118,15 @@ greedy_sample_kernel(const T *__restrict__ logits, int64_t vocab, int64_t row_st
         const int64_t slot = (int64_t)row * kSamplerSplits + split;
         __hip_atomic_store(scratch.part_value + slot, best.value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(scratch.part_index + slot, best.index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __threadfence();
+        // the release half of the ticket orders the two stores before it
         const int32_t ticket = __hip_atomic_fetch_add(scratch.tickets + row, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        last = ticket == kSamplerSplits - 1;
+        last = ticket == splits - 1;
     }
     last = __shfl(last, 0, 64);
     if (!last) return;
     __threadfence();
-    const int64_t slot = (int64_t)row * kSamplerSplits + (tid & (kSamplerSplits - 1));
+    const int from = tid & (kSamplerSplits - 1);
+    const int64_t slot = (int64_t)row * kSamplerSplits + (from < splits ? from : 0);
     best.value = __hip_atomic_load(scratch.part_value + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     best.index = __hip_atomic_load(scratch.part_index + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
@@ -172,11 +173,15 @@ extern "C" int nq_greedy_sample(const void *logits_dev, int logits_dtype, int ro
     scratch.tickets = reinterpret_cast<int32_t *>(workspace_dev);
     scratch.part_index = reinterpret_cast<int64_t *>(reinterpret_cast<char *>(workspace_dev) + nq::sampler_ticket_bytes(rows));
     scratch.part_value = reinterpret_cast<float *>(scratch.part_index + (size_t)rows * nq::kSamplerSplits);
+    // about 128 workgroups in all: every one pays a release of its cache at the ticket, which is
+    // what a launch of many rows spends its time on (16 rows: 12.8 us with 8 stretches, 16.7 with 32)
+    int splits = 128 / rows;
+    splits = splits < 8 ? 8 : (splits > nq::kSamplerSplits ? nq::kSamplerSplits : splits);
     const hipStream_t s = (hipStream_t)stream;
 #define NQ_LAUNCH_SAMPLER(T)                                                                                   \
     do {                                                                                                       \
         const int vector_loads = nq::aligned(logits_dev, 16) && (row_stride * sizeof(T)) % 16 == 0;            \
-        hipLaunchKernelGGL(nq::greedy_sample_kernel<T>, dim3(nq::kSamplerSplits, (unsigned)rows), dim3(256), 0, s, \
+        hipLaunchKernelGGL(nq::greedy_sample_kernel<T>, dim3((unsigned)splits, (unsigned)rows), dim3(256), 0, s,   \
                            reinterpret_cast<const T *>(logits_dev), vocab, row_stride, active_mask_dev,        \
                            tokens_dev, positions_dev, history_dev, history_steps, rows, cursors_dev,           \
                            vector_loads, scratch);                                                             \
