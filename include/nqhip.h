@@ -281,6 +281,22 @@ int nq_nqkv_advance(const int32_t *slot_ids_dev, const uint8_t *active_mask_dev,
                     int32_t *hot_lengths_dev, void *stream);
 
 /*
+ * The head of a decode step in one launch: nq_nqkv_advance with a count of one token per row,
+ * embedded[r] = embedding[tokens[r]] (BF16 rows of `hidden` values; a token outside [0, vocab)
+ * embeds as zero) and the rotary embedding's rows of positions[r] (clamped to the table):
+ * rotary is BF16 [2, rotary_positions, head_dim] (cos rows, then sin rows), rotary_rows BF16
+ * [2, batch, head_dim].  Replaces: embed_tokens and LlamaRotaryEmbedding at the top of the model
+ * forward of a decode step (nestquant/runtime/nqkv_batched_runner.py:162-169) together with the
+ * step's metadata update (nqkv_graph_writer.py:15-80).
+ */
+int nq_decode_step_begin(const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch, int slots,
+                         int page_size, int max_tokens, int32_t *sequence_lengths_dev, int32_t *page_counts_dev,
+                         int32_t *last_page_lens_dev, int32_t *hot_lengths_dev, const int64_t *tokens_dev,
+                         const void *embedding_bf16_dev, int64_t vocab, int hidden, void *embedded_bf16_dev,
+                         const int64_t *positions_dev, const void *rotary_bf16_dev, int64_t rotary_positions,
+                         int head_dim, void *rotary_rows_bf16_dev, void *stream);
+
+/*
  * Paged ragged writer for one layer.  key/value: BF16 [batch, tokens, kv_heads, head_dim];
  * row r contributes its first counts[r] tokens (uniform_count when counts is NULL) at
  * positions sequence_lengths[s] - count .. sequence_lengths[s] - 1 (lengths already advanced).

@@ -48,6 +48,8 @@ SIGNATURES = {
                                           _size, _ptr]),
     "nq_w4a4_gemm_workspace_bytes": (_size, [_i32, _i32, _i32, _i32, _i32]),
     "nq_nqkv_advance": (_i32, [_ptr, _ptr, _ptr, _i32, _i32, _i32, _i32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "nq_decode_step_begin": (_i32, [_ptr, _ptr, _i32, _i32, _i32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i32,
+                                    _ptr, _ptr, _ptr, _i64, _i32, _ptr, _ptr]),
     "nq_nqkv_write": (_i32, [_ptr, _ptr, _i32, _ptr, _ptr, _ptr, _i32, _ptr, _ptr] + [_ptr] * 6
                       + [_ptr, _i32, _ptr, _i32, _ptr, _ptr] + [_i32] * 8 + [_ptr, _ptr, _ptr]),
     "nq_nqkv_attention_decode": (_i32, [_ptr, _i32] + [_ptr] * 17 + [_i32] * 7 + [_c.c_float, _i32, _ptr, _ptr,

@@ -49,6 +49,53 @@ kv_advance_kernel(const int32_t *__restrict__ slot_ids, const uint8_t *__restric
     hot_lengths[slot] = length % page_size;
 }
 
+// One launch at the head of a decode step: workgroup r advances row r's tables by one token
+// (as kv_advance_kernel), copies the embedding row of its input token and the rotary
+// embedding's cos and sin rows of its position.
+struct StepBeginArgs {
+    const int32_t *slot_ids;
+    const uint8_t *active_mask;
+    int batch, slots, page_size, max_tokens;
+    int32_t *sequence_lengths, *page_counts, *last_page_lens, *hot_lengths;
+    const int64_t *tokens;          // [batch]
+    const uint4 *embedding;         // BF16 [vocab][hidden]
+    uint4 *embedded;                // BF16 [batch][hidden]
+    int64_t vocab;
+    int hidden_vectors;             // hidden / 8
+    const int64_t *positions;       // [batch]
+    const uint4 *rotary;            // BF16 [2][rotary_positions][rotary_vectors * 8]: cos rows, then sin rows
+    uint4 *rotary_rows;             // BF16 [2][batch][rotary_vectors * 8]
+    int64_t rotary_positions;
+    int rotary_vectors;             // head_dim / 8
+};
+
+__global__ void __launch_bounds__(256) decode_step_begin_kernel(StepBeginArgs a) {
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const int64_t token = a.tokens[r];
+    const bool known = token >= 0 && token < a.vocab;                  // an unknown token embeds as zero
+    const uint4 *source = a.embedding + (known ? token : 0) * a.hidden_vectors;
+    for (int v = tid; v < a.hidden_vectors; v += blockDim.x) {
+        const uint4 value = source[v];
+        a.embedded[(int64_t)r * a.hidden_vectors + v] = known ? value : make_uint4(0, 0, 0, 0);
+    }
+    if (tid < 2 * a.rotary_vectors) {
+        int64_t position = a.positions[r];
+        position = position < 0 ? 0 : (position >= a.rotary_positions ? a.rotary_positions - 1 : position);
+        const int side = tid / a.rotary_vectors, v = tid % a.rotary_vectors;
+        a.rotary_rows[((int64_t)side * a.batch + r) * a.rotary_vectors + v] =
+            a.rotary[((int64_t)side * a.rotary_positions + position) * a.rotary_vectors + v];
+    }
+    if (tid != 0 || !a.active_mask[r]) return;
+    const int slot = a.slot_ids[r];
+    if (slot < 0 || slot >= a.slots) return;                          // a stale replay writes nothing
+    int length = a.sequence_lengths[slot];
+    if (length < a.max_tokens) length += 1;                           // clamp at capacity
+    a.sequence_lengths[slot] = length;
+    a.page_counts[slot] = length / a.page_size;
+    a.last_page_lens[slot] = length >= a.page_size ? a.page_size : 0;
+    a.hot_lengths[slot] = length % a.page_size;
+}
+
 struct KvWriteArgs {
     const uint16_t *key, *value;            // BF16 [batch, tokens, kv_heads, D]
     const int32_t *slot_ids, *counts;       // counts may be null (uniform_count)
@@ -225,6 +272,42 @@ extern "C" int nq_nqkv_advance(const int32_t *slot_ids_dev, const uint8_t *activ
                        slot_ids_dev, active_mask_dev, counts_dev, uniform_count, batch, slots, page_size, max_tokens,
                        sequence_lengths_dev, page_counts_dev, last_page_lens_dev, hot_lengths_dev);
     return nq::check_launch("nq_nqkv_advance");
+}
+
+extern "C" int nq_decode_step_begin(const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch, int slots,
+                                    int page_size, int max_tokens, int32_t *sequence_lengths_dev,
+                                    int32_t *page_counts_dev, int32_t *last_page_lens_dev, int32_t *hot_lengths_dev,
+                                    const int64_t *tokens_dev, const void *embedding_bf16_dev, int64_t vocab,
+                                    int hidden, void *embedded_bf16_dev, const int64_t *positions_dev,
+                                    const void *rotary_bf16_dev, int64_t rotary_positions, int head_dim,
+                                    void *rotary_rows_bf16_dev, void *stream) {
+    NQ_REQUIRE(batch >= 1 && batch <= 65535 && slots >= 1 && page_size >= 1 && max_tokens >= 1, NQ_ERR_SHAPE,
+               "nq_decode_step_begin: batch (at most 65535), slots, page_size and max_tokens must be positive");
+    NQ_REQUIRE(vocab >= 1 && hidden >= 8 && hidden % 8 == 0 && rotary_positions >= 1 && head_dim >= 8 &&
+                   head_dim % 8 == 0 && head_dim <= 1024,
+               NQ_ERR_SHAPE, "nq_decode_step_begin: hidden and head_dim (at most 1024) must be positive multiples of 8");
+    NQ_REQUIRE(slot_ids_dev && active_mask_dev && sequence_lengths_dev && page_counts_dev && last_page_lens_dev &&
+                   hot_lengths_dev && tokens_dev && embedding_bf16_dev && embedded_bf16_dev && positions_dev &&
+                   rotary_bf16_dev && rotary_rows_bf16_dev,
+               NQ_ERR_ARGUMENT, "nq_decode_step_begin: null pointer");
+    NQ_REQUIRE(nq::aligned(embedding_bf16_dev, 16) && nq::aligned(embedded_bf16_dev, 16) &&
+                   nq::aligned(rotary_bf16_dev, 16) && nq::aligned(rotary_rows_bf16_dev, 16),
+               NQ_ERR_ARGUMENT, "nq_decode_step_begin: tables and outputs must be 16-byte aligned");
+    nq::StepBeginArgs a;
+    a.slot_ids = slot_ids_dev; a.active_mask = active_mask_dev;
+    a.batch = batch; a.slots = slots; a.page_size = page_size; a.max_tokens = max_tokens;
+    a.sequence_lengths = sequence_lengths_dev; a.page_counts = page_counts_dev;
+    a.last_page_lens = last_page_lens_dev; a.hot_lengths = hot_lengths_dev;
+    a.tokens = tokens_dev;
+    a.embedding = reinterpret_cast<const uint4 *>(embedding_bf16_dev);
+    a.embedded = reinterpret_cast<uint4 *>(embedded_bf16_dev);
+    a.vocab = vocab; a.hidden_vectors = hidden / 8;
+    a.positions = positions_dev;
+    a.rotary = reinterpret_cast<const uint4 *>(rotary_bf16_dev);
+    a.rotary_rows = reinterpret_cast<uint4 *>(rotary_rows_bf16_dev);
+    a.rotary_positions = rotary_positions; a.rotary_vectors = head_dim / 8;
+    hipLaunchKernelGGL(nq::decode_step_begin_kernel, dim3((unsigned)batch), dim3(256), 0, (hipStream_t)stream, a);
+    return nq::check_launch("nq_decode_step_begin");
 }
 
 extern "C" int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_dtype, const int32_t *slot_ids_dev,

@@ -18,7 +18,9 @@ per layer:
     SiLU(gate) * up + Hadamard + A4 encode             nq_fused_input_stage (mode 2)
     down_proj                                          nq_w4a4_gemv
 
-and the LM head of up to 16 rows as one stream over its BF16 weight (nq_bf16_rows_linear).
+preceded by one launch that advances the cache's tables and gathers the embedding and rotary
+rows (nq_decode_step_begin) and followed by the LM head of up to 16 rows as one stream over its
+BF16 weight (nq_bf16_rows_linear).
 
 FusedLlamaPrefillStep runs a prompt (or a chunk of one) the same way over [rows * tokens]
 activation rows: the input stages and linears as above (the linears on the matrix cores), RoPE
@@ -128,18 +130,35 @@ class FusedLlamaDecodeStep:
             return linear_packed_w4a4_gemv_grouped(activation, prepared, output_dtype=torch.bfloat16)
         return [self._linear(activation, weight) for weight in prepared]
 
+    def _table_rope(self) -> bool:
+        return getattr(self.inner.rotary_emb, "rope_type", "default") in ("default", "llama3", "linear")
+
     @torch.inference_mode()
-    def __call__(self, tokens: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+    def __call__(self, tokens: torch.Tensor, positions: torch.Tensor, *, advance: bool = False) -> torch.Tensor:
+        """`advance`: the step itself advances the cache's tables by one token per active row
+        (`BatchedNQKVLlamaCache.begin_decode_step`, which the caller has otherwise done), in the
+        launch that also gathers the embedding and rotary rows when the model allows it."""
         cache, inner = self.cache, self.inner
         manager = cache.manager
         rows = tokens.shape[0]
         if tokens.shape != (rows, 1) or positions.shape != (rows, 1) or rows != cache._rows:
             raise ValueError("the fused decode step takes [rows, 1] tokens and positions for the rows in flight")
         device = tokens.device
-        embedded = inner.embed_tokens(tokens)                               # [rows, 1, hidden]
-        if embedded.dtype != torch.bfloat16:
+        table = inner.embed_tokens.weight
+        if table.dtype != torch.bfloat16:
             raise TypeError("the fused decode step runs BF16 models")
-        query_rope = self._rope(embedded, positions)                        # 2 x [rows, head_dim]
+        if (advance and self._table_rope() and type(inner.embed_tokens) is torch.nn.Embedding
+                and table.is_contiguous() and table.shape[1] % 8 == 0 and tokens.is_contiguous()
+                and positions.is_contiguous() and tokens.dtype == positions.dtype == torch.int64):
+            if self._rope_tables is None:
+                self._rope(torch.empty((1, 1, self.hidden), dtype=torch.bfloat16, device=device), positions)
+            embedded, query_rope = manager.begin_decode_step(rows=rows, tokens=tokens, embedding=table,
+                                                             positions=positions, rotary=self._rope_tables)
+        else:
+            if advance:
+                cache.begin_decode_step()
+            embedded = inner.embed_tokens(tokens)                           # [rows, 1, hidden]
+            query_rope = self._rope(embedded, positions)                    # 2 x [rows, head_dim]
         cos, sin = query_rope[0].view(rows, 1, -1), query_rope[1].view(rows, 1, -1)
         heads, kv_heads, dim = cache.num_query_heads, cache.num_kv_heads, cache.head_dim
         workspace = cache._workspace(rows, torch.bfloat16)

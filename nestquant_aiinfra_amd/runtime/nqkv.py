@@ -596,6 +596,34 @@ class BatchedNQKVCacheManager:
             meta.sequence_lengths.data_ptr(), meta.page_counts.data_ptr(), meta.last_page_lens.data_ptr(),
             meta.hot_lengths.data_ptr(), _native.stream_handle(self.device)))
 
+    def begin_decode_step(self, *, rows: int, tokens: torch.Tensor, embedding: torch.Tensor,
+                          positions: torch.Tensor, rotary: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        """`begin_step(rows=rows, uniform_count=1)` and, in the same launch, the embedding rows of
+        `tokens` (int64, `rows` entries; `embedding` BF16 [vocab, hidden]) and the rows of
+        `positions` (int64, `rows` entries) of `rotary` (BF16 [2, positions, head_dim]: cos, sin).
+        Returns (embedded [rows, hidden], rotary rows [2, rows, head_dim]).  Graph-capturable."""
+        for name, tensor in (("tokens", tokens), ("positions", positions)):
+            if tensor.dtype != torch.int64 or tensor.numel() != rows or not tensor.is_contiguous() or \
+                    tensor.device != self.device:
+                raise ValueError(f"{name} must be {rows} contiguous int64 entries on the cache's device")
+        for name, tensor, ndim in (("embedding", embedding, 2), ("rotary", rotary, 3)):
+            if tensor.dtype != torch.bfloat16 or tensor.ndim != ndim or not tensor.is_contiguous() or \
+                    tensor.device != self.device or tensor.shape[-1] % 8:
+                raise ValueError(f"{name} must be a contiguous BF16 table on the cache's device")
+        if rotary.shape[0] != 2:
+            raise ValueError("rotary holds the cos rows, then the sin rows: [2, positions, head_dim]")
+        self._step_rows, self._step_uniform = rows, 1
+        meta = self.metadata
+        embedded = torch.empty((rows, embedding.shape[1]), dtype=torch.bfloat16, device=self.device)
+        rotary_rows = torch.empty((2, rows, rotary.shape[2]), dtype=torch.bfloat16, device=self.device)
+        _native.check(_native.library().nq_decode_step_begin(
+            self.step_slot_ids.data_ptr(), self.step_active.data_ptr(), rows, self.capacity, self.page_size,
+            self.max_tokens, meta.sequence_lengths.data_ptr(), meta.page_counts.data_ptr(),
+            meta.last_page_lens.data_ptr(), meta.hot_lengths.data_ptr(), tokens.data_ptr(), embedding.data_ptr(),
+            embedding.shape[0], embedding.shape[1], embedded.data_ptr(), positions.data_ptr(), rotary.data_ptr(),
+            rotary.shape[1], rotary.shape[2], rotary_rows.data_ptr(), _native.stream_handle(self.device)))
+        return embedded, rotary_rows
+
     def write_layer(self, layer_index: int, key: torch.Tensor, value: torch.Tensor, *,
                     rotate_keys: bool = False,
                     rope: tuple[torch.Tensor, torch.Tensor] | None = None) -> None:

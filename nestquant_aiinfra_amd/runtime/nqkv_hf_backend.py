@@ -401,9 +401,9 @@ class BatchedNQKVLlamaRunner:
 
     # -- decode --------------------------------------------------------------------------------
     def _step(self, tokens: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
-        self.cache.begin_decode_step()
         if self.fused_step is not None:
-            return self.fused_step(tokens, positions)
+            return self.fused_step(tokens, positions, advance=True)
+        self.cache.begin_decode_step()
         return self.model(input_ids=tokens, position_ids=positions, past_key_values=self.cache,
                           use_cache=True).logits
 

@@ -427,3 +427,42 @@ def test_page_container_fill_levels(kv, oracle, golden, valid):
         PackedNQKVPage.from_tensors(key, value, page_size=PAGE, q=Q, betas=KEY_BETAS, key_betas=KEY_BETAS)
     with pytest.raises(ValueError):
         PackedNQKVPage.from_tensors(key, value, page_size=PAGE, q=Q, key_betas=KEY_BETAS)
+
+
+def test_decode_step_begin_is_advance_plus_two_gathers():
+    """The head-of-step launch against nq_nqkv_advance (uniform count 1) on a copy of the tables,
+    torch's embedding and an index_select of the rotary table: inactive rows and rows with a slot
+    out of range advance nothing, a slot at capacity stays there, positions past the table take
+    its last row, an unknown token embeds as zero."""
+    from nestquant_aiinfra_amd import _native
+    lib = _native.library()
+    g = torch.Generator().manual_seed(909)
+    rows, slots, page, max_tokens, vocab, hidden, dim, max_pos = 6, 8, 16, 64, 300, 2048, 64, 96
+    slot_ids = torch.tensor([3, 0, 7, 9, 5, 1], dtype=torch.int32, device="cuda")         # 9: out of range; 7: inactive
+    active = torch.tensor([True, True, False, True, True, True], device="cuda")
+    lengths = torch.tensor([15, 31, 0, 64, 5, 47, 1, 16], dtype=torch.int32, device="cuda")  # slot 3: at capacity
+    tokens = torch.tensor([[5], [299], [0], [17], [300], [-1]], dtype=torch.long, device="cuda")
+    positions = torch.tensor([[0], [95], [96], [1000], [7], [50]], dtype=torch.long, device="cuda")
+    embedding = torch.randn((vocab, hidden), generator=g).to(torch.bfloat16).cuda()
+    rotary = torch.randn((2, max_pos, dim), generator=g).to(torch.bfloat16).cuda()
+    stream = _native.stream_handle(torch.device("cuda"))
+
+    def tables():
+        return [lengths.clone(), lengths // page, torch.where(lengths >= page, page, 0).int(), lengths % page]
+    want, got = tables(), tables()
+    _native.check(lib.nq_nqkv_advance(slot_ids.data_ptr(), active.data_ptr(), None, 1, rows, slots, page, max_tokens,
+                                      *[t.data_ptr() for t in want], stream))
+    embedded = torch.full((rows, hidden), 7.0, dtype=torch.bfloat16, device="cuda")
+    rotary_rows = torch.full((2, rows, dim), 7.0, dtype=torch.bfloat16, device="cuda")
+    _native.check(lib.nq_decode_step_begin(
+        slot_ids.data_ptr(), active.data_ptr(), rows, slots, page, max_tokens, *[t.data_ptr() for t in got],
+        tokens.data_ptr(), embedding.data_ptr(), vocab, hidden, embedded.data_ptr(), positions.data_ptr(),
+        rotary.data_ptr(), max_pos, dim, rotary_rows.data_ptr(), stream))
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    assert got[0].tolist() == [16, 32, 0, 64, 5, 48, 1, 16]
+    known = ((tokens >= 0) & (tokens < vocab)).view(-1)
+    reference = torch.nn.functional.embedding(tokens.view(-1).clamp(0, vocab - 1), embedding)
+    reference[~known] = 0
+    assert torch.equal(embedded.view(torch.int16), reference.view(torch.int16))
+    assert torch.equal(rotary_rows, rotary.index_select(1, positions.view(-1).clamp(0, max_pos - 1)))
