@@ -413,6 +413,29 @@ def tpot_extra(device, batches=(1, 8), prompt=128, generate=128):
                 "prefill_ms": prefill_s * 1e3, "prefill_ms_last_token_logits": prefill_last_s * 1e3, "tokens_per_s": batch / (sum(steps) / len(steps)),
                 "tokens_per_s_device_sampler": batch / greedy_s,
             }
+        # the same decode with BF16 copies of the projection weights kept beside the packed ones
+        # (16 instead of 6 bits per weight in HBM; the step streams them instead of decoding)
+        runner.fused_step.expand_weights = True
+        runner._graphs.clear()
+        for batch in batches:
+            slots = list(range(batch))
+            ids = torch.randint(0, config.vocab_size, (batch, prompt), generator=g).to(device)
+            logits = runner.prefill_slots(ids, slots=slots, lengths=[prompt] * batch, last_token_logits=True)
+            token = logits[:, 0].argmax(-1).reshape(batch, 1)
+            if not runner.graph_captured:
+                runner.capture()
+            position = torch.full((batch, 1), prompt, dtype=torch.long, device=device)
+            runner.decode_greedy(token, slots=slots, positions=position, steps=generate)       # to the same context
+            position = position + generate
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            runner.decode_greedy(token, slots=slots, positions=position, steps=greedy_steps).tolist()
+            greedy_s = (time.perf_counter() - t0) / greedy_steps
+            runner.release_slots(slots)
+            results[f"batch{batch}"]["tpot_ms_device_sampler_expanded_weights"] = greedy_s * 1e3
+        results["expanded_weight_bytes"] = sum(
+            sum(t.numel() * 2 for t in entry if isinstance(t, torch.Tensor))
+            for entry in runner.fused_step._expanded.values() if entry is not None)
         results["checkpoint_bytes"] = packed_bytes
     return results
 

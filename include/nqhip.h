@@ -422,16 +422,22 @@ int nq_greedy_sample(const void *logits_dev, int logits_dtype, int rows, int64_t
 size_t nq_greedy_sample_workspace_bytes(int rows);
 
 /*
- * out[r, j] = sum_k act[r, k] weight[j, k] for a few rows (rows in [1, 16], K 2048 or 4096) of a
- * BF16 activation [rows, K] against a BF16 weight [N, K], both dense row-major and 16-byte
+ * out[r, j] = sum_k act[r, k] weight[j, k] for a few rows (rows in [1, 16], K 2048, 4096 or 8192)
+ * of a BF16 activation [rows, K] against a BF16 weight [N, K], both dense row-major and 16-byte
  * aligned; FP32 accumulation, BF16 out [rows, N].  One stream over the weight on the matrix
- * cores, for the LM head of a decode step where a library GEMM of this shape leaves a third of
- * the memory rate unused.  No bias.
+ * cores: the LM head of a decode step (a library GEMM of this shape leaves a third of the memory
+ * rate unused), or a packed projection whose weight nq_w4a4_decode_weight has expanded to the
+ * BF16 values the packed kernels multiply by, applied to the decoded activation the encoder
+ * emits.  No bias.  The grouped form splits the N rows of one concatenated weight into up to
+ * three outputs (q, k, v or gate, up of one activation): group g holds group_n[g] rows and writes
+ * outs_bf16_dev[g], BF16 [rows, group_n[g]]; group_n and outs_bf16_dev are host arrays.
  * Replaces: the lm_head call inside the model forward of a decode step
  * (nestquant/runtime/nqkv_batched_runner.py:162-169).
  */
 int nq_bf16_rows_linear(const void *act_bf16_dev, const void *weight_bf16_dev, int rows, int64_t k, int64_t n,
                         void *out_bf16_dev, void *stream);
+int nq_bf16_rows_linear_grouped(const void *act_bf16_dev, const void *weight_bf16_dev, int rows, int64_t k, int groups,
+                                const int64_t *group_n, void *const *outs_bf16_dev, void *stream);
 
 #ifdef __cplusplus
 }

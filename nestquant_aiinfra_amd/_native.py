@@ -60,6 +60,7 @@ SIGNATURES = {
     "nq_greedy_sample": (_i32, [_ptr, _i32, _i32, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _size, _ptr]),
     "nq_greedy_sample_workspace_bytes": (_size, [_i32]),
     "nq_bf16_rows_linear": (_i32, [_ptr, _ptr, _i32, _i64, _i64, _ptr, _ptr]),
+    "nq_bf16_rows_linear_grouped": (_i32, [_ptr, _ptr, _i32, _i64, _i32, _ptr, _ptr, _ptr]),
     "nq_attention_output_stage": (_i32, [_ptr, _i64, _i32, _i32, _i32, _ptr, _i32, _ptr, _i32, _i32, _ptr, _ptr, _ptr,
                                          _ptr, _ptr]),
 }

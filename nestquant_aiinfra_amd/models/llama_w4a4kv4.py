@@ -63,7 +63,7 @@ def build_w4a4kv4_runner(model: nn.Module, checkpoint: str | Path, *, capacity: 
                          key_betas: Sequence[float] = KEY_BETAS, value_betas: Sequence[float] = VALUE_BETAS,
                          enable_m1_down_splitk: bool = False,
                          fused_decode: bool | None = None, fused_prefill: bool | None = None,
-                         packed_prefill: bool = False) -> BatchedNQKVLlamaRunner:
+                         packed_prefill: bool = False, expand_weights: bool = False) -> BatchedNQKVLlamaRunner:
     """Swap the projections of `model` (BF16, on the GPU, eval mode) for packed W4A4 modules
     read from `checkpoint` and attach a batched NQKV4 cache; returns the runner."""
     reader = NQMCFileReader(checkpoint)
@@ -80,4 +80,5 @@ def build_w4a4kv4_runner(model: nn.Module, checkpoint: str | Path, *, capacity: 
         page_size=page_size, q=14, key_betas=key_betas, value_betas=value_betas, dtype=torch.bfloat16, device=device,
         packed_prefill=packed_prefill)
     install_batched_nqkv_llama_backend(model, cache)
-    return BatchedNQKVLlamaRunner(model, cache, fused_decode=fused_decode, fused_prefill=fused_prefill)
+    return BatchedNQKVLlamaRunner(model, cache, fused_decode=fused_decode, fused_prefill=fused_prefill,
+                                  expand_weights=expand_weights)

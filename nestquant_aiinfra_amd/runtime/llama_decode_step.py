@@ -37,8 +37,9 @@ import torch
 import torch.nn.functional as F
 
 from .nqkv import attention_output_stage, launch_nqkv_decode_attention, nqkv_prefill_attention
-from .w4a4_linear import (MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, _gemm, _gemv, bf16_rows_linear,
-                          can_use_bf16_rows_linear, fused_input_stage,
+from .w4a4_linear import (BF16_ROWS_LINEAR_K, MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, _gemm, _gemv,
+                          bf16_rows_linear, bf16_rows_linear_grouped, can_use_bf16_rows_linear, decode_weight_bf16,
+                          fused_input_stage,
                           linear_packed_w4a4_gemv_grouped, quantize_activation_cuda, rope_hadamard_cuda)
 
 
@@ -56,7 +57,11 @@ class FusedLlamaDecodeStep:
     LlamaForCausalLM whose projections are FusedNQRTLinear modules and a BatchedNQKVLlamaCache.
     Raises UnsupportedForFusedDecode at construction for anything else."""
 
-    def __init__(self, model: torch.nn.Module, cache) -> None:
+    def __init__(self, model: torch.nn.Module, cache, *, expand_weights: bool = False) -> None:
+        """`expand_weights`: keep, beside every packed projection, the BF16 values its kernels
+        multiply by (16 bits per weight in HBM instead of 6) and stream those for steps of up to
+        16 rows: the same products without the per-step decode, which is what bounds the packed
+        kernels.  The container on disk and the prefill path are unchanged."""
         from ..models.fused_linear import FusedNQRTLinear
 
         inner = getattr(model, "model", None)
@@ -88,6 +93,8 @@ class FusedLlamaDecodeStep:
         _require(hidden & (hidden - 1) == 0 and hidden % 32 == 0, "hidden size is not a power of two")
         self.hidden = hidden
         self._rope_tables: torch.Tensor | None = None
+        self.expand_weights = bool(expand_weights)
+        self._expanded: dict[int, tuple] = {}
 
     def _rope(self, embedded: torch.Tensor, positions: torch.Tensor, *, padded: bool = False
               ) -> tuple[torch.Tensor, torch.Tensor]:
@@ -130,6 +137,19 @@ class FusedLlamaDecodeStep:
             return linear_packed_w4a4_gemv_grouped(activation, prepared, output_dtype=torch.bfloat16)
         return [self._linear(activation, weight) for weight in prepared]
 
+    def _expanded_layer(self, index: int, device) -> tuple | None:
+        """(q|k|v rows, their sizes, o, gate|up rows, their sizes, down) of layer `index` as BF16
+        [N, K] tensors, decoded once; None when a projection's K is not one the stream kernel takes."""
+        if index not in self._expanded:
+            prepared = [self._prepared(linear, device) for linear in self.layers[index][3]]
+            if any(weight.record.feature_count not in BF16_ROWS_LINEAR_K for weight in prepared):
+                self._expanded[index] = None
+            else:
+                q, k, v, o, gate, up, down = (decode_weight_bf16(weight) for weight in prepared)
+                self._expanded[index] = (torch.cat((q, k, v)), [q.shape[0], k.shape[0], v.shape[0]], o,
+                                         torch.cat((gate, up)), [gate.shape[0], up.shape[0]], down)
+        return self._expanded[index]
+
     def _table_rope(self) -> bool:
         return getattr(self.inner.rotary_emb, "rope_type", "default") in ("default", "llama3", "linear")
 
@@ -170,7 +190,11 @@ class FusedLlamaDecodeStep:
             activation, residual, _ = fused_input_stage(
                 delta, mode="rmsnorm", residual=residual, norm_weight=layer.input_layernorm.weight,
                 eps=layer.input_layernorm.variance_epsilon, beta_table=table, want_residual=True)
-            query, key, value = self._linears(activation, [q_w, k_w, v_w])
+            expanded = self._expanded_layer(index, device) if self.expand_weights and rows <= 16 else None
+            if expanded is not None:
+                query, key, value = bf16_rows_linear_grouped(activation.decoded, expanded[0], expanded[1])
+            else:
+                query, key, value = self._linears(activation, [q_w, k_w, v_w])
             manager.write_layer(index, key.view(rows, 1, kv_heads, dim), value.view(rows, 1, kv_heads, dim),
                                 rotate_keys=True, rope=(cos, sin))
             # the attention leaves per-chunk results; o_proj's input stage merges them as it loads its rows
@@ -179,13 +203,17 @@ class FusedLlamaDecodeStep:
                 active_mask=manager.step_active, attention_scale=float(attention.scaling), workspace=workspace,
                 rotate_query=True, rope=query_rope, merge=False)
             o_input, _ = attention_output_stage(workspace, q=14, beta_table=table, hadamard=True)
-            delta = self._linear(o_input, o_w)
+            delta = self._linear(o_input, o_w) if expanded is None else bf16_rows_linear(o_input.decoded, expanded[2])
             activation, residual, _ = fused_input_stage(
                 delta, mode="rmsnorm", residual=residual, norm_weight=layer.post_attention_layernorm.weight,
                 eps=layer.post_attention_layernorm.variance_epsilon, beta_table=table, want_residual=True)
-            gate, up = self._linears(activation, [gate_w, up_w])
+            if expanded is not None:
+                gate, up = bf16_rows_linear_grouped(activation.decoded, expanded[3], expanded[4])
+            else:
+                gate, up = self._linears(activation, [gate_w, up_w])
             activation, _, _ = fused_input_stage(up, mode="swiglu", gate=gate, beta_table=table)
-            delta = self._linear(activation, down_w)
+            delta = (self._linear(activation, down_w) if expanded is None
+                     else bf16_rows_linear(activation.decoded, expanded[5]))
         _, _, normed = fused_input_stage(delta, mode="rmsnorm", residual=residual, norm_weight=inner.norm.weight,
                                          eps=inner.norm.variance_epsilon, encode=False, want_staged=True)
         return self._lm_head(normed.view(rows, self.hidden)).view(rows, 1, -1)

@@ -323,10 +323,12 @@ class BatchedNQKVLlamaRunner:
     GREEDY_HISTORY_STEPS = 256
 
     def __init__(self, model: torch.nn.Module, cache: BatchedNQKVLlamaCache, *,
-                 fused_decode: bool | None = None, fused_prefill: bool | None = None) -> None:
+                 fused_decode: bool | None = None, fused_prefill: bool | None = None,
+                 expand_weights: bool = False) -> None:
         """`fused_decode` / `fused_prefill`: run decode steps through FusedLlamaDecodeStep (ten
         launches per layer) and prompts through FusedLlamaPrefillStep instead of the module
-        graph; None = whenever the model qualifies."""
+        graph; None = whenever the model qualifies.  `expand_weights`: the fused decode step keeps
+        and streams BF16 copies of the projection weights (see FusedLlamaDecodeStep)."""
         if not isinstance(model, torch.nn.Module):
             raise TypeError("model must be a torch module")
         if not isinstance(cache, BatchedNQKVLlamaCache):
@@ -347,7 +349,7 @@ class BatchedNQKVLlamaRunner:
         if fused_decode is None or fused_decode:
             from .llama_decode_step import FusedLlamaDecodeStep, UnsupportedForFusedDecode
             try:
-                self.fused_step = FusedLlamaDecodeStep(model, cache)
+                self.fused_step = FusedLlamaDecodeStep(model, cache, expand_weights=expand_weights)
             except UnsupportedForFusedDecode:
                 if fused_decode:
                     raise

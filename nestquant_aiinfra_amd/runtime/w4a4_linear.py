@@ -10,6 +10,7 @@ Every operator calls the HIP library through its C ABI; there is no other comput
 
 from __future__ import annotations
 
+import ctypes
 import math
 from dataclasses import dataclass
 from typing import Any, Sequence
@@ -553,6 +554,7 @@ LIBRARY_GEMM_ROWS = 288
 # which from five rows on multiplies on the matrix cores
 MATRIX_CORE_GEMV_ROWS = 16
 BF16_ROWS_LINEAR_MAX_ROWS = 16
+BF16_ROWS_LINEAR_K = (2048, 4096, 8192)
 
 
 def decode_weight_bf16(weight: PreparedNQRTLinear) -> torch.Tensor:
@@ -575,22 +577,35 @@ def can_use_bf16_rows_linear(rows: torch.Tensor, weight: torch.Tensor) -> bool:
     return (rows.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and rows.device.type == "cuda"
             and weight.device == rows.device and rows.ndim == 2 and weight.ndim == 2
             and 1 <= rows.shape[0] <= BF16_ROWS_LINEAR_MAX_ROWS and rows.shape[1] == weight.shape[1]
-            and weight.shape[1] in (2048, 4096) and rows.is_contiguous() and weight.is_contiguous()
+            and weight.shape[1] in BF16_ROWS_LINEAR_K and rows.is_contiguous() and weight.is_contiguous()
             and rows.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
 def bf16_rows_linear(rows: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """`rows @ weight.T` for at most 16 BF16 rows against a BF16 [N, K] weight (K 2048 or 4096),
-    FP32 accumulation, BF16 out: the LM head of a decode step
+    """`rows @ weight.T` for at most 16 BF16 rows against a BF16 [N, K] weight (K 2048, 4096 or
+    8192), FP32 accumulation, BF16 out: the LM head of a decode step
     (nestquant/runtime/nqkv_batched_runner.py:162-169) as one stream over the weight."""
+    return bf16_rows_linear_grouped(rows, weight, [weight.shape[0]])[0]
+
+
+def bf16_rows_linear_grouped(rows: torch.Tensor, weight: torch.Tensor, sizes: Sequence[int]) -> list[torch.Tensor]:
+    """`bf16_rows_linear` against a weight whose N rows are the rows of up to three projections of
+    the same activation, one after the other (`sizes` rows each): one launch, one dense BF16
+    [rows, size] output per projection."""
     if not can_use_bf16_rows_linear(rows, weight):
-        raise ValueError("bf16_rows_linear takes contiguous BF16 [rows <= 16, K] and [N, K] on one GPU, K 2048 or 4096")
+        raise ValueError("bf16_rows_linear takes contiguous BF16 [rows <= 16, K] and [N, K] on one GPU, "
+                         "K 2048, 4096 or 8192")
+    sizes = [int(size) for size in sizes]
+    if not 1 <= len(sizes) <= 3 or min(sizes) < 1 or sum(sizes) != weight.shape[0]:
+        raise ValueError("between one and three positive sizes that add up to the weight's rows")
     device = _native.require_cuda(rows)
-    out = torch.empty((rows.shape[0], weight.shape[0]), dtype=torch.bfloat16, device=device)
-    _native.check(_native.library().nq_bf16_rows_linear(
-        rows.data_ptr(), weight.data_ptr(), rows.shape[0], rows.shape[1], weight.shape[0], out.data_ptr(),
+    outs = [torch.empty((rows.shape[0], size), dtype=torch.bfloat16, device=device) for size in sizes]
+    group_n = (ctypes.c_int64 * len(sizes))(*sizes)
+    pointers = (ctypes.c_void_p * len(sizes))(*[out.data_ptr() for out in outs])
+    _native.check(_native.library().nq_bf16_rows_linear_grouped(
+        rows.data_ptr(), weight.data_ptr(), rows.shape[0], rows.shape[1], len(sizes), group_n, pointers,
         _native.stream_handle(device)))
-    return out
+    return outs
 
 
 def _gemm(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *,

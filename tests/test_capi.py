@@ -64,9 +64,11 @@ def test_host_side_validation_needs_no_gpu():
     status = lib.nq_bf16_rows_linear(None, None, 17, 2048, 128256, None, None)
     assert status == _native.NQ_ERR_SHAPE and b"outside [1, 16]" in lib.nq_last_error()
     status = lib.nq_bf16_rows_linear(None, None, 8, 1024, 128256, None, None)
-    assert status == _native.NQ_ERR_SHAPE and b"not 2048 or 4096" in lib.nq_last_error()
+    assert status == _native.NQ_ERR_SHAPE and b"not 2048, 4096 or 8192" in lib.nq_last_error()
     status = lib.nq_bf16_rows_linear(None, None, 8, 2048, 128256, None, None)
     assert status == _native.NQ_ERR_ARGUMENT and b"null pointer" in lib.nq_last_error()
+    status = lib.nq_bf16_rows_linear_grouped(None, None, 8, 8192, 4, None, None, None)
+    assert status == _native.NQ_ERR_ARGUMENT and b"between one and three outputs" in lib.nq_last_error()
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

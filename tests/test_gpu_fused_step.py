@@ -471,7 +471,8 @@ def test_bf16_rows_linear_against_float64():
     both K."""
     from nestquant_aiinfra_amd.runtime.w4a4_linear import bf16_rows_linear, can_use_bf16_rows_linear
     g = torch.Generator().manual_seed(4242)
-    for rows, n, k in ((1, 128256, 2048), (8, 4099, 2048), (16, 1000, 4096), (5, 77, 2048), (13, 16, 4096), (3, 1, 2048)):
+    for rows, n, k in ((1, 128256, 2048), (8, 4099, 2048), (16, 1000, 4096), (5, 77, 2048), (13, 16, 4096), (3, 1, 2048),
+                       (8, 2048, 8192), (16, 77, 8192)):
         act = torch.randint(-3, 4, (rows, k), generator=g).to(torch.bfloat16).cuda()
         weight = torch.randint(-3, 4, (n, k), generator=g).to(torch.bfloat16).cuda()
         assert can_use_bf16_rows_linear(act, weight)
@@ -483,6 +484,17 @@ def test_bf16_rows_linear_against_float64():
         got = bf16_rows_linear(act, weight).double()
         bound = exact.abs() * 2.0 ** -8 + (act.double().abs() @ weight.double().abs().T) * k * 2.0 ** -24
         assert bool(((got - exact).abs() <= bound).all()), (rows, n, k, float(((got - exact).abs() / bound).max()))
+    # one weight, three outputs: the rows of q, k and v one after the other, ragged on purpose
+    from nestquant_aiinfra_amd.runtime.w4a4_linear import bf16_rows_linear_grouped
+    for rows, k, sizes in ((8, 2048, [2048, 512, 512]), (3, 8192, [40, 9]), (16, 4096, [5, 1, 30])):
+        act = torch.randn((rows, k), generator=g).to(torch.bfloat16).cuda()
+        weight = (0.05 * torch.randn((sum(sizes), k), generator=g)).to(torch.bfloat16).cuda()
+        outs = bf16_rows_linear_grouped(act, weight, sizes)
+        whole = bf16_rows_linear(act, weight)
+        assert [tuple(out.shape) for out in outs] == [(rows, size) for size in sizes]
+        assert torch.equal(torch.cat(outs, 1), whole)
+    with pytest.raises(ValueError, match="add up"):
+        bf16_rows_linear_grouped(act, weight, [5, 1])
     for bad_rows, bad_weight in ((torch.zeros((17, 2048)), torch.zeros((32, 2048))), (torch.zeros((4, 1024)), torch.zeros((32, 1024)))):
         assert not can_use_bf16_rows_linear(bad_rows.to(torch.bfloat16).cuda(), bad_weight.to(torch.bfloat16).cuda())
         with pytest.raises(ValueError):
@@ -537,3 +549,40 @@ def test_last_token_logits_and_the_lm_head_stream(tmp_path, monkeypatch):
     assert len(calls) == 1
     assert float((streamed - library).abs().max()) <= 2.0 ** -7 * float(library.abs().max())
     assert int(streamed.argmax()) == int(library.argmax())
+
+
+def test_expanded_weights_step_tracks_the_packed_step(tmp_path):
+    """`expand_weights`: the decode step that streams BF16 copies of the weights (the values the
+    packed kernels decode, multiplied in another order) against the packed step on the same
+    prompt in another slot, eager and captured; K = 2048 and 4096 projections.  Every linear agrees
+    with its packed form to a BF16 step of a few outputs (the kernel tests hold that); a step or
+    two of difference moves some activation codes, which a random-init network amplifies from
+    layer to layer, hence the loose bound on the logits."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
+    from nestquant_aiinfra_amd.runtime.llama_decode_step import FusedLlamaDecodeStep
+
+    torch.manual_seed(7001)
+    config = LlamaConfig(hidden_size=2048, intermediate_size=4096, num_hidden_layers=2, num_attention_heads=32,
+                         num_key_value_heads=8, head_dim=64, vocab_size=1000, max_position_embeddings=256,
+                         rope_theta=500000.0, tie_word_embeddings=True)
+    model = LlamaForCausalLM(config).to(torch.bfloat16).cuda().eval()
+    path = tmp_path / "wide.nqmc"
+    asm.write_w4_checkpoint(model, path)
+    runner = asm.build_w4a4kv4_runner(model, path, capacity=2, max_cache_len=96, expand_weights=True)
+    streamed_step = runner.fused_step
+    assert streamed_step.expand_weights
+    packed_step = FusedLlamaDecodeStep(model, runner.cache)
+    ids = torch.randint(0, 1000, (1, 20), generator=torch.Generator().manual_seed(7002)).cuda().repeat(2, 1)
+    runner.prefill_slots(ids, slots=[0, 1], lengths=[20, 20], last_token_logits=True)
+    token, position = torch.tensor([[7]], device="cuda"), torch.tensor([[20]], device="cuda")
+    streamed = runner.decode_eager(token, slots=[0], positions=position).float()
+    assert streamed_step._expanded and all(entry is not None for entry in streamed_step._expanded.values())
+    runner.fused_step = packed_step
+    packed = runner.decode_eager(token, slots=[1], positions=position).float()
+    runner.fused_step = streamed_step
+    cosine = torch.nn.functional.cosine_similarity(streamed.flatten(), packed.flatten(), dim=0)
+    assert float(cosine) > 0.95, float(cosine)
+    runner.capture()
+    chosen = runner.decode_greedy(token, slots=[0], positions=position + 1, steps=4)
+    assert chosen.shape == (4, 1) and bool(((chosen >= 0) & (chosen < 1000)).all())
