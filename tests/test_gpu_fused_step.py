@@ -472,7 +472,7 @@ def test_bf16_rows_linear_against_float64():
     from nestquant_aiinfra_amd.runtime.w4a4_linear import bf16_rows_linear, can_use_bf16_rows_linear
     g = torch.Generator().manual_seed(4242)
     for rows, n, k in ((1, 128256, 2048), (8, 4099, 2048), (16, 1000, 4096), (5, 77, 2048), (13, 16, 4096), (3, 1, 2048),
-                       (8, 2048, 8192), (16, 77, 8192)):
+                       (8, 2048, 8192), (16, 77, 8192), (5, 1000, 4096), (1, 4099, 8192)):
         act = torch.randint(-3, 4, (rows, k), generator=g).to(torch.bfloat16).cuda()
         weight = torch.randint(-3, 4, (n, k), generator=g).to(torch.bfloat16).cuda()
         assert can_use_bf16_rows_linear(act, weight)
