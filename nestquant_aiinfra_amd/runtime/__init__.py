@@ -33,6 +33,9 @@ _EXPORTS = {
     "linear_packed_w4a4_mma_small_m": "w4a4_linear",
     "linear_packed_w4a4_mma_small_m_splitk_probe": "w4a4_linear",
     "decode_weight_bf16": "w4a4_linear",
+    "can_use_bf16_rows_linear": "w4a4_linear",
+    "bf16_rows_linear": "w4a4_linear",
+    "bf16_rows_linear_grouped": "w4a4_linear",
     "linear_packed_w4a4_mma_m16": "w4a4_linear",
     "linear_packed_w4a4_mma_large_m_staged": "w4a4_linear",
     "linear_packed_w4a4_mma_m128_staged": "w4a4_linear",
