@@ -63,7 +63,7 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--profile-copy", action="store_true",
                         help="also run three 256 MiB device-to-device copies (a kernel of known traffic, "
                              "to calibrate FETCH_SIZE / WRITE_SIZE counters under rocprofv3)")
-    parser.add_argument("--only", choices=("tpot", "gemm", "attention", "encode"), default=None,
+    parser.add_argument("--only", choices=("tpot", "gemm", "attention", "encode", "rowlinear"), default=None,
                         help="run one of the extra measurements alone (for profiling) and print its JSON")
     parser.add_argument("--skip-extras", action="store_true",
                         help="only the headline GEMV workload (no prefill GEMM, attention, TPOT)")
@@ -288,6 +288,29 @@ def encode_extra(rt, device):
     return results
 
 
+def row_linear_extra(rt, device):
+    """The BF16 stream kernel: the LM head of the 1B model (128256 x 2048) and, for the optional
+    expanded-weights decode, the 1B projection shapes, at 1 and 8 rows.  Algorithmic bytes: the
+    BF16 weight once, the activation and the output."""
+    import torch
+    results = {}
+    g = torch.Generator().manual_seed(6100)
+    shapes = (("lm_head", 2048, [128256]), ("qkv", 2048, [2048, 512, 512]), ("o_proj", 2048, [2048]),
+              ("gate_up", 2048, [8192, 8192]), ("down_proj", 8192, [2048]))
+    for name, k, sizes in shapes:
+        n = sum(sizes)
+        copies = max(2, min(8, (600 << 20) // (n * k * 2)))            # rotate past the 256 MB of last-level cache
+        weights = [(0.05 * torch.randn((n, k), generator=g)).to(torch.bfloat16).to(device) for _ in range(copies)]
+        for rows in (1, 8):
+            act = torch.randn((rows, k), generator=g).to(torch.bfloat16).to(device)
+            seconds = time_graph(lambda i: rt.bf16_rows_linear_grouped(act, weights[i % copies], sizes), 2 * copies)
+            nbytes = 2 * (n * k + rows * k + rows * n)
+            results[f"{name}_m{rows}"] = {"us": seconds * 1e6, "bytes": nbytes, "GBps": nbytes / seconds / 1e9,
+                                          "hbm_frac": nbytes / seconds / 1e9 / HBM_PEAK_GBPS}
+        del weights
+    return results
+
+
 def attention_extra(device):
     """Paged NQKV4 decode attention: 32 / 8 heads, D 64, batch 8, contexts uniform in [128, 4096]."""
     import torch
@@ -465,7 +488,8 @@ def main() -> None:
 
     if args.only:
         extra = {"tpot": lambda: tpot_extra(device), "gemm": lambda: prefill_gemm_extra(rt, device),
-                 "attention": lambda: attention_extra(device), "encode": lambda: encode_extra(rt, device)}[args.only]()
+                 "attention": lambda: attention_extra(device), "encode": lambda: encode_extra(rt, device),
+                 "rowlinear": lambda: row_linear_extra(rt, device)}[args.only]()
         print(json.dumps({args.only: extra}))
         return
 
@@ -520,6 +544,7 @@ def main() -> None:
         result["extra"]["e8_encode"] = encode_extra(rt, device)
         result["extra"]["prefill_gemm"] = prefill_gemm_extra(rt, device)
         result["extra"]["nqkv_attention"] = attention_extra(device)
+        result["extra"]["bf16_row_linear"] = row_linear_extra(rt, device)
         result["extra"]["llama_1b_w4a4kv4"] = tpot_extra(device)
     print(json.dumps(result))
 
