@@ -205,6 +205,28 @@ int nq_w4a4_gemv(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
 size_t nq_w4a4_gemv_workspace_bytes(int m, int k, int n, int split_k, int have_decoded_activation);
 
 /*
+ * nq_w4a4_gemv without a caller workspace: the decoded activation and the split-K partial sums
+ * live in a 4 MiB buffer inside the library's own device image (one copy per GPU, held until the
+ * process ends), so the call allocates nothing and asks for nothing that was allocated for it.
+ * Same arguments, kernels and results (bit for bit) as nq_w4a4_gemv; shapes whose workspace
+ * (nq_w4a4_gemv_workspace_bytes) exceeds the buffer are rejected with NQ_ERR_WORKSPACE.  The
+ * first call on a device looks up the buffer's address (hipGetSymbolAddress) and should
+ * therefore happen outside a graph capture.  All calls on one GPU share the buffer: calls that
+ * may overlap there (different streams, different threads) race and must be serialised by the
+ * caller.  Nothing in the buffer needs clearing between calls.
+ * No counterpart in the reference (its extension allocates partials with torch::empty on every
+ * call, nestquant/runtime/nqrt4_w4a4_mma.cu:1213-1214); it is for callers that cannot allocate
+ * device memory: code under HIP graph capture, tight serving loops, harnesses that forbid it.
+ */
+int nq_w4a4_gemv_static(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
+                        const float *act_norms_dev, const float *act_betas_dev,
+                        const void *act_decoded_dev, const uint8_t *w_codes_dev,
+                        const uint8_t *w_beta_ids_dev, const uint32_t *w_resolved_words_dev,
+                        const uint16_t *w_resolved_tails_dev, const float *w_norms_dev,
+                        const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
+                        int64_t weight_seed, int split_k, void *out_dev, int out_dtype, void *stream);
+
+/*
  * nq_w4a4_gemv for `count` (1..4) weights that share one activation (q/k/v_proj, gate/up_proj)
  * in a single launch.  Every array argument is a host array of `count` entries; weights are
  * given in resolved form (nq_w4a4_resolve_weight) and the activation as its decoded BF16

@@ -586,3 +586,66 @@ extern "C" int nq_w4a4_gemv_grouped(const void *act_decoded_dev, int count, cons
 #undef NQ_LAUNCH_GROUPED
     return nq::check_launch("nq_w4a4_gemv_grouped");
 }
+
+// ---------------------------------------------------------------------------------------
+// nq_w4a4_gemv for callers that cannot allocate device memory: the workspace (decoded
+// activation, split-K partials) is a fixed array in the library's own device image.
+namespace {
+
+constexpr size_t kStaticScratchBytes = (size_t)4 << 20;
+constexpr int kStaticScratchMaxDevices = 64;
+
+// One copy per GPU the library's code object is loaded on, at that GPU's own address.  In
+// host code the name is only a handle for hipGetSymbolAddress: it is never passed to a kernel.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch_address(void **address) {
+    static void *known[kStaticScratchMaxDevices] = {nullptr};
+    int device = -1;
+    hipError_t status = hipGetDevice(&device);
+    if (status != hipSuccess)
+        return nq::fail(NQ_ERR_LAUNCH, "nq_w4a4_gemv_static: hipGetDevice: %s", hipGetErrorString(status));
+    NQ_REQUIRE(device >= 0 && device < kStaticScratchMaxDevices, NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemv_static: device ordinal %d is outside [0, %d)", device, kStaticScratchMaxDevices);
+    void *pointer = __atomic_load_n(&known[device], __ATOMIC_ACQUIRE);
+    if (!pointer) {
+        status = hipGetSymbolAddress(&pointer, HIP_SYMBOL(scratch));
+        if (status != hipSuccess || !pointer)
+            return nq::fail(NQ_ERR_LAUNCH, "nq_w4a4_gemv_static: hipGetSymbolAddress(scratch): %s",
+                            hipGetErrorString(status));
+        __atomic_store_n(&known[device], pointer, __ATOMIC_RELEASE);    // every thread finds the same address
+    }
+    *address = pointer;
+    return NQ_OK;
+}
+
+}  // namespace
+
+extern "C" int nq_w4a4_gemv_static(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
+                                   const float *act_norms_dev, const float *act_betas_dev,
+                                   const void *act_decoded_dev, const uint8_t *w_codes_dev,
+                                   const uint8_t *w_beta_ids_dev, const uint32_t *w_resolved_words_dev,
+                                   const uint16_t *w_resolved_tails_dev, const float *w_norms_dev,
+                                   const float *w_betas_dev, int m, int k, int n, int64_t weight_offset,
+                                   int64_t weight_seed, int split_k, void *out_dev, int out_dtype, void *stream) {
+    NQ_REQUIRE(m >= 1 && m <= 16 && k >= 32 && n >= 1, NQ_ERR_SHAPE,
+               "nq_w4a4_gemv_static: M = %d, K = %d, N = %d: M must be in [1, 16], K at least 32, N positive", m, k, n);
+    NQ_REQUIRE(split_k == 0 || split_k == 1 || split_k == 2 || split_k == 4 || split_k == 8, NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemv_static: split_k must be 0, 1, 2, 4 or 8");
+    // what nq_w4a4_gemv will ask of its workspace (a launch on the matrix cores needs less, never more)
+    const size_t need = nq_w4a4_gemv_workspace_bytes(m, k, n, split_k, act_decoded_dev != nullptr);
+    NQ_REQUIRE(need <= kStaticScratchBytes, NQ_ERR_WORKSPACE,
+               "nq_w4a4_gemv_static: M = %d, K = %d, N = %d, split_k = %d needs %zu bytes of scratch; the "
+               "built-in buffer holds %zu (use nq_w4a4_gemv with a caller-owned workspace)",
+               m, k, n, split_k, need, kStaticScratchBytes);
+    void *workspace = nullptr;
+    const int status = static_scratch_address(&workspace);
+    if (status != NQ_OK) return status;
+    // Every partial sum and every decoded activation value a launch reads was written by that
+    // same launch sequence, so what an earlier call left in the buffer needs no clearing.
+    return nq_w4a4_gemv(act_codes_dev, act_beta_ids_dev, act_norms_dev, act_betas_dev, act_decoded_dev, w_codes_dev,
+                        w_beta_ids_dev, w_resolved_words_dev, w_resolved_tails_dev, w_norms_dev, w_betas_dev, m, k, n,
+                        weight_offset, weight_seed, split_k, out_dev, out_dtype, need ? workspace : nullptr,
+                        need ? kStaticScratchBytes : 0, stream);
+}
