@@ -149,8 +149,8 @@ int nq_dequantize_rows(const uint8_t *codes_dev, const uint8_t *beta_ids_dev,
  * seed and the block index.  This entry runs the exact decode and stores the lattice point
  * s = G c + Q_E8(u) - 14 Q_E8(...) of every block, so that the linear kernels compute w = s - u
  * with the hash alone (no search, no division; about a third of the vector instructions).
- *   words_dev  uint32[rows * K / 8]: floor(s_j) + 15 for j = 0..5 in 5-bit fields from bit 0,
- *              the block's beta id in bits 30..31
+ *   words_dev  uint32[rows * K / 8]: the block's beta id in bits 0..1, floor(s_j) + 15 for
+ *              j = 0..5 in 5-bit fields from bit 2
  *   tails_dev  uint16[rows * K / 8]: fields 6 and 7 in bits 0..9, bit 10 set when s lies in
  *              the half-integer coset
  *   out_of_range_dev  int32 counter (caller zeroes it): blocks whose s does not fit the

@@ -245,14 +245,17 @@ __device__ __forceinline__ void decode_codeword(uint32_t word, float q, uint32_t
 // lattice searches depend only on the stored code, the seed and the block index, so they can
 // be done once when a weight is prepared: s = p + n - 14 k is a point of E8 and  w = s - u.
 // resolve_codeword() runs the exact decode and stores s in 43 bits: the eight floors
-// floor(s_j) + 15 as 5-bit fields (w and u bound s_j to [-14, 16]), one bit saying that
-// the point lies in the half-integer coset, and the block's 2-bit beta id, as a 32-bit word
-// (fields 0..5, beta id in bits 30..31) and a 16-bit word (fields 6..7, half flag in bit 10).
-// decode_resolved() then needs the hash and six instructions per weight, no search and no
-// division.  It returns (s - u) * 2^26 computed in integers from the hash value with its
-// four lowest bits dropped: a 2^-26 absolute deviation from the float decode, far below the
-// BF16 rounding that follows, and the lattice points themselves are the exact ones.
-constexpr float kResolvedUnit = 1.0f / 67108864.0f;   // 2^-26
+// f_j = floor(s_j) + 15 as 5-bit fields (w and u bound s_j to [-14, 16]), one bit saying that
+// the point lies in the half-integer coset, and the block's 2-bit beta id:
+//   32-bit word  beta id in bits 0..1, f_0..f_5 at bits 2 + 5 j
+//   16-bit word  f_6 at bits 0..4, f_7 at bits 5..9, half-coset flag in bit 10
+// decode_resolved() then needs the hash and a handful of instructions per weight, no search and
+// no division.  It builds the float 2^23 + (f_j 2^17 + 2^18 - 1 - U_j) in its mantissa, U_j being
+// the top 18 bits of the 31-bit hash value (u_j 2^17, truncated), and subtracts the constant
+// that leaves (s_j - u_j) 2^17: the lattice points are the exact ones, the dither is taken to
+// 2^-17 of a lattice unit (the reference rounds it to 24 significant bits), far below the BF16
+// rounding that follows.
+constexpr float kResolvedUnit = 1.0f / 131072.0f;   // 2^-17
 
 __device__ __forceinline__ bool resolve_codeword(uint32_t word, uint32_t counter_plus_seed, uint32_t beta_id,
                                                  uint32_t &lo, uint32_t &hi) {
@@ -277,22 +280,63 @@ __device__ __forceinline__ bool resolve_codeword(uint32_t word, uint32_t counter
         field[j] = (uint32_t)(int)biased & 31u;
         if (j == 0) { first = s; first_floor = __builtin_floorf(s); }
     }
-    lo = field[0] | (field[1] << 5) | (field[2] << 10) | (field[3] << 15) | (field[4] << 20) |
-         (field[5] << 25) | (beta_id << 30);
+    lo = beta_id | (field[0] << 2) | (field[1] << 7) | (field[2] << 12) | (field[3] << 17) | (field[4] << 22) |
+         (field[5] << 27);
     hi = field[6] | (field[7] << 5) | (first != first_floor ? 1024u : 0u);
     return in_range;
 }
 
-__device__ __forceinline__ void decode_resolved(uint32_t lo, uint32_t hi, uint32_t counter_plus_seed,
+// x * c + a, low 32 bits, as one instruction (c and a are the same for every lane).
+__device__ __forceinline__ uint32_t mad_u32(uint32_t x, uint32_t c, uint64_t a) {
+    uint64_t r;
+    asm("v_mad_u64_u32 %0, vcc, %1, %2, %3" : "=v"(r) : "v"(x), "s"(c), "v"(a) : "vcc");
+    return (uint32_t)r;
+}
+
+// Keeps the compiler from merging a shift with the shifts applied to its result.
+__device__ __forceinline__ uint32_t as_computed(uint32_t x) {
+    asm("" : "+v"(x));
+    return x;
+}
+
+__device__ __forceinline__ uint32_t resolved_beta_id(uint32_t lo) { return lo & 3u; }
+
+// out[j] = (s_j - u_j) * 2^17 * scale  (pass scale = weight scale * kResolvedUnit).
+// The hash is evaluated on values shifted left by one bit, so that "modulo 2^31" is the
+// register's own wrap-around: stage 1 is t (2 A) + 2 C, the second shift-xor masks bit 0, stage 2
+// multiplies by -B and adds -3, which leaves the complement of (v B + 1) << 1, whose top 18 bits
+// are 2^18 - 1 - U.  The last shift-xor of lcg31_mix_v1 only touches bits 0..14 of the value: two
+// of the 18 bits used here (13 and 14), which then carry an unmixed but equally uniform bit.
+// The eight counters of a block share bits 16..30 unless the block straddles a multiple of 2^16
+// (or of 2^31): those blocks take the counter-by-counter form of the first shift-xor.
+__device__ __forceinline__ void decode_resolved(uint32_t lo, uint32_t hi, uint32_t counter_plus_seed, float scale,
                                                 float (&out)[8]) {
-    // (half ? 2^25 : 0) - 15 * 2^26, wrapping like the sums below
-    const uint32_t base = ((hi << 15) & (1u << 25)) - (15u << 26);
+    const uint32_t base = counter_plus_seed & 0x7fffffffu;
+    const uint32_t high = base >> 16;
+    // 2^23 + (2^18 - 1) + 15 * 2^17, less 2^16 in the half-integer coset
+    const float origin = (hi & 1024u) ? 10551295.0f : 10616831.0f;
+    const uint32_t low_fields = as_computed(lo << 15), tail_fields = as_computed(hi << 17);
+    const uint32_t field[8] = {low_fields, low_fields >> 5, low_fields >> 10, lo, lo >> 5, lo >> 10,
+                               tail_fields, tail_fields >> 5};
+    uint32_t t[8];
+    if (__builtin_expect((base & 0xffffu) > 0xfff8u || base > 0x7ffffff8u, 0)) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t x = (counter_plus_seed + (uint32_t)j) & 0x7fffffffu;
+            t[j] = x ^ (x >> 16);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) t[j] = (base + (uint32_t)j) ^ high;
+    }
+    const uint64_t twice_c = 2u * 12345u;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-        const uint32_t field = j < 6 ? (lo >> (5 * j)) & 31u : (hi >> (5 * (j - 6))) & 31u;
-        const uint32_t point = (field << 26) + base;                                    // s_j * 2^26
-        const uint32_t uniform = (lcg31_mix_bits(counter_plus_seed + (uint32_t)j) >> 4) & 0x7ffffffu;
-        out[j] = (float)(int32_t)(point - uniform);
+        const uint32_t v1 = mad_u32(t[j], 2u * 1103515245u, twice_c);
+        const uint32_t v1x = v1 ^ ((v1 >> 13) & 0x7fffeu);
+        const uint32_t v2_complement = v1x * (0u - 134775813u) - 3u;
+        const uint32_t bits = ((field[j] & (31u << 17)) | 0x4b000000u) + (v2_complement >> 14);
+        out[j] = (__uint_as_float(bits) - origin) * scale;
     }
 }
 

@@ -126,16 +126,16 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
         }
         if (s < steps) {
             float v[8];
-            float scale;
             if (kResolved) {
-                decode_resolved(word, side, seed_plus_offset + (uint32_t)g * 8u, v);
-                scale = wbeta[word >> 30] * wscale;
+                decode_resolved(word, side, seed_plus_offset + (uint32_t)g * 8u, wbeta[resolved_beta_id(word)] * wscale, v);
             } else {
                 decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
-                scale = wbeta[(side >> (2 * (g & 3))) & 3] * wscale;
+                const float scale = wbeta[(side >> (2 * (g & 3))) & 3] * wscale;
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = v[j] * scale;
             }
-            const bf16x2 h0 = pack_bf16x2(v[0] * scale, v[1] * scale), h1 = pack_bf16x2(v[2] * scale, v[3] * scale);
-            const bf16x2 h2 = pack_bf16x2(v[4] * scale, v[5] * scale), h3 = pack_bf16x2(v[6] * scale, v[7] * scale);
+            const bf16x2 h0 = pack_bf16x2(v[0], v[1]), h1 = pack_bf16x2(v[2], v[3]);
+            const bf16x2 h2 = pack_bf16x2(v[4], v[5]), h3 = pack_bf16x2(v[6], v[7]);
             *((s & 1) ? dec_slot1 : dec_slot0) =
                 make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
                            __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
@@ -179,16 +179,18 @@ decode_weight_kernel(const uint32_t *__restrict__ w_words, const uint16_t *__res
     const int64_t row = g / blocks_per_row;
     const uint32_t word = w_words[g];
     const float unit = w_norms[row] / sqrt_k;
-    float v[8], scale;
+    float v[8];
     if (kResolved) {
-        decode_resolved(word, w_tails[g], seed_plus_offset + (uint32_t)g * 8u, v);
-        scale = w_betas[word >> 30] * (unit * kResolvedUnit);
+        decode_resolved(word, w_tails[g], seed_plus_offset + (uint32_t)g * 8u,
+                        w_betas[resolved_beta_id(word)] * (unit * kResolvedUnit), v);
     } else {
         decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
-        scale = w_betas[(w_beta_ids[g >> 2] >> (2 * (g & 3))) & 3] * unit;
+        const float scale = w_betas[(w_beta_ids[g >> 2] >> (2 * (g & 3))) & 3] * unit;
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = v[j] * scale;
     }
-    const bf16x2 h0 = pack_bf16x2(v[0] * scale, v[1] * scale), h1 = pack_bf16x2(v[2] * scale, v[3] * scale);
-    const bf16x2 h2 = pack_bf16x2(v[4] * scale, v[5] * scale), h3 = pack_bf16x2(v[6] * scale, v[7] * scale);
+    const bf16x2 h0 = pack_bf16x2(v[0], v[1]), h1 = pack_bf16x2(v[2], v[3]);
+    const bf16x2 h2 = pack_bf16x2(v[4], v[5]), h3 = pack_bf16x2(v[6], v[7]);
     out[g] = make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
                         __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
 }

@@ -117,17 +117,18 @@ gemv_rows(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8
         for (int r = 0; r < R; r++) {
             const int64_t g = row_first_block[r] + b;
             float v[8];
-            float scale;
             if (kResolved) {
-                decode_resolved(word[r], side[r], seed_plus_offset + (uint32_t)g * 8u, v);
-                scale = wbeta[word[r] >> 30] * wscale[r];
+                decode_resolved(word[r], side[r], seed_plus_offset + (uint32_t)g * 8u,
+                                wbeta[resolved_beta_id(word[r])] * wscale[r], v);
             } else {
                 decode_codeword<true>(word[r], 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
-                scale = wbeta[(side[r] >> (2 * (g & 3))) & 3] * wscale[r];
+                const float scale = wbeta[(side[r] >> (2 * (g & 3))) & 3] * wscale[r];
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = v[j] * scale;
             }
             bf16x2 w[4];
 #pragma unroll
-            for (int j = 0; j < 4; j++) w[j] = pack_bf16x2(v[2 * j] * scale, v[2 * j + 1] * scale);
+            for (int j = 0; j < 4; j++) w[j] = pack_bf16x2(v[2 * j], v[2 * j + 1]);
 #pragma unroll
             for (int m = 0; m < M; m++) {
                 acc[r][m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].x), w[0], acc[r][m], false);
@@ -289,10 +290,10 @@ w4a4_gemv_mfma_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, 
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             float v[8];
-            decode_resolved(word[t], tail[t], seed_plus_offset + (uint32_t)(g + t) * 8u, v);
-            const float scale = wbeta[word[t] >> 30] * wscale;
-            const bf16x2 h0 = pack_bf16x2(v[0] * scale, v[1] * scale), h1 = pack_bf16x2(v[2] * scale, v[3] * scale);
-            const bf16x2 h2 = pack_bf16x2(v[4] * scale, v[5] * scale), h3 = pack_bf16x2(v[6] * scale, v[7] * scale);
+            decode_resolved(word[t], tail[t], seed_plus_offset + (uint32_t)(g + t) * 8u,
+                            wbeta[resolved_beta_id(word[t])] * wscale, v);
+            const bf16x2 h0 = pack_bf16x2(v[0], v[1]), h1 = pack_bf16x2(v[2], v[3]);
+            const bf16x2 h2 = pack_bf16x2(v[4], v[5]), h3 = pack_bf16x2(v[6], v[7]);
             const uint4 a = make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
                                        __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
 #pragma unroll

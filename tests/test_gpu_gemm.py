@@ -121,15 +121,15 @@ def test_long_prefill_decodes_the_weight_once(rt, oracle, k, n_out):
     w_hat = oracle.bf16_round(oracle.dequantize_rows(wc, wb, wn, WEIGHT_BETAS, Q, seed=seed))
     # the kernels form beta * (norm / sqrt(K)) first (the oracle multiplies by beta, then by the
     # row scale): same lattice points, FP32 products that differ in the last place, hence rare
-    # one-step differences after the BF16 rounding.  The resolved form adds at most 2^-26 lattice
+    # one-step differences after the BF16 rounding.  The resolved form takes the dither to 2^-17 lattice
     # units before the scale, which only shows on weights that are themselves almost zero.
     row_peak = np.abs(w_hat).max(axis=1, keepdims=True)
-    for form in (streams_only, weight):
+    for form, deviation, share in ((streams_only, 2.0 ** -22, 500), (weight, 2.0 ** -16, 50)):
         decoded = bits(rt.decode_weight_bf16(form).float())
-        assert np.all(np.abs(decoded - w_hat) <= np.maximum(np.abs(w_hat) * 2.0 ** -7, row_peak * 2.0 ** -22))
-        assert np.count_nonzero(decoded != w_hat) <= decoded.size // 500 + 1
+        assert np.all(np.abs(decoded - w_hat) <= np.abs(w_hat) * 2.0 ** -7 + row_peak * deviation)
+        assert np.count_nonzero(decoded != w_hat) <= decoded.size // share + 1
     from_streams, from_resolved = (bits(rt.decode_weight_bf16(form).float()) for form in (streams_only, weight))
-    assert np.count_nonzero(from_streams != from_resolved) <= from_streams.size // 500 + 1
+    assert np.count_nonzero(from_streams != from_resolved) <= from_streams.size // 50 + 1
 
     m = rt.LIBRARY_GEMM_ROWS + 37
     activation = _activation(rt, oracle, m, k, seed=77)

@@ -151,8 +151,9 @@ def _one_hot_activation(rt, columns, k):
 def test_resolved_weight_decodes_to_the_oracle_weight(rt, oracle, k, n_out, seed):
     """Unit-vector activations read single decoded weights out of the linear kernels.  From the
     resolved form they must be the oracle's dequantized weights after the same BF16 rounding;
-    the resolved arithmetic deviates by at most 2^-26 lattice units before that rounding, so
-    all but a few values agree bit for bit and none is off by more than one BF16 step."""
+    the resolved arithmetic takes the dither to 2^-17 of a lattice unit before that rounding, so
+    nearly all values agree bit for bit and none is off by more than one BF16 step plus that
+    deviation (which only shows on weights that are themselves almost zero)."""
     _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=77 + k, dither_seed=seed)
     resolved = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
     assert resolved.resolved_words is not None and resolved.resolved_words.numel() == n_out * k // 8
@@ -173,11 +174,11 @@ def test_resolved_weight_decodes_to_the_oracle_weight(rt, oracle, k, n_out, seed
         for kernel in ("gemv", "gemm"):
             got = bits(rt._gemv(activation, resolved, split_k=1, output_dtype=torch.float32, kernel=kernel))
             want = w_hat[:, cols].T
-            # one BF16 step is <= 2^-7 relative; weights that are almost zero may move by 2^-26 lattice units
-            step = np.maximum(np.abs(want) * 2.0 ** -7, np.abs(w_hat).max() * 2.0 ** -22)
+            # one BF16 step is <= 2^-7 relative; 2^-17 lattice units are below 2^-16 of a row's peak
+            step = np.abs(want) * 2.0 ** -7 + np.abs(w_hat).max() * 2.0 ** -16
             assert np.all(np.abs(got - want) <= step)
             mismatches += int(np.count_nonzero(got != want))
-    assert mismatches <= 2 * len(columns) * n_out // 1000 + 1
+    assert mismatches <= 2 * len(columns) * n_out // 50 + 1
 
 
 @pytest.mark.parametrize("k,n_out,seed", [(2048, 2048, 20261101), (8192, 256, 5)])
@@ -192,4 +193,5 @@ def test_resolved_and_searching_linears_agree(rt, oracle, k, n_out, seed):
         for kernel in kernels:
             a = bits(rt._gemv(activation, resolved, split_k=0, output_dtype=torch.float32, kernel=kernel))
             b = bits(rt._gemv(activation, searching, split_k=0, output_dtype=torch.float32, kernel=kernel))
-            assert relative_error(a, b) <= 2e-4
+            # same lattice points; the resolved form's 2^-17 dither step flips the BF16 rounding of about 1 % of the weights
+            assert relative_error(a, b) <= 5e-4
