@@ -247,6 +247,9 @@ int nq_w4a4_gemv_grouped(const void *act_decoded_dev, int count, const uint32_t 
  * weight tile is decoded once per call into double-buffered LDS as MFMA B fragments; ragged
  * M is padded to a multiple of 32 with zero rows inside the kernel and M above 512 is
  * processed in chunks of 512 rows.  split_k in {0 (library picks), 1, 2, 4, 8, 16}.
+ * From 288 rows on, with split_k = 0 and BF16 output, the weight is instead decoded once into a
+ * BF16 scratch [N, K] inside the workspace (nq_w4a4_decode_weight) and multiplied by
+ * nq_bf16_gemm; nq_w4a4_gemm_workspace_bytes includes that scratch.
  * Requires q = 14, K % 128 == 0, (K / split_k) % 128 == 0.
  * Replaces: run_m16 / run_large_m_staged of the torch extension
  * (nestquant/runtime/nqrt4_w4a4_mma_binding.cpp:3-46, kernels
@@ -278,6 +281,19 @@ int nq_w4a4_decode_weight(const uint8_t *w_codes_dev, const uint8_t *w_beta_ids_
                           const uint32_t *w_resolved_words_dev, const uint16_t *w_resolved_tails_dev,
                           const float *w_norms_dev, const float *w_betas_dev, int64_t n, int64_t k,
                           int64_t weight_offset, int64_t weight_seed, void *out_bf16_dev, void *stream);
+
+/*
+ * Dense BF16 GEMM on the matrix cores: c[m, n] = sum_k a[m, k] b[n, k], a [M, K] and b [N, K]
+ * row-major BF16 (16-byte aligned), FP32 accumulation, c [M, N] BF16.  K a multiple of 128.
+ * tile = -1 lets the library choose the workgroup tile from the shape; 0..6 force
+ * 256x256, 128x256, 256x128, 128x128, 64x128, 128x64, 64x64 (for measurements).
+ * nq_w4a4_gemm calls it on the weight it has decoded once when M is large; it is exported for
+ * callers that keep a decoded weight themselves.
+ * Replaces: the multiply of run_large_m_staged for long prefills,
+ * nestquant/runtime/nqrt4_w4a4_mma.cu:606-667 (which decodes inside the multiply).
+ */
+int nq_bf16_gemm(const void *a_bf16_dev, const void *b_bf16_dev, int64_t m, int64_t n, int64_t k,
+                 void *c_bf16_dev, int tile, void *stream);
 
 /*
  * NQKV cache, device-resident state.  Per slot (int32[slots]): sequence_lengths,

@@ -1,0 +1,256 @@
+// Dense BF16 GEMM on the matrix cores for long prefills: C[M, N] = A[M, K] * B[N, K]^T, both
+// operands K-contiguous, FP32 accumulation, BF16 out.  A is the decoded NQA4 activation, B the
+// BF16 weight nq_w4a4_decode_weight wrote once for the call, so that a prefill of hundreds or
+// thousands of rows decodes every weight block once and multiplies at matrix-core speed.
+//
+// Tiling.  A workgroup of four wavefronts (2 x 2) owns a (64 WM) x (64 WN) tile of C; each
+// wavefront owns WM x WN tiles of 32 x 32 (v_mfma_f32_32x32x16_bf16), e.g. 4 x 4 = 128 x 128 with
+// 256 accumulator registers.  K is walked in steps of 64: the A and B slabs of a step sit in LDS
+// as rows of 128 bytes whose eight 16-byte pieces are stored at piece ^ ((row / 2) % 8).  The LDS
+// has 64 banks and serves sixteen lanes of a 16-byte read per cycle: sixteen consecutive rows of
+// one fragment read (lane l: row l % 32, piece 2 s + l / 32) then fall on sixteen different groups
+// of four banks (even rows in one half of the banks, odd rows in the other, eight different pieces
+// in each), and so do the eight lanes that store one row.  LDS is double-buffered: the loads of step s + 1 are
+// requested before the products of step s and stored after them, one barrier per step.
+// Workgroups are numbered so that the ones that run together on one XCD (every eighth) form a
+// compact block of tiles, i.e. share rows of A and of B in that XCD's L2.
+// Replaces (together with nq_w4a4_decode_weight): run_large_m_staged and the chunk-and-pad wrapper for
+// M beyond a few hundred rows, nestquant/runtime/nqrt4_w4a4_mma.cu:606-667 and
+// nestquant/runtime/cuda_w4a4_mma.py:450-474.
+#include "nq_host.h"
+
+#include <stdint.h>
+
+namespace nq {
+
+typedef __bf16 gemm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float gemm_floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // a native vector: stays in registers across the loop
+
+constexpr int kDenseBK = 64;
+
+__device__ __forceinline__ uint16_t dense_f32_to_bf16(float x) {
+    uint32_t bits = __float_as_uint(x);
+    bits += 0x7fffu + ((bits >> 16) & 1u);
+    return (uint16_t)(bits >> 16);
+}
+
+// WM x WN: 32 x 32 tiles per wavefront; GM x GN: wavefronts per workgroup along M and N.
+template <int WM, int WN, int GM, int GN>
+__global__ void __launch_bounds__(64 * GM * GN)
+bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b, uint16_t *__restrict__ c,
+                 int m_size, int n_size, int k_size, int tiles_m, int tiles_n, int group_m) {
+    constexpr int kThreads = 64 * GM * GN;
+    constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN;
+    constexpr int kRowsPerPass = kThreads / 8;                     // rows one pass of 16-byte loads covers
+    constexpr int kLoadsA = BM / kRowsPerPass, kLoadsB = BN / kRowsPerPass;
+    static_assert(BM % kRowsPerPass == 0 && BN % kRowsPerPass == 0 && kRowsPerPass % 8 == 0, "tile and workgroup shapes");
+    extern __shared__ u32x4 lds[];                                 // [2][BM + BN][8] pieces
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave / GN, wave_n = wave % GN;
+
+    // tile of this workgroup: every eighth workgroup shares an XCD; within an XCD's share, tiles are
+    // walked in groups of group_m rows of tiles so that neighbours in time share operands
+    int pid = blockIdx.x;
+    const int total = tiles_m * tiles_n;
+    if (total % 8 == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+    const int per_group = group_m * tiles_n;
+    const int group = pid / per_group, first_m = group * group_m;
+    const int rows_in_group = tiles_m - first_m < group_m ? tiles_m - first_m : group_m;
+    const int in_group = pid - group * per_group;
+    const int tile_m = first_m + in_group % rows_in_group, tile_n = in_group / rows_in_group;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    // global -> LDS role: piece (tid & 7) of rows (tid >> 3) + kRowsPerPass i
+    const int load_row = tid >> 3, load_piece = tid & 7;
+    const int store_slot = load_row * 8 + (load_piece ^ ((load_row >> 1) & 7));
+    int a_offset[kLoadsA], b_offset[kLoadsB];                      // in elements, below 2^31 (checked by the host)
+#pragma unroll
+    for (int i = 0; i < kLoadsA; i++) {
+        const int row = m0 + load_row + kRowsPerPass * i;
+        a_offset[i] = (row < m_size ? row : m_size - 1) * k_size + load_piece * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < kLoadsB; i++) {
+        const int row = n0 + load_row + kRowsPerPass * i;
+        b_offset[i] = (row < n_size ? row : n_size - 1) * k_size + load_piece * 8;
+    }
+
+    // fragment role: A rows wave_m * 32 WM + 32 i + lane % 32, B rows likewise; piece 2 s + lane / 32
+    const int frag_row = lane & 31, frag_half = lane >> 5, frag_mask = (lane >> 1) & 7;
+    const int a_frag_base = (wave_m * 32 * WM + frag_row) * 8;
+    const int b_frag_base = (BM + wave_n * 32 * WN + frag_row) * 8;
+
+    gemm_floatx16 acc[WM][WN];
+#pragma unroll
+    for (int i = 0; i < WM; i++)
+#pragma unroll
+        for (int j = 0; j < WN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    // Slabs are requested two steps ahead: registers `early` hold slab s + 1 (requested a step ago,
+    // stored to LDS at the end of step s), registers `late` receive slab s + 2 at the top of step s.
+    // A step of 64 k lasts about as long as a trip to the L2 and back under load, so one step of
+    // lead leaves the matrix cores waiting for the stores.
+    const int steps = k_size / kDenseBK;
+    u32x4 pa0[kLoadsA], pa1[kLoadsA], pb0[kLoadsB], pb1[kLoadsB];
+    {
+        u32x4 ra[kLoadsA], rb[kLoadsB];
+#pragma unroll
+        for (int i = 0; i < kLoadsA; i++) ra[i] = *reinterpret_cast<const u32x4 *>(a + a_offset[i]);
+#pragma unroll
+        for (int i = 0; i < kLoadsB; i++) rb[i] = *reinterpret_cast<const u32x4 *>(b + b_offset[i]);
+        const int k_one = steps > 1 ? kDenseBK : 0;
+#pragma unroll
+        for (int i = 0; i < kLoadsA; i++) pa1[i] = *reinterpret_cast<const u32x4 *>(a + a_offset[i] + k_one);
+#pragma unroll
+        for (int i = 0; i < kLoadsB; i++) pb1[i] = *reinterpret_cast<const u32x4 *>(b + b_offset[i] + k_one);
+#pragma unroll
+        for (int i = 0; i < kLoadsA; i++) lds[store_slot + kRowsPerPass * 8 * i] = ra[i];
+#pragma unroll
+        for (int i = 0; i < kLoadsB; i++) lds[BM * 8 + store_slot + kRowsPerPass * 8 * i] = rb[i];
+    }
+    __syncthreads();
+
+    // one step: request slab step + 2 into set `late`, multiply slab `step` from LDS, store set `early`
+    // (slab step + 1) into the other LDS buffer
+    auto dense_step = [&](int step, u32x4 (&late_a)[kLoadsA], u32x4 (&late_b)[kLoadsB],
+                          const u32x4 (&early_a)[kLoadsA], const u32x4 (&early_b)[kLoadsB]) {
+        const u32x4 *now = lds + (step & 1) * (BM + BN) * 8;
+        u32x4 *next = lds + ((step + 1) & 1) * (BM + BN) * 8;
+        const int ahead = step + 2 < steps ? step + 2 : steps - 1;      // past the end: any valid slab
+#pragma unroll
+        for (int i = 0; i < kLoadsA; i++) late_a[i] = *reinterpret_cast<const u32x4 *>(a + a_offset[i] + ahead * kDenseBK);
+#pragma unroll
+        for (int i = 0; i < kLoadsB; i++) late_b[i] = *reinterpret_cast<const u32x4 *>(b + b_offset[i] + ahead * kDenseBK);
+        // fragments of sub-step s + 1 are read while the products of sub-step s run
+        gemm_bf16x8 fa[2][WM], fb[2][WN];
+#pragma unroll
+        for (int i = 0; i < WM; i++) fa[0][i] = __builtin_bit_cast(gemm_bf16x8, now[a_frag_base + 256 * i + (frag_half ^ frag_mask)]);
+#pragma unroll
+        for (int j = 0; j < WN; j++) fb[0][j] = __builtin_bit_cast(gemm_bf16x8, now[b_frag_base + 256 * j + (frag_half ^ frag_mask)]);
+#pragma unroll
+        for (int s = 0; s < kDenseBK / 16; s++) {
+            if (s + 1 < kDenseBK / 16) {
+                const int piece = (2 * (s + 1) + frag_half) ^ frag_mask;
+#pragma unroll
+                for (int i = 0; i < WM; i++)
+                    fa[(s + 1) & 1][i] = __builtin_bit_cast(gemm_bf16x8, now[a_frag_base + 256 * i + piece]);
+#pragma unroll
+                for (int j = 0; j < WN; j++)
+                    fb[(s + 1) & 1][j] = __builtin_bit_cast(gemm_bf16x8, now[b_frag_base + 256 * j + piece]);
+            }
+#pragma unroll
+            for (int i = 0; i < WM; i++)
+#pragma unroll
+                for (int j = 0; j < WN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
+        }
+        // (after the last step this stores a slab nobody reads, into the buffer nobody is reading)
+#pragma unroll
+        for (int i = 0; i < kLoadsA; i++) next[store_slot + kRowsPerPass * 8 * i] = early_a[i];
+#pragma unroll
+        for (int i = 0; i < kLoadsB; i++) next[BM * 8 + store_slot + kRowsPerPass * 8 * i] = early_b[i];
+        __syncthreads();
+    };
+    for (int step = 0; step < steps; step += 2) {          // the host checks that the step count is even
+        dense_step(step, pa0, pb0, pa1, pb1);
+        dense_step(step + 1, pa1, pb1, pa0, pb0);
+    }
+
+    // accumulator r of lane l: row (r % 4) + 8 (r / 4) + 4 (l / 32) of the 32 x 32 tile, column l % 32
+#pragma unroll
+    for (int i = 0; i < WM; i++) {
+        const int row_base = m0 + wave_m * 32 * WM + 32 * i + 4 * frag_half;
+#pragma unroll
+        for (int j = 0; j < WN; j++) {
+            const int col = n0 + wave_n * 32 * WN + 32 * j + frag_row;
+            if (col < n_size) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = row_base + (r & 3) + 8 * (r >> 2);
+                    if (row < m_size) c[(int64_t)row * n_size + col] = dense_f32_to_bf16(acc[i][j][r]);
+                }
+            }
+        }
+    }
+}
+
+}  // namespace nq
+
+namespace {
+
+struct DenseTile { int bm, bn; float efficiency; };
+
+// Workgroup tiles from the fastest per product to the slowest; `efficiency` is the measured rate
+// relative to the 256 x 256 tile on a problem that fills the chip (8192^3: 1.13, 0.92, 0.92, 0.93,
+// 0.74, 0.74, 0.61 PFLOP/s).
+const DenseTile kDenseTiles[] = {
+    {256, 256, 1.00f}, {128, 256, 0.81f}, {256, 128, 0.81f}, {128, 128, 0.82f}, {64, 128, 0.65f}, {128, 64, 0.65f},
+    {64, 64, 0.55f},
+};
+
+template <int WM, int WN, int GM, int GN>
+void launch_dense(const void *a, const void *b, void *c, int m, int n, int k, hipStream_t stream) {
+    constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN;
+    const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+    const size_t lds_bytes = (size_t)2 * (BM + BN) * 128;
+    static bool raised = false;                  // once per process: permission for more than 64 KiB of LDS
+    if (!raised) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(nq::bf16_gemm_kernel<WM, WN, GM, GN>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        raised = true;
+    }
+    const int group_m = tiles_m < 4 ? tiles_m : 4;
+    hipLaunchKernelGGL((nq::bf16_gemm_kernel<WM, WN, GM, GN>), dim3((unsigned)(tiles_m * tiles_n)), dim3(64 * GM * GN),
+                       lds_bytes, stream, reinterpret_cast<const uint16_t *>(a), reinterpret_cast<const uint16_t *>(b),
+                       reinterpret_cast<uint16_t *>(c), m, n, k, tiles_m, tiles_n, group_m);
+}
+
+}  // namespace
+
+namespace nq {
+
+// Shared with nq_w4a4_gemm: picks the tile shape with the least estimated time and launches.
+int launch_bf16_gemm(const void *a, const void *b, void *c, int m, int n, int k, int forced_tile, hipStream_t stream) {
+    int best = 0;
+    float best_cost = 0.0f;
+    const int count = (int)(sizeof(kDenseTiles) / sizeof(kDenseTiles[0]));
+    for (int t = 0; t < count; t++) {
+        const DenseTile &tile = kDenseTiles[t];
+        const int64_t tiles = (int64_t)((m + tile.bm - 1) / tile.bm) * ((n + tile.bn - 1) / tile.bn);
+        // the busiest of the 256 compute units works through ceil(tiles / 256) tiles, whether one
+        // after the other or side by side at a share of its rate
+        const float cost = (float)((tiles + 255) / 256) * (float)(tile.bm * tile.bn) / tile.efficiency;
+        if (t == 0 || cost < best_cost) { best = t; best_cost = cost; }
+    }
+    if (forced_tile >= 0 && forced_tile < count) best = forced_tile;
+    switch (best) {
+        case 0: launch_dense<2, 4, 4, 2>(a, b, c, m, n, k, stream); break;
+        case 1: launch_dense<2, 4, 2, 2>(a, b, c, m, n, k, stream); break;
+        case 2: launch_dense<4, 2, 2, 2>(a, b, c, m, n, k, stream); break;
+        case 3: launch_dense<2, 2, 2, 2>(a, b, c, m, n, k, stream); break;
+        case 4: launch_dense<1, 2, 2, 2>(a, b, c, m, n, k, stream); break;
+        case 5: launch_dense<2, 1, 2, 2>(a, b, c, m, n, k, stream); break;
+        default: launch_dense<1, 1, 2, 2>(a, b, c, m, n, k, stream); break;
+    }
+    return check_launch("nq_bf16_gemm");
+}
+
+}  // namespace nq
+
+extern "C" int nq_bf16_gemm(const void *a_bf16_dev, const void *b_bf16_dev, int64_t m, int64_t n, int64_t k,
+                            void *c_bf16_dev, int tile, void *stream) {
+    NQ_REQUIRE(m >= 1 && n >= 1 && m < ((int64_t)1 << 30) && n < ((int64_t)1 << 30), NQ_ERR_SHAPE,
+               "nq_bf16_gemm: M and N must be positive");
+    NQ_REQUIRE(k >= 2 * nq::kDenseBK && k % (2 * nq::kDenseBK) == 0 && k < ((int64_t)1 << 30), NQ_ERR_SHAPE,
+               "nq_bf16_gemm: K = %lld must be a positive multiple of 128", (long long)k);
+    NQ_REQUIRE(a_bf16_dev && b_bf16_dev && c_bf16_dev, NQ_ERR_ARGUMENT, "nq_bf16_gemm: null pointer");
+    NQ_REQUIRE(nq::aligned(a_bf16_dev, 16) && nq::aligned(b_bf16_dev, 16) && nq::aligned(c_bf16_dev, 2), NQ_ERR_ARGUMENT,
+               "nq_bf16_gemm: operands must be 16-byte aligned");
+    NQ_REQUIRE(m * k < ((int64_t)1 << 31) && n * k < ((int64_t)1 << 31), NQ_ERR_SHAPE,
+               "nq_bf16_gemm: operands of 2^31 elements or more are not supported");
+    NQ_REQUIRE(tile >= -1 && tile <= 6, NQ_ERR_ARGUMENT, "nq_bf16_gemm: tile must be -1 (automatic) or 0..6");
+    return nq::launch_bf16_gemm(a_bf16_dev, b_bf16_dev, c_bf16_dev, (int)m, (int)n, (int)k, tile, (hipStream_t)stream);
+}

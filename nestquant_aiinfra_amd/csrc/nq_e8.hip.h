@@ -309,15 +309,10 @@ __device__ __forceinline__ uint32_t resolved_beta_id(uint32_t lo) { return lo & 
 // of the 18 bits used here (13 and 14), which then carry an unmixed but equally uniform bit.
 // The eight counters of a block share bits 16..30 unless the block straddles a multiple of 2^16
 // (or of 2^31): those blocks take the counter-by-counter form of the first shift-xor.
-__device__ __forceinline__ void decode_resolved(uint32_t lo, uint32_t hi, uint32_t counter_plus_seed, float scale,
-                                                float (&out)[8]) {
+// The part of the decode that needs no memory: bits[j] = 2^18 - 1 - U_j from the counters alone.
+__device__ __forceinline__ void resolved_dither_bits(uint32_t counter_plus_seed, uint32_t (&bits)[8]) {
     const uint32_t base = counter_plus_seed & 0x7fffffffu;
     const uint32_t high = base >> 16;
-    // 2^23 + (2^18 - 1) + 15 * 2^17, less 2^16 in the half-integer coset
-    const float origin = (hi & 1024u) ? 10551295.0f : 10616831.0f;
-    const uint32_t low_fields = as_computed(lo << 15), tail_fields = as_computed(hi << 17);
-    const uint32_t field[8] = {low_fields, low_fields >> 5, low_fields >> 10, lo, lo >> 5, lo >> 10,
-                               tail_fields, tail_fields >> 5};
     uint32_t t[8];
     if (__builtin_expect((base & 0xffffu) > 0xfff8u || base > 0x7ffffff8u, 0)) {
 #pragma unroll
@@ -335,9 +330,30 @@ __device__ __forceinline__ void decode_resolved(uint32_t lo, uint32_t hi, uint32
         const uint32_t v1 = mad_u32(t[j], 2u * 1103515245u, twice_c);
         const uint32_t v1x = v1 ^ ((v1 >> 13) & 0x7fffeu);
         const uint32_t v2_complement = v1x * (0u - 134775813u) - 3u;
-        const uint32_t bits = ((field[j] & (31u << 17)) | 0x4b000000u) + (v2_complement >> 14);
-        out[j] = (__uint_as_float(bits) - origin) * scale;
+        bits[j] = v2_complement >> 14;
     }
+}
+
+// The part that needs the stored block: out[j] = (s_j - u_j) * 2^17 * scale.
+__device__ __forceinline__ void resolved_apply(uint32_t lo, uint32_t hi, const uint32_t (&bits)[8], float scale,
+                                               float (&out)[8]) {
+    // 2^23 + (2^18 - 1) + 15 * 2^17, less 2^16 in the half-integer coset
+    const float origin = (hi & 1024u) ? 10551295.0f : 10616831.0f;
+    const uint32_t low_fields = as_computed(lo << 15), tail_fields = as_computed(hi << 17);
+    const uint32_t field[8] = {low_fields, low_fields >> 5, low_fields >> 10, lo, lo >> 5, lo >> 10,
+                               tail_fields, tail_fields >> 5};
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t pattern = ((field[j] & (31u << 17)) | 0x4b000000u) + bits[j];
+        out[j] = (__uint_as_float(pattern) - origin) * scale;
+    }
+}
+
+__device__ __forceinline__ void decode_resolved(uint32_t lo, uint32_t hi, uint32_t counter_plus_seed, float scale,
+                                                float (&out)[8]) {
+    uint32_t bits[8];
+    resolved_dither_bits(counter_plus_seed, bits);
+    resolved_apply(lo, hi, bits, scale, out);
 }
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t bits) {

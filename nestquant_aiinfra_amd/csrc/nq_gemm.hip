@@ -197,9 +197,19 @@ decode_weight_kernel(const uint32_t *__restrict__ w_words, const uint16_t *__res
 
 }  // namespace nq
 
+namespace nq {
+int launch_bf16_gemm(const void *a, const void *b, void *c, int m, int n, int k, int forced_tile, hipStream_t stream);
+}
+
 namespace {
 
 constexpr int kChunkRows = 512;    // 8 wavefronts x 2 tiles x 32 rows
+// From this many rows on (BF16 output, automatic split) the weight is decoded once into a BF16
+// scratch [N][K] in the workspace and a dense BF16 GEMM multiplies: the fused kernel decodes a
+// block once per 512 rows and re-reads the activation once per 32 channels.
+constexpr int kDecodeOnceRows = 288;
+
+bool decodes_once(int m, int k, int split_k) { return split_k == 0 && m >= kDecodeOnceRows && k % 128 == 0; }
 
 // enough workgroups for 256 CUs; slabs stay multiples of 128
 int pick_gemm_split(int k, int n, int requested) {
@@ -217,9 +227,12 @@ extern "C" size_t nq_w4a4_gemm_workspace_bytes(int m, int k, int n, int split_k,
     const int split = pick_gemm_split(k, n, split_k);
     size_t bytes = 0;
     if (!have_decoded_activation) bytes += nq::align256((size_t)m * k * 2);
+    // the output dtype is not known here: enough for the decode-once scratch (BF16 output) and for the
+    // fused kernel's partial sums (FP32 output) alike
     const int chunk = m < kChunkRows ? m : kChunkRows;
-    if (split > 1) bytes += (size_t)split * (size_t)chunk * (size_t)n * sizeof(float);
-    return bytes;
+    const size_t partials = split > 1 ? (size_t)split * (size_t)chunk * (size_t)n * sizeof(float) : 0;
+    const size_t scratch = decodes_once(m, k, split_k) ? nq::align256((size_t)n * k * 2) : 0;
+    return bytes + (scratch > partials ? scratch : partials);
 }
 
 extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
@@ -252,12 +265,14 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
                "nq_w4a4_gemm: seed must be in [0, 2**31)");
     NQ_REQUIRE(weight_offset >= 0 && weight_offset + (int64_t)n * (k / 8) <= ((int64_t)1 << 28),
                NQ_ERR_SHAPE, "nq_w4a4_gemm: block range exceeds the stateless dither counter space");
-    const int split = pick_gemm_split(k, n, split_k);
+    const bool once = decodes_once(m, k, split_k) && out_dtype == NQ_BF16;
+    const int split = once ? 1 : pick_gemm_split(k, n, split_k);
     NQ_REQUIRE(k % split == 0 && (k / split) % nq::kGemmBK == 0, NQ_ERR_SHAPE,
                "nq_w4a4_gemm: K / split_k = %d / %d must be a multiple of 128", k, split);
     const int chunk_rows = m < kChunkRows ? m : kChunkRows;
     const size_t decoded_bytes = act_decoded_dev ? 0 : nq::align256((size_t)m * k * 2);
-    const size_t need = decoded_bytes + (split > 1 ? (size_t)split * chunk_rows * n * sizeof(float) : 0);
+    const size_t need = decoded_bytes + (once ? nq::align256((size_t)n * k * 2)
+                                              : (split > 1 ? (size_t)split * chunk_rows * n * sizeof(float) : 0));
     NQ_REQUIRE(need == 0 || (workspace_dev && workspace_bytes >= need), NQ_ERR_WORKSPACE,
                "nq_w4a4_gemm: needs a %zu-byte workspace, got %zu", need, workspace_bytes);
     NQ_REQUIRE(need == 0 || nq::aligned(workspace_dev, 16), NQ_ERR_ARGUMENT,
@@ -272,6 +287,14 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
         act = reinterpret_cast<const uint16_t *>(workspace_dev);
     }
     float *partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace_dev) + decoded_bytes);
+    if (once) {
+        void *weight_bf16 = partials;
+        const int status = nq_w4a4_decode_weight(w_codes_dev, w_beta_ids_dev, w_resolved_words_dev, w_resolved_tails_dev,
+                                                 w_norms_dev, w_betas_dev, n, k, weight_offset, weight_seed, weight_bf16,
+                                                 stream);
+        if (status != NQ_OK) return status;
+        return nq::launch_bf16_gemm(act, weight_bf16, out_dev, m, n, k, -1, s);
+    }
     const uint32_t seed_plus_offset = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
     const float sqrt_k = (float)sqrt((double)k);
     const dim3 grid((unsigned)((n + nq::kGemmBN - 1) / nq::kGemmBN), (unsigned)split);

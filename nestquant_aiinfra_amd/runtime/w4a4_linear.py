@@ -420,6 +420,24 @@ def can_use_w4a4_mma_chunked_staged(activation: PreparedNQA4Activation,
 # linear kernels, M = 1..8
 # --------------------------------------------------------------------------------------
 
+# Workspaces above this size (the BF16 scratch of a decode-once prefill: 33 MB for gate_proj) are
+# kept per device and stream and reused by later calls there; smaller ones are allocated
+# per call from torch's caching allocator, which is what a captured graph wants.
+_KEPT_WORKSPACE_BYTES = 4 << 20
+_kept_workspaces: dict[tuple[int | None, int], torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, need: int) -> torch.Tensor:
+    if need < _KEPT_WORKSPACE_BYTES or torch.cuda.is_current_stream_capturing():
+        return torch.empty(need, dtype=torch.uint8, device=device)
+    key = (device.index, _native.stream_handle(device))
+    kept = _kept_workspaces.get(key)
+    if kept is None or kept.numel() < need:
+        kept = torch.empty(need, dtype=torch.uint8, device=device)
+        _kept_workspaces[key] = kept
+    return kept
+
+
 def _gemv(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *, split_k: int,
           output_dtype: torch.dtype, kernel: str = "gemv") -> torch.Tensor:
     lib = _native.library()
@@ -431,7 +449,7 @@ def _gemv(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *, spl
     out = torch.empty((m, n), dtype=output_dtype, device=device)
     decoded = activation.decoded
     need = workspace_bytes(m, k, n, split_k, int(decoded is not None))
-    workspace = torch.empty(need, dtype=torch.uint8, device=device) if need else None
+    workspace = _workspace(device, need) if need else None
     _native.check(launch(
         activation.code_payload.data_ptr(), activation.beta_payload.data_ptr(),
         activation.row_norms.data_ptr(), activation.beta_table.data_ptr(),
@@ -544,12 +562,11 @@ def linear_packed_w4a4_mma_small_m_splitk_probe(activation: PreparedNQA4Activati
 # linear kernels, prefill (matrix cores)
 # --------------------------------------------------------------------------------------
 
-# From this many rows on (BF16 output, automatic split) a packed linear decodes its weight once
-# into a BF16 scratch (nq_w4a4_decode_weight) and hands the plain BF16 GEMM to the BLAS library
-# behind torch.matmul.  The fused kernel decodes a block once per 512 rows but re-reads the
-# activation once per 32 channels, which is what it waits for beyond a few hundred rows;
-# measured crossover on MI355X at the 1B shapes: between 256 and 384 rows.
-LIBRARY_GEMM_ROWS = 288
+# From this many rows on (BF16 output, automatic split) nq_w4a4_gemm decodes the weight once into a
+# BF16 scratch inside its workspace and multiplies with the dense matrix-core GEMM of the library
+# (nq_bf16_gemm); below, the fused kernel decodes inside the multiply.  Measured crossover on MI355X
+# at the 1B shapes: between 256 and 384 rows.
+DECODE_ONCE_ROWS = 288
 # up to this many rows a linear over resolved weights (K a multiple of 128) takes the decode GEMV,
 # which from five rows on multiplies on the matrix cores
 MATRIX_CORE_GEMV_ROWS = 16
@@ -611,18 +628,25 @@ def bf16_rows_linear_grouped(rows: torch.Tensor, weight: torch.Tensor, sizes: Se
 def _gemm(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *,
           output_dtype: torch.dtype | None = None, split_k: int = 0) -> torch.Tensor:
     dtype = _kernel_dtype(activation) if output_dtype is None else output_dtype
-    if (dtype == torch.bfloat16 and split_k == 0 and activation.token_count >= LIBRARY_GEMM_ROWS
-            and activation.feature_count % 32 == 0):
-        rows = activation.decoded
-        if rows is None:
-            rows = decode_packed_a4(activation, output_dtype=torch.bfloat16).reshape(-1, activation.feature_count)
-        out = torch.matmul(rows, decode_weight_bf16(weight).t())
-        return out.reshape(*activation.original_shape[:-1], out.shape[-1])
     if (split_k == 0 and activation.token_count <= MATRIX_CORE_GEMV_ROWS and weight.resolved_words is not None
             and activation.feature_count % 128 == 0):
         # up to sixteen rows the decode-in-register kernel feeds the matrix cores directly
         return _gemv(activation, weight, split_k=0, output_dtype=dtype)
     return _gemv(activation, weight, split_k=split_k, output_dtype=dtype, kernel="gemm")
+
+
+def bf16_gemm(rows: torch.Tensor, weight: torch.Tensor, *, tile: int = -1) -> torch.Tensor:
+    """`rows @ weight.T` for BF16 [M, K] and [N, K] (K a multiple of 128) on the library's dense
+    matrix-core GEMM, FP32 accumulation, BF16 out.  `tile` forces a workgroup tile (measurements)."""
+    device = _native.require_cuda(rows, weight)
+    if rows.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or rows.ndim != 2 or weight.ndim != 2:
+        raise TypeError("bf16_gemm takes two BF16 matrices")
+    if rows.shape[1] != weight.shape[1]:
+        raise ValueError("operands disagree on K")
+    out = torch.empty((rows.shape[0], weight.shape[0]), dtype=torch.bfloat16, device=device)
+    _native.check(_native.library().nq_bf16_gemm(rows.data_ptr(), weight.data_ptr(), rows.shape[0], weight.shape[0],
+                                                 rows.shape[1], out.data_ptr(), tile, _native.stream_handle(device)))
+    return out
 
 
 def linear_packed_w4a4_mma_m16(activation: PreparedNQA4Activation,

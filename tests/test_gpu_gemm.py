@@ -87,6 +87,11 @@ def test_llama_1b_prefill_shapes(rt, oracle, name, k, n_out, wseed, dseed):
         y = rt.linear_packed_w4a4_mma_chunked_staged(activation, weight)
         assert y.dtype == torch.bfloat16 and tuple(y.shape) == (m, n_out)
         assert relative_error(bits(y.float())[:, rows], ref32) <= TOLERANCE, (name, m)
+        if m == 384:
+            # 384 rows take the decode-once route by default; an explicit single slice keeps the fused
+            # kernel (the weight decoded inside the multiply): both must meet the oracle
+            fused = rt._gemm(activation, weight, output_dtype=torch.bfloat16, split_k=1)
+            assert relative_error(bits(fused.float())[:, rows], ref32) <= TOLERANCE, (name, m, "fused")
 
 
 def test_slice_and_pad_matches_reference_chunking(rt, oracle):
@@ -108,8 +113,8 @@ def test_slice_and_pad_matches_reference_chunking(rt, oracle):
 
 @pytest.mark.parametrize("k,n_out", [(2048, 2048), (512, 200)])
 def test_long_prefill_decodes_the_weight_once(rt, oracle, k, n_out):
-    """From LIBRARY_GEMM_ROWS rows on, BF16 outputs come from nq_w4a4_decode_weight + a library
-    GEMM: the decoded weight equals the oracle's BF16-rounded weight (resolved form: but for
+    """From DECODE_ONCE_ROWS rows on, BF16 outputs come from nq_w4a4_decode_weight + the dense
+    matrix-core GEMM inside nq_w4a4_gemm: the decoded weight equals the oracle's BF16-rounded weight (resolved form: but for
     rare one-step roundings) and the product stays within the bar; below the threshold and for
     FP32 outputs the fused kernel runs."""
     from test_gpu_gemv import _record
@@ -131,7 +136,7 @@ def test_long_prefill_decodes_the_weight_once(rt, oracle, k, n_out):
     from_streams, from_resolved = (bits(rt.decode_weight_bf16(form).float()) for form in (streams_only, weight))
     assert np.count_nonzero(from_streams != from_resolved) <= from_streams.size // 50 + 1
 
-    m = rt.LIBRARY_GEMM_ROWS + 37
+    m = rt.DECODE_ONCE_ROWS + 37
     activation = _activation(rt, oracle, m, k, seed=77)
     a_codes = oracle.unpack_unsigned(bits(activation.code_payload), m * k, 4)
     a_beta = oracle.unpack_unsigned(bits(activation.beta_payload), m * k // 8, 2)
@@ -142,3 +147,20 @@ def test_long_prefill_decodes_the_weight_once(rt, oracle, k, n_out):
     assert relative_error(bits(y.float()), ref) <= TOLERANCE
     fused = rt._gemm(activation, weight, output_dtype=torch.bfloat16, split_k=1)      # explicit split: fused kernel
     assert relative_error(bits(y.float()), bits(fused.float())) <= 5e-3
+
+
+@pytest.mark.parametrize("m,n,k", [(300, 200, 128), (257, 520, 384), (64, 64, 128), (1000, 72, 256), (384, 8192, 2048)])
+def test_dense_bf16_gemm_against_float32(rt, m, n, k):
+    """nq_bf16_gemm (the multiply of the decode-once route) against the FP32 product of the same BF16
+    operands: FP32 accumulation and one BF16 rounding of the result leave <= 2^-8 relative to the
+    largest output; every workgroup tile shape, ragged edges included."""
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16).cuda()
+    b = torch.randn(n, k, generator=g).to(torch.bfloat16).cuda()
+    ref = bits(a.float() @ b.float().t())
+    for tile in range(-1, 7):
+        c = rt.bf16_gemm(a, b, tile=tile)
+        assert c.dtype == torch.bfloat16 and tuple(c.shape) == (m, n)
+        assert relative_error(bits(c.float()), ref) <= 2.0 ** -8, (tile,)
+    with pytest.raises(ValueError, match="multiple of 128"):
+        rt.bf16_gemm(a[:, :64].contiguous(), b[:, :64].contiguous())
