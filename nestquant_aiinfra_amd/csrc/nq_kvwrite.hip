@@ -227,6 +227,7 @@ __global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
         __syncthreads();
         staged_row_norms(&rows[0][0], 2 * P, D, sqrt_d, row_scale, row_norm);
         const int64_t page = a.page_indices[(int64_t)slot * a.max_pages + ordinal];
+        if (page < 0) continue;                  // ordinal not mapped to a physical page: nothing to write to
         if (tid < 2 * P) {
             const int t = tid % P;
             (tid < P ? a.key_norms : a.value_norms)[page * page_rows + t * a.kv_heads + g] = row_norm[tid];

@@ -56,11 +56,24 @@ _EXPORTS = {
     "nqkv_decode_attention_batched_k1": "nqkv",
     "nqkv_prefill_attention": "nqkv",
     "BatchedNQKVCacheManager": "nqkv",
+    "append_hot_k1_graph_safe": "nqkv",
+    "launch_pack_full_hot_pages_graph_safe": "nqkv",
+    "cuda_e8_available": "cuda_e8",
+    "e8_nearest_cuda": "cuda_e8",
+    "bf16_gemm": "w4a4_linear",
     "BatchedNQKVLlamaCache": "nqkv_hf_backend",
     "install_batched_nqkv_llama_backend": "nqkv_hf_backend",
     "greedy_sample_": "nqkv_hf_backend",
     "greedy_sample_workspace": "nqkv_hf_backend",
     "BatchedNQKVLlamaRunner": "nqkv_hf_backend",
+    "RequestStatus": "continuous_batching",
+    "DecodeRequest": "continuous_batching",
+    "ContinuousBatchScheduler": "continuous_batching",
+    "RaggedDecodeBackend": "inference_engine",
+    "EngineStep": "inference_engine",
+    "AdmissionPolicy": "inference_engine",
+    "GreedyHostSampler": "inference_engine",
+    "ContinuousBatchInferenceEngine": "inference_engine",
     "UnsupportedForFusedDecode": "llama_decode_step",
     "FusedLlamaDecodeStep": "llama_decode_step",
     "FusedLlamaPrefillStep": "llama_decode_step",

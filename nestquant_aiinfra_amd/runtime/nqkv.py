@@ -503,6 +503,105 @@ def nqkv_prefill_attention(query: torch.Tensor, cache: NQKVHotColdCache, *, slot
 
 
 # --------------------------------------------------------------------------------------
+# single-cache writer under the reference's names
+# --------------------------------------------------------------------------------------
+
+def _check_hot_k1_inputs(key: torch.Tensor, value: torch.Tensor, cache: NQKVHotColdCache,
+                         slot_ids: torch.Tensor, active_mask: torch.Tensor) -> int:
+    if not isinstance(cache, NQKVHotColdCache):
+        raise TypeError("cache must be an NQKVHotColdCache")
+    pool = cache.pool
+    if not isinstance(key, torch.Tensor) or not isinstance(value, torch.Tensor):
+        raise TypeError("key and value must be tensors")
+    if key.ndim != 3 or key.shape != value.shape or tuple(key.shape[1:]) != (pool.num_kv_heads, pool.head_dim):
+        raise ValueError("key and value must have shape [batch, kv_heads, head_dim]")
+    batch = key.shape[0]
+    if not 1 <= batch <= cache.max_sequences:
+        raise ValueError("batch must be within cache capacity")
+    if key.dtype != torch.bfloat16 or value.dtype != torch.bfloat16:
+        raise ValueError("key and value must be BF16 like the hot tails")
+    if slot_ids.dtype != torch.int32 or tuple(slot_ids.shape) != (batch,):
+        raise ValueError("slot_ids must be int32 with shape [batch]")
+    if active_mask.dtype != torch.bool or tuple(active_mask.shape) != (batch,):
+        raise ValueError("active_mask must be bool with shape [batch]")
+    if any(t.device != pool.device for t in (key, value, slot_ids, active_mask)):
+        raise ValueError("append inputs must be on the cache device")
+    if not all(t.is_contiguous() for t in (key, value, slot_ids, active_mask)):
+        raise RuntimeError("append inputs must be contiguous")
+    return batch
+
+
+def _launch_append_hot_k1_graph_safe(key: torch.Tensor, value: torch.Tensor, cache: NQKVHotColdCache, *,
+                                     slot_ids: torch.Tensor, active_mask: torch.Tensor) -> None:
+    """Fixed-address GPU work only: one table update and one writer launch, no host reads."""
+    pool, meta = cache.pool, cache.metadata
+    batch = key.shape[0]
+    lib, stream = _native.library(), _native.stream_handle(pool.device)
+    max_tokens = cache.max_pages_per_sequence * pool.page_size
+    _native.check(lib.nq_nqkv_advance(
+        slot_ids.data_ptr(), active_mask.data_ptr(), None, 1, batch, cache.max_sequences, pool.page_size, max_tokens,
+        meta.sequence_lengths.data_ptr(), meta.page_counts.data_ptr(), meta.last_page_lens.data_ptr(),
+        meta.hot_lengths.data_ptr(), stream))
+    _native.check(lib.nq_nqkv_write(
+        key.data_ptr(), value.data_ptr(), _native.dtype_tag(key.dtype), slot_ids.data_ptr(), active_mask.data_ptr(),
+        None, 1, meta.sequence_lengths.data_ptr(), meta.page_indices.data_ptr(),
+        pool.key_codes.data_ptr(), pool.key_betas.data_ptr(), pool.key_norms.data_ptr(),
+        pool.value_codes.data_ptr(), pool.value_betas.data_ptr(), pool.value_norms.data_ptr(),
+        pool.beta_table.data_ptr(), pool.beta_table.numel(), pool.value_beta_table.data_ptr(),
+        pool.value_beta_table.numel(), cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(),
+        batch, 1, cache.max_sequences, cache.max_pages_per_sequence, pool.num_kv_heads, pool.head_dim, pool.page_size,
+        0, None, None, stream))
+
+
+def append_hot_k1_graph_safe(key: torch.Tensor, value: torch.Tensor, cache: NQKVHotColdCache, *,
+                             slot_ids: torch.Tensor, active_mask: torch.Tensor) -> None:
+    """Append one token per active row of one cache (nestquant/runtime/nqkv_graph_writer.py:263-289):
+    key / value BF16 [batch, kv_heads, head_dim] land in the hot tail of slot_ids[r], and the
+    device tables of the cache advance by one token.  An append that completes a page encodes
+    and publishes that page into physical page page_indices[slot, ordinal] in the same launch, so
+    the "hot page is full" state the reference refuses here never exists; what is refused instead
+    is a sequence that already holds max_pages * page_size tokens, and a page ordinal that is not
+    mapped to a physical page.  The checks read the tables on the host; the launch itself
+    (`_launch_append_hot_k1_graph_safe`) does not and is capturable.
+
+    A cache that shares its tables with other layers (BatchedNQKVCacheManager) must not be
+    advanced once per layer: there `begin_step` + `write_layer` are the entry points."""
+    _check_hot_k1_inputs(key, value, cache, slot_ids, active_mask)
+    slots = slot_ids[active_mask].detach().cpu().tolist()
+    if len(slots) != len(set(slots)):
+        raise ValueError("active slot_ids must be unique")
+    if any(not 0 <= slot < cache.max_sequences for slot in slots):
+        raise ValueError("active slot_ids must be inside the cache")
+    if slots:
+        pool, meta = cache.pool, cache.metadata
+        index = torch.tensor(slots, dtype=torch.long, device=pool.device)
+        lengths = meta.sequence_lengths[index]
+        if bool((lengths >= cache.max_pages_per_sequence * pool.page_size).any().item()):
+            raise RuntimeError("sequence already fills its pages")
+        completes = (lengths + 1) % pool.page_size == 0
+        targets = meta.page_indices[index, lengths // pool.page_size]
+        if bool((completes & ((targets < 0) | (targets >= pool.capacity))).any().item()):
+            raise RuntimeError("the page this append completes is not mapped to a physical page")
+    _launch_append_hot_k1_graph_safe(key, value, cache, slot_ids=slot_ids, active_mask=active_mask)
+
+
+def launch_pack_full_hot_pages_graph_safe(cache: NQKVHotColdCache, *, boundary_mask: torch.Tensor,
+                                          batched_encode: bool = False) -> None:
+    """The page-boundary stage of the reference's decode graph
+    (nestquant/runtime/nqkv_graph_pack.py:76-135): encode the full hot pages of the rows in
+    `boundary_mask` and publish them.  Here the append that fills a page has already done both
+    (`append_hot_k1_graph_safe`, `write_layer`), so after validating its arguments this launches
+    nothing: the cache is in the state the reference reaches after this call."""
+    del batched_encode
+    if not isinstance(cache, NQKVHotColdCache):
+        raise TypeError("cache must be an NQKVHotColdCache")
+    if boundary_mask.dtype != torch.bool or tuple(boundary_mask.shape) != (cache.max_sequences,):
+        raise ValueError("boundary_mask must be bool with cache capacity shape")
+    if boundary_mask.device != cache.pool.device:
+        raise ValueError("boundary_mask must be on the cache device")
+
+
+# --------------------------------------------------------------------------------------
 # multi-layer manager: step bookkeeping + the ragged writer
 # --------------------------------------------------------------------------------------
 

@@ -79,24 +79,68 @@ class BatchedNQKVLlamaCache(Cache):
         return self.manager.release_slots(slots)
 
     # -- step state ------------------------------------------------------------------------
-    def set_batch_state(self, *, slot_ids: Sequence[int], counts: Sequence[int]) -> None:
-        """Eager (prefill) step: row i writes its first counts[i] tokens into slot_ids[i].
-        Copies the row state to the fixed step tensors and advances the device tables."""
+    def set_batch_state(self, *, slot_ids: Sequence[int] | None = None, counts: Sequence[int] | None = None,
+                        active_mask: torch.Tensor | None = None, write_mask: torch.Tensor | None = None,
+                        width: int | None = None) -> None:
+        """Eager (prefill) step.  Two forms:
+          * slot_ids / counts: row i writes its first counts[i] tokens into slot_ids[i] (`width`, when
+            given, bounds every count);
+          * active_mask / write_mask, the reference's form (nestquant/runtime/nqkv_batched_hf_backend.py:147):
+            bool [capacity] and bool [capacity, width]; row r is slot r and writes the prefix of
+            `write_mask[r]` (masks that are not prefixes are rejected).
+        Validates before anything changes, copies the row state to the fixed step tensors and advances
+        the device tables."""
+        if write_mask is not None or active_mask is not None:
+            if slot_ids is not None or counts is not None:
+                raise ValueError("give slot_ids / counts or active_mask / write_mask, not both")
+            if (not isinstance(write_mask, torch.Tensor) or write_mask.dtype != torch.bool or write_mask.ndim != 2
+                    or write_mask.shape[0] != self.capacity):
+                raise ValueError("write_mask must be bool with shape [capacity, width]")
+            if active_mask is None:
+                active_mask = write_mask.any(dim=1)
+            if active_mask.dtype != torch.bool or tuple(active_mask.shape) != (self.capacity,):
+                raise ValueError("active_mask must be bool with shape [capacity]")
+            host_mask = write_mask.detach().cpu()
+            host_active = active_mask.detach().cpu().tolist()
+            width = write_mask.shape[1]
+            counts = [int(row.sum()) if live else 0 for row, live in zip(host_mask, host_active)]
+            for row, count in zip(host_mask, counts):
+                if count and not bool(row[:count].all()):
+                    raise ValueError("write_mask rows must be prefixes: written tokens lead each row")
+            slot_ids = list(range(self.capacity))
+        if slot_ids is None or counts is None:
+            raise ValueError("set_batch_state needs slot_ids and counts (or the two masks)")
+        slot_ids, counts = [int(s) for s in slot_ids], [int(c) for c in counts]
         rows = len(slot_ids)
         if rows < 1 or rows > self.capacity or len(counts) != rows:
             raise ValueError("slot_ids and counts must describe 1..capacity rows")
+        if len(set(slot_ids)) != rows:
+            raise ValueError("a slot may appear once per step")
         for slot, count in zip(slot_ids, counts):
-            if self._host_lengths[slot] + count > self.manager.max_tokens:
+            if not 0 <= slot < self.capacity:
+                raise ValueError("slot is outside cache capacity")
+            if count < 0 or (width is not None and count > width):
+                raise ValueError("a row writes between 0 and `width` tokens")
+            if count and self.manager.sequence_id(slot) is None:
+                raise RuntimeError("slot has no registered sequence")
+            if self._host_lengths[slot] + count > self._max_cache_len:
                 raise RuntimeError("sequence would exceed max_cache_len")
         self._continuation = any(self._host_lengths[slot] > 0 and count > 0 for slot, count in zip(slot_ids, counts))
         m = self.manager
-        m.step_slot_ids[:rows].copy_(torch.tensor(list(slot_ids), dtype=torch.int32))
-        m.step_counts[:rows].copy_(torch.tensor(list(counts), dtype=torch.int32))
+        m.step_slot_ids[:rows].copy_(torch.tensor(slot_ids, dtype=torch.int32))
+        m.step_counts[:rows].copy_(torch.tensor(counts, dtype=torch.int32))
         m.step_active[:rows].copy_(torch.tensor([c > 0 for c in counts]))
         for slot, count in zip(slot_ids, counts):
             self._host_lengths[slot] += count
         self._rows, self._tokens = rows, max(counts)
         m.begin_step(rows=rows, uniform_count=None)
+
+    def fail_closed(self, slots: Sequence[int]) -> None:
+        """After a forward that raised: the step's table advance is not backed by keys and values in
+        every layer, so the sequences it touched are dropped (tables zeroed, slots free), as the
+        reference does on a failed prefill (nestquant/runtime/nqkv_batched_hf_backend.py:493-531)."""
+        self.release_slots([slot for slot in slots if self.manager.sequence_id(slot) is not None])
+        self._tokens = None
 
     def set_decode_execution_state(self, *, slot_ids: torch.Tensor, active_mask: torch.Tensor) -> None:
         """Decode rows for the steps that follow (device tensors of equal length <= capacity);
@@ -121,7 +165,7 @@ class BatchedNQKVLlamaCache(Cache):
         """Raises before a step that would take a slot past the cache length (the device tables
         clamp there, so the step itself would overwrite the newest tokens instead)."""
         for slot in slots:
-            if self._host_lengths[slot] + tokens > self.manager.max_tokens:
+            if self._host_lengths[slot] + tokens > self._max_cache_len:
                 raise RuntimeError("sequence would exceed max_cache_len")
 
     # -- Cache protocol -------------------------------------------------------------------------
@@ -367,18 +411,97 @@ class BatchedNQKVLlamaRunner:
         return bool(self._graphs)
 
     # -- prefill -------------------------------------------------------------------------------
+    def _check_reference_rows(self, input_ids: torch.Tensor, positions: torch.Tensor, mask: torch.Tensor,
+                              valid_lengths: torch.Tensor) -> None:
+        """Argument checks of the reference's runner (nestquant/runtime/nqkv_batched_runner.py:72-100)."""
+        if input_ids.dtype != torch.long or input_ids.ndim != 2:
+            raise ValueError("input_ids must be rank-2 torch.long")
+        if input_ids.shape[0] != self.batch_size:
+            raise ValueError("input batch must equal fixed runner capacity")
+        if positions.dtype != torch.long or positions.shape != input_ids.shape:
+            raise ValueError("positions must be torch.long and match input_ids")
+        if mask.dtype != torch.bool or mask.shape != input_ids.shape:
+            raise ValueError("write_mask must be bool and match input_ids")
+        if valid_lengths.dtype != torch.long or tuple(valid_lengths.shape) != (self.batch_size,):
+            raise ValueError("valid_lengths must have shape [batch_size]")
+        if any(tensor.device != self.device for tensor in (input_ids, positions, mask, valid_lengths)):
+            raise ValueError("runner inputs must be on the model CUDA device")
+        if bool(mask.any().item()):
+            written = positions[mask]
+            if int(written.min().item()) < 0:
+                raise ValueError("written positions must be non-negative")
+            if int(written.max().item()) >= self.max_cache_len:
+                raise ValueError("written positions exceed the NQKV cache")
+
     @torch.inference_mode()
-    def prefill_slots(self, input_ids: torch.Tensor, *, slots: Sequence[int], lengths: Sequence[int],
-                      positions: torch.Tensor | None = None, last_token_logits: bool = False) -> torch.Tensor:
+    def prefill(self, input_ids: torch.Tensor) -> torch.Tensor:
+        """Every fixed row takes its whole row of input_ids [capacity, width] as a fresh prompt (the
+        warm-up call of the reference's engine, nestquant/runtime/nqkv_batched_runner.py:171-187)."""
+        if input_ids.dtype != torch.long or input_ids.ndim != 2:
+            raise ValueError("input_ids must be rank-2 torch.long")
+        if input_ids.shape[0] != self.batch_size or input_ids.device != self.device:
+            raise ValueError("input_ids batch or device does not match the runner")
+        width = input_ids.shape[1]
+        if width < 1 or width > self.max_cache_len:
+            raise ValueError("prefill width is outside the NQKV cache")
+        return self.prefill_slots(input_ids, slots=list(range(self.batch_size)), lengths=[width] * self.batch_size)
+
+    @torch.inference_mode()
+    def prefill_slots(self, input_ids: torch.Tensor, *, slots: Sequence[int] | None = None,
+                      lengths: Sequence[int] | None = None, positions: torch.Tensor | None = None,
+                      last_token_logits: bool = False, write_mask: torch.Tensor | None = None,
+                      valid_lengths: torch.Tensor | None = None) -> torch.Tensor:
         """Prefill `slots[i]` with the first `lengths[i]` tokens of row i of input_ids
         [rows, width] (right padded).  New slots are registered.  Returns logits [rows, width, vocab],
         or, with `last_token_logits`, only those of every row's last token, [rows, 1, vocab]
-        (what sampling the first new token needs: the LM head then runs on `rows` vectors)."""
+        (what sampling the first new token needs: the LM head then runs on `rows` vectors).
+
+        The reference's form (RaggedDecodeBackend, nestquant/runtime/inference_engine.py:14-32) is
+        taken too: input_ids / positions / write_mask [capacity, width] and valid_lengths [capacity],
+        row r being slot r and writing the prefix `write_mask[r]` marks; logits then come back as
+        [capacity, width, vocab] with zero rows for slots that wrote nothing.
+
+        A forward that raises leaves no slot half written: the sequences of the rows that were
+        writing are dropped and their slots freed before the exception travels on."""
+        if write_mask is not None:
+            if slots is not None or lengths is not None:
+                raise ValueError("give slots / lengths or write_mask / valid_lengths, not both")
+            if positions is None or valid_lengths is None:
+                raise ValueError("the masked form needs positions and valid_lengths")
+            self._check_reference_rows(input_ids, positions, write_mask, valid_lengths)
+            host_mask = write_mask.detach().cpu()
+            counts = [int(row.sum()) for row in host_mask]
+            for row, count in zip(host_mask, counts):
+                if count and not bool(row[:count].all()):
+                    raise ValueError("write_mask rows must be prefixes: written tokens lead each row")
+            live = [slot for slot, count in enumerate(counts) if count]
+            full = None
+            if live:
+                index = torch.tensor(live, dtype=torch.long, device=self.device)
+                part = self.prefill_slots(input_ids[index], slots=live, lengths=[counts[s] for s in live],
+                                          positions=positions[index], last_token_logits=last_token_logits)
+                full = torch.zeros((self.batch_size, *part.shape[1:]), dtype=part.dtype, device=self.device)
+                full[index] = part
+            else:
+                vocab = self.model.config.vocab_size
+                full = torch.zeros((self.batch_size, 1 if last_token_logits else input_ids.shape[1], vocab),
+                                   dtype=next(self.model.parameters()).dtype, device=self.device)
+            return full
+        if slots is None or lengths is None:
+            raise ValueError("prefill_slots needs slots and lengths (or write_mask and valid_lengths)")
         rows, width = input_ids.shape
+        slots, lengths = [int(s) for s in slots], [int(n) for n in lengths]
         if len(slots) != rows or len(lengths) != rows:
             raise ValueError("slots and lengths must have one entry per row")
-        if last_token_logits and not all(1 <= int(length) <= width for length in lengths):
+        if len(set(slots)) != rows or any(not 0 <= slot < self.batch_size for slot in slots):
+            raise ValueError("slots must be distinct and inside the runner's capacity")
+        if any(not 0 <= length <= width for length in lengths):
+            raise ValueError("a row holds between 0 and `width` prompt tokens")
+        if last_token_logits and not all(1 <= length <= width for length in lengths):
             raise ValueError("last_token_logits needs at least one token in every row")
+        for slot, length in zip(slots, lengths):
+            if self.cache._host_lengths[slot] + length > self.max_cache_len:
+                raise RuntimeError("sequence would exceed max_cache_len")
         for slot in slots:
             if self.cache.manager.sequence_id(slot) is None:
                 self._generation[slot] += 1
@@ -386,20 +509,40 @@ class BatchedNQKVLlamaRunner:
         if positions is None:
             starts = torch.tensor([self.cache._host_lengths[s] for s in slots], device=self.device)
             positions = starts[:, None] + torch.arange(width, device=self.device)[None, :]
+        else:
+            if positions.dtype != torch.long or tuple(positions.shape) != (rows, width) or positions.device != self.device:
+                raise ValueError("positions must be torch.long [rows, width] on the model device")
+            written = torch.arange(width, device=self.device)[None, :] < torch.tensor(lengths, device=self.device)[:, None]
+            if bool(written.any().item()):
+                inside = positions[written]
+                if int(inside.min().item()) < 0 or int(inside.max().item()) >= self.max_cache_len:
+                    raise ValueError("written positions must lie in [0, max_cache_len)")
         self._decode_state = None
-        self.cache.set_batch_state(slot_ids=slots, counts=lengths)
+        self.cache.set_batch_state(slot_ids=slots, counts=lengths, width=width)
         keep = None
         if last_token_logits:
-            keep = torch.tensor([int(length) - 1 for length in lengths], dtype=torch.long, device=self.device)
-        if self.fused_prefill is not None:
-            return self.fused_prefill(input_ids, positions, keep=keep)
-        output = self.model(input_ids=input_ids, position_ids=positions, past_key_values=self.cache, use_cache=True)
+            keep = torch.tensor([length - 1 for length in lengths], dtype=torch.long, device=self.device)
+        try:
+            if self.fused_prefill is not None:
+                return self.fused_prefill(input_ids, positions, keep=keep)
+            output = self.model(input_ids=input_ids, position_ids=positions, past_key_values=self.cache, use_cache=True)
+        except Exception:
+            self.cache.fail_closed([slot for slot, length in zip(slots, lengths) if length])
+            raise
         if keep is not None:
             return output.logits[torch.arange(rows, device=self.device), keep].unsqueeze(1)
         return output.logits
 
     def release_slots(self, slots: Sequence[int]) -> None:
         self.cache.release_slots(slots)
+
+    def clear_slots(self, slot_mask: torch.Tensor) -> None:
+        """Release the slots marked in a bool mask [capacity] (the reference's name for release)."""
+        if slot_mask.dtype != torch.bool or tuple(slot_mask.shape) != (self.batch_size,):
+            raise ValueError("slot_mask must be bool with shape [batch_size]")
+        if slot_mask.device != self.device:
+            raise ValueError("slot_mask must be on the model device")
+        self.release_slots(slot_mask.nonzero(as_tuple=False).flatten().cpu().tolist())
 
     # -- decode --------------------------------------------------------------------------------
     def _step(self, tokens: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
@@ -423,9 +566,16 @@ class BatchedNQKVLlamaRunner:
         return logits
 
     @torch.inference_mode()
-    def capture(self, widths: Sequence[int] | None = None) -> None:
-        """Capture one decode graph per batch width.  Captured on slots that hold at least one
-        token; the tables are restored afterwards, so capture leaves the cache unchanged."""
+    def capture(self, sample_token: torch.Tensor | Sequence[int] | None = None, *, positions: torch.Tensor | None = None,
+                active_mask: torch.Tensor | None = None, valid_lengths: torch.Tensor | None = None,
+                widths: Sequence[int] | None = None) -> None:
+        """Capture one decode graph per batch width.  The tables are restored afterwards, so capture
+        leaves the cache unchanged.  The reference's arguments (sample_token, positions, active_mask,
+        valid_lengths: nestquant/runtime/nqkv_batched_runner.py:227-299) are accepted and not needed:
+        the graphs are captured on inactive rows and read their inputs from fixed tensors."""
+        del positions, active_mask, valid_lengths
+        if widths is None and sample_token is not None and not isinstance(sample_token, torch.Tensor):
+            widths = list(sample_token)
         if widths is None:
             widths, width = [], 1
             while width < self.batch_size:
@@ -464,8 +614,28 @@ class BatchedNQKVLlamaRunner:
             tensor.copy_(value)
 
     @torch.inference_mode()
-    def decode(self, tokens: torch.Tensor, *, slots: Sequence[int], positions: torch.Tensor) -> torch.Tensor:
-        """One captured decode step: tokens / positions [rows, 1] for `slots`; logits [rows, 1, vocab]."""
+    def decode(self, tokens: torch.Tensor, *, slots: Sequence[int] | None = None, positions: torch.Tensor,
+               active_mask: torch.Tensor | None = None, valid_lengths: torch.Tensor | None = None) -> torch.Tensor:
+        """One captured decode step: tokens / positions [rows, 1] for `slots`; logits [rows, 1, vocab].
+        The reference's form (tokens / positions / active_mask [capacity, 1], valid_lengths [capacity];
+        row r is slot r) returns [capacity, 1, vocab] with zero rows for inactive slots."""
+        if active_mask is not None:
+            if slots is not None:
+                raise ValueError("give slots or active_mask, not both")
+            if valid_lengths is None:
+                raise ValueError("the masked form needs valid_lengths")
+            self._check_reference_rows(tokens, positions, active_mask, valid_lengths)
+            live = active_mask[:, 0].nonzero(as_tuple=False).flatten().cpu().tolist()
+            vocab = self.model.config.vocab_size
+            if not live:
+                return torch.zeros((*tokens.shape, vocab), dtype=next(self.model.parameters()).dtype, device=self.device)
+            index = torch.tensor(live, dtype=torch.long, device=self.device)
+            part = self.decode(tokens[index], slots=live, positions=positions[index])
+            full = torch.zeros((self.batch_size, *part.shape[1:]), dtype=part.dtype, device=self.device)
+            full[index] = part
+            return full
+        if slots is None:
+            raise ValueError("decode needs slots (or active_mask and valid_lengths)")
         rows = len(slots)
         width = next((w for w in sorted(self._graphs) if w >= rows), None)
         if width is None:

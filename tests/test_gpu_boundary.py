@@ -1,0 +1,245 @@
+"""The reference's Python-facing names for the hot path that adapt to this build's kernels:
+the masked (RaggedDecodeBackend) form of the runner, fail-closed prefill, the single-cache
+append / pack pair, the stand-alone E8 projection, and the continuous-batching engine on a
+tiny random-init Llama (reference: tests/unit/runtime/test_nqkv_batched_hf_backend.py:399-567,
+tests/unit/runtime/test_nqkv_graph_writer.py, nestquant/runtime/cuda_e8.py)."""
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import KEY_BETAS, Q, VALUE_BETAS
+from gpu_util import bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tiny(tmp_path_factory):
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
+
+    torch.manual_seed(5011)
+    config = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                         num_key_value_heads=2, head_dim=64, vocab_size=128, max_position_embeddings=512,
+                         rope_theta=500000.0, tie_word_embeddings=True)
+    model = LlamaForCausalLM(config).to(torch.bfloat16).cuda().eval()
+    path = tmp_path_factory.mktemp("nqmc") / "tiny.nqmc"
+    asm.write_w4_checkpoint(model, path)
+    # a cache length that is not a multiple of the page size: positions stop at 100, pages hold 112
+    runner = asm.build_w4a4kv4_runner(model, path, capacity=4, max_cache_len=100)
+    return model, runner
+
+
+def _ids(rows, width, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(1, 128, (rows, width), generator=g).cuda()
+
+
+def test_masked_form_equals_slot_form(tiny):
+    model, runner = tiny
+    cache = runner.cache
+    ids = _ids(4, 21, 1)
+    lengths = [21, 0, 9, 17]
+    write_mask = torch.arange(21, device="cuda")[None, :] < torch.tensor(lengths, device="cuda")[:, None]
+    positions = torch.arange(21, device="cuda").repeat(4, 1)
+    valid = torch.tensor([21, 1, 9, 17], device="cuda")
+    masked = runner.prefill_slots(ids, positions=positions, write_mask=write_mask, valid_lengths=valid)
+    assert tuple(masked.shape) == (4, 21, 128) and not masked[1].any()
+    tables = [t.clone() for t in (cache.manager.metadata.sequence_lengths, cache.manager.metadata.hot_lengths)]
+    assert tables[0].tolist() == [21, 0, 9, 17]
+    runner.clear_slots(torch.tensor([True, True, True, True], device="cuda"))
+    live = [0, 2, 3]
+    by_slot = runner.prefill_slots(ids[live], slots=live, lengths=[lengths[s] for s in live])
+    assert torch.equal(masked[live], by_slot)
+
+    runner.capture(ids[:, :1], positions=positions[:, :1], active_mask=write_mask[:, :1], valid_lengths=valid)
+    token = torch.zeros((4, 1), dtype=torch.long, device="cuda")
+    at = torch.zeros((4, 1), dtype=torch.long, device="cuda")
+    for slot in live:
+        token[slot, 0] = by_slot[live.index(slot), lengths[slot] - 1].argmax()
+        at[slot, 0] = lengths[slot]
+    active = torch.tensor([[True], [False], [True], [True]], device="cuda")
+    out = runner.decode(token, positions=at, active_mask=active, valid_lengths=at[:, 0] + 1)
+    assert tuple(out.shape) == (4, 1, 128) and not out[1].any() and torch.isfinite(out).all()
+    assert cache.manager.metadata.sequence_lengths.tolist() == [22, 0, 10, 18]
+    with pytest.raises(ValueError, match="prefixes"):
+        holes = write_mask.clone()
+        holes[0, 3] = False
+        runner.prefill_slots(ids, positions=positions, write_mask=holes, valid_lengths=valid)
+    with pytest.raises(ValueError, match="exceed the NQKV cache"):
+        runner.prefill_slots(ids, positions=positions + 90, write_mask=write_mask, valid_lengths=valid)
+    runner.clear_slots(torch.ones(4, dtype=torch.bool, device="cuda"))
+
+
+def test_cache_length_that_is_not_a_page_multiple(tiny):
+    """Positions end at max_cache_len = 100 although the pages could hold 112 tokens: the host
+    refuses the 101st token instead of letting the kernels reuse the last rotary row."""
+    model, runner = tiny
+    ids = _ids(1, 100, 2)
+    logits = runner.prefill_slots(ids[:, :99], slots=[1], lengths=[99])
+    token = logits[:, 98].argmax(-1).reshape(1, 1)
+    out = runner.decode(token, slots=[1], positions=torch.tensor([[99]], device="cuda"))
+    assert torch.isfinite(out).all() and runner.cache.manager.total_tokens(1) == 100
+    with pytest.raises(RuntimeError, match="exceed max_cache_len"):
+        runner.decode(token, slots=[1], positions=torch.tensor([[100]], device="cuda"))
+    with pytest.raises(RuntimeError, match="exceed max_cache_len"):
+        runner.prefill_slots(ids[:, :1], slots=[1], lengths=[1])
+    assert runner.cache.manager.total_tokens(1) == 100            # refused before anything changed
+    runner.release_slots([1])
+    with pytest.raises(RuntimeError, match="exceed max_cache_len"):
+        runner.prefill_slots(_ids(1, 101, 3), slots=[1], lengths=[101])
+    assert runner.cache.manager.sequence_id(1) is None or runner.cache.manager.total_tokens(1) == 0
+    runner.release_slots([1])
+
+
+def test_prefill_input_validation_changes_nothing(tiny):
+    model, runner = tiny
+    ids = _ids(2, 8, 4)
+    before = runner.cache.manager.metadata.sequence_lengths.clone()
+    for kwargs, error in (({"slots": [0, 0], "lengths": [3, 3]}, ValueError),          # duplicate slot
+                          ({"slots": [0, 9], "lengths": [3, 3]}, ValueError),          # slot outside the runner
+                          ({"slots": [0, 1], "lengths": [3, 9]}, ValueError),          # longer than the row
+                          ({"slots": [0, 1], "lengths": [3, -1]}, ValueError),         # negative
+                          ({"slots": [0], "lengths": [3]}, ValueError)):               # one entry per row
+        with pytest.raises(error):
+            runner.prefill_slots(ids, **kwargs)
+    assert torch.equal(runner.cache.manager.metadata.sequence_lengths, before)
+    assert all(runner.cache.manager.sequence_id(slot) is None for slot in range(4))
+
+
+def test_forward_failure_releases_the_rows_that_were_writing(tiny):
+    model, runner = tiny
+    cache = runner.cache
+    keep = runner.prefill_slots(_ids(1, 20, 5), slots=[3], lengths=[20])           # a bystander in another slot
+    runner.prefill_slots(_ids(2, 12, 6), slots=[0, 1], lengths=[12, 5])
+    # the forward runs to its end (every layer has written its keys and values), then fails
+    fused = runner.fused_prefill
+    real = fused if fused is not None else model.forward
+
+    def failing(*args, **kwargs):
+        real(*args, **kwargs)
+        raise RuntimeError("injected post-KV failure")
+
+    if fused is not None:
+        runner.fused_prefill = failing
+    else:
+        model.forward = failing
+    try:
+        with pytest.raises(RuntimeError, match="injected post-KV failure"):
+            runner.prefill_slots(_ids(2, 30, 7), slots=[0, 2], lengths=[30, 8])      # slot 0 continues, slot 2 is new
+    finally:
+        if fused is not None:
+            runner.fused_prefill = fused
+        else:
+            del model.forward
+    meta = cache.manager.metadata
+    assert meta.sequence_lengths.tolist() == [0, 5, 0, 20] and meta.page_counts.tolist() == [0, 0, 0, 1]
+    assert cache._host_lengths == [0, 5, 0, 20]
+    assert cache.manager.sequence_id(0) is None and cache.manager.sequence_id(2) is None
+    assert cache.manager.sequence_id(1) is not None and cache.manager.sequence_id(3) is not None
+    # the freed slots take new prompts; the bystander still decodes
+    runner.prefill_slots(_ids(1, 6, 8), slots=[0], lengths=[6])
+    out = runner.decode_eager(keep[:, 19].argmax(-1).reshape(1, 1), slots=[3], positions=torch.tensor([[20]], device="cuda"))
+    assert torch.isfinite(out).all()
+    runner.release_slots([0, 1, 2, 3])
+
+
+def test_engine_end_to_end_with_slot_reuse_and_bursts(tiny):
+    from nestquant_aiinfra_amd.runtime import AdmissionPolicy, ContinuousBatchInferenceEngine, DecodeRequest, RequestStatus
+    model, runner = tiny
+
+    def drain(burst):
+        engine = ContinuousBatchInferenceEngine(runner, decode_burst=burst,
+                                                admission_policy=AdmissionPolicy(min_prefill_batch=1, max_wait_steps=0))
+        g = torch.Generator().manual_seed(11)
+        requests = [DecodeRequest(f"r{i}", tuple(torch.randint(1, 128, (int(n),), generator=g).tolist()), int(t))
+                    for i, (n, t) in enumerate(((5, 20), (19, 7), (33, 18), (2, 30), (16, 9), (40, 12), (7, 5)))]
+        for request in requests[:5]:
+            engine.submit(request)
+        steps = 0
+        while engine.has_work() and steps < 200:
+            if steps == 3:
+                for request in requests[5:]:
+                    engine.submit(request)
+            engine.step()
+            steps += 1
+        assert not engine.has_work()
+        assert all(r.status is RequestStatus.FINISHED and len(r.generated_token_ids) == r.max_new_tokens for r in requests)
+        assert runner.cache.manager.metadata.sequence_lengths.tolist() == [0, 0, 0, 0]       # every slot was given back
+        return {r.request_id: list(r.generated_token_ids) for r in requests}
+
+    single = drain(1)
+    burst = drain(6)
+    assert single == burst           # the device sampler picks what the host argmax picks
+    # each request's text equals its own solo run: slots never see each other's cache
+    solo_engine = ContinuousBatchInferenceEngine(runner, admission_policy=AdmissionPolicy(1, 0))
+    g = torch.Generator().manual_seed(11)
+    first_prompt = tuple(torch.randint(1, 128, (5,), generator=g).tolist())
+    alone = DecodeRequest("alone", first_prompt, 20)
+    solo_engine.submit(alone)
+    while solo_engine.has_work():
+        solo_engine.step()
+    assert alone.generated_token_ids == single["r0"]
+
+
+def test_single_cache_append_under_the_reference_names():
+    from nestquant_aiinfra_amd.runtime import (BatchedNQKVCacheManager, append_hot_k1_graph_safe,
+                                               launch_pack_full_hot_pages_graph_safe)
+    kwargs = dict(capacity=3, num_layers=1, num_kv_heads=2, head_dim=64, max_cache_len=48, page_size=16, q=Q,
+                  key_betas=KEY_BETAS, value_betas=VALUE_BETAS, dtype=torch.bfloat16, device="cuda")
+    by_names, by_manager = BatchedNQKVCacheManager(**kwargs), BatchedNQKVCacheManager(**kwargs)
+    for manager in (by_names, by_manager):
+        manager.register("a", slot=0)
+        manager.register("b", slot=2)
+    slot_ids = torch.tensor([2, 0, 1], dtype=torch.int32, device="cuda")
+    active = torch.tensor([True, True, False], device="cuda")
+    by_manager.step_slot_ids.copy_(slot_ids)
+    by_manager.step_active.copy_(active)
+    g = torch.Generator().manual_seed(3)
+    cache = by_names.layers[0]
+    for step in range(35):                                   # two page boundaries
+        key = torch.randn(3, 2, 64, generator=g).to(torch.bfloat16).cuda()
+        value = torch.randn(3, 2, 64, generator=g).to(torch.bfloat16).cuda()
+        append_hot_k1_graph_safe(key, value, cache, slot_ids=slot_ids, active_mask=active)
+        launch_pack_full_hot_pages_graph_safe(cache, boundary_mask=torch.ones(3, dtype=torch.bool, device="cuda"))
+        by_manager.begin_step(rows=3, uniform_count=1)
+        by_manager.write_layer(0, key[:, None].contiguous(), value[:, None].contiguous())
+    other = by_manager.layers[0]
+    assert cache.metadata.sequence_lengths.tolist() == [35, 0, 35] and cache.metadata.page_counts.tolist() == [2, 0, 2]
+    for name in ("sequence_lengths", "page_counts", "last_page_lens", "hot_lengths"):
+        assert torch.equal(getattr(cache.metadata, name), getattr(other.metadata, name))
+    for name in ("key_codes", "key_betas", "key_norms", "value_codes", "value_betas", "value_norms"):
+        assert torch.equal(getattr(cache.pool, name), getattr(other.pool, name))
+    assert torch.equal(cache.hot_keys, other.hot_keys) and torch.equal(cache.hot_values, other.hot_values)
+    # the checked boundary: duplicates, a full sequence, an unmapped page
+    key = torch.zeros(3, 2, 64, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError, match="unique"):
+        append_hot_k1_graph_safe(key, key, cache, slot_ids=torch.tensor([0, 0, 1], dtype=torch.int32, device="cuda"),
+                                 active_mask=torch.tensor([True, True, False], device="cuda"))
+    for _ in range(13):
+        append_hot_k1_graph_safe(key, key, cache, slot_ids=slot_ids, active_mask=active)
+    with pytest.raises(RuntimeError, match="fills its pages"):
+        append_hot_k1_graph_safe(key, key, cache, slot_ids=slot_ids, active_mask=active)
+    by_names.register("c", slot=1)
+    cache.metadata.page_indices[1, 0] = -1
+    only_one = torch.tensor([False, False, True], device="cuda")
+    for _ in range(15):
+        append_hot_k1_graph_safe(key, key, cache, slot_ids=slot_ids, active_mask=only_one)
+    with pytest.raises(RuntimeError, match="not mapped"):
+        append_hot_k1_graph_safe(key, key, cache, slot_ids=slot_ids, active_mask=only_one)
+    with pytest.raises(ValueError, match="capacity shape"):
+        launch_pack_full_hot_pages_graph_safe(cache, boundary_mask=torch.ones(2, dtype=torch.bool, device="cuda"))
+
+
+def test_e8_nearest_cuda_wrapper(golden):
+    from nestquant_aiinfra_amd.runtime import cuda_e8_available, e8_nearest_cuda
+    assert cuda_e8_available()
+    x = torch.from_numpy(golden["e8_x"]).cuda()
+    assert np.array_equal(bits(e8_nearest_cuda(x)), golden["e8_point"])
+    assert np.array_equal(bits(e8_nearest_cuda(torch.full((1, 8), 0.25, device="cuda"))), np.full((1, 8), 0.5, np.float32))
+    assert tuple(e8_nearest_cuda(torch.empty((0, 8), device="cuda")).shape) == (0, 8)
+    with pytest.raises(ValueError, match="CUDA tensor"):
+        e8_nearest_cuda(torch.zeros(1, 8))
+    with pytest.raises(ValueError, match="shape"):
+        e8_nearest_cuda(torch.zeros(8, device="cuda"))
