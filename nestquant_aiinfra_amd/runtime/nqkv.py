@@ -18,6 +18,7 @@ reservation, no host read of hot lengths and no separate page-boundary graph.
 from __future__ import annotations
 
 import math
+from collections import deque
 from dataclasses import dataclass
 from typing import Hashable, Sequence
 
@@ -142,141 +143,155 @@ class NQKVPageHandle:
     generation: int
 
 
+@dataclass
+class _PageRecord:
+    """Host-side state of one physical page."""
+
+    generation: int = 0          # bumped on release: handles of an earlier owner stop matching
+    owned: bool = False
+    valid_tokens: int = 0        # 0 until a payload has been stored
+
+
+def _positive(**values: int) -> None:
+    for name, value in values.items():
+        if isinstance(value, bool) or not isinstance(value, int) or value < 1:
+            raise ValueError(f"{name} must be a positive integer")
+
+
 class NQKVPagePool:
-    """Preallocated SoA page storage; the tensors never move, so kernels captured in a HIP
-    graph keep valid addresses.  Allocation metadata is host-side and generation-checked."""
+    """Preallocated SoA page storage (same tensors as the reference's pool,
+    nestquant/runtime/nqkv_pool.py:94-110); the tensors never move, so kernels captured in a HIP
+    graph keep valid addresses.  Ownership is host-side: one record per page, handles carry the
+    page's generation and go stale when the page is released."""
+
+    _STREAMS = ("key_codes", "key_betas", "key_norms", "value_codes", "value_betas", "value_norms")
 
     def __init__(self, *, capacity: int, page_size: int, num_kv_heads: int, head_dim: int, q: int,
                  betas: Sequence[float] | None = None, key_betas: Sequence[float] | None = None,
                  value_betas: Sequence[float] | None = None,
                  output_dtype: torch.dtype = torch.bfloat16, device: torch.device | str = "cuda") -> None:
-        for name, value in (("capacity", capacity), ("page_size", page_size),
-                            ("num_kv_heads", num_kv_heads), ("head_dim", head_dim)):
-            if isinstance(value, bool) or not isinstance(value, int) or value < 1:
-                raise ValueError(f"{name} must be a positive integer")
+        _positive(capacity=capacity, page_size=page_size, num_kv_heads=num_kv_heads, head_dim=head_dim)
         if head_dim % 8:
             raise ValueError("head_dim must be divisible by 8")
-        if betas is not None:
-            if key_betas is not None or value_betas is not None:
-                raise ValueError("pass legacy betas or key_betas/value_betas, not both")
-            key_values = value_values = tuple(float(b) for b in betas)
-        else:
-            if key_betas is None or value_betas is None:
-                raise ValueError("v2 requires both key_betas and value_betas")
-            key_values = tuple(float(b) for b in key_betas)
-            value_values = tuple(float(b) for b in value_betas)
-        if not key_values or not value_values:
+        shared_table = betas is not None                    # format v1: one table for keys and values
+        if shared_table and (key_betas is not None or value_betas is not None):
+            raise ValueError("pass legacy betas or key_betas/value_betas, not both")
+        if not shared_table and (key_betas is None or value_betas is None):
+            raise ValueError("v2 requires both key_betas and value_betas")
+        key_table = tuple(map(float, betas if shared_table else key_betas))
+        value_table = key_table if shared_table else tuple(map(float, value_betas))
+        if not key_table or not value_table:
             raise ValueError("beta tables must be nonempty")
-        target = torch.device(device)
-        if target.type != "cuda" or not torch.cuda.is_available():
+        where = torch.device(device)
+        if where.type != "cuda" or not torch.cuda.is_available():
             raise ValueError("NQKVPagePool requires an available CUDA device")
-        if target.index is None:
-            target = torch.device("cuda", torch.cuda.current_device())
-        self.capacity, self.page_size = capacity, page_size
-        self.num_kv_heads, self.head_dim, self.q = num_kv_heads, head_dim, q
-        self.betas, self.value_beta_values = key_values, value_values
-        self.format_version = 1 if betas is not None else 2
-        self.output_dtype, self.device = output_dtype, target
-        self.code_width, self.beta_width = 4, 2
-        self._row_count = page_size * num_kv_heads
-        self._code_bytes = self._row_count * head_dim // 2
-        self._beta_bytes = self._row_count * head_dim // 32
-        self.key_codes = torch.zeros((capacity, self._code_bytes), device=target, dtype=torch.uint8)
-        self.key_betas = torch.zeros((capacity, self._beta_bytes), device=target, dtype=torch.uint8)
-        self.key_norms = torch.zeros((capacity, self._row_count), device=target, dtype=torch.float32)
-        self.value_codes = torch.zeros_like(self.key_codes)
-        self.value_betas = torch.zeros_like(self.key_betas)
-        self.value_norms = torch.zeros_like(self.key_norms)
-        self.beta_table = torch.tensor(key_values, device=target, dtype=torch.float32)
-        self.value_beta_table = (self.beta_table if betas is not None
-                                 else torch.tensor(value_values, device=target, dtype=torch.float32))
-        self._free = list(range(capacity - 1, -1, -1))
-        self._generation = [0] * capacity
-        self._allocated = [False] * capacity
-        self._stored = [False] * capacity
-        self._valid_tokens = [0] * capacity
+        if where.index is None:
+            where = torch.device("cuda", torch.cuda.current_device())
 
+        self.capacity, self.page_size, self.num_kv_heads, self.head_dim, self.q = (
+            capacity, page_size, num_kv_heads, head_dim, q)
+        self.betas, self.value_beta_values = key_table, value_table
+        self.format_version = 1 if shared_table else 2
+        self.output_dtype, self.device = output_dtype, where
+        self.code_width, self.beta_width = 4, 2
+        rows = page_size * num_kv_heads                     # one row per (token, head)
+        self._stream_shapes = {"codes": (rows * head_dim // 2, torch.uint8), "betas": (rows * head_dim // 32, torch.uint8),
+                               "norms": (rows, torch.float32)}
+        for side in ("key", "value"):
+            for kind, (width, dtype) in self._stream_shapes.items():
+                setattr(self, f"{side}_{kind}", torch.zeros((capacity, width), dtype=dtype, device=where))
+        self.beta_table = torch.tensor(key_table, dtype=torch.float32, device=where)
+        self.value_beta_table = self.beta_table if shared_table else torch.tensor(value_table, dtype=torch.float32,
+                                                                                  device=where)
+        self._pages = [_PageRecord() for _ in range(capacity)]
+        self._unowned = deque(range(capacity))              # lowest page first
+
+    # -- sizes -------------------------------------------------------------------------------
     @property
     def free_pages(self) -> int:
-        return len(self._free)
+        return len(self._unowned)
 
     @property
     def allocated_pages(self) -> int:
-        return self.capacity - len(self._free)
+        return self.capacity - len(self._unowned)
 
     @property
     def page_payload_bytes(self) -> int:
-        return 2 * (self._code_bytes + self._beta_bytes + 4 * self._row_count)
+        return 2 * sum(width * dtype.itemsize for width, dtype in self._stream_shapes.values())
 
     @property
     def resident_bytes(self) -> int:
-        tensors = [self.key_codes, self.key_betas, self.key_norms, self.value_codes, self.value_betas,
-                   self.value_norms, self.beta_table]
+        held = [getattr(self, name) for name in self._STREAMS] + [self.beta_table]
         if self.value_beta_table is not self.beta_table:
-            tensors.append(self.value_beta_table)
-        return sum(t.numel() * t.element_size() for t in tensors)
+            held.append(self.value_beta_table)
+        return sum(tensor.numel() * tensor.element_size() for tensor in held)
 
+    # -- ownership ---------------------------------------------------------------------------
     def allocate(self) -> NQKVPageHandle:
-        if not self._free:
+        if not self._unowned:
             raise RuntimeError("NQKV page pool is exhausted")
-        page_id = self._free.pop()
-        self._allocated[page_id], self._stored[page_id], self._valid_tokens[page_id] = True, False, 0
-        return NQKVPageHandle(page_id, self._generation[page_id])
+        page_id = self._unowned.popleft()
+        record = self._pages[page_id]
+        record.owned, record.valid_tokens = True, 0
+        return NQKVPageHandle(page_id, record.generation)
 
     def release(self, handle: NQKVPageHandle) -> None:
-        page_id = self._validate_handle(handle)
-        self._allocated[page_id], self._stored[page_id], self._valid_tokens[page_id] = False, False, 0
-        self._generation[page_id] += 1
-        self._free.append(page_id)
+        page_id = self._owned_page(handle)
+        record = self._pages[page_id]
+        record.owned, record.valid_tokens = False, 0
+        record.generation += 1
+        self._unowned.appendleft(page_id)                   # reused next, while it may still be cached
 
-    def store_prepared(self, handle: NQKVPageHandle, page: PreparedNQKVPage) -> None:
-        """Copy a GPU-produced packed page into its fixed physical slot."""
-        page_id = self._validate_handle(handle)
-        if not isinstance(page, PreparedNQKVPage):
-            raise TypeError("page must be a PreparedNQKVPage")
-        if (page.page_size, page.num_kv_heads, page.head_dim, page.q, page.device) != (
-                self.page_size, self.num_kv_heads, self.head_dim, self.q, self.device):
-            raise ValueError("prepared NQKV page configuration does not match the pool")
-        if (not torch.equal(page.key_beta_table, self.beta_table)
-                or not torch.equal(page.value_beta_table, self.value_beta_table)):
-            raise ValueError("prepared NQKV beta tables do not match the pool")
-        for destination, source in zip(
-                (self.key_codes[page_id], self.key_betas[page_id], self.key_norms[page_id],
-                 self.value_codes[page_id], self.value_betas[page_id], self.value_norms[page_id]),
-                (page.key_code_payload, page.key_beta_payload, page.key_norms,
-                 page.value_code_payload, page.value_beta_payload, page.value_norms)):
-            if destination.numel() != source.numel():
-                raise ValueError("prepared NQKV payload sizes do not match the pool")
-            destination.copy_(source)
-        self._valid_tokens[page_id], self._stored[page_id] = page.valid_tokens, True
-
-    def mark_graph_stored(self, handle: NQKVPageHandle, *, valid_tokens: int) -> None:
-        page_id = self._validate_handle(handle)
-        if not 1 <= valid_tokens <= self.page_size:
-            raise ValueError("valid_tokens must be in [1, page_size]")
-        self._valid_tokens[page_id], self._stored[page_id] = valid_tokens, True
-
-    def prepared(self, handle: NQKVPageHandle) -> PreparedNQKVPage:
-        page_id = self._validate_handle(handle)
-        if not self._stored[page_id]:
-            raise RuntimeError("NQKV page has not been stored")
-        return self.page_view(page_id, self._valid_tokens[page_id])
-
-    def page_view(self, page_id: int, valid_tokens: int) -> PreparedNQKVPage:
-        return PreparedNQKVPage(
-            self.key_codes[page_id], self.key_betas[page_id], self.key_norms[page_id],
-            self.value_codes[page_id], self.value_betas[page_id], self.value_norms[page_id],
-            self.beta_table, self.value_beta_table, self.page_size, valid_tokens, self.num_kv_heads,
-            self.head_dim, self.q, self.code_width, self.beta_width, self.output_dtype)
-
-    def _validate_handle(self, handle: NQKVPageHandle) -> int:
+    def _owned_page(self, handle: NQKVPageHandle) -> int:
         if not isinstance(handle, NQKVPageHandle):
             raise TypeError("handle must be an NQKVPageHandle")
         if not 0 <= handle.page_id < self.capacity:
             raise ValueError("NQKV page ID is outside pool capacity")
-        if not self._allocated[handle.page_id] or self._generation[handle.page_id] != handle.generation:
+        record = self._pages[handle.page_id]
+        if not record.owned or record.generation != handle.generation:
             raise RuntimeError("stale or released NQKV page handle")
         return handle.page_id
+
+    # -- payloads ----------------------------------------------------------------------------
+    def store_prepared(self, handle: NQKVPageHandle, page: PreparedNQKVPage) -> None:
+        """Copy a GPU-produced packed page into its fixed physical slot."""
+        page_id = self._owned_page(handle)
+        if not isinstance(page, PreparedNQKVPage):
+            raise TypeError("page must be a PreparedNQKVPage")
+        geometry = (self.page_size, self.num_kv_heads, self.head_dim, self.q, self.device)
+        if (page.page_size, page.num_kv_heads, page.head_dim, page.q, page.device) != geometry:
+            raise ValueError("prepared NQKV page configuration does not match the pool")
+        if not (torch.equal(page.key_beta_table, self.beta_table)
+                and torch.equal(page.value_beta_table, self.value_beta_table)):
+            raise ValueError("prepared NQKV beta tables do not match the pool")
+        incoming = (page.key_code_payload, page.key_beta_payload, page.key_norms,
+                    page.value_code_payload, page.value_beta_payload, page.value_norms)
+        slots = [getattr(self, name)[page_id] for name in self._STREAMS]
+        if any(slot.numel() != stream.numel() for slot, stream in zip(slots, incoming)):
+            raise ValueError("prepared NQKV payload sizes do not match the pool")
+        for slot, stream in zip(slots, incoming):
+            slot.copy_(stream)
+        self._pages[page_id].valid_tokens = page.valid_tokens
+
+    def mark_graph_stored(self, handle: NQKVPageHandle, *, valid_tokens: int) -> None:
+        """Record that a kernel (not store_prepared) has filled the page."""
+        page_id = self._owned_page(handle)
+        if not 1 <= valid_tokens <= self.page_size:
+            raise ValueError("valid_tokens must be in [1, page_size]")
+        self._pages[page_id].valid_tokens = valid_tokens
+
+    def prepared(self, handle: NQKVPageHandle) -> PreparedNQKVPage:
+        page_id = self._owned_page(handle)
+        tokens = self._pages[page_id].valid_tokens
+        if not tokens:
+            raise RuntimeError("NQKV page has not been stored")
+        return self.page_view(page_id, tokens)
+
+    def page_view(self, page_id: int, valid_tokens: int) -> PreparedNQKVPage:
+        return PreparedNQKVPage(
+            *(getattr(self, name)[page_id] for name in self._STREAMS), self.beta_table, self.value_beta_table,
+            self.page_size, valid_tokens, self.num_kv_heads, self.head_dim, self.q, self.code_width, self.beta_width,
+            self.output_dtype)
 
 
 # --------------------------------------------------------------------------------------
