@@ -311,8 +311,20 @@ def row_linear_extra(rt, device):
     return results
 
 
+def rope_gpu(x, positions, theta=500000.0):
+    """Llama rotary embedding (rotate-half form) of [..., tokens, heads, dim] rows at `positions` [tokens]."""
+    import torch
+    dim = x.shape[-1]
+    inv_freq = 1.0 / theta ** (torch.arange(0, dim, 2, device=x.device, dtype=torch.float64) / dim)
+    angle = positions.to(torch.float64)[:, None] * inv_freq[None, :]
+    cos, sin = (torch.cat((f(angle), f(angle)), dim=-1)[:, None, :].float() for f in (torch.cos, torch.sin))
+    half = torch.cat((-x[..., dim // 2:], x[..., :dim // 2]), dim=-1)
+    return x * cos + half * sin
+
+
 def attention_extra(device):
-    """Paged NQKV4 decode attention: 32 / 8 heads, D 64, batch 8, contexts uniform in [128, 4096]."""
+    """Paged NQKV4 decode attention: 32 / 8 heads, D 64, batch 8, contexts uniform in [128, 4096],
+    RoPE (theta = 500000) on keys and queries before their Hadamard."""
     import torch
     from nestquant_aiinfra_amd.runtime import nqkv
     key_betas = tuple(v / 14 for v in (3.50, 4.58, 6.47, 17.06))
@@ -328,11 +340,15 @@ def attention_extra(device):
     manager.step_counts.copy_(torch.tensor(lengths, dtype=torch.int32))
     manager.step_active.fill_(True)
     manager.begin_step(rows=8, uniform_count=None)
+    positions = torch.arange(width, device=device)
     for layer in range(4):                       # distinct layers = distinct (cold) pages per launch
-        key = hadamard_gpu(torch.randn(8, width, 8, 64, generator=g).to(device)).to(torch.bfloat16)
+        key = hadamard_gpu(rope_gpu(torch.randn(8, width, 8, 64, generator=g).to(device), positions)).to(torch.bfloat16)
         value = torch.randn(8, width, 8, 64, generator=g).to(device).to(torch.bfloat16)
         manager.write_layer(layer, key, value)
-    query = hadamard_gpu(torch.randn(8, 32, 64, generator=g).to(device)).to(torch.bfloat16)
+    last = torch.tensor(lengths, device=device) - 1
+    query = torch.randn(8, 32, 64, generator=g).to(device)
+    query = hadamard_gpu(torch.stack([rope_gpu(query[row:row + 1], last[row:row + 1])[0] for row in range(8)]))
+    query = query.to(torch.bfloat16)
     slot_ids = torch.arange(8, dtype=torch.int32, device=device)
     active = torch.ones(8, dtype=torch.bool, device=device)
     workspace = nqkv.BatchedNQKVAttentionWorkspace.create(manager.layers[0], batch_size=8, query_heads=32,

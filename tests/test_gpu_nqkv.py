@@ -254,19 +254,32 @@ def test_attention_merged_inside_the_output_encoder(kv, oracle, batch, max_len, 
         assert torch.equal(getattr(activation, name), getattr(plain, name)), name
 
 
+def _rope(x: np.ndarray, positions: np.ndarray, theta: float = 500000.0) -> np.ndarray:
+    """Llama rotary embedding of [tokens, heads, DIM] rows at the given positions (rotate-half form)."""
+    inv_freq = 1.0 / theta ** (np.arange(0, DIM, 2, dtype=np.float64) / DIM)
+    angle = positions.astype(np.float64)[:, None] * inv_freq[None, :]
+    cos, sin = (np.concatenate((f(angle), f(angle)), axis=-1)[:, None, :].astype(np.float32) for f in (np.cos, np.sin))
+    half = np.concatenate((-x[..., DIM // 2:], x[..., :DIM // 2]), axis=-1)
+    return (x * cos + half * sin).astype(np.float32)
+
+
 def test_attention_ragged_batch_at_full_size(kv, oracle):
-    """Batch 8, 32 query / 8 KV heads, contexts uniform in [128, 4096] (up to 256 pages)."""
+    """Batch 8, 32 query / 8 KV heads, contexts uniform in [128, 4096] (up to 256 pages); keys and
+    queries carry RoPE (theta = 500000) at their positions before the Hadamard, as the model makes them."""
     g = torch.Generator().manual_seed(4001)
     lengths = torch.randint(128, 4097, (8,), generator=g).tolist()
     lengths[0], lengths[1] = 4096, 128
     rng = np.random.default_rng(4002)
     manager = _manager(kv, capacity=8, max_len=4096)
-    keys = [_bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for n in lengths]
+    keys = [_bf16(oracle.hadamard(_rope(rng.standard_normal((n, HEADS, DIM)).astype(np.float32), np.arange(n))))
+            for n in lengths]
     values = [_bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for n in lengths]
     for s in range(8):
         manager.register(s, slot=s)
     _append(manager, list(range(8)), keys, values)
-    query = _bf16(oracle.hadamard(rng.standard_normal((8, 32, DIM)).astype(np.float32))).cuda()
+    query = rng.standard_normal((8, 32, DIM)).astype(np.float32)
+    query = np.stack([_rope(query[row:row + 1], np.array([n - 1]))[0] for row, n in enumerate(lengths)])
+    query = _bf16(oracle.hadamard(query)).cuda()
     slot_ids = torch.arange(8, dtype=torch.int32, device="cuda")
     active = torch.ones(8, dtype=torch.bool, device="cuda")
     out = kv.nqkv_decode_attention_batched_k1(query, manager.layers[0], slot_ids=slot_ids, active_mask=active)
