@@ -44,11 +44,41 @@ def linear_bytes(m: int, k: int, n: int) -> int:
     return n * k // 2 + n * k // 32 + 4 * n + 16 + m * (k // 2 + k // 32 + 4) + 16 + 2 * m * n
 
 
-# HBM bytes per launch of the linear kernel (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by
-# what the same counters read for a 256 MiB copy; runs and factors in
-# profiles/w4a4_gemv_decode_rocprofv3.md).  Counters cannot be read from inside this process.
-MEASURED_TRAFFIC_BYTES = {"q_proj_m1": 3_414_000, "q_proj_m8": 3_613_000, "down_proj_m1": 12_948_000,
-                          "down_proj_m8": 13_836_000}
+# HBM bytes per launch of the linear kernel come from counters (FETCH_SIZE + WRITE_SIZE of rocprofv3
+# --pmc, scaled by what the same counters read for a 256 MiB copy), which cannot be read from inside
+# this process: the profile summary below holds them in its "traffic bytes" column, together with a
+# fingerprint of the kernel sources it was taken on.  A summary taken on other sources is stale and
+# reads as None.
+TRAFFIC_PROFILE = ROOT / "profiles" / "w4a4_gemv_decode_rocprofv3.md"
+KERNEL_SOURCES = ("nq_gemv.hip", "nq_e8.hip.h", "nq_linear_common.hip.h")
+
+
+def kernel_source_fingerprint() -> str:
+    import hashlib
+    digest = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        digest.update((ROOT / "nestquant_aiinfra_amd" / "csrc" / name).read_bytes())
+    return digest.hexdigest()[:16]
+
+
+def measured_traffic_bytes(case_name: str):
+    """`traffic bytes` of e.g. "down_proj_m1" from the profile summary, or None when the summary is
+    missing, does not list the case, or was taken on kernel sources other than the current ones."""
+    try:
+        lines = TRAFFIC_PROFILE.read_text().splitlines()
+    except OSError:
+        return None
+    if not any(line.startswith("Kernel source fingerprint:") and kernel_source_fingerprint() in line for line in lines):
+        return None
+    name, rows = case_name.rsplit("_m", 1)
+    label = f"{name} M={rows} |"
+    for line in lines:
+        cells = [cell.strip() for cell in line.strip().strip("|").split("|")]
+        if label in line and len(cells) == 8 and cells[-1].isdigit():
+            return int(cells[-1])
+    return None
+
+
 # the kernel each case launches (one row: vector units; eight rows: matrix cores, two K ranges per tile)
 CASE_KERNEL = {"q_proj_m1": "w4a4_gemv_kernel<1, 2, true>", "down_proj_m1": "w4a4_gemv_kernel<1, 2, true>",
                "q_proj_m8": "w4a4_gemv_mfma_kernel<2>", "down_proj_m8": "w4a4_gemv_mfma_kernel<2>"}
@@ -167,9 +197,52 @@ def time_kernel_alone(rt, case, copies, launches_per_graph=None):
     return begin.elapsed_time(end) * 1e-3 / (repeats * count)
 
 
-def cpu_baseline(cases, budget_s: float = 12.0):
+def cpu_baseline_torch(cases, budget_s: float):
+    """The same four-linear step with whole-tensor torch operations on the CPU, as the reference's own
+    CPU path evaluates it: one encode + decode pass per beta over the full tensor, argmin over the
+    passes; dither regenerated; dequantise; torch.matmul in FP32."""
+    import numpy as np
+    import torch
+    import oracle
+    from oracle import torch_port
+
+    prepared = []
+    for case in cases:
+        record, n, k = case["record"], case["n"], case["k"]
+        codes = oracle.unpack_unsigned(np.frombuffer(record.indices.code_payload, np.uint8), n * k, 4)
+        ids = oracle.unpack_unsigned(np.frombuffer(record.indices.beta_payload, np.uint8), n * k // 8, 2)
+        prepared.append((case, torch.from_numpy(codes.astype(np.int64)).reshape(n, k // 8, 8),
+                         torch.from_numpy(ids.astype(np.int64)).reshape(n, k // 8), record.row_norms.float().cpu(),
+                         case["x"].float().cpu()))
+
+    def one_step():
+        for case, codes, ids, norms, x in prepared:
+            n, k = case["n"], case["k"]
+            a_codes, a_ids, a_norms = torch_port.quantize_rows(x, Q, ACTIVATION_BETAS)
+            a_hat = torch_port.dequantize_rows(a_codes, a_ids, a_norms, ACTIVATION_BETAS, Q)
+            dither = torch_port.dither_stateless(n * k // 8, case["record"].dither_seed).reshape(n, k // 8, 8)
+            w_hat = torch_port.dequantize_rows(codes, ids, norms, WEIGHT_BETAS, Q, dither)
+            torch.matmul(a_hat, w_hat.t())
+
+    one_step()
+    steps, begin = 0, time.perf_counter()
+    while True:
+        one_step()
+        steps += 1
+        elapsed = time.perf_counter() - begin
+        if elapsed >= budget_s or steps >= 1000:
+            break
+    step_bytes = sum(case["bytes"] for case in cases)
+    return {"value": step_bytes * steps / elapsed / 1e9, "unit": "GB/s", "ms_per_step": elapsed / steps * 1e3,
+            "torch_threads": torch.get_num_threads(), "os_cpu_count": os.cpu_count(),
+            "sample": f"{steps} full steps of the same four-linear workload in {elapsed:.1f} s "
+                      f"(whole-tensor torch operations on the CPU, {torch.get_num_threads()} threads)"}
+
+
+def cpu_baseline(cases, budget_s: float = 10.0):
     """The CPU oracle on the same workload: NQA4-encode the activation, dequantise the
-    NQRT4 weight (dither regenerated), FP32 matvec.  Bounded to about `budget_s` seconds."""
+    NQRT4 weight (dither regenerated), FP32 matvec.  Bounded to about `budget_s` seconds for
+    the C restatement and as much again for the torch-vectorised one reported beside it."""
     import numpy as np
     import oracle
 
@@ -204,6 +277,7 @@ def cpu_baseline(cases, budget_s: float = 12.0):
         "sample": f"{steps} full steps of the same four-linear workload in {elapsed:.1f} s "
                   f"(C oracle, OpenMP, {threads} threads)",
         "ms_per_step": elapsed / steps * 1e3,
+        "torch_vectorised": cpu_baseline_torch(cases, budget_s),
     }
 
 
@@ -479,6 +553,30 @@ def tpot_extra(device, batches=(1, 8), prompt=128, generate=128):
     return results
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def extra_rooflines(extra):
+    """One roofline object per secondary kernel, from the measurements already taken: the prefill
+    GEMM at its largest row count against the dense BF16 matrix-core peak, decode attention and the
+    decode-size encoder against HBM."""
+    gemm = extra["prefill_gemm"]["gate_proj_m4096"]
+    attention = extra["nqkv_attention"]
+    encoders = {name: extra["e8_encode"][name] for name in ("a4_bf16_m1_n2048", "a4_bf16_m1_n8192", "a4_bf16_m4096_n8192")}
+    return {
+        "prefill_gemm": {"bound": "mfma", "workload": "gate_proj K2048 N8192 M4096 (decode of the weight included)",
+                         "achieved": gemm["TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": gemm["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, "launch_us": gemm["us"]},
+        "nqkv_attention": {"bound": "hbm", "workload": "batch 8, 32 / 8 heads, D 64, contexts uniform in [128, 4096]",
+                           "achieved": attention["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                           "frac": attention["hbm_frac"], "launch_us": attention["us"],
+                           "algorithmic_bytes": attention["algorithmic_bytes"]},
+        "e8_encode": {name: {"bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                             "frac": row["hbm_frac"], "launch_us": row["us"], "algorithmic_bytes": row["bytes"]}
+                      for name, row in encoders.items()},
+    }
+
+
 def main() -> None:
     args = parse_args()
     if args.gpus != 1:
@@ -534,7 +632,7 @@ def main() -> None:
     roofline = {
         "bound": "hbm", "kernel": f"{CASE_KERNEL.get(dominant, 'w4a4_gemv_kernel')} ({dominant})",
         "achieved": per_case[dominant]["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": per_case[dominant]["GBps"] / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
+        "frac": per_case[dominant]["GBps"] / HBM_PEAK_GBPS, "traffic": measured_traffic_bytes(dominant),
         "launch_us": per_case[dominant]["us"], "algorithmic_bytes": per_case[dominant]["bytes"],
     }
 
@@ -562,6 +660,7 @@ def main() -> None:
         result["extra"]["nqkv_attention"] = attention_extra(device)
         result["extra"]["bf16_row_linear"] = row_linear_extra(rt, device)
         result["extra"]["llama_1b_w4a4kv4"] = tpot_extra(device)
+        result["extra"]["rooflines"] = extra_rooflines(result["extra"])
     print(json.dumps(result))
 
 
