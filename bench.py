@@ -93,7 +93,10 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--profile-copy", action="store_true",
                         help="also run three 256 MiB device-to-device copies (a kernel of known traffic, "
                              "to calibrate FETCH_SIZE / WRITE_SIZE counters under rocprofv3)")
-    parser.add_argument("--only", choices=("tpot", "gemm", "attention", "encode", "rowlinear"), default=None,
+    parser.add_argument("--library", default=None,
+                        help="another build of libnqhip.so to load (the measuring build that --only encode_phases needs: "
+                             "python -m nestquant_aiinfra_amd.build --define NQ_PHASE_STAMPS --output PATH)")
+    parser.add_argument("--only", choices=("tpot", "gemm", "attention", "encode", "rowlinear", "encode_phases"), default=None,
                         help="run one of the extra measurements alone (for profiling) and print its JSON")
     parser.add_argument("--skip-extras", action="store_true",
                         help="only the headline GEMV workload (no prefill GEMM, attention, TPOT)")
@@ -362,6 +365,50 @@ def encode_extra(rt, device):
     return results
 
 
+def encode_phases_extra(rt, device):
+    """Where one launch of the decode-size encoder spends its time: the wall-clock stamps that lane 0
+    of workgroup 0 leaves at the phase boundaries in a measuring build (--library), beside the
+    launch-to-launch time of the same call in a graph.  Nanoseconds; `outside` is what the launch
+    costs before the first and after the last stamp of that workgroup."""
+    import ctypes
+    import torch
+    from nestquant_aiinfra_amd import _native
+    lib = _native.library()
+    if not hasattr(lib, "nq_debug_phase_stamps"):
+        sys.exit("bench.py: --only encode_phases needs a library built with --define NQ_PHASE_STAMPS (see --library)")
+    lib.nq_debug_phase_stamps.restype = ctypes.c_int
+    lib.nq_debug_phase_stamps.argtypes = [ctypes.c_void_p]
+    table = torch.tensor(ACTIVATION_BETAS, dtype=torch.float32, device=device)
+    g = torch.Generator().manual_seed(59)
+    results = {}
+    for rows, n in ((1, 2048), (8, 2048), (1, 8192), (8, 8192)):
+        x = torch.randn(rows, n, generator=g).to(torch.bfloat16).to(device)
+        other = torch.randn(rows, n, generator=g).to(torch.bfloat16).to(device)
+        weight = (1.0 + 0.1 * torch.randn(n, generator=g)).to(torch.bfloat16).to(device)
+        calls = {
+            "plain": lambda: rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS, beta_table=table, hadamard=True),
+            "rmsnorm": lambda: rt.fused_input_stage(x, mode="rmsnorm", residual=other, norm_weight=weight, eps=1e-5,
+                                                    beta_table=table, want_residual=True),
+            "swiglu": lambda: rt.fused_input_stage(x, mode="swiglu", gate=other, beta_table=table),
+        }
+        for name, call in calls.items():
+            seconds = time_graph(lambda i: call(), 16)
+            call()
+            stamps = (ctypes.c_ulonglong * 16)()
+            _native.check(lib.nq_debug_phase_stamps(stamps))
+            s = [int(v) * 10 for v in stamps[:12]]                      # 100 MHz ticks -> ns
+            inside = s[4] - s[0]
+            results[f"{name}_m{rows}_n{n}"] = {
+                "launch_ns": round(seconds * 1e9), "outside_ns": round(seconds * 1e9) - inside,
+                "stage_ns": s[1] - s[0], "hadamard_ns": s[2] - s[1], "norm_ns": s[3] - s[2], "encode_ns": s[4] - s[3],
+                "hadamard_parts_ns": {"registers_and_lanes": s[8] - s[1], "barrier": s[9] - s[8], "lds_passes": s[2] - s[9]},
+                "norm_parts_ns": {"chains": s[10] - s[2], "sum_sqrt_divide": s[11] - s[10], "barrier": s[3] - s[11]},
+                "encode_parts_ns": {"load_scale_divide": s[5] - s[3], "nearest_point_and_code": s[6] - s[5],
+                                    "decode_and_error": s[7] - s[6], "argmin_and_stores": s[4] - s[7]},
+            }
+    return results
+
+
 def row_linear_extra(rt, device):
     """The BF16 stream kernel: the LM head of the 1B model (128256 x 2048) and, for the optional
     expanded-weights decode, the 1B projection shapes, at 1 and 8 rows.  Algorithmic bytes: the
@@ -582,6 +629,8 @@ def main() -> None:
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only; run with --gpus 1 "
                  "(nothing in the path uses a second GPU)")
+    if args.library:
+        os.environ["NQHIP_LIBRARY"] = str(Path(args.library).resolve())
     import torch
     from nestquant_aiinfra_amd import _native
     from nestquant_aiinfra_amd.runtime import w4a4_linear as rt
@@ -603,7 +652,8 @@ def main() -> None:
     if args.only:
         extra = {"tpot": lambda: tpot_extra(device), "gemm": lambda: prefill_gemm_extra(rt, device),
                  "attention": lambda: attention_extra(device), "encode": lambda: encode_extra(rt, device),
-                 "rowlinear": lambda: row_linear_extra(rt, device)}[args.only]()
+                 "rowlinear": lambda: row_linear_extra(rt, device),
+                 "encode_phases": lambda: encode_phases_extra(rt, device)}[args.only]()
         print(json.dumps({args.only: extra}))
         return
 

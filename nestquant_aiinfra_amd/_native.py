@@ -11,7 +11,10 @@ from pathlib import Path
 
 import torch
 
-LIBRARY_PATH = Path(__file__).resolve().parent / "libnqhip.so"
+import os
+
+# NQHIP_LIBRARY names another build of the same library (a measuring build, say); never a fallback
+LIBRARY_PATH = Path(os.environ.get("NQHIP_LIBRARY") or Path(__file__).resolve().parent / "libnqhip.so")
 
 NQ_OK = 0
 NQ_ERR_ARGUMENT = -1

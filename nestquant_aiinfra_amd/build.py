@@ -1,6 +1,10 @@
 """Builds libnqhip.so (the gfx950 kernels behind the C ABI in include/nqhip.h) in-tree.
 
-    python -m nestquant_aiinfra_amd.build
+    python -m nestquant_aiinfra_amd.build [-v] [--define NAME ...] [--output PATH]
+
+`--define NQ_PHASE_STAMPS --output PATH` makes a measuring build beside the product library: the
+row encoder then stamps the wall clock at its phase boundaries (read with nq_debug_phase_stamps;
+`bench.py --only encode_phases --library PATH` prints the table).
 
 hipcc cross-compiles for gfx950 without a GPU.  Flags that are part of the contract:
   -ffp-contract=off   the codec's float32 operation order is specified; fused
@@ -34,14 +38,16 @@ def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
 
-def build(verbose: bool = False) -> Path:
-    """Compile every csrc/*.hip for gfx950 and link libnqhip.so.  Always recompiles."""
+def build(verbose: bool = False, defines: tuple[str, ...] = (), output: Path = LIBRARY) -> Path:
+    """Compile every csrc/*.hip for gfx950 and link the library (libnqhip.so unless `output`
+    names another file).  Always recompiles."""
     hipcc = os.environ.get("HIPCC", "hipcc")
     objects = []
+    suffix = ".o" if output == LIBRARY else f".{Path(output).stem}.o"
 
     def compile_one(source: Path) -> Path:
-        obj = source.with_suffix(".o")
-        command = [hipcc, *FLAGS, "-c", str(source), "-o", str(obj)]
+        obj = source.with_suffix(suffix)
+        command = [hipcc, *FLAGS, *(f"-D{name}" for name in defines), "-c", str(source), "-o", str(obj)]
         if verbose:
             print(" ".join(command), flush=True)
         result = subprocess.run(command, capture_output=True, text=True)
@@ -56,14 +62,20 @@ def build(verbose: bool = False) -> Path:
 
     with ThreadPoolExecutor(max_workers=min(8, len(sources()) or 1)) as pool:
         objects = list(pool.map(compile_one, sources()))
-    link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(LIBRARY), *map(str, objects)]
+    link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(output), *map(str, objects)]
     result = subprocess.run(link, capture_output=True, text=True)
     if result.returncode != 0:
         raise RuntimeError(f"link failed:\n{result.stderr}")
     for obj in objects:
         obj.unlink(missing_ok=True)
-    return LIBRARY
+    return Path(output)
 
 
 if __name__ == "__main__":
-    print(build(verbose="-v" in sys.argv))
+    import argparse
+    parser = argparse.ArgumentParser()
+    parser.add_argument("-v", action="store_true")
+    parser.add_argument("--define", action="append", default=[])
+    parser.add_argument("--output", type=Path, default=LIBRARY)
+    options = parser.parse_args()
+    print(build(verbose=options.v, defines=tuple(options.define), output=options.output.resolve()))

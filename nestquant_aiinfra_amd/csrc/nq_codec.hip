@@ -1,10 +1,21 @@
 // E8 codec kernels: nearest point, row quantiser with multi-beta selection (NQA4 / NQKV4
 // encoder) and its inverse.  Reference: nestquant/core/quantizer.py:214-301, 39-51;
 // nestquant/runtime/nqkv_page.py:97-185, 332-372, 446-456, 22-95; nestquant/runtime/cuda_e8.cu:8-59.
+#define NQ_PHASE_STAMP_UNIT
 #include "nq_rowquant.hip.h"
 #include "nq_host.h"
 
 #include <math.h>
+#include <type_traits>
+
+#ifdef NQ_PHASE_STAMPS
+// Measuring builds only: the stamps the last encoder launch left (wall clock, 10 ns units).
+extern "C" int nq_debug_phase_stamps(unsigned long long *out16) {
+    if (hipDeviceSynchronize() != hipSuccess) return NQ_ERR_LAUNCH;
+    return hipMemcpyFromSymbol(out16, HIP_SYMBOL(nq::g_phase_stamps), 16 * sizeof(unsigned long long)) == hipSuccess
+               ? NQ_OK : NQ_ERR_LAUNCH;
+}
+#endif
 
 namespace nq {
 
@@ -329,6 +340,7 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
     const int blocks_per_row = n >> 3;
 
     // phase 1
+    NQ_STAMP(0);
     const int64_t first = row0 * n, limit = rows * (int64_t)n;
     if (kPrologue != 0) {
         stage_with_prologue<kPrologue>(reinterpret_cast<const uint16_t *>(x), pro, lds, row_scale, row_norm + rows_per_wg,
@@ -355,13 +367,16 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
         }
     }
     __syncthreads();
+    NQ_STAMP(1);
 
     // optional input rotation, in the arithmetic of the caller's tensor dtype
     if (hadamard_stage_dtype >= 0) staged_hadamard(lds, rows_per_wg, n, hadamard_stage_dtype);
+    NQ_STAMP(2);
 
     // phase 2
     staged_row_norms(lds, rows_per_wg, n, sqrt_n, row_scale, row_norm);
     if (slice == 0 && tid < rows_per_wg && row0 + tid < rows) norms[row0 + tid] = row_norm[tid];
+    NQ_STAMP(3);
 
     // phase 3
     const int slice_pairs = rows_per_wg * blocks_per_row * 4 / slices;     // a multiple of 16
@@ -369,6 +384,322 @@ quantize_rows_kernel(const T *__restrict__ x, int64_t rows, int n, float q, floa
     const SharedBetas betas_of{betas};
     quantize_staged_pairs<kDithered>(lds, row_scale, n, q, inv_q, betas_of, beta_count, seed_plus_offset,
                                      slice_pairs * slice, slice_pairs * (slice + 1), sink);
+    NQ_STAMP(4);
+}
+
+// ---------------------------------------------------------------------------------------
+// One BF16 row per launch slice, one lane per eight neighbouring values (n / 8 lanes, n a power of
+// two from 2048 to 8192, q = 14): the form for decode steps, where the latency of one row is all
+// that counts.  The row never makes the trip through LDS that the general kernel's phases are built
+// around:
+//   * the element-wise stage (residual + RMSNorm, SwiGLU, attention merge) runs on the lane's eight
+//     values in registers; the RMS sum is a sum per lane, a DPP tree per wavefront, one barrier;
+//   * the rotation's butterflies of distance 1 .. 256 follow in the same registers (hadamard_chunk);
+//     rows above 512 values need one pass through LDS for the distances from 512 up;
+//   * the last writer leaves the row in LDS transposed -- element i at (i % 8) * pitch + i / 8 -- so
+//     that each of the eight fused-multiply-add chains of the row norm (element i feeds chain i % 8)
+//     reads its operands four at a time with 128-bit loads instead of one 32-bit load per step;
+//   * the wavefronts that encode run the chains themselves (no hand-over through LDS), and divide
+//     by beta through its reciprocal where that gives the IEEE quotient.
+// Every workgroup of a row repeats all of this and encodes its own slice of the blocks.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum_in_lane_order(float v) {
+    // sum over the 64 lanes: pairs, quads, eights and sixteens by DPP, then the four rows of 16 in order
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+    const int bits = __builtin_bit_cast(int, v);
+    return ((__builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0)) +
+             __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16))) +
+            __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32))) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
+}
+
+// The lane's eight values after the element-wise stage of `pro` (see InputPrologue); g is the index
+// of the first of them in the row-major input.  Mode 1 needs the whole workgroup (one barrier);
+// `wave_sums` is LDS for one float per wavefront.
+template <int kPrologue>
+__device__ __forceinline__ void lane_prologue(const uint16_t *__restrict__ x, const InputPrologue &pro, int64_t g, int n,
+                                              bool writes_outputs, float *wave_sums, float (&y)[8]) {
+    const int chunk = threadIdx.x;
+    if (kPrologue == 3) {
+        constexpr int kBatch = 8;
+        const float kNone = -__builtin_inff();
+#pragma unroll
+        for (int j = 0; j < 8; j++) y[j] = 0.0f;
+        const int64_t head = (g / n) * pro.heads + (g % n) / 64;
+        const float *m = pro.part_max + head * pro.parts, *sum = pro.part_sum + head * pro.parts;
+        const float *acc = pro.part_acc + head * pro.parts * 64 + (g % 64);
+        float top = kNone, denom = 0.0f;
+        for (int c0 = 0; c0 < pro.parts; c0 += kBatch) {
+            float mc[kBatch], sc[kBatch];
+            float4 lo[kBatch], hi[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; j++) {
+                const int c = min(c0 + j, pro.parts - 1);
+                mc[j] = m[c];
+                sc[j] = sum[c];
+                lo[j] = *reinterpret_cast<const float4 *>(acc + (int64_t)c * 64);
+                hi[j] = *reinterpret_cast<const float4 *>(acc + (int64_t)c * 64 + 4);
+            }
+            float batch_top = kNone;
+#pragma unroll
+            for (int j = 0; j < kBatch; j++) {
+                if (c0 + j >= pro.parts) sc[j] = 0.0f;
+                batch_top = fmaxf(batch_top, mc[j]);
+            }
+            const float next_top = fmaxf(top, batch_top);
+            if (next_top > kNone) {
+                const float keep = top > kNone ? __expf(top - next_top) : 0.0f;
+                denom = denom * keep;
+#pragma unroll
+                for (int i = 0; i < 8; i++) y[i] = y[i] * keep;
+#pragma unroll
+                for (int j = 0; j < kBatch; j++) {
+                    const float w = sc[j] > 0.0f ? __expf(mc[j] - next_top) : 0.0f;
+                    denom = denom + sc[j] * w;
+                    const bool used = w > 0.0f;
+                    y[0] += used ? lo[j].x * w : 0.0f; y[1] += used ? lo[j].y * w : 0.0f;
+                    y[2] += used ? lo[j].z * w : 0.0f; y[3] += used ? lo[j].w * w : 0.0f;
+                    y[4] += used ? hi[j].x * w : 0.0f; y[5] += used ? hi[j].y * w : 0.0f;
+                    y[6] += used ? hi[j].z * w : 0.0f; y[7] += used ? hi[j].w * w : 0.0f;
+                }
+                top = next_top;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            y[j] = denom > 0.0f ? y[j] / denom : 0.0f;               // inactive or empty rows give zeros
+            y[j + 1] = denom > 0.0f ? y[j + 1] / denom : 0.0f;
+            round_pair<1>(y[j], y[j + 1]);
+        }
+        if (writes_outputs && pro.normed_out) reinterpret_cast<uint4 *>(pro.normed_out)[g >> 3] = pack_bf16x8_exact(y);
+        return;
+    }
+    // every global operand is requested before any is used: one memory round trip
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    const uint4 raw_x = reinterpret_cast<const uint4 *>(x)[g >> 3];
+    uint4 raw_a = zero, raw_w = zero;
+    if (kPrologue == 1) {
+        if (pro.residual) raw_a = reinterpret_cast<const uint4 *>(pro.residual)[g >> 3];
+        raw_w = reinterpret_cast<const uint4 *>(pro.weight)[chunk];
+    } else if (kPrologue == 2) {
+        raw_a = reinterpret_cast<const uint4 *>(pro.gate)[g >> 3];
+    }
+    unpack_bf16x8(raw_x, y);
+    if (kPrologue == 0) return;
+    float a[8];
+    unpack_bf16x8(raw_a, a);
+    if (kPrologue == 2) {
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            float s0 = a[j] / (1.0f + __expf(-a[j])), s1 = a[j + 1] / (1.0f + __expf(-a[j + 1]));
+            round_pair<1>(s0, s1);
+            y[j] = s0 * y[j];
+            y[j + 1] = s1 * y[j + 1];
+            round_pair<1>(y[j], y[j + 1]);
+        }
+        if (writes_outputs && pro.normed_out) reinterpret_cast<uint4 *>(pro.normed_out)[g >> 3] = pack_bf16x8_exact(y);
+        return;
+    }
+    // LlamaRMSNorm: bf16(weight * bf16(h * rsqrt(mean(h^2) + eps))) with h = x + residual
+    if (pro.residual) {
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            y[j] = y[j] + a[j];
+            y[j + 1] = y[j + 1] + a[j + 1];
+            round_pair<1>(y[j], y[j + 1]);
+        }
+    }
+    if (writes_outputs && pro.residual_out) reinterpret_cast<uint4 *>(pro.residual_out)[g >> 3] = pack_bf16x8_exact(y);
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) sum = __builtin_fmaf(y[j], y[j], sum);
+    sum = wave_sum_in_lane_order(sum);
+    const int waves = (int)(blockDim.x >> 6);
+    if ((threadIdx.x & 63) == 0) wave_sums[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    float total = 0.0f;
+    for (int w = 0; w < waves; w++) total = total + wave_sums[w];
+    const float scale = 1.0f / __builtin_sqrtf(total / (float)n + pro.eps);
+    float w[8];
+    unpack_bf16x8(raw_w, w);
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+        y[j] = y[j] * scale;
+        y[j + 1] = y[j + 1] * scale;
+        round_pair<1>(y[j], y[j + 1]);
+        y[j] = w[j] * y[j];
+        y[j + 1] = w[j + 1] * y[j + 1];
+        round_pair<1>(y[j], y[j + 1]);
+    }
+    if (writes_outputs && pro.normed_out) reinterpret_cast<uint4 *>(pro.normed_out)[g >> 3] = pack_bf16x8_exact(y);
+}
+
+// Pitch (floats) of one chain of the transposed row: 8 more than the chain's length, so that the
+// lanes of a wavefront fall into different banks whether they write chains side by side or read
+// along them.
+__device__ __forceinline__ int chain_pitch(int n) { return (n >> 3) + 8; }
+
+// The rotation's butterflies of distance 512 .. 2^(8 + S) on a row of 2^(9 + S) values staged in
+// order in `natural`, then the scale by `inv`: work item t takes the 2^S values t, t + 512, ... (all
+// of chain t % 8) and leaves them in the transposed row `chains`.  Every result is rounded to BF16.
+template <int S>
+__device__ __forceinline__ void late_stages_to_chains(const float *natural, float *chains, int pitch, float inv) {
+    constexpr int kValues = 1 << S;
+    for (int t = threadIdx.x; t < 512; t += blockDim.x) {
+        float u[kValues];
+#pragma unroll
+        for (int j = 0; j < kValues; j++) u[j] = natural[t + (j << 9)];
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+#pragma unroll
+            for (int j = 0; j < kValues; j++) {
+                if (j & (1 << s)) continue;
+                const float left = u[j], right = u[j + (1 << s)];
+                u[j] = left + right;
+                u[j + (1 << s)] = left - right;
+                round_pair<1>(u[j], u[j + (1 << s)]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kValues; j += 2) {
+            u[j] = u[j] * inv;
+            u[j + 1] = u[j + 1] * inv;
+            round_pair<1>(u[j], u[j + 1]);
+        }
+        float *out = chains + (t & 7) * pitch + (t >> 3);
+#pragma unroll
+        for (int j = 0; j < kValues; j++) out[j << 6] = u[j];
+    }
+}
+
+template <int kPrologue>
+__global__ void __launch_bounds__(1024)
+quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, const float *__restrict__ betas,
+                          int beta_count, float sqrt_n, uint32_t *__restrict__ codes, uint8_t *__restrict__ beta_ids,
+                          float *__restrict__ norms, uint4 *__restrict__ decoded, int slices, int rotate,
+                          InputPrologue pro) {
+    extern __shared__ float lds[];
+    const int pitch = chain_pitch(n);
+    float *chains = lds;                                  // 8 * pitch floats: the row, transposed
+    float *natural = chains + 8 * pitch;                  // n floats: the row in order (rows above 512 values, rotated)
+    __shared__ float wave_sums[16];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int slice = blockIdx.x % slices;
+    const int64_t row = blockIdx.x / slices;
+    const int log_n = 31 - __builtin_clz(n);
+    const bool live = (tid & 3) < beta_count;
+    // requested first, used last; a launch that only runs the element-wise stage has no table
+    const float beta = codes != nullptr ? betas[live ? (tid & 3) : 0] : 1.0f;
+    NQ_STAMP(0);
+
+    float v[8];
+    lane_prologue<kPrologue>(x, pro, row * n + 8 * tid, n, slice == 0, wave_sums, v);
+    if (codes == nullptr) return;                         // element-wise stage only
+    NQ_STAMP(1);
+
+    const bool late_stages = rotate && log_n > 9;
+    if (rotate) hadamard_chunk<1>(v, lane, log_n - 3 < 6 ? log_n - 3 : 6, log_n <= 9, 1.0f / __builtin_sqrtf((float)n));
+    NQ_STAMP(8);
+    if (late_stages) {
+        *reinterpret_cast<float4 *>(natural + 8 * tid) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4 *>(natural + 8 * tid + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        __syncthreads();
+        NQ_STAMP(9);
+        const float inv = 1.0f / __builtin_sqrtf((float)n);
+        switch (log_n - 9) {
+            case 1: late_stages_to_chains<1>(natural, chains, pitch, inv); break;
+            case 2: late_stages_to_chains<2>(natural, chains, pitch, inv); break;
+            case 3: late_stages_to_chains<3>(natural, chains, pitch, inv); break;
+            default: late_stages_to_chains<4>(natural, chains, pitch, inv); break;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) chains[j * pitch + tid] = v[j];
+    }
+    __syncthreads();
+    NQ_STAMP(2);
+
+    // only the first four wavefronts encode (256 pairs of the slice); the others are done
+    if (tid >= 256) return;
+
+    // row norm in the reference's order (quantizer.py:257): chain k sums the squares of elements
+    // k, k + 8, ... with fused multiply-adds; chains added 0..7; sqrt.  Lanes 8 .. 63 run along
+    // (on chain lane % 8) so that the wavefront stays uniform.
+    float norm;
+    {
+        const float4 *chain = reinterpret_cast<const float4 *>(chains + (lane & 7) * pitch);
+        const int quads = n >> 5;                          // 128-bit loads per chain, a multiple of 16
+        float acc = 0.0f;
+        float4 a[8], b[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) a[k] = chain[k];
+        for (int at = 0; at < quads; at += 16) {
+#pragma unroll
+            for (int k = 0; k < 8; k++) b[k] = chain[at + 8 + k];
+            __builtin_amdgcn_sched_barrier(0);            // keep the requests ahead of the chain
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                acc = __builtin_fmaf(a[k].x, a[k].x, acc);
+                acc = __builtin_fmaf(a[k].y, a[k].y, acc);
+                acc = __builtin_fmaf(a[k].z, a[k].z, acc);
+                acc = __builtin_fmaf(a[k].w, a[k].w, acc);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const int after = at + 16 < quads ? at + 16 : at;      // a request past the end repeats the last batch, unused
+#pragma unroll
+            for (int k = 0; k < 8; k++) a[k] = chain[after + k];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                acc = __builtin_fmaf(b[k].x, b[k].x, acc);
+                acc = __builtin_fmaf(b[k].y, b[k].y, acc);
+                acc = __builtin_fmaf(b[k].z, b[k].z, acc);
+                acc = __builtin_fmaf(b[k].w, b[k].w, acc);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        NQ_STAMP(10);
+        float total = 0.0f;
+        const int bits = __builtin_bit_cast(int, acc);
+#pragma unroll
+        for (int k = 0; k < 8; k++) total = total + __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, k));
+        norm = __builtin_sqrtf(total);
+    }
+    // math.sqrt(n) / norm is evaluated as (1 / norm) * float32(sqrt(n))
+    const float scale = norm > 0.0f ? (1.0f / norm) * sqrt_n : 0.0f;
+    if (slice == 0 && tid == 0) norms[row] = norm;
+    NQ_STAMP(3);
+
+    // one lane per (block, beta) pair of the slice
+    const int blocks_per_row = n >> 3;
+    const int p = slice * 256 + tid, b = p >> 2, bi = p & 3;
+    float raw[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) raw[j] = chains[j * pitch + b];
+    struct LaneSink {
+        uint32_t *codes; uint8_t *beta_ids; uint4 *decoded; int64_t first_block; float back;
+        __device__ __forceinline__ bool wants(int) const { return true; }
+        __device__ __forceinline__ void code(int, int b, uint32_t word, const float (&recon)[8], float beta) const {
+            codes[first_block + b] = word;
+            if (decoded) {
+                uint32_t h[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) h[j] = f32_to_bf16((recon[j] * beta) * back);
+                decoded[first_block + b] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16),
+                                                      h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+            }
+        }
+        __device__ __forceinline__ void beta_byte(int, int b, uint32_t byte) const {
+            beta_ids[(first_block + b) >> 2] = (uint8_t)byte;
+        }
+        __device__ __forceinline__ uint32_t counter(int, int) const { return 0; }
+    };
+    const LaneSink sink{codes, beta_ids, decoded, row * blocks_per_row, norm / sqrt_n};
+    quantize_pair_lane<false, true>(raw, scale, beta, live, bi, 0, b, p, 14.0f, 1.0f / 14.0f, 0u, sink);
+    NQ_STAMP(4);
 }
 
 // Many rows: 256 lanes per workgroup, `rows_per_wg` rows of together at least 2048 values, one
@@ -672,6 +1003,27 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
                            (float)sqrt((double)n), reinterpret_cast<uint32_t *>(codes), beta_ids, norms,
                            reinterpret_cast<uint4 *>(decoded), rows_per_wg, (int)nq::aligned(x, 16),
                            hadamard_stage_dtype, prologue);
+        return nq::check_launch("nq_quantize_rows");
+    }
+    // decode steps: up to 16 BF16 rows of 2048, 4096 or 8192 values, q = 14, every operand
+    // 16-byte aligned: one lane per eight values, each row repeated over as many workgroups as it has
+    // slices of 256 (block, beta) pairs
+    if (std::is_same<T, uint16_t>::value && !kDithered && q == 14 && (n == 2048 || n == 4096 || n == 8192) &&
+        rows <= 16 && nq::aligned(x, 16)) {
+        const int slices = n / 512;                       // 4 * (n / 8) pairs in slices of 256
+        const size_t lds_bytes = (size_t)(8 * ((n >> 3) + 8) + n) * sizeof(float);
+        auto kernel = nq::quantize_row_lanes_kernel<kPrologue>;
+        if (lds_bytes > 48 * 1024) {
+            hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (status != hipSuccess)
+                return nq::fail(NQ_ERR_LAUNCH, "nq_quantize_rows: cannot reserve %zu bytes of LDS: %s",
+                                lds_bytes, hipGetErrorString(status));
+        }
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(rows * slices)), dim3(n / 8), lds_bytes, stream,
+                           reinterpret_cast<const uint16_t *>(x), rows, n, betas, beta_count, (float)sqrt((double)n),
+                           reinterpret_cast<uint32_t *>(codes), beta_ids, norms, reinterpret_cast<uint4 *>(decoded),
+                           slices, hadamard_stage_dtype >= 0 ? 1 : 0, prologue);
         return nq::check_launch("nq_quantize_rows");
     }
     const int pairs_per_row = n / 2;

@@ -12,6 +12,17 @@
 
 #include "nq_e8.hip.h"
 
+// Phase stamps of the row encoder (a measuring build only, -DNQ_PHASE_STAMPS, and only in the
+// translation unit that asks for them with NQ_PHASE_STAMP_UNIT): lane 0 of workgroup 0 writes the
+// 100 MHz wall clock at the phase boundaries into a device array that nq_debug_phase_stamps
+// copies out.  Otherwise the macro is empty.
+#if defined(NQ_PHASE_STAMPS) && defined(NQ_PHASE_STAMP_UNIT)
+namespace nq { __device__ unsigned long long g_phase_stamps[16]; }
+#define NQ_STAMP(i) do { if (blockIdx.x == 0 && threadIdx.x == 0) nq::g_phase_stamps[i] = wall_clock64(); } while (0)
+#else
+#define NQ_STAMP(i) do { } while (0)
+#endif
+
 namespace nq {
 
 // exchange with the lane whose id differs in bit 0 / bit 1 (inside a quad)
@@ -132,6 +143,39 @@ __device__ __forceinline__ void lane_stage(float (&v)[8], int lane) {
     for (int j = 0; j < 8; j += 2) round_pair<kDtype>(v[j], v[j + 1]);
 }
 
+// The butterflies of distance 1 .. 2^(2 + lane_stages) on the eight neighbouring values every lane of
+// a wavefront holds (value j of lane l is element 8 l + j of the wavefront's 512): distances 1, 2, 4
+// in registers, 8 .. 256 between lanes.  With scale_here the results are multiplied by `inv` and
+// rounded once more.
+template <int kDtype>
+__device__ __forceinline__ void hadamard_chunk(float (&v)[8], int lane, int lane_stages, bool scale_here, float inv) {
+#pragma unroll
+    for (int s = 0; s < 3; s++) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            if (j & (1 << s)) continue;
+            const float left = v[j], right = v[j + (1 << s)];
+            v[j] = left + right;
+            v[j + (1 << s)] = left - right;
+            round_pair<kDtype>(v[j], v[j + (1 << s)]);
+        }
+    }
+    if (lane_stages > 0) lane_stage<1, kDtype>(v, lane);
+    if (lane_stages > 1) lane_stage<2, kDtype>(v, lane);
+    if (lane_stages > 2) lane_stage<4, kDtype>(v, lane);
+    if (lane_stages > 3) lane_stage<8, kDtype>(v, lane);
+    if (lane_stages > 4) lane_stage<16, kDtype>(v, lane);
+    if (lane_stages > 5) lane_stage<32, kDtype>(v, lane);
+    if (scale_here) {
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            v[j] = v[j] * inv;
+            v[j + 1] = v[j + 1] * inv;
+            round_pair<kDtype>(v[j], v[j + 1]);
+        }
+    }
+}
+
 // Normalized Sylvester-Hadamard transform of rows staged in LDS (nestquant/core/rotation.py:12-27):
 // butterflies of growing width, each sum and difference rounded to `stage_dtype` (the dtype
 // the reference's tensor ops would run in), then one multiplication by float32(1 / sqrt(n))
@@ -167,37 +211,15 @@ __device__ __forceinline__ void staged_hadamard_as(float *rows, int row_count, i
         float4 *slot = reinterpret_cast<float4 *>(rows + 8 * chunk);
         const float4 lo = slot[0], hi = slot[1];
         float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-#pragma unroll
-        for (int s = 0; s < 3; s++) {
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                if (j & (1 << s)) continue;
-                const float left = v[j], right = v[j + (1 << s)];
-                v[j] = left + right;
-                v[j + (1 << s)] = left - right;
-                round_pair<kDtype>(v[j], v[j + (1 << s)]);
-            }
-        }
         // a row's chunks sit in neighbouring lanes (n / 8 of them, a power of two), so the
         // stage count is the same for the whole wavefront
-        if (lane_stages > 0) lane_stage<1, kDtype>(v, lane);
-        if (lane_stages > 1) lane_stage<2, kDtype>(v, lane);
-        if (lane_stages > 2) lane_stage<4, kDtype>(v, lane);
-        if (lane_stages > 3) lane_stage<8, kDtype>(v, lane);
-        if (lane_stages > 4) lane_stage<16, kDtype>(v, lane);
-        if (lane_stages > 5) lane_stage<32, kDtype>(v, lane);
-        if (scale_here) {
-#pragma unroll
-            for (int j = 0; j < 8; j += 2) {
-                v[j] = v[j] * inv;
-                v[j + 1] = v[j + 1] * inv;
-                round_pair<kDtype>(v[j], v[j + 1]);
-            }
-        }
+        hadamard_chunk<kDtype>(v, lane, lane_stages, scale_here, inv);
         slot[0] = make_float4(v[0], v[1], v[2], v[3]);
         slot[1] = make_float4(v[4], v[5], v[6], v[7]);
     }
+    NQ_STAMP(8);
     __syncthreads();
+    NQ_STAMP(9);
     int log_w = 9;
     for (; log_n - log_w > 4; log_w += 3) hadamard_pass<3, kDtype, false>(rows, total, log_w, inv);
     switch (log_n - log_w) {
@@ -268,6 +290,7 @@ __device__ __forceinline__ void staged_row_norms(const float *rows, int row_coun
                 acc = __builtin_fmaf(v2, v2, acc);
                 acc = __builtin_fmaf(v3, v3, acc);
             }
+            NQ_STAMP(10);
             float total = 0.0f;
 #pragma unroll
             for (int k = 0; k < 8; k++) total = total + __shfl(acc, (tid & 56) + k, 64);
@@ -279,7 +302,80 @@ __device__ __forceinline__ void staged_row_norms(const float *rows, int row_coun
             }
         }
     }
+    NQ_STAMP(11);
     __syncthreads();
+}
+
+// One lane's share of a block: its values `raw` (to be scaled by `scale`) against the beta of index
+// bi (quantizer.py:273-289); the quad of lanes bi = 0..3 then settles the first minimum by two
+// exchanges, the winner hands the code word to the sink, and sixteen lanes merge the beta byte of
+// four neighbouring blocks.  p = (row * blocks_per_row + block) * 4 + bi.  With kFastDivide the
+// division by beta goes through its reciprocal where that gives the IEEE quotient (a zero quotient
+// may then carry the other sign; the lattice search treats both alike).
+template <bool kDithered, bool kFastDivide, class Sink>
+__device__ __forceinline__ void quantize_pair_lane(const float (&raw)[8], float scale, float beta, bool live, int bi,
+                                                   int r, int b, int p, float q, float inv_q,
+                                                   uint32_t seed_plus_offset, const Sink &sink) {
+    float y[8], z[8], code[8], p8[8], recon[8], dither[8];
+    if (kDithered) dither_block(seed_plus_offset + sink.counter(r, b), dither);
+#pragma unroll
+    for (int j = 0; j < 8; j++) y[j] = raw[j] * scale;
+    // the same decision for the whole wavefront; the quotients are the IEEE ones either way
+    const bool by_reciprocal = kFastDivide && beta >= 0x1p-40f && beta <= 0x1p40f &&
+                               __builtin_amdgcn_ballot_w64(has_tiny_nonzero(y)) == 0;
+    if (by_reciprocal) {
+        const float rcp = 1.0f / beta;
+#pragma unroll
+        for (int j = 0; j < 8; j++) z[j] = divide_by_reciprocal(y[j], beta, rcp);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) z[j] = y[j] / beta;     // IEEE division
+    }
+    if (kDithered) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) z[j] = z[j] + dither[j];
+    }
+    NQ_STAMP(5);
+    encode_block(z, q, inv_q, code);
+    NQ_STAMP(6);
+    e8_coset_point(code, p8);
+    if (kDithered) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) p8[j] = p8[j] - dither[j];
+    }
+    reduce_coset_point(p8, q, recon);
+    float err = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float d = recon[j] * beta - y[j];
+        err = err + d * d;
+    }
+    if (!live) err = __builtin_inff();
+    NQ_STAMP(7);
+
+    // first minimum over the quad: order by (err, beta index)
+    uint32_t best_err = __float_as_uint(err), best = (uint32_t)bi;
+    {
+        const uint32_t oe = quad_xor1(best_err), oi = quad_xor1(best);
+        const float fe = __uint_as_float(oe), me = __uint_as_float(best_err);
+        const bool take = fe < me || (fe == me && oi < best);
+        best_err = take ? oe : best_err;
+        best = take ? oi : best;
+    }
+    {
+        const uint32_t oe = quad_xor2(best_err), oi = quad_xor2(best);
+        const float fe = __uint_as_float(oe), me = __uint_as_float(best_err);
+        const bool take = fe < me || (fe == me && oi < best);
+        best = take ? oi : best;
+    }
+    const bool wanted = sink.wants(r);
+    if (best == (uint32_t)bi && wanted) sink.code(r, b, pack_codeword(code), recon, beta);
+
+    // four consecutive blocks (16 lanes) share one beta byte
+    uint32_t byte = best << (2 * (b & 3));
+    byte |= (uint32_t)__shfl_xor((int)byte, 4, 64);
+    byte |= (uint32_t)__shfl_xor((int)byte, 8, 64);
+    if ((p & 15) == 0 && wanted) sink.beta_byte(r, b, byte);
 }
 
 // Pairs [pair_begin, pair_end) of the staged rows (pair = (row * n / 8 + block) * 4 + beta
@@ -300,53 +396,8 @@ __device__ __forceinline__ void quantize_staged_pairs(const float *rows, const f
         const float4 hi = *reinterpret_cast<const float4 *>(rows + (size_t)r * n + 8 * b + 4);
         const float raw[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
         const bool live = bi < beta_count;
-        const float beta = betas_of(r)[live ? bi : 0];
-        float y[8], z[8], code[8], p8[8], recon[8], dither[8];
-        if (kDithered) dither_block(seed_plus_offset + sink.counter(r, b), dither);
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            y[j] = raw[j] * scale;
-            z[j] = y[j] / beta;                 // IEEE division
-            if (kDithered) z[j] = z[j] + dither[j];
-        }
-        encode_block(z, q, inv_q, code);
-        e8_coset_point(code, p8);
-        if (kDithered) {
-#pragma unroll
-            for (int j = 0; j < 8; j++) p8[j] = p8[j] - dither[j];
-        }
-        reduce_coset_point(p8, q, recon);
-        float err = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const float d = recon[j] * beta - y[j];
-            err = err + d * d;
-        }
-        if (!live) err = __builtin_inff();
-
-        // first minimum over the quad: order by (err, beta index)
-        uint32_t best_err = __float_as_uint(err), best = (uint32_t)bi;
-        {
-            const uint32_t oe = quad_xor1(best_err), oi = quad_xor1(best);
-            const float fe = __uint_as_float(oe), me = __uint_as_float(best_err);
-            const bool take = fe < me || (fe == me && oi < best);
-            best_err = take ? oe : best_err;
-            best = take ? oi : best;
-        }
-        {
-            const uint32_t oe = quad_xor2(best_err), oi = quad_xor2(best);
-            const float fe = __uint_as_float(oe), me = __uint_as_float(best_err);
-            const bool take = fe < me || (fe == me && oi < best);
-            best = take ? oi : best;
-        }
-        const bool wanted = sink.wants(r);
-        if (best == (uint32_t)bi && wanted) sink.code(r, b, pack_codeword(code), recon, beta);
-
-        // four consecutive blocks (16 lanes) share one beta byte
-        uint32_t byte = best << (2 * (b & 3));
-        byte |= (uint32_t)__shfl_xor((int)byte, 4, 64);
-        byte |= (uint32_t)__shfl_xor((int)byte, 8, 64);
-        if ((p & 15) == 0 && wanted) sink.beta_byte(r, b, byte);
+        quantize_pair_lane<kDithered, false>(raw, scale, betas_of(r)[live ? bi : 0], live, bi, r, b, p, q, inv_q,
+                                             seed_plus_offset, sink);
     }
 }
 
