@@ -633,13 +633,18 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
         const float4 *chain = reinterpret_cast<const float4 *>(chains + (lane & 7) * pitch);
         const int quads = n >> 5;                          // 128-bit loads per chain, a multiple of 16
         float acc = 0.0f;
+        // Batches of 32 chain steps, double-buffered by hand: the next batch is requested from LDS
+        // before the chain runs over the current one.  The address of a request waits for the chain
+        // (adding zero unless the sum is NaN), so that it reuses the registers the chain has just
+        // released and the loop carries no copies.
         float4 a[8], b[8];
 #pragma unroll
         for (int k = 0; k < 8; k++) a[k] = chain[k];
-        for (int at = 0; at < quads; at += 16) {
+        int at = 0;
+        for (; at + 16 < quads; at += 16) {
 #pragma unroll
             for (int k = 0; k < 8; k++) b[k] = chain[at + 8 + k];
-            __builtin_amdgcn_sched_barrier(0);            // keep the requests ahead of the chain
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int k = 0; k < 8; k++) {
                 acc = __builtin_fmaf(a[k].x, a[k].x, acc);
@@ -648,9 +653,9 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
                 acc = __builtin_fmaf(a[k].w, a[k].w, acc);
             }
             __builtin_amdgcn_sched_barrier(0);
-            const int after = at + 16 < quads ? at + 16 : at;      // a request past the end repeats the last batch, unused
+            const float4 *next = chain + at + 16 + (acc != acc ? 1 : 0);
 #pragma unroll
-            for (int k = 0; k < 8; k++) a[k] = chain[after + k];
+            for (int k = 0; k < 8; k++) a[k] = next[k];
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int k = 0; k < 8; k++) {
@@ -660,6 +665,22 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
                 acc = __builtin_fmaf(b[k].w, b[k].w, acc);
             }
             __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) b[k] = chain[at + 8 + k];
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            acc = __builtin_fmaf(a[k].x, a[k].x, acc);
+            acc = __builtin_fmaf(a[k].y, a[k].y, acc);
+            acc = __builtin_fmaf(a[k].z, a[k].z, acc);
+            acc = __builtin_fmaf(a[k].w, a[k].w, acc);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            acc = __builtin_fmaf(b[k].x, b[k].x, acc);
+            acc = __builtin_fmaf(b[k].y, b[k].y, acc);
+            acc = __builtin_fmaf(b[k].z, b[k].z, acc);
+            acc = __builtin_fmaf(b[k].w, b[k].w, acc);
         }
         NQ_STAMP(10);
         float total = 0.0f;
