@@ -96,7 +96,7 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--library", default=None,
                         help="another build of libnqhip.so to load (the measuring build that --only encode_phases needs: "
                              "python -m nestquant_aiinfra_amd.build --define NQ_PHASE_STAMPS --output PATH)")
-    parser.add_argument("--only", choices=("tpot", "gemm", "attention", "encode", "rowlinear", "encode_phases"), default=None,
+    parser.add_argument("--only", choices=("tpot", "gemm", "attention", "encode", "rowlinear", "encode_phases", "attention_phases"), default=None,
                         help="run one of the extra measurements alone (for profiling) and print its JSON")
     parser.add_argument("--skip-extras", action="store_true",
                         help="only the headline GEMV workload (no prefill GEMM, attention, TPOT)")
@@ -409,6 +409,56 @@ def encode_phases_extra(rt, device):
     return results
 
 
+def attention_phases_extra(device):
+    """Where one launch of the decode attention (stage 1) spends its time, from the wall-clock stamps
+    that lane 0 of the first workgroup (row 0, KV head 0, first chunk of pages) leaves in a measuring
+    build (--library): contexts of a decode step after a 128-token prompt, and the ragged long ones."""
+    import ctypes
+    import torch
+    from nestquant_aiinfra_amd import _native
+    from nestquant_aiinfra_amd.runtime import nqkv
+    lib = _native.library()
+    if not hasattr(lib, "nq_debug_attention_stamps"):
+        sys.exit("bench.py: --only attention_phases needs a library built with --define NQ_PHASE_STAMPS (see --library)")
+    lib.nq_debug_attention_stamps.restype = ctypes.c_int
+    lib.nq_debug_attention_stamps.argtypes = [ctypes.c_void_p]
+    key_betas = tuple(v / 14 for v in (3.50, 4.58, 6.47, 17.06))
+    value_betas = tuple(v / 14 for v in (3.53, 5.59, 9.62, 29.03))
+    g = torch.Generator().manual_seed(4001)
+    results = {}
+    for name, lengths in (("decode_after_128", [200] * 8), ("ragged_128_4096", torch.randint(128, 4097, (8,), generator=g).tolist())):
+        manager = nqkv.BatchedNQKVCacheManager(capacity=8, num_layers=4, num_kv_heads=8, head_dim=64, max_cache_len=4096,
+                                               page_size=16, q=Q, key_betas=key_betas, value_betas=value_betas,
+                                               dtype=torch.bfloat16, device=device)
+        width = max(lengths)
+        for slot in range(8):
+            manager.register(slot, slot=slot)
+        manager.step_counts.copy_(torch.tensor(lengths, dtype=torch.int32))
+        manager.step_active.fill_(True)
+        manager.begin_step(rows=8, uniform_count=None)
+        for layer in range(4):
+            key = hadamard_gpu(torch.randn(8, width, 8, 64, generator=g).to(device)).to(torch.bfloat16)
+            value = torch.randn(8, width, 8, 64, generator=g).to(device).to(torch.bfloat16)
+            manager.write_layer(layer, key, value)
+        query = hadamard_gpu(torch.randn(8, 32, 64, generator=g).to(device)).to(torch.bfloat16)
+        slot_ids = torch.arange(8, dtype=torch.int32, device=device)
+        active = torch.ones(8, dtype=torch.bool, device=device)
+        workspace = nqkv.BatchedNQKVAttentionWorkspace.create(manager.layers[0], batch_size=8, query_heads=32,
+                                                              output_dtype=torch.bfloat16)
+        call = lambda i: nqkv.launch_nqkv_decode_attention(query, manager.layers[i % 4], slot_ids=slot_ids, active_mask=active,
+                                                           attention_scale=0.125, workspace=workspace).clone()
+        seconds = time_graph(call, 8)
+        call(0)
+        stamps = (ctypes.c_ulonglong * 16)()
+        _native.check(lib.nq_debug_attention_stamps(stamps))
+        s = [int(v) * 10 for v in stamps[:8]]
+        results[name] = {"launch_ns_with_merge": round(seconds * 1e9), "tables_ns": s[1] - s[0],
+                         "key_requests_and_query_ns": s[2] - s[1], "query_to_registers_ns": s[3] - s[2],
+                         "key_pass_ns": s[4] - s[3], "softmax_ns": s[5] - s[4], "value_pass_ns": s[6] - s[5],
+                         "fold_and_store_ns": s[7] - s[6], "inside_ns": s[7] - s[0]}
+    return results
+
+
 def row_linear_extra(rt, device):
     """The BF16 stream kernel: the LM head of the 1B model (128256 x 2048) and, for the optional
     expanded-weights decode, the 1B projection shapes, at 1 and 8 rows.  Algorithmic bytes: the
@@ -653,7 +703,8 @@ def main() -> None:
         extra = {"tpot": lambda: tpot_extra(device), "gemm": lambda: prefill_gemm_extra(rt, device),
                  "attention": lambda: attention_extra(device), "encode": lambda: encode_extra(rt, device),
                  "rowlinear": lambda: row_linear_extra(rt, device),
-                 "encode_phases": lambda: encode_phases_extra(rt, device)}[args.only]()
+                 "encode_phases": lambda: encode_phases_extra(rt, device),
+                 "attention_phases": lambda: attention_phases_extra(device)}[args.only]()
         print(json.dumps({args.only: extra}))
         return
 

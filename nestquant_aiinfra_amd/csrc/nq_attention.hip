@@ -19,14 +19,24 @@
 // beyond the table width (the reference stops at 64 pages, nqkv_attention_k1.py:696-698).
 // Decoded K/V stay FP32 (as in the reference's fused kernel); K/V decode follows the exact
 // float32 order of nq_e8.hip.h because undithered codes sit on exact Voronoi ties.
+#define NQ_PHASE_STAMP_ARRAY g_attention_stamps
 #include "nq_rowquant.hip.h"
 #include "nq_host.h"
 
 #include <math.h>
 
+#ifdef NQ_PHASE_STAMPS
+// Measuring builds only: the stamps the last stage-1 launch left (wall clock, 10 ns units).
+extern "C" int nq_debug_attention_stamps(unsigned long long *out16) {
+    if (hipDeviceSynchronize() != hipSuccess) return NQ_ERR_LAUNCH;
+    return hipMemcpyFromSymbol(out16, HIP_SYMBOL(nq::g_attention_stamps), 16 * sizeof(unsigned long long)) == hipSuccess
+               ? NQ_OK : NQ_ERR_LAUNCH;
+}
+#endif
+
 namespace nq {
 
-constexpr int kAttnThreads = 256;
+constexpr int kAttnThreads = 512;
 constexpr int kAttnMaxPagesPerChunk = 16;
 constexpr int kAttnMaxGroup = 8;
 
@@ -75,6 +85,45 @@ __device__ __forceinline__ float sum8(float v) {
     return v;
 }
 
+// maximum / sum over the 64 lanes of a wavefront, the same value in every lane: register exchanges
+// inside rows of 16 lanes, then the four rows through scalar registers
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_quad_xor1(v));
+    v = fmaxf(v, dpp_quad_xor2(v));
+    v = fmaxf(v, dpp_half_mirror(v));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true)));
+    const int bits = __builtin_bit_cast(int, v);
+    return fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0)),
+                       __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16))),
+                 fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32)),
+                       __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48))));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v = v + dpp_quad_xor1(v);
+    v = v + dpp_quad_xor2(v);
+    v = v + dpp_half_mirror(v);
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+    const int bits = __builtin_bit_cast(int, v);
+    return (__builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0)) +
+            __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16))) +
+           (__builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32)) +
+            __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48)));
+}
+// v + the value of the lane 16 / 32 further on (the same in both lanes)
+__device__ __forceinline__ float fold_rows(float v) {
+    const int bits = __builtin_bit_cast(int, v);
+    const auto by16 = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    const float half = __builtin_bit_cast(float, (int)by16[0]) + __builtin_bit_cast(float, (int)by16[1]);
+    const int half_bits = __builtin_bit_cast(int, half);
+    const auto by32 = __builtin_amdgcn_permlane32_swap(half_bits, half_bits, false, false);
+    return __builtin_bit_cast(float, (int)by32[0]) + __builtin_bit_cast(float, (int)by32[1]);
+}
+
+// The dependent loads of a workgroup are what a short context pays for, so they are arranged in
+// three rounds, each requested as early as its addresses are known: (1) the row's slot and
+// activity flag, the group's queries and their rotary rows; (2) the slot's lengths and the page
+// ids of the chunk (requested for every ordinal of the chunk before the count says which exist);
+// (3) the packed keys and values of every pass together.
 template <int D, int P, int G, int kAttnPagesPerChunk>     // head_dim, page_size, query heads per KV head, pages per chunk
 __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(AttentionArgs a) {
     constexpr int kBlocks = D / 8;                       // E8 blocks per head vector
@@ -82,18 +131,16 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     constexpr int kPagesPerPass = kAttnThreads / kTokenBlocks;
     constexpr int kPasses = kAttnPagesPerChunk / kPagesPerPass;
     constexpr int kChunkTokens = kAttnPagesPerChunk * P;
+    constexpr int kWaves = kAttnThreads / 64;
     static_assert(kTokenBlocks * kPagesPerPass == kAttnThreads && kPasses * kPagesPerPass == kAttnPagesPerChunk,
                   "page does not tile the workgroup");
+    static_assert(D == 64 && G * 8 <= 64 && kBlocks == 8, "eight lanes of the first wavefront prepare one head's query");
+    static_assert(kChunkTokens % 64 == 0, "every lane of a wavefront takes the same number of scores");
     __shared__ float scores[G][kChunkTokens];
-    __shared__ float reduce_buf[kAttnThreads / 64][G];
-    __shared__ float chunk_max[G], chunk_sum[G];
-    __shared__ float acc_lds[kAttnThreads / 16][kBlocks][G * 8];   // one entry per 16-lane row
+    __shared__ float acc_lds[kWaves][G * 8][kBlocks];    // one entry per wavefront; holds the queries first
 
-    // The part of (block, row) that does not reach the bank index through the address, as an XOR mask
-    // for the G * 8 columns of acc_lds: the block bits that overflow 32 banks, and two row bits.
-    constexpr int kOverflowShift = G >= 4 ? 0 : (G == 2 ? 1 : 2);
-    auto acc_swizzle = [](int block, int row16) { return 4 * (block >> kOverflowShift) + (row16 & 3); };
     const int tid = threadIdx.x;
+    NQ_STAMP(0);
     // Workgroups go to the eight XCDs in turn by their linear index, and every XCD has its own L2.
     // A page stores the blocks of all KV heads of a token side by side, so the workgroups of one
     // (row, chunk) -- one per KV head -- fetch the same cache lines: they are numbered so that they
@@ -103,13 +150,59 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     const int chunk = pair % (a.chunks + 1), row = pair / (a.chunks + 1);
     if (row >= a.batch) return;                          // padding of the last group of eight pairs
     const bool is_hot = chunk == a.chunks;
-    int slot = a.slot_ids[row];
-    slot = slot < 0 ? 0 : (slot >= a.slots ? a.slots - 1 : slot);
-    const int page_count = a.page_counts[slot], last_len = a.last_page_lens[slot], hot_len = a.hot_lengths[slot];
-    const bool live = a.active_mask[row] && (!a.cache_active || a.cache_active[slot]);
     const int first_page = chunk * kAttnPagesPerChunk;
     const int64_t part = ((int64_t)row * a.q_heads + (int64_t)g * G) * (a.chunks + 1) + chunk;   // + h * (chunks + 1)
 
+    // lane role inside a pass
+    const int pass_page = tid / kTokenBlocks, token = (tid % kTokenBlocks) / kBlocks, blk = tid % kBlocks;
+    const int row_in_page = token * a.kv_heads + g;
+    const int64_t page_words = (int64_t)P * a.kv_heads * kBlocks, page_rows = (int64_t)P * a.kv_heads;
+
+    // ---- round 1: slot, activity, queries ------------------------------------------------------
+    int slot = a.slot_ids[row];
+    const bool row_active = a.active_mask[row] != 0;
+    // lane 8 h + piece of the first wavefront holds elements 8 piece .. 8 piece + 7 of head h
+    const int qh = tid >> 3, piece = tid & 7;
+    float qv[8], rope_c[8], rope_s[8];
+    if (tid < G * 8) {
+        const int64_t at = ((int64_t)row * a.q_heads + g * G + qh) * D + piece * 8;
+        if (a.query_dtype == NQ_BF16) {
+            const uint4 raw = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.query) + at);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                qv[2 * j] = __uint_as_float(w[j] << 16);
+                qv[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) qv[j] = load_query(a.query, a.query_dtype, at + j);
+        }
+        if (a.rope_cos) {
+            const int64_t rope_at = (int64_t)row * D + piece * 8;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                rope_c[j] = bf16_to_f32(a.rope_cos[rope_at + j]);
+                rope_s[j] = bf16_to_f32(a.rope_sin[rope_at + j]);
+            }
+        }
+    }
+    // beta tables in registers: a table lookup from memory would sit behind every decode
+    const float key_beta[4] = {a.key_betas[0], a.key_betas[1], a.key_betas[2], a.key_betas[3]};
+    const float value_beta[4] = {a.value_betas[0], a.value_betas[1], a.value_betas[2], a.value_betas[3]};
+
+    // ---- round 2: lengths and page ids of the slot ------------------------------------------------
+    slot = slot < 0 ? 0 : (slot >= a.slots ? a.slots - 1 : slot);
+    const int page_count = a.page_counts[slot], last_len = a.last_page_lens[slot], hot_len = a.hot_lengths[slot];
+    const bool cache_live = !a.cache_active || a.cache_active[slot];
+    int64_t pass_pageid[kPasses];
+#pragma unroll
+    for (int pass = 0; pass < kPasses; pass++) {
+        const int ordinal = first_page + pass * kPagesPerPass + pass_page;
+        pass_pageid[pass] = (!is_hot && ordinal < a.max_pages) ? a.page_indices[(int64_t)slot * a.max_pages + ordinal] : 0;
+    }
+    NQ_STAMP(1);
+    const bool live = row_active && cache_live;
     const bool empty = !live || (is_hot ? hot_len <= 0 : first_page >= page_count);
     if (empty) {                                         // uniform over the workgroup
         if (tid < G) {
@@ -119,66 +212,54 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
         return;
     }
 
-    // beta tables in registers: a table lookup from memory would sit behind every decode
-    const float key_beta[4] = {a.key_betas[0], a.key_betas[1], a.key_betas[2], a.key_betas[3]};
-    const float value_beta[4] = {a.value_betas[0], a.value_betas[1], a.value_betas[2], a.value_betas[3]};
-
-    // lane role inside a pass
-    const int pass_page = tid / kTokenBlocks, token = (tid % kTokenBlocks) / kBlocks, blk = tid % kBlocks;
-    const int row_in_page = token * a.kv_heads + g;
-    const int64_t page_words = (int64_t)P * a.kv_heads * kBlocks, page_rows = (int64_t)P * a.kv_heads;
-
-    // Which (page, token) this lane serves in every pass, and the packed key operands of all
-    // passes, requested together so that a chunk pays one memory round trip, not one per pass.
+    // ---- round 3: the packed operands of all passes, keys and values -----------------------------------
     bool pass_valid[kPasses];
-    int64_t pass_word[kPasses], pass_norm[kPasses];
-    uint32_t k_code[kPasses], k_ids[kPasses];
-    float k_norm[kPasses];
+    uint32_t k_code[kPasses], k_ids[kPasses], v_code[kPasses], v_ids[kPasses];
+    float k_norm[kPasses], v_norm[kPasses];
+    uint4 hot_k = make_uint4(0, 0, 0, 0), hot_v = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int pass = 0; pass < kPasses; pass++) {
         const int ordinal = first_page + pass * kPagesPerPass + pass_page;
         pass_valid[pass] = is_hot ? (pass == 0 && pass_page == 0 && token < hot_len)
                                   : (ordinal < page_count && (ordinal < page_count - 1 || token < last_len));
-        pass_word[pass] = 0;
-        pass_norm[pass] = 0;
         k_code[pass] = 0u; k_ids[pass] = 0u; k_norm[pass] = 0.0f;
+        v_code[pass] = 0u; v_ids[pass] = 0u; v_norm[pass] = 0.0f;
         if (!is_hot && pass_valid[pass]) {
-            const int64_t page = a.page_indices[(int64_t)slot * a.max_pages + ordinal];
-            pass_word[pass] = page * page_words + (int64_t)row_in_page * kBlocks + blk;
-            pass_norm[pass] = page * page_rows + row_in_page;
-            k_code[pass] = a.key_codes[pass_word[pass]];
-            k_ids[pass] = a.key_beta_ids[pass_word[pass] >> 2];
-            k_norm[pass] = a.key_norms[pass_norm[pass]];
+            const int64_t word = pass_pageid[pass] * page_words + (int64_t)row_in_page * kBlocks + blk;
+            const int64_t norm = pass_pageid[pass] * page_rows + row_in_page;
+            k_code[pass] = a.key_codes[word];
+            k_ids[pass] = a.key_beta_ids[word >> 2];
+            k_norm[pass] = a.key_norms[norm];
+            v_code[pass] = a.value_codes[word];
+            v_ids[pass] = a.value_beta_ids[word >> 2];
+            v_norm[pass] = a.value_norms[norm];
         }
     }
-    // the group's queries, optionally Hadamard-rotated here (float32 butterflies over the head,
-    // scaled by 1 / sqrt(D), rounded to the query dtype: hadamard(query.float()).to(dtype),
+    if (is_hot && pass_valid[0]) {
+        const int64_t at = (((int64_t)slot * P + token) * a.kv_heads + g) * D + blk * 8;
+        hot_k = *reinterpret_cast<const uint4 *>(a.hot_keys + at);
+        hot_v = *reinterpret_cast<const uint4 *>(a.hot_values + at);
+    }
+
+    // the group's queries: rotary embedding ((q * cos) + (rotate_half(q) * sin) in BF16 tensor
+    // arithmetic), then optionally the Hadamard rotation (float32 butterflies over the head, scaled
+    // by 1 / sqrt(D), rounded to the query dtype: hadamard(query.float()).to(dtype),
     // nestquant/runtime/nqkv_batched_hf_backend.py:549)
-    static_assert(sizeof(acc_lds) >= sizeof(float) * G * D, "the query staging fits the accumulator buffer");
-    static_assert(D == 64 && G * 8 <= 64, "eight lanes of the first wavefront prepare one head's query");
     float *q_lds = &acc_lds[0][0][0];                    // free until the V pass ends
+    static_assert(sizeof(acc_lds) >= sizeof(float) * G * D, "the query staging fits the accumulator buffer");
     if (tid < G * 8) {
-        // lane 8 h + part holds elements 8 part .. 8 part + 7 of head h: the embedding pairs it with
-        // the lane four further on, the rotation runs in registers and between the eight lanes
-        const int h = tid >> 3, part = tid & 7;
-        float v[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++)
-            v[j] = load_query(a.query, a.query_dtype, ((int64_t)row * a.q_heads + g * G + h) * D + part * 8 + j);
         if (a.rope_cos) {
-            // (q * cos) + (rotate_half(q) * sin) in BF16 tensor arithmetic, before the rotation
-            const int64_t at = (int64_t)row * D + part * 8;
-            const bool upper = part >= 4;
+            const bool upper = piece >= 4;
 #pragma unroll
             for (int j = 0; j < 8; j += 2) {
-                const float o0 = lane_xor<4>(v[j]), o1 = lane_xor<4>(v[j + 1]);
-                float a0 = v[j] * bf16_to_f32(a.rope_cos[at + j]), a1 = v[j + 1] * bf16_to_f32(a.rope_cos[at + j + 1]);
+                const float o0 = lane_xor<4>(qv[j]), o1 = lane_xor<4>(qv[j + 1]);
+                float a0 = qv[j] * rope_c[j], a1 = qv[j + 1] * rope_c[j + 1];
                 round_pair<1>(a0, a1);
-                float b0 = o0 * bf16_to_f32(a.rope_sin[at + j]), b1 = o1 * bf16_to_f32(a.rope_sin[at + j + 1]);
+                float b0 = o0 * rope_s[j], b1 = o1 * rope_s[j + 1];
                 round_pair<1>(b0, b1);
-                v[j] = upper ? a0 + b0 : a0 - b0;
-                v[j + 1] = upper ? a1 + b1 : a1 - b1;
-                round_pair<1>(v[j], v[j + 1]);
+                qv[j] = upper ? a0 + b0 : a0 - b0;
+                qv[j + 1] = upper ? a1 + b1 : a1 - b1;
+                round_pair<1>(qv[j], qv[j + 1]);
             }
         }
         if (a.rotate_query) {
@@ -187,35 +268,36 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
                     if (j & (1 << s)) continue;
-                    const float left = v[j], right = v[j + (1 << s)];
-                    v[j] = left + right;
-                    v[j + (1 << s)] = left - right;
+                    const float left = qv[j], right = qv[j + (1 << s)];
+                    qv[j] = left + right;
+                    qv[j + (1 << s)] = left - right;
                 }
             }
-            lane_stage<1, 0>(v, tid);
-            lane_stage<2, 0>(v, tid);
-            lane_stage<4, 0>(v, tid);
+            lane_stage<1, 0>(qv, tid);
+            lane_stage<2, 0>(qv, tid);
+            lane_stage<4, 0>(qv, tid);
             const float inv = 1.0f / __builtin_sqrtf((float)D);
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                const float scaled = v[j] * inv;
-                v[j] = a.query_dtype == NQ_BF16 ? bf16_to_f32(f32_to_bf16(scaled))
-                                                : (a.query_dtype == NQ_F16 ? (float)(_Float16)scaled : scaled);
+                const float scaled = qv[j] * inv;
+                qv[j] = a.query_dtype == NQ_BF16 ? bf16_to_f32(f32_to_bf16(scaled))
+                                                 : (a.query_dtype == NQ_F16 ? (float)(_Float16)scaled : scaled);
             }
         }
 #pragma unroll
-        for (int j = 0; j < 8; j++) q_lds[h * D + part * 8 + j] = v[j];
+        for (int j = 0; j < 8; j++) q_lds[qh * D + piece * 8 + j] = qv[j];
     }
     __syncthreads();
+    NQ_STAMP(2);
     float q[G][8];
 #pragma unroll
     for (int h = 0; h < G; h++)
 #pragma unroll
         for (int j = 0; j < 8; j++) q[h][j] = q_lds[h * D + blk * 8 + j];
-    __syncthreads();
     const float sqrt_d = __builtin_sqrtf((float)D);
 
     // ---- K pass -----------------------------------------------------------------------------
+    NQ_STAMP(3);
 #pragma unroll
     for (int pass = 0; pass < kPasses; pass++) {
         const int page_in_chunk = pass * kPagesPerPass + pass_page;
@@ -224,15 +306,11 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
 #pragma unroll
         for (int j = 0; j < 8; j++) k[j] = 0.0f;
         if (is_hot) {
-            if (valid) {
-                const uint4 raw = *reinterpret_cast<const uint4 *>(
-                    a.hot_keys + (((int64_t)slot * P + token) * a.kv_heads + g) * D + blk * 8);
-                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+            const uint32_t w[4] = {hot_k.x, hot_k.y, hot_k.z, hot_k.w};
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    k[2 * j] = __uint_as_float(w[j] << 16);
-                    k[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
-                }
+            for (int j = 0; j < 4; j++) {
+                k[2 * j] = __uint_as_float(w[j] << 16);
+                k[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
             }
         } else if (valid) {
             decode_codeword<false>(k_code[pass], 14.0f, 0u, k);
@@ -251,56 +329,26 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
             if (blk == 0) scores[h][page_in_chunk * P + token] = valid ? s * a.scale : -INFINITY;
         }
     }
-    // the packed value operands of all passes, in flight during the softmax
-    uint32_t v_code[kPasses], v_ids[kPasses];
-    float v_norm[kPasses];
-#pragma unroll
-    for (int pass = 0; pass < kPasses; pass++) {
-        v_code[pass] = 0u; v_ids[pass] = 0u; v_norm[pass] = 0.0f;
-        if (!is_hot && pass_valid[pass]) {
-            v_code[pass] = a.value_codes[pass_word[pass]];
-            v_ids[pass] = a.value_beta_ids[pass_word[pass] >> 2];
-            v_norm[pass] = a.value_norms[pass_norm[pass]];
-        }
-    }
-    __syncthreads();
+    __syncthreads();                                     // scores complete; the queries in acc_lds are no longer needed
+    NQ_STAMP(4);
 
-    // ---- softmax over the chunk (one score per lane and head) -----------------------------------
-    static_assert(kChunkTokens <= kAttnThreads, "at most one token per lane in the softmax phase");
-    float mine[G];
+    // ---- softmax over the chunk: every wavefront works out the maximum and the denominator for
+    // itself (no hand-over between wavefronts), every lane the weights of its own tokens -------------
+    float chunk_max[G], chunk_sum[G];
 #pragma unroll
     for (int h = 0; h < G; h++) {
-        mine[h] = tid < kChunkTokens ? scores[h][tid] : -INFINITY;
-        float m = mine[h];
+        float m = -INFINITY;
 #pragma unroll
-        for (int offset = 32; offset >= 1; offset >>= 1) m = fmaxf(m, __shfl_xor(m, offset, 64));
-        if ((tid & 63) == 0) reduce_buf[tid >> 6][h] = m;
-    }
-    __syncthreads();
-    if (tid < G) {
-        float m = reduce_buf[0][tid];
-        for (int w = 1; w < kAttnThreads / 64; w++) m = fmaxf(m, reduce_buf[w][tid]);
-        chunk_max[tid] = m;
-    }
-    __syncthreads();
+        for (int t = 0; t < kChunkTokens / 64; t++) m = fmaxf(m, scores[h][(tid & 63) + 64 * t]);
+        chunk_max[h] = wave_max(m);                      // finite: the chunk holds at least one token
+        float s = 0.0f;
 #pragma unroll
-    for (int h = 0; h < G; h++) {
-        const float p = mine[h] == -INFINITY ? 0.0f : __expf(mine[h] - chunk_max[h]);
-        if (tid < kChunkTokens) scores[h][tid] = p;
-        float s = p;
-#pragma unroll
-        for (int offset = 32; offset >= 1; offset >>= 1) s = s + __shfl_xor(s, offset, 64);
-        if ((tid & 63) == 0) reduce_buf[tid >> 6][h] = s;
+        for (int t = 0; t < kChunkTokens / 64; t++) s = s + __expf(scores[h][(tid & 63) + 64 * t] - chunk_max[h]);
+        chunk_sum[h] = wave_sum(s);
     }
-    __syncthreads();
-    if (tid < G) {
-        float s = reduce_buf[0][tid];
-        for (int w = 1; w < kAttnThreads / 64; w++) s = s + reduce_buf[w][tid];
-        chunk_sum[tid] = s;
-    }
-    // (scores now hold probabilities; the barrier above ordered their writes)
 
     // ---- V pass ------------------------------------------------------------------------------
+    NQ_STAMP(5);
     float acc[G][8];
 #pragma unroll
     for (int h = 0; h < G; h++)
@@ -311,16 +359,14 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
         const int page_in_chunk = pass * kPagesPerPass + pass_page;
         const bool valid = pass_valid[pass];
         float v[8];
-        if (is_hot) {
-            if (valid) {
-                const uint4 raw = *reinterpret_cast<const uint4 *>(
-                    a.hot_values + (((int64_t)slot * P + token) * a.kv_heads + g) * D + blk * 8);
-                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    v[2 * j] = __uint_as_float(w[j] << 16);
-                    v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
-                }
+        for (int j = 0; j < 8; j++) v[j] = 0.0f;
+        if (is_hot) {
+            const uint32_t w[4] = {hot_v.x, hot_v.y, hot_v.z, hot_v.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                v[2 * j] = __uint_as_float(w[j] << 16);
+                v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
             }
         } else if (valid) {
             decode_codeword<false>(v_code[pass], 14.0f, 0u, v);
@@ -329,39 +375,43 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
 #pragma unroll
             for (int j = 0; j < 8; j++) v[j] = (v[j] * beta) * back;
         }
-        if (valid) {
 #pragma unroll
-            for (int h = 0; h < G; h++) {
-                const float p = scores[h][page_in_chunk * P + token];
+        for (int h = 0; h < G; h++) {
+            // exp(-inf - max) = 0 for a token that does not exist
+            const float p = __expf(scores[h][page_in_chunk * P + token] - chunk_max[h]);
 #pragma unroll
-                for (int j = 0; j < 8; j++) acc[h][j] = __builtin_fmaf(p, v[j], acc[h][j]);
-            }
+            for (int j = 0; j < 8; j++) acc[h][j] = __builtin_fmaf(p, v[j], acc[h][j]);
         }
     }
-    // lanes that share a block index hold partial sums of the same 8 output dims: the two
-    // tokens of a 16-lane row are folded with a register exchange, rows through LDS in order
-    static_assert(kBlocks == 8, "lane bits 0..2 index the block");
+    NQ_STAMP(6);
+    // lanes that share a block index hold partial sums of the same 8 output dims: folded inside the
+    // wavefront with register exchanges (the two tokens of a 16-lane row, then the four rows),
+    // wavefronts through LDS in order
 #pragma unroll
     for (int h = 0; h < G; h++)
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const float v = acc[h][j] + dpp_rotate8(acc[h][j]);
-            // column swizzled by (block, row): the 32 lanes of a wavefront that store one (h, j) hit 32
-            // banks (unswizzled they all met in one: blocks lie G * 32 bytes apart, rows G * 256)
-            if ((tid & 8) == 0) acc_lds[tid >> 4][tid & 7][(h * 8 + j) ^ acc_swizzle(tid & 7, tid >> 4)] = v;
+            const float v = fold_rows(acc[h][j] + dpp_rotate8(acc[h][j]));
+            if ((tid & 63) < 8) acc_lds[tid >> 6][h * 8 + j][tid & 7] = v;
         }
     __syncthreads();
     for (int o = tid; o < G * D; o += kAttnThreads) {
         const int h = o / D, d = o % D;
-        float total = acc_lds[0][d / 8][(h * 8 + d % 8) ^ acc_swizzle(d / 8, 0)];
+        float total = acc_lds[0][h * 8 + d % 8][d / 8];
 #pragma unroll
-        for (int w = 1; w < kAttnThreads / 16; w++) total = total + acc_lds[w][d / 8][(h * 8 + d % 8) ^ acc_swizzle(d / 8, w)];
+        for (int w = 1; w < kWaves; w++) total = total + acc_lds[w][h * 8 + d % 8][d / 8];
         a.part_acc[(part + (int64_t)h * (a.chunks + 1)) * D + d] = total;
     }
     if (tid < G) {
-        a.part_max[part + (int64_t)tid * (a.chunks + 1)] = chunk_max[tid];
-        a.part_sum[part + (int64_t)tid * (a.chunks + 1)] = chunk_sum[tid];
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            if (tid == h) {
+                a.part_max[part + (int64_t)h * (a.chunks + 1)] = chunk_max[h];
+                a.part_sum[part + (int64_t)h * (a.chunks + 1)] = chunk_sum[h];
+            }
+        }
     }
+    NQ_STAMP(7);
 }
 
 // Stage 2, one wavefront per (row, head): out[d] = sum_c acc_c[d] w_c / sum_c sum_c w_c with

@@ -1,7 +1,7 @@
 // E8 codec kernels: nearest point, row quantiser with multi-beta selection (NQA4 / NQKV4
 // encoder) and its inverse.  Reference: nestquant/core/quantizer.py:214-301, 39-51;
 // nestquant/runtime/nqkv_page.py:97-185, 332-372, 446-456, 22-95; nestquant/runtime/cuda_e8.cu:8-59.
-#define NQ_PHASE_STAMP_UNIT
+#define NQ_PHASE_STAMP_ARRAY g_phase_stamps
 #include "nq_rowquant.hip.h"
 #include "nq_host.h"
 

@@ -12,13 +12,13 @@
 
 #include "nq_e8.hip.h"
 
-// Phase stamps of the row encoder (a measuring build only, -DNQ_PHASE_STAMPS, and only in the
-// translation unit that asks for them with NQ_PHASE_STAMP_UNIT): lane 0 of workgroup 0 writes the
-// 100 MHz wall clock at the phase boundaries into a device array that nq_debug_phase_stamps
-// copies out.  Otherwise the macro is empty.
-#if defined(NQ_PHASE_STAMPS) && defined(NQ_PHASE_STAMP_UNIT)
-namespace nq { __device__ unsigned long long g_phase_stamps[16]; }
-#define NQ_STAMP(i) do { if (blockIdx.x == 0 && threadIdx.x == 0) nq::g_phase_stamps[i] = wall_clock64(); } while (0)
+// Phase stamps (a measuring build only, -DNQ_PHASE_STAMPS, and only in a translation unit that
+// names its stamp array with NQ_PHASE_STAMP_ARRAY before this header): lane 0 of workgroup 0 writes
+// the 100 MHz wall clock at the phase boundaries into that device array, which the unit's
+// nq_debug_*_stamps call copies out.  Otherwise the macro is empty.
+#if defined(NQ_PHASE_STAMPS) && defined(NQ_PHASE_STAMP_ARRAY)
+namespace nq { __device__ unsigned long long NQ_PHASE_STAMP_ARRAY[16]; }
+#define NQ_STAMP(i) do { if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) nq::NQ_PHASE_STAMP_ARRAY[i] = wall_clock64(); } while (0)
 #else
 #define NQ_STAMP(i) do { } while (0)
 #endif
