@@ -287,13 +287,18 @@ int nq_w4a4_decode_weight(const uint8_t *w_codes_dev, const uint8_t *w_beta_ids_
  * row-major BF16 (16-byte aligned), FP32 accumulation, c [M, N] BF16.  K a multiple of 128.
  * tile = -1 lets the library choose the workgroup tile from the shape; 0..6 force
  * 256x256, 128x256, 256x128, 128x128, 64x128, 128x64, 64x64 (for measurements).
+ * A product with few tiles (a few hundred rows) is split along K into 2, 4 or 8 slabs whose
+ * float32 partial results meet in a second launch: split_k = 0 lets the library decide, 1 forbids
+ * it, 2 / 4 / 8 force it (K a multiple of 128 split_k).  The partial results need
+ * split_k * M * N * 4 bytes of workspace (16-byte aligned); without a workspace nothing is split.
  * nq_w4a4_gemm calls it on the weight it has decoded once when M is large; it is exported for
  * callers that keep a decoded weight themselves.
  * Replaces: the multiply of run_large_m_staged for long prefills,
  * nestquant/runtime/nqrt4_w4a4_mma.cu:606-667 (which decodes inside the multiply).
  */
 int nq_bf16_gemm(const void *a_bf16_dev, const void *b_bf16_dev, int64_t m, int64_t n, int64_t k,
-                 void *c_bf16_dev, int tile, void *stream);
+                 void *c_bf16_dev, int tile, int split_k, void *workspace_dev, size_t workspace_bytes,
+                 void *stream);
 
 /*
  * NQKV cache, device-resident state.  Per slot (int32[slots]): sequence_lengths,

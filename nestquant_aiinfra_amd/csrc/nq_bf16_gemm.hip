@@ -17,7 +17,7 @@
 // Replaces (together with nq_w4a4_decode_weight): run_large_m_staged and the chunk-and-pad wrapper for
 // M beyond a few hundred rows, nestquant/runtime/nqrt4_w4a4_mma.cu:606-667 and
 // nestquant/runtime/cuda_w4a4_mma.py:450-474.
-#include "nq_host.h"
+#include "nq_linear_common.hip.h"
 
 #include <stdint.h>
 
@@ -39,7 +39,8 @@ __device__ __forceinline__ uint16_t dense_f32_to_bf16(float x) {
 template <int WM, int WN, int GM, int GN>
 __global__ void __launch_bounds__(64 * GM * GN)
 bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b, uint16_t *__restrict__ c,
-                 int m_size, int n_size, int k_size, int tiles_m, int tiles_n, int group_m) {
+                 int m_size, int n_size, int k_size, int tiles_m, int tiles_n, int group_m, int k_slab,
+                 float *__restrict__ partials) {
     constexpr int kThreads = 64 * GM * GN;
     constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN;
     constexpr int kRowsPerPass = kThreads / 8;                     // rows one pass of 16-byte loads covers
@@ -61,6 +62,10 @@ bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b,
     const int tile_m = first_m + in_group % rows_in_group, tile_n = in_group / rows_in_group;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
+    // with a K split, workgroup row blockIdx.y multiplies the K range [k_begin, k_begin + k_slab) and
+    // leaves a float32 partial result
+    const int k_begin = blockIdx.y * k_slab;
+
     // global -> LDS role: piece (tid & 7) of rows (tid >> 3) + kRowsPerPass i
     const int load_row = tid >> 3, load_piece = tid & 7;
     const int store_slot = load_row * 8 + (load_piece ^ ((load_row >> 1) & 7));
@@ -68,12 +73,12 @@ bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b,
 #pragma unroll
     for (int i = 0; i < kLoadsA; i++) {
         const int row = m0 + load_row + kRowsPerPass * i;
-        a_offset[i] = (row < m_size ? row : m_size - 1) * k_size + load_piece * 8;
+        a_offset[i] = (row < m_size ? row : m_size - 1) * k_size + k_begin + load_piece * 8;
     }
 #pragma unroll
     for (int i = 0; i < kLoadsB; i++) {
         const int row = n0 + load_row + kRowsPerPass * i;
-        b_offset[i] = (row < n_size ? row : n_size - 1) * k_size + load_piece * 8;
+        b_offset[i] = (row < n_size ? row : n_size - 1) * k_size + k_begin + load_piece * 8;
     }
 
     // fragment role: A rows wave_m * 32 WM + 32 i + lane % 32, B rows likewise; piece 2 s + lane / 32
@@ -93,7 +98,7 @@ bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b,
     // stored to LDS at the end of step s), registers `late` receive slab s + 2 at the top of step s.
     // A step of 64 k lasts about as long as a trip to the L2 and back under load, so one step of
     // lead leaves the matrix cores waiting for the stores.
-    const int steps = k_size / kDenseBK;
+    const int steps = k_slab / kDenseBK;
     u32x4 pa0[kLoadsA], pa1[kLoadsA], pb0[kLoadsB], pb1[kLoadsB];
     {
         u32x4 ra[kLoadsA], rb[kLoadsB];
@@ -170,7 +175,10 @@ bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b,
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int row = row_base + (r & 3) + 8 * (r >> 2);
-                    if (row < m_size) c[(int64_t)row * n_size + col] = dense_f32_to_bf16(acc[i][j][r]);
+                    if (row < m_size) {
+                        if (partials) partials[((int64_t)blockIdx.y * m_size + row) * n_size + col] = acc[i][j][r];
+                        else c[(int64_t)row * n_size + col] = dense_f32_to_bf16(acc[i][j][r]);
+                    }
                 }
             }
         }
@@ -192,7 +200,8 @@ const DenseTile kDenseTiles[] = {
 };
 
 template <int WM, int WN, int GM, int GN>
-void launch_dense(const void *a, const void *b, void *c, int m, int n, int k, hipStream_t stream) {
+void launch_dense(const void *a, const void *b, void *c, int m, int n, int k, int split, float *partials,
+                  hipStream_t stream) {
     constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN;
     const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     const size_t lds_bytes = (size_t)2 * (BM + BN) * 128;
@@ -203,45 +212,70 @@ void launch_dense(const void *a, const void *b, void *c, int m, int n, int k, hi
         raised = true;
     }
     const int group_m = tiles_m < 4 ? tiles_m : 4;
-    hipLaunchKernelGGL((nq::bf16_gemm_kernel<WM, WN, GM, GN>), dim3((unsigned)(tiles_m * tiles_n)), dim3(64 * GM * GN),
-                       lds_bytes, stream, reinterpret_cast<const uint16_t *>(a), reinterpret_cast<const uint16_t *>(b),
-                       reinterpret_cast<uint16_t *>(c), m, n, k, tiles_m, tiles_n, group_m);
+    hipLaunchKernelGGL((nq::bf16_gemm_kernel<WM, WN, GM, GN>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)split),
+                       dim3(64 * GM * GN), lds_bytes, stream, reinterpret_cast<const uint16_t *>(a),
+                       reinterpret_cast<const uint16_t *>(b), reinterpret_cast<uint16_t *>(c), m, n, k, tiles_m, tiles_n,
+                       group_m, k / split, split > 1 ? partials : nullptr);
 }
 
 }  // namespace
 
 namespace nq {
 
-// Shared with nq_w4a4_gemm: picks the tile shape with the least estimated time and launches.
-int launch_bf16_gemm(const void *a, const void *b, void *c, int m, int n, int k, int forced_tile, hipStream_t stream) {
+// K split of a product whose tiles would leave most of the chip idle: 1 (none), 2, 4 or 8 slabs of
+// at least 2048 k, as long as the 128 x 128 tiles times the slabs stay within one per compute unit,
+// within a partial-result buffer of `partial_bytes`.  (Measured at 384 rows: K = 8192, N = 2048 runs
+// in 29 us with four slabs against 42 us without; at K = 2048, N = 8192 the partial results cost
+// more than the idle units, 35 against 27 us.)
+int dense_split_for(int m, int n, int k, size_t partial_bytes) {
+    const int64_t tiles = (int64_t)((m + 127) / 128) * ((n + 127) / 128);
+    int split = 1;
+    while (split < 8 && tiles * split * 2 <= 256 && k / (split * 2) >= 2048 && k % (split * 2 * 128) == 0 &&
+           (size_t)(split * 2) * m * n * sizeof(float) <= partial_bytes)
+        split *= 2;
+    return split;
+}
+
+// Shared with nq_w4a4_gemm: picks the tile shape with the least estimated time (and, given a buffer
+// for partial results, a K split) and launches.
+int launch_bf16_gemm(const void *a, const void *b, void *c, int m, int n, int k, int forced_tile, int forced_split,
+                     void *partials, size_t partial_bytes, hipStream_t stream) {
+    int split = forced_split > 0 ? forced_split : dense_split_for(m, n, k, partials ? partial_bytes : 0);
+    if (split > 1 && (k % (split * 128) != 0 || !partials || (size_t)split * m * n * sizeof(float) > partial_bytes))
+        return fail(NQ_ERR_WORKSPACE, "nq_bf16_gemm: a K split of %d needs K a multiple of %d and %zu bytes for partial results",
+                    split, split * 128, (size_t)split * m * n * sizeof(float));
     int best = 0;
     float best_cost = 0.0f;
     const int count = (int)(sizeof(kDenseTiles) / sizeof(kDenseTiles[0]));
     for (int t = 0; t < count; t++) {
         const DenseTile &tile = kDenseTiles[t];
-        const int64_t tiles = (int64_t)((m + tile.bm - 1) / tile.bm) * ((n + tile.bn - 1) / tile.bn);
+        const int64_t tiles = (int64_t)((m + tile.bm - 1) / tile.bm) * ((n + tile.bn - 1) / tile.bn) * split;
         // the busiest of the 256 compute units works through ceil(tiles / 256) tiles, whether one
         // after the other or side by side at a share of its rate
         const float cost = (float)((tiles + 255) / 256) * (float)(tile.bm * tile.bn) / tile.efficiency;
         if (t == 0 || cost < best_cost) { best = t; best_cost = cost; }
     }
     if (forced_tile >= 0 && forced_tile < count) best = forced_tile;
+    float *p = reinterpret_cast<float *>(partials);
     switch (best) {
-        case 0: launch_dense<2, 4, 4, 2>(a, b, c, m, n, k, stream); break;
-        case 1: launch_dense<2, 4, 2, 2>(a, b, c, m, n, k, stream); break;
-        case 2: launch_dense<4, 2, 2, 2>(a, b, c, m, n, k, stream); break;
-        case 3: launch_dense<2, 2, 2, 2>(a, b, c, m, n, k, stream); break;
-        case 4: launch_dense<1, 2, 2, 2>(a, b, c, m, n, k, stream); break;
-        case 5: launch_dense<2, 1, 2, 2>(a, b, c, m, n, k, stream); break;
-        default: launch_dense<1, 1, 2, 2>(a, b, c, m, n, k, stream); break;
+        case 0: launch_dense<2, 4, 4, 2>(a, b, c, m, n, k, split, p, stream); break;
+        case 1: launch_dense<2, 4, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
+        case 2: launch_dense<4, 2, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
+        case 3: launch_dense<2, 2, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
+        case 4: launch_dense<1, 2, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
+        case 5: launch_dense<2, 1, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
+        default: launch_dense<1, 1, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
     }
-    return check_launch("nq_bf16_gemm");
+    const int status = check_launch("nq_bf16_gemm");
+    if (status != NQ_OK || split == 1) return status;
+    return launch_splitk_reduce(p, split, (int64_t)m * n, c, NQ_BF16, stream);
 }
 
 }  // namespace nq
 
 extern "C" int nq_bf16_gemm(const void *a_bf16_dev, const void *b_bf16_dev, int64_t m, int64_t n, int64_t k,
-                            void *c_bf16_dev, int tile, void *stream) {
+                            void *c_bf16_dev, int tile, int split_k, void *workspace_dev, size_t workspace_bytes,
+                            void *stream) {
     NQ_REQUIRE(m >= 1 && n >= 1 && m < ((int64_t)1 << 30) && n < ((int64_t)1 << 30), NQ_ERR_SHAPE,
                "nq_bf16_gemm: M and N must be positive");
     NQ_REQUIRE(k >= 2 * nq::kDenseBK && k % (2 * nq::kDenseBK) == 0 && k < ((int64_t)1 << 30), NQ_ERR_SHAPE,
@@ -252,5 +286,9 @@ extern "C" int nq_bf16_gemm(const void *a_bf16_dev, const void *b_bf16_dev, int6
     NQ_REQUIRE(m * k < ((int64_t)1 << 31) && n * k < ((int64_t)1 << 31), NQ_ERR_SHAPE,
                "nq_bf16_gemm: operands of 2^31 elements or more are not supported");
     NQ_REQUIRE(tile >= -1 && tile <= 6, NQ_ERR_ARGUMENT, "nq_bf16_gemm: tile must be -1 (automatic) or 0..6");
-    return nq::launch_bf16_gemm(a_bf16_dev, b_bf16_dev, c_bf16_dev, (int)m, (int)n, (int)k, tile, (hipStream_t)stream);
+    NQ_REQUIRE(split_k == 0 || split_k == 1 || split_k == 2 || split_k == 4 || split_k == 8, NQ_ERR_ARGUMENT,
+               "nq_bf16_gemm: split_k must be 0 (automatic), 1, 2, 4 or 8");
+    NQ_REQUIRE(!workspace_dev || nq::aligned(workspace_dev, 16), NQ_ERR_ARGUMENT, "nq_bf16_gemm: workspace must be 16-byte aligned");
+    return nq::launch_bf16_gemm(a_bf16_dev, b_bf16_dev, c_bf16_dev, (int)m, (int)n, (int)k, tile, split_k, workspace_dev,
+                                workspace_dev ? workspace_bytes : 0, (hipStream_t)stream);
 }

@@ -198,7 +198,9 @@ decode_weight_kernel(const uint32_t *__restrict__ w_words, const uint16_t *__res
 }  // namespace nq
 
 namespace nq {
-int launch_bf16_gemm(const void *a, const void *b, void *c, int m, int n, int k, int forced_tile, hipStream_t stream);
+int dense_split_for(int m, int n, int k, size_t partial_bytes);
+int launch_bf16_gemm(const void *a, const void *b, void *c, int m, int n, int k, int forced_tile, int forced_split,
+                     void *partials, size_t partial_bytes, hipStream_t stream);
 }
 
 namespace {
@@ -231,7 +233,12 @@ extern "C" size_t nq_w4a4_gemm_workspace_bytes(int m, int k, int n, int split_k,
     // fused kernel's partial sums (FP32 output) alike
     const int chunk = m < kChunkRows ? m : kChunkRows;
     const size_t partials = split > 1 ? (size_t)split * (size_t)chunk * (size_t)n * sizeof(float) : 0;
-    const size_t scratch = decodes_once(m, k, split_k) ? nq::align256((size_t)n * k * 2) : 0;
+    // decode-once: the BF16 weight, then the partial results of the dense product's own K split
+    size_t scratch = 0;
+    if (decodes_once(m, k, split_k)) {
+        const int dense_split = nq::dense_split_for(m, n, k, ~(size_t)0);
+        scratch = nq::align256((size_t)n * k * 2) + (dense_split > 1 ? (size_t)dense_split * m * n * sizeof(float) : 0);
+    }
     return bytes + (scratch > partials ? scratch : partials);
 }
 
@@ -293,7 +300,10 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
                                                  w_norms_dev, w_betas_dev, n, k, weight_offset, weight_seed, weight_bf16,
                                                  stream);
         if (status != NQ_OK) return status;
-        return nq::launch_bf16_gemm(act, weight_bf16, out_dev, m, n, k, -1, s);
+        char *dense_partials = reinterpret_cast<char *>(weight_bf16) + nq::align256((size_t)n * k * 2);
+        const size_t used = (size_t)(dense_partials - reinterpret_cast<char *>(workspace_dev));
+        return nq::launch_bf16_gemm(act, weight_bf16, out_dev, m, n, k, -1, 0, dense_partials,
+                                    workspace_bytes > used ? workspace_bytes - used : 0, s);
     }
     const uint32_t seed_plus_offset = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
     const float sqrt_k = (float)sqrt((double)k);

@@ -635,17 +635,22 @@ def _gemm(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *,
     return _gemv(activation, weight, split_k=split_k, output_dtype=dtype, kernel="gemm")
 
 
-def bf16_gemm(rows: torch.Tensor, weight: torch.Tensor, *, tile: int = -1) -> torch.Tensor:
+def bf16_gemm(rows: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split_k: int = 0) -> torch.Tensor:
     """`rows @ weight.T` for BF16 [M, K] and [N, K] (K a multiple of 128) on the library's dense
-    matrix-core GEMM, FP32 accumulation, BF16 out.  `tile` forces a workgroup tile (measurements)."""
+    matrix-core GEMM, FP32 accumulation, BF16 out.  `tile` forces a workgroup tile and `split_k` a K
+    split (measurements); by default the library splits K when the product has few tiles."""
     device = _native.require_cuda(rows, weight)
     if rows.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or rows.ndim != 2 or weight.ndim != 2:
         raise TypeError("bf16_gemm takes two BF16 matrices")
     if rows.shape[1] != weight.shape[1]:
         raise ValueError("operands disagree on K")
-    out = torch.empty((rows.shape[0], weight.shape[0]), dtype=torch.bfloat16, device=device)
-    _native.check(_native.library().nq_bf16_gemm(rows.data_ptr(), weight.data_ptr(), rows.shape[0], weight.shape[0],
-                                                 rows.shape[1], out.data_ptr(), tile, _native.stream_handle(device)))
+    m, n = rows.shape[0], weight.shape[0]
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    need = 8 * m * n * 4 if m * n <= (1 << 22) else 0               # room for the widest split of a small product
+    workspace = _workspace(device, need) if need else None
+    _native.check(_native.library().nq_bf16_gemm(rows.data_ptr(), weight.data_ptr(), m, n, rows.shape[1], out.data_ptr(),
+                                                 tile, split_k, None if workspace is None else workspace.data_ptr(), need,
+                                                 _native.stream_handle(device)))
     return out
 
 

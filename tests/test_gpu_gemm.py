@@ -149,7 +149,8 @@ def test_long_prefill_decodes_the_weight_once(rt, oracle, k, n_out):
     assert relative_error(bits(y.float()), bits(fused.float())) <= 5e-3
 
 
-@pytest.mark.parametrize("m,n,k", [(300, 200, 128), (257, 520, 384), (64, 64, 128), (1000, 72, 256), (384, 8192, 2048)])
+@pytest.mark.parametrize("m,n,k", [(300, 200, 128), (257, 520, 384), (64, 64, 128), (1000, 72, 256), (384, 8192, 2048),
+                                   (384, 2048, 8192), (130, 136, 1024)])
 def test_dense_bf16_gemm_against_float32(rt, m, n, k):
     """nq_bf16_gemm (the multiply of the decode-once route) against the FP32 product of the same BF16
     operands: FP32 accumulation and one BF16 rounding of the result leave <= 2^-8 relative to the
@@ -162,5 +163,15 @@ def test_dense_bf16_gemm_against_float32(rt, m, n, k):
         c = rt.bf16_gemm(a, b, tile=tile)
         assert c.dtype == torch.bfloat16 and tuple(c.shape) == (m, n)
         assert relative_error(bits(c.float()), ref) <= 2.0 ** -8, (tile,)
+    # K split: slabs of float32 partial results added in ascending order by a second launch
+    for split in (2, 4, 8):
+        if k % (128 * split):
+            with pytest.raises(RuntimeError, match="K split"):
+                rt.bf16_gemm(a, b, split_k=split)
+            continue
+        for tile in (-1, 3, 6):
+            c = rt.bf16_gemm(a, b, tile=tile, split_k=split)
+            assert relative_error(bits(c.float()), ref) <= 2.0 ** -8, (tile, split)
+    assert torch.equal(rt.bf16_gemm(a, b, split_k=1), rt.bf16_gemm(a, b, split_k=1))
     with pytest.raises(ValueError, match="multiple of 128"):
         rt.bf16_gemm(a[:, :64].contiguous(), b[:, :64].contiguous())
