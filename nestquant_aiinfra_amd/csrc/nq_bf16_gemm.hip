@@ -185,6 +185,164 @@ bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b,
     }
 }
 
+
+// The same product with the wavefronts of a workgroup split by role: four of the eight (one per
+// SIMD) only move data -- global loads three steps ahead into a ring of registers, then into a ring
+// of three LDS stages -- and four only multiply, each a quarter (WM x WN tiles of 32 x 32) of the
+// workgroup's 64 WM x 64 WN tile.  A wavefront that waits for memory therefore never holds back
+// matrix instructions: the multiplying wavefront of its SIMD keeps issuing.  One barrier per step of
+// 64 k; before it the movers wait for their LDS stores only (their global loads stay in flight).
+template <int WM, int WN>
+__global__ void __launch_bounds__(512)
+bf16_gemm_roles_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b, uint16_t *__restrict__ c,
+                       int m_size, int n_size, int k_size, int tiles_m, int tiles_n, int group_m, int k_slab,
+                       float *__restrict__ partials) {
+    constexpr int BM = 64 * WM, BN = 64 * WN;
+    constexpr int kStage = (BM + BN) * 8;                          // 16-byte pieces per LDS stage
+    constexpr int kLoadsA = BM / 32, kLoadsB = BN / 32;            // 256 mover lanes cover 32 rows of 128 bytes per pass
+    constexpr int kLoads = kLoadsA + kLoadsB;
+    extern __shared__ u32x4 lds[];                                 // [3][BM + BN][8] pieces
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    int pid = blockIdx.x;
+    const int total = tiles_m * tiles_n;
+    if (total % 8 == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+    const int per_group = group_m * tiles_n;
+    const int group = pid / per_group, first_m = group * group_m;
+    const int rows_in_group = tiles_m - first_m < group_m ? tiles_m - first_m : group_m;
+    const int in_group = pid - group * per_group;
+    const int tile_m = first_m + in_group % rows_in_group, tile_n = in_group / rows_in_group;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int k_begin = blockIdx.y * k_slab;
+    const int steps = k_slab / kDenseBK;
+    // a workgroup barrier that orders LDS traffic only: the movers' global loads stay in flight across it
+    auto lds_barrier = [] {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    };
+
+    if (wave >= 4) {
+        // ---- movers ---------------------------------------------------------------------------------
+        const int mover = tid - 256;
+        const int load_row = mover >> 3, load_piece = mover & 7;
+        const int store_slot = load_row * 8 + (load_piece ^ ((load_row >> 1) & 7));
+        int offset[kLoads], slot[kLoads];
+#pragma unroll
+        for (int i = 0; i < kLoadsA; i++) {
+            const int row = m0 + load_row + 32 * i;
+            offset[i] = (row < m_size ? row : m_size - 1) * k_size + k_begin + load_piece * 8;
+            slot[i] = store_slot + 256 * i;
+        }
+#pragma unroll
+        for (int i = 0; i < kLoadsB; i++) {
+            const int row = n0 + load_row + 32 * i;
+            offset[kLoadsA + i] = (row < n_size ? row : n_size - 1) * k_size + k_begin + load_piece * 8;
+            slot[kLoadsA + i] = BM * 8 + store_slot + 256 * i;
+        }
+        auto request = [&](int step, u32x4 (&into)[kLoads]) {
+            const int at = (step < steps ? step : steps - 1) * kDenseBK;        // past the end: any valid slab, never stored
+#pragma unroll
+            for (int i = 0; i < kLoads; i++) {
+                const uint16_t *base = i < kLoadsA ? a : b;
+                into[i] = *reinterpret_cast<const u32x4 *>(base + offset[i] + at);
+            }
+        };
+        auto park = [&](int step, const u32x4 (&from)[kLoads]) {
+            if (step < steps) {
+                u32x4 *stage = lds + (step % 3) * kStage;
+#pragma unroll
+                for (int i = 0; i < kLoads; i++) stage[slot[i]] = from[i];
+            }
+        };
+        u32x4 r0[kLoads], r1[kLoads], r2[kLoads];
+        request(0, r0);
+        request(1, r1);
+        request(2, r2);
+        park(0, r0);
+        park(1, r1);
+        request(3, r0);
+        request(4, r1);
+        lds_barrier();
+        // at step s: slab s + 2 goes to its stage (the one the multipliers finished with at step s - 1),
+        // slab s + 5 is requested into the registers that held it
+        for (int s = 0; s < steps; s += 3) {
+            park(s + 2, r2);
+            request(s + 5, r2);
+            lds_barrier();
+            if (s + 1 < steps) {
+                park(s + 3, r0);
+                request(s + 6, r0);
+                lds_barrier();
+            }
+            if (s + 2 < steps) {
+                park(s + 4, r1);
+                request(s + 7, r1);
+                lds_barrier();
+            }
+        }
+        return;
+    }
+
+    // ---- multipliers --------------------------------------------------------------------------------
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const int frag_row = lane & 31, frag_half = lane >> 5, frag_mask = (lane >> 1) & 7;
+    const int a_frag_base = (wave_m * 32 * WM + frag_row) * 8;
+    const int b_frag_base = (BM + wave_n * 32 * WN + frag_row) * 8;
+    gemm_floatx16 acc[WM][WN];
+#pragma unroll
+    for (int i = 0; i < WM; i++)
+#pragma unroll
+        for (int j = 0; j < WN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+    lds_barrier();                                                 // slabs 0 and 1 are parked
+    for (int step = 0; step < steps; step++) {
+        const u32x4 *now = lds + (step % 3) * kStage;
+        gemm_bf16x8 fa[2][WM], fb[2][WN];
+#pragma unroll
+        for (int i = 0; i < WM; i++) fa[0][i] = __builtin_bit_cast(gemm_bf16x8, now[a_frag_base + 256 * i + (frag_half ^ frag_mask)]);
+#pragma unroll
+        for (int j = 0; j < WN; j++) fb[0][j] = __builtin_bit_cast(gemm_bf16x8, now[b_frag_base + 256 * j + (frag_half ^ frag_mask)]);
+#pragma unroll
+        for (int s = 0; s < kDenseBK / 16; s++) {
+            if (s + 1 < kDenseBK / 16) {
+                const int piece = (2 * (s + 1) + frag_half) ^ frag_mask;
+#pragma unroll
+                for (int i = 0; i < WM; i++)
+                    fa[(s + 1) & 1][i] = __builtin_bit_cast(gemm_bf16x8, now[a_frag_base + 256 * i + piece]);
+#pragma unroll
+                for (int j = 0; j < WN; j++)
+                    fb[(s + 1) & 1][j] = __builtin_bit_cast(gemm_bf16x8, now[b_frag_base + 256 * j + piece]);
+            }
+#pragma unroll
+            for (int i = 0; i < WM; i++)
+#pragma unroll
+                for (int j = 0; j < WN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
+        }
+        lds_barrier();                                             // every fragment of the stage has arrived
+    }
+#pragma unroll
+    for (int i = 0; i < WM; i++) {
+        const int row_base = m0 + wave_m * 32 * WM + 32 * i + 4 * frag_half;
+#pragma unroll
+        for (int j = 0; j < WN; j++) {
+            const int col = n0 + wave_n * 32 * WN + 32 * j + frag_row;
+            if (col < n_size) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = row_base + (r & 3) + 8 * (r >> 2);
+                    if (row < m_size) {
+                        if (partials) partials[((int64_t)blockIdx.y * m_size + row) * n_size + col] = acc[i][j][r];
+                        else c[(int64_t)row * n_size + col] = dense_f32_to_bf16(acc[i][j][r]);
+                    }
+                }
+            }
+        }
+    }
+}
+
 }  // namespace nq
 
 namespace {
@@ -192,10 +350,14 @@ namespace {
 struct DenseTile { int bm, bn; float efficiency; };
 
 // Workgroup tiles from the fastest per product to the slowest; `efficiency` is the measured rate
-// relative to the 256 x 256 tile on a problem that fills the chip (8192^3: 1.13, 0.92, 0.92, 0.93,
-// 0.74, 0.74, 0.61 PFLOP/s).
+// relative to the 256 x 256 tile on a problem that fills the chip (8192^3: 1.13, 0.92, 0.99, 0.93,
+// 0.74, 0.74, 0.61 PFLOP/s).  The 256 x 128 tile runs on the kernel with movers and multipliers
+// (0.94 PFLOP/s with every wavefront doing both; the same split gave 0.87 against 0.92 at 128 x 128,
+// which keeps the plain kernel).  All of them sit at the LDS's 128 bytes per clock: a wavefront that
+// owns 2 x 4 tiles reads 0.75 KB of fragments per matrix instruction, which with the stores of the
+// next slab is about 125 bytes per clock at full matrix rate.
 const DenseTile kDenseTiles[] = {
-    {256, 256, 1.00f}, {128, 256, 0.81f}, {256, 128, 0.81f}, {128, 128, 0.82f}, {64, 128, 0.65f}, {128, 64, 0.65f},
+    {256, 256, 1.00f}, {128, 256, 0.81f}, {256, 128, 0.89f}, {128, 128, 0.82f}, {64, 128, 0.65f}, {128, 64, 0.65f},
     {64, 64, 0.55f},
 };
 
@@ -214,6 +376,25 @@ void launch_dense(const void *a, const void *b, void *c, int m, int n, int k, in
     const int group_m = tiles_m < 4 ? tiles_m : 4;
     hipLaunchKernelGGL((nq::bf16_gemm_kernel<WM, WN, GM, GN>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)split),
                        dim3(64 * GM * GN), lds_bytes, stream, reinterpret_cast<const uint16_t *>(a),
+                       reinterpret_cast<const uint16_t *>(b), reinterpret_cast<uint16_t *>(c), m, n, k, tiles_m, tiles_n,
+                       group_m, k / split, split > 1 ? partials : nullptr);
+}
+
+template <int WM, int WN>
+void launch_roles(const void *a, const void *b, void *c, int m, int n, int k, int split, float *partials,
+                  hipStream_t stream) {
+    constexpr int BM = 64 * WM, BN = 64 * WN;
+    const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+    const size_t lds_bytes = (size_t)3 * (BM + BN) * 128;
+    static bool raised = false;
+    if (!raised) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(nq::bf16_gemm_roles_kernel<WM, WN>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        raised = true;
+    }
+    const int group_m = tiles_m < 4 ? tiles_m : 4;
+    hipLaunchKernelGGL((nq::bf16_gemm_roles_kernel<WM, WN>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)split),
+                       dim3(512), lds_bytes, stream, reinterpret_cast<const uint16_t *>(a),
                        reinterpret_cast<const uint16_t *>(b), reinterpret_cast<uint16_t *>(c), m, n, k, tiles_m, tiles_n,
                        group_m, k / split, split > 1 ? partials : nullptr);
 }
@@ -260,7 +441,7 @@ int launch_bf16_gemm(const void *a, const void *b, void *c, int m, int n, int k,
     switch (best) {
         case 0: launch_dense<2, 4, 4, 2>(a, b, c, m, n, k, split, p, stream); break;
         case 1: launch_dense<2, 4, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
-        case 2: launch_dense<4, 2, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
+        case 2: launch_roles<4, 2>(a, b, c, m, n, k, split, p, stream); break;      // movers and multipliers
         case 3: launch_dense<2, 2, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
         case 4: launch_dense<1, 2, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
         case 5: launch_dense<2, 1, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
