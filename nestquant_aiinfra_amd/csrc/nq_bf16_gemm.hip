@@ -35,6 +35,32 @@ __device__ __forceinline__ uint16_t dense_f32_to_bf16(float x) {
     return (uint16_t)(bits >> 16);
 }
 
+// The order a step's instructions should issue in (a hint to the scheduler, sched_group_barrier):
+// the first fragments, then kGroups groups of four matrix instructions, each followed by its share
+// of the kReads LDS reads of the next fragments, of the kMoves LDS stores of the next slab and of
+// the kMoves global requests.  Left to itself the compiler issues the step as requests, reads and
+// matrix instructions, stores: with the phases interleaved a wavefront's waits fall behind matrix
+// instructions that are still running (8192^3: 1049 -> 945 us).
+template <int kGroups, int kReads, int kMoves, int g = 0>
+__device__ __forceinline__ void issue_order_groups() {
+    if constexpr (g < kGroups) {
+        constexpr int reads = kReads / kGroups + (g >= kGroups - kReads % kGroups ? 1 : 0);
+        constexpr int moves = kMoves / kGroups + (g >= kGroups - kMoves % kGroups ? 1 : 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);                       // matrix instructions
+        if constexpr (reads > 0) __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);       // LDS reads
+        if constexpr (moves > 0) {
+            __builtin_amdgcn_sched_group_barrier(0x200, moves, 0);              // LDS stores
+            __builtin_amdgcn_sched_group_barrier(0x020, moves, 0);              // global loads
+        }
+        issue_order_groups<kGroups, kReads, kMoves, g + 1>();
+    }
+}
+template <int kGroups, int kReads, int kMoves>
+__device__ __forceinline__ void issue_order(int) {
+    __builtin_amdgcn_sched_group_barrier(0x100, kReads / 3, 0);
+    issue_order_groups<kGroups, kReads, kMoves>();
+}
+
 // WM x WN: 32 x 32 tiles per wavefront; GM x GN: wavefronts per workgroup along M and N.
 template <int WM, int WN, int GM, int GN>
 __global__ void __launch_bounds__(64 * GM * GN)
@@ -157,7 +183,11 @@ bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b,
         for (int i = 0; i < kLoadsA; i++) next[store_slot + kRowsPerPass * 8 * i] = early_a[i];
 #pragma unroll
         for (int i = 0; i < kLoadsB; i++) next[BM * 8 + store_slot + kRowsPerPass * 8 * i] = early_b[i];
-        __syncthreads();
+        issue_order<WM * WN, 3 * (WM + WN), kLoadsA + kLoadsB>(WM + WN);
+        // a barrier that orders LDS traffic only: the requests for slab step + 2 stay in flight across it
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     };
     for (int step = 0; step < steps; step += 2) {          // the host checks that the step count is even
         dense_step(step, pa0, pb0, pa1, pb1);
@@ -321,6 +351,7 @@ bf16_gemm_roles_kernel(const uint16_t *__restrict__ a, const uint16_t *__restric
                 for (int j = 0; j < WN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
         }
+        issue_order<WM * WN, 3 * (WM + WN), 0>(WM + WN);
         lds_barrier();                                             // every fragment of the stage has arrived
     }
 #pragma unroll
