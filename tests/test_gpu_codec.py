@@ -229,3 +229,24 @@ def test_errors_are_reported_like_the_reference(rt):
         rt.quantize_activation_cuda(torch.randn(2, 32), q=Q, betas=ACTIVATION_BETAS)  # CPU tensor
     with pytest.raises(RuntimeError, match="contiguous"):
         rt.quantize_rows_packed(torch.randn(64, 4, device="cuda").t(), q=Q, beta_table=_table(ACTIVATION_BETAS))
+
+
+@pytest.mark.parametrize("n", [2048, 4096, 8192])
+@pytest.mark.parametrize("rows", [1, 3, 16])
+def test_decode_size_encoder_equals_the_many_row_encoder(rt, rows, n):
+    """Up to 16 BF16 rows of 2048, 4096 or 8192 values take the one-lane-per-eight-values kernel,
+    more rows the row-at-a-time or the bulk kernel: the same rows must come out of either bit for bit
+    (rotation included), zero rows and rows of huge and tiny magnitude among them."""
+    g = torch.Generator().manual_seed(rows * n)
+    x = torch.randn(17, n, generator=g) * torch.logspace(-15, 15, 17).unsqueeze(-1)
+    x[min(2, rows - 1)] = 0.0
+    x = x.to(torch.bfloat16).cuda()
+    table = _table(ACTIVATION_BETAS)
+    for rotate in (True, False):
+        few = rt.quantize_activation_cuda(x[:rows].contiguous(), q=Q, betas=ACTIVATION_BETAS, beta_table=table,
+                                          hadamard=rotate)
+        many = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS, beta_table=table, hadamard=rotate)
+        assert torch.equal(few.code_payload, many.code_payload[: rows * n // 2]), rotate
+        assert torch.equal(few.beta_payload, many.beta_payload[: rows * n // 32]), rotate
+        assert torch.equal(few.row_norms, many.row_norms[:rows]), rotate
+        assert torch.equal(few.decoded, many.decoded[:rows]), rotate
