@@ -527,6 +527,10 @@ def attention_extra(device):
     seconds = time_graph(lambda i: nqkv.launch_nqkv_decode_attention(
         query, manager.layers[i % 4], slot_ids=slot_ids, active_mask=active, attention_scale=0.125,
         workspace=workspace).clone(), 8)
+    # the first stage alone (the decode step merges its partial results inside the next encoder)
+    stage1 = time_graph(lambda i: nqkv.launch_nqkv_decode_attention(
+        query, manager.layers[i % 4], slot_ids=slot_ids, active_mask=active, attention_scale=0.125,
+        workspace=workspace, merge=False), 8)
     bytes_moved = sum(608 * 16 * (n // 16) + (n % 16) * 8 * 64 * 2 * 2 + 2 * 32 * 64 * 2 for n in lengths)
     step_key = torch.randn(8, 1, 8, 64, device=device).to(torch.bfloat16)
     manager.step_active.fill_(False)             # time the writer's launch without growing the cache
@@ -540,6 +544,7 @@ def attention_extra(device):
     prefill_flops = sum(4 * 32 * 64 * sum(n - chunk + t + 1 for t in range(chunk)) for n in lengths)
     return {"contexts": lengths, "us": seconds * 1e6, "algorithmic_bytes": bytes_moved,
             "GBps": bytes_moved / seconds / 1e9, "hbm_frac": bytes_moved / seconds / 1e9 / HBM_PEAK_GBPS,
+            "stage1_us": stage1 * 1e6, "stage1_hbm_frac": bytes_moved / stage1 / 1e9 / HBM_PEAK_GBPS,
             "append_launch_us": write * 1e6,
             "prefill_chunk128": {"us": prefill * 1e6, "flops": prefill_flops,
                                  "TFLOPs": prefill_flops / prefill / 1e12}}
@@ -667,7 +672,8 @@ def extra_rooflines(extra):
         "nqkv_attention": {"bound": "hbm", "workload": "batch 8, 32 / 8 heads, D 64, contexts uniform in [128, 4096]",
                            "achieved": attention["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                            "frac": attention["hbm_frac"], "launch_us": attention["us"],
-                           "algorithmic_bytes": attention["algorithmic_bytes"]},
+                           "algorithmic_bytes": attention["algorithmic_bytes"],
+                           "stage1_launch_us": attention["stage1_us"], "stage1_frac": attention["stage1_hbm_frac"]},
         "e8_encode": {name: {"bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                              "frac": row["hbm_frac"], "launch_us": row["us"], "algorithmic_bytes": row["bytes"]}
                       for name, row in encoders.items()},
