@@ -420,17 +420,18 @@ __device__ __forceinline__ float wave_sum_in_lane_order(float v) {
 // of the first of them in the row-major input.  Mode 1 needs the whole workgroup (one barrier);
 // `wave_sums` is LDS for one float per wavefront.
 template <int kPrologue>
-__device__ __forceinline__ void lane_prologue(const uint16_t *__restrict__ x, const InputPrologue &pro, int64_t g, int n,
+__device__ __forceinline__ void lane_prologue(const uint16_t *__restrict__ x, const InputPrologue &pro, int64_t row, int n,
                                               bool writes_outputs, float *wave_sums, float (&y)[8]) {
     const int chunk = threadIdx.x;
+    const int64_t g = row * n + 8 * chunk;
     if (kPrologue == 3) {
         constexpr int kBatch = 8;
         const float kNone = -__builtin_inff();
 #pragma unroll
         for (int j = 0; j < 8; j++) y[j] = 0.0f;
-        const int64_t head = (g / n) * pro.heads + (g % n) / 64;
+        const int64_t head = row * pro.heads + (chunk >> 3);      // eight lanes per head of 64
         const float *m = pro.part_max + head * pro.parts, *sum = pro.part_sum + head * pro.parts;
-        const float *acc = pro.part_acc + head * pro.parts * 64 + (g % 64);
+        const float *acc = pro.part_acc + head * pro.parts * 64 + 8 * (chunk & 7);
         float top = kNone, denom = 0.0f;
         for (int c0 = 0; c0 < pro.parts; c0 += kBatch) {
             float mc[kBatch], sc[kBatch];
@@ -596,7 +597,7 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
     NQ_STAMP(0);
 
     float v[8];
-    lane_prologue<kPrologue>(x, pro, row * n + 8 * tid, n, slice == 0, wave_sums, v);
+    lane_prologue<kPrologue>(x, pro, row, n, slice == 0, wave_sums, v);
     if (codes == nullptr) return;                         // element-wise stage only
     NQ_STAMP(1);
 
