@@ -342,10 +342,13 @@ __device__ __forceinline__ void resolved_apply(uint32_t lo, uint32_t hi, const u
     const uint32_t low_fields = as_computed(lo << 15), tail_fields = as_computed(hi << 17);
     const uint32_t field[8] = {low_fields, low_fields >> 5, low_fields >> 10, lo, lo >> 5, lo >> 10,
                                tail_fields, tail_fields >> 5};
+    // (float - origin) * scale as one fused multiply-add: one rounding instead of two (the difference
+    // is exact in the first form, so only the final rounding can move, by half a unit in the last place)
+    const float shift = -origin * scale;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const uint32_t pattern = ((field[j] & (31u << 17)) | 0x4b000000u) + bits[j];
-        out[j] = (__uint_as_float(pattern) - origin) * scale;
+        out[j] = __builtin_fmaf(__uint_as_float(pattern), scale, shift);
     }
 }
 
