@@ -400,6 +400,37 @@ int nq_nqkv_attention_decode(
 size_t nq_nqkv_attention_workspace_bytes(int batch, int q_heads, int head_dim, int max_pages);
 
 /*
+ * One decode step's KV append and attention of a layer in one launch: what nq_nqkv_write (one
+ * new BF16 token per row, uniform count 1) followed by nq_nqkv_attention_decode computes, for
+ * tables nq_nqkv_advance / nq_decode_step_begin have already advanced by this token.  The
+ * workgroup that attends over a row's hot tail takes the row's new key and value
+ * [batch, kv_heads, head_dim] as the projections left them, applies the rotary tables (the
+ * same BF16 [batch, head_dim] rows serve the query and the key: they share the position) and,
+ * with rotate != 0, the Hadamard rotation to both, and appends the pair to the slot's hot tail;
+ * a token that completes a page is encoded with the page (codes, beta ids and norms bit-equal
+ * to nq_nqkv_write's) into page_indices[slot, (length - 1) / page_size], and this launch
+ * attends over that page through the codes it has just made.  Rows write under
+ * nq_nqkv_write's conditions (active, slot in range, length > 0) whether or not cache_active
+ * lets them attend.  The attention output equals the two-call form but for the order in which
+ * the completed page's part is merged (float32 rounding).  out_dev may be NULL as for
+ * nq_nqkv_attention_decode.  BF16 only; same shape limits as the two calls it replaces.
+ * Replaces: append_hot_k1_graph_safe + launch_pack_full_hot_pages_graph_safe
+ * (nestquant/runtime/nqkv_graph_writer.py:263-473, nqkv_graph_pack.py:76-193) followed by
+ * nqkv_decode_attention_batched_k1 (nestquant/runtime/nqkv_attention_k1.py:763-942) in
+ * BatchedNQKVLlamaCache's decode update (nestquant/runtime/nqkv_batched_hf_backend.py:357-631).
+ */
+int nq_nqkv_append_attention_decode(
+    const void *query_dev, const void *key_dev, const void *value_dev, const int32_t *sequence_lengths_dev,
+    uint8_t *key_codes_dev, uint8_t *key_beta_ids_dev, float *key_norms_dev, uint8_t *value_codes_dev,
+    uint8_t *value_beta_ids_dev, float *value_norms_dev, const float *key_betas_dev, int key_beta_count,
+    const float *value_betas_dev, int value_beta_count, const int32_t *page_indices_dev,
+    const int32_t *page_counts_dev, const int32_t *last_page_lens_dev, const int32_t *hot_lengths_dev,
+    const uint8_t *cache_active_dev, void *hot_keys_dev, void *hot_values_dev, const int32_t *slot_ids_dev,
+    const uint8_t *active_mask_dev, int batch, int slots, int max_pages, int q_heads, int kv_heads, int head_dim,
+    int page_size, float scale, int rotate, const void *rope_cos_dev, const void *rope_sin_dev, void *out_dev,
+    void *workspace_dev, size_t workspace_bytes, void *stream);
+
+/*
  * The second stage of the decode attention done where its result is consumed.  With
  * out_dev == NULL nq_nqkv_attention_decode leaves the per-chunk partial results (maxima, sums
  * and numerators of nq_nqkv_attention_parts(batch, max_pages) chunks per head) in its workspace;

@@ -59,6 +59,8 @@ SIGNATURES = {
                       + [_ptr, _i32, _ptr, _i32, _ptr, _ptr] + [_i32] * 8 + [_ptr, _ptr, _ptr]),
     "nq_nqkv_attention_decode": (_i32, [_ptr, _i32] + [_ptr] * 17 + [_i32] * 7 + [_c.c_float, _i32, _ptr, _ptr,
                                                                                 _ptr, _ptr, _size, _ptr]),
+    "nq_nqkv_append_attention_decode": (_i32, [_ptr] * 10 + [_ptr, _i32, _ptr, _i32] + [_ptr] * 9 + [_i32] * 7
+                                        + [_c.c_float, _i32, _ptr, _ptr, _ptr, _ptr, _size, _ptr]),
     "nq_nqkv_attention_prefill": (_i32, [_ptr] * 19 + [_i32] * 9 + [_c.c_float, _ptr, _ptr]),
     "nq_nqkv_attention_workspace_bytes": (_size, [_i32, _i32, _i32, _i32]),
     "nq_nqkv_attention_parts": (_i32, [_i32, _i32]),

@@ -19,6 +19,14 @@
 // beyond the table width (the reference stops at 64 pages, nqkv_attention_k1.py:696-698).
 // Decoded K/V stay FP32 (as in the reference's fused kernel); K/V decode follows the exact
 // float32 order of nq_e8.hip.h because undithered codes sit on exact Voronoi ties.
+//
+// A decode step can append as it attends (kWrites launches): the hot-tail workgroup of a row
+// takes the row's new key and value straight from the projections, applies the rotary embedding
+// and the Hadamard rotation to the key, stores the pair in the slot's hot tail and attends over
+// the tail from LDS.  When the new token completes a page the workgroup encodes the page as the
+// KV writer does (same device routine, same bits), stores it in the pool and attends over the
+// 16 tokens through the codes it has just made; the workgroups of the cold chunks leave that
+// page alone in this launch.  One launch per layer instead of the writer's and the attention's.
 #define NQ_PHASE_STAMP_ARRAY g_attention_stamps
 #include "nq_rowquant.hip.h"
 #include "nq_host.h"
@@ -56,7 +64,63 @@ struct AttentionArgs {
     int batch, slots, max_pages, q_heads, kv_heads, chunks, query_dtype, rotate_query;
     float scale;
     float *part_max, *part_sum, *part_acc;        // [batch, q_heads, chunks + 1] (x D)
+    // kWrites launches only: one new token per active row
+    const uint16_t *new_key, *new_value;          // BF16 [batch, kv_heads, D], the key before RoPE and rotation
+    const int32_t *sequence_lengths;              // [slots], this step's token already counted
+    int key_beta_count, rotate_keys;
 };
+
+// Rotary embedding ((x * cos) + (rotate_half(x) * sin) in BF16 tensor arithmetic), then optionally
+// the Hadamard rotation (float32 butterflies over the head, scaled by 1 / sqrt(D), rounded to
+// `dtype`: hadamard(x.float()).to(dtype), nestquant/runtime/nqkv_batched_hf_backend.py:381, 549) of a
+// head vector of 64 held by eight neighbouring lanes, lane `piece` elements 8 piece .. 8 piece + 7.
+__device__ __forceinline__ void rope_then_rotate(float (&x)[8], const float (&rope_c)[8], const float (&rope_s)[8],
+                                                 bool rope, bool rotate, int dtype, int lane) {
+    if (rope) {
+        const bool upper = (lane & 7) >= 4;
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            const float o0 = lane_xor<4>(x[j]), o1 = lane_xor<4>(x[j + 1]);
+            float a0 = x[j] * rope_c[j], a1 = x[j + 1] * rope_c[j + 1];
+            round_pair<1>(a0, a1);
+            float b0 = o0 * rope_s[j], b1 = o1 * rope_s[j + 1];
+            round_pair<1>(b0, b1);
+            x[j] = upper ? a0 + b0 : a0 - b0;
+            x[j + 1] = upper ? a1 + b1 : a1 - b1;
+            round_pair<1>(x[j], x[j + 1]);
+        }
+    }
+    if (rotate) {
+#pragma unroll
+        for (int s = 0; s < 3; s++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                if (j & (1 << s)) continue;
+                const float left = x[j], right = x[j + (1 << s)];
+                x[j] = left + right;
+                x[j + (1 << s)] = left - right;
+            }
+        }
+        lane_stage<1, 0>(x, lane);
+        lane_stage<2, 0>(x, lane);
+        lane_stage<4, 0>(x, lane);
+        const float inv = 1.0f / __builtin_sqrtf(64.0f);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float scaled = x[j] * inv;
+            x[j] = dtype == NQ_BF16 ? bf16_to_f32(f32_to_bf16(scaled)) : (dtype == NQ_F16 ? (float)(_Float16)scaled : scaled);
+        }
+    }
+}
+
+__device__ __forceinline__ void unpack_bf16_row(const uint4 &raw, float (&x)[8]) {
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        x[2 * j] = __uint_as_float(w[j] << 16);
+        x[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+}
 
 __device__ __forceinline__ float load_query(const void *q, int dtype, int64_t i) {
     if (dtype == NQ_BF16) return bf16_to_f32(reinterpret_cast<const uint16_t *>(q)[i]);
@@ -124,7 +188,7 @@ __device__ __forceinline__ float fold_rows(float v) {
 // activity flag, the group's queries and their rotary rows; (2) the slot's lengths and the page
 // ids of the chunk (requested for every ordinal of the chunk before the count says which exist);
 // (3) the packed keys and values of every pass together.
-template <int D, int P, int G, int kAttnPagesPerChunk>     // head_dim, page_size, query heads per KV head, pages per chunk
+template <int D, int P, int G, int kAttnPagesPerChunk, bool kWrites>   // head_dim, page_size, query heads per KV head, pages per chunk
 __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(AttentionArgs a) {
     constexpr int kBlocks = D / 8;                       // E8 blocks per head vector
     constexpr int kTokenBlocks = P * kBlocks;            // lanes needed per page
@@ -136,8 +200,14 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
                   "page does not tile the workgroup");
     static_assert(D == 64 && G * 8 <= 64 && kBlocks == 8, "eight lanes of the first wavefront prepare one head's query");
     static_assert(kChunkTokens % 64 == 0, "every lane of a wavefront takes the same number of scores");
+    static_assert(2 * kTokenBlocks <= kAttnThreads, "one lane per block of the tail's keys and values");
     __shared__ float scores[G][kChunkTokens];
     __shared__ float acc_lds[kWaves][G * 8][kBlocks];    // one entry per wavefront; holds the queries first
+    // kWrites: the slot's hot tail with the new token (keys, then values), and the page made from it
+    __shared__ float tail[kWrites ? 2 * P : 1][kWrites ? D : 1];
+    __shared__ float tail_scale[kWrites ? 2 * P : 1], tail_norm[kWrites ? 2 * P : 1];
+    __shared__ uint32_t tail_code[kWrites ? 2 * P : 1][kWrites ? kBlocks : 1];
+    __shared__ uint32_t tail_ids[kWrites ? 2 * P : 1][kWrites ? kBlocks / 4 : 1];
 
     const int tid = threadIdx.x;
     NQ_STAMP(0);
@@ -150,6 +220,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     const int chunk = pair % (a.chunks + 1), row = pair / (a.chunks + 1);
     if (row >= a.batch) return;                          // padding of the last group of eight pairs
     const bool is_hot = chunk == a.chunks;
+    const bool appends = kWrites && is_hot;              // this workgroup owns the row's new token
     const int first_page = chunk * kAttnPagesPerChunk;
     const int64_t part = ((int64_t)row * a.q_heads + (int64_t)g * G) * (a.chunks + 1) + chunk;   // + h * (chunks + 1)
 
@@ -158,25 +229,26 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     const int row_in_page = token * a.kv_heads + g;
     const int64_t page_words = (int64_t)P * a.kv_heads * kBlocks, page_rows = (int64_t)P * a.kv_heads;
 
-    // ---- round 1: slot, activity, queries ------------------------------------------------------
-    int slot = a.slot_ids[row];
+    // ---- round 1: slot, activity, queries (and the new key and value) ------------------------------
+    const int given_slot = a.slot_ids[row];
     const bool row_active = a.active_mask[row] != 0;
-    // lane 8 h + piece of the first wavefront holds elements 8 piece .. 8 piece + 7 of head h
+    // lane 8 h + piece of the first wavefront holds elements 8 piece .. 8 piece + 7 of head h; the
+    // first eight lanes of the second wavefront hold the new key the same way
     const int qh = tid >> 3, piece = tid & 7;
+    const bool key_lane = appends && tid >= 64 && tid < 72;
     float qv[8], rope_c[8], rope_s[8];
-    if (tid < G * 8) {
-        const int64_t at = ((int64_t)row * a.q_heads + g * G + qh) * D + piece * 8;
-        if (a.query_dtype == NQ_BF16) {
-            const uint4 raw = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.query) + at);
-            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                qv[2 * j] = __uint_as_float(w[j] << 16);
-                qv[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
-            }
+    uint4 new_value = make_uint4(0, 0, 0, 0);
+    if (tid < G * 8 || key_lane) {
+        if (key_lane) {
+            unpack_bf16_row(*reinterpret_cast<const uint4 *>(a.new_key + ((int64_t)row * a.kv_heads + g) * D + piece * 8), qv);
         } else {
+            const int64_t at = ((int64_t)row * a.q_heads + g * G + qh) * D + piece * 8;
+            if (a.query_dtype == NQ_BF16) {
+                unpack_bf16_row(*reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.query) + at), qv);
+            } else {
 #pragma unroll
-            for (int j = 0; j < 8; j++) qv[j] = load_query(a.query, a.query_dtype, at + j);
+                for (int j = 0; j < 8; j++) qv[j] = load_query(a.query, a.query_dtype, at + j);
+            }
         }
         if (a.rope_cos) {
             const int64_t rope_at = (int64_t)row * D + piece * 8;
@@ -187,13 +259,18 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
             }
         }
     }
+    // lanes 128 .. 255 stage the tail's values: each requests the new value's piece it may need
+    if (appends && tid >= kTokenBlocks && tid < 2 * kTokenBlocks)
+        new_value = *reinterpret_cast<const uint4 *>(a.new_value + ((int64_t)row * a.kv_heads + g) * D + blk * 8);
     // beta tables in registers: a table lookup from memory would sit behind every decode
     const float key_beta[4] = {a.key_betas[0], a.key_betas[1], a.key_betas[2], a.key_betas[3]};
     const float value_beta[4] = {a.value_betas[0], a.value_betas[1], a.value_betas[2], a.value_betas[3]};
 
     // ---- round 2: lengths and page ids of the slot ------------------------------------------------
-    slot = slot < 0 ? 0 : (slot >= a.slots ? a.slots - 1 : slot);
+    const bool slot_known = given_slot >= 0 && given_slot < a.slots;
+    const int slot = given_slot < 0 ? 0 : (given_slot >= a.slots ? a.slots - 1 : given_slot);
     const int page_count = a.page_counts[slot], last_len = a.last_page_lens[slot], hot_len = a.hot_lengths[slot];
+    const int length = kWrites ? a.sequence_lengths[slot] : 0;
     const bool cache_live = !a.cache_active || a.cache_active[slot];
     int64_t pass_pageid[kPasses];
 #pragma unroll
@@ -202,9 +279,17 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
         pass_pageid[pass] = (!is_hot && ordinal < a.max_pages) ? a.page_indices[(int64_t)slot * a.max_pages + ordinal] : 0;
     }
     NQ_STAMP(1);
+    // the row's new token (as the KV writer decides it: an active row with a known slot that holds
+    // at least this token) sits at position length - 1; it completes a page when length % P == 0
+    const bool writes = kWrites && row_active && slot_known && length > 0;
+    const bool packs = writes && length % P == 0;
+    const int new_at = writes ? (length - 1) % P : -1;           // the new token's place in the tail
+    const int tail_old = writes ? new_at : hot_len;              // tokens the tail held before this step
+    const int hot_tokens = packs ? P : hot_len;                  // tokens the hot workgroup attends over
+    const int cold_pages = page_count - (packs ? 1 : 0);         // the page being made is the hot workgroup's
     const bool live = row_active && cache_live;
-    const bool empty = !live || (is_hot ? hot_len <= 0 : first_page >= page_count);
-    if (empty) {                                         // uniform over the workgroup
+    const bool empty = !live || (is_hot ? hot_tokens <= 0 : first_page >= cold_pages);
+    if (empty && !(appends && writes)) {                 // uniform over the workgroup
         if (tid < G) {
             a.part_max[part + (int64_t)tid * (a.chunks + 1)] = -INFINITY;
             a.part_sum[part + (int64_t)tid * (a.chunks + 1)] = 0.0f;
@@ -220,8 +305,8 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
 #pragma unroll
     for (int pass = 0; pass < kPasses; pass++) {
         const int ordinal = first_page + pass * kPagesPerPass + pass_page;
-        pass_valid[pass] = is_hot ? (pass == 0 && pass_page == 0 && token < hot_len)
-                                  : (ordinal < page_count && (ordinal < page_count - 1 || token < last_len));
+        pass_valid[pass] = is_hot ? (pass == 0 && pass_page == 0 && token < hot_tokens)
+                                  : (ordinal < cold_pages && (ordinal < cold_pages - 1 || token < last_len));
         k_code[pass] = 0u; k_ids[pass] = 0u; k_norm[pass] = 0.0f;
         v_code[pass] = 0u; v_ids[pass] = 0u; v_norm[pass] = 0.0f;
         if (!is_hot && pass_valid[pass]) {
@@ -235,60 +320,108 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
             v_norm[pass] = a.value_norms[norm];
         }
     }
-    if (is_hot && pass_valid[0]) {
+    int64_t new_page = -1;
+    if (appends) {
+        // lanes 0 .. 127 stage the tail's keys, lanes 128 .. 255 its values (lane = token * 8 + block)
+        if (tid < 2 * kTokenBlocks && token < tail_old) {
+            const int64_t at = (((int64_t)slot * P + token) * a.kv_heads + g) * D + blk * 8;
+            hot_k = *reinterpret_cast<const uint4 *>((tid < kTokenBlocks ? a.hot_keys : a.hot_values) + at);
+        }
+        if (packs) new_page = a.page_indices[(int64_t)slot * a.max_pages + (length - 1) / P];
+    } else if (is_hot && pass_valid[0]) {
         const int64_t at = (((int64_t)slot * P + token) * a.kv_heads + g) * D + blk * 8;
         hot_k = *reinterpret_cast<const uint4 *>(a.hot_keys + at);
         hot_v = *reinterpret_cast<const uint4 *>(a.hot_values + at);
     }
 
-    // the group's queries: rotary embedding ((q * cos) + (rotate_half(q) * sin) in BF16 tensor
-    // arithmetic), then optionally the Hadamard rotation (float32 butterflies over the head, scaled
-    // by 1 / sqrt(D), rounded to the query dtype: hadamard(query.float()).to(dtype),
-    // nestquant/runtime/nqkv_batched_hf_backend.py:549)
+    // the group's queries (and the new key): rotary embedding, then the Hadamard rotation
     float *q_lds = &acc_lds[0][0][0];                    // free until the V pass ends
     static_assert(sizeof(acc_lds) >= sizeof(float) * G * D, "the query staging fits the accumulator buffer");
-    if (tid < G * 8) {
-        if (a.rope_cos) {
-            const bool upper = piece >= 4;
+    if (tid < G * 8 || key_lane) {
+        rope_then_rotate(qv, rope_c, rope_s, a.rope_cos != nullptr, key_lane ? a.rotate_keys != 0 : a.rotate_query != 0,
+                         key_lane ? (int)NQ_BF16 : a.query_dtype, tid);
+        if (!key_lane) {
 #pragma unroll
-            for (int j = 0; j < 8; j += 2) {
-                const float o0 = lane_xor<4>(qv[j]), o1 = lane_xor<4>(qv[j + 1]);
-                float a0 = qv[j] * rope_c[j], a1 = qv[j + 1] * rope_c[j + 1];
-                round_pair<1>(a0, a1);
-                float b0 = o0 * rope_s[j], b1 = o1 * rope_s[j + 1];
-                round_pair<1>(b0, b1);
-                qv[j] = upper ? a0 + b0 : a0 - b0;
-                qv[j + 1] = upper ? a1 + b1 : a1 - b1;
-                round_pair<1>(qv[j], qv[j + 1]);
+            for (int j = 0; j < 8; j++) q_lds[qh * D + piece * 8 + j] = qv[j];
+        } else if (writes) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) tail[new_at][piece * 8 + j] = qv[j];
+            if (!packs) {                                // the rotated key joins the slot's hot tail
+                uint4 packed;
+                packed.x = f32_to_bf16(qv[0]) | ((uint32_t)f32_to_bf16(qv[1]) << 16);
+                packed.y = f32_to_bf16(qv[2]) | ((uint32_t)f32_to_bf16(qv[3]) << 16);
+                packed.z = f32_to_bf16(qv[4]) | ((uint32_t)f32_to_bf16(qv[5]) << 16);
+                packed.w = f32_to_bf16(qv[6]) | ((uint32_t)f32_to_bf16(qv[7]) << 16);
+                *reinterpret_cast<uint4 *>(const_cast<uint16_t *>(a.hot_keys) +
+                                           (((int64_t)slot * P + new_at) * a.kv_heads + g) * D + piece * 8) = packed;
             }
         }
-        if (a.rotate_query) {
+    }
+    if (appends && tid < 2 * kTokenBlocks) {
+        const bool of_values = tid >= kTokenBlocks;
+        const bool is_new = token == new_at;             // never for a row that writes nothing
+        if (is_new && of_values && !packs)
+            *reinterpret_cast<uint4 *>(const_cast<uint16_t *>(a.hot_values) +
+                                       (((int64_t)slot * P + new_at) * a.kv_heads + g) * D + blk * 8) = new_value;
+        if (!is_new || of_values) {                      // the new key comes from its eight lanes above
+            float x[8];
+            unpack_bf16_row(is_new ? new_value : hot_k, x);      // rows past the tail are zeros
 #pragma unroll
-            for (int s = 0; s < 3; s++) {
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    if (j & (1 << s)) continue;
-                    const float left = qv[j], right = qv[j + (1 << s)];
-                    qv[j] = left + right;
-                    qv[j + (1 << s)] = left - right;
-                }
-            }
-            lane_stage<1, 0>(qv, tid);
-            lane_stage<2, 0>(qv, tid);
-            lane_stage<4, 0>(qv, tid);
-            const float inv = 1.0f / __builtin_sqrtf((float)D);
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const float scaled = qv[j] * inv;
-                qv[j] = a.query_dtype == NQ_BF16 ? bf16_to_f32(f32_to_bf16(scaled))
-                                                 : (a.query_dtype == NQ_F16 ? (float)(_Float16)scaled : scaled);
-            }
+            for (int j = 0; j < 8; j++) tail[(of_values ? P : 0) + token][blk * 8 + j] = x[j];
         }
-#pragma unroll
-        for (int j = 0; j < 8; j++) q_lds[qh * D + piece * 8 + j] = qv[j];
     }
     __syncthreads();
     NQ_STAMP(2);
+    if constexpr (kWrites) {
+        if (packs) {
+            // the tail is a complete page: norms, codes and beta ids as the KV writer makes them, kept in
+            // LDS for this launch's attention and stored in the pool
+            const float sqrt_d = __builtin_sqrtf((float)D);
+            staged_row_norms(&tail[0][0], 2 * P, D, sqrt_d, tail_scale, tail_norm);
+            if (new_page >= 0 && tid < 2 * P)
+                const_cast<float *>(tid < P ? a.key_norms : a.value_norms)[new_page * page_rows + (tid % P) * a.kv_heads + g] =
+                    tail_norm[tid];
+            struct Sink {
+                uint32_t *key_codes, *value_codes; uint8_t *key_beta_ids, *value_beta_ids;
+                uint32_t (*code_lds)[kBlocks]; uint32_t (*ids_lds)[kBlocks / 4];
+                int64_t page_word0; int kv_heads, g; bool mapped;
+                __device__ __forceinline__ bool wants(int) const { return true; }
+                __device__ __forceinline__ int64_t word(int r, int b) const {
+                    return page_word0 + ((int64_t)(r % P) * kv_heads + g) * kBlocks + b;
+                }
+                __device__ __forceinline__ void code(int r, int b, uint32_t w, const float (&)[8], float) const {
+                    code_lds[r][b] = w;
+                    if (mapped) (r < P ? key_codes : value_codes)[word(r, b)] = w;
+                }
+                __device__ __forceinline__ void beta_byte(int r, int b, uint32_t byte) const {
+                    ids_lds[r][b >> 2] = byte;
+                    if (mapped) (r < P ? key_beta_ids : value_beta_ids)[word(r, b) >> 2] = (uint8_t)byte;
+                }
+                __device__ __forceinline__ uint32_t counter(int, int) const { return 0u; }
+            } sink{const_cast<uint32_t *>(a.key_codes), const_cast<uint32_t *>(a.value_codes),
+                   const_cast<uint8_t *>(a.key_beta_ids), const_cast<uint8_t *>(a.value_beta_ids), tail_code, tail_ids,
+                   new_page * page_words, a.kv_heads, g, new_page >= 0};
+            struct Betas {
+                const float *key, *value;
+                __device__ __forceinline__ const float *operator()(int r) const { return r < P ? key : value; }
+            } betas_of{a.key_betas, a.value_betas};
+            quantize_staged_pairs<false>(&tail[0][0], tail_scale, D, 14.0f, 1.0f / 14.0f, betas_of, a.key_beta_count,
+                                         0u, 0, 2 * P * kBlocks * 4, sink);
+            __syncthreads();
+        }
+    }
+    if (empty) {                                         // the row's cache is switched off: the append was all
+        if (tid < G) {
+            a.part_max[part + (int64_t)tid * (a.chunks + 1)] = -INFINITY;
+            a.part_sum[part + (int64_t)tid * (a.chunks + 1)] = 0.0f;
+        }
+        return;
+    }
+    if (appends && packs && pass_valid[0]) {
+        k_code[0] = tail_code[token][blk]; k_ids[0] = tail_ids[token][blk >> 2]; k_norm[0] = tail_norm[token];
+        v_code[0] = tail_code[P + token][blk]; v_ids[0] = tail_ids[P + token][blk >> 2]; v_norm[0] = tail_norm[P + token];
+    }
+    const bool bf16_rows = is_hot && !packs;             // the pass reads BF16 rows, not codes
     float q[G][8];
 #pragma unroll
     for (int h = 0; h < G; h++)
@@ -305,12 +438,14 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
         float k[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) k[j] = 0.0f;
-        if (is_hot) {
-            const uint32_t w[4] = {hot_k.x, hot_k.y, hot_k.z, hot_k.w};
+        if (bf16_rows) {
+            if (appends) {
+                if (valid) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                k[2 * j] = __uint_as_float(w[j] << 16);
-                k[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+                    for (int j = 0; j < 8; j++) k[j] = tail[token][blk * 8 + j];
+                }
+            } else {
+                unpack_bf16_row(hot_k, k);
             }
         } else if (valid) {
             decode_codeword<false>(k_code[pass], 14.0f, 0u, k);
@@ -361,12 +496,14 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
         float v[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) v[j] = 0.0f;
-        if (is_hot) {
-            const uint32_t w[4] = {hot_v.x, hot_v.y, hot_v.z, hot_v.w};
+        if (bf16_rows) {
+            if (appends) {
+                if (valid) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                v[2 * j] = __uint_as_float(w[j] << 16);
-                v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+                    for (int j = 0; j < 8; j++) v[j] = tail[P + token][blk * 8 + j];
+                }
+            } else {
+                unpack_bf16_row(hot_v, v);
             }
         } else if (valid) {
             decode_codeword<false>(v_code[pass], 14.0f, 0u, v);
@@ -490,7 +627,17 @@ extern "C" size_t nq_nqkv_attention_workspace_bytes(int batch, int q_heads, int 
     return (size_t)batch * q_heads * parts * ((size_t)head_dim + 2) * sizeof(float);
 }
 
-extern "C" int nq_nqkv_attention_decode(
+namespace {
+
+// What a launch that appends as it attends adds to the attention's operands.
+struct AppendOperands {
+    const void *key, *value;               // BF16 [batch, kv_heads, head_dim]
+    const int32_t *sequence_lengths;
+    int key_beta_count, value_beta_count, rotate_keys;
+};
+
+int launch_decode_attention(
+    const char *entry, const AppendOperands *append,
     const void *query_dev, int query_dtype, const uint8_t *key_codes_dev, const uint8_t *key_beta_ids_dev,
     const float *key_norms_dev, const uint8_t *value_codes_dev, const uint8_t *value_beta_ids_dev,
     const float *value_norms_dev, const float *key_betas_dev, const float *value_betas_dev,
@@ -501,30 +648,30 @@ extern "C" int nq_nqkv_attention_decode(
     int rotate_query, const void *rope_cos_dev, const void *rope_sin_dev, void *out_dev, void *workspace_dev,
     size_t workspace_bytes, void *stream) {
     NQ_REQUIRE(batch >= 1 && slots >= 1 && max_pages >= 1, NQ_ERR_SHAPE,
-               "nq_nqkv_attention_decode: batch, slots and max_pages must be positive");
+               "%s: batch, slots and max_pages must be positive", entry);
     NQ_REQUIRE(kv_heads >= 1 && q_heads >= kv_heads && q_heads % kv_heads == 0, NQ_ERR_SHAPE,
-               "nq_nqkv_attention_decode: q_heads must be a positive multiple of kv_heads");
+               "%s: q_heads must be a positive multiple of kv_heads", entry);
     const int group = q_heads / kv_heads;
     NQ_REQUIRE(head_dim == 64 && page_size == 16, NQ_ERR_SHAPE,
-               "nq_nqkv_attention_decode: built for head_dim 64 and 16-token pages (got %d, %d)", head_dim, page_size);
+               "%s: built for head_dim 64 and 16-token pages (got %d, %d)", entry, head_dim, page_size);
     NQ_REQUIRE(group == 1 || group == 2 || group == 4 || group == 8, NQ_ERR_SHAPE,
-               "nq_nqkv_attention_decode: %d query heads per KV head is not 1, 2, 4 or 8", group);
+               "%s: %d query heads per KV head is not 1, 2, 4 or 8", entry, group);
     NQ_REQUIRE(query_dtype == NQ_F32 || query_dtype == NQ_BF16 || query_dtype == NQ_F16, NQ_ERR_ARGUMENT,
-               "nq_nqkv_attention_decode: unknown dtype tag %d", query_dtype);
+               "%s: unknown dtype tag %d", entry, query_dtype);
     NQ_REQUIRE(query_dev && key_codes_dev && key_beta_ids_dev && key_norms_dev && value_codes_dev &&
                    value_beta_ids_dev && value_norms_dev && key_betas_dev && value_betas_dev && page_indices_dev &&
                    page_counts_dev && last_page_lens_dev && hot_lengths_dev && hot_keys_dev && hot_values_dev &&
                    slot_ids_dev && active_mask_dev,
-               NQ_ERR_ARGUMENT, "nq_nqkv_attention_decode: null pointer");
+               NQ_ERR_ARGUMENT, "%s: null pointer", entry);
     NQ_REQUIRE(nq::aligned(key_codes_dev, 4) && nq::aligned(value_codes_dev, 4) && nq::aligned(hot_keys_dev, 16) &&
                    nq::aligned(hot_values_dev, 16),
-               NQ_ERR_ARGUMENT, "nq_nqkv_attention_decode: page streams need 4-byte, hot tails 16-byte alignment");
-    NQ_REQUIRE(isfinite(scale), NQ_ERR_ARGUMENT, "nq_nqkv_attention_decode: scale must be finite");
+               NQ_ERR_ARGUMENT, "%s: page streams need 4-byte, hot tails 16-byte alignment", entry);
+    NQ_REQUIRE(isfinite(scale), NQ_ERR_ARGUMENT, "%s: scale must be finite", entry);
     NQ_REQUIRE(chunks_for(batch, max_pages) + 1 <= 512, NQ_ERR_SHAPE,
-               "nq_nqkv_attention_decode: a page table of %d pages needs more than 512 context chunks", max_pages);
+               "%s: a page table of %d pages needs more than 512 context chunks", entry, max_pages);
     const size_t need = nq_nqkv_attention_workspace_bytes(batch, q_heads, head_dim, max_pages);
     NQ_REQUIRE(workspace_dev && workspace_bytes >= need, NQ_ERR_WORKSPACE,
-               "nq_nqkv_attention_decode: needs a %zu-byte workspace, got %zu", need, workspace_bytes);
+               "%s: needs a %zu-byte workspace, got %zu", entry, need, workspace_bytes);
 
     nq::AttentionArgs a;
     a.query = query_dev;
@@ -543,11 +690,28 @@ extern "C" int nq_nqkv_attention_decode(
     a.chunks = chunks_for(batch, max_pages); a.query_dtype = query_dtype; a.scale = scale;
     a.rotate_query = rotate_query;
     NQ_REQUIRE((rope_cos_dev == nullptr) == (rope_sin_dev == nullptr), NQ_ERR_ARGUMENT,
-               "nq_nqkv_attention_decode: rotary cos and sin tables come together");
+               "%s: rotary cos and sin tables come together", entry);
     NQ_REQUIRE(!rope_cos_dev || query_dtype == NQ_BF16, NQ_ERR_ARGUMENT,
-               "nq_nqkv_attention_decode: the fused rotary embedding takes BF16 queries");
+               "%s: the fused rotary embedding takes BF16 queries", entry);
     a.rope_cos = reinterpret_cast<const uint16_t *>(rope_cos_dev);
     a.rope_sin = reinterpret_cast<const uint16_t *>(rope_sin_dev);
+    a.new_key = a.new_value = nullptr;
+    a.sequence_lengths = nullptr;
+    a.key_beta_count = 4; a.rotate_keys = 0;
+    if (append) {
+        NQ_REQUIRE(append->key && append->value && append->sequence_lengths, NQ_ERR_ARGUMENT, "%s: null pointer", entry);
+        NQ_REQUIRE(nq::aligned(append->key, 16) && nq::aligned(append->value, 16), NQ_ERR_ARGUMENT,
+                   "%s: the new keys and values need 16-byte alignment", entry);
+        NQ_REQUIRE(append->key_beta_count >= 1 && append->key_beta_count <= 4 &&
+                       append->value_beta_count == append->key_beta_count,
+                   NQ_ERR_SHAPE, "%s: key and value tables must hold the same number (1..4) of betas", entry);
+        NQ_REQUIRE(query_dtype == NQ_BF16, NQ_ERR_ARGUMENT, "%s: a step that appends takes BF16 queries, keys and values",
+                   entry);
+        a.new_key = reinterpret_cast<const uint16_t *>(append->key);
+        a.new_value = reinterpret_cast<const uint16_t *>(append->value);
+        a.sequence_lengths = append->sequence_lengths;
+        a.key_beta_count = append->key_beta_count; a.rotate_keys = append->rotate_keys;
+    }
     const size_t parts = (size_t)a.chunks + 1, heads_total = (size_t)batch * q_heads;
     a.part_max = reinterpret_cast<float *>(workspace_dev);
     a.part_sum = a.part_max + heads_total * parts;
@@ -556,23 +720,68 @@ extern "C" int nq_nqkv_attention_decode(
     hipStream_t s = (hipStream_t)stream;
     const size_t pairs = parts * (size_t)batch;                    // (row, chunk) pairs, padded to whole groups of eight
     const dim3 grid((unsigned)((pairs + 7) / 8 * 8 * kv_heads));
-#define NQ_LAUNCH_STAGE1(GROUP)                                                                                   \
+#define NQ_LAUNCH_STAGE1_AS(GROUP, PAGES, WRITES)                                                                 \
+    hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, PAGES, WRITES>), grid, dim3(nq::kAttnThreads), 0, s, a)
+#define NQ_LAUNCH_STAGE1(GROUP, WRITES)                                                                           \
     switch (pages_per_chunk_for(batch, max_pages)) {                                                              \
-        case 4: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 4>), grid, dim3(nq::kAttnThreads), 0, s, a); break;  \
-        case 8: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 8>), grid, dim3(nq::kAttnThreads), 0, s, a); break;  \
-        default: hipLaunchKernelGGL((nq::attention_stage1_kernel<64, 16, GROUP, 16>), grid, dim3(nq::kAttnThreads), 0, s, a); break; \
+        case 4: NQ_LAUNCH_STAGE1_AS(GROUP, 4, WRITES); break;                                                     \
+        case 8: NQ_LAUNCH_STAGE1_AS(GROUP, 8, WRITES); break;                                                     \
+        default: NQ_LAUNCH_STAGE1_AS(GROUP, 16, WRITES); break;                                                   \
     }
-    switch (group) {
-        case 1: NQ_LAUNCH_STAGE1(1); break;
-        case 2: NQ_LAUNCH_STAGE1(2); break;
-        case 4: NQ_LAUNCH_STAGE1(4); break;
-        default: NQ_LAUNCH_STAGE1(8); break;
+#define NQ_LAUNCH_STAGE1_GROUPS(WRITES)                                                                           \
+    switch (group) {                                                                                              \
+        case 1: NQ_LAUNCH_STAGE1(1, WRITES); break;                                                               \
+        case 2: NQ_LAUNCH_STAGE1(2, WRITES); break;                                                               \
+        case 4: NQ_LAUNCH_STAGE1(4, WRITES); break;                                                               \
+        default: NQ_LAUNCH_STAGE1(8, WRITES); break;                                                              \
     }
+    if (append) { NQ_LAUNCH_STAGE1_GROUPS(true) } else { NQ_LAUNCH_STAGE1_GROUPS(false) }
+#undef NQ_LAUNCH_STAGE1_GROUPS
 #undef NQ_LAUNCH_STAGE1
-    int status = nq::check_launch("nq_nqkv_attention_decode (stage 1)");
+#undef NQ_LAUNCH_STAGE1_AS
+    int status = nq::check_launch(entry);
     // without an output the partial results stay in the workspace for nq_attention_output_stage
     if (status != NQ_OK || out_dev == nullptr) return status;
     hipLaunchKernelGGL(nq::attention_merge_kernel<64>, dim3((unsigned)heads_total), dim3(64), 0, s,
                        a.part_max, a.part_sum, a.part_acc, (int)parts, (int64_t)heads_total, out_dev, query_dtype);
-    return nq::check_launch("nq_nqkv_attention_decode (merge)");
+    return nq::check_launch(entry);
+}
+
+}  // namespace
+
+extern "C" int nq_nqkv_attention_decode(
+    const void *query_dev, int query_dtype, const uint8_t *key_codes_dev, const uint8_t *key_beta_ids_dev,
+    const float *key_norms_dev, const uint8_t *value_codes_dev, const uint8_t *value_beta_ids_dev,
+    const float *value_norms_dev, const float *key_betas_dev, const float *value_betas_dev,
+    const int32_t *page_indices_dev, const int32_t *page_counts_dev, const int32_t *last_page_lens_dev,
+    const int32_t *hot_lengths_dev, const uint8_t *cache_active_dev, const void *hot_keys_dev,
+    const void *hot_values_dev, const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch,
+    int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
+    int rotate_query, const void *rope_cos_dev, const void *rope_sin_dev, void *out_dev, void *workspace_dev,
+    size_t workspace_bytes, void *stream) {
+    return launch_decode_attention(
+        "nq_nqkv_attention_decode", nullptr, query_dev, query_dtype, key_codes_dev, key_beta_ids_dev, key_norms_dev,
+        value_codes_dev, value_beta_ids_dev, value_norms_dev, key_betas_dev, value_betas_dev, page_indices_dev,
+        page_counts_dev, last_page_lens_dev, hot_lengths_dev, cache_active_dev, hot_keys_dev, hot_values_dev,
+        slot_ids_dev, active_mask_dev, batch, slots, max_pages, q_heads, kv_heads, head_dim, page_size, scale,
+        rotate_query, rope_cos_dev, rope_sin_dev, out_dev, workspace_dev, workspace_bytes, stream);
+}
+
+extern "C" int nq_nqkv_append_attention_decode(
+    const void *query_dev, const void *key_dev, const void *value_dev, const int32_t *sequence_lengths_dev,
+    uint8_t *key_codes_dev, uint8_t *key_beta_ids_dev, float *key_norms_dev, uint8_t *value_codes_dev,
+    uint8_t *value_beta_ids_dev, float *value_norms_dev, const float *key_betas_dev, int key_beta_count,
+    const float *value_betas_dev, int value_beta_count, const int32_t *page_indices_dev,
+    const int32_t *page_counts_dev, const int32_t *last_page_lens_dev, const int32_t *hot_lengths_dev,
+    const uint8_t *cache_active_dev, void *hot_keys_dev, void *hot_values_dev, const int32_t *slot_ids_dev,
+    const uint8_t *active_mask_dev, int batch, int slots, int max_pages, int q_heads, int kv_heads, int head_dim,
+    int page_size, float scale, int rotate, const void *rope_cos_dev, const void *rope_sin_dev, void *out_dev,
+    void *workspace_dev, size_t workspace_bytes, void *stream) {
+    const AppendOperands append{key_dev, value_dev, sequence_lengths_dev, key_beta_count, value_beta_count, rotate};
+    return launch_decode_attention(
+        "nq_nqkv_append_attention_decode", &append, query_dev, NQ_BF16, key_codes_dev, key_beta_ids_dev, key_norms_dev,
+        value_codes_dev, value_beta_ids_dev, value_norms_dev, key_betas_dev, value_betas_dev, page_indices_dev,
+        page_counts_dev, last_page_lens_dev, hot_lengths_dev, cache_active_dev, hot_keys_dev, hot_values_dev,
+        slot_ids_dev, active_mask_dev, batch, slots, max_pages, q_heads, kv_heads, head_dim, page_size, scale,
+        rotate, rope_cos_dev, rope_sin_dev, out_dev, workspace_dev, workspace_bytes, stream);
 }

@@ -4,13 +4,13 @@ The reference runs the Hugging Face module graph for a decode step: per layer ab
 small tensor kernels (residual adds, LlamaRMSNorm, rotary embedding, SiLU and multiply,
 Hadamard passes) surround the packed linears and the NQKV attention
 (nestquant/models/fused_linear.py:276-421, nestquant/runtime/nqkv_batched_hf_backend.py:357-631).
-Here the same arithmetic, in the same BF16 tensor-operation rounding, runs in ten launches
+Here the same arithmetic, in the same BF16 tensor-operation rounding, runs in nine launches
 per layer:
 
     residual add + RMSNorm + Hadamard + A4 encode      nq_fused_input_stage (mode 1)
     q_proj, k_proj, v_proj                             nq_w4a4_gemv_grouped
-    RoPE(k) + Hadamard(k) + KV append / page pack      nq_nqkv_write
-    RoPE(q) + Hadamard(q) + paged attention, stage 1   nq_nqkv_attention_decode (no output given)
+    RoPE + Hadamard of q and k, KV append / page pack,
+      paged attention, stage 1                         nq_nqkv_append_attention_decode (no output given)
     attention stage 2 + Hadamard + A4 encode           nq_attention_output_stage
     o_proj                                             nq_w4a4_gemv
     residual add + RMSNorm + Hadamard + A4 encode      nq_fused_input_stage (mode 1)
@@ -179,7 +179,6 @@ class FusedLlamaDecodeStep:
                 cache.begin_decode_step()
             embedded = inner.embed_tokens(tokens)                           # [rows, 1, hidden]
             query_rope = self._rope(embedded, positions)                    # 2 x [rows, head_dim]
-        cos, sin = query_rope[0].view(rows, 1, -1), query_rope[1].view(rows, 1, -1)
         heads, kv_heads, dim = cache.num_query_heads, cache.num_kv_heads, cache.head_dim
         workspace = cache._workspace(rows, torch.bfloat16)
 
@@ -195,13 +194,12 @@ class FusedLlamaDecodeStep:
                 query, key, value = bf16_rows_linear_grouped(activation.decoded, expanded[0], expanded[1])
             else:
                 query, key, value = self._linears(activation, [q_w, k_w, v_w])
-            manager.write_layer(index, key.view(rows, 1, kv_heads, dim), value.view(rows, 1, kv_heads, dim),
-                                rotate_keys=True, rope=(cos, sin))
-            # the attention leaves per-chunk results; o_proj's input stage merges them as it loads its rows
-            launch_nqkv_decode_attention(
-                query.view(rows, heads, dim), manager.layers[index], slot_ids=manager.step_slot_ids,
-                active_mask=manager.step_active, attention_scale=float(attention.scaling), workspace=workspace,
-                rotate_query=True, rope=query_rope, merge=False)
+            # the new token joins the cache inside the attention launch, which leaves per-chunk results;
+            # o_proj's input stage merges them as it loads its rows
+            manager.append_and_attend(
+                index, query.view(rows, heads, dim), key.view(rows, kv_heads, dim), value.view(rows, kv_heads, dim),
+                attention_scale=float(attention.scaling), workspace=workspace, rotate=True, rope=query_rope,
+                merge=False)
             o_input, _ = attention_output_stage(workspace, q=14, beta_table=table, hadamard=True)
             delta = self._linear(o_input, o_w) if expanded is None else bf16_rows_linear(o_input.decoded, expanded[2])
             activation, residual, _ = fused_input_stage(

@@ -762,6 +762,40 @@ class BatchedNQKVCacheManager:
             int(rotate_keys), None if rope is None else rope[0].data_ptr(),
             None if rope is None else rope[1].data_ptr(), _native.stream_handle(self.device)))
 
+    def append_and_attend(self, layer_index: int, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, *,
+                          attention_scale: float, workspace: BatchedNQKVAttentionWorkspace, rotate: bool = False,
+                          rope: tuple[torch.Tensor, torch.Tensor] | None = None, merge: bool = True
+                          ) -> torch.Tensor | None:
+        """One decode token per row: `write_layer` of this step's key/value rows [rows, kv_heads,
+        head_dim] and `launch_nqkv_decode_attention` of the query [rows, query_heads, head_dim] over
+        the layer in one launch (BF16; the same `rope` rows and `rotate` serve keys and queries).
+        Graph-safe: no host reads, no allocation.  Returns workspace.output, or None when `merge`
+        is false (the per-chunk results then wait in workspace.buffer for attention_output_stage)."""
+        cache = self.layers[layer_index]
+        pool, meta = cache.pool, self.metadata
+        rows, heads, dim = query.shape
+        if rows != self._step_rows or self._step_uniform != 1:
+            raise ValueError("append_and_attend takes the rows of a decode step in flight, one token each")
+        if not (query.dtype == key.dtype == value.dtype == torch.bfloat16):
+            raise TypeError("append_and_attend takes BF16 queries, keys and values")
+        if tuple(key.shape) != (rows, pool.num_kv_heads, dim) or key.shape != value.shape:
+            raise ValueError("keys and values must have shape [rows, kv_heads, head_dim]")
+        if not (query.is_contiguous() and key.is_contiguous() and value.is_contiguous()):
+            raise ValueError("queries, keys and values must be contiguous")
+        _native.check(_native.library().nq_nqkv_append_attention_decode(
+            query.data_ptr(), key.data_ptr(), value.data_ptr(), meta.sequence_lengths.data_ptr(),
+            pool.key_codes.data_ptr(), pool.key_betas.data_ptr(), pool.key_norms.data_ptr(),
+            pool.value_codes.data_ptr(), pool.value_betas.data_ptr(), pool.value_norms.data_ptr(),
+            pool.beta_table.data_ptr(), pool.beta_table.numel(), pool.value_beta_table.data_ptr(),
+            pool.value_beta_table.numel(), meta.page_indices.data_ptr(), meta.page_counts.data_ptr(),
+            meta.last_page_lens.data_ptr(), meta.hot_lengths.data_ptr(), meta.active_mask.data_ptr(),
+            cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(), self.step_slot_ids.data_ptr(),
+            self.step_active.data_ptr(), rows, self.capacity, self.max_pages, heads, pool.num_kv_heads, dim,
+            self.page_size, attention_scale, int(rotate), None if rope is None else rope[0].data_ptr(),
+            None if rope is None else rope[1].data_ptr(), workspace.output.data_ptr() if merge else None,
+            workspace.buffer.data_ptr(), workspace.buffer.numel(), _native.stream_handle(self.device)))
+        return workspace.output if merge else None
+
     def resident_bytes(self) -> int:
         total = 0
         for cache in self.layers:

@@ -479,3 +479,79 @@ def test_decode_step_begin_is_advance_plus_two_gathers():
     reference[~known] = 0
     assert torch.equal(embedded.view(torch.int16), reference.view(torch.int16))
     assert torch.equal(rotary_rows, rotary.index_select(1, positions.view(-1).clamp(0, max_pos - 1)))
+
+
+@pytest.mark.parametrize("q_heads,max_len,steps", [(32, 256, 40), (8, 256, 20), (64, 64, 34), (16, 1024, 20)])
+def test_append_inside_the_attention_launch_equals_writer_then_attention(kv, oracle, q_heads, max_len, steps):
+    """One launch per layer and decode step (`append_and_attend`) against the two it replaces
+    (`write_layer`, then `launch_nqkv_decode_attention`), on two caches fed the same tokens: after
+    every step the pools, hot tails and tables are bit for bit the same.  The attention rows are
+    bit for bit the same on steps where the row's token does not complete a page; where it does,
+    the fused launch merges that page as a part of its own, so the rows agree to the rounding of the
+    BF16 result.  Covers rows that complete pages at different steps, a row that is not in the
+    step, a slot whose cache is switched off for some steps (it still appends), RoPE(theta = 500000)
+    on keys and queries, and (max_len 64) a slot that reaches its capacity."""
+    rng = np.random.default_rng(700 + q_heads)
+    slots, lengths = [3, 0, 2, 1], [5, 16, 37, 9]
+    if max_len == 1024:
+        lengths = [700, 16, 1003, 9]                  # chunks of eight pages; one row ends near the table's end
+    rows = len(slots)
+    managers = [_manager(kv, capacity=4, max_len=max_len) for _ in range(2)]
+    keys = [_bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for n in lengths]
+    values = [_bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for n in lengths]
+    for manager in managers:
+        for s in slots:
+            manager.register(f"seq{s}", slot=s)
+        _append(manager, slots, keys, values)
+    workspaces = [kv.BatchedNQKVAttentionWorkspace.create(m.layers[0], batch_size=rows, query_heads=q_heads,
+                                                          output_dtype=torch.bfloat16) for m in managers]
+    totals = list(lengths)
+    for step in range(steps):
+        in_step = [True, True, True, step % 5 != 3]                  # the last row sits out every fifth step
+        cache_on = not (7 <= step < 11)                              # slot 0's cache is off for four steps
+        key = _bf16(rng.standard_normal((rows, HEADS, DIM)).astype(np.float32)).cuda()
+        value = _bf16(rng.standard_normal((rows, HEADS, DIM)).astype(np.float32)).cuda()
+        query = _bf16(rng.standard_normal((rows, q_heads, DIM)).astype(np.float32)).cuda()
+        positions = np.asarray(totals, dtype=np.float64)
+        angles = positions[:, None] * (500000.0 ** (-np.arange(0, DIM, 2) / DIM))[None, :]
+        cos = _bf16(np.concatenate([np.cos(angles)] * 2, axis=1).astype(np.float32)).cuda()
+        sin = _bf16(np.concatenate([np.sin(angles)] * 2, axis=1).astype(np.float32)).cuda()
+        packs = []
+        for i in range(rows):
+            grows = in_step[i] and totals[i] < managers[0].max_tokens
+            totals[i] += 1 if grows else 0
+            packs.append(in_step[i] and totals[i] % PAGE == 0)
+        outputs = []
+        for which, (manager, workspace) in enumerate(zip(managers, workspaces)):
+            manager.step_slot_ids[:rows] = torch.tensor(slots, dtype=torch.int32)
+            manager.step_active[:rows] = torch.tensor(in_step)
+            manager.metadata.active_mask[0] = cache_on
+            manager.begin_step(rows=rows, uniform_count=1)
+            if which == 0:
+                manager.write_layer(0, key.view(rows, 1, HEADS, DIM), value.view(rows, 1, HEADS, DIM), rotate_keys=True,
+                                    rope=(cos.view(rows, 1, DIM), sin.view(rows, 1, DIM)))
+                out = kv.launch_nqkv_decode_attention(query, manager.layers[0], slot_ids=manager.step_slot_ids,
+                                                      active_mask=manager.step_active, attention_scale=0.125,
+                                                      workspace=workspace, rotate_query=True, rope=(cos, sin))
+            else:
+                out = manager.append_and_attend(0, query, key, value, attention_scale=0.125, workspace=workspace,
+                                                rotate=True, rope=(cos, sin))
+            outputs.append(out.clone())
+        torch.cuda.synchronize()
+        two, one = outputs
+        for i in range(rows):
+            if packs[i]:
+                assert relative_error(_f32(one[i]), _f32(two[i])) <= 2.0 ** -7, (step, i)
+            else:
+                assert torch.equal(one[i], two[i]), (step, i)
+        if not cache_on:
+            assert not one[1].any()                                  # slot 0 is row 1
+        a, b = managers
+        for name in ("sequence_lengths", "page_counts", "last_page_lens", "hot_lengths"):
+            assert torch.equal(getattr(a.metadata, name), getattr(b.metadata, name)), (step, name)
+        assert [a.total_tokens(s) for s in slots] == totals
+        for name in ("key_codes", "key_betas", "key_norms", "value_codes", "value_betas", "value_norms"):
+            assert torch.equal(getattr(a.layers[0].pool, name), getattr(b.layers[0].pool, name)), (step, name)
+        assert torch.equal(a.layers[0].hot_keys, b.layers[0].hot_keys), step
+        assert torch.equal(a.layers[0].hot_values, b.layers[0].hot_values), step
+    assert any(t % PAGE < steps for t in totals)                     # pages were completed on the way
