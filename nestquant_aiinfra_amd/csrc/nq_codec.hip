@@ -135,10 +135,11 @@ __device__ __forceinline__ void stage_with_prologue(const uint16_t *__restrict__
     const uint4 zero = make_uint4(0, 0, 0, 0);
     if (kPrologue == 3) {
         // one lane per eight output dimensions of one head: out = sum_c acc_c w_c / sum_c sum_c w_c with
-        // w_c = exp(max_c - max).  Online over batches of eight chunks whose maxima, sums and numerators
-        // are all requested before the first is used (one memory latency per batch, not per chunk);
-        // chunks without tokens carry no numerator (their entry is read, never used) and weigh nothing.
-        constexpr int kBatch = 8;
+        // w_c = exp(max_c - max).  Online over batches of four chunks (the batch of lane_prologue, so
+        // that both encoders round alike) whose maxima, sums and numerators are all requested before
+        // the first is used (one memory latency per batch, not per chunk); chunks without tokens carry
+        // no numerator (their entry is read, never used) and weigh nothing.
+        constexpr int kBatch = 4;
         const float kNone = -__builtin_inff();
         for (int v = tid; v < vectors; v += blockDim.x) {
             const int64_t g = first + (int64_t)v * 8;
@@ -425,30 +426,34 @@ __device__ __forceinline__ void lane_prologue(const uint16_t *__restrict__ x, co
     const int chunk = threadIdx.x;
     const int64_t g = row * n + 8 * chunk;
     if (kPrologue == 3) {
-        constexpr int kBatch = 8;
+        // Parts are taken four at a time, and the next four are requested before the current four are
+        // used: the workspace was written by the previous launch on other XCDs, so a round of loads
+        // costs over a microsecond and the rounds of a long table would otherwise add up.
+        constexpr int kBatch = 4;
         const float kNone = -__builtin_inff();
 #pragma unroll
         for (int j = 0; j < 8; j++) y[j] = 0.0f;
         const int64_t head = row * pro.heads + (chunk >> 3);      // eight lanes per head of 64
         const float *m = pro.part_max + head * pro.parts, *sum = pro.part_sum + head * pro.parts;
         const float *acc = pro.part_acc + head * pro.parts * 64 + 8 * (chunk & 7);
-        float top = kNone, denom = 0.0f;
-        for (int c0 = 0; c0 < pro.parts; c0 += kBatch) {
-            float mc[kBatch], sc[kBatch];
-            float4 lo[kBatch], hi[kBatch];
+        struct Batch { float mc[kBatch], sc[kBatch]; float4 lo[kBatch], hi[kBatch]; };
+        const auto request = [&](int c0, Batch &b) {
 #pragma unroll
             for (int j = 0; j < kBatch; j++) {
                 const int c = min(c0 + j, pro.parts - 1);
-                mc[j] = m[c];
-                sc[j] = sum[c];
-                lo[j] = *reinterpret_cast<const float4 *>(acc + (int64_t)c * 64);
-                hi[j] = *reinterpret_cast<const float4 *>(acc + (int64_t)c * 64 + 4);
+                b.mc[j] = m[c];
+                b.sc[j] = sum[c];
+                b.lo[j] = *reinterpret_cast<const float4 *>(acc + (int64_t)c * 64);
+                b.hi[j] = *reinterpret_cast<const float4 *>(acc + (int64_t)c * 64 + 4);
             }
+        };
+        float top = kNone, denom = 0.0f;
+        const auto fold = [&](int c0, Batch &b) {
             float batch_top = kNone;
 #pragma unroll
             for (int j = 0; j < kBatch; j++) {
-                if (c0 + j >= pro.parts) sc[j] = 0.0f;
-                batch_top = fmaxf(batch_top, mc[j]);
+                if (c0 + j >= pro.parts) b.sc[j] = 0.0f;
+                batch_top = fmaxf(batch_top, b.mc[j]);
             }
             const float next_top = fmaxf(top, batch_top);
             if (next_top > kNone) {
@@ -458,16 +463,25 @@ __device__ __forceinline__ void lane_prologue(const uint16_t *__restrict__ x, co
                 for (int i = 0; i < 8; i++) y[i] = y[i] * keep;
 #pragma unroll
                 for (int j = 0; j < kBatch; j++) {
-                    const float w = sc[j] > 0.0f ? __expf(mc[j] - next_top) : 0.0f;
-                    denom = denom + sc[j] * w;
+                    const float w = b.sc[j] > 0.0f ? __expf(b.mc[j] - next_top) : 0.0f;
+                    denom = denom + b.sc[j] * w;
                     const bool used = w > 0.0f;
-                    y[0] += used ? lo[j].x * w : 0.0f; y[1] += used ? lo[j].y * w : 0.0f;
-                    y[2] += used ? lo[j].z * w : 0.0f; y[3] += used ? lo[j].w * w : 0.0f;
-                    y[4] += used ? hi[j].x * w : 0.0f; y[5] += used ? hi[j].y * w : 0.0f;
-                    y[6] += used ? hi[j].z * w : 0.0f; y[7] += used ? hi[j].w * w : 0.0f;
+                    y[0] += used ? b.lo[j].x * w : 0.0f; y[1] += used ? b.lo[j].y * w : 0.0f;
+                    y[2] += used ? b.lo[j].z * w : 0.0f; y[3] += used ? b.lo[j].w * w : 0.0f;
+                    y[4] += used ? b.hi[j].x * w : 0.0f; y[5] += used ? b.hi[j].y * w : 0.0f;
+                    y[6] += used ? b.hi[j].z * w : 0.0f; y[7] += used ? b.hi[j].w * w : 0.0f;
                 }
                 top = next_top;
             }
+        };
+        Batch even, odd;
+        request(0, even);
+        for (int c0 = 0; c0 < pro.parts; c0 += 2 * kBatch) {
+            if (c0 + kBatch < pro.parts) request(c0 + kBatch, odd);
+            fold(c0, even);
+            if (c0 + kBatch >= pro.parts) break;
+            if (c0 + 2 * kBatch < pro.parts) request(c0 + 2 * kBatch, even);
+            fold(c0 + kBatch, odd);
         }
 #pragma unroll
         for (int j = 0; j < 8; j += 2) {
