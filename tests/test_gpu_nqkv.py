@@ -481,7 +481,8 @@ def test_decode_step_begin_is_advance_plus_two_gathers():
     assert torch.equal(rotary_rows, rotary.index_select(1, positions.view(-1).clamp(0, max_pos - 1)))
 
 
-@pytest.mark.parametrize("q_heads,max_len,steps", [(32, 256, 40), (8, 256, 20), (64, 64, 34), (16, 1024, 20)])
+@pytest.mark.parametrize("q_heads,max_len,steps", [(32, 256, 40), (8, 256, 20), (64, 64, 34), (16, 1024, 20),
+                                                   (32, 2048, 20), (32, 16384, 18)])
 def test_append_inside_the_attention_launch_equals_writer_then_attention(kv, oracle, q_heads, max_len, steps):
     """One launch per layer and decode step (`append_and_attend`) against the two it replaces
     (`write_layer`, then `launch_nqkv_decode_attention`), on two caches fed the same tokens: after
@@ -490,11 +491,12 @@ def test_append_inside_the_attention_launch_equals_writer_then_attention(kv, ora
     the fused launch merges that page as a part of its own, so the rows agree to the rounding of the
     BF16 result.  Covers rows that complete pages at different steps, a row that is not in the
     step, a slot whose cache is switched off for some steps (it still appends), RoPE(theta = 500000)
-    on keys and queries, and (max_len 64) a slot that reaches its capacity."""
+    on keys and queries, (max_len 64) a slot that reaches its capacity, and tables wide enough for
+    chunks of 8 and 16 pages."""
     rng = np.random.default_rng(700 + q_heads)
     slots, lengths = [3, 0, 2, 1], [5, 16, 37, 9]
-    if max_len == 1024:
-        lengths = [700, 16, 1003, 9]                  # chunks of eight pages; one row ends near the table's end
+    if max_len >= 1024:                               # chunks of 4, 8 and 16 pages; one row ends near the table's end
+        lengths = [max_len * 11 // 16 + 12, 16, max_len - 21, 9]
     rows = len(slots)
     managers = [_manager(kv, capacity=4, max_len=max_len) for _ in range(2)]
     keys = [_bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for n in lengths]
