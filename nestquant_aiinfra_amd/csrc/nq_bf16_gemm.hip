@@ -61,6 +61,94 @@ __device__ __forceinline__ void issue_order(int) {
     issue_order_groups<kGroups, kReads, kMoves>();
 }
 
+// The wavefront's tiles go to C.  The products are taken as B A^T (the weight fragment is the matrix
+// instruction's first operand), so accumulator r of lane l belongs to row l % 32 and column
+// (r % 4) + 8 (r / 4) + 4 (l / 32) of its 32 x 32 tile: four neighbouring columns per lane and group of
+// four accumulators, which leave as one 8-byte piece of BF16 (16 bytes of a float32 partial result).
+// With one column per lane (A B^T) the same tile took 16 two-byte stores per lane instead of 4 wide
+// ones, and the store instructions of a 256 x 128 tile took 7 us of the 44 us its workgroup ran.
+template <int WM, int WN>
+__device__ __forceinline__ void store_tiles(const gemm_floatx16 (&acc)[WM][WN], int row0, int col0, int lane,
+                                            uint16_t *__restrict__ c, float *__restrict__ partial, int m_size,
+                                            int n_size) {
+    const bool wide = (n_size & 3) == 0 && (reinterpret_cast<uintptr_t>(c) & 7) == 0 &&
+                      (reinterpret_cast<uintptr_t>(partial) & 15) == 0;
+#pragma unroll
+    for (int i = 0; i < WM; i++) {
+        const int row = row0 + 32 * i + (lane & 31);
+        if (row >= m_size) continue;
+#pragma unroll
+        for (int j = 0; j < WN; j++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int col = col0 + 32 * j + 8 * g + 4 * (lane >> 5);
+                const float v0 = acc[i][j][4 * g], v1 = acc[i][j][4 * g + 1], v2 = acc[i][j][4 * g + 2],
+                            v3 = acc[i][j][4 * g + 3];
+                const int64_t at = (int64_t)row * n_size + col;
+                if (wide && col + 3 < n_size) {
+                    if (partial) {
+                        *reinterpret_cast<float4 *>(partial + at) = make_float4(v0, v1, v2, v3);
+                    } else {
+                        uint2 packed;
+                        packed.x = __builtin_bit_cast(uint32_t, pack_bf16x2(v0, v1));
+                        packed.y = __builtin_bit_cast(uint32_t, pack_bf16x2(v2, v3));
+                        *reinterpret_cast<uint2 *>(c + at) = packed;
+                    }
+                } else {
+                    const float v[4] = {v0, v1, v2, v3};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (col + e >= n_size) continue;
+                        if (partial) partial[at + e] = v[e];
+                        else c[at + e] = dense_f32_to_bf16(v[e]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// The same tiles as BF16 by way of LDS, for whole rows of C: the wavefront parks its 32 WM x 32 WN
+// values in `stage` (its own 2048 WM WN bytes, rows of 64 WN bytes whose 16-byte pieces sit at
+// piece ^ (row % pieces)), then every lane takes one piece and the wavefront stores whole rows of its
+// tile: 64 WN contiguous bytes per row instead of 16, a quarter of the requests to the L2 (which,
+// with every workgroup of a round storing at once, is what the direct form waits for: 3.5 us per
+// 256 x 128 tile against 7 us with two-byte stores).  Needs rows of C that are multiples of 16 bytes.
+template <int WM, int WN>
+__device__ __forceinline__ void store_tiles_by_rows(const gemm_floatx16 (&acc)[WM][WN], int row0, int col0, int lane,
+                                                    uint16_t *__restrict__ c, int m_size, int n_size,
+                                                    u32x4 *__restrict__ stage) {
+    constexpr int kPieces = 4 * WN;                                // 16-byte pieces per row of the wavefront's tile
+    uint2 *halves = reinterpret_cast<uint2 *>(stage);
+#pragma unroll
+    for (int i = 0; i < WM; i++) {
+        const int row = 32 * i + (lane & 31);
+#pragma unroll
+        for (int j = 0; j < WN; j++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                uint2 packed;
+                packed.x = __builtin_bit_cast(uint32_t, pack_bf16x2(acc[i][j][4 * g], acc[i][j][4 * g + 1]));
+                packed.y = __builtin_bit_cast(uint32_t, pack_bf16x2(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]));
+                const int piece = (4 * j + g) ^ (row & (kPieces - 1));
+                halves[(row * kPieces + piece) * 2 + (lane >> 5)] = packed;
+            }
+        }
+    }
+    // the pieces are read by other lanes than wrote them: LDS serves a wavefront's accesses in order,
+    // and the compiler must keep them in this order too
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    constexpr int kRowsPerStore = 64 / kPieces;
+#pragma unroll
+    for (int pass = 0; pass < 32 * WM / kRowsPerStore; pass++) {
+        const int row = pass * kRowsPerStore + lane / kPieces, piece = lane % kPieces;
+        const u32x4 value = stage[row * kPieces + (piece ^ (row & (kPieces - 1)))];
+        const int out_row = row0 + row, out_col = col0 + 8 * piece;
+        if (out_row < m_size && out_col < n_size)                   // n_size is a multiple of 8 here
+            *reinterpret_cast<u32x4 *>(c + (int64_t)out_row * n_size + out_col) = value;
+    }
+}
+
 // WM x WN: 32 x 32 tiles per wavefront; GM x GN: wavefronts per workgroup along M and N.
 template <int WM, int WN, int GM, int GN>
 __global__ void __launch_bounds__(64 * GM * GN)
@@ -176,7 +264,7 @@ bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b,
             for (int i = 0; i < WM; i++)
 #pragma unroll
                 for (int j = 0; j < WN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[s & 1][j], fa[s & 1][i], acc[i][j], 0, 0, 0);
         }
         // (after the last step this stores a slab nobody reads, into the buffer nobody is reading)
 #pragma unroll
@@ -194,25 +282,13 @@ bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b,
         dense_step(step + 1, pa1, pb1, pa0, pb0);
     }
 
-    // accumulator r of lane l: row (r % 4) + 8 (r / 4) + 4 (l / 32) of the 32 x 32 tile, column l % 32
-#pragma unroll
-    for (int i = 0; i < WM; i++) {
-        const int row_base = m0 + wave_m * 32 * WM + 32 * i + 4 * frag_half;
-#pragma unroll
-        for (int j = 0; j < WN; j++) {
-            const int col = n0 + wave_n * 32 * WN + 32 * j + frag_row;
-            if (col < n_size) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int row = row_base + (r & 3) + 8 * (r >> 2);
-                    if (row < m_size) {
-                        if (partials) partials[((int64_t)blockIdx.y * m_size + row) * n_size + col] = acc[i][j][r];
-                        else c[(int64_t)row * n_size + col] = dense_f32_to_bf16(acc[i][j][r]);
-                    }
-                }
-            }
-        }
-    }
+    // (the last step's barrier has passed: nobody reads the slabs any more)
+    if (!partials && (n_size & 7) == 0 && (reinterpret_cast<uintptr_t>(c) & 15) == 0)
+        store_tiles_by_rows<WM, WN>(acc, m0 + wave_m * 32 * WM, n0 + wave_n * 32 * WN, lane, c, m_size, n_size,
+                                    lds + wave * (128 * WM * WN));
+    else
+        store_tiles<WM, WN>(acc, m0 + wave_m * 32 * WM, n0 + wave_n * 32 * WN, lane, c,
+                            partials ? partials + (int64_t)blockIdx.y * m_size * n_size : nullptr, m_size, n_size);
 }
 
 
@@ -349,29 +425,18 @@ bf16_gemm_roles_kernel(const uint16_t *__restrict__ a, const uint16_t *__restric
             for (int i = 0; i < WM; i++)
 #pragma unroll
                 for (int j = 0; j < WN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[s & 1][j], fa[s & 1][i], acc[i][j], 0, 0, 0);
         }
         issue_order<WM * WN, 3 * (WM + WN), 0>(WM + WN);
         lds_barrier();                                             // every fragment of the stage has arrived
     }
-#pragma unroll
-    for (int i = 0; i < WM; i++) {
-        const int row_base = m0 + wave_m * 32 * WM + 32 * i + 4 * frag_half;
-#pragma unroll
-        for (int j = 0; j < WN; j++) {
-            const int col = n0 + wave_n * 32 * WN + 32 * j + frag_row;
-            if (col < n_size) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int row = row_base + (r & 3) + 8 * (r >> 2);
-                    if (row < m_size) {
-                        if (partials) partials[((int64_t)blockIdx.y * m_size + row) * n_size + col] = acc[i][j][r];
-                        else c[(int64_t)row * n_size + col] = dense_f32_to_bf16(acc[i][j][r]);
-                    }
-                }
-            }
-        }
-    }
+    // (the last step's barrier has passed: nobody reads the slabs any more)
+    if (!partials && (n_size & 7) == 0 && (reinterpret_cast<uintptr_t>(c) & 15) == 0)
+        store_tiles_by_rows<WM, WN>(acc, m0 + wave_m * 32 * WM, n0 + wave_n * 32 * WN, lane, c, m_size, n_size,
+                                    lds + wave * (128 * WM * WN));
+    else
+        store_tiles<WM, WN>(acc, m0 + wave_m * 32 * WM, n0 + wave_n * 32 * WN, lane, c,
+                            partials ? partials + (int64_t)blockIdx.y * m_size * n_size : nullptr, m_size, n_size);
 }
 
 }  // namespace nq
