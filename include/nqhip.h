@@ -286,7 +286,9 @@ int nq_w4a4_decode_weight(const uint8_t *w_codes_dev, const uint8_t *w_beta_ids_
  * Dense BF16 GEMM on the matrix cores: c[m, n] = sum_k a[m, k] b[n, k], a [M, K] and b [N, K]
  * row-major BF16 (16-byte aligned), FP32 accumulation, c [M, N] BF16.  K a multiple of 128.
  * tile = -1 lets the library choose the workgroup tile from the shape; 0..6 force
- * 256x256, 128x256, 256x128, 128x128, 64x128, 128x64, 64x64 (for measurements).
+ * 256x256, 128x256, 256x128, 128x128, 64x128, 128x64, 64x64, and 7..9 the 128x128, 64x128 and
+ * 64x64 tiles on the kernel that splits its wavefronts into movers and multipliers, which the
+ * library takes by itself when every compute unit gets at most one tile (for measurements).
  * A product with few tiles (a few hundred rows) is split along K into 2, 4 or 8 slabs whose
  * float32 partial results meet in a second launch: split_k = 0 lets the library decide, 1 forbids
  * it, 2 / 4 / 8 force it (K a multiple of 128 split_k).  The partial results need

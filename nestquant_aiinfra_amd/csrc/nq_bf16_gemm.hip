@@ -443,18 +443,24 @@ bf16_gemm_roles_kernel(const uint16_t *__restrict__ a, const uint16_t *__restric
 
 namespace {
 
-struct DenseTile { int bm, bn; float efficiency; };
+struct DenseTile { int bm, bn; float efficiency, alone; };
 
 // Workgroup tiles from the fastest per product to the slowest; `efficiency` is the measured rate
 // relative to the 256 x 256 tile on a problem that fills the chip (8192^3: 1.13, 0.92, 0.99, 0.93,
-// 0.74, 0.74, 0.61 PFLOP/s).  The 256 x 128 tile runs on the kernel with movers and multipliers
-// (0.94 PFLOP/s with every wavefront doing both; the same split gave 0.87 against 0.92 at 128 x 128,
-// which keeps the plain kernel).  All of them sit at the LDS's 128 bytes per clock: a wavefront that
-// owns 2 x 4 tiles reads 0.75 KB of fragments per matrix instruction, which with the stores of the
-// next slab is about 125 bytes per clock at full matrix rate.
+// 0.74, 0.74, 0.61 PFLOP/s).  The 256 x 128 tile always runs on the kernel with movers and
+// multipliers (0.94 PFLOP/s with every wavefront doing both).  For 128 x 128, 64 x 128 and 64 x 64
+// that kernel's three LDS stages leave room for one workgroup per compute unit where the plain
+// kernel fits two or more, so it loses when a product has more tiles than compute units (M = 1024,
+// N = 8192, K = 2048 at 128 x 128: 52 against 45 us) and wins when every compute unit holds at
+// most one tile, because it keeps five slabs in flight instead of two and a lone workgroup is bound
+// by the latency of its loads (M = 384, same N and K: 24.6 against 27.7 us; M = 128 at 64 x 64:
+// 16.5 against 20.1 us): `alone` is the rate in that case, 0 where the plain kernel stays.
+// All of them sit at the LDS's 128 bytes per clock: a wavefront that owns 2 x 4 tiles reads 0.75 KB
+// of fragments per matrix instruction, which with the stores of the next slab is about 125 bytes
+// per clock at full matrix rate.
 const DenseTile kDenseTiles[] = {
-    {256, 256, 1.00f}, {128, 256, 0.81f}, {256, 128, 0.89f}, {128, 128, 0.82f}, {64, 128, 0.65f}, {128, 64, 0.65f},
-    {64, 64, 0.55f},
+    {256, 256, 1.00f, 0.0f}, {128, 256, 0.81f, 0.0f}, {256, 128, 0.89f, 0.0f}, {128, 128, 0.82f, 0.92f},
+    {64, 128, 0.65f, 0.73f}, {128, 64, 0.65f, 0.0f},  {64, 64, 0.55f, 0.67f},
 };
 
 template <int WM, int WN, int GM, int GN>
@@ -523,25 +529,41 @@ int launch_bf16_gemm(const void *a, const void *b, void *c, int m, int n, int k,
                     split, split * 128, (size_t)split * m * n * sizeof(float));
     int best = 0;
     float best_cost = 0.0f;
+    bool best_alone = false;
     const int count = (int)(sizeof(kDenseTiles) / sizeof(kDenseTiles[0]));
     for (int t = 0; t < count; t++) {
         const DenseTile &tile = kDenseTiles[t];
         const int64_t tiles = (int64_t)((m + tile.bm - 1) / tile.bm) * ((n + tile.bn - 1) / tile.bn) * split;
         // the busiest of the 256 compute units works through ceil(tiles / 256) tiles, whether one
         // after the other or side by side at a share of its rate
-        const float cost = (float)((tiles + 255) / 256) * (float)(tile.bm * tile.bn) / tile.efficiency;
-        if (t == 0 || cost < best_cost) { best = t; best_cost = cost; }
+        const bool alone = tiles <= 256 && tile.alone > 0.0f;
+        const float cost = (float)((tiles + 255) / 256) * (float)(tile.bm * tile.bn) / (alone ? tile.alone : tile.efficiency);
+        if (t == 0 || cost < best_cost) { best = t; best_cost = cost; best_alone = alone; }
     }
-    if (forced_tile >= 0 && forced_tile < count) best = forced_tile;
+    // measurements may force a tile: 0..6 the table's entries on their usual kernel, 7..9 the 128 x 128,
+    // 64 x 128 and 64 x 64 tiles on the kernel with movers and multipliers
+    if (forced_tile >= 0 && forced_tile < count) { best = forced_tile; best_alone = false; }
+    if (forced_tile == 7) { best = 3; best_alone = true; }
+    if (forced_tile == 8) { best = 4; best_alone = true; }
+    if (forced_tile == 9) { best = 6; best_alone = true; }
     float *p = reinterpret_cast<float *>(partials);
     switch (best) {
         case 0: launch_dense<2, 4, 4, 2>(a, b, c, m, n, k, split, p, stream); break;
         case 1: launch_dense<2, 4, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
         case 2: launch_roles<4, 2>(a, b, c, m, n, k, split, p, stream); break;      // movers and multipliers
-        case 3: launch_dense<2, 2, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
-        case 4: launch_dense<1, 2, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
+        case 3:
+            if (best_alone) launch_roles<2, 2>(a, b, c, m, n, k, split, p, stream);
+            else launch_dense<2, 2, 2, 2>(a, b, c, m, n, k, split, p, stream);
+            break;
+        case 4:
+            if (best_alone) launch_roles<1, 2>(a, b, c, m, n, k, split, p, stream);
+            else launch_dense<1, 2, 2, 2>(a, b, c, m, n, k, split, p, stream);
+            break;
         case 5: launch_dense<2, 1, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
-        default: launch_dense<1, 1, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
+        default:
+            if (best_alone) launch_roles<1, 1>(a, b, c, m, n, k, split, p, stream);
+            else launch_dense<1, 1, 2, 2>(a, b, c, m, n, k, split, p, stream);
+            break;
     }
     const int status = check_launch("nq_bf16_gemm");
     if (status != NQ_OK || split == 1) return status;
@@ -562,7 +584,7 @@ extern "C" int nq_bf16_gemm(const void *a_bf16_dev, const void *b_bf16_dev, int6
                "nq_bf16_gemm: operands must be 16-byte aligned");
     NQ_REQUIRE(m * k < ((int64_t)1 << 31) && n * k < ((int64_t)1 << 31), NQ_ERR_SHAPE,
                "nq_bf16_gemm: operands of 2^31 elements or more are not supported");
-    NQ_REQUIRE(tile >= -1 && tile <= 6, NQ_ERR_ARGUMENT, "nq_bf16_gemm: tile must be -1 (automatic) or 0..6");
+    NQ_REQUIRE(tile >= -1 && tile <= 9, NQ_ERR_ARGUMENT, "nq_bf16_gemm: tile must be -1 (automatic) or 0..9");
     NQ_REQUIRE(split_k == 0 || split_k == 1 || split_k == 2 || split_k == 4 || split_k == 8, NQ_ERR_ARGUMENT,
                "nq_bf16_gemm: split_k must be 0 (automatic), 1, 2, 4 or 8");
     NQ_REQUIRE(!workspace_dev || nq::aligned(workspace_dev, 16), NQ_ERR_ARGUMENT, "nq_bf16_gemm: workspace must be 16-byte aligned");
