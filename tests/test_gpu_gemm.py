@@ -150,16 +150,18 @@ def test_long_prefill_decodes_the_weight_once(rt, oracle, k, n_out):
 
 
 @pytest.mark.parametrize("m,n,k", [(300, 200, 128), (257, 520, 384), (64, 64, 128), (1000, 72, 256), (384, 8192, 2048),
-                                   (384, 2048, 8192), (130, 136, 1024)])
+                                   (384, 2048, 8192), (130, 136, 1024), (100, 36, 128), (70, 33, 256), (33, 12, 128)])
 def test_dense_bf16_gemm_against_float32(rt, m, n, k):
     """nq_bf16_gemm (the multiply of the decode-once route) against the FP32 product of the same BF16
     operands: FP32 accumulation and one BF16 rounding of the result leave <= 2^-8 relative to the
-    largest output; every workgroup tile shape, ragged edges included."""
+    largest output; every workgroup tile shape on both kernels (7..9: the small tiles on the kernel
+    with movers and multipliers), ragged edges included, and rows of C that are multiples of 16 bytes
+    (stored by whole rows through LDS), of 8 bytes (four columns per lane) and of neither."""
     g = torch.Generator().manual_seed(m + n + k)
     a = torch.randn(m, k, generator=g).to(torch.bfloat16).cuda()
     b = torch.randn(n, k, generator=g).to(torch.bfloat16).cuda()
     ref = bits(a.float() @ b.float().t())
-    for tile in range(-1, 7):
+    for tile in range(-1, 10):
         c = rt.bf16_gemm(a, b, tile=tile)
         assert c.dtype == torch.bfloat16 and tuple(c.shape) == (m, n)
         assert relative_error(bits(c.float()), ref) <= 2.0 ** -8, (tile,)
@@ -169,7 +171,7 @@ def test_dense_bf16_gemm_against_float32(rt, m, n, k):
             with pytest.raises(RuntimeError, match="K split"):
                 rt.bf16_gemm(a, b, split_k=split)
             continue
-        for tile in (-1, 3, 6):
+        for tile in (-1, 3, 6, 7, 9):
             c = rt.bf16_gemm(a, b, tile=tile, split_k=split)
             assert relative_error(bits(c.float()), ref) <= 2.0 ** -8, (tile, split)
     assert torch.equal(rt.bf16_gemm(a, b, split_k=1), rt.bf16_gemm(a, b, split_k=1))
