@@ -293,13 +293,26 @@ __device__ __forceinline__ uint32_t mad_u32(uint32_t x, uint32_t c, uint64_t a) 
     return (uint32_t)r;
 }
 
-// Keeps the compiler from merging a shift with the shifts applied to its result.
-__device__ __forceinline__ uint32_t as_computed(uint32_t x) {
-    asm("" : "+v"(x));
-    return x;
-}
-
 __device__ __forceinline__ uint32_t resolved_beta_id(uint32_t lo) { return lo & 3u; }
+
+// The four products beta_i * (row scale * kResolvedUnit) a lane keeps for its row, and the block's
+// scale out of them: two compares and three selects on the id's bits.  (The empty asm keeps the four
+// in registers: a select between two loads would become one load through a selected address, and the
+// table would move to LDS.)
+struct ResolvedScales {
+    float s0, s1, s2, s3;
+};
+__device__ __forceinline__ ResolvedScales resolved_scales(const float (&beta)[4], float row_scale) {
+    return ResolvedScales{beta[0] * row_scale, beta[1] * row_scale, beta[2] * row_scale, beta[3] * row_scale};
+}
+__device__ __forceinline__ float resolved_scale(const ResolvedScales &scales, uint32_t lo) {
+    float s0 = scales.s0, s1 = scales.s1, s2 = scales.s2, s3 = scales.s3;
+    asm("" : "+v"(s0), "+v"(s1), "+v"(s2), "+v"(s3));    // values in registers, whatever memory they came from
+    const bool odd = (lo & 1u) != 0u;
+    const float low = odd ? s1 : s0;
+    const float high = odd ? s3 : s2;
+    return (lo & 2u) ? high : low;
+}
 
 // out[j] = (s_j - u_j) * 2^17 * scale  (pass scale = weight scale * kResolvedUnit).
 // The hash is evaluated on values shifted left by one bit, so that "modulo 2^31" is the
@@ -309,7 +322,23 @@ __device__ __forceinline__ uint32_t resolved_beta_id(uint32_t lo) { return lo & 
 // of the 18 bits used here (13 and 14), which then carry an unmixed but equally uniform bit.
 // The eight counters of a block share bits 16..30 unless the block straddles a multiple of 2^16
 // (or of 2^31): those blocks take the counter-by-counter form of the first shift-xor.
-// The part of the decode that needs no memory: bits[j] = 2^18 - 1 - U_j from the counters alone.
+
+// From t_j = counter_j ^ (counter_j >> 16) to the float pattern's dither part: 2^18 - 1 - U_j in
+// bits 0..17 under the exponent of 2^23 (the funnel shift that takes the hash's top 18 bits brings
+// the exponent in from its other operand).  Five instructions per weight.
+__device__ __forceinline__ void resolved_hash_bits(const uint32_t (&t)[8], uint32_t (&bits)[8]) {
+    const uint64_t twice_c = 2u * 12345u;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t v1 = mad_u32(t[j], 2u * 1103515245u, twice_c);
+        const uint32_t v1x = v1 ^ ((v1 >> 13) & 0x7fffeu);
+        const uint32_t v2_complement = v1x * (0u - 134775813u) - 3u;
+        bits[j] = __builtin_amdgcn_alignbit(0x4b000000u >> 18, v2_complement, 14);
+    }
+}
+
+// The part of the decode that needs no memory: bits[j] as resolved_hash_bits leaves them, from the
+// block's first counter.
 __device__ __forceinline__ void resolved_dither_bits(uint32_t counter_plus_seed, uint32_t (&bits)[8]) {
     const uint32_t base = counter_plus_seed & 0x7fffffffu;
     const uint32_t high = base >> 16;
@@ -324,30 +353,25 @@ __device__ __forceinline__ void resolved_dither_bits(uint32_t counter_plus_seed,
 #pragma unroll
         for (int j = 0; j < 8; j++) t[j] = (base + (uint32_t)j) ^ high;
     }
-    const uint64_t twice_c = 2u * 12345u;
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const uint32_t v1 = mad_u32(t[j], 2u * 1103515245u, twice_c);
-        const uint32_t v1x = v1 ^ ((v1 >> 13) & 0x7fffeu);
-        const uint32_t v2_complement = v1x * (0u - 134775813u) - 3u;
-        bits[j] = v2_complement >> 14;
-    }
+    resolved_hash_bits(t, bits);
 }
 
-// The part that needs the stored block: out[j] = (s_j - u_j) * 2^17 * scale.
+// The part that needs the stored block: out[j] = (s_j - u_j) * 2^17 * scale.  A weight's float
+// pattern is its dither part plus f_j 2^17: a bit-field extract and a shift-add.
 __device__ __forceinline__ void resolved_apply(uint32_t lo, uint32_t hi, const uint32_t (&bits)[8], float scale,
                                                float (&out)[8]) {
     // 2^23 + (2^18 - 1) + 15 * 2^17, less 2^16 in the half-integer coset
     const float origin = (hi & 1024u) ? 10551295.0f : 10616831.0f;
-    const uint32_t low_fields = as_computed(lo << 15), tail_fields = as_computed(hi << 17);
-    const uint32_t field[8] = {low_fields, low_fields >> 5, low_fields >> 10, lo, lo >> 5, lo >> 10,
-                               tail_fields, tail_fields >> 5};
     // (float - origin) * scale as one fused multiply-add: one rounding instead of two (the difference
     // is exact in the first form, so only the final rounding can move, by half a unit in the last place)
     const float shift = -origin * scale;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-        const uint32_t pattern = ((field[j] & (31u << 17)) | 0x4b000000u) + bits[j];
+        // spelled as instructions: left to itself the compiler turns the pair into shift, mask and add
+        uint32_t field, pattern;
+        if (j < 6) asm("v_bfe_u32 %0, %1, %2, 5" : "=v"(field) : "v"(lo), "n"(2 + 5 * (j < 6 ? j : 0)));
+        else asm("v_bfe_u32 %0, %1, %2, 5" : "=v"(field) : "v"(hi), "n"(5 * (j < 6 ? 0 : j - 6)));
+        asm("v_lshl_add_u32 %0, %1, 17, %2" : "=v"(pattern) : "v"(field), "v"(bits[j]));
         out[j] = __builtin_fmaf(__uint_as_float(pattern), scale, shift);
     }
 }

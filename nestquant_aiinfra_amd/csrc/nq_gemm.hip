@@ -58,6 +58,7 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
     const float unit = w_norms[dec_n] / sqrt_k;
     const float wscale = kResolved ? unit * kResolvedUnit : unit;
     const float wbeta[4] = {w_betas[0], w_betas[1], w_betas[2], w_betas[3]};
+    const ResolvedScales scaled_beta = resolved_scales(wbeta, wscale);
     const int64_t dec_first = (int64_t)dec_n * blocks_per_row + (k_begin >> 3) + dec_kb;
     // LDS entry of (K-step kk, fragment lane f): [kk][f ^ (2 (kk % 4) + f / 32)].  Eight neighbouring
     // decode lanes (one channel, blocks 8 i .. 8 i + 7, i.e. four K-steps x the two halves of the
@@ -127,7 +128,7 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
         if (s < steps) {
             float v[8];
             if (kResolved) {
-                decode_resolved(word, side, seed_plus_offset + (uint32_t)g * 8u, wbeta[resolved_beta_id(word)] * wscale, v);
+                decode_resolved(word, side, seed_plus_offset + (uint32_t)g * 8u, resolved_scale(scaled_beta, word), v);
             } else {
                 decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
                 const float scale = wbeta[(side >> (2 * (g & 3))) & 3] * wscale;

@@ -64,12 +64,14 @@ gemv_rows(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8
     const int n0 = group * R;
 
     float acc[R][M], wscale[R];
+    ResolvedScales scaled_beta[R];
     int64_t row_first_block[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int n = n0 + r < n_size ? n0 + r : n_size - 1;       // channels past the end repeat the last one
         const float unit = w_norms[n] / sqrt_k;
         wscale[r] = kResolved ? unit * kResolvedUnit : unit;
+        scaled_beta[r] = resolved_scales(wbeta, wscale[r]);
         row_first_block[r] = (int64_t)n * blocks_per_row + slice_first_block;
 #pragma unroll
         for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
@@ -119,7 +121,7 @@ gemv_rows(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8
             float v[8];
             if (kResolved) {
                 decode_resolved(word[r], side[r], seed_plus_offset + (uint32_t)g * 8u,
-                                wbeta[resolved_beta_id(word[r])] * wscale[r], v);
+                                resolved_scale(scaled_beta[r], word[r]), v);
             } else {
                 decode_codeword<true>(word[r], 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
                 const float scale = wbeta[(side[r] >> (2 * (g & 3))) & 3] * wscale[r];
@@ -219,9 +221,10 @@ constexpr int kMfmaGemvMaxWaves = 16;
 // weights would then leave part of the chip without a tile, so with R = 2 the rows are 8
 // channels times two interleaved ranges of 128 k: a super-step spans 128 R k, a lane still decodes
 // four consecutive blocks of its (channel, range), and every decoded block goes through R
-// instructions, the r-th with the activation fragment of range r and with the rows of the other
-// ranges zeroed, so that row (range, channel) only ever meets its own k.  The rows of a channel
-// are added at the end.
+// instructions, the r-th with the activation fragment of range r into an accumulator of its own:
+// in accumulator r only the rows of range r have met their own k, and only those are taken at the
+// end, where the rows of a channel are added.  (Zeroing the rows of the other ranges in the A
+// operand instead cost eight selects per block on the vector units, which are this kernel's limit.)
 template <int R>
 __global__ void __launch_bounds__(kMfmaGemvMaxWaves * 64)
 w4a4_gemv_mfma_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, int k_size, float sqrt_k,
@@ -241,6 +244,7 @@ w4a4_gemv_mfma_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, 
     const float wscale = (w.norms[which][n] / sqrt_k) * kResolvedUnit;
     const float *betas = w.betas[which];
     const float wbeta[4] = {betas[0], betas[1], betas[2], betas[3]};
+    const ResolvedScales scaled_beta = resolved_scales(wbeta, wscale);
     const uint32_t seed_plus_offset = w.seed_plus_offset[which];
     const int64_t row_first = (int64_t)n * blocks_per_row + 16 * range + 4 * quarter;
     const uint32_t *words = w.words[which];
@@ -249,7 +253,11 @@ w4a4_gemv_mfma_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, 
     const uint4 *act_row = act + (int64_t)(has_token ? column : 0) * blocks_per_row + 4 * quarter;
     const uint4 zero = make_uint4(0, 0, 0, 0);
 
-    floatx4 acc = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    // acc[r]: the products with the activation of range r.  Only the rows of range r are meant in it
+    // (a row of the other range has met the wrong k), and only those are read at the end.
+    floatx4 acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     uint4 word_next = zero, b_next[R][4];
 #pragma unroll
     for (int r = 0; r < R; r++)
@@ -286,27 +294,33 @@ w4a4_gemv_mfma_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, 
         }
         const uint32_t word[4] = {word4.x, word4.y, word4.z, word4.w};
         const uint32_t tail[4] = {tail2.x & 0xffffu, tail2.x >> 16, tail2.y & 0xffffu, tail2.y >> 16};
-        const int64_t g = row_first + 16 * R * ss;
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            float v[8];
-            decode_resolved(word[t], tail[t], seed_plus_offset + (uint32_t)(g + t) * 8u,
-                            wbeta[resolved_beta_id(word[t])] * wscale, v);
+        const uint32_t first_counter = seed_plus_offset + (uint32_t)(row_first + 16 * R * ss) * 8u;
+        const auto multiply = [&](int t, const float (&v)[8]) {
             const bf16x2 h0 = pack_bf16x2(v[0], v[1]), h1 = pack_bf16x2(v[2], v[3]);
             const bf16x2 h2 = pack_bf16x2(v[4], v[5]), h3 = pack_bf16x2(v[6], v[7]);
             const uint4 a = make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
                                        __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
 #pragma unroll
-            for (int r = 0; r < R; r++) {
-                const uint4 rows = (R == 1 || range == r) ? a : zero;
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rows),
-                                                              __builtin_bit_cast(bf16x8, b[r][t]), acc, 0, 0, 0);
-            }
+            for (int r = 0; r < R; r++)
+                acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                                 __builtin_bit_cast(bf16x8, b[r][t]), acc[r], 0, 0, 0);
+        };
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            float v[8];
+            decode_resolved(word[t], tail[t], first_counter + 8u * t, resolved_scale(scaled_beta, word[t]), v);
+            multiply(t, v);
         }
     }
-    // accumulator i of lane l: A row 4 (l / 16) + i = (range, channel), token l % 16
+    // accumulator i of lane l: A row 4 (l / 16) + i = (range, channel), token l % 16; the row's own
+    // range is (4 (l / 16) + i) / kChannels, the same for the lane's four rows
 #pragma unroll
-    for (int i = 0; i < 4; i++) part[wave][(4 * quarter + i) * 16 + column] = acc[i];
+    for (int i = 0; i < 4; i++) {
+        float mine = acc[0][i];
+#pragma unroll
+        for (int r = 1; r < R; r++) mine = (4 * quarter) / kChannels == r ? acc[r][i] : mine;
+        part[wave][(4 * quarter + i) * 16 + column] = mine;
+    }
     __syncthreads();
     if (tid < kChannels * 16) {
         const int channel = tid >> 4, token = tid & 15;
