@@ -557,3 +557,33 @@ def test_append_inside_the_attention_launch_equals_writer_then_attention(kv, ora
         assert torch.equal(a.layers[0].hot_keys, b.layers[0].hot_keys), step
         assert torch.equal(a.layers[0].hot_values, b.layers[0].hot_values), step
     assert any(t % PAGE < steps for t in totals)                     # pages were completed on the way
+
+
+def test_append_and_attend_rejects_what_it_cannot_take(kv):
+    """The one-launch form is for decode steps of one BF16 token per row: anything else is refused
+    before a launch, with the cache untouched."""
+    manager = _manager(kv, capacity=2, max_len=64)
+    for s in (0, 1):
+        manager.register(s, slot=s)
+    workspace = kv.BatchedNQKVAttentionWorkspace.create(manager.layers[0], batch_size=2, query_heads=32,
+                                                        output_dtype=torch.bfloat16)
+    query = torch.zeros((2, 32, DIM), dtype=torch.bfloat16, device="cuda")
+    key = torch.zeros((2, HEADS, DIM), dtype=torch.bfloat16, device="cuda")
+    manager.step_active[:2] = True
+    manager.begin_step(rows=2, uniform_count=3)                      # a step of three tokens per row
+    with pytest.raises(ValueError, match="one token each"):
+        manager.append_and_attend(0, query, key, key, attention_scale=0.125, workspace=workspace)
+    manager.begin_step(rows=2, uniform_count=1)
+    before = manager.layers[0].hot_keys.clone()
+    with pytest.raises(TypeError, match="BF16"):
+        manager.append_and_attend(0, query.half(), key, key, attention_scale=0.125, workspace=workspace)
+    with pytest.raises(ValueError, match="kv_heads"):
+        manager.append_and_attend(0, query, key[:, :4].contiguous(), key[:, :4].contiguous(), attention_scale=0.125,
+                                  workspace=workspace)
+    with pytest.raises(ValueError, match="contiguous"):
+        manager.append_and_attend(0, query, key.transpose(0, 1).contiguous().transpose(0, 1), key,
+                                  attention_scale=0.125, workspace=workspace)
+    with pytest.raises(ValueError, match="scale must be finite"):
+        manager.append_and_attend(0, query, key, key, attention_scale=float("nan"), workspace=workspace)
+    torch.cuda.synchronize()
+    assert torch.equal(manager.layers[0].hot_keys, before)
