@@ -303,6 +303,19 @@ int nq_bf16_gemm(const void *a_bf16_dev, const void *b_bf16_dev, int64_t m, int6
                  void *stream);
 
 /*
+ * The same product with its columns going to one to three outputs of their own: b stacks the
+ * weights of linears that share the activation a (q, k and v; gate and up), output i receives the
+ * next widths[i] columns as a row-major [M, widths[i]] BF16 matrix (16-byte aligned; every width
+ * a multiple of 256, so that no workgroup tile straddles two outputs).  One launch instead of one
+ * per linear: the narrow ones (k and v: 512 columns) no longer leave most of the chip idle.  No K
+ * split.  outs_bf16_dev and widths are host arrays of `count` entries.
+ * Replaces: the per-projection calls of FusedNQRTLinear.forward for projections that share their
+ * input (nestquant/models/fused_linear.py:49-127, SharedPackedActivationCache) in a long prefill.
+ */
+int nq_bf16_gemm_split(const void *a_bf16_dev, const void *b_bf16_dev, int64_t m, int64_t k,
+                       void *const *outs_bf16_dev, const int64_t *widths, int count, int tile, void *stream);
+
+/*
  * NQKV cache, device-resident state.  Per slot (int32[slots]): sequence_lengths,
  * page_counts, last_page_lens, hot_lengths; page_indices int32[slots, max_pages] maps a
  * slot's page ordinal to a physical page; hot tails BF16 [slots, page_size, kv_heads,

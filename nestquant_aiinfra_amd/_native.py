@@ -52,6 +52,7 @@ SIGNATURES = {
                                           _size, _ptr]),
     "nq_w4a4_gemm_workspace_bytes": (_size, [_i32, _i32, _i32, _i32, _i32]),
     "nq_bf16_gemm": (_i32, [_ptr, _ptr, _i64, _i64, _i64, _ptr, _i32, _i32, _ptr, _size, _ptr]),
+    "nq_bf16_gemm_split": (_i32, [_ptr, _ptr, _i64, _i64, _ptr, _ptr, _i32, _i32, _ptr]),
     "nq_nqkv_advance": (_i32, [_ptr, _ptr, _ptr, _i32, _i32, _i32, _i32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "nq_decode_step_begin": (_i32, [_ptr, _ptr, _i32, _i32, _i32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i32,
                                     _ptr, _ptr, _ptr, _i64, _i32, _ptr, _ptr]),

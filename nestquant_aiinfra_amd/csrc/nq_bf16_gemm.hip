@@ -61,6 +61,28 @@ __device__ __forceinline__ void issue_order(int) {
     issue_order_groups<kGroups, kReads, kMoves>();
 }
 
+// Column ranges of the product that go to outputs of their own (q, k and v of one activation
+// multiplied by their weights stacked in B): range i starts at column first[i] and goes to out[i],
+// a row-major matrix of its own width.  The host keeps every boundary a multiple of 256, so that no
+// workgroup tile straddles one.  count == 0: the single output c.
+struct DenseOutputs {
+    uint16_t *out[3];
+    int first[3], width[3];
+    int count;
+};
+
+// The output a workgroup whose tile starts at column n0 stores to, its width, and n0 inside it.
+__device__ __forceinline__ void tile_output(const DenseOutputs &outputs, int n0, uint16_t *&c, int &width, int &column0) {
+    if (outputs.count == 0) return;
+    int which = 0;
+#pragma unroll
+    for (int i = 1; i < 3; i++)
+        if (i < outputs.count && n0 >= outputs.first[i]) which = i;
+    c = which == 0 ? outputs.out[0] : (which == 1 ? outputs.out[1] : outputs.out[2]);
+    width = which == 0 ? outputs.width[0] : (which == 1 ? outputs.width[1] : outputs.width[2]);
+    column0 = n0 - (which == 0 ? outputs.first[0] : (which == 1 ? outputs.first[1] : outputs.first[2]));
+}
+
 // The wavefront's tiles go to C.  The products are taken as B A^T (the weight fragment is the matrix
 // instruction's first operand), so accumulator r of lane l belongs to row l % 32 and column
 // (r % 4) + 8 (r / 4) + 4 (l / 32) of its 32 x 32 tile: four neighbouring columns per lane and group of
@@ -154,7 +176,7 @@ template <int WM, int WN, int GM, int GN>
 __global__ void __launch_bounds__(64 * GM * GN)
 bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b, uint16_t *__restrict__ c,
                  int m_size, int n_size, int k_size, int tiles_m, int tiles_n, int group_m, int k_slab,
-                 float *__restrict__ partials) {
+                 float *__restrict__ partials, DenseOutputs outputs) {
     constexpr int kThreads = 64 * GM * GN;
     constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN;
     constexpr int kRowsPerPass = kThreads / 8;                     // rows one pass of 16-byte loads covers
@@ -283,12 +305,15 @@ bf16_gemm_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b,
     }
 
     // (the last step's barrier has passed: nobody reads the slabs any more)
-    if (!partials && (n_size & 7) == 0 && (reinterpret_cast<uintptr_t>(c) & 15) == 0)
-        store_tiles_by_rows<WM, WN>(acc, m0 + wave_m * 32 * WM, n0 + wave_n * 32 * WN, lane, c, m_size, n_size,
+    uint16_t *c_out = c;
+    int width = n_size, column0 = n0;
+    tile_output(outputs, n0, c_out, width, column0);
+    if (!partials && (width & 7) == 0 && (reinterpret_cast<uintptr_t>(c_out) & 15) == 0)
+        store_tiles_by_rows<WM, WN>(acc, m0 + wave_m * 32 * WM, column0 + wave_n * 32 * WN, lane, c_out, m_size, width,
                                     lds + wave * (128 * WM * WN));
     else
-        store_tiles<WM, WN>(acc, m0 + wave_m * 32 * WM, n0 + wave_n * 32 * WN, lane, c,
-                            partials ? partials + (int64_t)blockIdx.y * m_size * n_size : nullptr, m_size, n_size);
+        store_tiles<WM, WN>(acc, m0 + wave_m * 32 * WM, column0 + wave_n * 32 * WN, lane, c_out,
+                            partials ? partials + (int64_t)blockIdx.y * m_size * n_size : nullptr, m_size, width);
 }
 
 
@@ -302,7 +327,7 @@ template <int WM, int WN>
 __global__ void __launch_bounds__(512)
 bf16_gemm_roles_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ b, uint16_t *__restrict__ c,
                        int m_size, int n_size, int k_size, int tiles_m, int tiles_n, int group_m, int k_slab,
-                       float *__restrict__ partials) {
+                       float *__restrict__ partials, DenseOutputs outputs) {
     constexpr int BM = 64 * WM, BN = 64 * WN;
     constexpr int kStage = (BM + BN) * 8;                          // 16-byte pieces per LDS stage
     constexpr int kLoadsA = BM / 32, kLoadsB = BN / 32;            // 256 mover lanes cover 32 rows of 128 bytes per pass
@@ -431,12 +456,15 @@ bf16_gemm_roles_kernel(const uint16_t *__restrict__ a, const uint16_t *__restric
         lds_barrier();                                             // every fragment of the stage has arrived
     }
     // (the last step's barrier has passed: nobody reads the slabs any more)
-    if (!partials && (n_size & 7) == 0 && (reinterpret_cast<uintptr_t>(c) & 15) == 0)
-        store_tiles_by_rows<WM, WN>(acc, m0 + wave_m * 32 * WM, n0 + wave_n * 32 * WN, lane, c, m_size, n_size,
+    uint16_t *c_out = c;
+    int width = n_size, column0 = n0;
+    tile_output(outputs, n0, c_out, width, column0);
+    if (!partials && (width & 7) == 0 && (reinterpret_cast<uintptr_t>(c_out) & 15) == 0)
+        store_tiles_by_rows<WM, WN>(acc, m0 + wave_m * 32 * WM, column0 + wave_n * 32 * WN, lane, c_out, m_size, width,
                                     lds + wave * (128 * WM * WN));
     else
-        store_tiles<WM, WN>(acc, m0 + wave_m * 32 * WM, n0 + wave_n * 32 * WN, lane, c,
-                            partials ? partials + (int64_t)blockIdx.y * m_size * n_size : nullptr, m_size, n_size);
+        store_tiles<WM, WN>(acc, m0 + wave_m * 32 * WM, column0 + wave_n * 32 * WN, lane, c_out,
+                            partials ? partials + (int64_t)blockIdx.y * m_size * n_size : nullptr, m_size, width);
 }
 
 }  // namespace nq
@@ -465,7 +493,7 @@ const DenseTile kDenseTiles[] = {
 
 template <int WM, int WN, int GM, int GN>
 void launch_dense(const void *a, const void *b, void *c, int m, int n, int k, int split, float *partials,
-                  hipStream_t stream) {
+                  const nq::DenseOutputs &outputs, hipStream_t stream) {
     constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN;
     const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     const size_t lds_bytes = (size_t)2 * (BM + BN) * 128;
@@ -479,12 +507,12 @@ void launch_dense(const void *a, const void *b, void *c, int m, int n, int k, in
     hipLaunchKernelGGL((nq::bf16_gemm_kernel<WM, WN, GM, GN>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)split),
                        dim3(64 * GM * GN), lds_bytes, stream, reinterpret_cast<const uint16_t *>(a),
                        reinterpret_cast<const uint16_t *>(b), reinterpret_cast<uint16_t *>(c), m, n, k, tiles_m, tiles_n,
-                       group_m, k / split, split > 1 ? partials : nullptr);
+                       group_m, k / split, split > 1 ? partials : nullptr, outputs);
 }
 
 template <int WM, int WN>
 void launch_roles(const void *a, const void *b, void *c, int m, int n, int k, int split, float *partials,
-                  hipStream_t stream) {
+                  const nq::DenseOutputs &outputs, hipStream_t stream) {
     constexpr int BM = 64 * WM, BN = 64 * WN;
     const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     const size_t lds_bytes = (size_t)3 * (BM + BN) * 128;
@@ -498,7 +526,7 @@ void launch_roles(const void *a, const void *b, void *c, int m, int n, int k, in
     hipLaunchKernelGGL((nq::bf16_gemm_roles_kernel<WM, WN>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)split),
                        dim3(512), lds_bytes, stream, reinterpret_cast<const uint16_t *>(a),
                        reinterpret_cast<const uint16_t *>(b), reinterpret_cast<uint16_t *>(c), m, n, k, tiles_m, tiles_n,
-                       group_m, k / split, split > 1 ? partials : nullptr);
+                       group_m, k / split, split > 1 ? partials : nullptr, outputs);
 }
 
 }  // namespace
@@ -522,7 +550,12 @@ int dense_split_for(int m, int n, int k, size_t partial_bytes) {
 // Shared with nq_w4a4_gemm: picks the tile shape with the least estimated time (and, given a buffer
 // for partial results, a K split) and launches.
 int launch_bf16_gemm(const void *a, const void *b, void *c, int m, int n, int k, int forced_tile, int forced_split,
-                     void *partials, size_t partial_bytes, hipStream_t stream) {
+                     void *partials, size_t partial_bytes, hipStream_t stream, const DenseOutputs *split_outputs) {
+    DenseOutputs outputs;
+    outputs.count = 0;
+    if (split_outputs) outputs = *split_outputs;
+    // column ranges with outputs of their own are stored by the product's own launch: no K split
+    if (outputs.count > 0) forced_split = 1;
     int split = forced_split > 0 ? forced_split : dense_split_for(m, n, k, partials ? partial_bytes : 0);
     if (split > 1 && (k % (split * 128) != 0 || !partials || (size_t)split * m * n * sizeof(float) > partial_bytes))
         return fail(NQ_ERR_WORKSPACE, "nq_bf16_gemm: a K split of %d needs K a multiple of %d and %zu bytes for partial results",
@@ -548,21 +581,21 @@ int launch_bf16_gemm(const void *a, const void *b, void *c, int m, int n, int k,
     if (forced_tile == 9) { best = 6; best_alone = true; }
     float *p = reinterpret_cast<float *>(partials);
     switch (best) {
-        case 0: launch_dense<2, 4, 4, 2>(a, b, c, m, n, k, split, p, stream); break;
-        case 1: launch_dense<2, 4, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
-        case 2: launch_roles<4, 2>(a, b, c, m, n, k, split, p, stream); break;      // movers and multipliers
+        case 0: launch_dense<2, 4, 4, 2>(a, b, c, m, n, k, split, p, outputs, stream); break;
+        case 1: launch_dense<2, 4, 2, 2>(a, b, c, m, n, k, split, p, outputs, stream); break;
+        case 2: launch_roles<4, 2>(a, b, c, m, n, k, split, p, outputs, stream); break;      // movers and multipliers
         case 3:
-            if (best_alone) launch_roles<2, 2>(a, b, c, m, n, k, split, p, stream);
-            else launch_dense<2, 2, 2, 2>(a, b, c, m, n, k, split, p, stream);
+            if (best_alone) launch_roles<2, 2>(a, b, c, m, n, k, split, p, outputs, stream);
+            else launch_dense<2, 2, 2, 2>(a, b, c, m, n, k, split, p, outputs, stream);
             break;
         case 4:
-            if (best_alone) launch_roles<1, 2>(a, b, c, m, n, k, split, p, stream);
-            else launch_dense<1, 2, 2, 2>(a, b, c, m, n, k, split, p, stream);
+            if (best_alone) launch_roles<1, 2>(a, b, c, m, n, k, split, p, outputs, stream);
+            else launch_dense<1, 2, 2, 2>(a, b, c, m, n, k, split, p, outputs, stream);
             break;
-        case 5: launch_dense<2, 1, 2, 2>(a, b, c, m, n, k, split, p, stream); break;
+        case 5: launch_dense<2, 1, 2, 2>(a, b, c, m, n, k, split, p, outputs, stream); break;
         default:
-            if (best_alone) launch_roles<1, 1>(a, b, c, m, n, k, split, p, stream);
-            else launch_dense<1, 1, 2, 2>(a, b, c, m, n, k, split, p, stream);
+            if (best_alone) launch_roles<1, 1>(a, b, c, m, n, k, split, p, outputs, stream);
+            else launch_dense<1, 1, 2, 2>(a, b, c, m, n, k, split, p, outputs, stream);
             break;
     }
     const int status = check_launch("nq_bf16_gemm");
@@ -589,5 +622,37 @@ extern "C" int nq_bf16_gemm(const void *a_bf16_dev, const void *b_bf16_dev, int6
                "nq_bf16_gemm: split_k must be 0 (automatic), 1, 2, 4 or 8");
     NQ_REQUIRE(!workspace_dev || nq::aligned(workspace_dev, 16), NQ_ERR_ARGUMENT, "nq_bf16_gemm: workspace must be 16-byte aligned");
     return nq::launch_bf16_gemm(a_bf16_dev, b_bf16_dev, c_bf16_dev, (int)m, (int)n, (int)k, tile, split_k, workspace_dev,
-                                workspace_dev ? workspace_bytes : 0, (hipStream_t)stream);
+                                workspace_dev ? workspace_bytes : 0, (hipStream_t)stream, nullptr);
+}
+
+extern "C" int nq_bf16_gemm_split(const void *a_bf16_dev, const void *b_bf16_dev, int64_t m, int64_t k,
+                                  void *const *outs_bf16_dev, const int64_t *widths, int count, int tile, void *stream) {
+    NQ_REQUIRE(count >= 1 && count <= 3 && outs_bf16_dev && widths, NQ_ERR_ARGUMENT,
+               "nq_bf16_gemm_split: one to three outputs");
+    nq::DenseOutputs outputs;
+    outputs.count = count;
+    int64_t n = 0;
+    for (int i = 0; i < 3; i++) {
+        outputs.out[i] = nullptr; outputs.first[i] = 0; outputs.width[i] = 0;
+        if (i >= count) continue;
+        NQ_REQUIRE(widths[i] >= 256 && widths[i] % 256 == 0 && widths[i] < ((int64_t)1 << 30), NQ_ERR_SHAPE,
+                   "nq_bf16_gemm_split: width %lld of output %d is not a positive multiple of 256", (long long)widths[i], i);
+        NQ_REQUIRE(outs_bf16_dev[i] && nq::aligned(outs_bf16_dev[i], 16), NQ_ERR_ARGUMENT,
+                   "nq_bf16_gemm_split: outputs must be 16-byte aligned");
+        outputs.out[i] = reinterpret_cast<uint16_t *>(outs_bf16_dev[i]);
+        outputs.first[i] = (int)n;
+        outputs.width[i] = (int)widths[i];
+        n += widths[i];
+    }
+    NQ_REQUIRE(m >= 1 && m < ((int64_t)1 << 30) && n < ((int64_t)1 << 30), NQ_ERR_SHAPE,
+               "nq_bf16_gemm_split: M and N must be positive");
+    NQ_REQUIRE(k >= 2 * nq::kDenseBK && k % (2 * nq::kDenseBK) == 0 && k < ((int64_t)1 << 30), NQ_ERR_SHAPE,
+               "nq_bf16_gemm_split: K = %lld must be a positive multiple of 128", (long long)k);
+    NQ_REQUIRE(a_bf16_dev && b_bf16_dev && nq::aligned(a_bf16_dev, 16) && nq::aligned(b_bf16_dev, 16), NQ_ERR_ARGUMENT,
+               "nq_bf16_gemm_split: operands must be given and 16-byte aligned");
+    NQ_REQUIRE(m * k < ((int64_t)1 << 31) && n * k < ((int64_t)1 << 31), NQ_ERR_SHAPE,
+               "nq_bf16_gemm_split: operands of 2^31 elements or more are not supported");
+    NQ_REQUIRE(tile >= -1 && tile <= 9, NQ_ERR_ARGUMENT, "nq_bf16_gemm_split: tile must be -1 (automatic) or 0..9");
+    return nq::launch_bf16_gemm(a_bf16_dev, b_bf16_dev, outputs.out[0], (int)m, (int)n, (int)k, tile, 1, nullptr, 0,
+                                (hipStream_t)stream, &outputs);
 }

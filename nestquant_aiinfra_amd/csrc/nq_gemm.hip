@@ -200,8 +200,9 @@ decode_weight_kernel(const uint32_t *__restrict__ w_words, const uint16_t *__res
 
 namespace nq {
 int dense_split_for(int m, int n, int k, size_t partial_bytes);
+struct DenseOutputs;
 int launch_bf16_gemm(const void *a, const void *b, void *c, int m, int n, int k, int forced_tile, int forced_split,
-                     void *partials, size_t partial_bytes, hipStream_t stream);
+                     void *partials, size_t partial_bytes, hipStream_t stream, const DenseOutputs *split_outputs);
 }
 
 namespace {
@@ -304,7 +305,7 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
         char *dense_partials = reinterpret_cast<char *>(weight_bf16) + nq::align256((size_t)n * k * 2);
         const size_t used = (size_t)(dense_partials - reinterpret_cast<char *>(workspace_dev));
         return nq::launch_bf16_gemm(act, weight_bf16, out_dev, m, n, k, -1, 0, dense_partials,
-                                    workspace_bytes > used ? workspace_bytes - used : 0, s);
+                                    workspace_bytes > used ? workspace_bytes - used : 0, s, nullptr);
     }
     const uint32_t seed_plus_offset = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
     const float sqrt_k = (float)sqrt((double)k);

@@ -26,6 +26,8 @@ _EXPORTS = {
     "can_use_w4a4_mma_m128_staged": "w4a4_linear",
     "can_use_w4a4_mma_chunked_staged": "w4a4_linear",
     "linear_packed_w4a4_gemv_grouped": "w4a4_linear",
+    "can_use_w4a4_gemm_grouped": "w4a4_linear",
+    "linear_packed_w4a4_gemm_grouped": "w4a4_linear",
     "linear_packed_w4a4_gemv_m1": "w4a4_linear",
     "linear_packed_w4a4_gemv_m1_fp32_probe": "w4a4_linear",
     "linear_packed_w4a4_gemv_m1_splitk_probe": "w4a4_linear",

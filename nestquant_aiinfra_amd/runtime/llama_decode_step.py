@@ -39,7 +39,7 @@ import torch.nn.functional as F
 from .nqkv import attention_output_stage, launch_nqkv_decode_attention, nqkv_prefill_attention
 from .w4a4_linear import (BF16_ROWS_LINEAR_K, MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, _gemm, _gemv,
                           bf16_rows_linear, bf16_rows_linear_grouped, can_use_bf16_rows_linear, decode_weight_bf16,
-                          fused_input_stage,
+                          can_use_w4a4_gemm_grouped, fused_input_stage, linear_packed_w4a4_gemm_grouped,
                           linear_packed_w4a4_gemv_grouped, quantize_activation_cuda, rope_hadamard_cuda)
 
 
@@ -135,6 +135,8 @@ class FusedLlamaDecodeStep:
     def _linears(self, activation, prepared: list[PreparedNQRTLinear]) -> list[torch.Tensor]:
         if activation.token_count <= self._gemv_rows(activation):
             return linear_packed_w4a4_gemv_grouped(activation, prepared, output_dtype=torch.bfloat16)
+        if can_use_w4a4_gemm_grouped(activation, prepared):      # a long prefill: one product for the group
+            return linear_packed_w4a4_gemm_grouped(activation, prepared)
         return [self._linear(activation, weight) for weight in prepared]
 
     def _expanded_layer(self, index: int, device) -> tuple | None:

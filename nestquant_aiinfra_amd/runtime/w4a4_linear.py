@@ -574,11 +574,15 @@ BF16_ROWS_LINEAR_MAX_ROWS = 16
 BF16_ROWS_LINEAR_K = (2048, 4096, 8192)
 
 
-def decode_weight_bf16(weight: PreparedNQRTLinear) -> torch.Tensor:
-    """The BF16 weight [N, K] the packed linear kernels multiply by (transient scratch)."""
+def decode_weight_bf16(weight: PreparedNQRTLinear, *, out: torch.Tensor | None = None) -> torch.Tensor:
+    """The BF16 weight [N, K] the packed linear kernels multiply by (transient scratch); into `out`
+    (contiguous BF16 [N, K] on the weight's device) when given."""
     device = weight.row_norms.device
     n, k = weight.record.indices.shape[0], weight.record.feature_count
-    out = torch.empty((n, k), dtype=torch.bfloat16, device=device)
+    if out is None:
+        out = torch.empty((n, k), dtype=torch.bfloat16, device=device)
+    elif tuple(out.shape) != (n, k) or out.dtype != torch.bfloat16 or not out.is_contiguous() or out.device != device:
+        raise ValueError("out must be a contiguous BF16 [N, K] tensor on the weight's device")
     resolved = weight.resolved_words is not None
     _native.check(_native.library().nq_w4a4_decode_weight(
         weight.code_payload.data_ptr(), weight.beta_payload.data_ptr(),
@@ -652,6 +656,41 @@ def bf16_gemm(rows: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split
                                                  tile, split_k, None if workspace is None else workspace.data_ptr(), need,
                                                  _native.stream_handle(device)))
     return out
+
+
+def can_use_w4a4_gemm_grouped(activation: PreparedNQA4Activation, weights: Sequence[PreparedNQRTLinear]) -> bool:
+    """Whether `linear_packed_w4a4_gemm_grouped` takes these projections of one activation: a
+    long prefill (the decode-once route), two or three weights, every N a multiple of 256."""
+    k = activation.feature_count
+    return (2 <= len(weights) <= 3 and activation.token_count >= DECODE_ONCE_ROWS and k % 128 == 0
+            and activation.decoded is not None
+            and all(w.record.feature_count == k and w.record.indices.shape[0] % 256 == 0 for w in weights))
+
+
+def linear_packed_w4a4_gemm_grouped(activation: PreparedNQA4Activation,
+                                    weights: Sequence[PreparedNQRTLinear]) -> list[torch.Tensor]:
+    """The linears of two or three weights that share one activation (q, k and v; gate and up) in a
+    long prefill: every weight is decoded once into its rows of one BF16 scratch, and one dense
+    matrix-core GEMM over the stacked rows stores each projection's columns to a BF16 [M, N_i]
+    output of its own.  Same values as one `linear_packed_w4a4_mma_chunked_staged` per weight."""
+    if not can_use_w4a4_gemm_grouped(activation, weights):
+        raise ValueError("grouped prefill linears take 2 or 3 weights of one decoded activation of at least "
+                         f"{DECODE_ONCE_ROWS} rows, K a multiple of 128 and every N a multiple of 256")
+    rows = activation.decoded.reshape(activation.token_count, activation.feature_count)
+    device = _native.require_cuda(rows)
+    m, k = rows.shape
+    sizes = [int(w.record.indices.shape[0]) for w in weights]
+    stacked = _workspace(device, sum(sizes) * k * 2)[: sum(sizes) * k * 2].view(torch.bfloat16).view(sum(sizes), k)
+    first = 0
+    for weight, size in zip(weights, sizes):
+        decode_weight_bf16(weight, out=stacked[first:first + size])
+        first += size
+    outs = [torch.empty((m, size), dtype=torch.bfloat16, device=device) for size in sizes]
+    widths = (ctypes.c_int64 * len(sizes))(*sizes)
+    pointers = (ctypes.c_void_p * len(sizes))(*[out.data_ptr() for out in outs])
+    _native.check(_native.library().nq_bf16_gemm_split(rows.data_ptr(), stacked.data_ptr(), m, k, pointers, widths,
+                                                       len(sizes), -1, _native.stream_handle(device)))
+    return [out.reshape(*activation.original_shape[:-1], size) for out, size in zip(outs, sizes)]
 
 
 def linear_packed_w4a4_mma_m16(activation: PreparedNQA4Activation,

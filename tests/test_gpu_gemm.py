@@ -177,3 +177,30 @@ def test_dense_bf16_gemm_against_float32(rt, m, n, k):
     assert torch.equal(rt.bf16_gemm(a, b, split_k=1), rt.bf16_gemm(a, b, split_k=1))
     with pytest.raises(ValueError, match="multiple of 128"):
         rt.bf16_gemm(a[:, :64].contiguous(), b[:, :64].contiguous())
+
+
+@pytest.mark.parametrize("m,k,sizes", [(300, 512, (512, 256, 256)), (1024, 2048, (2048, 512, 512)), (384, 1024, (768, 768))])
+def test_grouped_prefill_linears_equal_one_call_per_weight(rt, oracle, m, k, sizes):
+    """q, k and v (or gate and up) of one activation through one dense product over their stacked
+    decoded weights (`linear_packed_w4a4_gemm_grouped`, `nq_bf16_gemm_split`): every output is bit
+    for bit what the decode-once route gives for its weight alone (same decoded BF16 operands,
+    same sum over K per element, whatever tile the product runs on)."""
+    weights = []
+    for i, n_out in enumerate(sizes):
+        g = torch.Generator().manual_seed(7000 + i)
+        w = torch.from_numpy(oracle.hadamard((0.02 * torch.randn(n_out, k, generator=g)).numpy()))
+        record = rt.quantize_weight_nqrt4(w.cuda(), q=Q, betas=WEIGHT_BETAS, dither_seed=20270000 + i, tensor_name=f"w{i}")
+        weights.append(rt.prepare_fused_linear(record, device="cuda"))
+    activation = _activation(rt, oracle, m, k, seed=7100)
+    assert rt.can_use_w4a4_gemm_grouped(activation, weights)
+    grouped = rt.linear_packed_w4a4_gemm_grouped(activation, weights)
+    for out, weight, n_out in zip(grouped, weights, sizes):
+        alone = rt.linear_packed_w4a4_mma_chunked_staged(activation, weight)
+        assert out.dtype == torch.bfloat16 and tuple(out.shape) == (m, n_out)
+        assert torch.equal(out, alone), n_out
+    # fewer rows than the decode-once route takes, or a width that a tile could straddle: refused
+    short = _activation(rt, oracle, 64, k, seed=7101)
+    assert not rt.can_use_w4a4_gemm_grouped(short, weights)
+    with pytest.raises(ValueError, match="grouped prefill linears"):
+        rt.linear_packed_w4a4_gemm_grouped(short, weights)
+    assert not rt.can_use_w4a4_gemm_grouped(activation, weights[:1])
