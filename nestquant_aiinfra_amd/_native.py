@@ -106,7 +106,15 @@ def dtype_tag(dtype: torch.dtype) -> int:
         raise TypeError(f"unsupported dtype {dtype}; expected float32, bfloat16 or float16") from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_handle(device: torch.device) -> int:
+    """The current stream of `device` as the integer the C ABI takes.  Every launch asks, so the
+    question goes to torch's raw-handle call where it exists (a fraction of a microsecond; building
+    a torch.cuda.Stream object for the answer takes several)."""
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
 
 
