@@ -600,14 +600,24 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
     const int pitch = chain_pitch(n);
     float *chains = lds;                                  // 8 * pitch floats: the row, transposed
     float *natural = chains + 8 * pitch;                  // n floats: the row in order (rows above 512 values, rotated)
+    // behind them (static LDS of odd size would be laid out in front of the dynamic part and leave the
+    // chains, which are read 128 bits at a time, misaligned): the row norm and a pass's beta choices
+    float *row_norm_shared = natural + n;
+    uint8_t *chosen = reinterpret_cast<uint8_t *>(natural + n + 4);       // 32 entries
     __shared__ float wave_sums[16];
     const int tid = threadIdx.x, lane = tid & 63;
     const int slice = blockIdx.x % slices;
     const int64_t row = blockIdx.x / slices;
     const int log_n = 31 - __builtin_clz(n);
-    const bool live = (tid & 3) < beta_count;
+    // Rows of up to 4096 values (workgroups of up to eight wavefronts) encode with eight lanes per
+    // (block, beta) pair, lane c the block's coordinate c, beta (lane / 8) % 4: a quarter of the
+    // instructions per lane.  With the sixteen wavefronts of an 8192-value row that would be four
+    // encoding wavefronts per SIMD taking turns, slower than the one lane per pair of its first four.
+    const bool eight_lanes = blockDim.x <= 512;
+    const int c = lane & 7, bi = eight_lanes ? (lane >> 3) & 3 : tid & 3;
+    const bool live = bi < beta_count;
     // requested first, used last; a launch that only runs the element-wise stage has no table
-    const float beta = codes != nullptr ? betas[live ? (tid & 3) : 0] : 1.0f;
+    const float beta = codes != nullptr ? betas[live ? bi : 0] : 1.0f;
     NQ_STAMP(0);
 
     float v[8];
@@ -637,14 +647,13 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
     __syncthreads();
     NQ_STAMP(2);
 
-    // only the first four wavefronts encode (256 pairs of the slice); the others are done
-    if (tid >= 256) return;
-
     // row norm in the reference's order (quantizer.py:257): chain k sums the squares of elements
-    // k, k + 8, ... with fused multiply-adds; chains added 0..7; sqrt.  Lanes 8 .. 63 run along
-    // (on chain lane % 8) so that the wavefront stays uniform.
-    float norm;
-    {
+    // k, k + 8, ... with fused multiply-adds; chains added 0..7; sqrt.  The first four wavefronts (one
+    // per SIMD: the chain is a latency, and wavefronts that shared a SIMD would take turns) run it,
+    // lanes 8 .. 63 running along (on chain lane % 8) so that the wavefront stays uniform; the others
+    // get the result through LDS.
+    float norm = 0.0f;
+    if (tid < 256) {
         const float4 *chain = reinterpret_cast<const float4 *>(chains + (lane & 7) * pitch);
         const int quads = n >> 5;                          // 128-bit loads per chain, a multiple of 16
         float acc = 0.0f;
@@ -703,38 +712,76 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
 #pragma unroll
         for (int k = 0; k < 8; k++) total = total + __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, k));
         norm = __builtin_sqrtf(total);
+        if (tid == 0) *row_norm_shared = norm;
+    }
+    if (!eight_lanes && tid >= 256) return;                // one lane per pair: the first four wavefronts encode
+    if (eight_lanes && blockDim.x > 256) {
+        __syncthreads();
+        norm = *row_norm_shared;
     }
     // math.sqrt(n) / norm is evaluated as (1 / norm) * float32(sqrt(n))
     const float scale = norm > 0.0f ? (1.0f / norm) * sqrt_n : 0.0f;
     if (slice == 0 && tid == 0) norms[row] = norm;
     NQ_STAMP(3);
 
-    // one lane per (block, beta) pair of the slice
-    const int blocks_per_row = n >> 3;
-    const int p = slice * 256 + tid, b = p >> 2, bi = p & 3;
-    float raw[8];
+    if (!eight_lanes) {
+        // one lane per (block, beta) pair of the slice (256 pairs)
+        const int p = slice * 256 + tid, b = p >> 2;
+        float raw[8];
 #pragma unroll
-    for (int j = 0; j < 8; j++) raw[j] = chains[j * pitch + b];
-    struct LaneSink {
-        uint32_t *codes; uint8_t *beta_ids; uint4 *decoded; int64_t first_block; float back;
-        __device__ __forceinline__ bool wants(int) const { return true; }
-        __device__ __forceinline__ void code(int, int b, uint32_t word, const float (&recon)[8], float beta) const {
-            codes[first_block + b] = word;
-            if (decoded) {
-                uint32_t h[8];
+        for (int j = 0; j < 8; j++) raw[j] = chains[j * pitch + b];
+        struct LaneSink {
+            uint32_t *codes; uint8_t *beta_ids; uint4 *decoded; int64_t first_block; float back;
+            __device__ __forceinline__ bool wants(int) const { return true; }
+            __device__ __forceinline__ void code(int, int b, uint32_t word, const float (&recon)[8], float beta) const {
+                codes[first_block + b] = word;
+                if (decoded) {
+                    uint32_t h[8];
 #pragma unroll
-                for (int j = 0; j < 8; j++) h[j] = f32_to_bf16((recon[j] * beta) * back);
-                decoded[first_block + b] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16),
-                                                      h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+                    for (int j = 0; j < 8; j++) h[j] = f32_to_bf16((recon[j] * beta) * back);
+                    decoded[first_block + b] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16),
+                                                          h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+                }
             }
+            __device__ __forceinline__ void beta_byte(int, int b, uint32_t byte) const {
+                beta_ids[(first_block + b) >> 2] = (uint8_t)byte;
+            }
+            __device__ __forceinline__ uint32_t counter(int, int) const { return 0; }
+        };
+        const LaneSink sink{codes, beta_ids, decoded, row * (n >> 3), norm / sqrt_n};
+        quantize_pair_lane<false, true>(raw, scale, beta, live, bi, 0, b, p, 14.0f, 1.0f / 14.0f, 0u, sink);
+        NQ_STAMP(4);
+        return;
+    }
+
+    // Encode: eight lanes per (block, beta) pair, lane c the block's coordinate c; a wavefront holds
+    // two blocks with their four betas each, the workgroup blockDim / 32 blocks per pass, and the
+    // slice's blocks take blocks_per_slice / (blockDim / 32) passes (one when a row has 32 slices).
+    const int blocks_per_row = n >> 3;
+    const int blocks_per_slice = blocks_per_row / slices, blocks_per_pass = (int)(blockDim.x >> 5);
+    const int64_t first_block = row * blocks_per_row;
+    const float back = norm / sqrt_n;
+    for (int first = 0; first < blocks_per_slice; first += blocks_per_pass) {
+        const int in_pass = 2 * (tid >> 6) + (lane >> 5);
+        const int b = slice * blocks_per_slice + first + in_pass;
+        const float raw = chains[c * pitch + b];
+        const PairOnEightLanes pair = quantize_pair_on_eight_lanes<true>(raw, scale, beta, live, bi, lane);
+        if (pair.wins) {
+            if (c == 0) codes[first_block + b] = pair.word;
+            if (decoded)
+                reinterpret_cast<uint16_t *>(decoded)[(first_block + b) * 8 + c] =
+                    f32_to_bf16((pair.recon * beta) * back);
         }
-        __device__ __forceinline__ void beta_byte(int, int b, uint32_t byte) const {
-            beta_ids[(first_block + b) >> 2] = (uint8_t)byte;
+        if ((lane & 31) == 7) chosen[in_pass] = (uint8_t)pair.best;
+        __syncthreads();
+        // four consecutive blocks share one beta byte
+        if (tid < (blocks_per_pass >> 2)) {
+            const uint32_t byte = chosen[4 * tid] | (chosen[4 * tid + 1] << 2) | (chosen[4 * tid + 2] << 4) |
+                                  (chosen[4 * tid + 3] << 6);
+            beta_ids[(first_block + slice * blocks_per_slice + first + 4 * tid) >> 2] = (uint8_t)byte;
         }
-        __device__ __forceinline__ uint32_t counter(int, int) const { return 0; }
-    };
-    const LaneSink sink{codes, beta_ids, decoded, row * blocks_per_row, norm / sqrt_n};
-    quantize_pair_lane<false, true>(raw, scale, beta, live, bi, 0, b, p, 14.0f, 1.0f / 14.0f, 0u, sink);
+        if (first + blocks_per_pass < blocks_per_slice) __syncthreads();      // `chosen` is written again
+    }
     NQ_STAMP(4);
 }
 
@@ -1046,8 +1093,11 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
     // slices of 256 (block, beta) pairs
     if (std::is_same<T, uint16_t>::value && !kDithered && q == 14 && (n == 2048 || n == 4096 || n == 8192) &&
         rows <= 16 && nq::aligned(x, 16)) {
-        const int slices = n / 512;                       // 4 * (n / 8) pairs in slices of 256
-        const size_t lds_bytes = (size_t)(8 * ((n >> 3) + 8) + n) * sizeof(float);
+        // a workgroup of n / 8 lanes encodes n / 256 blocks per pass (eight lanes per (block, beta) pair):
+        // 32 slices of one pass each while that keeps the launch within one workgroup per compute unit
+        // (n <= 4096; an 8192-value row keeps one lane per pair: slices of 256 pairs)
+        const int slices = n > 4096 ? n / 512 : (rows * 32 <= 256 ? 32 : 16);
+        const size_t lds_bytes = (size_t)(8 * ((n >> 3) + 8) + n + 4 + 8) * sizeof(float);   // + norm, beta choices
         auto kernel = nq::quantize_row_lanes_kernel<kPrologue>;
         if (lds_bytes > 48 * 1024) {
             hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),

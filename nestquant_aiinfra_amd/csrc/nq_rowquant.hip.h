@@ -378,6 +378,148 @@ __device__ __forceinline__ void quantize_pair_lane(const float (&raw)[8], float 
     if ((p & 15) == 0 && wanted) sink.beta_byte(r, b, byte);
 }
 
+// ---------------------------------------------------------------------------------------
+// One (block, beta) pair on eight neighbouring lanes, lane c (= lane id % 8) holding coordinate c.
+// For a few rows the encoder is a latency problem: with one lane per pair a wavefront walks about
+// 850 instructions that depend on each other; spread over its coordinates a pair takes about 250
+// per lane, and the eight-term sums whose order the reference fixes (squares added j = 0..7) become
+// scans along the eight lanes.  Every float32 operation is the one quantize_pair_lane performs, in
+// the same order, so codes, beta ids and decoded values are the same bits.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float dpp_from_lane_below(float v) {       // lane i <- lane i - 1 (row_shr:1)
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x111, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_from_lane_above(float v) {       // lane i <- lane i + 1 (row_shl:1)
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x101, 0xF, 0xF, true));
+}
+// ((v0 + v1) + v2) + ... + v7 of the eight lanes of a group, valid in its last lane (c == 7): after
+// step k lane i holds the left-to-right sum of lanes i - k .. i, so the window of lane 7 never
+// leaves the group.
+__device__ __forceinline__ float ordered_sum8_in_last(float v) {
+    float s = v;
+#pragma unroll
+    for (int k = 1; k < 8; k++) s = dpp_from_lane_below(s) + v;
+    return s;
+}
+// the value of the group's last lane in all eight: the last lane of each quad to its quad, then the
+// upper quad mirrored into the lower one
+__device__ __forceinline__ float from_last8(float v) {
+    const int quad = __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xFF, 0xF, 0xF, true);       // quad_perm [3,3,3,3]
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(quad, quad, 0x141, 0xF, 0x5, false)); // half mirror into lanes 0-3
+}
+__device__ __forceinline__ float max8(float v) {
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true)));
+    return v;
+}
+__device__ __forceinline__ uint32_t or8(uint32_t v) {
+    v |= (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);
+    v |= (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xF, 0xF, true);
+    v |= (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x141, 0xF, 0xF, true);
+    return v;
+}
+// whether this lane is the first of its group of eight whose flag is set
+__device__ __forceinline__ bool first_set8(bool flag, int lane) {
+    const uint64_t all = __builtin_amdgcn_ballot_w64(flag);
+    const uint32_t group = (uint32_t)(all >> (lane & 56)) & 0xffu;
+    return flag && (group & ((1u << (lane & 7)) - 1u)) == 0u;
+}
+
+// e8_nearest (nq_e8.hip.h) with x_c in lane c: returns coordinate c of the nearest point.
+__device__ __forceinline__ float e8_nearest_on_eight_lanes(float x, int lane) {
+    const float a = __builtin_rintf(x);
+    const float ea = x - a;                                    // exact
+    const float xm = x - 0.5f;
+    const float b = __builtin_rintf(xm);
+    const float eb = xm - b;
+    const float sum_a = from_last8(ordered_sum8_in_last(a)), sum_b = from_last8(ordered_sum8_in_last(b));
+    const float max_a = max8(fabsf(ea)), max_b = max8(fabsf(eb));
+    const float moved_a = max_a - 1.0f;
+    const float alt_a = moved_a * moved_a;
+    // the first coordinate with the largest |residual| moves when the coordinate sum is odd
+    const bool hit_a = first_set8(fabsf(ea) == max_a, lane) && is_odd(sum_a);
+    const bool hit_b = first_set8(fabsf(eb) == max_b, lane) && is_odd(sum_b);
+    const float sq = ea * ea;
+    const float term_a = hit_a ? alt_a : sq;
+    const float point_a = hit_a ? a + __builtin_copysignf(1.0f, ea) : a;
+    const float half_point = b + 0.5f;
+    const float point_b = hit_b ? half_point + __builtin_copysignf(1.0f, eb) : half_point;
+    const float t = x - point_b;
+    const float term_b = t * t;
+    const float dist_a = ordered_sum8_in_last(term_a), dist_b = ordered_sum8_in_last(term_b);
+    const bool pick_a = from_last8(dist_a < dist_b ? 1.0f : 0.0f) != 0.0f;       // ties go to the half-integer coset
+    return pick_a ? point_a : point_b;
+}
+
+struct PairOnEightLanes {
+    uint32_t word;      // the packed code word, in all eight lanes
+    uint32_t best;      // the block's winning beta index, in the last lane of each of the four groups
+    float recon;        // coordinate c of the pair's decoded lattice point
+    bool wins;          // this pair's beta is the block's choice, in all eight lanes
+};
+
+// quantize_pair_lane for the pair whose coordinate c this lane holds (`raw`), q = 14.  The four
+// betas of a block sit in four neighbouring groups of eight lanes (beta index bi = (lane / 8) % 4).
+template <bool kFastDivide>
+__device__ __forceinline__ PairOnEightLanes quantize_pair_on_eight_lanes(float raw, float scale, float beta, bool live,
+                                                                         int bi, int lane) {
+    const int c = lane & 7;
+    const float y = raw * scale;
+    const uint32_t key = (__float_as_uint(y) << 1) - 1u;                         // as has_tiny_nonzero
+    const bool tiny = key < ((66u << 24) - 1u);
+    const bool by_reciprocal = kFastDivide && beta >= 0x1p-40f && beta <= 0x1p40f && __builtin_amdgcn_ballot_w64(tiny) == 0;
+    float z;
+    if (by_reciprocal) z = divide_by_reciprocal(y, beta, 1.0f / beta);
+    else z = y / beta;                                                           // IEEE division
+    // encode_block: nearest point, generator coordinates (the recurrence of e8_coords, one step per
+    // coordinate from c = 5 down), residues modulo q
+    const float point = e8_nearest_on_eight_lanes(z, lane);
+    const float last = from_last8(point);
+    float coord = c == 7 ? 2.0f * point : point - last;                          // c[7], c[6]
+#pragma unroll
+    for (int step = 5; step >= 0; step--) {
+        const float candidate = (point + dpp_from_lane_above(coord)) - last;
+        coord = c == step ? (step == 0 ? 0.5f * candidate : candidate) : coord;
+    }
+    const float code = mod_q(coord, 14.0f, 1.0f / 14.0f);
+    // e8_coset_point
+    const float h = 0.5f * from_last8(code);
+    const float next = dpp_from_lane_above(code);
+    const float p8 = c == 0 ? (2.0f * code - next) + h : (c <= 5 ? (code - next) + h : (c == 6 ? code + h : h));
+    // reduce_coset_point
+    const float k = e8_nearest_on_eight_lanes(div_by_14(p8), lane);
+    const float recon = p8 - 14.0f * k;                                          // exact
+    const float d = recon * beta - y;
+    float err = ordered_sum8_in_last(d * d);
+    if (!live) err = __builtin_inff();
+    // first minimum over the four betas: order by (err, beta index); partners 8 and 16 lanes away
+    uint32_t best_err = __float_as_uint(err), best = (uint32_t)bi;
+    {
+        const uint32_t oe = (uint32_t)__builtin_amdgcn_mov_dpp((int)best_err, 0x128, 0xF, 0xF, true);   // row_ror:8
+        const uint32_t oi = (uint32_t)__builtin_amdgcn_mov_dpp((int)best, 0x128, 0xF, 0xF, true);
+        const float fe = __uint_as_float(oe), me = __uint_as_float(best_err);
+        const bool take = fe < me || (fe == me && oi < best);
+        best_err = take ? oe : best_err;
+        best = take ? oi : best;
+    }
+    {
+        const auto e2 = __builtin_amdgcn_permlane16_swap(best_err, best_err, false, false);
+        const auto i2 = __builtin_amdgcn_permlane16_swap(best, best, false, false);
+        const bool upper = (lane & 16) != 0;
+        const uint32_t oe = upper ? (uint32_t)e2[0] : (uint32_t)e2[1], oi = upper ? (uint32_t)i2[0] : (uint32_t)i2[1];
+        const float fe = __uint_as_float(oe), me = __uint_as_float(best_err);
+        const bool take = fe < me || (fe == me && oi < best);
+        best = take ? oi : best;
+    }
+    PairOnEightLanes out;
+    out.best = best;
+    out.wins = from_last8(best == (uint32_t)bi ? 1.0f : 0.0f) != 0.0f;
+    out.word = or8(((uint32_t)code) << (4 * c));
+    out.recon = recon;
+    return out;
+}
+
 // Pairs [pair_begin, pair_end) of the staged rows (pair = (row * n / 8 + block) * 4 + beta
 // index; both bounds multiples of 16).  betas_of(row) returns that row's beta table.
 // Sink: wants(row), code(row, block, word, recon, beta), beta_byte(row, block, byte),
