@@ -166,34 +166,68 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
 }
 
 
-// The BF16 weight [N][K] the linear kernels multiply by, written out: one lane per E8 block,
-// the same decode, scale and rounding as the decode role of the kernel above.  Long prefills
-// decode the weight once with the whole chip and hand the plain GEMM to a library.
-template <bool kResolved>
+// The BF16 weight [N][K] the linear kernels multiply by, written out: the same decode, scale and
+// rounding as the decode role of the kernel above.  Long prefills decode the weight once with the
+// whole chip and multiply with the dense BF16 GEMM.  The packed form: one lane per E8 block.
 __global__ void __launch_bounds__(256)
-decode_weight_kernel(const uint32_t *__restrict__ w_words, const uint16_t *__restrict__ w_tails,
-                     const uint8_t *__restrict__ w_beta_ids, const float *__restrict__ w_norms,
-                     const float *__restrict__ w_betas, int64_t blocks, int blocks_per_row,
-                     uint32_t seed_plus_offset, float sqrt_k, uint4 *__restrict__ out) {
+decode_weight_kernel(const uint32_t *__restrict__ w_words, const uint8_t *__restrict__ w_beta_ids,
+                     const float *__restrict__ w_norms, const float *__restrict__ w_betas, int64_t blocks,
+                     int blocks_per_row, uint32_t seed_plus_offset, float sqrt_k, uint4 *__restrict__ out) {
     const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (g >= blocks) return;
     const int64_t row = g / blocks_per_row;
     const uint32_t word = w_words[g];
     const float unit = w_norms[row] / sqrt_k;
     float v[8];
-    if (kResolved) {
-        decode_resolved(word, w_tails[g], seed_plus_offset + (uint32_t)g * 8u,
-                        w_betas[resolved_beta_id(word)] * (unit * kResolvedUnit), v);
-    } else {
-        decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
-        const float scale = w_betas[(w_beta_ids[g >> 2] >> (2 * (g & 3))) & 3] * unit;
+    decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
+    const float scale = w_betas[(w_beta_ids[g >> 2] >> (2 * (g & 3))) & 3] * unit;
 #pragma unroll
-        for (int j = 0; j < 8; j++) v[j] = v[j] * scale;
-    }
+    for (int j = 0; j < 8; j++) v[j] = v[j] * scale;
     const bf16x2 h0 = pack_bf16x2(v[0], v[1]), h1 = pack_bf16x2(v[2], v[3]);
     const bf16x2 h2 = pack_bf16x2(v[4], v[5]), h3 = pack_bf16x2(v[6], v[7]);
     out[g] = make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
                         __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
+}
+
+// The resolved form of the weight, four blocks per lane.  A wavefront takes 256 consecutive blocks,
+// lane l the blocks l, 64 + l, 128 + l and 192 + l of them: every load and store instruction of the
+// wavefront covers one contiguous stretch, the four word loads of a lane are in flight together and
+// the hashes of the next block overlap the stores of the last.  kWholeStretch: the blocks of a row
+// are a multiple of 256, so a wavefront's stretch lies in one row and the lane keeps that row's four
+// beta scales in registers.
+constexpr int kDecodeBlocksPerLane = 4;
+
+template <bool kWholeStretch>
+__global__ void __launch_bounds__(256)
+decode_resolved_weight_kernel(const uint32_t *__restrict__ w_words, const uint16_t *__restrict__ w_tails,
+                              const float *__restrict__ w_norms, const float *__restrict__ w_betas, uint32_t blocks,
+                              uint32_t blocks_per_row, uint32_t seed_plus_offset, float sqrt_k,
+                              uint4 *__restrict__ out) {
+    const uint32_t first = (blockIdx.x * 4u + (threadIdx.x >> 6)) * (64u * kDecodeBlocksPerLane) + (threadIdx.x & 63u);
+    if (first >= blocks) return;
+    uint32_t word[kDecodeBlocksPerLane], tail[kDecodeBlocksPerLane];
+#pragma unroll
+    for (int i = 0; i < kDecodeBlocksPerLane; i++) {
+        const uint32_t g = first + 64u * i;
+        const bool live = g < blocks;
+        word[i] = live ? w_words[g] : 0u;
+        tail[i] = live ? (uint32_t)w_tails[g] : 0u;
+    }
+    const float beta[4] = {w_betas[0], w_betas[1], w_betas[2], w_betas[3]};
+    ResolvedScales scales = resolved_scales(beta, (w_norms[first / blocks_per_row] / sqrt_k) * kResolvedUnit);
+#pragma unroll
+    for (int i = 0; i < kDecodeBlocksPerLane; i++) {
+        const uint32_t g = first + 64u * i;
+        if (g >= blocks) break;
+        if (!kWholeStretch && i > 0)
+            scales = resolved_scales(beta, (w_norms[g / blocks_per_row] / sqrt_k) * kResolvedUnit);
+        float v[8];
+        decode_resolved(word[i], tail[i], seed_plus_offset + g * 8u, resolved_scale(scales, word[i]), v);
+        const bf16x2 h0 = pack_bf16x2(v[0], v[1]), h1 = pack_bf16x2(v[2], v[3]);
+        const bf16x2 h2 = pack_bf16x2(v[4], v[5]), h3 = pack_bf16x2(v[6], v[7]);
+        out[g] = make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
+                            __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
+    }
 }
 
 }  // namespace nq
@@ -361,15 +395,24 @@ extern "C" int nq_w4a4_decode_weight(const uint8_t *w_codes_dev, const uint8_t *
                "nq_w4a4_decode_weight: block range exceeds the stateless dither counter space");
     const uint32_t seed_plus_offset = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
     const float sqrt_k = (float)sqrt((double)k);
-    const dim3 grid((unsigned)((blocks + 255) / 256));
-    const uint32_t *words = resolved ? w_resolved_words_dev : reinterpret_cast<const uint32_t *>(w_codes_dev);
-    if (resolved)
-        hipLaunchKernelGGL(nq::decode_weight_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, words,
-                           w_resolved_tails_dev, w_beta_ids_dev, w_norms_dev, w_betas_dev, blocks, (int)(k / 8),
-                           seed_plus_offset, sqrt_k, reinterpret_cast<uint4 *>(out_bf16_dev));
-    else
-        hipLaunchKernelGGL(nq::decode_weight_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, words,
-                           w_resolved_tails_dev, w_beta_ids_dev, w_norms_dev, w_betas_dev, blocks, (int)(k / 8),
-                           seed_plus_offset, sqrt_k, reinterpret_cast<uint4 *>(out_bf16_dev));
+    const hipStream_t s = (hipStream_t)stream;
+    const uint32_t blocks_per_row = (uint32_t)(k / 8);
+    if (resolved) {
+        constexpr int64_t per_group = 256 * nq::kDecodeBlocksPerLane;
+        const dim3 grid((unsigned)((blocks + per_group - 1) / per_group));
+        if (blocks_per_row % (64 * nq::kDecodeBlocksPerLane) == 0)
+            hipLaunchKernelGGL(nq::decode_resolved_weight_kernel<true>, grid, dim3(256), 0, s, w_resolved_words_dev,
+                               w_resolved_tails_dev, w_norms_dev, w_betas_dev, (uint32_t)blocks, blocks_per_row,
+                               seed_plus_offset, sqrt_k, reinterpret_cast<uint4 *>(out_bf16_dev));
+        else
+            hipLaunchKernelGGL(nq::decode_resolved_weight_kernel<false>, grid, dim3(256), 0, s, w_resolved_words_dev,
+                               w_resolved_tails_dev, w_norms_dev, w_betas_dev, (uint32_t)blocks, blocks_per_row,
+                               seed_plus_offset, sqrt_k, reinterpret_cast<uint4 *>(out_bf16_dev));
+    } else {
+        hipLaunchKernelGGL(nq::decode_weight_kernel, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0, s,
+                           reinterpret_cast<const uint32_t *>(w_codes_dev), w_beta_ids_dev, w_norms_dev, w_betas_dev,
+                           blocks, (int)blocks_per_row, seed_plus_offset, sqrt_k,
+                           reinterpret_cast<uint4 *>(out_bf16_dev));
+    }
     return nq::check_launch("nq_w4a4_decode_weight");
 }

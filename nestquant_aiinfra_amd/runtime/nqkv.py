@@ -659,35 +659,46 @@ class BatchedNQKVCacheManager:
 
     # -- slots ---------------------------------------------------------------------------
     def register(self, sequence_id: Hashable, *, slot: int) -> None:
-        if not 0 <= slot < self.capacity:
-            raise ValueError("slot is outside cache capacity")
-        if self._sequence_of_slot[slot] is not None:
-            raise RuntimeError("slot is already occupied")
-        if sequence_id in self._sequence_of_slot:
-            raise RuntimeError("sequence is already registered")
-        self._sequence_of_slot[slot] = sequence_id
-        self.metadata.active_mask[slot] = True
-        for tensor in (self.metadata.sequence_lengths, self.metadata.page_counts,
-                       self.metadata.last_page_lens, self.metadata.hot_lengths):
-            tensor[slot] = 0
+        self.register_batch([(sequence_id, slot)])
 
     def register_batch(self, assignments: Sequence[tuple[Hashable, int]]) -> None:
-        for sequence_id, slot in assignments:
-            self.register(sequence_id, slot=slot)
+        """All-or-nothing: every assignment is checked before the first slot is taken."""
+        assignments = list(assignments)
+        slots = [slot for _, slot in assignments]
+        names = [name for name, _ in assignments]
+        if any(not 0 <= slot < self.capacity for slot in slots):
+            raise ValueError("slot is outside cache capacity")
+        if len(set(names)) != len(names) or any(name in self._sequence_of_slot for name in names):
+            raise ValueError("sequence is already registered")      # nqkv_batch_manager.py:395-396
+        if len(set(slots)) != len(slots) or any(self._sequence_of_slot[slot] is not None for slot in slots):
+            raise RuntimeError("slot is already occupied")          # nqkv_batch_manager.py:398-399
+        for name, slot in assignments:
+            self._sequence_of_slot[slot] = name
+        self._reset_slot_tables(slots, active=True)
+
+    def _reset_slot_tables(self, slots: Sequence[int], *, active: bool) -> None:
+        """Zero lengths and counts of `slots` and set their activity flag: one fill per table and run
+        of neighbouring slots (a batch admitted into slots 0..b-1 costs five launches, not 5 b)."""
+        ordered = sorted(slots)
+        meta = self.metadata
+        start = 0
+        while start < len(ordered):
+            stop = start
+            while stop + 1 < len(ordered) and ordered[stop + 1] == ordered[stop] + 1:
+                stop += 1
+            first, last = ordered[start], ordered[stop] + 1
+            meta.active_mask[first:last] = active
+            for tensor in (meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths):
+                tensor[first:last] = 0
+            start = stop + 1
 
     def release_slots(self, slots: Sequence[int]) -> tuple[Hashable, ...]:
-        released = []
-        for slot in slots:
-            sequence_id = self._sequence_of_slot[slot]
-            if sequence_id is None:
-                continue
-            released.append(sequence_id)
+        held = [slot for slot in dict.fromkeys(slots) if self._sequence_of_slot[slot] is not None]
+        released = tuple(self._sequence_of_slot[slot] for slot in held)
+        for slot in held:
             self._sequence_of_slot[slot] = None
-            self.metadata.active_mask[slot] = False
-            for tensor in (self.metadata.sequence_lengths, self.metadata.page_counts,
-                           self.metadata.last_page_lens, self.metadata.hot_lengths):
-                tensor[slot] = 0
-        return tuple(released)
+        self._reset_slot_tables(held, active=False)
+        return released
 
     def sequence_id(self, slot: int) -> Hashable | None:
         return self._sequence_of_slot[slot]

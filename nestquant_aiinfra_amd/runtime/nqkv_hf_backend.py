@@ -70,8 +70,10 @@ class BatchedNQKVLlamaCache(Cache):
         self._host_lengths[slot] = 0
 
     def register_batch(self, assignments: Sequence[tuple[Hashable, int]]) -> None:
-        for sequence_id, slot in assignments:
-            self.register(sequence_id, slot=slot)
+        assignments = list(assignments)
+        self.manager.register_batch(assignments)
+        for _, slot in assignments:
+            self._host_lengths[slot] = 0
 
     def release_slots(self, slots: Sequence[int]) -> tuple[Hashable, ...]:
         for slot in slots:
@@ -502,10 +504,10 @@ class BatchedNQKVLlamaRunner:
         for slot, length in zip(slots, lengths):
             if self.cache._host_lengths[slot] + length > self.max_cache_len:
                 raise RuntimeError("sequence would exceed max_cache_len")
-        for slot in slots:
-            if self.cache.manager.sequence_id(slot) is None:
-                self._generation[slot] += 1
-                self.cache.register(f"slot-{slot}-generation-{self._generation[slot]}", slot=slot)
+        fresh = [slot for slot in slots if self.cache.manager.sequence_id(slot) is None]
+        for slot in fresh:
+            self._generation[slot] += 1
+        self.cache.register_batch([(f"slot-{slot}-generation-{self._generation[slot]}", slot) for slot in fresh])
         if positions is None:
             starts = torch.tensor([self.cache._host_lengths[s] for s in slots], device=self.device)
             positions = starts[:, None] + torch.arange(width, device=self.device)[None, :]

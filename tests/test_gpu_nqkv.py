@@ -390,6 +390,37 @@ def test_pool_handles_are_generation_checked(kv):
     assert pool.page_payload_bytes == 9728 and b.page_id != c.page_id
 
 
+def test_slot_registration_in_batches_is_atomic_and_resets_the_tables(kv):
+    """register_batch / release_slots (nestquant/runtime/nqkv_batch_manager.py:394-445): a rejected
+    batch leaves no slot taken; admitted slots, neighbours or not, start from zeroed tables."""
+    manager = _manager(kv, 8, 64)
+    meta = manager.metadata
+    tables = (meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths)
+    for table in tables:
+        table.fill_(7)
+    manager.register_batch([("a", 0), ("b", 1), ("c", 2), ("d", 5), ("e", 7)])
+    taken = [0, 1, 2, 5, 7]
+    assert meta.active_mask.tolist() == [slot in taken for slot in range(8)]
+    for table in tables:
+        assert table.tolist() == [0 if slot in taken else 7 for slot in range(8)]
+    with pytest.raises(RuntimeError, match="occupied"):
+        manager.register_batch([("f", 3), ("g", 5)])
+    with pytest.raises(ValueError, match="already registered"):
+        manager.register_batch([("h", 3), ("a", 4)])
+    with pytest.raises(ValueError, match="capacity"):
+        manager.register_batch([("i", 3), ("j", 8)])
+    assert [manager.sequence_id(slot) for slot in range(8)] == ["a", "b", "c", None, None, "d", None, "e"]
+    assert meta.active_mask.tolist() == [slot in taken for slot in range(8)]
+    key = torch.randn(3, HEADS, DIM).to(torch.bfloat16)
+    _append(manager, [1, 5], [key, key[:2]], [key, key[:2]])
+    assert meta.sequence_lengths.tolist()[:6] == [0, 3, 0, 7, 7, 2]
+    assert manager.release_slots([5, 1, 3, 5]) == ("d", "b")
+    assert meta.active_mask.tolist() == [True, False, True, False, False, False, False, True]
+    assert meta.sequence_lengths.tolist() == [0, 0, 0, 7, 7, 0, 7, 0] and meta.hot_lengths.tolist()[1] == 0
+    manager.register("k", slot=1)
+    assert manager.sequence_id(1) == "k" and meta.active_mask.tolist()[1]
+
+
 def test_page_container_from_the_gpu_encoder_equals_the_reference_file(kv, golden, golden_meta):
     """PackedNQKVPage.from_tensors (HIP encoder) serialises to the bytes the reference's CPU path
     wrote for the same page (SHA-256 in the golden metadata), decodes to the reference's values, and
