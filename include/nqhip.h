@@ -268,6 +268,24 @@ int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
 size_t nq_w4a4_gemm_workspace_bytes(int m, int k, int n, int split_k, int have_decoded_activation);
 
 /*
+ * nq_w4a4_gemm for up to four weights that share one activation (q, k and v; gate and up) of at
+ * most 512 rows, in one launch: decoded BF16 activation [M, K], resolved weights, every N[i] a
+ * positive multiple of 32, BF16 outputs [M, N[i]] of their own.  The K split follows the sum of the
+ * N[i]; with a split the partial sums wait in the workspace (nq_w4a4_gemm_grouped_workspace_bytes
+ * for M, K and the sum of N) and one more launch adds them in slab order.  Same values as one
+ * nq_w4a4_gemm per weight with that split.
+ * Replaces: the three (two) calls of run_large_m_staged a prefill makes for one input
+ * (nestquant/models/fused_linear.py:316-407, nestquant/runtime/nqrt4_w4a4_mma.cu:606-667).
+ */
+int nq_w4a4_gemm_grouped(const void *act_decoded_dev, int count, const uint32_t *const *w_resolved_words_dev,
+                         const uint16_t *const *w_resolved_tails_dev, const float *const *w_norms_dev,
+                         const float *const *w_betas_dev, const int *n, const int64_t *weight_offsets,
+                         const int64_t *weight_seeds, void *const *out_bf16_dev, int m, int k,
+                         void *workspace_dev, size_t workspace_bytes, void *stream);
+
+size_t nq_w4a4_gemm_grouped_workspace_bytes(int m, int k, int n_total);
+
+/*
  * The BF16 weight [N, K] that nq_w4a4_gemv / nq_w4a4_gemm multiply by, written out:
  * bf16(decode * beta * (norm / sqrt(K))) per element, from the resolved form when given, else
  * from the NQRT4 streams.  For prefills long enough that decoding the weight once and running

@@ -51,6 +51,8 @@ SIGNATURES = {
     "nq_w4a4_gemm": (_i32, [_ptr] * 11 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
                                           _size, _ptr]),
     "nq_w4a4_gemm_workspace_bytes": (_size, [_i32, _i32, _i32, _i32, _i32]),
+    "nq_w4a4_gemm_grouped": (_i32, [_ptr, _i32] + [_ptr] * 8 + [_i32, _i32, _ptr, _size, _ptr]),
+    "nq_w4a4_gemm_grouped_workspace_bytes": (_size, [_i32, _i32, _i32]),
     "nq_bf16_gemm": (_i32, [_ptr, _ptr, _i64, _i64, _i64, _ptr, _i32, _i32, _ptr, _size, _ptr]),
     "nq_bf16_gemm_split": (_i32, [_ptr, _ptr, _i64, _i64, _ptr, _ptr, _i32, _i32, _ptr]),
     "nq_nqkv_advance": (_i32, [_ptr, _ptr, _ptr, _i32, _i32, _i32, _i32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),

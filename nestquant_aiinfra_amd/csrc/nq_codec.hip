@@ -590,12 +590,14 @@ __device__ __forceinline__ void late_stages_to_chains(const float *natural, floa
     }
 }
 
+enum LaneEncodeForm { kEightLanes = 0, kFirstLanes = 1, kEveryLane = 2 };
+
 template <int kPrologue>
 __global__ void __launch_bounds__(1024)
 quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, const float *__restrict__ betas,
                           int beta_count, float sqrt_n, uint32_t *__restrict__ codes, uint8_t *__restrict__ beta_ids,
-                          float *__restrict__ norms, uint4 *__restrict__ decoded, int slices, int rotate,
-                          InputPrologue pro) {
+                          float *__restrict__ norms, uint4 *__restrict__ decoded, int slices, int encode_form,
+                          int rotate, InputPrologue pro) {
     extern __shared__ float lds[];
     const int pitch = chain_pitch(n);
     float *chains = lds;                                  // 8 * pitch floats: the row, transposed
@@ -609,11 +611,17 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
     const int slice = blockIdx.x % slices;
     const int64_t row = blockIdx.x / slices;
     const int log_n = 31 - __builtin_clz(n);
-    // Rows of up to 4096 values (workgroups of up to eight wavefronts) encode with eight lanes per
-    // (block, beta) pair, lane c the block's coordinate c, beta (lane / 8) % 4: a quarter of the
-    // instructions per lane.  With the sixteen wavefronts of an 8192-value row that would be four
-    // encoding wavefronts per SIMD taking turns, slower than the one lane per pair of its first four.
-    const bool eight_lanes = blockDim.x <= 512;
+    // How the slice's (block, beta) pairs meet the lanes (`encode_form`):
+    //   kEightLanes  eight lanes per pair, lane c the block's coordinate c, beta (lane / 8) % 4: a quarter
+    //                of the instructions per lane, the shortest path for the few rows of a decode step
+    //                (rows of up to 4096 values; with the sixteen wavefronts of an 8192-value row that
+    //                would be four encoding wavefronts per SIMD taking turns);
+    //   kFirstLanes  one lane per pair on the first four wavefronts, one per SIMD (256 pairs a slice):
+    //                an 8192-value row of a decode step;
+    //   kEveryLane   one lane per pair on every lane, blockDim pairs at a time (four slices a row, fewer
+    //                and several turns when that would be more than two workgroups of an 8192-value row
+    //                per compute unit): the fewest instructions per pair, for prefills of some tens of rows.
+    const bool eight_lanes = encode_form == kEightLanes;
     const int c = lane & 7, bi = eight_lanes ? (lane >> 3) & 3 : tid & 3;
     const bool live = bi < beta_count;
     // requested first, used last; a launch that only runs the element-wise stage has no table
@@ -714,8 +722,8 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
         norm = __builtin_sqrtf(total);
         if (tid == 0) *row_norm_shared = norm;
     }
-    if (!eight_lanes && tid >= 256) return;                // one lane per pair: the first four wavefronts encode
-    if (eight_lanes && blockDim.x > 256) {
+    if (encode_form == kFirstLanes && tid >= 256) return;
+    if (encode_form != kFirstLanes && blockDim.x > 256) {
         __syncthreads();
         norm = *row_norm_shared;
     }
@@ -725,11 +733,7 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
     NQ_STAMP(3);
 
     if (!eight_lanes) {
-        // one lane per (block, beta) pair of the slice (256 pairs)
-        const int p = slice * 256 + tid, b = p >> 2;
-        float raw[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) raw[j] = chains[j * pitch + b];
+        // one lane per (block, beta) pair of the slice, blockDim pairs at a time
         struct LaneSink {
             uint32_t *codes; uint8_t *beta_ids; uint4 *decoded; int64_t first_block; float back;
             __device__ __forceinline__ bool wants(int) const { return true; }
@@ -749,7 +753,14 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
             __device__ __forceinline__ uint32_t counter(int, int) const { return 0; }
         };
         const LaneSink sink{codes, beta_ids, decoded, row * (n >> 3), norm / sqrt_n};
-        quantize_pair_lane<false, true>(raw, scale, beta, live, bi, 0, b, p, 14.0f, 1.0f / 14.0f, 0u, sink);
+        const int pairs_per_slice = encode_form == kFirstLanes ? 256 : (n >> 1) / slices;
+        for (int at = tid; at < pairs_per_slice; at += (int)blockDim.x) {
+            const int p = slice * pairs_per_slice + at, b = p >> 2;
+            float raw[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) raw[j] = chains[j * pitch + b];
+            quantize_pair_lane<false, true>(raw, scale, beta, live, bi, 0, b, p, 14.0f, 1.0f / 14.0f, 0u, sink);
+        }
         NQ_STAMP(4);
         return;
     }
@@ -1062,6 +1073,10 @@ namespace {
 
 // from this many values on, undithered rows go to the kernel built for throughput
 constexpr int64_t kBulkElements = 1 << 21;
+// up to this many BF16 rows of 2048, 4096 or 8192 values take the kernel with one lane per eight
+// values (measured against the row-at-a-time kernel, us, 128 / 384 rows: 7.9 / 17.2 against
+// 9.2 / 14.7 at 2048 values)
+constexpr int64_t kLanesKernelRows = 192;
 
 template <typename T, bool kDithered, int kPrologue = 0>
 int launch_quantize(const void *x, int64_t rows, int n, int q, const float *betas, int beta_count,
@@ -1088,15 +1103,22 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
                            hadamard_stage_dtype, prologue);
         return nq::check_launch("nq_quantize_rows");
     }
-    // decode steps: up to 16 BF16 rows of 2048, 4096 or 8192 values, q = 14, every operand
-    // 16-byte aligned: one lane per eight values, each row repeated over as many workgroups as it has
-    // slices of 256 (block, beta) pairs
+    // BF16 rows of 2048, 4096 or 8192 values, q = 14, every operand 16-byte aligned, fewer than the
+    // throughput kernel's: one lane per eight values, each row repeated over as many workgroups as
+    // it has slices.  Up to 16 rows (a decode step) are laid out for the shortest path through one row,
+    // more rows (a prefill chunk) for the fewest instructions.
     if (std::is_same<T, uint16_t>::value && !kDithered && q == 14 && (n == 2048 || n == 4096 || n == 8192) &&
-        rows <= 16 && nq::aligned(x, 16)) {
-        // a workgroup of n / 8 lanes encodes n / 256 blocks per pass (eight lanes per (block, beta) pair):
-        // 32 slices of one pass each while that keeps the launch within one workgroup per compute unit
-        // (n <= 4096; an 8192-value row keeps one lane per pair: slices of 256 pairs)
-        const int slices = n > 4096 ? n / 512 : (rows * 32 <= 256 ? 32 : 16);
+        nq::aligned(x, 16) && (rows <= 16 || (kPrologue != 3 && rows <= kLanesKernelRows))) {
+        // decode step: a workgroup of n / 8 lanes encodes n / 256 blocks per pass with eight lanes per
+        // (block, beta) pair: 32 slices of one pass each while that keeps the launch within one
+        // workgroup per compute unit (n <= 4096); an 8192-value row keeps one lane per pair, slices of
+        // 256 pairs.  Prefill chunk: every lane one pair, four slices a row.
+        const int form = rows > 16 ? nq::kEveryLane : (n > 4096 ? nq::kFirstLanes : nq::kEightLanes);
+        int slices = n > 4096 ? n / 512 : (rows * 32 <= 256 ? 32 : 16);
+        if (form == nq::kEveryLane) {
+            // a workgroup of 1024 (512) lanes per compute unit (two) at most: 4 slices, else 2
+            slices = n <= 2048 || rows * 4 * (n / 2048) <= 1024 ? 4 : 2;
+        }
         const size_t lds_bytes = (size_t)(8 * ((n >> 3) + 8) + n + 4 + 8) * sizeof(float);   // + norm, beta choices
         auto kernel = nq::quantize_row_lanes_kernel<kPrologue>;
         if (lds_bytes > 48 * 1024) {
@@ -1109,7 +1131,7 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
         hipLaunchKernelGGL(kernel, dim3((unsigned)(rows * slices)), dim3(n / 8), lds_bytes, stream,
                            reinterpret_cast<const uint16_t *>(x), rows, n, betas, beta_count, (float)sqrt((double)n),
                            reinterpret_cast<uint32_t *>(codes), beta_ids, norms, reinterpret_cast<uint4 *>(decoded),
-                           slices, hadamard_stage_dtype >= 0 ? 1 : 0, prologue);
+                           slices, form, hadamard_stage_dtype >= 0 ? 1 : 0, prologue);
         return nq::check_launch("nq_quantize_rows");
     }
     const int pairs_per_row = n / 2;

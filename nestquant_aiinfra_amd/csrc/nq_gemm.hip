@@ -36,19 +36,43 @@ constexpr int kGemmBK = 128;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-// TILES: token tiles (of 32 rows) per wavefront.  kResolved: the weight comes as resolved
-// blocks (w_words / w_tails, see nq_e8.hip.h) instead of NQRT4 code words and beta bytes.
+// Up to four weights that share an activation (q, k and v; gate and up): one launch takes their
+// channels one after the other, a workgroup's 32 channels always inside one weight (every weight but
+// the last has a multiple of 32 channels).
+constexpr int kGemmMaxGroups = 4;
+struct GemmWeights {
+    const uint32_t *words[kGemmMaxGroups];        // NQRT4 code words, or resolved words
+    const uint16_t *tails[kGemmMaxGroups];        // resolved tails
+    const uint8_t *beta_ids[kGemmMaxGroups];
+    const float *norms[kGemmMaxGroups];
+    const float *betas[kGemmMaxGroups];
+    uint16_t *out_bf16[kGemmMaxGroups];           // BF16 [m_rows][channels of the weight], or null
+    uint32_t seed_plus_offset[kGemmMaxGroups];
+    int end[kGemmMaxGroups];                      // channels of the weights up to and including this one
+};
+
+// TILES: token tiles (of 32 rows) per wavefront.  kResolved: the weights come as resolved
+// blocks (words / tails, see nq_e8.hip.h) instead of NQRT4 code words and beta bytes.
+// FP32 results (partial sums of K slab blockIdx.y, or the output itself) are laid out weight by
+// weight: out_f32[(slab * n_total + first channel of the weight) * m_rows + m * channels + n].
 template <int TILES, bool kResolved>
 __global__ void __launch_bounds__(kGemmThreads)
 w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
-                 const uint32_t *__restrict__ w_words, const uint16_t *__restrict__ w_tails,
-                 const uint8_t *__restrict__ w_beta_ids,
-                 const float *__restrict__ w_norms, const float *__restrict__ w_betas,
-                 int m_rows, int k_size, int n_size, int k_slab, uint32_t seed_plus_offset,
-                 float sqrt_k, float *__restrict__ out_f32, uint16_t *__restrict__ out_bf16) {
+                 GemmWeights weights, int m_rows, int k_size, int n_total, int k_slab, float sqrt_k,
+                 float *__restrict__ out_f32) {
     __shared__ uint4 b_tile[2][kGemmBK / 16][64];          // 2 x 8 K-steps x 64 lanes x 16 B = 16 KiB
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n0 = blockIdx.x * kGemmBN;
+    const int channel0 = blockIdx.x * kGemmBN;
+    const int group = (channel0 >= weights.end[0]) + (channel0 >= weights.end[1]) + (channel0 >= weights.end[2]);
+    const int group_first = group ? weights.end[group - 1] : 0;
+    const int n0 = channel0 - group_first, n_size = weights.end[group] - group_first;
+    const uint32_t *__restrict__ w_words = weights.words[group];
+    const uint16_t *__restrict__ w_tails = weights.tails[group];
+    const uint8_t *__restrict__ w_beta_ids = weights.beta_ids[group];
+    const float *__restrict__ w_norms = weights.norms[group];
+    const float *__restrict__ w_betas = weights.betas[group];
+    uint16_t *__restrict__ out_bf16 = weights.out_bf16[group];
+    const uint32_t seed_plus_offset = weights.seed_plus_offset[group];
     const int k_begin = blockIdx.y * k_slab;
     const int blocks_per_row = k_size >> 3;
 
@@ -156,7 +180,7 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
                 const int m = m_base + (r & 3) + 8 * (r >> 2);
                 if (m < m_rows) {
                     if (out_f32)
-                        out_f32[((int64_t)blockIdx.y * m_rows + m) * n_size + n] = acc[t][r];
+                        out_f32[((int64_t)blockIdx.y * n_total + group_first) * m_rows + (int64_t)m * n_size + n] = acc[t][r];
                     else
                         out_bf16[(int64_t)m * n_size + n] = f32_to_bf16(acc[t][r]);
                 }
@@ -258,6 +282,25 @@ int pick_gemm_split(int k, int n, int requested) {
     return split;
 }
 
+// One launch of the fused kernel over `rows` tokens and the n_total channels of `weights`.
+int launch_fused_gemm(const uint16_t *act, const nq::GemmWeights &weights, bool resolved, int rows, int k, int n_total,
+                      int split, float *out_f32, hipStream_t s) {
+    const dim3 grid((unsigned)((n_total + nq::kGemmBN - 1) / nq::kGemmBN), (unsigned)split);
+    const float sqrt_k = (float)sqrt((double)k);
+#define NQ_LAUNCH_GEMM(TILES, RESOLVED)                                                                     \
+    hipLaunchKernelGGL((nq::w4a4_gemm_kernel<TILES, RESOLVED>), grid, dim3(nq::kGemmThreads), 0, s, act,    \
+                       weights, rows, k, n_total, k / split, sqrt_k, out_f32)
+    if (rows <= 8 * 32) {
+        if (resolved) NQ_LAUNCH_GEMM(1, true);
+        else NQ_LAUNCH_GEMM(1, false);
+    } else {
+        if (resolved) NQ_LAUNCH_GEMM(2, true);
+        else NQ_LAUNCH_GEMM(2, false);
+    }
+#undef NQ_LAUNCH_GEMM
+    return nq::check_launch("nq_w4a4_gemm");
+}
+
 }  // namespace
 
 extern "C" size_t nq_w4a4_gemm_workspace_bytes(int m, int k, int n, int split_k, int have_decoded_activation) {
@@ -341,31 +384,21 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
         return nq::launch_bf16_gemm(act, weight_bf16, out_dev, m, n, k, -1, 0, dense_partials,
                                     workspace_bytes > used ? workspace_bytes - used : 0, s, nullptr);
     }
-    const uint32_t seed_plus_offset = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
-    const float sqrt_k = (float)sqrt((double)k);
-    const dim3 grid((unsigned)((n + nq::kGemmBN - 1) / nq::kGemmBN), (unsigned)split);
-    const uint32_t *wc = resolved ? w_resolved_words_dev : reinterpret_cast<const uint32_t *>(w_codes_dev);
+    nq::GemmWeights weights = {};
+    weights.words[0] = resolved ? w_resolved_words_dev : reinterpret_cast<const uint32_t *>(w_codes_dev);
+    weights.tails[0] = w_resolved_tails_dev;
+    weights.beta_ids[0] = w_beta_ids_dev;
+    weights.norms[0] = w_norms_dev;
+    weights.betas[0] = w_betas_dev;
+    weights.seed_plus_offset[0] = (uint32_t)((uint64_t)weight_seed + (uint64_t)weight_offset * 8u);
+    for (int g = 0; g < nq::kGemmMaxGroups; g++) weights.end[g] = n;
     const size_t out_row_bytes = (size_t)n * (out_dtype == NQ_F32 ? 4 : 2);
-
     for (int m0 = 0; m0 < m; m0 += kChunkRows) {
         const int rows = m - m0 < kChunkRows ? m - m0 : kChunkRows;
         char *out_chunk = reinterpret_cast<char *>(out_dev) + (size_t)m0 * out_row_bytes;
         float *target_f32 = split > 1 ? partials : (out_dtype == NQ_F32 ? (float *)out_chunk : nullptr);
-        uint16_t *target_bf16 = (split > 1 || out_dtype == NQ_F32) ? nullptr : (uint16_t *)out_chunk;
-        const uint16_t *act_chunk = act + (size_t)m0 * k;
-#define NQ_LAUNCH_GEMM(TILES, RESOLVED)                                                                       \
-    hipLaunchKernelGGL((nq::w4a4_gemm_kernel<TILES, RESOLVED>), grid, dim3(nq::kGemmThreads), 0, s, act_chunk, \
-                       wc, w_resolved_tails_dev, w_beta_ids_dev, w_norms_dev, w_betas_dev, rows, k, n,          \
-                       k / split, seed_plus_offset, sqrt_k, target_f32, target_bf16)
-        if (rows <= 8 * 32) {
-            if (resolved) NQ_LAUNCH_GEMM(1, true);
-            else NQ_LAUNCH_GEMM(1, false);
-        } else {
-            if (resolved) NQ_LAUNCH_GEMM(2, true);
-            else NQ_LAUNCH_GEMM(2, false);
-        }
-#undef NQ_LAUNCH_GEMM
-        int status = nq::check_launch("nq_w4a4_gemm");
+        weights.out_bf16[0] = (split > 1 || out_dtype == NQ_F32) ? nullptr : (uint16_t *)out_chunk;
+        int status = launch_fused_gemm(act + (size_t)m0 * k, weights, resolved, rows, k, n, split, target_f32, s);
         if (status != NQ_OK) return status;
         if (split > 1) {
             status = nq::launch_splitk_reduce(partials, split, (int64_t)rows * n, out_chunk, out_dtype, s);
@@ -373,6 +406,75 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
         }
     }
     return NQ_OK;
+}
+
+extern "C" size_t nq_w4a4_gemm_grouped_workspace_bytes(int m, int k, int n_total) {
+    if (m < 1 || n_total < 1 || k < 1) return 0;
+    const int split = pick_gemm_split(k, n_total, 0);
+    return split > 1 ? (size_t)split * (size_t)m * (size_t)n_total * sizeof(float) : 0;
+}
+
+extern "C" int nq_w4a4_gemm_grouped(const void *act_decoded_dev, int count, const uint32_t *const *w_resolved_words_dev,
+                                    const uint16_t *const *w_resolved_tails_dev, const float *const *w_norms_dev,
+                                    const float *const *w_betas_dev, const int *n, const int64_t *weight_offsets,
+                                    const int64_t *weight_seeds, void *const *out_bf16_dev, int m, int k,
+                                    void *workspace_dev, size_t workspace_bytes, void *stream) {
+    NQ_REQUIRE(count >= 1 && count <= nq::kGemmMaxGroups, NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemm_grouped: between one and four weights, got %d", count);
+    NQ_REQUIRE(m >= 1 && m <= kChunkRows, NQ_ERR_SHAPE, "nq_w4a4_gemm_grouped: M = %d is outside [1, 512]", m);
+    NQ_REQUIRE(k >= nq::kGemmBK && k % nq::kGemmBK == 0, NQ_ERR_SHAPE,
+               "nq_w4a4_gemm_grouped: K = %d must be a positive multiple of 128", k);
+    NQ_REQUIRE(act_decoded_dev && w_resolved_words_dev && w_resolved_tails_dev && w_norms_dev && w_betas_dev && n &&
+                   weight_offsets && weight_seeds && out_bf16_dev,
+               NQ_ERR_ARGUMENT, "nq_w4a4_gemm_grouped: null pointer");
+    NQ_REQUIRE(nq::aligned(act_decoded_dev, 16), NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemm_grouped: the decoded activation must be 16-byte aligned");
+    nq::GemmWeights weights = {};
+    nq::ReduceOutputs outputs = {};
+    int64_t n_total = 0;
+    for (int g = 0; g < count; g++) {
+        NQ_REQUIRE(n[g] >= 32 && n[g] % 32 == 0, NQ_ERR_SHAPE,
+                   "nq_w4a4_gemm_grouped: N = %d of weight %d is not a positive multiple of 32", n[g], g);
+        NQ_REQUIRE(w_resolved_words_dev[g] && w_resolved_tails_dev[g] && w_norms_dev[g] && w_betas_dev[g] &&
+                       out_bf16_dev[g], NQ_ERR_ARGUMENT, "nq_w4a4_gemm_grouped: null pointer for weight %d", g);
+        NQ_REQUIRE(nq::aligned(w_resolved_words_dev[g], 4) && nq::aligned(w_resolved_tails_dev[g], 2) &&
+                       nq::aligned(out_bf16_dev[g], 2), NQ_ERR_ARGUMENT,
+                   "nq_w4a4_gemm_grouped: misaligned stream or output of weight %d", g);
+        NQ_REQUIRE(weight_seeds[g] >= 0 && weight_seeds[g] < ((int64_t)1 << 31), NQ_ERR_ARGUMENT,
+                   "nq_w4a4_gemm_grouped: seed must be in [0, 2**31)");
+        NQ_REQUIRE(weight_offsets[g] >= 0 && weight_offsets[g] + (int64_t)n[g] * (k / 8) <= ((int64_t)1 << 28),
+                   NQ_ERR_SHAPE, "nq_w4a4_gemm_grouped: block range exceeds the stateless dither counter space");
+        n_total += n[g];
+        NQ_REQUIRE(n_total <= ((int64_t)1 << 24), NQ_ERR_SHAPE, "nq_w4a4_gemm_grouped: too many channels");
+        weights.words[g] = w_resolved_words_dev[g];
+        weights.tails[g] = w_resolved_tails_dev[g];
+        weights.norms[g] = w_norms_dev[g];
+        weights.betas[g] = w_betas_dev[g];
+        weights.out_bf16[g] = reinterpret_cast<uint16_t *>(out_bf16_dev[g]);
+        weights.seed_plus_offset[g] = (uint32_t)((uint64_t)weight_seeds[g] + (uint64_t)weight_offsets[g] * 8u);
+        weights.end[g] = (int)n_total;
+        outputs.out[g] = weights.out_bf16[g];
+        outputs.end[g] = (int64_t)m * n_total;
+    }
+    for (int g = count; g < nq::kGemmMaxGroups; g++) {
+        weights.end[g] = (int)n_total;
+        outputs.out[g] = outputs.out[count - 1];
+        outputs.end[g] = (int64_t)m * n_total;
+    }
+    const int split = pick_gemm_split(k, (int)n_total, 0);
+    const size_t need = split > 1 ? (size_t)split * m * n_total * sizeof(float) : 0;
+    NQ_REQUIRE(need == 0 || (workspace_dev && workspace_bytes >= need), NQ_ERR_WORKSPACE,
+               "nq_w4a4_gemm_grouped: needs a %zu-byte workspace, got %zu", need, workspace_bytes);
+    NQ_REQUIRE(need == 0 || nq::aligned(workspace_dev, 16), NQ_ERR_ARGUMENT,
+               "nq_w4a4_gemm_grouped: workspace must be 16-byte aligned");
+    const hipStream_t s = (hipStream_t)stream;
+    float *partials = split > 1 ? reinterpret_cast<float *>(workspace_dev) : nullptr;
+    if (split > 1)
+        for (int g = 0; g < nq::kGemmMaxGroups; g++) weights.out_bf16[g] = nullptr;
+    int status = launch_fused_gemm(reinterpret_cast<const uint16_t *>(act_decoded_dev), weights, true, m, k, (int)n_total,
+                                   split, partials, s);
+    if (status != NQ_OK || split == 1) return status;
+    return nq::launch_splitk_reduce_grouped(partials, split, (int64_t)m * n_total, outputs, s);
 }
 
 extern "C" int nq_w4a4_decode_weight(const uint8_t *w_codes_dev, const uint8_t *w_beta_ids_dev,

@@ -56,6 +56,34 @@ inline int launch_splitk_reduce(const float *partials, int split, int64_t count,
     return check_launch("split-K reduce");
 }
 
+// The same sum for partial results laid out weight by weight (the grouped launch of the fused
+// kernel): elements [end[g - 1], end[g]) of a slice belong to out[g], BF16, in the same order.
+constexpr int kReduceMaxOutputs = 4;
+struct ReduceOutputs {
+    uint16_t *out[kReduceMaxOutputs];
+    int64_t end[kReduceMaxOutputs];
+};
+
+static __global__ void __launch_bounds__(256)
+splitk_reduce_grouped_kernel(const float *__restrict__ partial, int split, int64_t count, ReduceOutputs outputs) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float total = 0.0f;
+    for (int s = 0; s < split; s++) total = total + partial[(int64_t)s * count + i];
+    // selects, not an index into the argument: the struct stays in scalar registers
+    const bool first = i < outputs.end[0], second = i < outputs.end[1], third = i < outputs.end[2];
+    uint16_t *out = first ? outputs.out[0] : (second ? outputs.out[1] : (third ? outputs.out[2] : outputs.out[3]));
+    const int64_t begin = first ? 0 : (second ? outputs.end[0] : (third ? outputs.end[1] : outputs.end[2]));
+    out[i - begin] = f32_to_bf16(total);
+}
+
+inline int launch_splitk_reduce_grouped(const float *partials, int split, int64_t count, const ReduceOutputs &outputs,
+                                        hipStream_t stream) {
+    hipLaunchKernelGGL(splitk_reduce_grouped_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                       partials, split, count, outputs);
+    return check_launch("split-K reduce");
+}
+
 inline size_t align256(size_t bytes) { return (bytes + 255) & ~(size_t)255; }
 
 }  // namespace nq

@@ -658,38 +658,68 @@ def bf16_gemm(rows: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split
     return out
 
 
+FUSED_GROUP_MAX_ROWS = 512                  # one chunk of the fused kernel
+
+
+def _fused_group(activation: PreparedNQA4Activation, weights: Sequence[PreparedNQRTLinear]) -> bool:
+    """A group the fused kernel takes in one launch: a prefill below the decode-once size."""
+    return (MATRIX_CORE_GEMV_ROWS < activation.token_count < DECODE_ONCE_ROWS and 2 <= len(weights) <= 4
+            and all(w.resolved_words is not None and w.record.indices.shape[0] % 32 == 0 for w in weights))
+
+
 def can_use_w4a4_gemm_grouped(activation: PreparedNQA4Activation, weights: Sequence[PreparedNQRTLinear]) -> bool:
-    """Whether `linear_packed_w4a4_gemm_grouped` takes these projections of one activation: a
-    long prefill (the decode-once route), two or three weights, every N a multiple of 256."""
+    """Whether `linear_packed_w4a4_gemm_grouped` takes these projections of one decoded activation:
+    a long prefill (the decode-once route: two or three weights, every N a multiple of 256), or a
+    shorter one of more than 16 rows (the fused kernel: up to four resolved weights, every N a
+    multiple of 32)."""
     k = activation.feature_count
-    return (2 <= len(weights) <= 3 and activation.token_count >= DECODE_ONCE_ROWS and k % 128 == 0
-            and activation.decoded is not None
-            and all(w.record.feature_count == k and w.record.indices.shape[0] % 256 == 0 for w in weights))
+    if k % 128 != 0 or activation.decoded is None or any(w.record.feature_count != k for w in weights):
+        return False
+    if _fused_group(activation, weights):
+        return True
+    return (2 <= len(weights) <= 3 and activation.token_count >= DECODE_ONCE_ROWS
+            and all(w.record.indices.shape[0] % 256 == 0 for w in weights))
 
 
 def linear_packed_w4a4_gemm_grouped(activation: PreparedNQA4Activation,
                                     weights: Sequence[PreparedNQRTLinear]) -> list[torch.Tensor]:
-    """The linears of two or three weights that share one activation (q, k and v; gate and up) in a
-    long prefill: every weight is decoded once into its rows of one BF16 scratch, and one dense
-    matrix-core GEMM over the stacked rows stores each projection's columns to a BF16 [M, N_i]
-    output of its own.  Same values as one `linear_packed_w4a4_mma_chunked_staged` per weight."""
+    """The linears of the weights that share one activation (q, k and v; gate and up) in a prefill,
+    as one product.  From 288 rows on every weight is decoded once into its rows of one BF16 scratch
+    and one dense matrix-core GEMM over the stacked rows stores each projection's columns to a BF16
+    [M, N_i] output of its own; below, one launch of the fused kernel walks the channels of all the
+    weights.  Same values as one `linear_packed_w4a4_mma_chunked_staged` per weight."""
     if not can_use_w4a4_gemm_grouped(activation, weights):
-        raise ValueError("grouped prefill linears take 2 or 3 weights of one decoded activation of at least "
-                         f"{DECODE_ONCE_ROWS} rows, K a multiple of 128 and every N a multiple of 256")
+        raise ValueError("grouped prefill linears take the weights of one decoded activation, K a multiple of 128: "
+                         f"2 or 3 with every N a multiple of 256 from {DECODE_ONCE_ROWS} rows on, up to 4 resolved "
+                         f"ones with every N a multiple of 32 between {MATRIX_CORE_GEMV_ROWS + 1} rows and that")
     rows = activation.decoded.reshape(activation.token_count, activation.feature_count)
     device = _native.require_cuda(rows)
     m, k = rows.shape
     sizes = [int(w.record.indices.shape[0]) for w in weights]
-    stacked = _workspace(device, sum(sizes) * k * 2)[: sum(sizes) * k * 2].view(torch.bfloat16).view(sum(sizes), k)
-    first = 0
-    for weight, size in zip(weights, sizes):
-        decode_weight_bf16(weight, out=stacked[first:first + size])
-        first += size
+    count = len(sizes)
     outs = [torch.empty((m, size), dtype=torch.bfloat16, device=device) for size in sizes]
-    widths = (ctypes.c_int64 * len(sizes))(*sizes)
-    pointers = (ctypes.c_void_p * len(sizes))(*[out.data_ptr() for out in outs])
-    _native.check(_native.library().nq_bf16_gemm_split(rows.data_ptr(), stacked.data_ptr(), m, k, pointers, widths,
-                                                       len(sizes), -1, _native.stream_handle(device)))
+    pointers = (ctypes.c_void_p * count)(*[out.data_ptr() for out in outs])
+    lib = _native.library()
+    if _fused_group(activation, weights):
+        array = ctypes.c_void_p * count
+        need = lib.nq_w4a4_gemm_grouped_workspace_bytes(m, k, sum(sizes))
+        workspace = _workspace(device, need) if need else None
+        _native.check(lib.nq_w4a4_gemm_grouped(
+            rows.data_ptr(), count, array(*[w.resolved_words.data_ptr() for w in weights]),
+            array(*[w.resolved_tails.data_ptr() for w in weights]), array(*[w.row_norms.data_ptr() for w in weights]),
+            array(*[w.beta_table.data_ptr() for w in weights]), (ctypes.c_int * count)(*sizes),
+            (ctypes.c_int64 * count)(*([0] * count)),
+            (ctypes.c_int64 * count)(*[int(w.record.dither_seed) for w in weights]), pointers, m, k,
+            None if workspace is None else workspace.data_ptr(), need, _native.stream_handle(device)))
+    else:
+        stacked = _workspace(device, sum(sizes) * k * 2)[: sum(sizes) * k * 2].view(torch.bfloat16).view(sum(sizes), k)
+        first = 0
+        for weight, size in zip(weights, sizes):
+            decode_weight_bf16(weight, out=stacked[first:first + size])
+            first += size
+        widths = (ctypes.c_int64 * count)(*sizes)
+        _native.check(lib.nq_bf16_gemm_split(rows.data_ptr(), stacked.data_ptr(), m, k, pointers, widths, count, -1,
+                                             _native.stream_handle(device)))
     return [out.reshape(*activation.original_shape[:-1], size) for out, size in zip(outs, sizes)]
 
 

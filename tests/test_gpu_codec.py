@@ -86,6 +86,10 @@ def test_quantize_rows_long_rows_match_reference_golden(rt, golden_long_rows):
     (1, 2048, "student", torch.bfloat16),
     (8, 8192, "student", torch.bfloat16),
     (17, 2048, "outlier", torch.bfloat16),
+    (40, 8192, "student", torch.bfloat16),      # prefill chunks: every lane of the lanes kernel one (block, beta) pair
+    (130, 4096, "outlier", torch.bfloat16),
+    (190, 2048, "student", torch.bfloat16),
+    (100, 8192, "outlier", torch.bfloat16),     # two slices a row, two turns a lane
     (40, 2048, "outlier", torch.float32),
     (128, 64, "normal", torch.bfloat16),        # one KV page side: 16 tokens x 8 heads
     (5, 32, "normal", torch.float32),
@@ -234,19 +238,26 @@ def test_errors_are_reported_like_the_reference(rt):
 @pytest.mark.parametrize("n", [2048, 4096, 8192])
 @pytest.mark.parametrize("rows", [1, 3, 16])
 def test_decode_size_encoder_equals_the_many_row_encoder(rt, rows, n):
-    """Up to 16 BF16 rows of 2048, 4096 or 8192 values take the one-lane-per-eight-values kernel,
-    more rows the row-at-a-time or the bulk kernel: the same rows must come out of either bit for bit
-    (rotation included), zero rows and rows of huge and tiny magnitude among them."""
+    """BF16 rows of 2048, 4096 or 8192 values take the one-lane-per-eight-values kernel while they
+    are fewer than two million values (up to 16 rows with eight lanes or the first four wavefronts
+    on the (block, beta) pairs, more rows with every lane on one pair), and the bulk kernel from
+    there on: the same rows must come out of all three bit for bit (rotation included), zero rows
+    and rows of huge and tiny magnitude among them."""
     g = torch.Generator().manual_seed(rows * n)
-    x = torch.randn(17, n, generator=g) * torch.logspace(-15, 15, 17).unsqueeze(-1)
+    total = (1 << 21) // n
+    x = torch.randn(total, n, generator=g) * torch.logspace(-15, 15, total).unsqueeze(-1)
+    x[:17] = torch.randn(17, n, generator=g) * torch.logspace(-15, 15, 17).unsqueeze(-1)
     x[min(2, rows - 1)] = 0.0
     x = x.to(torch.bfloat16).cuda()
     table = _table(ACTIVATION_BETAS)
     for rotate in (True, False):
         few = rt.quantize_activation_cuda(x[:rows].contiguous(), q=Q, betas=ACTIVATION_BETAS, beta_table=table,
                                           hadamard=rotate)
+        some = rt.quantize_activation_cuda(x[:41].contiguous(), q=Q, betas=ACTIVATION_BETAS, beta_table=table,
+                                           hadamard=rotate)
         many = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS, beta_table=table, hadamard=rotate)
-        assert torch.equal(few.code_payload, many.code_payload[: rows * n // 2]), rotate
-        assert torch.equal(few.beta_payload, many.beta_payload[: rows * n // 32]), rotate
-        assert torch.equal(few.row_norms, many.row_norms[:rows]), rotate
-        assert torch.equal(few.decoded, many.decoded[:rows]), rotate
+        for part, count in ((few, rows), (some, 41)):
+            assert torch.equal(part.code_payload, many.code_payload[: count * n // 2]), (rotate, count)
+            assert torch.equal(part.beta_payload, many.beta_payload[: count * n // 32]), (rotate, count)
+            assert torch.equal(part.row_norms, many.row_norms[:count]), (rotate, count)
+            assert torch.equal(part.decoded, many.decoded[:count]), (rotate, count)

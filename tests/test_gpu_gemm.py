@@ -198,9 +198,37 @@ def test_grouped_prefill_linears_equal_one_call_per_weight(rt, oracle, m, k, siz
         alone = rt.linear_packed_w4a4_mma_chunked_staged(activation, weight)
         assert out.dtype == torch.bfloat16 and tuple(out.shape) == (m, n_out)
         assert torch.equal(out, alone), n_out
-    # fewer rows than the decode-once route takes, or a width that a tile could straddle: refused
-    short = _activation(rt, oracle, 64, k, seed=7101)
+    # a decode step's rows (the grouped GEMV's), or a single weight: refused
+    short = _activation(rt, oracle, 16, k, seed=7101)
     assert not rt.can_use_w4a4_gemm_grouped(short, weights)
     with pytest.raises(ValueError, match="grouped prefill linears"):
         rt.linear_packed_w4a4_gemm_grouped(short, weights)
     assert not rt.can_use_w4a4_gemm_grouped(activation, weights[:1])
+
+
+@pytest.mark.parametrize("m,k,sizes", [(17, 512, (256, 64, 64)), (128, 2048, (2048, 512, 512)), (287, 1024, (512, 512)),
+                                       (40, 256, (32, 64, 96, 32)), (128, 2048, (8192, 8192)), (100, 8192, (64, 32))])
+def test_grouped_short_prefill_linears_equal_one_launch_per_weight(rt, oracle, m, k, sizes):
+    """Below the decode-once size one launch of the fused kernel walks the channels of all the
+    weights (`nq_w4a4_gemm_grouped`): every output is bit for bit what the kernel gives for its
+    weight alone with the K split the group runs with (the split follows the sum of the widths)."""
+    from nestquant_aiinfra_amd.runtime.w4a4_linear import _gemm
+    weights = []
+    for i, n_out in enumerate(sizes):
+        g = torch.Generator().manual_seed(7200 + i)
+        w = torch.from_numpy(oracle.hadamard((0.02 * torch.randn(n_out, k, generator=g)).numpy()))
+        record = rt.quantize_weight_nqrt4(w.cuda(), q=Q, betas=WEIGHT_BETAS, dither_seed=20280000 + i, tensor_name=f"w{i}")
+        weights.append(rt.prepare_fused_linear(record, device="cuda"))
+    activation = _activation(rt, oracle, m, k, seed=7300)
+    assert rt.can_use_w4a4_gemm_grouped(activation, weights)
+    grouped = rt.linear_packed_w4a4_gemm_grouped(activation, weights)
+    split, tiles = 1, sum(sizes) // 32
+    while split < 16 and tiles * split < 256 and (k // (split * 2)) % 128 == 0:
+        split *= 2
+    for out, weight, n_out in zip(grouped, weights, sizes):
+        alone = _gemm(activation, weight, output_dtype=torch.bfloat16, split_k=split)
+        assert out.dtype == torch.bfloat16 and tuple(out.shape) == (m, n_out)
+        assert torch.equal(out, alone), (n_out, split)
+    # the same call twice gives the same bits (the slabs are added in order)
+    again = rt.linear_packed_w4a4_gemm_grouped(activation, weights)
+    assert all(torch.equal(a, b) for a, b in zip(grouped, again))
