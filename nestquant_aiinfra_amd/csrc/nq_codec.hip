@@ -590,11 +590,11 @@ __device__ __forceinline__ void late_stages_to_chains(const float *natural, floa
     }
 }
 
-enum LaneEncodeForm { kEightLanes = 0, kFirstLanes = 1, kEveryLane = 2 };
+enum LaneEncodeForm { kEightLanes = 0, kFirstLanes = 1, kEveryLane = 2, kBlockLanes = 3 };
 
 template <int kPrologue>
 __global__ void __launch_bounds__(1024)
-quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, const float *__restrict__ betas,
+quantize_row_lanes_kernel(const void *__restrict__ x_any, int x_is_f32, int64_t rows, int n, const float *__restrict__ betas,
                           int beta_count, float sqrt_n, uint32_t *__restrict__ codes, uint8_t *__restrict__ beta_ids,
                           float *__restrict__ norms, uint4 *__restrict__ decoded, int slices, int encode_form,
                           int rotate, InputPrologue pro) {
@@ -620,7 +620,11 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
     //                an 8192-value row of a decode step;
     //   kEveryLane   one lane per pair on every lane, blockDim pairs at a time (four slices a row, fewer
     //                and several turns when that would be more than two workgroups of an 8192-value row
-    //                per compute unit): the fewest instructions per pair, for prefills of some tens of rows.
+    //                per compute unit): for prefills of some tens of rows;
+    //   kBlockLanes  one lane per block, its betas in turn, only the winner turned into a code word and
+    //                the coset reduction skipped where every block of the wavefront lies inside the
+    //                Voronoi cell (quantize_block_betas_in_turn): the fewest instructions per block, for
+    //                hundreds of rows and more, one workgroup a row.
     const bool eight_lanes = encode_form == kEightLanes;
     const int c = lane & 7, bi = eight_lanes ? (lane >> 3) & 3 : tid & 3;
     const bool live = bi < beta_count;
@@ -629,7 +633,13 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
     NQ_STAMP(0);
 
     float v[8];
-    lane_prologue<kPrologue>(x, pro, row, n, slice == 0, wave_sums, v);
+    if (kPrologue == 0 && x_is_f32) {                     // plain float32 rows (never rotated here)
+        const float4 *at = reinterpret_cast<const float4 *>(x_any) + ((row * n) >> 2) + 2 * tid;
+        const float4 lo = at[0], hi = at[1];
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    } else {
+        lane_prologue<kPrologue>(reinterpret_cast<const uint16_t *>(x_any), pro, row, n, slice == 0, wave_sums, v);
+    }
     if (codes == nullptr) return;                         // element-wise stage only
     NQ_STAMP(1);
 
@@ -753,6 +763,18 @@ quantize_row_lanes_kernel(const uint16_t *__restrict__ x, int64_t rows, int n, c
             __device__ __forceinline__ uint32_t counter(int, int) const { return 0; }
         };
         const LaneSink sink{codes, beta_ids, decoded, row * (n >> 3), norm / sqrt_n};
+        if (encode_form == kBlockLanes) {
+            const int blocks_per_slice = (n >> 3) / slices;
+            for (int at = tid; at < blocks_per_slice; at += (int)blockDim.x) {
+                const int b = slice * blocks_per_slice + at;
+                float raw[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) raw[j] = chains[j * pitch + b];
+                quantize_block_betas_in_turn(raw, scale, betas, beta_count, 14.0f, 1.0f / 14.0f, 0, b, sink);
+            }
+            NQ_STAMP(4);
+            return;
+        }
         const int pairs_per_slice = encode_form == kFirstLanes ? 256 : (n >> 1) / slices;
         for (int at = tid; at < pairs_per_slice; at += (int)blockDim.x) {
             const int p = slice * pairs_per_slice + at, b = p >> 2;
@@ -1073,16 +1095,55 @@ namespace {
 
 // from this many values on, undithered rows go to the kernel built for throughput
 constexpr int64_t kBulkElements = 1 << 21;
-// up to this many BF16 rows of 2048, 4096 or 8192 values take the kernel with one lane per eight
-// values (measured against the row-at-a-time kernel, us, 128 / 384 rows: 7.9 / 17.2 against
-// 9.2 / 14.7 at 2048 values)
+// Rows of 2048, 4096 or 8192 values on the kernel with one lane per eight values: up to
+// kLanesKernelRows rows with every lane on one (block, beta) pair (us against the row-at-a-time kernel,
+// 128 / 384 rows of 2048 values: 7.9 / 17.2 against 9.2 / 14.7), from there to kBlockLanesRows rows (and
+// whatever is too small for the many-row kernel) with one lane per block (384 rows of 2048 / 8192 values:
+// 13.5 / 42.1 against 14.6 / 47.5; 1024 rows: 21.5 / 84.0 against the many-row kernel's 21.5 / 77.5)
 constexpr int64_t kLanesKernelRows = 192;
+constexpr int64_t kBlockLanesRows = 512;
 
 template <typename T, bool kDithered, int kPrologue = 0>
 int launch_quantize(const void *x, int64_t rows, int n, int q, const float *betas, int beta_count,
                     uint32_t seed_plus_offset, uint8_t *codes, uint8_t *beta_ids, float *norms,
                     void *decoded, int hadamard_stage_dtype, hipStream_t stream,
                     nq::InputPrologue prologue = nq::InputPrologue{}) {
+    // Rows of 2048, 4096 or 8192 values, q = 14, every operand 16-byte aligned, BF16 (or float32
+    // without a rotation): the kernel with one lane per eight values.  Up to 16 rows (a decode step) are
+    // laid out for the shortest path through one row, a prefill chunk of up to 192 rows for the fewest
+    // instructions per (block, beta) pair with four workgroups a row, some hundreds of rows for the
+    // fewest instructions per block with one workgroup a row; the many-row kernel takes over from there.
+    constexpr bool kBf16 = std::is_same<T, uint16_t>::value, kF32 = std::is_same<T, float>::value;
+    const bool lanes_input = kBf16 || (kF32 && kPrologue == 0 && hadamard_stage_dtype < 0);
+    if ((kBf16 || kF32) && lanes_input && !kDithered && q == 14 && (n == 2048 || n == 4096 || n == 8192) &&
+        nq::aligned(x, 16) && (kPrologue != 3 || rows <= 16) && (kBf16 || rows > kLanesKernelRows) &&
+        (rows <= kBlockLanesRows || rows * (int64_t)n < kBulkElements)) {
+        // decode step: a workgroup of n / 8 lanes encodes n / 256 blocks per pass with eight lanes per
+        // (block, beta) pair: 32 slices of one pass each while that keeps the launch within one
+        // workgroup per compute unit (n <= 4096); an 8192-value row keeps one lane per pair, slices of
+        // 256 pairs.  Prefill chunk: every lane one pair, four slices a row (two, when four would put
+        // more than two 1024-lane workgroups on a compute unit).
+        const int form = rows > kLanesKernelRows ? nq::kBlockLanes
+                         : (rows > 16 ? nq::kEveryLane : (n > 4096 ? nq::kFirstLanes : nq::kEightLanes));
+        int slices = n > 4096 ? n / 512 : (rows * 32 <= 256 ? 32 : 16);
+        if (form == nq::kEveryLane) slices = n <= 2048 || rows * 4 * (n / 2048) <= 1024 ? 4 : 2;
+        if (form == nq::kBlockLanes) slices = 1;
+        if (rows * slices > 0x7fffffff) return nq::fail(NQ_ERR_SHAPE, "nq_quantize_rows: too many rows");
+        const size_t lds_bytes = (size_t)(8 * ((n >> 3) + 8) + n + 4 + 8) * sizeof(float);   // + norm, beta choices
+        auto kernel = nq::quantize_row_lanes_kernel<kPrologue>;
+        if (lds_bytes > 48 * 1024) {
+            hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (status != hipSuccess)
+                return nq::fail(NQ_ERR_LAUNCH, "nq_quantize_rows: cannot reserve %zu bytes of LDS: %s",
+                                lds_bytes, hipGetErrorString(status));
+        }
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(rows * slices)), dim3(n / 8), lds_bytes, stream, x, (int)kF32, rows, n,
+                           betas, beta_count, (float)sqrt((double)n), reinterpret_cast<uint32_t *>(codes), beta_ids,
+                           norms, reinterpret_cast<uint4 *>(decoded), slices, form, hadamard_stage_dtype >= 0 ? 1 : 0,
+                           prologue);
+        return nq::check_launch("nq_quantize_rows");
+    }
     if (!kDithered && kPrologue != 3 && rows * (int64_t)n >= kBulkElements) {
         int rows_per_wg = n >= 2048 ? 1 : 2048 / n;
         const size_t lds_bytes = ((size_t)rows_per_wg * n + 2 * rows_per_wg + (kPrologue == 1 ? n : 0)) * sizeof(float);
@@ -1101,37 +1162,6 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
                            (float)sqrt((double)n), reinterpret_cast<uint32_t *>(codes), beta_ids, norms,
                            reinterpret_cast<uint4 *>(decoded), rows_per_wg, (int)nq::aligned(x, 16),
                            hadamard_stage_dtype, prologue);
-        return nq::check_launch("nq_quantize_rows");
-    }
-    // BF16 rows of 2048, 4096 or 8192 values, q = 14, every operand 16-byte aligned, fewer than the
-    // throughput kernel's: one lane per eight values, each row repeated over as many workgroups as
-    // it has slices.  Up to 16 rows (a decode step) are laid out for the shortest path through one row,
-    // more rows (a prefill chunk) for the fewest instructions.
-    if (std::is_same<T, uint16_t>::value && !kDithered && q == 14 && (n == 2048 || n == 4096 || n == 8192) &&
-        nq::aligned(x, 16) && (rows <= 16 || (kPrologue != 3 && rows <= kLanesKernelRows))) {
-        // decode step: a workgroup of n / 8 lanes encodes n / 256 blocks per pass with eight lanes per
-        // (block, beta) pair: 32 slices of one pass each while that keeps the launch within one
-        // workgroup per compute unit (n <= 4096); an 8192-value row keeps one lane per pair, slices of
-        // 256 pairs.  Prefill chunk: every lane one pair, four slices a row.
-        const int form = rows > 16 ? nq::kEveryLane : (n > 4096 ? nq::kFirstLanes : nq::kEightLanes);
-        int slices = n > 4096 ? n / 512 : (rows * 32 <= 256 ? 32 : 16);
-        if (form == nq::kEveryLane) {
-            // a workgroup of 1024 (512) lanes per compute unit (two) at most: 4 slices, else 2
-            slices = n <= 2048 || rows * 4 * (n / 2048) <= 1024 ? 4 : 2;
-        }
-        const size_t lds_bytes = (size_t)(8 * ((n >> 3) + 8) + n + 4 + 8) * sizeof(float);   // + norm, beta choices
-        auto kernel = nq::quantize_row_lanes_kernel<kPrologue>;
-        if (lds_bytes > 48 * 1024) {
-            hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            if (status != hipSuccess)
-                return nq::fail(NQ_ERR_LAUNCH, "nq_quantize_rows: cannot reserve %zu bytes of LDS: %s",
-                                lds_bytes, hipGetErrorString(status));
-        }
-        hipLaunchKernelGGL(kernel, dim3((unsigned)(rows * slices)), dim3(n / 8), lds_bytes, stream,
-                           reinterpret_cast<const uint16_t *>(x), rows, n, betas, beta_count, (float)sqrt((double)n),
-                           reinterpret_cast<uint32_t *>(codes), beta_ids, norms, reinterpret_cast<uint4 *>(decoded),
-                           slices, form, hadamard_stage_dtype >= 0 ? 1 : 0, prologue);
         return nq::check_launch("nq_quantize_rows");
     }
     const int pairs_per_row = n / 2;

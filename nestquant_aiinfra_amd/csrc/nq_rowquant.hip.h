@@ -553,84 +553,91 @@ __device__ __forceinline__ void quantize_staged_pairs(const float *rows, const f
 // wavefront the coset reduction (a second lattice search) is skipped.  The first minimum over
 // the betas is a strict comparison in ascending order, and only the winner is turned into a
 // code word.
+// One block, its betas in turn (see quantize_staged_blocks): raw holds the block's eight staged
+// values, `betas` the row's table.  Every lane of the wavefront must call it together.
+template <class Sink>
+__device__ __forceinline__ void quantize_block_betas_in_turn(const float (&raw)[8], float scale, const float *betas,
+                                                             int beta_count, float q, float inv_q, int r, int b,
+                                                             const Sink &sink) {
+    const float inside_limit = 0.5f * q * q - 2.0f;
+    float y[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) y[j] = raw[j] * scale;
+    // the same for the whole wavefront, so that the betas stay a uniform loop
+    const bool fast_division = __builtin_amdgcn_ballot_w64(has_tiny_nonzero(y)) == 0;
+    float best_err = __builtin_inff(), best_beta = betas[0], best_point[8], best_recon[8];
+    uint32_t best = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) best_point[j] = best_recon[j] = 0.0f;
+#pragma unroll 1
+    for (int bi = 0; bi < beta_count; bi++) {
+        const float beta = betas[bi];
+        float z[8], point[8], recon[8];
+        if (fast_division && beta >= 0x1p-40f && beta <= 0x1p40f) {
+            const float rcp = 1.0f / beta;
+#pragma unroll
+            for (int j = 0; j < 8; j++) z[j] = divide_by_reciprocal(y[j], beta, rcp);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) z[j] = y[j] / beta;         // IEEE division
+        }
+        e8_nearest(z, point);
+        float energy = 0.0f;                                       // small half-integers: exact
+#pragma unroll
+        for (int j = 0; j < 8; j++) energy = __builtin_fmaf(point[j], point[j], energy);
+        if (__builtin_amdgcn_ballot_w64(!(energy <= inside_limit)) == 0) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) recon[j] = point[j] + 0.0f;  // the decode never returns -0
+        } else {
+            float c[8], code[8], p8[8];
+            e8_coords(point, c);
+#pragma unroll
+            for (int j = 0; j < 8; j++) code[j] = mod_q(c[j], q, inv_q);
+            e8_coset_point(code, p8);
+            reduce_coset_point(p8, q, recon);
+        }
+        float err = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float d = recon[j] * beta - y[j];
+            err = err + d * d;
+        }
+        const bool take = err < best_err;                          // first minimum
+        best_err = take ? err : best_err;
+        best = take ? (uint32_t)bi : best;
+        best_beta = take ? beta : best_beta;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            best_point[j] = take ? point[j] : best_point[j];
+            best_recon[j] = take ? recon[j] : best_recon[j];
+        }
+    }
+    const bool wanted = sink.wants(r);
+    if (wanted) {
+        float c[8], code[8];
+        e8_coords(best_point, c);
+#pragma unroll
+        for (int j = 0; j < 8; j++) code[j] = mod_q(c[j], q, inv_q);
+        sink.code(r, b, pack_codeword(code), best_recon, best_beta);
+    }
+    // four consecutive blocks (a quad of lanes) share one beta byte
+    uint32_t byte = best << (2 * (b & 3));
+    byte |= quad_xor1(byte);
+    byte |= quad_xor2(byte);
+    if ((b & 3) == 0 && wanted) sink.beta_byte(r, b, byte);
+}
+
 template <class BetasOf, class Sink>
 __device__ __forceinline__ void quantize_staged_blocks(const float *rows, const float *row_scale, int n, float q,
                                                        float inv_q, BetasOf betas_of, int beta_count,
                                                        int block_begin, int block_end, const Sink &sink) {
     const int blocks_per_row = n >> 3;
-    const float inside_limit = 0.5f * q * q - 2.0f;
     for (int blk = block_begin + (int)threadIdx.x; blk < block_end; blk += blockDim.x) {
         const int r = blk / blocks_per_row, b = blk - r * blocks_per_row;
-        const float scale = row_scale[r];
         const float4 lo = *reinterpret_cast<const float4 *>(rows + (size_t)r * n + 8 * b);
         const float4 hi = *reinterpret_cast<const float4 *>(rows + (size_t)r * n + 8 * b + 4);
         const float raw[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        const float *betas = betas_of(r);
-        float y[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) y[j] = raw[j] * scale;
-        // the same for the whole wavefront, so that the betas stay a uniform loop
-        const bool fast_division = __builtin_amdgcn_ballot_w64(has_tiny_nonzero(y)) == 0;
-        float best_err = __builtin_inff(), best_beta = betas[0], best_point[8], best_recon[8];
-        uint32_t best = 0;
-#pragma unroll
-        for (int j = 0; j < 8; j++) best_point[j] = best_recon[j] = 0.0f;
-#pragma unroll 1
-        for (int bi = 0; bi < beta_count; bi++) {
-            const float beta = betas[bi];
-            float z[8], point[8], recon[8];
-            if (fast_division && beta >= 0x1p-40f && beta <= 0x1p40f) {
-                const float rcp = 1.0f / beta;
-#pragma unroll
-                for (int j = 0; j < 8; j++) z[j] = divide_by_reciprocal(y[j], beta, rcp);
-            } else {
-#pragma unroll
-                for (int j = 0; j < 8; j++) z[j] = y[j] / beta;         // IEEE division
-            }
-            e8_nearest(z, point);
-            float energy = 0.0f;                                       // small half-integers: exact
-#pragma unroll
-            for (int j = 0; j < 8; j++) energy = __builtin_fmaf(point[j], point[j], energy);
-            if (__builtin_amdgcn_ballot_w64(!(energy <= inside_limit)) == 0) {
-#pragma unroll
-                for (int j = 0; j < 8; j++) recon[j] = point[j] + 0.0f;  // the decode never returns -0
-            } else {
-                float c[8], code[8], p8[8];
-                e8_coords(point, c);
-#pragma unroll
-                for (int j = 0; j < 8; j++) code[j] = mod_q(c[j], q, inv_q);
-                e8_coset_point(code, p8);
-                reduce_coset_point(p8, q, recon);
-            }
-            float err = 0.0f;
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const float d = recon[j] * beta - y[j];
-                err = err + d * d;
-            }
-            const bool take = err < best_err;                          // first minimum
-            best_err = take ? err : best_err;
-            best = take ? (uint32_t)bi : best;
-            best_beta = take ? beta : best_beta;
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                best_point[j] = take ? point[j] : best_point[j];
-                best_recon[j] = take ? recon[j] : best_recon[j];
-            }
-        }
-        const bool wanted = sink.wants(r);
-        if (wanted) {
-            float c[8], code[8];
-            e8_coords(best_point, c);
-#pragma unroll
-            for (int j = 0; j < 8; j++) code[j] = mod_q(c[j], q, inv_q);
-            sink.code(r, b, pack_codeword(code), best_recon, best_beta);
-        }
-        // four consecutive blocks (a quad of lanes) share one beta byte
-        uint32_t byte = best << (2 * (b & 3));
-        byte |= quad_xor1(byte);
-        byte |= quad_xor2(byte);
-        if ((b & 3) == 0 && wanted) sink.beta_byte(r, b, byte);
+        quantize_block_betas_in_turn(raw, row_scale[r], betas_of(r), beta_count, q, inv_q, r, b, sink);
     }
 }
 

@@ -90,6 +90,10 @@ def test_quantize_rows_long_rows_match_reference_golden(rt, golden_long_rows):
     (130, 4096, "outlier", torch.bfloat16),
     (190, 2048, "student", torch.bfloat16),
     (100, 8192, "outlier", torch.bfloat16),     # two slices a row, two turns a lane
+    (400, 2048, "student", torch.bfloat16),     # some hundreds of rows: one lane per block, betas in turn
+    (700, 2048, "outlier", torch.bfloat16),
+    (300, 2048, "student", torch.float32),
+    (200, 4096, "outlier", torch.float32),
     (40, 2048, "outlier", torch.float32),
     (128, 64, "normal", torch.bfloat16),        # one KV page side: 16 tokens x 8 heads
     (5, 32, "normal", torch.float32),
@@ -238,13 +242,13 @@ def test_errors_are_reported_like_the_reference(rt):
 @pytest.mark.parametrize("n", [2048, 4096, 8192])
 @pytest.mark.parametrize("rows", [1, 3, 16])
 def test_decode_size_encoder_equals_the_many_row_encoder(rt, rows, n):
-    """BF16 rows of 2048, 4096 or 8192 values take the one-lane-per-eight-values kernel while they
-    are fewer than two million values (up to 16 rows with eight lanes or the first four wavefronts
-    on the (block, beta) pairs, more rows with every lane on one pair), and the bulk kernel from
-    there on: the same rows must come out of all three bit for bit (rotation included), zero rows
+    """BF16 rows of 2048, 4096 or 8192 values take the one-lane-per-eight-values kernel up to 512
+    rows (up to 16 rows with eight lanes or the first four wavefronts on the (block, beta) pairs, up
+    to 192 with every lane on one pair, beyond with one lane per block), and the many-row kernel from
+    there on: the same rows must come out of all four bit for bit (rotation included), zero rows
     and rows of huge and tiny magnitude among them."""
     g = torch.Generator().manual_seed(rows * n)
-    total = (1 << 21) // n
+    total = max((1 << 21) // n, 520)
     x = torch.randn(total, n, generator=g) * torch.logspace(-15, 15, total).unsqueeze(-1)
     x[:17] = torch.randn(17, n, generator=g) * torch.logspace(-15, 15, 17).unsqueeze(-1)
     x[min(2, rows - 1)] = 0.0
@@ -256,7 +260,9 @@ def test_decode_size_encoder_equals_the_many_row_encoder(rt, rows, n):
         some = rt.quantize_activation_cuda(x[:41].contiguous(), q=Q, betas=ACTIVATION_BETAS, beta_table=table,
                                            hadamard=rotate)
         many = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS, beta_table=table, hadamard=rotate)
-        for part, count in ((few, rows), (some, 41)):
+        more = rt.quantize_activation_cuda(x[:300].contiguous(), q=Q, betas=ACTIVATION_BETAS, beta_table=table,
+                                           hadamard=rotate)
+        for part, count in ((few, rows), (some, 41), (more, 300)):
             assert torch.equal(part.code_payload, many.code_payload[: count * n // 2]), (rotate, count)
             assert torch.equal(part.beta_payload, many.beta_payload[: count * n // 32]), (rotate, count)
             assert torch.equal(part.row_norms, many.row_norms[:count]), (rotate, count)
