@@ -451,11 +451,12 @@ def attention_phases_extra(device):
         call(0)
         stamps = (ctypes.c_ulonglong * 16)()
         _native.check(lib.nq_debug_attention_stamps(stamps))
-        s = [int(v) * 10 for v in stamps[:8]]
+        s = [int(v) * 10 for v in stamps[:10]]
         results[name] = {"launch_ns_with_merge": round(seconds * 1e9), "tables_ns": s[1] - s[0],
                          "key_requests_and_query_ns": s[2] - s[1], "query_to_registers_ns": s[3] - s[2],
                          "key_pass_ns": s[4] - s[3], "softmax_ns": s[5] - s[4], "value_pass_ns": s[6] - s[5],
-                         "fold_and_store_ns": s[7] - s[6], "inside_ns": s[7] - s[0]}
+                         "fold_and_store_ns": s[7] - s[6], "of_which_fold_ns": s[8] - s[6],
+                         "of_which_wait_for_the_workgroup_ns": s[9] - s[8], "inside_ns": s[7] - s[0]}
     return results
 
 

@@ -202,7 +202,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     static_assert(kChunkTokens % 64 == 0, "every lane of a wavefront takes the same number of scores");
     static_assert(2 * kTokenBlocks <= kAttnThreads, "one lane per block of the tail's keys and values");
     __shared__ float scores[G][kChunkTokens];
-    __shared__ float acc_lds[kWaves][G * 8][kBlocks];    // one entry per wavefront; holds the queries first
+    __shared__ __align__(16) float acc_lds[kWaves][kBlocks][G * 8];    // one entry per wavefront; holds the queries first
     // kWrites: the slot's hot tail with the new token (keys, then values), and the page made from it
     __shared__ float tail[kWrites ? 2 * P : 1][kWrites ? D : 1];
     __shared__ float tail_scale[kWrites ? 2 * P : 1], tail_norm[kWrites ? 2 * P : 1];
@@ -454,14 +454,20 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
 #pragma unroll
             for (int j = 0; j < 8; j++) k[j] = (k[j] * beta) * back;
         }
-        // every pass writes its scores, so a hot or ragged chunk leaves no stale entry
+        // every pass writes its scores, so a hot or ragged chunk leaves no stale entry (the sums of
+        // all heads first, then one predicated stretch of stores: a store between two sums would end
+        // the basic block and keep the sums from overlapping)
+        float s[G];
 #pragma unroll
         for (int h = 0; h < G; h++) {
-            float s = 0.0f;
+            s[h] = 0.0f;
 #pragma unroll
-            for (int j = 0; j < 8; j++) s = __builtin_fmaf(q[h][j], k[j], s);
-            s = sum8(s);
-            if (blk == 0) scores[h][page_in_chunk * P + token] = valid ? s * a.scale : -INFINITY;
+            for (int j = 0; j < 8; j++) s[h] = __builtin_fmaf(q[h][j], k[j], s[h]);
+            s[h] = sum8(s[h]);
+        }
+        if (blk == 0) {
+#pragma unroll
+            for (int h = 0; h < G; h++) scores[h][page_in_chunk * P + token] = valid ? s[h] * a.scale : -INFINITY;
         }
     }
     __syncthreads();                                     // scores complete; the queries in acc_lds are no longer needed
@@ -524,19 +530,27 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     // lanes that share a block index hold partial sums of the same 8 output dims: folded inside the
     // wavefront with register exchanges (the two tokens of a 16-lane row, then the four rows),
     // wavefronts through LDS in order
+    // (all the sums first, then one predicated stretch of 128-bit stores, as above)
 #pragma unroll
     for (int h = 0; h < G; h++)
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const float v = fold_rows(acc[h][j] + dpp_rotate8(acc[h][j]));
-            if ((tid & 63) < 8) acc_lds[tid >> 6][h * 8 + j][tid & 7] = v;
+        for (int j = 0; j < 8; j++) acc[h][j] = fold_rows(acc[h][j] + dpp_rotate8(acc[h][j]));
+    if ((tid & 63) < 8) {
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            float4 *to = reinterpret_cast<float4 *>(&acc_lds[tid >> 6][tid & 7][h * 8]);
+            to[0] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+            to[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
         }
+    }
+    NQ_STAMP(8);
     __syncthreads();
+    NQ_STAMP(9);
     for (int o = tid; o < G * D; o += kAttnThreads) {
         const int h = o / D, d = o % D;
-        float total = acc_lds[0][h * 8 + d % 8][d / 8];
+        float total = acc_lds[0][d / 8][h * 8 + d % 8];
 #pragma unroll
-        for (int w = 1; w < kWaves; w++) total = total + acc_lds[w][h * 8 + d % 8][d / 8];
+        for (int w = 1; w < kWaves; w++) total = total + acc_lds[w][d / 8][h * 8 + d % 8];
         a.part_acc[(part + (int64_t)h * (a.chunks + 1)) * D + d] = total;
     }
     if (tid < G) {
