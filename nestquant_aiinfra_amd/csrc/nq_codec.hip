@@ -592,12 +592,12 @@ __device__ __forceinline__ void late_stages_to_chains(const float *natural, floa
 
 enum LaneEncodeForm { kEightLanes = 0, kFirstLanes = 1, kEveryLane = 2, kBlockLanes = 3 };
 
-template <int kPrologue>
+template <int kPrologue, int kForm>
 __global__ void __launch_bounds__(1024)
 quantize_row_lanes_kernel(const void *__restrict__ x_any, int x_is_f32, int64_t rows, int n, const float *__restrict__ betas,
                           int beta_count, float sqrt_n, uint32_t *__restrict__ codes, uint8_t *__restrict__ beta_ids,
-                          float *__restrict__ norms, uint4 *__restrict__ decoded, int slices, int encode_form,
-                          int rotate, InputPrologue pro) {
+                          float *__restrict__ norms, uint4 *__restrict__ decoded, int slices, int rotate,
+                          InputPrologue pro) {
     extern __shared__ float lds[];
     const int pitch = chain_pitch(n);
     float *chains = lds;                                  // 8 * pitch floats: the row, transposed
@@ -611,7 +611,7 @@ quantize_row_lanes_kernel(const void *__restrict__ x_any, int x_is_f32, int64_t 
     const int slice = blockIdx.x % slices;
     const int64_t row = blockIdx.x / slices;
     const int log_n = 31 - __builtin_clz(n);
-    // How the slice's (block, beta) pairs meet the lanes (`encode_form`):
+    // How the slice's (block, beta) pairs meet the lanes (kForm, one instantiation each):
     //   kEightLanes  eight lanes per pair, lane c the block's coordinate c, beta (lane / 8) % 4: a quarter
     //                of the instructions per lane, the shortest path for the few rows of a decode step
     //                (rows of up to 4096 values; with the sixteen wavefronts of an 8192-value row that
@@ -625,7 +625,7 @@ quantize_row_lanes_kernel(const void *__restrict__ x_any, int x_is_f32, int64_t 
     //                the coset reduction skipped where every block of the wavefront lies inside the
     //                Voronoi cell (quantize_block_betas_in_turn): the fewest instructions per block, for
     //                hundreds of rows and more, one workgroup a row.
-    const bool eight_lanes = encode_form == kEightLanes;
+    constexpr bool eight_lanes = kForm == kEightLanes;
     const int c = lane & 7, bi = eight_lanes ? (lane >> 3) & 3 : tid & 3;
     const bool live = bi < beta_count;
     // requested first, used last; a launch that only runs the element-wise stage has no table
@@ -633,7 +633,7 @@ quantize_row_lanes_kernel(const void *__restrict__ x_any, int x_is_f32, int64_t 
     NQ_STAMP(0);
 
     float v[8];
-    if (kPrologue == 0 && x_is_f32) {                     // plain float32 rows (never rotated here)
+    if (kForm == kBlockLanes && kPrologue == 0 && x_is_f32) {      // plain float32 rows (never rotated here)
         const float4 *at = reinterpret_cast<const float4 *>(x_any) + ((row * n) >> 2) + 2 * tid;
         const float4 lo = at[0], hi = at[1];
         v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
@@ -732,8 +732,8 @@ quantize_row_lanes_kernel(const void *__restrict__ x_any, int x_is_f32, int64_t 
         norm = __builtin_sqrtf(total);
         if (tid == 0) *row_norm_shared = norm;
     }
-    if (encode_form == kFirstLanes && tid >= 256) return;
-    if (encode_form != kFirstLanes && blockDim.x > 256) {
+    if (kForm == kFirstLanes && tid >= 256) return;
+    if (kForm != kFirstLanes && blockDim.x > 256) {
         __syncthreads();
         norm = *row_norm_shared;
     }
@@ -763,7 +763,7 @@ quantize_row_lanes_kernel(const void *__restrict__ x_any, int x_is_f32, int64_t 
             __device__ __forceinline__ uint32_t counter(int, int) const { return 0; }
         };
         const LaneSink sink{codes, beta_ids, decoded, row * (n >> 3), norm / sqrt_n};
-        if (encode_form == kBlockLanes) {
+        if (kForm == kBlockLanes) {
             const int blocks_per_slice = (n >> 3) / slices;
             for (int at = tid; at < blocks_per_slice; at += (int)blockDim.x) {
                 const int b = slice * blocks_per_slice + at;
@@ -775,7 +775,7 @@ quantize_row_lanes_kernel(const void *__restrict__ x_any, int x_is_f32, int64_t 
             NQ_STAMP(4);
             return;
         }
-        const int pairs_per_slice = encode_form == kFirstLanes ? 256 : (n >> 1) / slices;
+        const int pairs_per_slice = kForm == kFirstLanes ? 256 : (n >> 1) / slices;
         for (int at = tid; at < pairs_per_slice; at += (int)blockDim.x) {
             const int p = slice * pairs_per_slice + at, b = p >> 2;
             float raw[8];
@@ -1130,7 +1130,12 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
         if (form == nq::kBlockLanes) slices = 1;
         if (rows * slices > 0x7fffffff) return nq::fail(NQ_ERR_SHAPE, "nq_quantize_rows: too many rows");
         const size_t lds_bytes = (size_t)(8 * ((n >> 3) + 8) + n + 4 + 8) * sizeof(float);   // + norm, beta choices
-        auto kernel = nq::quantize_row_lanes_kernel<kPrologue>;
+        using Kernel = void (*)(const void *, int, int64_t, int, const float *, int, float, uint32_t *, uint8_t *, float *,
+                                uint4 *, int, int, nq::InputPrologue);
+        Kernel kernel = form == nq::kEightLanes   ? (Kernel)nq::quantize_row_lanes_kernel<kPrologue, nq::kEightLanes>
+                        : form == nq::kFirstLanes ? (Kernel)nq::quantize_row_lanes_kernel<kPrologue, nq::kFirstLanes>
+                        : form == nq::kEveryLane  ? (Kernel)nq::quantize_row_lanes_kernel<kPrologue, nq::kEveryLane>
+                                                  : (Kernel)nq::quantize_row_lanes_kernel<kPrologue, nq::kBlockLanes>;
         if (lds_bytes > 48 * 1024) {
             hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -1140,8 +1145,7 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
         }
         hipLaunchKernelGGL(kernel, dim3((unsigned)(rows * slices)), dim3(n / 8), lds_bytes, stream, x, (int)kF32, rows, n,
                            betas, beta_count, (float)sqrt((double)n), reinterpret_cast<uint32_t *>(codes), beta_ids,
-                           norms, reinterpret_cast<uint4 *>(decoded), slices, form, hadamard_stage_dtype >= 0 ? 1 : 0,
-                           prologue);
+                           norms, reinterpret_cast<uint4 *>(decoded), slices, hadamard_stage_dtype >= 0 ? 1 : 0, prologue);
         return nq::check_launch("nq_quantize_rows");
     }
     if (!kDithered && kPrologue != 3 && rows * (int64_t)n >= kBulkElements) {
