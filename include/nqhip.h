@@ -505,7 +505,17 @@ int nq_nqkv_attention_prefill(
     const int32_t *sequence_lengths_dev, const void *hot_keys_dev, const void *hot_values_dev,
     const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, const int32_t *counts_dev, int uniform_count,
     int batch, int tokens, int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size,
-    float scale, void *out_dev, void *stream);
+    float scale, void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
+
+/*
+ * Bytes of the optional workspace of nq_nqkv_attention_prefill (0 when the launch has enough
+ * workgroups as it is).  Given at least this much (16-byte aligned), the call splits every slot's page
+ * table into ranges that workgroups of their own attend over, and a second launch merges the
+ * partial results per query vector in range order: the work of a row then spreads over the chip in
+ * proportion to its context.  Without it (NULL, 0) one workgroup walks a (row, token tile, KV head)
+ * from the first page to the last.  Same result up to the rounding of the merged sums.
+ */
+size_t nq_nqkv_attention_prefill_workspace_bytes(int batch, int tokens, int max_pages, int q_heads, int kv_heads);
 
 /*
  * Greedy sampling inside the decode step: for every row r (all rows when active_mask_dev is NULL,

@@ -64,7 +64,8 @@ SIGNATURES = {
                                                                                 _ptr, _ptr, _size, _ptr]),
     "nq_nqkv_append_attention_decode": (_i32, [_ptr] * 10 + [_ptr, _i32, _ptr, _i32] + [_ptr] * 9 + [_i32] * 7
                                         + [_c.c_float, _i32, _ptr, _ptr, _ptr, _ptr, _size, _ptr]),
-    "nq_nqkv_attention_prefill": (_i32, [_ptr] * 19 + [_i32] * 9 + [_c.c_float, _ptr, _ptr]),
+    "nq_nqkv_attention_prefill": (_i32, [_ptr] * 19 + [_i32] * 9 + [_c.c_float, _ptr, _ptr, _size, _ptr]),
+    "nq_nqkv_attention_prefill_workspace_bytes": (_size, [_i32] * 5),
     "nq_nqkv_attention_workspace_bytes": (_size, [_i32, _i32, _i32, _i32]),
     "nq_nqkv_attention_parts": (_i32, [_i32, _i32]),
     "nq_greedy_sample": (_i32, [_ptr, _i32, _i32, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _size, _ptr]),

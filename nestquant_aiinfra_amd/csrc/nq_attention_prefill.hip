@@ -17,12 +17,21 @@
 //   * scores on the matrix cores, transposed: S^T[token, vector] = K . Q^T with two
 //     v_mfma_f32_16x16x32_bf16 per wavefront (Q^T fragments live in registers for the whole
 //     kernel).  A lane then holds 4 tokens of one query vector: causal and length masks, the
-//     online softmax in FP32 (two cross-row exchanges per statistic), and its four
+//     online softmax in FP32 (two register exchanges per statistic), and its four
 //     probabilities are already laid out as the B operand of the next product;
 //   * output, transposed: O^T[dim, vector] += V^T . P^T over the pair's 32 tokens, four
 //     v_mfma_f32_16x16x32_bf16.
 // LDS tiles are double-buffered (one barrier per pair of pages).  Pages past the last position of the
 // tile are never visited.
+//
+// kSets: a lane serves kSets query vectors (vector v, v + 128, ...), so a workgroup owns kSets x 128
+// of them and a decoded page serves them all: the decode is the kernel's largest cost, and the G
+// heads x 128 / G tokens of one set would decode every page once per 32 tokens (G = 4).
+// With a workspace the context is also split: workgroup (pair, head, s) takes pages
+// [s L, (s + 1) L) of the slot's table and leaves its unnormalised outputs, maxima and denominators
+// per query vector for attention_prefill_merge_kernel; a row's work then spreads over the chip in
+// proportion to its context instead of running on one workgroup per (tile, head) from the first page
+// to the last (batch 8, contexts 495 .. 3967, 128 new tokens: the longest row alone set the time).
 #include "nq_e8.hip.h"
 #include "nq_host.h"
 
@@ -46,20 +55,41 @@ struct PrefillAttentionArgs {
     const uint8_t *active_mask;
     int batch, tokens, uniform_count, slots, max_pages, q_heads, kv_heads;
     float scale;
+    // split form: pages per split (even), number of splits (grid.y), partial results
+    int pages_per_split, splits;
+    float *part_out;                   // [batch, tokens, q_heads, splits, D] unnormalised
+    float *part_stats;                 // [batch, tokens, q_heads, splits, 2]: maximum, denominator
 };
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-// the value held by the lane whose id differs in bit 4 / bit 5
-__device__ __forceinline__ float lane_xor16(float v) { return __shfl_xor(v, 16, 64); }
-__device__ __forceinline__ float lane_xor32(float v) { return __shfl_xor(v, 32, 64); }
+// maximum / sum over the four lanes l % 16, + 16, + 32, + 48 (the four quarters of a query vector's
+// column), the same in all four: two register exchanges each (v_permlane16_swap, v_permlane32_swap
+// hand a lane its own value and that of the lane 16 / 32 further on), no trip through the LDS crossbar
+__device__ __forceinline__ float quarters_max(float v) {
+    const int bits = __builtin_bit_cast(int, v);
+    const auto by16 = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    const float half = fmaxf(__builtin_bit_cast(float, (int)by16[0]), __builtin_bit_cast(float, (int)by16[1]));
+    const int half_bits = __builtin_bit_cast(int, half);
+    const auto by32 = __builtin_amdgcn_permlane32_swap(half_bits, half_bits, false, false);
+    return fmaxf(__builtin_bit_cast(float, (int)by32[0]), __builtin_bit_cast(float, (int)by32[1]));
+}
+__device__ __forceinline__ float quarters_sum(float v) {
+    const int bits = __builtin_bit_cast(int, v);
+    const auto by16 = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    const float half = __builtin_bit_cast(float, (int)by16[0]) + __builtin_bit_cast(float, (int)by16[1]);
+    const int half_bits = __builtin_bit_cast(int, half);
+    const auto by32 = __builtin_amdgcn_permlane32_swap(half_bits, half_bits, false, false);
+    return __builtin_bit_cast(float, (int)by32[0]) + __builtin_bit_cast(float, (int)by32[1]);
+}
 
-template <int D, int P, int G>
+template <int D, int P, int G, int kSets, bool kSplit>
 __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(PrefillAttentionArgs a) {
     static_assert(D == 64 && P == 16, "lane roles assume 64-dim heads and 16-token pages");
     constexpr int kBlocks = D / 8;
-    constexpr int kTileTokens = 128 / G;                 // query tokens per workgroup
+    constexpr int kSetTokens = 128 / G;                  // query tokens per set of 128 vectors
+    constexpr int kTileTokens = kSets * kSetTokens;      // query tokens per workgroup
     constexpr int kKeyRow = D + 8;                       // BF16 elements per key row: 144 bytes, conflict-free 16-byte reads
     __shared__ __attribute__((aligned(16))) uint16_t k_page[2][2][P][kKeyRow];   // [buffer][page of the pair][token][dim]
     // transposed: [dim][token], rows of 40 bytes, and the rows of dims 32..63 keep their two halves of
@@ -77,11 +107,16 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     const int place = blockIdx.x >> 3, pair = (place / a.kv_heads) * 8 + (blockIdx.x & 7);
     const int g = place % a.kv_heads, tile = pair % tiles, row = pair / tiles;
     if (row >= a.batch) return;                          // padding of the last group of eight pairs
-    const int vec = 16 * wave + (lane & 15);             // this lane's query vector (column of S^T and O^T)
+    const int vec = 16 * wave + (lane & 15);             // this lane's query vector of every set (column of S^T and O^T)
     const int quarter = lane >> 4;                       // which 4 tokens / 4 dims of a 16-row tile the lane holds
-    const int t = tile * kTileTokens + vec / G;          // token of the query vector inside the chunk
     const int head = g * G + vec % G;
-    const int64_t q_at = (((int64_t)row * a.tokens + t) * a.q_heads + head) * D;
+    int t[kSets];                                        // token of the set's query vector inside the chunk
+    int64_t q_at[kSets];
+#pragma unroll
+    for (int i = 0; i < kSets; i++) {
+        t[i] = tile * kTileTokens + i * kSetTokens + vec / G;
+        q_at[i] = (((int64_t)row * a.tokens + t[i]) * a.q_heads + head) * D;
+    }
 
     int slot = a.slot_ids[row];
     const bool live = a.active_mask[row] && slot >= 0 && slot < a.slots;
@@ -92,27 +127,43 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     if (count > length) count = length;
     if (!live) count = 0;
     const int start = length - count;
-    const bool has_query = t < count;
-    const int position = start + t;                      // attends to cache tokens 0 .. position
+    bool has_query[kSets];
+    int position[kSets];                                 // attends to cache tokens 0 .. position
+#pragma unroll
+    for (int i = 0; i < kSets; i++) {
+        has_query[i] = t[i] < count;
+        position[i] = start + t[i];
+    }
     const int page_count = a.page_counts[slot], last_len = a.last_page_lens[slot], hot_len = a.hot_lengths[slot];
 
     // last position any vector of this tile looks at (uniform over the workgroup)
     const int tile_first = tile * kTileTokens;
     const int tile_last_token = (tile_first + kTileTokens < count ? tile_first + kTileTokens : count) - 1;
-    const int pages_needed = tile_last_token >= tile_first ? (start + tile_last_token) / P + 1 : 0;
+    const int all_pages = tile_last_token >= tile_first ? (start + tile_last_token) / P + 1 : 0;
+    // this workgroup's pages of the table: [first_page, pages_needed)
+    // (the last ranges, which only long contexts have, are dispatched first: the launch then ends on the
+    // first ranges, which every row has)
+    const int split_index = kSplit ? (int)(gridDim.y - 1 - blockIdx.y) : 0;
+    const int first_page = split_index * a.pages_per_split;
+    const int pages_needed = kSplit && first_page + a.pages_per_split < all_pages ? first_page + a.pages_per_split : all_pages;
 
     // Q^T fragments of the two 32-dim steps: lane (vector, quarter) holds dims 32 step + 8 quarter .. + 8
-    bf16x8 q_frag[2];
+    bf16x8 q_frag[kSets][2];
+    floatx4 o[kSets][4];                                 // O^T tiles: dims 16 tile + 4 quarter + r of this lane's vector
+    float running_max[kSets], denom[kSets];
 #pragma unroll
-    for (int step = 0; step < 2; step++) {
-        uint4 raw = make_uint4(0, 0, 0, 0);
-        if (has_query) raw = *reinterpret_cast<const uint4 *>(a.query + q_at + 32 * step + 8 * quarter);
-        q_frag[step] = __builtin_bit_cast(bf16x8, raw);
+    for (int i = 0; i < kSets; i++) {
+#pragma unroll
+        for (int step = 0; step < 2; step++) {
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (has_query[i]) raw = *reinterpret_cast<const uint4 *>(a.query + q_at[i] + 32 * step + 8 * quarter);
+            q_frag[i][step] = __builtin_bit_cast(bf16x8, raw);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) o[i][j] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        running_max[i] = -INFINITY;
+        denom[i] = 0.0f;
     }
-    floatx4 o[4];                                        // O^T tiles: dims 16 tile + 4 quarter + r of this lane's vector
-#pragma unroll
-    for (int i = 0; i < 4; i++) o[i] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-    float running_max = -INFINITY, denom = 0.0f;
 
     // decode role: lanes 0..255 stage the first page of a pair, 256..511 the second; of each
     // half, 128 lanes take keys and 128 values; (token, block) of the page
@@ -171,55 +222,64 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     // kMasked = false when all 32 tokens exist and are visible to every vector of the tile
     auto attend = [&](auto masked, int buf, int first) {
         constexpr bool kMasked = decltype(masked)::value;
-        float s[8], trip_max = -INFINITY;
+        bf16x8 k_frag[2][2];
 #pragma unroll
-        for (int half = 0; half < 2; half++) {
-            floatx4 st = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int half = 0; half < 2; half++)
 #pragma unroll
-            for (int step = 0; step < 2; step++) {
-                const bf16x8 k_frag = __builtin_bit_cast(
+            for (int step = 0; step < 2; step++)
+                k_frag[half][step] = __builtin_bit_cast(
                     bf16x8, *reinterpret_cast<const uint4 *>(&k_page[buf][half][lane & 15][32 * step + 8 * quarter]));
-                st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag, q_frag[step], st, 0, 0, 0);
-            }
-            const int tokens_here = kMasked ? tokens_of(first + half) : P;
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int tok = 4 * quarter + r;
-                const bool visible = !kMasked || (has_query && tok < tokens_here && (first + half) * P + tok <= position);
-                s[4 * half + r] = visible ? st[r] * a.scale : -INFINITY;
-                trip_max = fmaxf(trip_max, s[4 * half + r]);
-            }
-        }
-        trip_max = fmaxf(trip_max, lane_xor16(trip_max));
-        trip_max = fmaxf(trip_max, lane_xor32(trip_max));
-        const float new_max = fmaxf(running_max, trip_max);
-        // a vector that has seen nothing yet keeps max = -inf: exponents are forced to zero weight
-        const float keep = (kMasked && new_max == -INFINITY) ? 1.0f : __expf(running_max - new_max);
-        float p[8], trip_sum = 0.0f;
-#pragma unroll
-        for (int r = 0; r < 8; r++) {
-            p[r] = (kMasked && s[r] == -INFINITY) ? 0.0f : __expf(s[r] - new_max);
-            trip_sum = trip_sum + p[r];
-        }
-        trip_sum = trip_sum + lane_xor16(trip_sum);
-        trip_sum = trip_sum + lane_xor32(trip_sum);
-        denom = denom * keep + trip_sum;
-        running_max = new_max;
-        // B operand of the 32-deep product: slots 0..3 = this lane's tokens of the first page, 4..7 of the second
-        const uint4 p_bits = make_uint4(__builtin_bit_cast(uint32_t, pack_bf16x2(p[0], p[1])),
-                                        __builtin_bit_cast(uint32_t, pack_bf16x2(p[2], p[3])),
-                                        __builtin_bit_cast(uint32_t, pack_bf16x2(p[4], p[5])),
-                                        __builtin_bit_cast(uint32_t, pack_bf16x2(p[6], p[7])));
-        const bf16x8 p_frag = __builtin_bit_cast(bf16x8, p_bits);
+        bf16x8 v_frag[4];
 #pragma unroll
         for (int tile = 0; tile < 4; tile++) {
             const int column = (4 * quarter) ^ (8 * (tile >> 1));
             const uint2 v0 = *reinterpret_cast<const uint2 *>(&v_page[buf][0][16 * tile + (lane & 15)][column]);
             const uint2 v1 = *reinterpret_cast<const uint2 *>(&v_page[buf][1][16 * tile + (lane & 15)][column]);
+            v_frag[tile] = __builtin_bit_cast(bf16x8, make_uint4(v0.x, v0.y, v1.x, v1.y));
+        }
 #pragma unroll
-            for (int r = 0; r < 4; r++) o[tile][r] = o[tile][r] * keep;
-            o[tile] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, make_uint4(v0.x, v0.y, v1.x, v1.y)),
-                                                             p_frag, o[tile], 0, 0, 0);
+        for (int i = 0; i < kSets; i++) {
+            float s[8], trip_max = -INFINITY;
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+                floatx4 st = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int step = 0; step < 2; step++)
+                    st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag[half][step], q_frag[i][step], st, 0, 0, 0);
+                const int tokens_here = kMasked ? tokens_of(first + half) : P;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int tok = 4 * quarter + r;
+                    const bool visible = !kMasked || (has_query[i] && tok < tokens_here && (first + half) * P + tok <= position[i]);
+                    s[4 * half + r] = visible ? st[r] * a.scale : -INFINITY;
+                    trip_max = fmaxf(trip_max, s[4 * half + r]);
+                }
+            }
+            trip_max = quarters_max(trip_max);
+            const float new_max = fmaxf(running_max[i], trip_max);
+            // a vector that has seen nothing yet keeps max = -inf: exponents are forced to zero weight
+            const float keep = (kMasked && new_max == -INFINITY) ? 1.0f : __expf(running_max[i] - new_max);
+            float p[8], trip_sum = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 8; r++) {
+                p[r] = (kMasked && s[r] == -INFINITY) ? 0.0f : __expf(s[r] - new_max);
+                trip_sum = trip_sum + p[r];
+            }
+            trip_sum = quarters_sum(trip_sum);
+            denom[i] = denom[i] * keep + trip_sum;
+            running_max[i] = new_max;
+            // B operand of the 32-deep product: slots 0..3 = this lane's tokens of the first page, 4..7 of the second
+            const uint4 p_bits = make_uint4(__builtin_bit_cast(uint32_t, pack_bf16x2(p[0], p[1])),
+                                            __builtin_bit_cast(uint32_t, pack_bf16x2(p[2], p[3])),
+                                            __builtin_bit_cast(uint32_t, pack_bf16x2(p[4], p[5])),
+                                            __builtin_bit_cast(uint32_t, pack_bf16x2(p[6], p[7])));
+            const bf16x8 p_frag = __builtin_bit_cast(bf16x8, p_bits);
+#pragma unroll
+            for (int tile = 0; tile < 4; tile++) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) o[i][tile][r] = o[i][tile][r] * keep;
+                o[i][tile] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_frag[tile], p_frag, o[i][tile], 0, 0, 0);
+            }
         }
     };
 
@@ -231,10 +291,11 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     if (fast_pages > pages_needed) fast_pages = pages_needed;
     if (tile_first >= count || fast_pages < 0) fast_pages = 0;
     fast_pages &= ~1;
+    if (fast_pages < first_page) fast_pages = first_page;          // (first_page is even)
     int trip = 0;
-    if (fast_pages > 0) {
-        ColdOperands next = request_cold(dec_half);
-        for (int first = 0; first < fast_pages; first += 2, trip++) {
+    if (fast_pages > first_page) {
+        ColdOperands next = request_cold(first_page + dec_half);
+        for (int first = first_page; first < fast_pages; first += 2, trip++) {
             const ColdOperands now = next;
             if (first + 2 < fast_pages) next = request_cold(first + 2 + dec_half);
             write_page(trip & 1, dec_half, decode_cold(now));
@@ -255,18 +316,94 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
         __syncthreads();
         attend(std::true_type{}, trip & 1, first);
     }
-    if (t < a.tokens) {
-        const float inv = (has_query && denom > 0.0f) ? 1.0f / denom : 0.0f;   // padding tokens and inactive rows give zeros
 #pragma unroll
-        for (int tile = 0; tile < 4; tile++) {
-            const uint32_t lo = (uint32_t)f32_to_bf16(o[tile][0] * inv) | ((uint32_t)f32_to_bf16(o[tile][1] * inv) << 16);
-            const uint32_t hi = (uint32_t)f32_to_bf16(o[tile][2] * inv) | ((uint32_t)f32_to_bf16(o[tile][3] * inv) << 16);
-            *reinterpret_cast<uint2 *>(a.out + q_at + 16 * tile + 4 * quarter) = make_uint2(lo, hi);
+    for (int i = 0; i < kSets; i++) {
+        if (t[i] >= a.tokens) continue;
+        if (kSplit) {
+            // unnormalised sums, maximum and denominator of this split (a split without a visible
+            // token leaves -inf and 0: the merge gives it no weight)
+            const int64_t at = (q_at[i] / D) * a.splits + split_index;
+            if (first_page < all_pages) {                // (uniform; the merge reads no sums of a split without a denominator)
+#pragma unroll
+                for (int tile = 0; tile < 4; tile++)
+                    *reinterpret_cast<float4 *>(a.part_out + at * D + 16 * tile + 4 * quarter) =
+                        make_float4(o[i][tile][0], o[i][tile][1], o[i][tile][2], o[i][tile][3]);
+            }
+            // (a padding token's vector multiplied zeros on the unmasked trips: it gets no weight either)
+            if (quarter == 0)
+                *reinterpret_cast<float2 *>(a.part_stats + at * 2) =
+                    has_query[i] ? make_float2(running_max[i], denom[i]) : make_float2(-INFINITY, 0.0f);
+        } else {
+            const float inv = (has_query[i] && denom[i] > 0.0f) ? 1.0f / denom[i] : 0.0f;   // padding tokens and inactive rows give zeros
+#pragma unroll
+            for (int tile = 0; tile < 4; tile++) {
+                const uint32_t lo = (uint32_t)f32_to_bf16(o[i][tile][0] * inv) | ((uint32_t)f32_to_bf16(o[i][tile][1] * inv) << 16);
+                const uint32_t hi = (uint32_t)f32_to_bf16(o[i][tile][2] * inv) | ((uint32_t)f32_to_bf16(o[i][tile][3] * inv) << 16);
+                *reinterpret_cast<uint2 *>(a.out + q_at[i] + 16 * tile + 4 * quarter) = make_uint2(lo, hi);
+            }
         }
     }
 }
 
+// One wavefront per query vector: out[d] = sum_s o_s[d] w_s / sum_s denom_s w_s with
+// w_s = exp(max_s - max), splits in index order; a vector no split saw anything of gives zeros.
+// All statistics are requested together, then all sums: two memory round trips per vector.
+constexpr int kPrefillMaxSplits = 16;
+
+template <int kSplits>
+__global__ void __launch_bounds__(256)
+attention_prefill_merge_kernel(const float *__restrict__ part_out, const float *__restrict__ part_stats, int64_t vectors,
+                               uint16_t *__restrict__ out) {
+    const int64_t vector = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int d = threadIdx.x & 63;
+    if (vector >= vectors) return;
+    const float2 *stats = reinterpret_cast<const float2 *>(part_stats) + vector * kSplits;
+    float2 st[kSplits];
+#pragma unroll
+    for (int s = 0; s < kSplits; s++) st[s] = stats[s];
+    float top = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < kSplits; s++) top = fmaxf(top, st[s].x);
+    float sums[kSplits];
+#pragma unroll
+    for (int s = 0; s < kSplits; s++)                    // (a split without a denominator wrote no sums)
+        sums[s] = st[s].y > 0.0f ? part_out[(vector * kSplits + s) * 64 + d] : 0.0f;
+    float total = 0.0f, weight_sum = 0.0f;
+#pragma unroll
+    for (int s = 0; s < kSplits; s++) {
+        const float w = st[s].y > 0.0f ? __expf(st[s].x - top) : 0.0f;
+        weight_sum = weight_sum + st[s].y * w;
+        total = total + sums[s] * w;
+    }
+    out[vector * 64 + d] = f32_to_bf16(weight_sum > 0.0f ? total / weight_sum : 0.0f);
+}
+
 }  // namespace nq
+
+namespace {
+
+constexpr int kPrefillSets = 1;        // query-vector sets per lane (see the kernel)
+constexpr int kPrefillWorkgroups = 2048;
+
+// Splits of the page table: enough workgroups for the chip however few (row, tile, head) triples a
+// launch has, with at least eight pages (four trips) per split.
+int prefill_splits(int batch, int tokens, int max_pages, int group, int kv_heads) {
+    const int tile_tokens = kPrefillSets * 128 / group;
+    const int64_t workgroups = (int64_t)((tokens + tile_tokens - 1) / tile_tokens) * batch * kv_heads;
+    int splits = 1;
+    while (splits < nq::kPrefillMaxSplits && workgroups * splits < kPrefillWorkgroups && (max_pages + splits * 2 - 1) / (splits * 2) >= 8) splits *= 2;
+    return splits;
+}
+
+}  // namespace
+
+extern "C" size_t nq_nqkv_attention_prefill_workspace_bytes(int batch, int tokens, int max_pages, int q_heads,
+                                                            int kv_heads) {
+    if (batch < 1 || tokens < 1 || max_pages < 1 || kv_heads < 1 || q_heads < kv_heads || q_heads % kv_heads) return 0;
+    const int splits = prefill_splits(batch, tokens, max_pages, q_heads / kv_heads, kv_heads);
+    if (splits == 1) return 0;
+    return (size_t)batch * tokens * q_heads * splits * (64 + 2) * sizeof(float);
+}
 
 extern "C" int nq_nqkv_attention_prefill(
     const void *query_dev, const uint8_t *key_codes_dev, const uint8_t *key_beta_ids_dev, const float *key_norms_dev,
@@ -276,7 +413,7 @@ extern "C" int nq_nqkv_attention_prefill(
     const int32_t *sequence_lengths_dev, const void *hot_keys_dev, const void *hot_values_dev,
     const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, const int32_t *counts_dev, int uniform_count,
     int batch, int tokens, int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size,
-    float scale, void *out_dev, void *stream) {
+    float scale, void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream) {
     NQ_REQUIRE(batch >= 1 && tokens >= 1 && slots >= 1 && max_pages >= 1, NQ_ERR_SHAPE,
                "nq_nqkv_attention_prefill: batch, tokens, slots and max_pages must be positive");
     NQ_REQUIRE(kv_heads >= 1 && q_heads >= kv_heads && q_heads % kv_heads == 0, NQ_ERR_SHAPE,
@@ -312,15 +449,43 @@ extern "C" int nq_nqkv_attention_prefill(
     a.slot_ids = slot_ids_dev; a.counts = counts_dev; a.active_mask = active_mask_dev;
     a.batch = batch; a.tokens = tokens; a.uniform_count = uniform_count; a.slots = slots; a.max_pages = max_pages;
     a.q_heads = q_heads; a.kv_heads = kv_heads; a.scale = scale;
-    const int tile_tokens = 128 / group;
+    // the context is split when the caller's workspace has room for the partial results
+    const size_t need = nq_nqkv_attention_prefill_workspace_bytes(batch, tokens, max_pages, q_heads, kv_heads);
+    const bool split = need > 0 && workspace_dev && workspace_bytes >= need && nq::aligned(workspace_dev, 16);
+    const int splits = split ? prefill_splits(batch, tokens, max_pages, group, kv_heads) : 1;
+    const int64_t vectors = (int64_t)batch * tokens * q_heads;
+    a.splits = splits;
+    a.pages_per_split = ((max_pages + splits - 1) / splits + 1) & ~1;
+    a.part_out = reinterpret_cast<float *>(workspace_dev);
+    a.part_stats = a.part_out ? a.part_out + vectors * splits * 64 : nullptr;
+    const int tile_tokens = kPrefillSets * 128 / group;
     const int64_t pairs = (int64_t)((tokens + tile_tokens - 1) / tile_tokens) * batch;     // (row, token tile), padded to eights
-    const dim3 grid((unsigned)((pairs + 7) / 8 * 8 * kv_heads));
+    const dim3 grid((unsigned)((pairs + 7) / 8 * 8 * kv_heads), (unsigned)splits);
     hipStream_t s = (hipStream_t)stream;
+#define NQ_LAUNCH_PREFILL(GROUP)                                                                                     \
+    if (split)                                                                                                       \
+        hipLaunchKernelGGL((nq::attention_prefill_kernel<64, 16, GROUP, kPrefillSets, true>), grid,                  \
+                           dim3(nq::kPrefillThreads), 0, s, a);                                                      \
+    else                                                                                                             \
+        hipLaunchKernelGGL((nq::attention_prefill_kernel<64, 16, GROUP, kPrefillSets, false>), grid,                 \
+                           dim3(nq::kPrefillThreads), 0, s, a)
     switch (group) {
-        case 1: hipLaunchKernelGGL((nq::attention_prefill_kernel<64, 16, 1>), grid, dim3(nq::kPrefillThreads), 0, s, a); break;
-        case 2: hipLaunchKernelGGL((nq::attention_prefill_kernel<64, 16, 2>), grid, dim3(nq::kPrefillThreads), 0, s, a); break;
-        case 4: hipLaunchKernelGGL((nq::attention_prefill_kernel<64, 16, 4>), grid, dim3(nq::kPrefillThreads), 0, s, a); break;
-        default: hipLaunchKernelGGL((nq::attention_prefill_kernel<64, 16, 8>), grid, dim3(nq::kPrefillThreads), 0, s, a); break;
+        case 1: NQ_LAUNCH_PREFILL(1); break;
+        case 2: NQ_LAUNCH_PREFILL(2); break;
+        case 4: NQ_LAUNCH_PREFILL(4); break;
+        default: NQ_LAUNCH_PREFILL(8); break;
+    }
+#undef NQ_LAUNCH_PREFILL
+    if (split) {
+        const int status = nq::check_launch("nq_nqkv_attention_prefill");
+        if (status != NQ_OK) return status;
+        const dim3 merge_grid((unsigned)((vectors + 3) / 4));
+        switch (splits) {                                // a power of two in [2, kPrefillMaxSplits]
+            case 2: hipLaunchKernelGGL(nq::attention_prefill_merge_kernel<2>, merge_grid, dim3(256), 0, s, a.part_out, a.part_stats, vectors, a.out); break;
+            case 4: hipLaunchKernelGGL(nq::attention_prefill_merge_kernel<4>, merge_grid, dim3(256), 0, s, a.part_out, a.part_stats, vectors, a.out); break;
+            case 8: hipLaunchKernelGGL(nq::attention_prefill_merge_kernel<8>, merge_grid, dim3(256), 0, s, a.part_out, a.part_stats, vectors, a.out); break;
+            default: hipLaunchKernelGGL(nq::attention_prefill_merge_kernel<16>, merge_grid, dim3(256), 0, s, a.part_out, a.part_stats, vectors, a.out); break;
+        }
     }
     return nq::check_launch("nq_nqkv_attention_prefill");
 }

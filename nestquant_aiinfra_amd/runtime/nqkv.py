@@ -482,11 +482,13 @@ def nqkv_decode_attention_batched_k1(query: torch.Tensor, cache: NQKVHotColdCach
 
 def nqkv_prefill_attention(query: torch.Tensor, cache: NQKVHotColdCache, *, slot_ids: torch.Tensor,
                            active_mask: torch.Tensor, counts: torch.Tensor | None = None, uniform_count: int | None = None,
-                           scale: float | None = None) -> torch.Tensor:
+                           scale: float | None = None, split_context: bool = True) -> torch.Tensor:
     """Causal attention of a chunk of new tokens over the packed cache, after the chunk was
     written: query BF16 [batch, tokens, query_heads, head_dim] (rotated like the stored keys);
     row r holds counts[r] (or uniform_count) new tokens that end at the slot's sequence length.
-    Returns BF16 [batch, tokens, query_heads, head_dim]; padding tokens give zeros."""
+    Returns BF16 [batch, tokens, query_heads, head_dim]; padding tokens give zeros.  `split_context`
+    lets the library split long page tables over more workgroups (partial results in a scratch buffer,
+    merged by a second launch); without it one workgroup walks a row's whole context."""
     if not isinstance(query, torch.Tensor) or query.ndim != 4 or query.dtype != torch.bfloat16:
         raise ValueError("query must be BF16 [batch, tokens, query_heads, head_dim]")
     pool, meta = cache.pool, cache.metadata
@@ -504,7 +506,13 @@ def nqkv_prefill_attention(query: torch.Tensor, cache: NQKVHotColdCache, *, slot
     attention_scale = 1.0 / math.sqrt(dim) if scale is None else float(scale)
     query = query.contiguous()
     out = torch.empty_like(query)
-    _native.check(_native.library().nq_nqkv_attention_prefill(
+    lib = _native.library()
+    # room for the partial results of a split context (long tables, few rows): the kernel then
+    # spreads every row over the chip in proportion to its context
+    need = 0 if not split_context else lib.nq_nqkv_attention_prefill_workspace_bytes(
+        batch, tokens, cache.max_pages_per_sequence, heads, pool.num_kv_heads)
+    workspace = torch.empty(need, dtype=torch.uint8, device=query.device) if need else None
+    _native.check(lib.nq_nqkv_attention_prefill(
         query.data_ptr(), pool.key_codes.data_ptr(), pool.key_betas.data_ptr(), pool.key_norms.data_ptr(),
         pool.value_codes.data_ptr(), pool.value_betas.data_ptr(), pool.value_norms.data_ptr(),
         pool.beta_table.data_ptr(), pool.value_beta_table.data_ptr(), meta.page_indices.data_ptr(),
@@ -513,7 +521,8 @@ def nqkv_prefill_attention(query: torch.Tensor, cache: NQKVHotColdCache, *, slot
         slot_ids.data_ptr(), active_mask.data_ptr(), None if counts is None else counts.data_ptr(),
         0 if uniform_count is None else int(uniform_count), batch, tokens, cache.max_sequences,
         cache.max_pages_per_sequence, heads, pool.num_kv_heads, dim, pool.page_size, attention_scale,
-        out.data_ptr(), _native.stream_handle(query.device)))
+        out.data_ptr(), None if workspace is None else workspace.data_ptr(), need,
+        _native.stream_handle(query.device)))
     return out
 
 

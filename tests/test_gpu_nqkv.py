@@ -317,8 +317,9 @@ def test_attention_chunk_sizes(kv, oracle, capacity, max_len, q_heads):
         assert relative_error(_f32(out[row]), ref) <= 1e-2, (row, lengths[row])
 
 
+@pytest.mark.parametrize("split_context", [False, True])
 @pytest.mark.parametrize("q_heads", [8, 32, 64])
-def test_prefill_attention_over_the_packed_cache(kv, oracle, q_heads):
+def test_prefill_attention_over_the_packed_cache(kv, oracle, q_heads, split_context):
     """Chunks of new tokens attend causally to everything their slot holds: a fresh prompt that
     crosses pages, a continuation of a sequence with cold pages, a one-token chunk, a padded row."""
     rng = np.random.default_rng(100 + q_heads)
@@ -349,7 +350,7 @@ def test_prefill_attention_over_the_packed_cache(kv, oracle, q_heads):
 
     query = _bf16(oracle.hadamard(rng.standard_normal((4, width, q_heads, DIM)).astype(np.float32))).cuda()
     out = kv.nqkv_prefill_attention(query, manager.layers[0], slot_ids=manager.step_slot_ids, active_mask=manager.step_active,
-                                    counts=manager.step_counts)
+                                    counts=manager.step_counts, split_context=split_context)
     assert out.dtype == torch.bfloat16 and tuple(out.shape) == (4, width, q_heads, DIM)
     for i in live:
         slot = slots[i]
@@ -368,6 +369,51 @@ def test_prefill_attention_over_the_packed_cache(kv, oracle, q_heads):
         query[:, counts[i] - 1].contiguous(), manager.layers[0], slot_ids=manager.step_slot_ids[:4].clone(),
         active_mask=torch.tensor([True, False, False, False], device="cuda"))
     assert relative_error(_f32(out[i, counts[i] - 1]), _f32(decode[0])) <= 2e-2
+
+
+def test_prefill_attention_with_the_context_split_over_workgroups(kv, oracle):
+    """Long contexts, few rows: with a workspace the page table of every slot is split into ranges
+    that workgroups of their own attend over and a second launch merges (`split_context`).  Same
+    attention as the single walk (up to the rounding of the merged sums) and as the oracle's dense
+    softmax; rows with short contexts, a padded row and ragged chunk lengths among them."""
+    rng = np.random.default_rng(2027)
+    q_heads = 32
+    manager = _manager(kv, capacity=4, max_len=2048)
+    for s in range(4):
+        manager.register(s, slot=s)
+    history = {0: 1500, 1: 40, 2: 0, 3: 700}
+    keys = {s: _bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for s, n in history.items()}
+    values = {s: _bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for s, n in history.items()}
+    old = [s for s in history if history[s]]
+    _append(manager, old, [keys[s] for s in old], [values[s] for s in old])
+    slots, counts = [0, 1, 2, 3], [100, 64, 0, 17]
+    new_k = [_bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for n in counts]
+    new_v = [_bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for n in counts]
+    width = max(counts)
+    key = torch.zeros((4, width, HEADS, DIM), dtype=torch.bfloat16)
+    value = torch.zeros_like(key)
+    for i, n in enumerate(counts):
+        key[i, :n], value[i, :n] = new_k[i], new_v[i]
+    manager.step_slot_ids[:4] = torch.tensor(slots, dtype=torch.int32)
+    manager.step_active[:4] = torch.tensor([n > 0 for n in counts])
+    manager.step_counts[:4] = torch.tensor(counts, dtype=torch.int32)
+    manager.begin_step(rows=4, uniform_count=None)
+    manager.write_layer(0, key.cuda(), value.cuda())
+    query = _bf16(oracle.hadamard(rng.standard_normal((4, width, q_heads, DIM)).astype(np.float32))).cuda()
+    call = lambda split: kv.nqkv_prefill_attention(query, manager.layers[0], slot_ids=manager.step_slot_ids,
+                                                   active_mask=manager.step_active, counts=manager.step_counts,
+                                                   split_context=split)
+    walked, split = call(False), call(True)
+    assert torch.equal(split, call(True))                       # the merge adds the ranges in order
+    assert relative_error(_f32(split), _f32(walked)) <= 4e-3
+    assert not split[2].any() and not split[3, counts[3]:].any() and not split[1, counts[1]:].any()
+    for i in (0, 3):
+        slot = slots[i]
+        k_view, v_view = _cache_view(oracle, torch.cat([keys[slot], new_k[i]]), torch.cat([values[slot], new_v[i]]))
+        for token in (0, counts[i] - 1):
+            visible = history[slot] + token + 1
+            ref = oracle.attention_dense(_f32(query[i, token].cpu()), k_view[:visible], v_view[:visible])
+            assert relative_error(_f32(split[i, token]), ref) <= 1e-2, (i, token)
 
 
 def test_pool_handles_are_generation_checked(kv):
