@@ -543,12 +543,24 @@ def attention_extra(device):
     prefill = time_graph(lambda i: nqkv.nqkv_prefill_attention(
         chunk_query, manager.layers[i % 4], slot_ids=slot_ids, active_mask=active, uniform_count=chunk, scale=0.125), 8)
     prefill_flops = sum(4 * 32 * 64 * sum(n - chunk + t + 1 for t in range(chunk)) for n in lengths)
+    # the same chunk with one workgroup per (row, token tile, KV head) walking the whole context, and the
+    # longest row alone (one sequence's chunked prefill), with and without the split of the context
+    walked = time_graph(lambda i: nqkv.nqkv_prefill_attention(
+        chunk_query, manager.layers[i % 4], slot_ids=slot_ids, active_mask=active, uniform_count=chunk, scale=0.125,
+        split_context=False), 8)
+    longest = max(range(8), key=lambda row: lengths[row])
+    one_slot = slot_ids[longest:longest + 1].clone()
+    one = {split: time_graph(lambda i: nqkv.nqkv_prefill_attention(
+        chunk_query[:1], manager.layers[i % 4], slot_ids=one_slot, active_mask=active[:1], uniform_count=chunk, scale=0.125,
+        split_context=split), 8) for split in (True, False)}
     return {"contexts": lengths, "us": seconds * 1e6, "algorithmic_bytes": bytes_moved,
             "GBps": bytes_moved / seconds / 1e9, "hbm_frac": bytes_moved / seconds / 1e9 / HBM_PEAK_GBPS,
             "stage1_us": stage1 * 1e6, "stage1_hbm_frac": bytes_moved / stage1 / 1e9 / HBM_PEAK_GBPS,
             "append_launch_us": write * 1e6,
             "prefill_chunk128": {"us": prefill * 1e6, "flops": prefill_flops,
-                                 "TFLOPs": prefill_flops / prefill / 1e12}}
+                                 "TFLOPs": prefill_flops / prefill / 1e12, "us_without_context_split": walked * 1e6,
+                                 "longest_row_alone_us": one[True] * 1e6,
+                                 "longest_row_alone_us_without_context_split": one[False] * 1e6}}
 
 
 def tpot_extra(device, batches=(1, 8), prompt=128, generate=128):
