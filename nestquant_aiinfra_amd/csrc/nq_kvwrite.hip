@@ -251,8 +251,11 @@ __global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
             const float *key, *value;
             __device__ __forceinline__ const float *operator()(int r) const { return r < P ? key : value; }
         } betas_of{a.key_betas, a.value_betas};
-        quantize_staged_pairs<false>(&rows[0][0], row_scale, D, 14.0f, 1.0f / 14.0f, betas_of, a.key_beta_count,
-                                     0u, 0, 2 * P * kBlocks * 4, sink);
+        // one lane per block, its betas in turn (the 2 P x 8 blocks of the page's key and value rows are the
+        // workgroup's 256 lanes; a wavefront holds rows of one kind): fewer instructions per block than
+        // a lane per (block, beta) pair, which is what a many-page prompt pays for
+        quantize_staged_blocks(&rows[0][0], row_scale, D, 14.0f, 1.0f / 14.0f, betas_of, a.key_beta_count, 0,
+                               2 * P * kBlocks, sink);
     }
 }
 
