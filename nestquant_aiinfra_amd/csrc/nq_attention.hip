@@ -229,7 +229,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     const int row_in_page = token * a.kv_heads + g;
     const int64_t page_words = (int64_t)P * a.kv_heads * kBlocks, page_rows = (int64_t)P * a.kv_heads;
 
-    // ---- round 1: slot, activity, queries (and the new key and value) ------------------------------
+    // ---- first loads: slot, activity, queries (and the new key and value) --------------------------
     const int given_slot = a.slot_ids[row];
     const bool row_active = a.active_mask[row] != 0;
     // lane 8 h + piece of the first wavefront holds elements 8 piece .. 8 piece + 7 of head h; the
@@ -266,7 +266,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     const float key_beta[4] = {a.key_betas[0], a.key_betas[1], a.key_betas[2], a.key_betas[3]};
     const float value_beta[4] = {a.value_betas[0], a.value_betas[1], a.value_betas[2], a.value_betas[3]};
 
-    // ---- round 2: lengths and page ids of the slot ------------------------------------------------
+    // ---- second loads: lengths and page ids of the slot -------------------------------------------
     const bool slot_known = given_slot >= 0 && given_slot < a.slots;
     const int slot = given_slot < 0 ? 0 : (given_slot >= a.slots ? a.slots - 1 : given_slot);
     const int page_count = a.page_counts[slot], last_len = a.last_page_lens[slot], hot_len = a.hot_lengths[slot];
@@ -297,7 +297,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
         return;
     }
 
-    // ---- round 3: the packed operands of all passes, keys and values -----------------------------------
+    // ---- third loads: the packed operands of all passes, keys and values --------------------------------
     bool pass_valid[kPasses];
     uint32_t k_code[kPasses], k_ids[kPasses], v_code[kPasses], v_ids[kPasses];
     float k_norm[kPasses], v_norm[kPasses];
