@@ -43,7 +43,8 @@ def _rms_norm(h, weight, eps):
     return weight * x.to(h.dtype)
 
 
-@pytest.mark.parametrize("rows,n", [(1, 2048), (8, 2048), (3, 256), (5, 8192), (40, 512), (1100, 2048), (4200, 512)])
+@pytest.mark.parametrize("rows,n", [(1, 2048), (8, 2048), (3, 256), (5, 8192), (40, 512), (1100, 2048), (4200, 512),
+                                    (64, 2048), (150, 4096), (128, 8192), (300, 2048), (500, 8192)])   # prefill chunks
 @pytest.mark.parametrize("with_residual", [False, True])
 def test_residual_rmsnorm_stage(rt, rows, n, with_residual):
     g = torch.Generator().manual_seed(rows * n + with_residual)
@@ -71,7 +72,7 @@ def test_residual_rmsnorm_stage(rt, rows, n, with_residual):
     assert none is None and torch.equal(staged_only, staged)
 
 
-@pytest.mark.parametrize("rows,n", [(1, 8192), (8, 8192), (2, 512), (300, 8192)])
+@pytest.mark.parametrize("rows,n", [(1, 8192), (8, 8192), (2, 512), (300, 8192), (40, 2048), (100, 8192), (192, 4096)])
 def test_swiglu_stage(rt, rows, n):
     g = torch.Generator().manual_seed(rows + n)
     gate = (2 * torch.randn(rows, n, generator=g)).to(torch.bfloat16).cuda()
