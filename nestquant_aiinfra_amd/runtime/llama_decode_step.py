@@ -95,6 +95,7 @@ class FusedLlamaDecodeStep:
         self._rope_tables: torch.Tensor | None = None
         self.expand_weights = bool(expand_weights)
         self._expanded: dict[int, tuple] = {}
+        self._weights: dict[int, tuple] = {}
 
     def _rope(self, embedded: torch.Tensor, positions: torch.Tensor, *, padded: bool = False
               ) -> tuple[torch.Tensor, torch.Tensor]:
@@ -123,6 +124,16 @@ class FusedLlamaDecodeStep:
         _require(prepared.resolved_words is not None, "weight has no resolved form")
         return prepared
 
+    def _layer_weights(self, index: int, device) -> tuple[PreparedNQRTLinear, ...]:
+        """The seven prepared projections of layer `index` (q, k, v, o, gate, up, down), looked up once
+        and kept while the modules still hold them on this device."""
+        linears = self.layers[index][3]
+        kept = self._weights.get(index)
+        if (kept is None or kept[0].code_payload.device != device
+                or not all(weight is linear._prepared for weight, linear in zip(kept, linears))):
+            kept = self._weights[index] = tuple(self._prepared(linear, device) for linear in linears)
+        return kept
+
     @staticmethod
     def _gemv_rows(activation) -> int:
         return MATRIX_CORE_GEMV_ROWS if activation.feature_count % 128 == 0 else 8
@@ -136,7 +147,7 @@ class FusedLlamaDecodeStep:
         if activation.token_count <= self._gemv_rows(activation):
             return linear_packed_w4a4_gemv_grouped(activation, prepared, output_dtype=torch.bfloat16)
         if can_use_w4a4_gemm_grouped(activation, prepared):      # a long prefill: one product for the group
-            return linear_packed_w4a4_gemm_grouped(activation, prepared)
+            return linear_packed_w4a4_gemm_grouped(activation, prepared, checked=True)
         return [self._linear(activation, weight) for weight in prepared]
 
     def _expanded_layer(self, index: int, device) -> tuple | None:
@@ -186,7 +197,7 @@ class FusedLlamaDecodeStep:
 
         delta, residual = embedded.view(rows, self.hidden), None
         for index, (layer, attention, mlp, linears) in enumerate(self.layers):
-            q_w, k_w, v_w, o_w, gate_w, up_w, down_w = (self._prepared(linear, device) for linear in linears)
+            q_w, k_w, v_w, o_w, gate_w, up_w, down_w = self._layer_weights(index, device)
             table = linears[0].activation_beta_table
             activation, residual, _ = fused_input_stage(
                 delta, mode="rmsnorm", residual=residual, norm_weight=layer.input_layernorm.weight,
@@ -256,7 +267,7 @@ class FusedLlamaPrefillStep(FusedLlamaDecodeStep):
 
         delta, residual = embedded.reshape(count, self.hidden), None
         for index, (layer, attention, mlp, linears) in enumerate(self.layers):
-            q_w, k_w, v_w, o_w, gate_w, up_w, down_w = (self._prepared(linear, device) for linear in linears)
+            q_w, k_w, v_w, o_w, gate_w, up_w, down_w = self._layer_weights(index, device)
             table = linears[0].activation_beta_table
             activation, residual, _ = fused_input_stage(
                 delta, mode="rmsnorm", residual=residual, norm_weight=layer.input_layernorm.weight,

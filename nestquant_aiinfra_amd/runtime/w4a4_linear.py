@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import weakref
 from dataclasses import dataclass
 from typing import Any, Sequence
 
@@ -203,16 +204,21 @@ def fused_input_stage(inputs: torch.Tensor, *, mode: str, q: int = 14, beta_tabl
     if mode not in ("rmsnorm", "swiglu"):
         raise ValueError("mode must be 'rmsnorm' or 'swiglu'")
     device = _native.require_cuda(inputs)
-    others = [t for t in (residual, norm_weight, gate) if t is not None]
-    if inputs.dtype != torch.bfloat16 or any(t.dtype != torch.bfloat16 for t in others):
-        raise TypeError("the fused input stage takes BF16 tensors")
-    if not inputs.is_contiguous() or any(not t.is_contiguous() for t in others):
-        raise RuntimeError("fused input stage tensors must be contiguous")
+    bf16 = torch.bfloat16
+    if inputs.dtype != bf16 or not inputs.is_contiguous():
+        raise (TypeError("the fused input stage takes BF16 tensors") if inputs.dtype != bf16
+               else RuntimeError("fused input stage tensors must be contiguous"))
+    for name, tensor in (("residual", residual), ("gate", gate), ("norm_weight", norm_weight)):
+        if tensor is None:
+            continue
+        if tensor.dtype != bf16:
+            raise TypeError("the fused input stage takes BF16 tensors")
+        if not tensor.is_contiguous():
+            raise RuntimeError("fused input stage tensors must be contiguous")
+        if name != "norm_weight" and tensor.shape != inputs.shape:
+            raise ValueError(f"{name} must have the shape of inputs")
     n = inputs.shape[-1]
     count = inputs.numel() // n
-    for name, tensor in (("residual", residual), ("gate", gate)):
-        if tensor is not None and tensor.shape != inputs.shape:
-            raise ValueError(f"{name} must have the shape of inputs")
     if mode == "rmsnorm" and (norm_weight is None or norm_weight.numel() != n):
         raise ValueError("mode 'rmsnorm' needs a norm weight of the feature size")
     if mode == "swiglu" and gate is None:
@@ -478,18 +484,12 @@ def linear_packed_w4a4_gemv_grouped(activation: PreparedNQA4Activation, weights:
     dtype = output_dtype or _kernel_dtype(activation)
     device = activation.decoded.device
     count = len(weights)
-    sizes = [w.record.indices.shape[0] for w in weights]
+    _, sizes, _, words, tails, norms, betas, widths, offsets, seeds, _ = _group_plan(weights)
     outs = [torch.empty((m, n), dtype=dtype, device=device) for n in sizes]
-    pointers = ctypes.c_void_p * count
     _native.check(_native.library().nq_w4a4_gemv_grouped(
-        activation.decoded.data_ptr(), count,
-        pointers(*[w.resolved_words.data_ptr() for w in weights]),
-        pointers(*[w.resolved_tails.data_ptr() for w in weights]),
-        pointers(*[w.row_norms.data_ptr() for w in weights]),
-        pointers(*[w.beta_table.data_ptr() for w in weights]),
-        (ctypes.c_int * count)(*sizes), (ctypes.c_int64 * count)(*([0] * count)),
-        (ctypes.c_int64 * count)(*[int(w.record.dither_seed) for w in weights]),
-        pointers(*[o.data_ptr() for o in outs]), m, k, _native.dtype_tag(dtype), _native.stream_handle(device)))
+        activation.decoded.data_ptr(), count, words, tails, norms, betas, widths, offsets, seeds,
+        (ctypes.c_void_p * count)(*[o.data_ptr() for o in outs]), m, k, _native.dtype_tag(dtype),
+        _native.stream_handle(device)))
     return [o.reshape(*activation.original_shape[:-1], n) for o, n in zip(outs, sizes)]
 
 
@@ -660,6 +660,34 @@ def bf16_gemm(rows: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split
 
 FUSED_GROUP_MAX_ROWS = 512                  # one chunk of the fused kernel
 
+# What a grouped launch passes for its weights never changes while the weights live: the pointer,
+# size, offset and seed arrays are built once per group (keyed by the weights' identities, dropped
+# with the first weight that is collected).
+_group_plans: dict[tuple[int, ...], tuple] = {}
+
+
+def _group_plan(weights: Sequence[PreparedNQRTLinear]) -> tuple:
+    """(weak references, sizes, their sum, words, tails, norms, betas, sizes as int, zero offsets,
+    seeds, sizes as int64) of the resolved weights of one grouped launch."""
+    key = tuple(id(w) for w in weights)
+    plan = _group_plans.get(key)
+    if plan is not None and all(ref() is w for ref, w in zip(plan[0], weights)):
+        return plan
+    count = len(weights)
+    array = ctypes.c_void_p * count
+    sizes = [int(w.record.indices.shape[0]) for w in weights]
+    forget = lambda _, key=key: _group_plans.pop(key, None)
+    plan = (tuple(weakref.ref(w, forget) for w in weights), sizes, sum(sizes),
+            array(*[w.resolved_words.data_ptr() for w in weights]),
+            array(*[w.resolved_tails.data_ptr() for w in weights]),
+            array(*[w.row_norms.data_ptr() for w in weights]),
+            array(*[w.beta_table.data_ptr() for w in weights]),
+            (ctypes.c_int * count)(*sizes), (ctypes.c_int64 * count)(*([0] * count)),
+            (ctypes.c_int64 * count)(*[int(w.record.dither_seed) for w in weights]),
+            (ctypes.c_int64 * count)(*sizes))
+    _group_plans[key] = plan
+    return plan
+
 
 def _fused_group(activation: PreparedNQA4Activation, weights: Sequence[PreparedNQRTLinear]) -> bool:
     """A group the fused kernel takes in one launch: a prefill below the decode-once size."""
@@ -681,37 +709,36 @@ def can_use_w4a4_gemm_grouped(activation: PreparedNQA4Activation, weights: Seque
             and all(w.record.indices.shape[0] % 256 == 0 for w in weights))
 
 
-def linear_packed_w4a4_gemm_grouped(activation: PreparedNQA4Activation,
-                                    weights: Sequence[PreparedNQRTLinear]) -> list[torch.Tensor]:
+def linear_packed_w4a4_gemm_grouped(activation: PreparedNQA4Activation, weights: Sequence[PreparedNQRTLinear], *,
+                                    checked: bool = False) -> list[torch.Tensor]:
     """The linears of the weights that share one activation (q, k and v; gate and up) in a prefill,
     as one product.  From 288 rows on every weight is decoded once into its rows of one BF16 scratch
     and one dense matrix-core GEMM over the stacked rows stores each projection's columns to a BF16
     [M, N_i] output of its own; below, one launch of the fused kernel walks the channels of all the
-    weights.  Same values as one `linear_packed_w4a4_mma_chunked_staged` per weight."""
-    if not can_use_w4a4_gemm_grouped(activation, weights):
+    weights.  Same values as one `linear_packed_w4a4_mma_chunked_staged` per weight.  `checked`:
+    the caller has just asked `can_use_w4a4_gemm_grouped`."""
+    if not checked and not can_use_w4a4_gemm_grouped(activation, weights):
         raise ValueError("grouped prefill linears take the weights of one decoded activation, K a multiple of 128: "
                          f"2 or 3 with every N a multiple of 256 from {DECODE_ONCE_ROWS} rows on, up to 4 resolved "
                          f"ones with every N a multiple of 32 between {MATRIX_CORE_GEMV_ROWS + 1} rows and that")
     rows = activation.decoded.reshape(activation.token_count, activation.feature_count)
     device = _native.require_cuda(rows)
     m, k = rows.shape
-    sizes = [int(w.record.indices.shape[0]) for w in weights]
-    count = len(sizes)
-    outs = [torch.empty((m, size), dtype=torch.bfloat16, device=device) for size in sizes]
-    pointers = (ctypes.c_void_p * count)(*[out.data_ptr() for out in outs])
+    count = len(weights)
     lib = _native.library()
     if _fused_group(activation, weights):
-        array = ctypes.c_void_p * count
-        need = lib.nq_w4a4_gemm_grouped_workspace_bytes(m, k, sum(sizes))
+        _, sizes, total, words, tails, norms, betas, widths, offsets, seeds, _ = _group_plan(weights)
+        outs = [torch.empty((m, size), dtype=torch.bfloat16, device=device) for size in sizes]
+        pointers = (ctypes.c_void_p * count)(*[out.data_ptr() for out in outs])
+        need = lib.nq_w4a4_gemm_grouped_workspace_bytes(m, k, total)
         workspace = _workspace(device, need) if need else None
         _native.check(lib.nq_w4a4_gemm_grouped(
-            rows.data_ptr(), count, array(*[w.resolved_words.data_ptr() for w in weights]),
-            array(*[w.resolved_tails.data_ptr() for w in weights]), array(*[w.row_norms.data_ptr() for w in weights]),
-            array(*[w.beta_table.data_ptr() for w in weights]), (ctypes.c_int * count)(*sizes),
-            (ctypes.c_int64 * count)(*([0] * count)),
-            (ctypes.c_int64 * count)(*[int(w.record.dither_seed) for w in weights]), pointers, m, k,
+            rows.data_ptr(), count, words, tails, norms, betas, widths, offsets, seeds, pointers, m, k,
             None if workspace is None else workspace.data_ptr(), need, _native.stream_handle(device)))
     else:
+        sizes = [int(w.record.indices.shape[0]) for w in weights]
+        outs = [torch.empty((m, size), dtype=torch.bfloat16, device=device) for size in sizes]
+        pointers = (ctypes.c_void_p * count)(*[out.data_ptr() for out in outs])
         stacked = _workspace(device, sum(sizes) * k * 2)[: sum(sizes) * k * 2].view(torch.bfloat16).view(sum(sizes), k)
         first = 0
         for weight, size in zip(weights, sizes):
