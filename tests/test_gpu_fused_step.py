@@ -205,7 +205,11 @@ def test_rotary_embedding_inside_writer_and_attention():
 
 @pytest.mark.parametrize("heads,dim", [(8, 64), (3, 128)])
 def test_rope_and_rotation_of_head_vectors_in_one_launch(rt, heads, dim):
-    from nestquant_aiinfra_amd.core.rotation import hadamard
+    from nestquant_aiinfra_amd.core.rotation import _staged
+
+    def hadamard(x):            # the tensor-operation butterflies, on the GPU (not the stand-alone kernel)
+        return _staged(x.reshape(-1, x.shape[-1]).contiguous(), x.shape[-1]).reshape(x.shape)
+
     rows = 37
     g = torch.Generator().manual_seed(heads * dim)
     x = torch.randn(rows, heads, dim, generator=g).to(torch.bfloat16).cuda()

@@ -173,8 +173,16 @@ def test_dispatch_counters_and_m_routes(tiny):
 def test_fused_rotation_matches_separate_rotation(oracle):
     """Encoding with the rotation fused equals rotating first with the stand-alone kernel,
     which equals the tensor-op Hadamard in the same dtype."""
-    from nestquant_aiinfra_amd.core.rotation import hadamard
+    from nestquant_aiinfra_amd.core import rotation
     from nestquant_aiinfra_amd.runtime import w4a4_linear as rt
+
+    def hadamard(x):
+        # the butterfly network written with tensor operations (what rotation.hadamard runs for host
+        # tensors), evaluated on the GPU: rotation.hadamard itself hands GPU tensors to the kernel
+        n = x.shape[-1]
+        return rotation._staged(x.reshape(-1, n).contiguous(), n).reshape(x.shape)
+
+    assert torch.equal(rotation.hadamard(torch.ones(2, 64, device="cuda")), hadamard(torch.ones(2, 64, device="cuda")))
     for dtype in (torch.bfloat16, torch.float32):
         x = torch.randn(5, 2048, device="cuda").to(dtype)
         rotated = rt.hadamard_cuda(x)
