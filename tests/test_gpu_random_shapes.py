@@ -172,3 +172,180 @@ def test_kv_writer_and_attention_over_random_batches(kv, oracle, sweep_seed):
                     visible = lengths[row] - tokens + t + 1
                     ref = oracle.attention_dense(_f32(queries[row, t].cpu()), views[s][0][:visible], views[s][1][:visible])
                     assert relative_error(_f32(got[row, t]), ref) <= 2e-2, ("prefill attention", split, row, t, case)
+
+
+@pytest.mark.parametrize("sweep_seed", [3, 41])
+def test_appending_attention_over_random_steps(kv, oracle, sweep_seed):
+    """The decode step's one-launch form (`append_and_attend`) against writer + attention on a second
+    cache fed the same tokens, as in test_gpu_nqkv.py, but with the rows in a step, the slots whose
+    cache is switched off, the slot order, the starting lengths and the head counts drawn at random."""
+    heads, dim, page = nqkv_cases.HEADS, nqkv_cases.DIM, nqkv_cases.PAGE
+    _bf16, _f32 = nqkv_cases._bf16, nqkv_cases._f32
+    rng = np.random.default_rng(sweep_seed)
+    for _ in range(30):
+        capacity = int(rng.choice([1, 2, 4, 8]))
+        max_len = int(rng.choice([64, 256, 1024, 2048]))
+        q_heads = int(rng.choice([8, 16, 32, 64]))
+        rows = int(rng.integers(1, capacity + 1))
+        slots = [int(s) for s in rng.permutation(capacity)[:rows]]
+        lengths = [int(rng.integers(1, max_len - 8)) if rng.integers(3) else int(rng.choice([1, 15, 16, 17, max_len - 20]))
+                   for _ in slots]
+        steps = int(rng.integers(18, 36))
+        case = (capacity, max_len, q_heads, slots, lengths, steps)
+        managers = [nqkv_cases._manager(kv, capacity=capacity, max_len=max_len) for _ in range(2)]
+        keys = [_bf16(oracle.hadamard(rng.standard_normal((n, heads, dim)).astype(np.float32))) for n in lengths]
+        values = [_bf16(rng.standard_normal((n, heads, dim)).astype(np.float32)) for n in lengths]
+        for manager in managers:
+            for s in slots:
+                manager.register(f"seq{s}", slot=s)
+            nqkv_cases._append(manager, slots, keys, values)
+        workspaces = [kv.BatchedNQKVAttentionWorkspace.create(m.layers[0], batch_size=rows, query_heads=q_heads,
+                                                              output_dtype=torch.bfloat16) for m in managers]
+        totals = list(lengths)
+        for step in range(steps):
+            in_step = [bool(rng.random() < 0.85) for _ in slots]
+            cache_on = [bool(rng.random() < 0.9) for _ in range(capacity)]
+            key = _bf16(rng.standard_normal((rows, heads, dim)).astype(np.float32)).cuda()
+            value = _bf16(rng.standard_normal((rows, heads, dim)).astype(np.float32)).cuda()
+            query = _bf16(rng.standard_normal((rows, q_heads, dim)).astype(np.float32)).cuda()
+            angles = np.asarray(totals, dtype=np.float64)[:, None] * (500000.0 ** (-np.arange(0, dim, 2) / dim))[None, :]
+            cos = _bf16(np.concatenate([np.cos(angles)] * 2, axis=1).astype(np.float32)).cuda()
+            sin = _bf16(np.concatenate([np.sin(angles)] * 2, axis=1).astype(np.float32)).cuda()
+            packs = []
+            for i in range(rows):
+                grows = in_step[i] and totals[i] < managers[0].max_tokens
+                totals[i] += 1 if grows else 0
+                packs.append(in_step[i] and totals[i] % page == 0)
+            outputs = []
+            for which, (manager, workspace) in enumerate(zip(managers, workspaces)):
+                manager.step_slot_ids[:rows] = torch.tensor(slots, dtype=torch.int32)
+                manager.step_active[:rows] = torch.tensor(in_step)
+                manager.metadata.active_mask[:capacity] = torch.tensor(cache_on)
+                manager.begin_step(rows=rows, uniform_count=1)
+                if which == 0:
+                    manager.write_layer(0, key.view(rows, 1, heads, dim), value.view(rows, 1, heads, dim), rotate_keys=True,
+                                        rope=(cos.view(rows, 1, dim), sin.view(rows, 1, dim)))
+                    out = kv.launch_nqkv_decode_attention(query, manager.layers[0], slot_ids=manager.step_slot_ids,
+                                                          active_mask=manager.step_active, attention_scale=0.125,
+                                                          workspace=workspace, rotate_query=True, rope=(cos, sin))
+                else:
+                    out = manager.append_and_attend(0, query, key, value, attention_scale=0.125, workspace=workspace,
+                                                    rotate=True, rope=(cos, sin))
+                outputs.append(out.clone())
+            torch.cuda.synchronize()
+            two, one = outputs
+            for i in range(rows):
+                if packs[i]:
+                    assert relative_error(_f32(one[i]), _f32(two[i])) <= 2.0 ** -7, (step, i, case)
+                else:
+                    assert torch.equal(one[i], two[i]), (step, i, case)
+                if not cache_on[slots[i]] or not in_step[i]:
+                    assert not one[i].any(), (step, i, case)
+            a, b = managers
+            for name in ("sequence_lengths", "page_counts", "last_page_lens", "hot_lengths"):
+                assert torch.equal(getattr(a.metadata, name), getattr(b.metadata, name)), (step, name, case)
+            assert [a.total_tokens(s) for s in slots] == totals, (step, case)
+            for name in ("key_codes", "key_betas", "key_norms", "value_codes", "value_betas", "value_norms"):
+                assert torch.equal(getattr(a.layers[0].pool, name), getattr(b.layers[0].pool, name)), (step, name, case)
+            assert torch.equal(a.layers[0].hot_keys, b.layers[0].hot_keys), (step, case)
+            assert torch.equal(a.layers[0].hot_values, b.layers[0].hot_values), (step, case)
+
+
+from test_gpu_model import tiny  # noqa: E402,F401  (the two-layer model and its runner, one instance for this file)
+
+
+@pytest.mark.parametrize("sweep_seed", [9, 58])
+def test_runner_graph_equals_eager_under_slot_churn(tiny, sweep_seed):
+    """A scripted engine on the tiny model: prompts of random lengths enter free slots, live slots take
+    further prompt chunks, random subsets of the live slots decode in random row order, slots are
+    released and reused.  Every decode step runs twice from the same cache state, through the
+    captured graph and un-captured, and must give the same logits, tables, hot tails and pages bit
+    for bit; bursts on the device sampler must choose the tokens that step-by-step argmax chooses."""
+    _, runner, *_ = tiny
+    cache, meta = runner.cache, runner.cache.manager.metadata
+    runner.release_slots([s for s in range(runner.batch_size) if cache.manager.sequence_id(s) is not None])
+    if not runner.graph_captured:
+        runner.capture()
+    rng = np.random.default_rng(sweep_seed)
+    generator = torch.Generator().manual_seed(sweep_seed)
+    tensors = [meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths]
+    for layer in cache.manager.layers:
+        pool = layer.pool
+        tensors += [layer.hot_keys, layer.hot_values, pool.key_codes, pool.key_betas, pool.key_norms,
+                    pool.value_codes, pool.value_betas, pool.value_norms]
+
+    def snapshot():
+        return [t.clone() for t in tensors], list(cache._host_lengths)
+
+    def restore(saved):
+        for tensor, value in zip(tensors, saved[0]):
+            tensor.copy_(value)
+        cache._host_lengths[:] = saved[1]
+
+    live: dict[int, list[int]] = {}                          # slot -> [tokens held, next token]
+    limit = runner.max_cache_len
+    decoded = 0
+    for event in range(50):
+        free = [s for s in range(runner.batch_size) if s not in live]
+        choice = rng.random()
+        if free and (not live or choice < 0.25):             # new prompts into free slots
+            slots = [int(s) for s in rng.permutation(free)[: int(rng.integers(1, len(free) + 1))]]
+            lengths = [int(rng.integers(1, 41)) for _ in slots]
+            ids = torch.randint(0, 128, (len(slots), max(lengths)), generator=generator).cuda()
+            logits = runner.prefill_slots(ids, slots=slots, lengths=lengths, last_token_logits=True)
+            for row, (slot, length) in enumerate(zip(slots, lengths)):
+                live[slot] = [length, int(logits[row, 0].argmax())]
+        elif live and choice < 0.35:                         # a further chunk of a live slot's prompt
+            slot = int(rng.choice(sorted(live)))
+            length = int(rng.integers(1, 21))
+            if live[slot][0] + length < limit - 8:
+                ids = torch.randint(0, 128, (1, length), generator=generator).cuda()
+                logits = runner.prefill_slots(ids, slots=[slot], lengths=[length], last_token_logits=True)
+                live[slot] = [live[slot][0] + length, int(logits[0, 0].argmax())]
+        elif live and choice < 0.45:                         # a sequence ends
+            slot = int(rng.choice(sorted(live)))
+            runner.release_slots([slot])
+            del live[slot]
+            assert cache.manager.total_tokens(slot) == 0
+        elif live:                                           # decode steps of a subset, in any row order
+            slots = [int(s) for s in rng.permutation(sorted(live))[: int(rng.integers(1, len(live) + 1))]]
+            steps = int(rng.integers(1, 7))
+            if any(live[s][0] + steps >= limit - 1 for s in slots):
+                for s in slots:
+                    runner.release_slots([s])
+                    del live[s]
+                continue
+            tokens = torch.tensor([[live[s][1]] for s in slots], device="cuda")
+            positions = torch.tensor([[live[s][0]] for s in slots], device="cuda")
+            case = (event, slots, steps, {s: tuple(v) for s, v in live.items()})
+            if rng.random() < 0.3:                           # a burst on the device sampler against single steps
+                saved = snapshot()
+                chosen = runner.decode_greedy(tokens, slots=slots, positions=positions, steps=steps)
+                burst_state = [t.clone() for t in tensors]
+                restore(saved)
+                runner._decode_state = None
+            else:
+                chosen = None
+            for step in range(steps):
+                saved = snapshot()
+                by_graph = runner.decode(tokens, slots=slots, positions=positions).clone()
+                graph_state = [t.clone() for t in tensors]
+                restore(saved)
+                runner._decode_state = None
+                eager = runner.decode_eager(tokens, slots=slots, positions=positions)
+                assert torch.equal(by_graph, eager), ("logits", step, case)
+                for a, b in zip(graph_state, tensors):
+                    assert torch.equal(a, b), ("cache state", step, case)
+                tokens = eager[:, 0].argmax(-1).reshape(-1, 1)
+                positions = positions + 1
+                if chosen is not None:
+                    assert torch.equal(chosen[step], tokens[:, 0]), ("device sampler", step, case)
+                decoded += 1
+            if chosen is not None:
+                for a, b in zip(burst_state, tensors):
+                    assert torch.equal(a, b), ("cache state after the burst", case)
+            for row, s in enumerate(slots):
+                live[s] = [live[s][0] + steps, int(tokens[row, 0])]
+                assert cache.manager.total_tokens(s) == live[s][0], case
+    assert decoded >= 20
+    runner.release_slots(sorted(live))
