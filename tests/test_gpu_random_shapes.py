@@ -349,3 +349,41 @@ def test_runner_graph_equals_eager_under_slot_churn(tiny, sweep_seed):
                 assert cache.manager.total_tokens(s) == live[s][0], case
     assert decoded >= 20
     runner.release_slots(sorted(live))
+
+
+@pytest.mark.parametrize("sweep_seed", [13, 87])
+def test_fused_input_stages_over_random_shapes(rt, sweep_seed):
+    """Residual + RMSNorm and SwiGLU in front of the encoder, over every kernel form's row counts: the
+    residual stream exact, the staged rows within one BF16 step of the tensor operations (two where a
+    norm weight above one stretches the step), and the codes those of the plain encoder on the staged rows."""
+    import test_gpu_fused_step as stage_cases
+    rng = np.random.default_rng(sweep_seed)
+    table = torch.tensor(ACTIVATION_BETAS, dtype=torch.float32, device="cuda")
+    for _ in range(120):
+        rows = int(rng.choice([1, 2, 5, 8, 16, 17, 40, 100, 192, 193, 300, 512, 513, 700, 1100]))
+        n = int(rng.choice([256, 512, 1024, 2048, 4096, 8192]))
+        rows = min(rows, max(1, (1 << 22) // n))
+        mode = str(rng.choice(["rmsnorm", "rmsnorm+residual", "swiglu"]))
+        scale = float(rng.choice([0.05, 1.0, 30.0]))
+        case = (rows, n, mode, scale)
+        g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+        x = (scale * torch.randn(rows, n, generator=g)).to(torch.bfloat16).cuda()
+        if mode == "swiglu":
+            gate = (2 * torch.randn(rows, n, generator=g)).to(torch.bfloat16).cuda()
+            activation, _, staged = rt.fused_input_stage(x, mode="swiglu", gate=gate, beta_table=table, want_staged=True)
+            expect = torch.nn.functional.silu(gate) * x
+        else:
+            residual = (3 * scale * torch.randn(rows, n, generator=g)).to(torch.bfloat16).cuda() if "+" in mode else None
+            weight = (1 + 0.1 * torch.randn(n, generator=g)).to(torch.bfloat16).cuda()
+            activation, h, staged = rt.fused_input_stage(x, mode="rmsnorm", residual=residual, norm_weight=weight, eps=1e-5,
+                                                         beta_table=table, want_residual=True, want_staged=True)
+            expect_h = x if residual is None else x + residual
+            assert torch.equal(h, expect_h), case
+            expect = stage_cases._rms_norm(expect_h, weight, 1e-5)
+        difference = (staged.float() - expect.float()).abs()
+        assert bool((difference <= expect.float().abs() * 2.0 ** -6 + 1e-30).all()), case
+        # a mean summed in another order moves a row's scale by a unit in the last place now and then, and with
+        # it the rounding of a few of the row's values: counted loosely, bounded tightly above
+        assert int((staged != expect).sum()) <= max(16, rows * n // 50), case
+        plain = rt.quantize_activation_cuda(staged, q=Q, betas=ACTIVATION_BETAS, hadamard=True)
+        assert stage_cases._same_activation(activation, plain), case
