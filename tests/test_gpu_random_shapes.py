@@ -387,3 +387,50 @@ def test_fused_input_stages_over_random_shapes(rt, sweep_seed):
         assert int((staged != expect).sum()) <= max(16, rows * n // 50), case
         plain = rt.quantize_activation_cuda(staged, q=Q, betas=ACTIVATION_BETAS, hadamard=True)
         assert stage_cases._same_activation(activation, plain), case
+
+
+@pytest.mark.parametrize("sweep_seed", [17, 63])
+def test_dense_gemm_and_grouped_linears_over_random_shapes(rt, oracle, sweep_seed):
+    """The dense BF16 product on every tile and K split over ragged M and N, and the grouped prefill
+    linears (both routes) against one call per weight, bit for bit."""
+    from conftest import WEIGHT_BETAS
+    rng = np.random.default_rng(sweep_seed)
+    for _ in range(25):
+        m, n = int(rng.integers(1, 1200)), int(rng.integers(1, 700))
+        k = 128 * int(rng.integers(1, 17))
+        case = (m, n, k)
+        g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+        a = torch.randn(m, k, generator=g).to(torch.bfloat16).cuda()
+        b = torch.randn(n, k, generator=g).to(torch.bfloat16).cuda()
+        ref = bits(a.float() @ b.float().t())
+        for tile in [-1] + [int(t) for t in rng.permutation(10)[:4]]:
+            split = int(rng.choice([0, 1, 2, 4, 8]))
+            if split > 1 and k % (128 * split):
+                split = 0
+            c = rt.bf16_gemm(a, b, tile=tile, split_k=split)
+            assert relative_error(bits(c.float()), ref) <= 2.0 ** -8, (tile, split, case)
+    for _ in range(12):
+        k = int(rng.choice([256, 512, 1024, 2048]))
+        m = int(rng.choice([17, 40, 100, 128, 287, 288, 300, 600]))
+        count = int(rng.integers(2, 5 if m < 288 else 4))
+        unit = 32 if m < 288 else 256
+        sizes = [unit * int(rng.integers(1, 4)) for _ in range(count)]
+        case = (m, k, sizes)
+        weights = []
+        for i, n_out in enumerate(sizes):
+            g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+            w = torch.from_numpy(oracle.hadamard((0.02 * torch.randn(n_out, k, generator=g)).numpy()))
+            record = rt.quantize_weight_nqrt4(w.cuda(), q=Q, betas=WEIGHT_BETAS, dither_seed=int(rng.integers(1 << 31)),
+                                              tensor_name=f"w{i}")
+            weights.append(rt.prepare_fused_linear(record, device="cuda"))
+        x = student_t_rows(m, k, seed=int(rng.integers(1 << 20))).to(torch.bfloat16).cuda()
+        activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS, hadamard=True)
+        assert rt.can_use_w4a4_gemm_grouped(activation, weights), case
+        grouped = rt.linear_packed_w4a4_gemm_grouped(activation, weights)
+        split, tiles = 1, sum(sizes) // 32
+        while split < 16 and tiles * split < 256 and (k // (split * 2)) % 128 == 0:
+            split *= 2
+        for out, weight in zip(grouped, weights):
+            alone = (rt._gemm(activation, weight, output_dtype=torch.bfloat16, split_k=split) if m < 288
+                     else rt.linear_packed_w4a4_mma_chunked_staged(activation, weight))
+            assert torch.equal(out, alone), case
