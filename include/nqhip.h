@@ -128,6 +128,17 @@ int nq_rope_hadamard(const void *x_dev, int64_t rows, int heads, int head_dim, c
                      const void *rope_sin_dev, int hadamard, void *out_dev, void *stream);
 
 /*
+ * nq_rope_hadamard for the queries [rows, query_heads, head_dim] and the keys [rows, key_heads,
+ * head_dim] of the same rows in one launch (same tables, same arithmetic, each tensor to an output
+ * of its own): a prefill applies both right after the q/k/v product.
+ * Replaces: the two apply_rotary_pos_emb results and their rotations,
+ * nestquant/runtime/nqkv_batched_hf_backend.py:381, 549.
+ */
+int nq_rope_hadamard_pair(const void *query_dev, int query_heads, void *query_out_dev, const void *key_dev,
+                          int key_heads, void *key_out_dev, int64_t rows, int head_dim, const void *rope_cos_dev,
+                          const void *rope_sin_dev, int hadamard, void *stream);
+
+/*
  * Inverse of nq_quantize_rows: out[r, :] = (decode(codes) * beta[id]) * (norm[r] / sqrt(n)).
  * With has_dither != 0 the stateless dither lcg31_mix_v1 of global block
  * block_offset + r * n/8 + b and `seed` is regenerated and subtracted (NQRT4 weights).

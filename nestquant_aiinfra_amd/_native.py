@@ -37,6 +37,7 @@ SIGNATURES = {
                                 _ptr, _ptr, _ptr, _ptr, _ptr]),
     "nq_hadamard": (_i32, [_ptr, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr]),
     "nq_rope_hadamard": (_i32, [_ptr, _i64, _i32, _i32, _ptr, _ptr, _i32, _ptr, _ptr]),
+    "nq_rope_hadamard_pair": (_i32, [_ptr, _i32, _ptr, _ptr, _i32, _ptr, _i64, _i32, _ptr, _ptr, _i32, _ptr]),
     "nq_dequantize_rows": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i64, _i64,
                                   _ptr, _i32, _ptr]),
     "nq_fused_input_stage": (_i32, [_ptr, _i64, _i64, _i32, _ptr, _ptr, _ptr, _c.c_float, _ptr, _ptr, _i32, _ptr, _i32,

@@ -959,14 +959,21 @@ hadamard_rows_kernel(const T *__restrict__ x, int64_t rows, int n, int rows_per_
 // (prefill queries and keys): eight values per lane, D / 8 neighbouring lanes per vector, no
 // LDS.  The embedding is (x * cos) + (rotate_half(x) * sin) in BF16 tensor arithmetic (every
 // product and the sum rounded to BF16); the rotation runs float32 butterflies and rounds once.
+// A second tensor of the same rows with a head count of its own (the keys beside the queries) may
+// follow the first in the same launch: its chunks are numbered after the first tensor's.
 template <int D>
 __global__ void __launch_bounds__(256)
 rope_hadamard_kernel(const uint16_t *__restrict__ x, int64_t vectors, int heads,
+                     const uint16_t *__restrict__ x2, int64_t vectors2, int heads2,
                      const uint16_t *__restrict__ rope_cos, const uint16_t *__restrict__ rope_sin,
-                     int rotate, uint16_t *__restrict__ out) {
+                     int rotate, uint16_t *__restrict__ out, uint16_t *__restrict__ out2) {
     constexpr int kLanes = D / 8;
-    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;        // one 8-value chunk each
-    if (g >= vectors * kLanes) return;                                        // whole vectors leave together
+    int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;              // one 8-value chunk each
+    if (g >= (vectors + vectors2) * kLanes) return;                           // whole vectors leave together
+    if (g >= vectors * kLanes) {                                              // (a vector never straddles the two)
+        g -= vectors * kLanes;
+        x = x2; out = out2; heads = heads2;
+    }
     const int lane = threadIdx.x & 63, part = (int)(g % kLanes);
     float v[8];
     unpack_bf16x8(reinterpret_cast<const uint4 *>(x)[g], v);
@@ -1048,32 +1055,45 @@ extern "C" int nq_hadamard(const void *x_dev, int x_dtype, int64_t rows, int64_t
     return nq::check_launch("nq_hadamard");
 }
 
+namespace {
+
+int launch_rope_hadamard(const char *entry, const void *x, int heads, void *out, const void *x2, int heads2, void *out2,
+                         int64_t rows, int head_dim, const void *rope_cos, const void *rope_sin, int hadamard,
+                         hipStream_t s) {
+    NQ_REQUIRE(rows >= 1 && heads >= 1 && heads2 >= 0, NQ_ERR_SHAPE, "%s: rows and heads must be positive", entry);
+    NQ_REQUIRE(head_dim == 64 || head_dim == 128, NQ_ERR_SHAPE, "%s: head_dim %d is not 64 or 128", entry, head_dim);
+    NQ_REQUIRE(x && out && (heads2 == 0 || (x2 && out2)), NQ_ERR_ARGUMENT, "%s: null pointer", entry);
+    NQ_REQUIRE((rope_cos == nullptr) == (rope_sin == nullptr), NQ_ERR_ARGUMENT, "%s: rotary tables come as a pair", entry);
+    NQ_REQUIRE(nq::aligned(x, 16) && nq::aligned(out, 16) && nq::aligned(x2, 16) && nq::aligned(out2, 16) &&
+                   nq::aligned(rope_cos, 16) && nq::aligned(rope_sin, 16),
+               NQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", entry);
+    const int64_t vectors = rows * heads, vectors2 = rows * heads2, chunks = (vectors + vectors2) * (head_dim / 8);
+    const int64_t grid = (chunks + 255) / 256;
+    NQ_REQUIRE(grid <= 0x7fffffff, NQ_ERR_SHAPE, "%s: too many vectors", entry);
+    // the second tensor's chunks start at a multiple of the 8 or 16 lanes of a vector, so the lanes that
+    // exchange values still sit side by side in one wavefront
+    auto kernel = head_dim == 64 ? nq::rope_hadamard_kernel<64> : nq::rope_hadamard_kernel<128>;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, reinterpret_cast<const uint16_t *>(x), vectors, heads,
+                       reinterpret_cast<const uint16_t *>(x2), vectors2, heads2,
+                       reinterpret_cast<const uint16_t *>(rope_cos), reinterpret_cast<const uint16_t *>(rope_sin), hadamard,
+                       reinterpret_cast<uint16_t *>(out), reinterpret_cast<uint16_t *>(out2));
+    return nq::check_launch(entry);
+}
+
+}  // namespace
+
 extern "C" int nq_rope_hadamard(const void *x_dev, int64_t rows, int heads, int head_dim, const void *rope_cos_dev,
                                 const void *rope_sin_dev, int hadamard, void *out_dev, void *stream) {
-    NQ_REQUIRE(rows >= 1 && heads >= 1, NQ_ERR_SHAPE, "nq_rope_hadamard: rows and heads must be positive");
-    NQ_REQUIRE(head_dim == 64 || head_dim == 128, NQ_ERR_SHAPE, "nq_rope_hadamard: head_dim %d is not 64 or 128", head_dim);
-    NQ_REQUIRE(x_dev && out_dev, NQ_ERR_ARGUMENT, "nq_rope_hadamard: null pointer");
-    NQ_REQUIRE((rope_cos_dev == nullptr) == (rope_sin_dev == nullptr), NQ_ERR_ARGUMENT,
-               "nq_rope_hadamard: rotary tables come as a pair");
-    NQ_REQUIRE(nq::aligned(x_dev, 16) && nq::aligned(out_dev, 16) && nq::aligned(rope_cos_dev, 16) &&
-                   nq::aligned(rope_sin_dev, 16), NQ_ERR_ARGUMENT, "nq_rope_hadamard: pointers must be 16-byte aligned");
-    const int64_t vectors = rows * heads, chunks = vectors * (head_dim / 8);
-    const int64_t grid = (chunks + 255) / 256;
-    NQ_REQUIRE(grid <= 0x7fffffff, NQ_ERR_SHAPE, "nq_rope_hadamard: too many vectors");
-    hipStream_t s = (hipStream_t)stream;
-    if (head_dim == 64)
-        hipLaunchKernelGGL(nq::rope_hadamard_kernel<64>, dim3((unsigned)grid), dim3(256), 0, s,
-                           reinterpret_cast<const uint16_t *>(x_dev), vectors, heads,
-                           reinterpret_cast<const uint16_t *>(rope_cos_dev),
-                           reinterpret_cast<const uint16_t *>(rope_sin_dev), hadamard,
-                           reinterpret_cast<uint16_t *>(out_dev));
-    else
-        hipLaunchKernelGGL(nq::rope_hadamard_kernel<128>, dim3((unsigned)grid), dim3(256), 0, s,
-                           reinterpret_cast<const uint16_t *>(x_dev), vectors, heads,
-                           reinterpret_cast<const uint16_t *>(rope_cos_dev),
-                           reinterpret_cast<const uint16_t *>(rope_sin_dev), hadamard,
-                           reinterpret_cast<uint16_t *>(out_dev));
-    return nq::check_launch("nq_rope_hadamard");
+    return launch_rope_hadamard("nq_rope_hadamard", x_dev, heads, out_dev, nullptr, 0, nullptr, rows, head_dim,
+                                rope_cos_dev, rope_sin_dev, hadamard, (hipStream_t)stream);
+}
+
+extern "C" int nq_rope_hadamard_pair(const void *query_dev, int query_heads, void *query_out_dev, const void *key_dev,
+                                     int key_heads, void *key_out_dev, int64_t rows, int head_dim,
+                                     const void *rope_cos_dev, const void *rope_sin_dev, int hadamard, void *stream) {
+    NQ_REQUIRE(key_heads >= 1, NQ_ERR_SHAPE, "nq_rope_hadamard_pair: rows and heads must be positive");
+    return launch_rope_hadamard("nq_rope_hadamard_pair", query_dev, query_heads, query_out_dev, key_dev, key_heads,
+                                key_out_dev, rows, head_dim, rope_cos_dev, rope_sin_dev, hadamard, (hipStream_t)stream);
 }
 
 extern "C" int nq_e8_nearest(const float *x_dev, float *out_dev, int64_t count, void *stream) {

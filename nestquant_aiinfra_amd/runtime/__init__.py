@@ -11,6 +11,7 @@ _EXPORTS = {
     "quantize_rows_packed": "w4a4_linear",
     "hadamard_cuda": "w4a4_linear",
     "rope_hadamard_cuda": "w4a4_linear",
+    "rope_hadamard_pair_cuda": "w4a4_linear",
     "quantize_activation_cuda": "w4a4_linear",
     "fused_input_stage": "w4a4_linear",
     "quantize_weight_nqrt4": "w4a4_linear",

@@ -40,7 +40,7 @@ from .nqkv import attention_output_stage, launch_nqkv_decode_attention, nqkv_pre
 from .w4a4_linear import (BF16_ROWS_LINEAR_K, MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, _gemm, _gemv,
                           bf16_rows_linear, bf16_rows_linear_grouped, can_use_bf16_rows_linear, decode_weight_bf16,
                           can_use_w4a4_gemm_grouped, fused_input_stage, linear_packed_w4a4_gemm_grouped,
-                          linear_packed_w4a4_gemv_grouped, quantize_activation_cuda, rope_hadamard_cuda)
+                          linear_packed_w4a4_gemv_grouped, quantize_activation_cuda, rope_hadamard_pair_cuda)
 
 
 class UnsupportedForFusedDecode(ValueError):
@@ -273,8 +273,8 @@ class FusedLlamaPrefillStep(FusedLlamaDecodeStep):
                 delta, mode="rmsnorm", residual=residual, norm_weight=layer.input_layernorm.weight,
                 eps=layer.input_layernorm.variance_epsilon, beta_table=table, want_residual=True)
             query, key, value = self._linears(activation, [q_w, k_w, v_w])
-            query = rope_hadamard_cuda(query.view(count, heads, dim), rope=rope).view(rows, width, heads, dim)
-            key = rope_hadamard_cuda(key.view(count, kv_heads, dim), rope=rope).view(rows, width, kv_heads, dim)
+            query, key = rope_hadamard_pair_cuda(query.view(count, heads, dim), key.view(count, kv_heads, dim), rope=rope)
+            query, key = query.view(rows, width, heads, dim), key.view(rows, width, kv_heads, dim)
             value = value.view(rows, width, kv_heads, dim)
             manager.write_layer(index, key, value)
             scale = float(attention.scaling)

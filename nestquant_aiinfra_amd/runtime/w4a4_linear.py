@@ -149,6 +149,30 @@ def rope_hadamard_cuda(vectors: torch.Tensor, *, rope: tuple[torch.Tensor, torch
     return out
 
 
+def rope_hadamard_pair_cuda(query: torch.Tensor, key: torch.Tensor, *,
+                            rope: tuple[torch.Tensor, torch.Tensor] | None = None, hadamard: bool = True
+                            ) -> tuple[torch.Tensor, torch.Tensor]:
+    """`rope_hadamard_cuda` of the queries [rows, query_heads, head_dim] and the keys [rows, key_heads,
+    head_dim] of the same rows in one launch."""
+    device = _native.require_cuda(query, key)
+    for vectors in (query, key):
+        if vectors.dtype != torch.bfloat16 or vectors.ndim != 3 or not vectors.is_contiguous():
+            raise ValueError("expected contiguous BF16 tensors [rows, heads, head_dim]")
+    rows, heads, dim = query.shape
+    if key.shape[0] != rows or key.shape[2] != dim:
+        raise ValueError("queries and keys must agree on rows and head_dim")
+    if rope is not None:
+        for table in rope:
+            if table.dtype != torch.bfloat16 or tuple(table.shape) != (rows, dim) or not table.is_contiguous():
+                raise ValueError("rotary tables must be contiguous BF16 [rows, head_dim]")
+    query_out, key_out = torch.empty_like(query), torch.empty_like(key)
+    _native.check(_native.library().nq_rope_hadamard_pair(
+        query.data_ptr(), heads, query_out.data_ptr(), key.data_ptr(), key.shape[1], key_out.data_ptr(), rows, dim,
+        None if rope is None else rope[0].data_ptr(), None if rope is None else rope[1].data_ptr(), int(hadamard),
+        _native.stream_handle(device)))
+    return query_out, key_out
+
+
 def quantize_activation_cuda(inputs: torch.Tensor, *, q: int, betas: Sequence[float],
                              beta_table: torch.Tensor | None = None,
                              hadamard: bool = False) -> PreparedNQA4Activation:

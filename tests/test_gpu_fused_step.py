@@ -219,6 +219,14 @@ def test_rope_and_rotation_of_head_vectors_in_one_launch(rt, heads, dim):
     assert torch.equal(rt.rope_hadamard_cuda(x, rope=(cos, sin), hadamard=False), embedded)
     assert torch.equal(rt.rope_hadamard_cuda(x, hadamard=True), hadamard(x.float()).to(torch.bfloat16))
     assert torch.equal(rt.rope_hadamard_cuda(x, rope=(cos, sin)), hadamard(embedded.float()).to(torch.bfloat16))
+    # queries and keys of the same rows in one launch: each as its own launch gives it
+    keys = torch.randn(rows, max(1, heads // 4), dim, generator=g).to(torch.bfloat16).cuda()
+    for tables, rotate in (((cos, sin), True), (None, True), ((cos, sin), False)):
+        q_out, k_out = rt.rope_hadamard_pair_cuda(x, keys, rope=tables, hadamard=rotate)
+        assert torch.equal(q_out, rt.rope_hadamard_cuda(x, rope=tables, hadamard=rotate))
+        assert torch.equal(k_out, rt.rope_hadamard_cuda(keys, rope=tables, hadamard=rotate))
+    with pytest.raises(ValueError):
+        rt.rope_hadamard_pair_cuda(x, keys[:5].contiguous(), rope=(cos, sin))
     with pytest.raises(ValueError):
         rt.rope_hadamard_cuda(x, rope=(cos[:5], sin[:5]))
     with pytest.raises(ValueError):
