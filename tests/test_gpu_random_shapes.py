@@ -434,3 +434,42 @@ def test_dense_gemm_and_grouped_linears_over_random_shapes(rt, oracle, sweep_see
             alone = (rt._gemm(activation, weight, output_dtype=torch.bfloat16, split_k=split) if m < 288
                      else rt.linear_packed_w4a4_mma_chunked_staged(activation, weight))
             assert torch.equal(out, alone), case
+
+
+@pytest.mark.parametrize("sweep_seed", [19, 71])
+def test_greedy_sampler_over_random_logits(sweep_seed):
+    """The device sampler against torch.argmax over random row counts, vocabulary sizes (odd ones
+    take the element loop), dtypes, strided rows, repeated maxima, infinities and NaN (the first NaN
+    of a row wins, as in torch.argmax)."""
+    from nestquant_aiinfra_amd.runtime.nqkv_hf_backend import greedy_sample_
+    rng = np.random.default_rng(sweep_seed)
+    g = torch.Generator().manual_seed(sweep_seed)
+    for _ in range(60):
+        rows = int(rng.integers(1, 33))
+        vocab = int(rng.choice([1, 5, 8, 777, 1000, 4096, 32000, 70001, 128256]))
+        stride = vocab + int(rng.choice([0, 0, 8, 13]))
+        dtype = [torch.bfloat16, torch.float32, torch.float16][rng.integers(3)]
+        case = (rows, vocab, stride, dtype)
+        storage = torch.randn((rows, stride), generator=g).to(dtype)
+        for row in range(rows):
+            kind = rng.integers(5)
+            if kind == 0:
+                storage[row, :vocab] = storage[row, :vocab].round()             # many equal maxima
+            elif kind == 1:
+                storage[row, int(rng.integers(vocab))] = float("inf")
+                storage[row, int(rng.integers(vocab))] = float("inf")
+            elif kind == 2:
+                storage[row, int(rng.integers(vocab))] = float("nan")
+                storage[row, int(rng.integers(vocab))] = float("nan")
+            elif kind == 3:
+                storage[row, :vocab] = float("-inf")                            # nothing to prefer: index 0
+        storage[:, vocab:] = 1e4                                                # beyond the vocabulary: never chosen
+        logits = storage.cuda()[:, :vocab]
+        values = logits.float().cpu()
+        want = values.argmax(-1)
+        for row in range(rows):                                                 # NaN is the largest, the first one wins
+            nans = torch.isnan(values[row]).nonzero()
+            if len(nans):
+                want[row] = int(nans[0])
+        plain = torch.zeros(rows, dtype=torch.long, device="cuda")
+        assert torch.equal(greedy_sample_(logits, plain).cpu(), want), case
