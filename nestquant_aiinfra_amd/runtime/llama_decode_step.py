@@ -36,7 +36,7 @@ import torch
 
 import torch.nn.functional as F
 
-from .nqkv import attention_output_stage, launch_nqkv_decode_attention, nqkv_prefill_attention
+from .nqkv import attention_output_stage, nqkv_prefill_attention
 from .w4a4_linear import (BF16_ROWS_LINEAR_K, MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, _gemm, _gemv,
                           bf16_rows_linear, bf16_rows_linear_grouped, can_use_bf16_rows_linear, decode_weight_bf16,
                           can_use_w4a4_gemm_grouped, fused_input_stage, linear_packed_w4a4_gemm_grouped,
