@@ -563,10 +563,56 @@ def attention_extra(device):
                                  "longest_row_alone_us_without_context_split": one[False] * 1e6}}
 
 
-def tpot_extra(device, batches=(1, 8), prompt=128, generate=128):
+def engine_tpot(model, capacity, prompt, generate, vocab, generator):
+    """The continuous-batching engine at `capacity` slots over `capacity` requests of `prompt` random
+    ids and `generate` new tokens each: per-request inter-token wall time, the clock read after a
+    device synchronisation at the end of every engine step, so that host scheduling, the graph replay
+    and the host argmax are all inside it (the reference's engine harness,
+    scripts/benchmark_service_workloads.py:148-151, 215-220)."""
+    import torch
+    from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
+    from nestquant_aiinfra_amd.runtime import AdmissionPolicy, ContinuousBatchInferenceEngine, DecodeRequest
+
+    runner = asm.attach_w4a4kv4_cache(model, capacity=capacity, max_cache_len=prompt + generate)
+    out = {}
+    for name, burst in (("host_sampler", 1), ("device_sampler_burst16", 16)):
+        engine = ContinuousBatchInferenceEngine(runner, decode_burst=burst,
+                                                admission_policy=AdmissionPolicy(min_prefill_batch=1, max_wait_steps=0))
+        engine.initialize()
+        requests = [DecodeRequest(f"r{i}", tuple(torch.randint(0, vocab, (prompt,), generator=generator).tolist()), generate)
+                    for i in range(capacity)]
+        for request in requests:
+            engine.submit(request)
+        token_times = {request.request_id: [] for request in requests}
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        while engine.has_work():
+            engine.step()
+            torch.cuda.synchronize()
+            now = time.perf_counter()
+            for request in requests:
+                times = token_times[request.request_id]
+                fresh = len(request.generated_token_ids) - len(times)
+                if fresh and not times:
+                    times.append(now)
+                    fresh -= 1
+                if fresh:
+                    # the tokens a burst hands over at once are spread evenly over the time since the one before
+                    previous = times[-1]
+                    times.extend(previous + (now - previous) * (i + 1) / fresh for i in range(fresh))
+        wall = time.perf_counter() - started
+        gaps = sorted((times[i] - times[i - 1]) * 1e3 for times in token_times.values() for i in range(1, len(times)))
+        out[name] = {"tpot_ms_p50": gaps[len(gaps) // 2], "tpot_ms_p95": gaps[int(0.95 * len(gaps))],
+                     "tpot_ms_mean": sum(gaps) / len(gaps), "ttft_ms": 1e3 * (min(t[0] for t in token_times.values()) - started),
+                     "tokens_per_s": sum(len(t) for t in token_times.values()) / wall}
+    return out
+
+
+def tpot_extra(device, batches=(1, 2, 4, 8), prompt=128, generate=128):
     """Random-init Llama-3.2-1B architecture, all 112 projections W4A4, KV4 cache, captured decode
     step.  Per batch size: mean decode-step wall time (host argmax included), the wall time per
-    step when the sampler runs inside the graph (one host read per 64 steps) and GPU graph time."""
+    step when the sampler runs inside the graph (one host read per 64 steps), GPU graph time, and
+    the engine's per-request TPOT at that capacity (`engine`)."""
     import tempfile
 
     import torch
@@ -669,6 +715,9 @@ def tpot_extra(device, batches=(1, 8), prompt=128, generate=128):
             greedy_s = (time.perf_counter() - t0) / greedy_steps
             runner.release_slots(slots)
             results[f"batch{batch}"]["tpot_ms_device_sampler_expanded_weights"] = greedy_s * 1e3
+        runner.fused_step.expand_weights = False
+        for batch in batches:
+            results[f"batch{batch}"]["engine"] = engine_tpot(model, batch, prompt, generate, config.vocab_size, g)
         results["expanded_weight_bytes"] = sum(
             sum(t.numel() * 2 for t in entry if isinstance(t, torch.Tensor))
             for entry in runner.fused_step._expanded.values() if entry is not None)

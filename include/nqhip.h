@@ -221,14 +221,17 @@ size_t nq_w4a4_gemv_workspace_bytes(int m, int k, int n, int split_k, int have_d
  * process ends), so the call allocates nothing and asks for nothing that was allocated for it.
  * Same arguments, kernels and results (bit for bit) as nq_w4a4_gemv; shapes whose workspace
  * (nq_w4a4_gemv_workspace_bytes) exceeds the buffer are rejected with NQ_ERR_WORKSPACE.  The
- * first call on a device looks up the buffer's address (hipGetSymbolAddress) and should
- * therefore happen outside a graph capture.  All calls on one GPU share the buffer: calls that
+ * first use on a device looks up the buffer's address (hipGetSymbolAddress), which a stream
+ * under capture must not see: nq_w4a4_gemv_static_init() does that lookup for the current
+ * device ahead of time, and a first call made inside a capture without it is rejected with
+ * NQ_ERR_ARGUMENT instead of being recorded.  All calls on one GPU share the buffer: calls that
  * may overlap there (different streams, different threads) race and must be serialised by the
  * caller.  Nothing in the buffer needs clearing between calls.
  * No counterpart in the reference (its extension allocates partials with torch::empty on every
  * call, nestquant/runtime/nqrt4_w4a4_mma.cu:1213-1214); it is for callers that cannot allocate
  * device memory: code under HIP graph capture, tight serving loops, harnesses that forbid it.
  */
+int nq_w4a4_gemv_static_init(void);
 int nq_w4a4_gemv_static(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
                         const float *act_norms_dev, const float *act_betas_dev,
                         const void *act_decoded_dev, const uint8_t *w_codes_dev,
@@ -423,7 +426,10 @@ int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_dtype, cons
  * query_dtype), matching keys stored with rotate_keys.  out_dev may be NULL: then only the first
  * stage runs (see nq_attention_output_stage).  rope_cos_dev / rope_sin_dev (optional,
  * both or neither): BF16 [batch, head_dim] rotary tables applied to the (BF16) query before
- * that, as nq_nqkv_write applies them to keys.  Workspace: at least
+ * that, as nq_nqkv_write applies them to keys.  Alignment: a BF16 query 16 bytes (its rows are
+ * read eight values at a time; a sliced view must be made contiguous first), float32 4, float16
+ * and the rotary rows 2, hot tails 16, page streams 4; anything else returns NQ_ERR_ARGUMENT.
+ * Workspace: at least
  * nq_nqkv_attention_workspace_bytes() bytes.  Requires head_dim = 64, page_size = 16,
  * q = 14, q_heads / kv_heads in {1, 2, 4, 8}; any max_pages.
  * Replaces: nqkv_decode_attention_batched_k1 and its three Triton kernels

@@ -48,6 +48,7 @@ SIGNATURES = {
     "nq_w4a4_gemv": (_i32, [_ptr] * 11 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
                                           _size, _ptr]),
     "nq_w4a4_gemv_workspace_bytes": (_size, [_i32, _i32, _i32, _i32, _i32]),
+    "nq_w4a4_gemv_static_init": (_i32, []),
     "nq_w4a4_gemv_static": (_i32, [_ptr] * 11 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr]),
     "nq_w4a4_gemm": (_i32, [_ptr] * 11 + [_i32, _i32, _i32, _i64, _i64, _i32, _ptr, _i32, _ptr,
                                           _size, _ptr]),

@@ -680,6 +680,12 @@ int launch_decode_attention(
     NQ_REQUIRE(nq::aligned(key_codes_dev, 4) && nq::aligned(value_codes_dev, 4) && nq::aligned(hot_keys_dev, 16) &&
                    nq::aligned(hot_values_dev, 16),
                NQ_ERR_ARGUMENT, "%s: page streams need 4-byte, hot tails 16-byte alignment", entry);
+    // a BF16 query row is read eight values (16 bytes) at a time; the other element types and the
+    // BF16 rotary rows one value at a time
+    NQ_REQUIRE(nq::aligned(query_dev, query_dtype == NQ_BF16 ? 16 : (query_dtype == NQ_F32 ? 4 : 2)), NQ_ERR_ARGUMENT,
+               "%s: a BF16 query needs 16-byte alignment (float32 4, float16 2)", entry);
+    NQ_REQUIRE(nq::aligned(rope_cos_dev, 2) && nq::aligned(rope_sin_dev, 2), NQ_ERR_ARGUMENT,
+               "%s: rotary rows need 2-byte alignment", entry);
     NQ_REQUIRE(isfinite(scale), NQ_ERR_ARGUMENT, "%s: scale must be finite", entry);
     NQ_REQUIRE(chunks_for(batch, max_pages) + 1 <= 512, NQ_ERR_SHAPE,
                "%s: a page table of %d pages needs more than 512 context chunks", entry, max_pages);

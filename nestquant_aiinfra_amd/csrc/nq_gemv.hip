@@ -397,15 +397,18 @@ bool takes_mfma_gemv(int m, int k, int64_t total_n, bool resolved) {
 
 int launch_mfma_gemv(const void *act, const nq::GemvWeights &w, int ranges, int groups, int m, int k,
                      int out_is_f32, hipStream_t stream) {
-    const int super_steps = k / (128 * ranges);
-    // two or more super-steps per wavefront, so that the requests of the next one hide behind a decode;
-    // four on a long K in two ranges (down_proj at 8 rows: 12.1 us with two, 11.8 to 11.9 with four, 13.2
-    // with eight).  Either way a K that runs in one range with w wavefronts runs in two ranges with w / 2,
-    // so the same 128-wide pieces of K meet in the same accumulators and are added in the same order:
-    // a weight gives the same bits alone (two ranges) and inside a group (one range).
-    const int per_wave = ranges == 2 && super_steps >= 32 ? 4 : 2;
-    int waves = super_steps / per_wave < nq::kMfmaGemvMaxWaves ? super_steps / per_wave : nq::kMfmaGemvMaxWaves;
-    if (waves < 4) waves = 4;                    // the last stage wants 256 lanes
+    // One range: two or more super-steps of 128 k per wavefront, so that the requests of the next one
+    // hide behind a decode; between 4 wavefronts (the last stage wants 256 lanes) and 16.  Two ranges:
+    // exactly half as many wavefronts as the same K takes in one range (the last stage wants 128
+    // lanes).  Wavefront v of the two-range launch then gathers, in its accumulator r, the pieces of
+    // 128 k that wavefront 2 v + r of the one-range launch gathers, in the same order, and the last
+    // stage adds the accumulators in that same wavefront order: a weight gives the same bits alone
+    // (two ranges) and inside a group (one range), for every K.  (down_proj at 8 rows, two ranges:
+    // 12.1 us with 16 wavefronts, 11.8 to 11.9 with 8, 13.2 with 4.)
+    const int pieces = k / 128;
+    int waves = pieces / 2 < nq::kMfmaGemvMaxWaves ? pieces / 2 : nq::kMfmaGemvMaxWaves;
+    if (waves < 4) waves = 4;
+    if (ranges == 2) waves /= 2;
     const uint4 *a = reinterpret_cast<const uint4 *>(act);
     const float sqrt_k = (float)sqrt((double)k);
     const dim3 grid((unsigned)groups), block(64 * waves);
@@ -619,8 +622,10 @@ constexpr int kStaticScratchMaxDevices = 64;
 // host code the name is only a handle for hipGetSymbolAddress: it is never passed to a kernel.
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
-// Device address of `scratch` on the current device, looked up once per device.
-int static_scratch_address(void **address) {
+// Device address of `scratch` on the current device, looked up once per device.  The lookup is a
+// runtime call that a stream under capture must not see: while `stream` is capturing only an
+// address that is already known is handed out (nq_w4a4_gemv_static_init makes it known).
+int static_scratch_address(void **address, hipStream_t stream, bool may_be_capturing) {
     static void *known[kStaticScratchMaxDevices] = {nullptr};
     int device = -1;
     hipError_t status = hipGetDevice(&device);
@@ -630,6 +635,15 @@ int static_scratch_address(void **address) {
                "nq_w4a4_gemv_static: device ordinal %d is outside [0, %d)", device, kStaticScratchMaxDevices);
     void *pointer = __atomic_load_n(&known[device], __ATOMIC_ACQUIRE);
     if (!pointer) {
+        if (may_be_capturing) {
+            hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+            status = hipStreamIsCapturing(stream, &capture);
+            if (status != hipSuccess)
+                return nq::fail(NQ_ERR_LAUNCH, "nq_w4a4_gemv_static: hipStreamIsCapturing: %s", hipGetErrorString(status));
+            NQ_REQUIRE(capture == hipStreamCaptureStatusNone, NQ_ERR_ARGUMENT,
+                       "nq_w4a4_gemv_static: first use on device %d inside a stream capture; call "
+                       "nq_w4a4_gemv_static_init() on this device before capturing", device);
+        }
         status = hipGetSymbolAddress(&pointer, HIP_SYMBOL(scratch));
         if (status != hipSuccess || !pointer)
             return nq::fail(NQ_ERR_LAUNCH, "nq_w4a4_gemv_static: hipGetSymbolAddress(scratch): %s",
@@ -641,6 +655,11 @@ int static_scratch_address(void **address) {
 }
 
 }  // namespace
+
+extern "C" int nq_w4a4_gemv_static_init(void) {
+    void *address = nullptr;
+    return static_scratch_address(&address, nullptr, false);
+}
 
 extern "C" int nq_w4a4_gemv_static(const uint8_t *act_codes_dev, const uint8_t *act_beta_ids_dev,
                                    const float *act_norms_dev, const float *act_betas_dev,
@@ -660,7 +679,7 @@ extern "C" int nq_w4a4_gemv_static(const uint8_t *act_codes_dev, const uint8_t *
                "built-in buffer holds %zu (use nq_w4a4_gemv with a caller-owned workspace)",
                m, k, n, split_k, need, kStaticScratchBytes);
     void *workspace = nullptr;
-    const int status = static_scratch_address(&workspace);
+    const int status = static_scratch_address(&workspace, (hipStream_t)stream, true);
     if (status != NQ_OK) return status;
     // Every partial sum and every decoded activation value a launch reads was written by that
     // same launch sequence, so what an earlier call left in the buffer needs no clearing.

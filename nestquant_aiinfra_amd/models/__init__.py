@@ -13,6 +13,7 @@ _EXPORTS = {
     "projection_names": "llama_w4a4kv4",
     "write_w4_checkpoint": "llama_w4a4kv4",
     "build_w4a4kv4_runner": "llama_w4a4kv4",
+    "attach_w4a4kv4_cache": "llama_w4a4kv4",
 }
 
 __all__ = sorted(_EXPORTS)

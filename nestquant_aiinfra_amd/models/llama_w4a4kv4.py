@@ -71,6 +71,19 @@ def build_w4a4kv4_runner(model: nn.Module, checkpoint: str | Path, *, capacity: 
     convert_linears_to_fused_nqrt_(model, reader, names, compute_backend="packed_w4a4_cuda_mma", activation_q=14,
                                    activation_betas=tuple(activation_betas),
                                    enable_m1_down_splitk=enable_m1_down_splitk)
+    return attach_w4a4kv4_cache(model, capacity=capacity, max_cache_len=max_cache_len, page_size=page_size,
+                                key_betas=key_betas, value_betas=value_betas, fused_decode=fused_decode,
+                                fused_prefill=fused_prefill, packed_prefill=packed_prefill,
+                                expand_weights=expand_weights)
+
+
+def attach_w4a4kv4_cache(model: nn.Module, *, capacity: int, max_cache_len: int, page_size: int = 16,
+                         key_betas: Sequence[float] = KEY_BETAS, value_betas: Sequence[float] = VALUE_BETAS,
+                         fused_decode: bool | None = None, fused_prefill: bool | None = None,
+                         packed_prefill: bool = False, expand_weights: bool = False) -> BatchedNQKVLlamaRunner:
+    """A batched NQKV4 cache of `capacity` slots and its runner over a model whose projections are
+    already packed modules (an engine of another capacity over the same weights: the packed weights
+    are shared, the attention modules point at the newest cache)."""
     config = model.config
     head_dim = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
     device = next(model.parameters()).device

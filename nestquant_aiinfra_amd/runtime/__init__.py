@@ -61,6 +61,11 @@ _EXPORTS = {
     "BatchedNQKVCacheManager": "nqkv",
     "append_hot_k1_graph_safe": "nqkv",
     "launch_pack_full_hot_pages_graph_safe": "nqkv",
+    "PagedNQKVCache": "nqkv_single",
+    "NQKVAttentionWorkspace": "nqkv_single",
+    "nqkv_decode_attention_k1": "nqkv_single",
+    "NQKVLlamaCache": "nqkv_single",
+    "install_nqkv_llama_backend": "nqkv_single",
     "cuda_e8_available": "cuda_e8",
     "e8_nearest_cuda": "cuda_e8",
     "bf16_gemm": "w4a4_linear",

@@ -273,6 +273,12 @@ class NQKVPagePool:
             slot.copy_(stream)
         self._pages[page_id].valid_tokens = page.valid_tokens
 
+    def store(self, handle: NQKVPageHandle, page) -> None:
+        """Copy a host container (core.kv_format.PackedNQKVPage) into the page's physical slot."""
+        if not hasattr(page, "to_prepared"):
+            raise TypeError("page must be a PackedNQKVPage")
+        self.store_prepared(handle, page.to_prepared(self.device))
+
     def mark_graph_stored(self, handle: NQKVPageHandle, *, valid_tokens: int) -> None:
         """Record that a kernel (not store_prepared) has filled the page."""
         page_id = self._owned_page(handle)
@@ -336,19 +342,143 @@ class BatchedNQKVMetadata:
 
 class NQKVHotColdCache:
     """One layer's cache: packed cold pages in a pool, a BF16 hot tail per slot, and the
-    (possibly shared) device tables that say how much of each is valid."""
+    (possibly shared) device tables that say how much of each is valid.
 
-    def __init__(self, pool: NQKVPagePool, metadata: BatchedNQKVMetadata, *, max_sequences: int,
-                 max_pages_per_sequence: int) -> None:
+    Two ways to build one.  `NQKVHotColdCache(pool, metadata, max_sequences=, max_pages_per_sequence=)`
+    is the flat form the batched manager uses: slots own fixed pages and the tables are shared between
+    layers.  `NQKVHotColdCache(cold_cache)` over a PagedNQKVCache is the reference's form
+    (nestquant/runtime/nqkv_hot_cache.py:14-37): sequences are registered by id, `append` takes pages
+    from the pool as tails fill, and `hot_view` / `materialize` / `total_tokens` read one sequence."""
+
+    def __init__(self, pool, metadata: BatchedNQKVMetadata | None = None, *, max_sequences: int | None = None,
+                 max_pages_per_sequence: int | None = None) -> None:
+        self._logical = None
+        if not isinstance(pool, NQKVPagePool):
+            logical = pool
+            if not all(hasattr(logical, name) for name in ("pool", "metadata", "reserve_page", "commit_graph_page")):
+                raise TypeError("cold_cache must be a PagedNQKVCache")
+            if metadata is not None or max_sequences is not None or max_pages_per_sequence is not None:
+                raise ValueError("a cache over a PagedNQKVCache takes its tables and sizes from it")
+            self._logical = logical
+            pool, metadata = logical.pool, logical.metadata
+            max_sequences, max_pages_per_sequence = logical.max_sequences, logical.max_pages_per_sequence
+        elif metadata is None or max_sequences is None or max_pages_per_sequence is None:
+            raise ValueError("the flat form needs metadata, max_sequences and max_pages_per_sequence")
         self.pool, self.metadata = pool, metadata
         self.max_sequences, self.max_pages_per_sequence = max_sequences, max_pages_per_sequence
         shape = (max_sequences, pool.page_size, pool.num_kv_heads, pool.head_dim)
         self.hot_keys = torch.zeros(shape, device=pool.device, dtype=torch.bfloat16)
         self.hot_values = torch.zeros_like(self.hot_keys)
+        self.hot_lengths = metadata.hot_lengths
+        self._hot_tokens = [0] * max_sequences          # host mirror of the tails (sequence form only)
 
     @property
-    def cold_cache(self) -> "NQKVHotColdCache":      # the reference nests a cold cache; flat here
-        return self
+    def cold_cache(self):
+        """The PagedNQKVCache underneath, or the cache itself in the flat form."""
+        return self if self._logical is None else self._logical
+
+    # -- one sequence at a time (over a PagedNQKVCache) --------------------------------------------
+    def _sequences(self):
+        if self._logical is None:
+            raise RuntimeError("this cache is driven by slot through its manager: it holds no sequence ids")
+        return self._logical
+
+    def register(self, sequence_id: Hashable, *, slot: int | None = None) -> int:
+        slot = self._sequences().register(sequence_id, slot=slot)
+        self._hot_tokens[slot] = 0
+        return slot
+
+    def release(self, sequence_id: Hashable) -> None:
+        logical = self._sequences()
+        slot = logical.slot(sequence_id)
+        logical.release(sequence_id)
+        self._hot_tokens[slot] = 0
+
+    def hot_length(self, slot: int) -> int:
+        self._sequences().sequence_id(slot)
+        return self._hot_tokens[slot]
+
+    def total_tokens(self, sequence_id: Hashable) -> int:
+        logical = self._sequences()
+        return logical.total_tokens(sequence_id) + self._hot_tokens[logical.slot(sequence_id)]
+
+    def hot_view(self, sequence_id: Hashable) -> tuple[torch.Tensor, torch.Tensor]:
+        slot = self._sequences().slot(sequence_id)
+        held = self._hot_tokens[slot]
+        return self.hot_keys[slot, :held], self.hot_values[slot, :held]
+
+    def append(self, sequence_id: Hashable, key: torch.Tensor, value: torch.Tensor) -> None:
+        """Append key / value BF16 [tokens, kv_heads, head_dim] (keys already rotated) to one sequence.
+        The pages this append completes are reserved from the pool and mapped into the sequence's page
+        table first; the writer kernel then fills the tail and encodes those pages in one launch."""
+        logical = self._sequences()
+        slot = logical.slot(sequence_id)
+        pool = self.pool
+        if (not isinstance(key, torch.Tensor) or key.ndim != 3 or key.shape != value.shape
+                or tuple(key.shape[1:]) != (pool.num_kv_heads, pool.head_dim)):
+            raise ValueError("key and value must share shape [tokens, kv_heads, head_dim]")
+        if key.dtype != torch.bfloat16 or value.dtype != torch.bfloat16 or key.device != pool.device:
+            raise ValueError("key and value must be BF16 on the cache device")
+        tokens = key.shape[0]
+        if tokens < 1:
+            return
+        held = self._hot_tokens[slot]
+        if logical.total_tokens(sequence_id) != len(logical.handles(sequence_id)) * pool.page_size:
+            raise RuntimeError("a sequence whose newest page is partial takes whole pages only")
+        if logical.total_tokens(sequence_id) + held + tokens > self.max_pages_per_sequence * pool.page_size:
+            raise RuntimeError("sequence exceeds max_pages_per_sequence")
+        completes = (held + tokens) // pool.page_size
+        first_ordinal = len(logical.handles(sequence_id))
+        handles = []
+        try:
+            for _ in range(completes):
+                handles.append(logical.reserve_page(sequence_id))
+        except Exception:
+            for handle in handles:
+                logical.cancel_reserved_page(sequence_id, handle)
+            raise
+        meta = self.metadata
+        if handles:
+            meta.page_indices[slot, first_ordinal:first_ordinal + completes] = torch.tensor(
+                [handle.page_id for handle in handles], dtype=torch.int32, device=pool.device)
+        slot_ids = torch.tensor([slot], dtype=torch.int32, device=pool.device)
+        active = torch.ones(1, dtype=torch.bool, device=pool.device)
+        lib, stream = _native.library(), _native.stream_handle(pool.device)
+        _native.check(lib.nq_nqkv_advance(
+            slot_ids.data_ptr(), active.data_ptr(), None, tokens, 1, self.max_sequences, pool.page_size,
+            self.max_pages_per_sequence * pool.page_size, meta.sequence_lengths.data_ptr(), meta.page_counts.data_ptr(),
+            meta.last_page_lens.data_ptr(), meta.hot_lengths.data_ptr(), stream))
+        key, value = key.contiguous(), value.contiguous()
+        _native.check(lib.nq_nqkv_write(
+            key.data_ptr(), value.data_ptr(), _native.dtype_tag(key.dtype), slot_ids.data_ptr(), active.data_ptr(),
+            None, tokens, meta.sequence_lengths.data_ptr(), meta.page_indices.data_ptr(),
+            pool.key_codes.data_ptr(), pool.key_betas.data_ptr(), pool.key_norms.data_ptr(),
+            pool.value_codes.data_ptr(), pool.value_betas.data_ptr(), pool.value_norms.data_ptr(),
+            pool.beta_table.data_ptr(), pool.beta_table.numel(), pool.value_beta_table.data_ptr(),
+            pool.value_beta_table.numel(), self.hot_keys.data_ptr(), self.hot_values.data_ptr(),
+            1, tokens, self.max_sequences, self.max_pages_per_sequence, pool.num_kv_heads, pool.head_dim,
+            pool.page_size, 0, None, None, stream))
+        for handle in handles:
+            logical.commit_graph_page(sequence_id, handle)
+        self._hot_tokens[slot] = (held + tokens) % pool.page_size
+
+    def materialize(self, sequence_id: Hashable) -> tuple[torch.Tensor, torch.Tensor]:
+        """The sequence as BF16 [tokens, kv_heads, head_dim]: its packed pages decoded, then the tail."""
+        logical = self._sequences()
+        keys, values = [], []
+        for handle in logical.handles(sequence_id):
+            key, value = dequantize_nqkv_page(self.pool.prepared(handle))
+            keys.append(key)
+            values.append(value)
+        hot_key, hot_value = self.hot_view(sequence_id)
+        if hot_key.shape[0]:
+            keys.append(hot_key)
+            values.append(hot_value)
+        if not keys:
+            empty = torch.empty((0, self.pool.num_kv_heads, self.pool.head_dim), device=self.pool.device,
+                                dtype=self.pool.output_dtype)
+            return empty, empty.clone()
+        return torch.cat(keys), torch.cat(values)
 
 
 @dataclass
@@ -385,6 +515,10 @@ def launch_nqkv_decode_attention(query: torch.Tensor, cache: NQKVHotColdCache, *
     attention_output_stage (returns None)."""
     pool, meta = cache.pool, cache.metadata
     batch, heads, dim = query.shape
+    if not query.is_contiguous() or query.data_ptr() % 16:
+        raise ValueError("query must be contiguous and 16-byte aligned (call .contiguous() on a sliced view)")
+    if rope is not None and any(not t.is_contiguous() or t.dtype != torch.bfloat16 for t in rope):
+        raise ValueError("rope must be a pair of contiguous BF16 tables")
     _native.check(_native.library().nq_nqkv_attention_decode(
         query.data_ptr(), _native.dtype_tag(query.dtype),
         pool.key_codes.data_ptr(), pool.key_betas.data_ptr(), pool.key_norms.data_ptr(),

@@ -477,6 +477,10 @@ class BatchedNQKVLlamaRunner:
                 if count and not bool(row[:count].all()):
                     raise ValueError("write_mask rows must be prefixes: written tokens lead each row")
             live = [slot for slot, count in enumerate(counts) if count]
+            held = valid_lengths.detach().cpu().tolist()
+            for slot in live:
+                if held[slot] != self.cache._host_lengths[slot] + counts[slot]:
+                    raise ValueError("valid_lengths of a writing row must equal the tokens it held plus those it writes")
             full = None
             if live:
                 index = torch.tensor(live, dtype=torch.long, device=self.device)
@@ -504,10 +508,6 @@ class BatchedNQKVLlamaRunner:
         for slot, length in zip(slots, lengths):
             if self.cache._host_lengths[slot] + length > self.max_cache_len:
                 raise RuntimeError("sequence would exceed max_cache_len")
-        fresh = [slot for slot in slots if self.cache.manager.sequence_id(slot) is None]
-        for slot in fresh:
-            self._generation[slot] += 1
-        self.cache.register_batch([(f"slot-{slot}-generation-{self._generation[slot]}", slot) for slot in fresh])
         if positions is None:
             starts = torch.tensor([self.cache._host_lengths[s] for s in slots], device=self.device)
             positions = starts[:, None] + torch.arange(width, device=self.device)[None, :]
@@ -519,6 +519,16 @@ class BatchedNQKVLlamaRunner:
                 inside = positions[written]
                 if int(inside.min().item()) < 0 or int(inside.max().item()) >= self.max_cache_len:
                     raise ValueError("written positions must lie in [0, max_cache_len)")
+                # tokens are appended at the cache's own length while RoPE turns them by `positions`: the
+                # two must name the same place, or keys would be stored at one position and rotated for another
+                starts = torch.tensor([self.cache._host_lengths[s] for s in slots], device=self.device)
+                expected = starts[:, None] + torch.arange(width, device=self.device)[None, :]
+                if bool(((positions != expected) & written).any().item()):
+                    raise ValueError("written positions must continue each slot's sequence: tokens already held + column")
+        fresh = [slot for slot in slots if self.cache.manager.sequence_id(slot) is None]
+        for slot in fresh:
+            self._generation[slot] += 1
+        self.cache.register_batch([(f"slot-{slot}-generation-{self._generation[slot]}", slot) for slot in fresh])
         self._decode_state = None
         self.cache.set_batch_state(slot_ids=slots, counts=lengths, width=width)
         keep = None

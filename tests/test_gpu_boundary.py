@@ -69,6 +69,16 @@ def test_masked_form_equals_slot_form(tiny):
         runner.prefill_slots(ids, positions=positions, write_mask=holes, valid_lengths=valid)
     with pytest.raises(ValueError, match="exceed the NQKV cache"):
         runner.prefill_slots(ids, positions=positions + 90, write_mask=write_mask, valid_lengths=valid)
+    # the slots still hold their tokens: a second prompt must say so in valid_lengths and continue their positions
+    with pytest.raises(ValueError, match="valid_lengths of a writing row"):
+        runner.prefill_slots(ids, positions=positions, write_mask=write_mask, valid_lengths=valid)
+    held = torch.tensor([22, 0, 10, 18], device="cuda")
+    with pytest.raises(ValueError, match="continue each slot"):
+        runner.prefill_slots(ids, positions=positions, write_mask=write_mask,
+                             valid_lengths=held + torch.tensor(lengths, device="cuda"))
+    with pytest.raises(ValueError, match="continue each slot"):
+        runner.prefill_slots(ids[:1, :5], slots=[1], lengths=[5], positions=positions[:1, :5] + 1)     # a fresh slot starts at 0
+    assert cache.manager.sequence_id(1) is None and cache.manager.metadata.sequence_lengths.tolist() == [22, 0, 10, 18]
     runner.clear_slots(torch.ones(4, dtype=torch.bool, device="cuda"))
 
 

@@ -151,6 +151,28 @@ def test_grouped_gemv_on_the_matrix_cores(rt, oracle, m):
     assert relative_error(bits(half.float()), bits(grouped[0])) < 1e-2
 
 
+@pytest.mark.parametrize("k", [256, 1024, 2048, 16384])
+def test_matrix_core_gemv_gives_the_same_bits_alone_and_in_a_group(rt, k):
+    """A narrow weight alone runs in tiles of 8 channels x 2 interleaved K ranges, the same weight
+    inside a group that fills the chip in tiles of 16 channels x 1 range; the two-range launch takes
+    half the wavefronts of the one-range launch, so the same 128-wide pieces of K meet in the same
+    accumulators in the same order: bit for bit, also at the K where the wavefront count is clamped."""
+    g = torch.Generator().manual_seed(77 + k)
+    weights = []
+    for index, n_out in enumerate((264, 3072)):
+        rotated = rt.hadamard_cuda((0.02 * torch.randn(n_out, k, generator=g)).cuda(), compute_dtype=torch.float32)
+        record = rt.quantize_weight_nqrt4(rotated, q=Q, betas=WEIGHT_BETAS, dither_seed=20261301 + index,
+                                          tensor_name=f"w{index}")
+        weights.append(rt.prepare_fused_linear(record, device="cuda"))
+    x = torch.randn(8, k, generator=g).to(torch.bfloat16).cuda()
+    activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS, hadamard=True)
+    for dtype in (torch.float32, torch.bfloat16):
+        grouped = rt.linear_packed_w4a4_gemv_grouped(activation, weights, output_dtype=dtype)
+        for out, weight in zip(grouped, weights):
+            alone = rt._gemv(activation, weight, split_k=1, output_dtype=dtype)
+            assert torch.equal(out, alone)
+
+
 def _rope_tables(rows, tokens, dim, seed):
     g = torch.Generator().manual_seed(seed)
     angle = 6.0 * torch.rand(rows, tokens, dim // 2, generator=g)

@@ -23,7 +23,9 @@ LENGTHS = [33, 9, 40, 16, 27, 31, 12, 38]           # hot tails of 1, 9, 8, 0, 1
 
 
 @pytest.fixture(scope="module")
-def llama_1b(tmp_path_factory):
+def llama_1b_model(tmp_path_factory):
+    """The random-weight model with its 112 projections swapped for packed modules (done once: the
+    conversion happens in place), and the runner of the first test."""
     from transformers import LlamaConfig, LlamaForCausalLM
     from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
 
@@ -38,6 +40,20 @@ def llama_1b(tmp_path_factory):
     assert len(names) == 16 * 7
     runner = asm.build_w4a4kv4_runner(model, path, capacity=BATCH, max_cache_len=96)
     return model, runner
+
+
+@pytest.fixture
+def llama_1b(llama_1b_model):
+    from nestquant_aiinfra_amd.runtime.nqkv_hf_backend import install_batched_nqkv_llama_backend
+    model, runner = llama_1b_model
+    install_batched_nqkv_llama_backend(model, runner.cache)      # another test may have attached its own cache
+    return model, runner
+
+
+def _runner_of_capacity(model, capacity, max_cache_len):
+    """A further cache and runner over the converted model (the packed weights are shared)."""
+    from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
+    return asm.attach_w4a4kv4_cache(model, capacity=capacity, max_cache_len=max_cache_len)
 
 
 def _cache_tensors(cache):
@@ -115,3 +131,133 @@ def test_graph_equals_eager_and_fused_tracks_modules_at_full_size(llama_1b):
     assert float(cosine.min()) > 0.8, cosine
     assert (fused.argmax(-1) == reference.argmax(-1)).float().mean() >= 0.85
     runner.release_slots(slots)
+
+
+# ---------------------------------------------------------------------------------------------
+# The continuous-batching workload at its stated size: 128-token random-id prompts, 128 generated
+# tokens, engine capacities 1, 2, 4 and 8, slots reused.  The reference pins this level with
+# graph == eager on a model driven through its runner
+# (tests/unit/runtime/test_nqkv_batched_hf_backend.py:533-567, 569-739) and measures it through
+# the engine loop (scripts/benchmark_service_workloads.py:148-151, 215-220).
+
+PROMPT, NEW_TOKENS = 128, 128
+
+
+class _RecordingBackend:
+    """RaggedDecodeBackend over a runner.  Keeps what the test compares: the logits of the newest
+    decode step and, at chosen decode-step counts, a copy of every cache tensor.  With `eager` the
+    decode steps run un-captured."""
+
+    def __init__(self, runner, *, eager, snapshot_at=()):
+        self.runner, self.eager, self.snapshot_at = runner, eager, set(snapshot_at)
+        self.batch_size, self.max_cache_len, self.device = runner.batch_size, runner.max_cache_len, runner.device
+        self.decode_steps, self.last_logits, self.snapshots = 0, None, {}
+
+    def prefill(self, input_ids):
+        return self.runner.prefill(input_ids)
+
+    def prefill_slots(self, input_ids, **kwargs):
+        return self.runner.prefill_slots(input_ids, **kwargs)
+
+    def capture(self, *args, **kwargs):
+        if not self.eager and not self.runner.graph_captured:
+            self.runner.capture()
+
+    def clear_slots(self, slot_mask):
+        self.runner.clear_slots(slot_mask)
+
+    def decode(self, token, *, positions, active_mask, valid_lengths):
+        if self.eager:
+            live = active_mask[:, 0].nonzero(as_tuple=False).flatten().cpu().tolist()
+            index = torch.tensor(live, dtype=torch.long, device=self.device)
+            part = self.runner.decode_eager(token[index], slots=live, positions=positions[index])
+            logits = torch.zeros((self.batch_size, *part.shape[1:]), dtype=part.dtype, device=self.device)
+            logits[index] = part
+        else:
+            logits = self.runner.decode(token, positions=positions, active_mask=active_mask, valid_lengths=valid_lengths)
+        self.decode_steps += 1
+        self.last_logits = logits.clone()
+        if self.decode_steps in self.snapshot_at:
+            self.snapshots[self.decode_steps] = [t.clone() for t in _cache_tensors(self.runner.cache)]
+        return logits
+
+
+def _requests(capacity):
+    """The first wave fills every slot; one of its requests stops early when there is a second slot,
+    so that a late request is prefilled into a reused slot while its neighbours decode."""
+    from nestquant_aiinfra_amd.runtime import DecodeRequest
+    g = torch.Generator().manual_seed(5002)
+    requests = []
+    for index in range(capacity + 1):
+        prompt = tuple(torch.randint(0, VOCAB, (PROMPT,), generator=g).tolist())
+        new_tokens = 96 if (capacity > 1 and index == 1) else NEW_TOKENS
+        requests.append(DecodeRequest(f"request-{index}", prompt, new_tokens))
+    return requests
+
+
+def _drain(backend, capacity, *, decode_burst=1):
+    from nestquant_aiinfra_amd.runtime import AdmissionPolicy, ContinuousBatchInferenceEngine, RequestStatus
+    engine = ContinuousBatchInferenceEngine(backend, decode_burst=decode_burst,
+                                            admission_policy=AdmissionPolicy(min_prefill_batch=1, max_wait_steps=0))
+    requests = _requests(capacity)
+    for request in requests:
+        engine.submit(request)
+    steps = 0
+    while engine.has_work() and steps < 4 * (PROMPT + NEW_TOKENS):
+        engine.step()
+        steps += 1
+    assert not engine.has_work()
+    assert all(r.status is RequestStatus.FINISHED and len(r.generated_token_ids) == r.max_new_tokens for r in requests)
+    return {r.request_id: list(r.generated_token_ids) for r in requests}
+
+
+@pytest.mark.parametrize("capacity", [1, 2, 4, 8])
+def test_engine_workload_at_full_size_graph_equals_eager(llama_1b_model, capacity):
+    model, _ = llama_1b_model
+    runner = _runner_of_capacity(model, capacity, PROMPT + NEW_TOKENS)
+    cache = runner.cache
+    meta = cache.manager.metadata
+    snapshot_at = (50, 120, 200)                    # decode steps: mid-page, after the slot reuse, late
+
+    def all_slots_returned():
+        assert meta.sequence_lengths.tolist() == [0] * capacity and meta.page_counts.tolist() == [0] * capacity
+        assert meta.hot_lengths.tolist() == [0] * capacity and not bool(meta.active_mask.any())
+        assert all(cache.manager.sequence_id(slot) is None for slot in range(capacity))
+        assert cache._host_lengths == [0] * capacity
+
+    graph = _RecordingBackend(runner, eager=False, snapshot_at=snapshot_at)
+    graph_tokens = _drain(graph, capacity)
+    assert runner.graph_captured and sum(runner.graph_replay_counts.values()) == graph.decode_steps
+    assert sorted(graph.snapshots) == list(snapshot_at) and torch.isfinite(graph.last_logits).all()
+    all_slots_returned()
+
+    eager = _RecordingBackend(runner, eager=True, snapshot_at=snapshot_at)
+    replays = sum(runner.graph_replay_counts.values())
+    eager_tokens = _drain(eager, capacity)
+    assert sum(runner.graph_replay_counts.values()) == replays            # no graph ran
+    assert eager.decode_steps == graph.decode_steps
+    assert eager_tokens == graph_tokens
+    assert torch.equal(eager.last_logits, graph.last_logits)              # bit for bit
+    for step in snapshot_at:
+        for a, b in zip(graph.snapshots[step], eager.snapshots[step]):
+            assert torch.equal(a, b)                                      # tables, hot tails, packed pages
+    all_slots_returned()
+
+    # sixteen replays between host reads, the sampler on the device: the step-by-step argmax tokens
+    burst_tokens = _drain(runner, capacity, decode_burst=16)
+    assert burst_tokens == graph_tokens
+    all_slots_returned()
+
+    if capacity == 1:
+        # the engine's text is what the runner alone produces: prefill, then decode + argmax
+        request = _requests(1)[0]
+        ids = torch.tensor([request.prompt_token_ids], device="cuda")
+        logits = runner.prefill_slots(ids, slots=[0], lengths=[PROMPT], last_token_logits=True)
+        token, alone = logits[:, 0].argmax(-1).reshape(1, 1), []
+        for step in range(NEW_TOKENS):
+            alone.append(int(token))
+            if step + 1 < NEW_TOKENS:
+                out = runner.decode(token, slots=[0], positions=torch.tensor([[PROMPT + step]], device="cuda"))
+                token = out[:, 0].argmax(-1).reshape(1, 1)
+        assert alone == graph_tokens["request-0"]
+        runner.release_slots([0])

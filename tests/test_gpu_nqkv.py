@@ -664,3 +664,32 @@ def test_append_and_attend_rejects_what_it_cannot_take(kv):
         manager.append_and_attend(0, query, key, key, attention_scale=float("nan"), workspace=workspace)
     torch.cuda.synchronize()
     assert torch.equal(manager.layers[0].hot_keys, before)
+
+
+def test_decode_attention_refuses_a_misaligned_query(kv):
+    """BF16 query rows are read 16 bytes at a time: a view that starts two bytes into a buffer is refused
+    by the wrapper, and by the library itself when a caller hands it the raw pointer."""
+    from nestquant_aiinfra_amd import _native
+    manager = _manager(kv, capacity=1, max_len=32)
+    manager.register(0, slot=0)
+    cache = manager.layers[0]
+    workspace = kv.BatchedNQKVAttentionWorkspace.create(cache, batch_size=1, query_heads=32, output_dtype=torch.bfloat16)
+    backing = torch.zeros(32 * DIM + 8, dtype=torch.bfloat16, device="cuda")
+    shifted = backing[1:1 + 32 * DIM].view(1, 32, DIM)
+    slot_ids = torch.zeros(1, dtype=torch.int32, device="cuda")
+    active = torch.ones(1, dtype=torch.bool, device="cuda")
+    with pytest.raises(ValueError, match="16-byte aligned"):
+        kv.launch_nqkv_decode_attention(shifted, cache, slot_ids=slot_ids, active_mask=active, attention_scale=0.125,
+                                        workspace=workspace)
+    pool, meta = cache.pool, cache.metadata
+    status = _native.library().nq_nqkv_attention_decode(
+        shifted.data_ptr(), _native.dtype_tag(torch.bfloat16),
+        pool.key_codes.data_ptr(), pool.key_betas.data_ptr(), pool.key_norms.data_ptr(),
+        pool.value_codes.data_ptr(), pool.value_betas.data_ptr(), pool.value_norms.data_ptr(),
+        pool.beta_table.data_ptr(), pool.value_beta_table.data_ptr(),
+        meta.page_indices.data_ptr(), meta.page_counts.data_ptr(), meta.last_page_lens.data_ptr(),
+        meta.hot_lengths.data_ptr(), meta.active_mask.data_ptr(), cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(),
+        slot_ids.data_ptr(), active.data_ptr(), 1, cache.max_sequences, cache.max_pages_per_sequence, 32, pool.num_kv_heads,
+        DIM, pool.page_size, 0.125, 0, None, None, workspace.output.data_ptr(), workspace.buffer.data_ptr(),
+        workspace.buffer.numel(), _native.stream_handle(shifted.device))
+    assert status == _native.NQ_ERR_ARGUMENT and b"16-byte alignment" in _native.library().nq_last_error()

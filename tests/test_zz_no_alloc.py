@@ -64,6 +64,32 @@ def test_static_scratch_gemv_equals_the_workspace_gemv(oracle, resolved):
             assert relative_error(bits(actual), ref32) <= 1e-2
 
 
+def test_static_scratch_gemv_allocates_no_device_memory(oracle):
+    """The property the entry point exists for: once the library is warm, a call changes neither
+    the device's free memory nor what the framework's allocator holds."""
+    from nestquant_aiinfra_amd import _native
+    from nestquant_aiinfra_amd.runtime import w4a4_linear as rt
+    lib = _native.library()
+    _native.check(lib.nq_w4a4_gemv_static_init())
+    activation, weight, ref32, seed = _case(oracle, rt, 8, 8192, 256, 20261203)
+    m, k, n = activation.token_count, activation.feature_count, weight.record.indices.shape[0]
+    out = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    arguments = [
+        activation.code_payload.data_ptr(), activation.beta_payload.data_ptr(), activation.row_norms.data_ptr(),
+        activation.beta_table.data_ptr(), None, weight.code_payload.data_ptr(), weight.beta_payload.data_ptr(),
+        weight.resolved_words.data_ptr(), weight.resolved_tails.data_ptr(), weight.row_norms.data_ptr(),
+        weight.beta_table.data_ptr(), m, k, n, 0, seed, 4, out.data_ptr(), _native.NQ_F32,
+        _native.stream_handle(out.device)]
+    _native.check(lib.nq_w4a4_gemv_static(*arguments))                   # warm: code objects loaded
+    torch.cuda.synchronize()
+    free_before, reserved_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
+    for _ in range(3):
+        _native.check(lib.nq_w4a4_gemv_static(*arguments))
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_reserved() == reserved_before
+    assert relative_error(bits(out), ref32) <= 1e-2
+
+
 def test_static_scratch_gemv_rejects_what_does_not_fit():
     from nestquant_aiinfra_amd import _native
     lib = _native.library()
