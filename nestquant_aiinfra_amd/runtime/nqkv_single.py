@@ -286,7 +286,7 @@ class NQKVLlamaCache(Cache):
         if dtype != torch.bfloat16:
             raise ValueError("the NQKV hot tails and writer are BF16")
         self.num_layers, self.num_query_heads, self.num_kv_heads = num_layers, num_query_heads, num_kv_heads
-        self.head_dim, self.max_cache_len, self.page_size, self.dtype = head_dim, max_cache_len, page_size, dtype
+        self.head_dim, self._max_cache_len, self.page_size, self.dtype = head_dim, max_cache_len, page_size, dtype
         target = torch.device(device)
         if target.type == "cuda" and target.index is None:
             target = torch.device("cuda", torch.cuda.current_device())
@@ -350,9 +350,13 @@ class NQKVLlamaCache(Cache):
     def get_max_length(self, layer_idx: int | None = None) -> int:
         if layer_idx is not None:
             self._validate_layer(layer_idx)
-        return self.max_cache_len
+        return self._max_cache_len
 
     get_max_cache_shape = get_max_length
+
+    @property
+    def max_cache_len(self) -> int:          # a read-only property of the transformers Cache base class
+        return self._max_cache_len
 
     def get_mask_sizes(self, query_length, layer_idx: int) -> tuple[int, int]:
         self._validate_layer(layer_idx)
