@@ -20,6 +20,33 @@ _MAGIC = b"NQPK"
 _VERSION = 1
 
 
+class ByteReader:
+    """Front-to-back reader over a bytes-like container: every read names what it wants and fails
+    with that name when the container is too short; `finish` fails when bytes are left over."""
+
+    def __init__(self, data, *, what: str) -> None:
+        self._view, self._at, self._what = memoryview(data).cast("B"), 0, what
+
+    def take(self, count: int, name: str) -> bytes:
+        if count < 0 or self._at + count > len(self._view):
+            raise ValueError(f"{self._what} is shorter than its {name} ({count} bytes at offset {self._at}, "
+                             f"{len(self._view)} in all)")
+        piece = bytes(self._view[self._at:self._at + count])
+        self._at += count
+        return piece
+
+    def unpack(self, layout: struct.Struct, name: str) -> tuple:
+        return layout.unpack(self.take(layout.size, name))
+
+    def remaining(self) -> int:
+        return len(self._view) - self._at
+
+    def finish(self) -> None:
+        if self._at != len(self._view):
+            raise ValueError(f"{self._what} has {len(self._view) - self._at} bytes after its last payload: "
+                             "stated lengths do not add up to the container size")
+
+
 def bits_for_cardinality(cardinality: int) -> int:
     if cardinality < 1:
         raise ValueError("cardinality must be positive")
@@ -99,31 +126,31 @@ class PackedNestQuantIndices:
 
     @classmethod
     def from_bytes(cls, data) -> "PackedNestQuantIndices":
-        view = memoryview(data)
-        if len(view) < _HEADER.size:
-            raise ValueError("input is shorter than the NestQuant packing header")
-        magic, version, ndim, q, beta_count, code_len, beta_len = _HEADER.unpack_from(view)
+        """Parse a container.  The header fixes every size that follows it, so the container is
+        taken apart by a reader that refuses to run past the end, and the sizes the header states
+        are then compared with the ones the shape implies."""
+        reader = ByteReader(data, what="NestQuant packing container")
+        magic, version, ndim, q, beta_count, code_bytes, beta_bytes = reader.unpack(_HEADER, "header")
         if magic != _MAGIC:
-            raise ValueError("invalid NestQuant packing magic")
+            raise ValueError(f"invalid NestQuant packing magic {bytes(magic)!r}")
         if version != _VERSION:
             raise ValueError(f"unsupported NestQuant packing version: {version}")
         if ndim < 2:
-            raise ValueError("packed code shape must include rows and 8D block dimension")
+            raise ValueError("a packed tensor has at least a row axis and the axis of eight block coordinates")
         _check_cardinalities(q, beta_count)
-        shape_end = _HEADER.size + 8 * ndim
-        if len(view) < shape_end:
-            raise ValueError("truncated tensor shape in packing header")
-        shape = struct.unpack_from(f"<{ndim}Q", view, _HEADER.size)
-        if any(d < 1 for d in shape) or shape[-1] != 8:
-            raise ValueError("shape must be positive and end with E8 dimension 8")
-        if code_len != _ceil_bytes(math.prod(shape), bits_for_cardinality(q)):
-            raise ValueError("residue payload length disagrees with header shape")
-        if beta_len != _ceil_bytes(math.prod(shape[:-1]), bits_for_cardinality(beta_count)):
-            raise ValueError("beta-index payload length disagrees with header shape")
-        if len(view) != shape_end + code_len + beta_len:
-            raise ValueError("packed container has trailing or truncated payload bytes")
-        return cls(tuple(shape), q, beta_count, bytes(view[shape_end:shape_end + code_len]),
-                   bytes(view[shape_end + code_len:]))
+        shape = reader.unpack(struct.Struct(f"<{ndim}Q"), "shape")
+        if min(shape) < 1 or shape[-1] != 8:
+            raise ValueError(f"shape {tuple(shape)} must be positive and end in the E8 dimension 8")
+        stated = {"residue": code_bytes, "beta-index": beta_bytes}
+        implied = {"residue": _ceil_bytes(math.prod(shape), bits_for_cardinality(q)),
+                   "beta-index": _ceil_bytes(math.prod(shape[:-1]), bits_for_cardinality(beta_count))}
+        for stream in stated:
+            if stated[stream] != implied[stream]:
+                raise ValueError(f"{stream} payload of {stated[stream]} bytes, but shape {tuple(shape)} implies "
+                                 f"{implied[stream]}")
+        codes, betas = reader.take(code_bytes, "residue payload"), reader.take(beta_bytes, "beta-index payload")
+        reader.finish()
+        return cls(tuple(shape), q, beta_count, codes, betas)
 
     def unpack(self, *, device: torch.device | str = "cpu") -> tuple[torch.Tensor, torch.Tensor]:
         """Host-side inspection helper: int64 codes ``shape`` and beta ids ``shape[:-1]``."""

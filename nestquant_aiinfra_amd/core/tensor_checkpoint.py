@@ -21,7 +21,7 @@ import torch
 
 from .codec import (CURRENT_CODEC_SEMANTICS, LEGACY_CODEC_SEMANTICS, STATELESS_DITHER_ALGORITHM,
                     STATELESS_MODULUS, UPSTREAM_CODEC_SEMANTICS)
-from .packing import PackedNestQuantIndices
+from .packing import ByteReader, PackedNestQuantIndices
 
 _HEADER = struct.Struct("<4sBBIQQQ")
 _MAGIC = b"NQRT"
@@ -50,6 +50,24 @@ def _validate_stateless(seed, algorithm) -> None:
         raise ValueError("dither_seed must be an integer in [0, 2**31)")
     if algorithm != STATELESS_DITHER_ALGORITHM:
         raise ValueError(f"unsupported stateless dither algorithm: {algorithm}")
+
+
+def _metadata_fields(blob: bytes) -> dict:
+    """The JSON metadata of a record as typed values; anything missing or of the wrong kind is one error."""
+    try:
+        raw = json.loads(blob.decode("utf-8"))
+    except (UnicodeDecodeError, json.JSONDecodeError) as error:
+        raise ValueError("invalid tensor checkpoint metadata") from error
+    try:
+        fields = {"tensor_name": raw["tensor_name"], "rows": int(raw["rows"]), "feature_count": int(raw["feature_count"]),
+                  "betas": tuple(float(value) for value in raw["betas"]), "output_dtype": _NAME_TO_DTYPE[raw["output_dtype"]]}
+    except (KeyError, TypeError, ValueError, AttributeError) as error:
+        raise ValueError("missing or invalid tensor checkpoint metadata fields") from error
+    if not isinstance(fields["tensor_name"], str):
+        raise ValueError("invalid tensor name")
+    for optional in ("q", "beta_count", "dither_seed", "dither_algorithm", "codec_semantics"):
+        fields[optional] = raw.get(optional)
+    return fields
 
 
 @dataclass(frozen=True)
@@ -118,61 +136,51 @@ class PackedNestQuantTensor:
 
     @classmethod
     def from_bytes(cls, data) -> "PackedNestQuantTensor":
-        view = memoryview(data)
-        if len(view) < 5:
+        """Parse an NQRT record (versions 2 to 4).  Only the payload-free dither modes reach the
+        packed path: none (0) and the stateless counter hash (3)."""
+        # magic and version sit in the first five bytes of every version: they are judged before the rest
+        prefix = bytes(memoryview(data).cast("B")[:5])
+        if len(prefix) < 5:
             raise ValueError("input is shorter than the tensor checkpoint header")
-        if bytes(view[:4]) != _MAGIC:
+        magic, version = struct.unpack("<4sB", prefix)
+        if magic != _MAGIC:
             raise ValueError("invalid tensor checkpoint magic")
-        version = int(view[4])
         if version not in (2, 3, 4):
             raise ValueError(f"unsupported tensor checkpoint version: {version}")
-        if len(view) < _HEADER.size:
-            raise ValueError("input is shorter than the v2 tensor checkpoint header")
-        _, _, dither_mode, metadata_len, indices_len, norms_len, dither_len = _HEADER.unpack_from(view)
-        if dither_mode not in (0, 1, 2, 3):
-            raise ValueError("invalid dither storage mode")
+        reader = ByteReader(data, what="tensor checkpoint")
+        _, _, dither_mode, *lengths = reader.unpack(_HEADER, "header")
         if dither_mode in (1, 2):
             raise ValueError("stored-dither and generator-state records are not supported by the packed path")
-        offset = _HEADER.size
-        if offset + metadata_len + indices_len + norms_len + dither_len != len(view):
+        if dither_mode not in (0, 3):
+            raise ValueError(f"invalid dither storage mode {dither_mode}")
+        metadata_bytes, indices_bytes, norms_bytes, dither_bytes = lengths
+        if metadata_bytes + indices_bytes + norms_bytes + dither_bytes != reader.remaining():
             raise ValueError("tensor checkpoint payload lengths do not match file size")
-        if dither_len:
-            raise ValueError("dither payload exists for a payload-free mode")
-        try:
-            metadata = json.loads(bytes(view[offset:offset + metadata_len]).decode("utf-8"))
-        except (UnicodeDecodeError, json.JSONDecodeError) as error:
-            raise ValueError("invalid tensor checkpoint metadata") from error
-        offset += metadata_len
-        indices = PackedNestQuantIndices.from_bytes(view[offset:offset + indices_len])
-        offset += indices_len
-        norms_blob = bytes(view[offset:offset + norms_len])
-        try:
-            dtype = _NAME_TO_DTYPE[metadata["output_dtype"]]
-            rows = int(metadata["rows"])
-            features = int(metadata["feature_count"])
-            name = metadata["tensor_name"]
-            betas = tuple(float(value) for value in metadata["betas"])
-        except (KeyError, TypeError, ValueError) as error:
-            raise ValueError("missing or invalid tensor checkpoint metadata fields") from error
-        if not isinstance(name, str):
-            raise ValueError("invalid tensor name")
-        if metadata.get("q") != indices.q or metadata.get("beta_count") != indices.beta_count:
+        if dither_bytes:
+            raise ValueError("a record whose dither is regenerated carries no dither payload")
+        fields = _metadata_fields(reader.take(metadata_bytes, "metadata"))
+        indices = PackedNestQuantIndices.from_bytes(reader.take(indices_bytes, "index container"))
+        norms_blob = reader.take(norms_bytes, "row norms")
+        reader.finish()
+
+        rows, features, dtype = fields["rows"], fields["feature_count"], fields["output_dtype"]
+        if (fields["q"], fields["beta_count"]) != (indices.q, indices.beta_count):
             raise ValueError("metadata disagrees with packed index parameters")
-        if indices.shape != (rows, features // 8, 8) or features <= 0 or features % 8:
-            raise ValueError("metadata feature shape disagrees with packed indices")
+        if features <= 0 or features % 8 or indices.shape != (rows, features // 8, 8):
+            raise ValueError(f"metadata says {rows} rows of {features} features, the index container holds "
+                             f"shape {indices.shape}")
         if len(norms_blob) != rows * torch.empty((), dtype=dtype).element_size():
             raise ValueError("row norm payload size disagrees with metadata")
-        seed = metadata.get("dither_seed") if dither_mode == 3 else None
-        algorithm = metadata.get("dither_algorithm") if dither_mode == 3 else None
+        seed = algorithm = None
         if dither_mode == 3:
             if version < 4:
                 raise ValueError("stateless dither requires NQRT v4")
+            seed, algorithm = fields["dither_seed"], fields["dither_algorithm"]
             _validate_stateless(seed, algorithm)
-        semantics = metadata.get("codec_semantics") if version >= 3 else LEGACY_CODEC_SEMANTICS
-        record = cls(tensor_name=name, indices=indices,
-                     row_norms=_tensor_from_bytes(norms_blob, (rows,), dtype), betas=betas,
-                     feature_count=features, output_dtype=dtype, dither_seed=seed,
-                     dither_algorithm=algorithm, codec_semantics=semantics)
+        record = cls(tensor_name=fields["tensor_name"], indices=indices,
+                     row_norms=_tensor_from_bytes(norms_blob, (rows,), dtype), betas=fields["betas"],
+                     feature_count=features, output_dtype=dtype, dither_seed=seed, dither_algorithm=algorithm,
+                     codec_semantics=fields["codec_semantics"] if version >= 3 else LEGACY_CODEC_SEMANTICS)
         record._validate()
         return record
 

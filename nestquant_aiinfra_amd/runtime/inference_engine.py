@@ -6,7 +6,10 @@ EngineStep, GreedyHostSampler, ContinuousBatchInferenceEngine.
 What is added for a backend that samples on the device (BatchedNQKVLlamaRunner.decode_greedy):
 with `decode_burst` > 1 a step in which nobody waits for a slot replays the captured decode
 graph up to that many times before the host reads the chosen tokens once; requests that meet
-their end-of-sequence token inside a burst are cut there."""
+their end-of-sequence token inside a burst are cut there.  A backend that says
+`takes_slot_lists` is driven by slot lists instead of capacity-wide masks: a step then uploads
+one row of tokens and positions per running request and reads nothing back before the launch,
+and a prompt's logits are computed for its last token only."""
 
 from __future__ import annotations
 
@@ -84,6 +87,7 @@ class ContinuousBatchInferenceEngine:
         self.scheduler = ContinuousBatchScheduler(self.capacity)
         # bursts need the device sampler, which is greedy: any other sampler keeps one token per step
         self.decode_burst = decode_burst if (sampler is None and hasattr(backend, "decode_greedy")) else 1
+        self._slot_lists = bool(getattr(backend, "takes_slot_lists", False))
         self._ready = False
         self._steps_taken = 0
         self._slots_idle_since: int | None = None
@@ -155,6 +159,13 @@ class ContinuousBatchInferenceEngine:
         if not admitted:
             return {}, ()
         width = max(len(request.prompt_token_ids) for request in admitted)
+        if self._slot_lists:
+            rows = [list(request.prompt_token_ids) + [self.pad_token_id] * (width - len(request.prompt_token_ids))
+                    for request in admitted]
+            logits = self.backend.prefill_slots(
+                torch.tensor(rows, dtype=torch.long, device=self.device), slots=[request.slot for request in admitted],
+                lengths=[len(request.prompt_token_ids) for request in admitted], last_token_logits=True)
+            return self._record(admitted, [[token] for token in self.sampler(logits[:, 0]).tolist()])
         input_ids = torch.full((self.capacity, width), self.pad_token_id, dtype=torch.long, device=self.device)
         write_mask = torch.zeros((self.capacity, width), dtype=torch.bool, device=self.device)
         # every column of a row gets its own position, padding included
@@ -201,6 +212,13 @@ class ContinuousBatchInferenceEngine:
                                      device=self.device)
             history = self.backend.decode_greedy(tokens, slots=slots, positions=positions, steps=burst).tolist()
             return self._record(running, [[history[step][row] for step in range(burst)] for row in range(len(running))])
+        if self._slot_lists:
+            tokens = torch.tensor([[request.generated_token_ids[-1]] for request in running], dtype=torch.long,
+                                  device=self.device)
+            positions = torch.tensor([[request.next_position] for request in running], dtype=torch.long,
+                                     device=self.device)
+            logits = self.backend.decode(tokens, slots=[request.slot for request in running], positions=positions)
+            return self._record(running, [[value] for value in self.sampler(logits[:, -1]).tolist()])
         token = self._column(self.pad_token_id, torch.long)
         positions = self._column(0, torch.long)
         active = self._column(False, torch.bool)

@@ -367,6 +367,7 @@ class BatchedNQKVLlamaRunner:
     """
 
     GREEDY_HISTORY_STEPS = 256
+    takes_slot_lists = True          # the engine may call prefill_slots / decode with slots= instead of masks
 
     def __init__(self, model: torch.nn.Module, cache: BatchedNQKVLlamaCache, *,
                  fused_decode: bool | None = None, fused_prefill: bool | None = None,

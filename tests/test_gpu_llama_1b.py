@@ -166,6 +166,9 @@ class _RecordingBackend:
     def clear_slots(self, slot_mask):
         self.runner.clear_slots(slot_mask)
 
+    def decode_greedy(self, tokens, *, slots, positions, steps):
+        return self.runner.decode_greedy(tokens, slots=slots, positions=positions, steps=steps)
+
     def decode(self, token, *, positions, active_mask, valid_lengths):
         if self.eager:
             live = active_mask[:, 0].nonzero(as_tuple=False).flatten().cpu().tolist()
@@ -247,7 +250,7 @@ def test_engine_workload_at_full_size_graph_equals_eager(llama_1b_model, capacit
     all_slots_returned()
 
     # sixteen replays between host reads, the sampler on the device: the step-by-step argmax tokens
-    burst_tokens = _drain(runner, capacity, decode_burst=16)
+    burst_tokens = _drain(_RecordingBackend(runner, eager=False), capacity, decode_burst=16)
     late = f"request-{capacity}"
     assert all(burst_tokens[name] == tokens for name, tokens in graph_tokens.items() if name != late)
     if capacity <= 4:
@@ -260,8 +263,14 @@ def test_engine_workload_at_full_size_graph_equals_eager(llama_1b_model, capacit
         assert burst_tokens[late][:16] == graph_tokens[late][:16] and len(burst_tokens[late]) == NEW_TOKENS
     all_slots_returned()
 
+    # The runner itself as the backend: the engine then hands it slot lists and asks for a prompt's last
+    # logits only (another LM-head kernel than the one that makes every position's logits, so a first token
+    # chosen between two near-equal BF16 logits may differ from the runs above).
+    direct_tokens = _drain(runner, capacity)
+    all_slots_returned()
     if capacity == 1:
-        # the engine's text is what the runner alone produces: prefill, then decode + argmax
+        # that text is what the runner alone produces: prefill, then decode + argmax
+        graph_tokens = direct_tokens
         request = _requests(1)[0]
         ids = torch.tensor([request.prompt_token_ids], device="cuda")
         logits = runner.prefill_slots(ids, slots=[0], lengths=[PROMPT], last_token_logits=True)
