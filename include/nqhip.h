@@ -500,6 +500,44 @@ int nq_attention_output_stage(const void *workspace_dev, int64_t rows, int q_hea
                               void *decoded_bf16_dev, void *stream);
 
 /*
+ * A decode step's input stage and the packed linear(s) that consume its rows, in one launch: what
+ * nq_fused_input_stage (mode 1: residual + RMSNorm, mode 2: SiLU(gate) * x) or
+ * nq_attention_output_stage (mode 3: attention merge) with the Hadamard rotation and q = 14 leaves
+ * in codes / beta ids / norms / decoded BF16 rows, followed by nq_w4a4_gemv_grouped of `count`
+ * (1..4) resolved weights on those rows; all outputs bit for bit those of the two calls.  The first
+ * rows * slices workgroups of the grid run the encoder; the others decode their weights while the
+ * encoder is still busy, wait until every encoder workgroup has set its flag word, and then
+ * multiply.  rows in [1, 16] (8 for n = 8192), n = K in {2048, 8192}, four betas.
+ *   flags_dev            nq_fused_stage_linear_flag_words(rows, n) words of device memory, zero when
+ *                        the launch starts and owned by it until the next launch on the stream that
+ *                        names them as previous_flags_dev (which clears them) has finished;
+ *   previous_flags_dev   the flag words of the launch before this one on the same stream (any
+ *                        earlier launch that has completed), cleared here; NULL with 0 words for
+ *                        none: a step of several launches hands each launch's words to the next and
+ *                        the last launch's words to the first launch of the next step;
+ *   status_dev           one word, device or pinned host memory: set to 1 by a workgroup whose wait
+ *                        ended after spin_limit polls without all flags set; that workgroup stores no
+ *                        outputs and exits, so the launch always ends.  A caller that finds it set
+ *                        must not trust the outputs and should go back to the two calls;
+ *   spin_limit           polls (about half a microsecond each) a consumer makes before it gives up;
+ *                        0 makes a consumer give up after one look (a test of the failure path).
+ * attention_workspace_dev / q_heads / parts: as for nq_attention_output_stage (mode 3 only); the
+ * other encoder arguments as for nq_fused_input_stage; the weight arrays as for nq_w4a4_gemv_grouped.
+ * No counterpart in the reference, which launches the input stage and the linear separately
+ * (nestquant/models/fused_linear.py:287-306, 316-407).
+ */
+int nq_fused_stage_linear_flag_words(int64_t rows, int64_t n);
+int nq_fused_stage_linear(
+    const void *x_dev, int64_t rows, int64_t n, int mode, const void *residual_dev, void *residual_out_dev,
+    const void *norm_weight_dev, float eps, const void *gate_dev, const void *attention_workspace_dev, int q_heads,
+    int parts, void *staged_out_dev, const float *betas_dev, int beta_count, uint8_t *codes_dev, uint8_t *beta_ids_dev,
+    float *norms_dev, void *decoded_bf16_dev, int count, const uint32_t *const *w_resolved_words_dev,
+    const uint16_t *const *w_resolved_tails_dev, const float *const *w_norms_dev, const float *const *w_betas_dev,
+    const int *w_n, const int64_t *weight_offsets, const int64_t *weight_seeds, void *const *out_dev, int out_dtype,
+    uint32_t *flags_dev, uint32_t *previous_flags_dev, int previous_flag_words, uint32_t *status_dev, int spin_limit,
+    void *stream);
+
+/*
  * Causal attention of a chunk of new tokens over the packed cache (prefill, chunked prefill,
  * continuation).  Call after nq_nqkv_advance + nq_nqkv_write of the same chunk: query token t
  * of batch row r (t < counts[r], or uniform_count when counts is NULL) sits at absolute

@@ -74,6 +74,9 @@ SIGNATURES = {
     "nq_greedy_sample_workspace_bytes": (_size, [_i32]),
     "nq_bf16_rows_linear": (_i32, [_ptr, _ptr, _i32, _i64, _i64, _ptr, _ptr]),
     "nq_bf16_rows_linear_grouped": (_i32, [_ptr, _ptr, _i32, _i64, _i32, _ptr, _ptr, _ptr]),
+    "nq_fused_stage_linear_flag_words": (_i32, [_i64, _i64]),
+    "nq_fused_stage_linear": (_i32, [_ptr, _i64, _i64, _i32, _ptr, _ptr, _ptr, _c.c_float, _ptr, _ptr, _i32, _i32, _ptr, _ptr, _i32,
+                                     _ptr, _ptr, _ptr, _ptr, _i32] + [_ptr] * 8 + [_i32, _ptr, _ptr, _i32, _ptr, _i32, _ptr]),
     "nq_attention_output_stage": (_i32, [_ptr, _i64, _i32, _i32, _i32, _ptr, _i32, _ptr, _i32, _i32, _ptr, _ptr, _ptr,
                                          _ptr, _ptr]),
 }

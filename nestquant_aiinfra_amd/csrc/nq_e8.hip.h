@@ -356,6 +356,29 @@ __device__ __forceinline__ void resolved_dither_bits(uint32_t counter_plus_seed,
     resolved_hash_bits(t, bits);
 }
 
+// The same for kBlocks consecutive blocks of one lane (counters counter_plus_seed .. + 8 kBlocks - 1), with
+// one test for the whole run, taken by the wavefront as a whole: a run that stays inside one stretch of
+// 2^16 counters in every lane shares the bits 16..30 of all its counters.  Same values as kBlocks calls
+// of resolved_dither_bits.
+template <int kBlocks>
+__device__ __forceinline__ void resolved_dither_bits_run(uint32_t counter_plus_seed, uint32_t (&bits)[kBlocks][8]) {
+    const uint32_t base = counter_plus_seed & 0x7fffffffu;
+    const bool leaves_its_stretch = (base & 0xffffu) > 0x10000u - 8u * kBlocks;
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(leaves_its_stretch) != 0, 0)) {
+#pragma unroll
+        for (int b = 0; b < kBlocks; b++) resolved_dither_bits(counter_plus_seed + 8u * b, bits[b]);
+        return;
+    }
+    const uint32_t high = base >> 16;
+#pragma unroll
+    for (int b = 0; b < kBlocks; b++) {
+        uint32_t t[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) t[j] = (base + (uint32_t)(8 * b + j)) ^ high;
+        resolved_hash_bits(t, bits[b]);
+    }
+}
+
 // The part that needs the stored block: out[j] = (s_j - u_j) * 2^17 * scale.  A weight's float
 // pattern is its dither part plus f_j 2^17: a bit-field extract and a shift-add.
 __device__ __forceinline__ void resolved_apply(uint32_t lo, uint32_t hi, const uint32_t (&bits)[8], float scale,

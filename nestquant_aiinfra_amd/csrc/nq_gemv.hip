@@ -31,16 +31,6 @@ constexpr int kGemvThreads = 256;
 constexpr int kGemvWaves = kGemvThreads / 64;
 constexpr int kGemvMaxRows = 8;
 
-// Sum over the 16 lanes of a DPP row, left in every lane of the row: exchanges inside quads,
-// then the mirrored half row, then the mirrored row.
-__device__ __forceinline__ float row16_sum(float v) {
-    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
-    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
-    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
-    return v;
-}
-
 // kResolved: the weight comes as resolved blocks (w_words = 32-bit words, w_tails = 16-bit
 // words, see nq_e8.hip.h) instead of NQRT4 code words and beta bytes.
 // R: output channels per workgroup.  A lane decodes block b of all R channels against one
@@ -177,19 +167,6 @@ w4a4_gemv_kernel(const uint4 *__restrict__ act, const uint32_t *__restrict__ w_w
                                k_slice, blockIdx.x, blockIdx.y, seed_plus_offset, sqrt_k, out_f32, out_bf16);
 }
 
-// Several weights that share one activation (q/k/v or gate/up) in one launch: the grid is the
-// concatenation of their channel groups.
-constexpr int kGemvMaxGroup = 4;
-struct GemvWeights {
-    const uint32_t *words[kGemvMaxGroup];
-    const uint16_t *tails[kGemvMaxGroup];
-    const float *norms[kGemvMaxGroup], *betas[kGemvMaxGroup];
-    void *out[kGemvMaxGroup];
-    int n[kGemvMaxGroup], first_group[kGemvMaxGroup];
-    uint32_t seed_plus_offset[kGemvMaxGroup];
-    int count;
-};
-
 template <int M, int R>
 __global__ void __launch_bounds__(kGemvThreads)
 w4a4_gemv_grouped_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, int k_size, float sqrt_k,
@@ -213,8 +190,6 @@ w4a4_gemv_grouped_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_row
 // 8 of tails and 64 of activation per super-step, requested one super-step ahead.  Partial
 // tiles meet in LDS and are added in wavefront order.  (The 4 x 4 x 4 block instruction would
 // allow four channels per workgroup, but issues at a quarter of this one's rate.)
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int kMfmaGemvMaxWaves = 16;
 
 // R: K ranges per tile.  With R = 1 the 16 rows of the A operand are 16 channels.  Narrow

@@ -86,4 +86,30 @@ inline int launch_splitk_reduce_grouped(const float *partials, int split, int64_
 
 inline size_t align256(size_t bytes) { return (bytes + 255) & ~(size_t)255; }
 
+// Sum over the 16 lanes of a DPP row, left in every lane of the row: exchanges inside quads,
+// then the mirrored half row, then the mirrored row.
+__device__ __forceinline__ float row16_sum(float v) {
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
+    return v;
+}
+
+// Several weights that share one activation (q/k/v or gate/up) in one launch: the grid is the
+// concatenation of their channel groups.
+constexpr int kGemvMaxGroup = 4;
+struct GemvWeights {
+    const uint32_t *words[kGemvMaxGroup];
+    const uint16_t *tails[kGemvMaxGroup];
+    const float *norms[kGemvMaxGroup], *betas[kGemvMaxGroup];
+    void *out[kGemvMaxGroup];
+    int n[kGemvMaxGroup], first_group[kGemvMaxGroup];
+    uint32_t seed_plus_offset[kGemvMaxGroup];
+    int count;
+};
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
 }  // namespace nq

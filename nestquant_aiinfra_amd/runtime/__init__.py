@@ -15,6 +15,9 @@ _EXPORTS = {
     "quantize_activation_cuda": "w4a4_linear",
     "fused_input_stage": "w4a4_linear",
     "quantize_weight_nqrt4": "w4a4_linear",
+    "StageLinearSync": "w4a4_linear",
+    "can_use_fused_stage_linear": "w4a4_linear",
+    "fused_stage_linear": "w4a4_linear",
     "resolve_weight": "w4a4_linear",
     "prepare_fused_linear": "w4a4_linear",
     "dequantize_rows_packed": "w4a4_linear",

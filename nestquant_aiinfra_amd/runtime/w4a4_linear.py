@@ -713,6 +713,141 @@ def _group_plan(weights: Sequence[PreparedNQRTLinear]) -> tuple:
     return plan
 
 
+class StageLinearSync:
+    """The hand-over state of `fused_stage_linear` launches that follow each other on one stream:
+    a ring of flag-word sets (each launch takes the next set and clears the one before it), the
+    status word a consumer sets when its bounded wait runs out (pinned host memory, so that the
+    host can look at it without a synchronisation), and the number of polls of that wait."""
+
+    FLAG_WORDS = 256          # words per set: the most producer workgroups a launch has
+
+    def __init__(self, device: torch.device, *, sets: int = 128, spin_limit: int = 400_000) -> None:
+        if sets < 2:
+            raise ValueError("the ring needs at least two sets of flag words")
+        self.flags = torch.zeros((sets, self.FLAG_WORDS), dtype=torch.int32, device=device)
+        self.status = torch.zeros(1, dtype=torch.int32).pin_memory()
+        self.spin_limit = int(spin_limit)
+        self._next = 0
+        self._previous: tuple[int, int] | None = None       # (set, words) of the launch before
+
+    def take(self, words: int) -> tuple[int, int | None, int]:
+        """(pointer to this launch's flag words, pointer to the previous launch's or None, their count)."""
+        if not 1 <= words <= self.FLAG_WORDS:
+            raise ValueError("a launch has between 1 and 256 producer workgroups")
+        current = self._next
+        self._next = (current + 1) % self.flags.shape[0]
+        previous = self._previous
+        self._previous = (current, words)
+        here = self.flags[current].data_ptr()
+        if previous is None:
+            return here, None, 0
+        return here, self.flags[previous[0]].data_ptr(), previous[1]
+
+    def position(self) -> tuple[int, tuple[int, int] | None]:
+        return self._next, self._previous
+
+    def rewind(self, position: tuple[int, tuple[int, int] | None]) -> None:
+        """Back to an earlier point of the ring: a captured graph replays the launches recorded from
+        that point on, so whatever is launched after the capture must continue where the graph ends."""
+        self._next, self._previous = position
+
+    @property
+    def timed_out(self) -> bool:
+        return bool(self.status[0].item())
+
+    def reset(self) -> None:
+        """After a time-out (or before a capture): every flag word and the status back to zero."""
+        self.flags.zero_()
+        self.status.zero_()
+        self._next, self._previous = 0, None
+
+
+def can_use_fused_stage_linear(rows: int, k: int, weights: Sequence[PreparedNQRTLinear]) -> bool:
+    """Whether `fused_stage_linear` takes this decode-step pair: up to 16 rows of 2048 values or up to
+    8 of 8192, one to four resolved weights of that K."""
+    return ((k == 2048 and 1 <= rows <= 16) or (k == 8192 and 1 <= rows <= 8)) and 1 <= len(weights) <= 4 and all(
+        w.resolved_words is not None and w.record.feature_count == k for w in weights)
+
+
+def fused_stage_linear(inputs: torch.Tensor | None, weights: Sequence[PreparedNQRTLinear], sync: StageLinearSync, *,
+                       mode: str, beta_table: torch.Tensor, residual: torch.Tensor | None = None,
+                       norm_weight: torch.Tensor | None = None, eps: float = 0.0, gate: torch.Tensor | None = None,
+                       attention_workspace=None, want_residual: bool = False, want_staged: bool = False,
+                       output_dtype: torch.dtype = torch.bfloat16
+                       ) -> tuple[list[torch.Tensor], PreparedNQA4Activation, torch.Tensor | None, torch.Tensor | None]:
+    """`fused_input_stage` (mode "rmsnorm" / "swiglu") or `attention_output_stage` (mode "attention", the
+    rows then come from `attention_workspace`, a BatchedNQKVAttentionWorkspace whose first stage has run)
+    with the Hadamard rotation, followed by `linear_packed_w4a4_gemv_grouped` of `weights` on the encoded
+    rows, as one launch whose linear workgroups decode their weights while the encoder runs.  Returns
+    (outputs, packed activation, residual sum when `want_residual`, staged rows when `want_staged`): the
+    same bits as the two calls.  `sync` orders the launch among its neighbours on the stream."""
+    if mode not in ("rmsnorm", "swiglu", "attention"):
+        raise ValueError("mode must be 'rmsnorm', 'swiglu' or 'attention'")
+    bf16 = torch.bfloat16
+    if mode == "attention":
+        if attention_workspace is None:
+            raise ValueError("mode 'attention' needs the attention workspace")
+        device = attention_workspace.buffer.device
+        rows, n = attention_workspace.batch_size, attention_workspace.query_heads * attention_workspace.head_dim
+        shape = (rows, n)
+    else:
+        device = _native.require_cuda(inputs)
+        if inputs.dtype != bf16:
+            raise TypeError("the fused input stage takes BF16 tensors")
+        if not inputs.is_contiguous():
+            raise RuntimeError("fused input stage tensors must be contiguous")
+        n = inputs.shape[-1]
+        rows = inputs.numel() // n
+        shape = tuple(inputs.shape)
+        for name, tensor in (("residual", residual), ("gate", gate), ("norm_weight", norm_weight)):
+            if tensor is None:
+                continue
+            if tensor.dtype != bf16:
+                raise TypeError("the fused input stage takes BF16 tensors")
+            if not tensor.is_contiguous():
+                raise RuntimeError("fused input stage tensors must be contiguous")
+            if name != "norm_weight" and tensor.shape != inputs.shape:
+                raise ValueError(f"{name} must have the shape of inputs")
+        if mode == "rmsnorm" and (norm_weight is None or norm_weight.numel() != n):
+            raise ValueError("mode 'rmsnorm' needs a norm weight of the feature size")
+        if mode == "swiglu" and gate is None:
+            raise ValueError("mode 'swiglu' needs the gate rows")
+    if not can_use_fused_stage_linear(rows, n, weights):
+        raise ValueError("rows, K or weights are outside what the fused stage + linear launch takes")
+    if beta_table is None or beta_table.numel() != 4:
+        raise ValueError("encoding needs a table of four betas")
+    if output_dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("outputs are BF16 or float32")
+    lib = _native.library()
+    residual_out = torch.empty(shape, dtype=bf16, device=device) if (want_residual and mode == "rmsnorm") else None
+    staged = torch.empty(shape, dtype=bf16, device=device) if want_staged else None
+    codes = torch.empty(rows * n // 2, dtype=torch.uint8, device=device)
+    beta_ids = torch.empty(rows * n // 32, dtype=torch.uint8, device=device)
+    norms = torch.empty(rows, dtype=torch.float32, device=device)
+    decoded = torch.empty((rows, n), dtype=bf16, device=device)
+    count = len(weights)
+    _, sizes, _, words, tails, w_norms, w_betas, widths, offsets, seeds, _ = _group_plan(weights)
+    outs = [torch.empty((rows, size), dtype=output_dtype, device=device) for size in sizes]
+    flags, previous, previous_words = sync.take(lib.nq_fused_stage_linear_flag_words(rows, n))
+
+    def ptr(tensor):
+        return None if tensor is None else tensor.data_ptr()
+
+    parts = 0 if mode != "attention" else lib.nq_nqkv_attention_parts(rows, attention_workspace.max_pages)
+    _native.check(lib.nq_fused_stage_linear(
+        ptr(inputs) if mode != "attention" else None, rows, n, {"rmsnorm": 1, "swiglu": 2, "attention": 3}[mode],
+        ptr(residual), ptr(residual_out), ptr(norm_weight), float(eps), ptr(gate),
+        attention_workspace.buffer.data_ptr() if mode == "attention" else None,
+        attention_workspace.query_heads if mode == "attention" else 0, parts, ptr(staged), beta_table.data_ptr(), 4,
+        codes.data_ptr(), beta_ids.data_ptr(), norms.data_ptr(), decoded.data_ptr(), count, words, tails, w_norms, w_betas,
+        widths, offsets, seeds, (ctypes.c_void_p * count)(*[o.data_ptr() for o in outs]), _native.dtype_tag(output_dtype),
+        flags, previous, previous_words, sync.status.data_ptr(), sync.spin_limit, _native.stream_handle(device)))
+    activation = PreparedNQA4Activation(
+        code_payload=codes, beta_payload=beta_ids, row_norms=norms, beta_table=beta_table, original_shape=shape, q=14,
+        code_width=4, beta_width=2, output_dtype=bf16, decoded=decoded)
+    return [o.reshape(*shape[:-1], size) for o, size in zip(outs, sizes)], activation, residual_out, staged
+
+
 def _fused_group(activation: PreparedNQA4Activation, weights: Sequence[PreparedNQRTLinear]) -> bool:
     """A group the fused kernel takes in one launch: a prefill below the decode-once size."""
     return (MATRIX_CORE_GEMV_ROWS < activation.token_count < DECODE_ONCE_ROWS and 2 <= len(weights) <= 4
