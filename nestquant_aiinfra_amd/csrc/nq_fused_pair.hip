@@ -101,7 +101,7 @@ __device__ __forceinline__ void load_pieces_device_scope(const uint4 *const (&at
 // All lanes of a consumer workgroup: true once every producer's flag is set, false when the first
 // wavefront's polls ran out (it has then written the status word).  Ends behind a barrier.
 __device__ __forceinline__ bool wait_for_producers(const PairSync &sync, int producers) {
-    __shared__ int ready_shared;
+    __shared__ __align__(16) int ready_shared[4];        // a multiple of 16 bytes, like every static array here
     if (threadIdx.x < 64) {
         int spins = 0;
         bool ready;
@@ -113,12 +113,12 @@ __device__ __forceinline__ bool wait_for_producers(const PairSync &sync, int pro
             __builtin_amdgcn_s_sleep(8);
         }
         if (threadIdx.x == 0) {
-            ready_shared = ready ? 1 : 0;
+            ready_shared[0] = ready ? 1 : 0;
             if (!ready) __hip_atomic_store(sync.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         }
     }
     __syncthreads();
-    return ready_shared != 0;
+    return ready_shared[0] != 0;
 }
 
 constexpr int kPairSubgroup = 256;       // lanes that share a group of channels in the vector form

@@ -278,7 +278,9 @@ row_lanes_encode(const void *__restrict__ x_any, int x_is_f32, int64_t rows, int
                  int beta_count, float sqrt_n, uint32_t *__restrict__ codes, uint8_t *__restrict__ beta_ids,
                  float *__restrict__ norms, uint4 *__restrict__ decoded, int slices, int rotate,
                  const InputPrologue &pro, int block_index) {
-    extern __shared__ float lds[];
+    // 16-byte aligned whatever static LDS the kernel around this code declares: the chains are read 128 bits
+    // at a time, and such reads from an address that is not a multiple of 16 take eight times as long
+    extern __shared__ __align__(16) float lds[];
     const int pitch = chain_pitch(n);
     float *chains = lds;                                  // 8 * pitch floats: the row, transposed
     float *natural = chains + 8 * pitch;                  // n floats: the row in order (rows above 512 values, rotated)
