@@ -63,7 +63,8 @@ def build_w4a4kv4_runner(model: nn.Module, checkpoint: str | Path, *, capacity: 
                          key_betas: Sequence[float] = KEY_BETAS, value_betas: Sequence[float] = VALUE_BETAS,
                          enable_m1_down_splitk: bool = False,
                          fused_decode: bool | None = None, fused_prefill: bool | None = None,
-                         packed_prefill: bool = False, expand_weights: bool = False) -> BatchedNQKVLlamaRunner:
+                         packed_prefill: bool = False, expand_weights: bool = False,
+                         stage_linear_pairs=None) -> BatchedNQKVLlamaRunner:
     """Swap the projections of `model` (BF16, on the GPU, eval mode) for packed W4A4 modules
     read from `checkpoint` and attach a batched NQKV4 cache; returns the runner."""
     reader = NQMCFileReader(checkpoint)
@@ -74,13 +75,14 @@ def build_w4a4kv4_runner(model: nn.Module, checkpoint: str | Path, *, capacity: 
     return attach_w4a4kv4_cache(model, capacity=capacity, max_cache_len=max_cache_len, page_size=page_size,
                                 key_betas=key_betas, value_betas=value_betas, fused_decode=fused_decode,
                                 fused_prefill=fused_prefill, packed_prefill=packed_prefill,
-                                expand_weights=expand_weights)
+                                expand_weights=expand_weights, stage_linear_pairs=stage_linear_pairs)
 
 
 def attach_w4a4kv4_cache(model: nn.Module, *, capacity: int, max_cache_len: int, page_size: int = 16,
                          key_betas: Sequence[float] = KEY_BETAS, value_betas: Sequence[float] = VALUE_BETAS,
                          fused_decode: bool | None = None, fused_prefill: bool | None = None,
-                         packed_prefill: bool = False, expand_weights: bool = False) -> BatchedNQKVLlamaRunner:
+                         packed_prefill: bool = False, expand_weights: bool = False,
+                         stage_linear_pairs=None) -> BatchedNQKVLlamaRunner:
     """A batched NQKV4 cache of `capacity` slots and its runner over a model whose projections are
     already packed modules (an engine of another capacity over the same weights: the packed weights
     are shared, the attention modules point at the newest cache)."""
@@ -94,4 +96,4 @@ def attach_w4a4kv4_cache(model: nn.Module, *, capacity: int, max_cache_len: int,
         packed_prefill=packed_prefill)
     install_batched_nqkv_llama_backend(model, cache)
     return BatchedNQKVLlamaRunner(model, cache, fused_decode=fused_decode, fused_prefill=fused_prefill,
-                                  expand_weights=expand_weights)
+                                  expand_weights=expand_weights, stage_linear_pairs=stage_linear_pairs)

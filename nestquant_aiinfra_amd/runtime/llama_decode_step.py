@@ -37,10 +37,11 @@ import torch
 import torch.nn.functional as F
 
 from .nqkv import attention_output_stage, nqkv_prefill_attention
-from .w4a4_linear import (BF16_ROWS_LINEAR_K, MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, _gemm, _gemv,
-                          bf16_rows_linear, bf16_rows_linear_grouped, can_use_bf16_rows_linear, decode_weight_bf16,
-                          can_use_w4a4_gemm_grouped, fused_input_stage, linear_packed_w4a4_gemm_grouped,
-                          linear_packed_w4a4_gemv_grouped, quantize_activation_cuda, rope_hadamard_pair_cuda)
+from .w4a4_linear import (BF16_ROWS_LINEAR_K, MATRIX_CORE_GEMV_ROWS, PreparedNQRTLinear, StageLinearSync, _gemm, _gemv,
+                          bf16_rows_linear, bf16_rows_linear_grouped, can_use_bf16_rows_linear, can_use_fused_stage_linear,
+                          decode_weight_bf16, can_use_w4a4_gemm_grouped, fused_input_stage, fused_stage_linear,
+                          linear_packed_w4a4_gemm_grouped, linear_packed_w4a4_gemv_grouped, quantize_activation_cuda,
+                          rope_hadamard_pair_cuda)
 
 
 class UnsupportedForFusedDecode(ValueError):
@@ -57,11 +58,21 @@ class FusedLlamaDecodeStep:
     LlamaForCausalLM whose projections are FusedNQRTLinear modules and a BatchedNQKVLlamaCache.
     Raises UnsupportedForFusedDecode at construction for anything else."""
 
-    def __init__(self, model: torch.nn.Module, cache, *, expand_weights: bool = False) -> None:
+    # Which (input stage, linear) pairs of a layer run as one launch (`fused_stage_linear`): the linear's
+    # workgroups decode their weights while the stage's few workgroups are still encoding.  Measured per
+    # pair inside a launch sequence with cold weights (microseconds, two launches -> one, at 1 / 8 rows):
+    # gate and up 24.0 -> 18.1 / 24.1 -> 20.4, down_proj 21.0 -> 16.5 / 23.6 -> 21.8, q, k and v
+    # 11.8 -> 10.7 / 13.3 -> 12.7, o_proj 10.4 -> 10.2 / 12.2 -> 11.3.
+    STAGE_LINEAR_PAIRS = frozenset({"qkv", "o", "gate_up", "down"})
+
+    def __init__(self, model: torch.nn.Module, cache, *, expand_weights: bool = False,
+                 stage_linear_pairs=None) -> None:
         """`expand_weights`: keep, beside every packed projection, the BF16 values its kernels
         multiply by (16 bits per weight in HBM instead of 6) and stream those for steps of up to
         16 rows: the same products without the per-step decode, which is what bounds the packed
-        kernels.  The container on disk and the prefill path are unchanged."""
+        kernels.  The container on disk and the prefill path are unchanged.
+        `stage_linear_pairs`: the pairs that run as one launch (a subset of STAGE_LINEAR_PAIRS, all of
+        them when None, none when empty); same logits bit for bit either way."""
         from ..models.fused_linear import FusedNQRTLinear
 
         inner = getattr(model, "model", None)
@@ -96,6 +107,26 @@ class FusedLlamaDecodeStep:
         self.expand_weights = bool(expand_weights)
         self._expanded: dict[int, tuple] = {}
         self._weights: dict[int, tuple] = {}
+        pairs = self.STAGE_LINEAR_PAIRS if stage_linear_pairs is None else frozenset(stage_linear_pairs)
+        if not pairs <= self.STAGE_LINEAR_PAIRS:
+            raise ValueError(f"stage_linear_pairs must be a subset of {sorted(self.STAGE_LINEAR_PAIRS)}")
+        self.stage_linear_pairs = pairs
+        self._pair_sync: StageLinearSync | None = None
+
+    # -- stage + linear as one launch -------------------------------------------------------------
+    def pairs_failed(self) -> bool:
+        """Whether a consumer of some earlier one-launch pair gave up its bounded wait (its outputs were
+        then not stored).  Reads a word of pinned host memory: no synchronisation."""
+        return self._pair_sync is not None and self._pair_sync.timed_out
+
+    def disable_pairs(self) -> None:
+        """Back to two launches per pair for good (after `pairs_failed`); call with the stream idle."""
+        self.stage_linear_pairs = frozenset()
+        if self._pair_sync is not None:
+            self._pair_sync.reset()
+
+    def _pair(self, name: str, rows: int, k: int, weights) -> bool:
+        return name in self.stage_linear_pairs and can_use_fused_stage_linear(rows, k, weights)
 
     def _rope(self, embedded: torch.Tensor, positions: torch.Tensor, *, padded: bool = False
               ) -> tuple[torch.Tensor, torch.Tensor]:
@@ -195,36 +226,60 @@ class FusedLlamaDecodeStep:
         heads, kv_heads, dim = cache.num_query_heads, cache.num_kv_heads, cache.head_dim
         workspace = cache._workspace(rows, torch.bfloat16)
 
+        sync = None
+        if self.stage_linear_pairs and not (self.expand_weights and rows <= 16):
+            if self._pair_sync is None:
+                self._pair_sync = StageLinearSync(device, sets=4 * len(self.layers))
+            sync = self._pair_sync
+            sync.begin_step()
         delta, residual = embedded.view(rows, self.hidden), None
         for index, (layer, attention, mlp, linears) in enumerate(self.layers):
             q_w, k_w, v_w, o_w, gate_w, up_w, down_w = self._layer_weights(index, device)
             table = linears[0].activation_beta_table
-            activation, residual, _ = fused_input_stage(
-                delta, mode="rmsnorm", residual=residual, norm_weight=layer.input_layernorm.weight,
-                eps=layer.input_layernorm.variance_epsilon, beta_table=table, want_residual=True)
             expanded = self._expanded_layer(index, device) if self.expand_weights and rows <= 16 else None
-            if expanded is not None:
-                query, key, value = bf16_rows_linear_grouped(activation.decoded, expanded[0], expanded[1])
+            if sync is not None and expanded is None and self._pair("qkv", rows, self.hidden, [q_w, k_w, v_w]):
+                (query, key, value), _, residual, _ = fused_stage_linear(
+                    delta, [q_w, k_w, v_w], sync, mode="rmsnorm", residual=residual, norm_weight=layer.input_layernorm.weight,
+                    eps=layer.input_layernorm.variance_epsilon, beta_table=table, want_residual=True)
             else:
-                query, key, value = self._linears(activation, [q_w, k_w, v_w])
+                activation, residual, _ = fused_input_stage(
+                    delta, mode="rmsnorm", residual=residual, norm_weight=layer.input_layernorm.weight,
+                    eps=layer.input_layernorm.variance_epsilon, beta_table=table, want_residual=True)
+                if expanded is not None:
+                    query, key, value = bf16_rows_linear_grouped(activation.decoded, expanded[0], expanded[1])
+                else:
+                    query, key, value = self._linears(activation, [q_w, k_w, v_w])
             # the new token joins the cache inside the attention launch, which leaves per-chunk results;
             # o_proj's input stage merges them as it loads its rows
             manager.append_and_attend(
                 index, query.view(rows, heads, dim), key.view(rows, kv_heads, dim), value.view(rows, kv_heads, dim),
                 attention_scale=float(attention.scaling), workspace=workspace, rotate=True, rope=query_rope,
                 merge=False)
-            o_input, _ = attention_output_stage(workspace, q=14, beta_table=table, hadamard=True)
-            delta = self._linear(o_input, o_w) if expanded is None else bf16_rows_linear(o_input.decoded, expanded[2])
-            activation, residual, _ = fused_input_stage(
-                delta, mode="rmsnorm", residual=residual, norm_weight=layer.post_attention_layernorm.weight,
-                eps=layer.post_attention_layernorm.variance_epsilon, beta_table=table, want_residual=True)
-            if expanded is not None:
-                gate, up = bf16_rows_linear_grouped(activation.decoded, expanded[3], expanded[4])
+            if sync is not None and expanded is None and self._pair("o", rows, heads * dim, [o_w]):
+                (delta,), _, _, _ = fused_stage_linear(None, [o_w], sync, mode="attention", beta_table=table,
+                                                       attention_workspace=workspace)
             else:
-                gate, up = self._linears(activation, [gate_w, up_w])
-            activation, _, _ = fused_input_stage(up, mode="swiglu", gate=gate, beta_table=table)
-            delta = (self._linear(activation, down_w) if expanded is None
-                     else bf16_rows_linear(activation.decoded, expanded[5]))
+                o_input, _ = attention_output_stage(workspace, q=14, beta_table=table, hadamard=True)
+                delta = self._linear(o_input, o_w) if expanded is None else bf16_rows_linear(o_input.decoded, expanded[2])
+            if sync is not None and expanded is None and self._pair("gate_up", rows, self.hidden, [gate_w, up_w]):
+                (gate, up), _, residual, _ = fused_stage_linear(
+                    delta, [gate_w, up_w], sync, mode="rmsnorm", residual=residual,
+                    norm_weight=layer.post_attention_layernorm.weight, eps=layer.post_attention_layernorm.variance_epsilon,
+                    beta_table=table, want_residual=True)
+            else:
+                activation, residual, _ = fused_input_stage(
+                    delta, mode="rmsnorm", residual=residual, norm_weight=layer.post_attention_layernorm.weight,
+                    eps=layer.post_attention_layernorm.variance_epsilon, beta_table=table, want_residual=True)
+                if expanded is not None:
+                    gate, up = bf16_rows_linear_grouped(activation.decoded, expanded[3], expanded[4])
+                else:
+                    gate, up = self._linears(activation, [gate_w, up_w])
+            if sync is not None and expanded is None and self._pair("down", rows, up.shape[-1], [down_w]):
+                (delta,), _, _, _ = fused_stage_linear(up, [down_w], sync, mode="swiglu", gate=gate, beta_table=table)
+            else:
+                activation, _, _ = fused_input_stage(up, mode="swiglu", gate=gate, beta_table=table)
+                delta = (self._linear(activation, down_w) if expanded is None
+                         else bf16_rows_linear(activation.decoded, expanded[5]))
         _, _, normed = fused_input_stage(delta, mode="rmsnorm", residual=residual, norm_weight=inner.norm.weight,
                                          eps=inner.norm.variance_epsilon, encode=False, want_staged=True)
         return self._lm_head(normed.view(rows, self.hidden)).view(rows, 1, -1)

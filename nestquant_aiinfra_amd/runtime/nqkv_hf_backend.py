@@ -371,11 +371,12 @@ class BatchedNQKVLlamaRunner:
 
     def __init__(self, model: torch.nn.Module, cache: BatchedNQKVLlamaCache, *,
                  fused_decode: bool | None = None, fused_prefill: bool | None = None,
-                 expand_weights: bool = False) -> None:
-        """`fused_decode` / `fused_prefill`: run decode steps through FusedLlamaDecodeStep (ten
-        launches per layer) and prompts through FusedLlamaPrefillStep instead of the module
-        graph; None = whenever the model qualifies.  `expand_weights`: the fused decode step keeps
-        and streams BF16 copies of the projection weights (see FusedLlamaDecodeStep)."""
+                 expand_weights: bool = False, stage_linear_pairs=None) -> None:
+        """`fused_decode` / `fused_prefill`: run decode steps through FusedLlamaDecodeStep and prompts
+        through FusedLlamaPrefillStep instead of the module graph; None = whenever the model
+        qualifies.  `expand_weights`: the fused decode step keeps and streams BF16 copies of the
+        projection weights; `stage_linear_pairs`: which input stages share a launch with their
+        linears (see FusedLlamaDecodeStep; None = all, () = none)."""
         if not isinstance(model, torch.nn.Module):
             raise TypeError("model must be a torch module")
         if not isinstance(cache, BatchedNQKVLlamaCache):
@@ -396,7 +397,8 @@ class BatchedNQKVLlamaRunner:
         if fused_decode is None or fused_decode:
             from .llama_decode_step import FusedLlamaDecodeStep, UnsupportedForFusedDecode
             try:
-                self.fused_step = FusedLlamaDecodeStep(model, cache, expand_weights=expand_weights)
+                self.fused_step = FusedLlamaDecodeStep(model, cache, expand_weights=expand_weights,
+                                                       stage_linear_pairs=stage_linear_pairs)
             except UnsupportedForFusedDecode:
                 if fused_decode:
                     raise
@@ -558,6 +560,20 @@ class BatchedNQKVLlamaRunner:
         self.release_slots(slot_mask.nonzero(as_tuple=False).flatten().cpu().tolist())
 
     # -- decode --------------------------------------------------------------------------------
+    def _check_pairs(self) -> None:
+        """A one-launch (input stage + linear) pair whose consumers gave up waiting for the encoder has
+        left outputs unwritten in some earlier step.  The step goes back to two launches per pair for
+        good, the captured graphs (which hold the one-launch form) are dropped, and the caller is told."""
+        step = self.fused_step
+        if step is not None and step.pairs_failed():
+            torch.cuda.synchronize(self.device)
+            step.disable_pairs()
+            self._graphs.clear()
+            self._greedy.clear()
+            self._decode_state = None
+            raise RuntimeError("a fused input stage + linear launch gave up waiting for its encoder: results since the "
+                               "last check are invalid; decode steps now use two launches per pair (capture again)")
+
     def _step(self, tokens: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
         if self.fused_step is not None:
             return self.fused_step(tokens, positions, advance=True)
@@ -569,6 +585,7 @@ class BatchedNQKVLlamaRunner:
     def decode_eager(self, tokens: torch.Tensor, *, slots: Sequence[int], positions: torch.Tensor) -> torch.Tensor:
         """One un-captured decode step for `slots` (tokens, positions: [rows, 1])."""
         rows = len(slots)
+        self._check_pairs()
         self.cache.require_room(slots)
         self._decode_state = None
         self.cache.set_decode_execution_state(
@@ -649,6 +666,7 @@ class BatchedNQKVLlamaRunner:
             return full
         if slots is None:
             raise ValueError("decode needs slots (or active_mask and valid_lengths)")
+        self._check_pairs()
         rows = len(slots)
         width = next((w for w in sorted(self._graphs) if w >= rows), None)
         if width is None:
@@ -680,6 +698,7 @@ class BatchedNQKVLlamaRunner:
         rows = len(slots)
         if isinstance(steps, bool) or not isinstance(steps, int) or not 1 <= steps <= self.GREEDY_HISTORY_STEPS:
             raise ValueError(f"steps must be an integer in [1, {self.GREEDY_HISTORY_STEPS}]")
+        self._check_pairs()
         width = next((w for w in sorted(self._graphs) if w >= rows), None)
         if width is None:
             raise RuntimeError("decode_greedy needs a captured graph of this width: call capture() first")

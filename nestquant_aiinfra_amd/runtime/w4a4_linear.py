@@ -714,27 +714,42 @@ def _group_plan(weights: Sequence[PreparedNQRTLinear]) -> tuple:
 
 
 class StageLinearSync:
-    """The hand-over state of `fused_stage_linear` launches that follow each other on one stream:
-    a ring of flag-word sets (each launch takes the next set and clears the one before it), the
-    status word a consumer sets when its bounded wait runs out (pinned host memory, so that the
-    host can look at it without a synchronisation), and the number of polls of that wait."""
+    """The hand-over state of `fused_stage_linear` launches on one stream: sets of flag words (one
+    set per launch), the status word a consumer sets when its bounded wait runs out (pinned host
+    memory: the host looks at it without a synchronisation), and the number of polls of that wait.
+
+    Two ways to hand out the sets.  A caller that issues a fixed sequence of launches again and
+    again (a decode step, also as a captured graph) calls `begin_step()` first: one fill clears
+    every set, and the launches of the step take sets 0, 1, ... .  Without `begin_step` the sets
+    form a ring in which every launch clears the set of the launch before it."""
 
     FLAG_WORDS = 256          # words per set: the most producer workgroups a launch has
 
     def __init__(self, device: torch.device, *, sets: int = 128, spin_limit: int = 400_000) -> None:
         if sets < 2:
-            raise ValueError("the ring needs at least two sets of flag words")
+            raise ValueError("at least two sets of flag words")
         self.flags = torch.zeros((sets, self.FLAG_WORDS), dtype=torch.int32, device=device)
         self.status = torch.zeros(1, dtype=torch.int32).pin_memory()
         self.spin_limit = int(spin_limit)
         self._next = 0
-        self._previous: tuple[int, int] | None = None       # (set, words) of the launch before
+        self._previous: tuple[int, int] | None = None       # (set, words) of the launch before, ring form
+        self._in_step = False
+
+    def begin_step(self) -> None:
+        """Clear every set with one fill (capturable) and hand the sets out from the first again."""
+        self.flags.zero_()
+        self._next, self._previous, self._in_step = 0, None, True
 
     def take(self, words: int) -> tuple[int, int | None, int]:
-        """(pointer to this launch's flag words, pointer to the previous launch's or None, their count)."""
+        """(pointer to this launch's flag words, pointer to the words this launch clears or None, their count)."""
         if not 1 <= words <= self.FLAG_WORDS:
             raise ValueError("a launch has between 1 and 256 producer workgroups")
         current = self._next
+        if self._in_step:
+            if current >= self.flags.shape[0]:
+                raise RuntimeError("more launches in a step than sets of flag words")
+            self._next = current + 1
+            return self.flags[current].data_ptr(), None, 0
         self._next = (current + 1) % self.flags.shape[0]
         previous = self._previous
         self._previous = (current, words)
@@ -743,23 +758,15 @@ class StageLinearSync:
             return here, None, 0
         return here, self.flags[previous[0]].data_ptr(), previous[1]
 
-    def position(self) -> tuple[int, tuple[int, int] | None]:
-        return self._next, self._previous
-
-    def rewind(self, position: tuple[int, tuple[int, int] | None]) -> None:
-        """Back to an earlier point of the ring: a captured graph replays the launches recorded from
-        that point on, so whatever is launched after the capture must continue where the graph ends."""
-        self._next, self._previous = position
-
     @property
     def timed_out(self) -> bool:
         return bool(self.status[0].item())
 
     def reset(self) -> None:
-        """After a time-out (or before a capture): every flag word and the status back to zero."""
+        """After a time-out: every flag word and the status back to zero (the stream must be idle)."""
         self.flags.zero_()
         self.status.zero_()
-        self._next, self._previous = 0, None
+        self._next, self._previous, self._in_step = 0, None, False
 
 
 def can_use_fused_stage_linear(rows: int, k: int, weights: Sequence[PreparedNQRTLinear]) -> bool:

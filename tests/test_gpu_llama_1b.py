@@ -282,3 +282,52 @@ def test_engine_workload_at_full_size_graph_equals_eager(llama_1b_model, capacit
                 token = out[:, 0].argmax(-1).reshape(1, 1)
         assert alone == graph_tokens["request-0"]
         runner.release_slots([0])
+
+
+def test_stage_and_linear_pairs_give_the_same_step_and_fail_closed(llama_1b_model):
+    """At this size every input stage of a decode step shares a launch with the linear(s) behind it
+    (nq_fused_stage_linear).  The step must give the logits and the cache of the step that launches
+    them separately, bit for bit, eager and captured; and when the consumers' bounded wait is made to
+    run out, the next call raises, the runner drops to two launches per pair for good, and goes on."""
+    from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
+    model, _ = llama_1b_model
+    g = torch.Generator().manual_seed(5201)
+    lengths = [29, 14, 40]
+    ids = torch.randint(0, VOCAB, (3, max(lengths)), generator=g).cuda()
+    start = torch.tensor(lengths, device="cuda").reshape(3, 1)
+
+    def run(pairs, steps=6, graph=False):
+        runner = asm.attach_w4a4kv4_cache(model, capacity=4, max_cache_len=64, stage_linear_pairs=pairs)
+        slots = [2, 0, 3]
+        logits = runner.prefill_slots(ids, slots=slots, lengths=lengths, last_token_logits=True)
+        token, position, outs = logits[:, 0].argmax(-1).reshape(3, 1), start, []
+        if graph:
+            runner.capture()
+        for _ in range(steps):
+            out = (runner.decode if graph else runner.decode_eager)(token, slots=slots, positions=position)
+            outs.append(out.clone())
+            token, position = out[:, 0].argmax(-1).reshape(3, 1), position + 1
+        return runner, torch.stack(outs), [t.clone() for t in _cache_tensors(runner.cache)]
+
+    plain_runner, plain, plain_state = run(())
+    assert plain_runner.fused_step.stage_linear_pairs == frozenset() and plain_runner.fused_step._pair_sync is None
+    for graph in (False, True):
+        runner, paired, state = run(None, graph=graph)
+        assert runner.fused_step.stage_linear_pairs == {"qkv", "o", "gate_up", "down"}
+        assert runner.fused_step._pair_sync is not None and not runner.fused_step.pairs_failed()
+        assert torch.equal(paired, plain)
+        assert all(torch.equal(a, b) for a, b in zip(state, plain_state))
+
+    # the failure path: with no polls allowed the consumers that look before their encoder is done give up
+    runner.fused_step._pair_sync.spin_limit = 0
+    token = torch.zeros((3, 1), dtype=torch.long, device="cuda")
+    position = start + 6
+    runner.decode_eager(token, slots=[2, 0, 3], positions=position)              # eager: the new limit takes effect
+    torch.cuda.synchronize()
+    assert runner.fused_step.pairs_failed()
+    with pytest.raises(RuntimeError, match="gave up waiting"):
+        runner.decode(token, slots=[2, 0, 3], positions=position + 1)
+    assert runner.fused_step.stage_linear_pairs == frozenset() and not runner.graph_captured
+    assert not runner.fused_step.pairs_failed()
+    again = runner.decode(token, slots=[2, 0, 3], positions=position + 1)         # two launches per pair, un-captured
+    assert torch.isfinite(again).all()
