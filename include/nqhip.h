@@ -508,7 +508,10 @@ int nq_attention_output_stage(const void *workspace_dev, int64_t rows, int q_hea
  * rows * slices workgroups of the grid run the encoder; the others decode their weights while the
  * encoder is still busy, wait until every encoder workgroup has set its flag word, and then
  * multiply.  rows in [1, 16] (8 for n = 8192), n = K in {2048, 8192}, four betas.
- *   flags_dev            nq_fused_stage_linear_flag_words(rows, n) words of device memory, zero when
+ *   flags_dev            nq_fused_stage_linear_flag_words(rows, n) words of device memory, 16-byte
+ *                        aligned (the library keeps several copies of a launch's flags, each in a
+ *                        memory channel of its own, because every consumer polls them at once; a poll
+ *                        reads four words per lane), zero when
  *                        the launch starts and owned by it until the next launch on the stream that
  *                        names them as previous_flags_dev (which clears them) has finished;
  *   previous_flags_dev   the flag words of the launch before this one on the same stream (any

@@ -31,10 +31,34 @@
 
 #include <math.h>
 
+#ifdef NQ_PHASE_STAMPS
+// Measuring builds only: lane 0 of the first and last producer and of the first and last consumer
+// (slots 0 to 3, eight stamps each) leave the 100 MHz wall clock at their phase boundaries.
+namespace nq { __device__ unsigned long long g_pair_stamps[32]; }
+#define NQ_PAIR_STAMP(slot, i) do { if ((slot) >= 0 && threadIdx.x == 0) nq::g_pair_stamps[(slot) * 8 + (i)] = wall_clock64(); } while (0)
+extern "C" int nq_debug_pair_stamps(unsigned long long *out32) {
+    if (hipDeviceSynchronize() != hipSuccess) return NQ_ERR_LAUNCH;
+    return hipMemcpyFromSymbol(out32, HIP_SYMBOL(nq::g_pair_stamps), 32 * sizeof(unsigned long long)) == hipSuccess
+               ? NQ_OK : NQ_ERR_LAUNCH;
+}
+#else
+#define NQ_PAIR_STAMP(slot, i) do { } while (0)
+#endif
+
 namespace nq {
 
+// Every consumer workgroup polls the flags at once, and polls of one cache line queue up at the one
+// memory channel that holds it: the flag words therefore exist in kFlagCopies copies, kFlagStride words
+// apart, a producer sets its word in all of them (one store instruction) and consumer g reads copy
+// g % kFlagCopies.
+#ifndef NQ_PAIR_FLAG_COPIES
+#define NQ_PAIR_FLAG_COPIES 16
+#endif
+constexpr int kFlagCopies = NQ_PAIR_FLAG_COPIES;
+constexpr int kFlagStride = 256;         // words: the most producer workgroups a launch has
+
 struct PairSync {
-    uint32_t *flags;         // one word per producer workgroup of this launch, zero when it starts
+    uint32_t *flags;         // kFlagCopies x kFlagStride words, one per producer workgroup and copy, zero when the launch starts
     uint32_t *previous;      // the flag words of the launch before this one on the stream (cleared here), or null
     int previous_count;
     uint32_t *status;        // set to 1 when a consumer's wait runs out (device or pinned host memory)
@@ -99,18 +123,28 @@ __device__ __forceinline__ void load_pieces_device_scope(const uint4 *const (&at
 }
 
 // All lanes of a consumer workgroup: true once every producer's flag is set, false when the first
-// wavefront's polls ran out (it has then written the status word).  Ends behind a barrier.
+// wavefront's polls ran out (it has then written the status word).  Ends behind a barrier.  A poll is
+// one 16-byte load per lane: four flag words each, so that the up to 256 flags of a launch cost one
+// trip to memory per poll (a load per flag and lane in turn made a poll of 256 flags four trips long).
 __device__ __forceinline__ bool wait_for_producers(const PairSync &sync, int producers) {
     __shared__ __align__(16) int ready_shared[4];        // a multiple of 16 bytes, like every static array here
     if (threadIdx.x < 64) {
+        const int first = 4 * (int)threadIdx.x;
+        const uint32_t *flags = sync.flags + ((int)blockIdx.x % kFlagCopies) * kFlagStride;
+        const bool polls = first < producers;             // the flag words come in multiples of four
         int spins = 0;
         bool ready;
         for (;;) {
             bool mine = true;
-            for (int p = (int)threadIdx.x; p < producers; p += 64) mine = mine && load_word_device_scope(sync.flags + p) != 0u;
+            if (polls) {
+                u32x4 four;
+                asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
+                             : "=&v"(four) : "v"(flags + first) : "memory");
+                mine = four.x != 0u && four.y != 0u && four.z != 0u && four.w != 0u;
+            }
             ready = __builtin_amdgcn_ballot_w64(!mine) == 0;
             if (ready || ++spins > sync.spin_limit) break;
-            __builtin_amdgcn_s_sleep(8);
+            __builtin_amdgcn_s_sleep(4);
         }
         if (threadIdx.x == 0) {
             ready_shared[0] = ready ? 1 : 0;
@@ -130,6 +164,8 @@ __device__ __forceinline__ void
 consume_on_vector_units(const uint4 *__restrict__ act, const GemvWeights &w, int which, int group, int m_rows, int k_size,
                         float sqrt_k, int out_is_f32, const PairSync &sync, int producers) {
     __shared__ float partial[4][16][R][MT];
+    [[maybe_unused]] const int stamp_slot = (int)blockIdx.x == producers ? 2 : ((int)blockIdx.x == (int)gridDim.x - 1 ? 3 : -1);
+    NQ_PAIR_STAMP(stamp_slot, 0);
     const int tid = threadIdx.x, sub = tid >> 8, t = tid & 255;
     const int subgroups = (int)blockDim.x >> 8;
     const int blocks_per_row = k_size >> 3;
@@ -180,7 +216,9 @@ consume_on_vector_units(const uint4 *__restrict__ act, const GemvWeights &w, int
         }
     }
 
+    NQ_PAIR_STAMP(stamp_slot, 1);
     const bool ready = wait_for_producers(sync, producers);
+    NQ_PAIR_STAMP(stamp_slot, 2);
 
     float acc[R][MT];
 #pragma unroll
@@ -216,6 +254,7 @@ consume_on_vector_units(const uint4 *__restrict__ act, const GemvWeights &w, int
             }
         }
     }
+    NQ_PAIR_STAMP(stamp_slot, 3);
     // sums over the 16 lanes of every row with register-only lane exchanges, then rows in index order
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -237,6 +276,7 @@ consume_on_vector_units(const uint4 *__restrict__ act, const GemvWeights &w, int
             else reinterpret_cast<uint16_t *>(w.out[which])[(int64_t)m * n_size + n] = f32_to_bf16(total);
         }
     }
+    NQ_PAIR_STAMP(stamp_slot, 4);
 }
 
 // Matrix-core consumer (w4a4_gemv_mfma_kernel<1>'s products and sums): a tile of 16 channels.  The
@@ -249,6 +289,8 @@ consume_on_matrix_cores(const uint4 *__restrict__ act, const GemvWeights &w, int
                         float sqrt_k, int out_is_f32, const PairSync &sync, int producers) {
     static_assert(kVirtualPerWave * kStepsPerVirtual == 4, "a lane holds sixteen decoded blocks");
     __shared__ float part[16][256];
+    [[maybe_unused]] const int stamp_slot = (int)blockIdx.x == producers ? 2 : ((int)blockIdx.x == (int)gridDim.x - 1 ? 3 : -1);
+    NQ_PAIR_STAMP(stamp_slot, 0);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = (int)blockDim.x >> 6;
     const int virtual_waves = waves * kVirtualPerWave;
     const int n_size = w.n[which], n0 = tile * 16;
@@ -295,7 +337,9 @@ consume_on_matrix_cores(const uint4 *__restrict__ act, const GemvWeights &w, int
         }
     }
 
+    NQ_PAIR_STAMP(stamp_slot, 1);
     const bool ready = wait_for_producers(sync, producers);
+    NQ_PAIR_STAMP(stamp_slot, 2);
 
     if (ready) {
         const bool has_token = column < m_rows;
@@ -304,18 +348,21 @@ consume_on_matrix_cores(const uint4 *__restrict__ act, const GemvWeights &w, int
         // the activation fragments of two pieces at a time (32 registers beside the 64 of decoded weights)
 #pragma unroll
         for (int half = 0; half < 2; half++) {
+            // lanes whose column is no token of this launch request nothing and multiply zeros
             u32x4 b[2][4];
-            load_2x4_device_scope(act_row + 16 * piece(2 * half), act_row + 16 * piece(2 * half + 1), b);
+#pragma unroll
+            for (int pair = 0; pair < 2; pair++)
+#pragma unroll
+                for (int t = 0; t < 4; t++) b[pair][t] = u32x4{0u, 0u, 0u, 0u};
+            if (has_token) load_2x4_device_scope(act_row + 16 * piece(2 * half), act_row + 16 * piece(2 * half + 1), b);
 #pragma unroll
             for (int pair = 0; pair < 2; pair++) {
                 const int e = 2 * half + pair;
                 if (e % kStepsPerVirtual == 0) acc = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    const u32x4 token = has_token ? b[pair][t] : u32x4{0u, 0u, 0u, 0u};
+                for (int t = 0; t < 4; t++)
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_fragment[e][t]),
-                                                                  __builtin_bit_cast(bf16x8, token), acc, 0, 0, 0);
-                }
+                                                                  __builtin_bit_cast(bf16x8, b[pair][t]), acc, 0, 0, 0);
                 if (e % kStepsPerVirtual == kStepsPerVirtual - 1) {
 #pragma unroll
                     for (int i = 0; i < 4; i++)
@@ -324,6 +371,7 @@ consume_on_matrix_cores(const uint4 *__restrict__ act, const GemvWeights &w, int
             }
         }
     }
+    NQ_PAIR_STAMP(stamp_slot, 3);
     __syncthreads();
     if (ready && tid < 256) {
         const int channel = tid >> 4, token = tid & 15;
@@ -335,6 +383,7 @@ consume_on_matrix_cores(const uint4 *__restrict__ act, const GemvWeights &w, int
             else reinterpret_cast<uint16_t *>(w.out[which])[at] = f32_to_bf16(total);
         }
     }
+    NQ_PAIR_STAMP(stamp_slot, 4);
 }
 
 struct EncoderArgs {
@@ -355,20 +404,32 @@ struct EncoderArgs {
 // kConsumer: 0 = vector units (MT rows, R channels per subgroup), 1 = matrix cores.
 template <int kPrologue, int kForm, int kConsumer, int MT, int R>
 __global__ void __launch_bounds__(kForm == kFirstLanes ? 1024 : 256)
-fused_stage_linear_kernel(EncoderArgs e, GemvWeights w, int producers, int m_rows, float sqrt_k, int out_is_f32, PairSync sync) {
+fused_stage_linear_kernel(EncoderArgs e, GemvWeights w, int producers, int late_first, int late_count, int m_rows,
+                          float sqrt_k, int out_is_f32, PairSync sync) {
     const int block = (int)blockIdx.x;
+    int group = block - producers;
     if (block < producers) {
         __builtin_amdgcn_s_setprio(3);           // a chain of latencies that the consumers' vector work would stretch
-        if (block == 0 && sync.previous)
-            for (int i = (int)threadIdx.x; i < sync.previous_count; i += (int)blockDim.x) sync.previous[i] = 0u;
+        [[maybe_unused]] const int stamp_slot = block == 0 ? 0 : (block == producers - 1 ? 1 : -1);
+        NQ_PAIR_STAMP(stamp_slot, 0);
         row_lanes_encode<kPrologue, kForm, true>(e.x, 0, e.rows, e.n, e.betas, e.beta_count, e.sqrt_n, e.codes, e.beta_ids,
                                                  e.norms, e.decoded, e.slices, e.rotate, e.prologue, block);
+        NQ_PAIR_STAMP(stamp_slot, 1);
         __builtin_amdgcn_s_waitcnt(0);           // this wavefront's write-through stores have been acknowledged
+        NQ_PAIR_STAMP(stamp_slot, 2);
         __syncthreads();
-        if (threadIdx.x == 0) store_word_device_scope(sync.flags + block, 1u);
-        return;
+        NQ_PAIR_STAMP(stamp_slot, 3);
+        if (threadIdx.x < kFlagCopies) store_word_device_scope(sync.flags + (int)threadIdx.x * kFlagStride + block, 1u);
+        // the groups of channels that found no free slot beside the others are the producers' second job
+        if (block >= late_count) return;
+        __builtin_amdgcn_s_setprio(0);
+        group = late_first + block;
     }
-    int group = block - producers, which = 0;
+    // the flag words of the launch before this one (finished: it came earlier on the stream) are cleared
+    // by a workgroup that has time to spare: the first consumer
+    if (block == producers && sync.previous)
+        for (int i = (int)threadIdx.x; i < sync.previous_count; i += (int)blockDim.x) sync.previous[i] = 0u;
+    int which = 0;
 #pragma unroll
     for (int i = 1; i < kGemvMaxGroup; i++)
         if (i < w.count && group >= w.first_group[i]) which = i;
@@ -394,9 +455,9 @@ bool pair_takes_matrix_cores(int m, int64_t total_n) { return m >= 5 || total_n 
 
 template <int kPrologue, int kForm>
 int launch_pair(const nq::EncoderArgs &e, const nq::GemvWeights &w, int consumer, int m_tile, int r, int producers,
-                int consumers, int m, float sqrt_k, int out_is_f32, const nq::PairSync &sync, size_t lds_bytes,
+                int consumers, int late, int m, float sqrt_k, int out_is_f32, const nq::PairSync &sync, size_t lds_bytes,
                 hipStream_t stream) {
-    using Kernel = void (*)(nq::EncoderArgs, nq::GemvWeights, int, int, float, int, nq::PairSync);
+    using Kernel = void (*)(nq::EncoderArgs, nq::GemvWeights, int, int, int, int, float, int, nq::PairSync);
     Kernel kernel = nullptr;
 #define NQ_PAIR(C, MT, R) (Kernel)nq::fused_stage_linear_kernel<kPrologue, kForm, C, MT, R>
     if (consumer == 1) kernel = NQ_PAIR(1, 1, 1);
@@ -410,16 +471,21 @@ int launch_pair(const nq::EncoderArgs &e, const nq::GemvWeights &w, int consumer
             return nq::fail(NQ_ERR_LAUNCH, "nq_fused_stage_linear: cannot reserve %zu bytes of LDS: %s", lds_bytes,
                             hipGetErrorString(status));
     }
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(producers + consumers)), dim3(e.n / 8), lds_bytes, stream, e, w, producers, m,
-                       sqrt_k, out_is_f32, sync);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(producers + consumers - late)), dim3(e.n / 8), lds_bytes, stream, e, w,
+                       producers, consumers - late, late, m, sqrt_k, out_is_f32, sync);
     return nq::check_launch("nq_fused_stage_linear");
 }
 
 }  // namespace
 
+namespace {
+// encoder workgroups of a launch: rows x slices (a multiple of four, at most 256)
+int pair_producers(int64_t rows, int64_t n) { return (int)(rows * (n > 4096 ? n / 512 : (rows * 32 <= 256 ? 32 : 16))); }
+}  // namespace
+
 extern "C" int nq_fused_stage_linear_flag_words(int64_t rows, int64_t n) {
     if (rows < 1 || rows > 16 || (n != 2048 && n != 8192)) return 0;
-    return (int)(rows * (n > 4096 ? n / 512 : (rows * 32 <= 256 ? 32 : 16)));
+    return nq::kFlagCopies * nq::kFlagStride;
 }
 
 extern "C" int nq_fused_stage_linear(
@@ -454,10 +520,11 @@ extern "C" int nq_fused_stage_linear(
                    weight_seeds && out_dev, NQ_ERR_ARGUMENT, "nq_fused_stage_linear: null argument array");
     NQ_REQUIRE(out_dtype == NQ_F32 || out_dtype == NQ_BF16, NQ_ERR_ARGUMENT,
                "nq_fused_stage_linear: output dtype tag %d is not F32 or BF16", out_dtype);
-    NQ_REQUIRE(flags_dev && status_dev && nq::aligned(flags_dev, 4) && nq::aligned(previous_flags_dev, 4) &&
-                   nq::aligned(status_dev, 4), NQ_ERR_ARGUMENT, "nq_fused_stage_linear: needs flag words and a status word");
-    NQ_REQUIRE(previous_flag_words >= 0 && previous_flag_words <= 1024 && (previous_flag_words == 0 || previous_flags_dev),
-               NQ_ERR_ARGUMENT, "nq_fused_stage_linear: at most 1024 flag words of the launch before");
+    NQ_REQUIRE(flags_dev && status_dev && nq::aligned(flags_dev, 16) && nq::aligned(previous_flags_dev, 4) &&
+                   nq::aligned(status_dev, 4), NQ_ERR_ARGUMENT,
+               "nq_fused_stage_linear: needs flag words (16-byte aligned) and a status word");
+    NQ_REQUIRE(previous_flag_words >= 0 && previous_flag_words <= 65536 && (previous_flag_words == 0 || previous_flags_dev),
+               NQ_ERR_ARGUMENT, "nq_fused_stage_linear: at most 65536 flag words of the launch before");
     NQ_REQUIRE(spin_limit >= 0, NQ_ERR_ARGUMENT, "nq_fused_stage_linear: spin_limit must not be negative");
 
     const int k = (int)n;
@@ -469,7 +536,7 @@ extern "C" int nq_fused_stage_linear(
     const int m = (int)rows;
     NQ_REQUIRE(n != 8192 || m <= 8, NQ_ERR_SHAPE, "nq_fused_stage_linear: rows of 8192 values come at most eight at a time");
     const int consumer = pair_takes_matrix_cores(m, total_n) ? 1 : 0;
-    const int producers = nq_fused_stage_linear_flag_words(rows, n);
+    const int producers = pair_producers(rows, n);
     const int slices = producers / m;
     const int lanes = k / 8, subgroups = lanes / nq::kPairSubgroup;
     // Every workgroup of the launch must be resident at once: a consumer that started after another
@@ -531,6 +598,10 @@ extern "C" int nq_fused_stage_linear(
         e.prologue.parts = parts;
         e.prologue.heads = q_heads;
     }
+    // Groups of channels beyond the slots of the chip would start when others finish and pay their
+    // whole decode behind the rest of the launch: as many of them as there are producers become the
+    // producers' second job (an encoder workgroup is done long before the first consumer).
+    const int late = groups + producers > slots ? (groups + producers - slots < producers ? groups + producers - slots : producers) : 0;
     nq::PairSync sync{flags_dev, previous_flags_dev, previous_flag_words, status_dev, spin_limit};
     const size_t lds_bytes = (size_t)(8 * ((k >> 3) + 8) + k + 4 + 8) * sizeof(float);
     const float sqrt_k = (float)sqrt((double)k);
@@ -538,7 +609,7 @@ extern "C" int nq_fused_stage_linear(
     const int out_is_f32 = out_dtype == NQ_F32;
     hipStream_t s = (hipStream_t)stream;
 #define NQ_LAUNCH_PAIR(PRO, FORM) \
-    launch_pair<PRO, FORM>(e, w, consumer, m_tile, r, producers, groups, m, sqrt_k, out_is_f32, sync, lds_bytes, s)
+    launch_pair<PRO, FORM>(e, w, consumer, m_tile, r, producers, groups, late, m, sqrt_k, out_is_f32, sync, lds_bytes, s)
     if (k == 8192) {
         if (mode == 1) return NQ_LAUNCH_PAIR(1, nq::kFirstLanes);
         if (mode == 2) return NQ_LAUNCH_PAIR(2, nq::kFirstLanes);

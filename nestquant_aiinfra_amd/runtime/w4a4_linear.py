@@ -723,12 +723,12 @@ class StageLinearSync:
     every set, and the launches of the step take sets 0, 1, ... .  Without `begin_step` the sets
     form a ring in which every launch clears the set of the launch before it."""
 
-    FLAG_WORDS = 256          # words per set: the most producer workgroups a launch has
-
     def __init__(self, device: torch.device, *, sets: int = 128, spin_limit: int = 400_000) -> None:
         if sets < 2:
             raise ValueError("at least two sets of flag words")
-        self.flags = torch.zeros((sets, self.FLAG_WORDS), dtype=torch.int32, device=device)
+        # words per set: what the largest launch asks for (the library keeps several copies of a launch's flags)
+        self.set_words = int(_native.library().nq_fused_stage_linear_flag_words(16, 2048))
+        self.flags = torch.zeros((sets, self.set_words), dtype=torch.int32, device=device)
         self.status = torch.zeros(1, dtype=torch.int32).pin_memory()
         self.spin_limit = int(spin_limit)
         self._next = 0
@@ -742,8 +742,8 @@ class StageLinearSync:
 
     def take(self, words: int) -> tuple[int, int | None, int]:
         """(pointer to this launch's flag words, pointer to the words this launch clears or None, their count)."""
-        if not 1 <= words <= self.FLAG_WORDS:
-            raise ValueError("a launch has between 1 and 256 producer workgroups")
+        if not 1 <= words <= self.set_words:
+            raise ValueError(f"a launch takes between 1 and {self.set_words} flag words")
         current = self._next
         if self._in_step:
             if current >= self.flags.shape[0]:
