@@ -130,7 +130,7 @@ def build_workload(device):
         record = rt.quantize_weight_nqrt4(w, q=Q, betas=WEIGHT_BETAS, dither_seed=dseed, tensor_name=name)
         base = rt.prepare_fused_linear(record, device=device)
         weights = [base] + [
-            rt.PreparedNQRTLinear(record, base.code_payload.clone(), base.beta_payload.clone(),
+            rt.PreparedNQRTLinear(record, None, None,
                                   base.row_norms.clone(), base.beta_table.clone(),
                                   None if base.resolved_words is None else base.resolved_words.clone(),
                                   None if base.resolved_tails is None else base.resolved_tails.clone())
@@ -317,7 +317,7 @@ def prefill_gemm_extra(rt, device):
         record = rt.quantize_weight_nqrt4(w, q=Q, betas=WEIGHT_BETAS, dither_seed=dseed, tensor_name=name)
         base = rt.prepare_fused_linear(record, device=device)
         copies = 32
-        weights = [base] + [rt.PreparedNQRTLinear(record, base.code_payload.clone(), base.beta_payload.clone(),
+        weights = [base] + [rt.PreparedNQRTLinear(record, None, None,
                                                   base.row_norms, base.beta_table,
                                                   None if base.resolved_words is None else base.resolved_words.clone(),
                                                   None if base.resolved_tails is None else base.resolved_tails.clone())

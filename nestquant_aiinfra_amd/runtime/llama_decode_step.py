@@ -160,7 +160,7 @@ class FusedLlamaDecodeStep:
         and kept while the modules still hold them on this device."""
         linears = self.layers[index][3]
         kept = self._weights.get(index)
-        if (kept is None or kept[0].code_payload.device != device
+        if (kept is None or kept[0].device != device
                 or not all(weight is linear._prepared for weight, linear in zip(kept, linears))):
             kept = self._weights[index] = tuple(self._prepared(linear, device) for linear in linears)
         return kept

@@ -65,15 +65,28 @@ class PreparedNQRTLinear:
     """GPU-resident packed streams and metadata of one NQRT4 weight."""
 
     record: Any          # PackedNestQuantTensor (ours or the reference's: same attributes)
-    code_payload: torch.Tensor
-    beta_payload: torch.Tensor
+    # The NQRT4 streams on the device, or None once the resolved form has replaced them (the record
+    # still holds them on the host; `prepare_fused_linear(..., keep_streams=True)` keeps both).
+    code_payload: torch.Tensor | None
+    beta_payload: torch.Tensor | None
     row_norms: torch.Tensor
     beta_table: torch.Tensor
     # Optional resolved form (int32 word + int16 tail per 8-weight block): the lattice point
     # each block's decode lands on, found once here so that the linear kernels need neither
-    # lattice search.  6 bits per weight on top of (or instead of) the 4.25-bit streams.
+    # lattice search.  6 bits per weight instead of (or, with keep_streams, beside) the 4.25-bit streams.
     resolved_words: torch.Tensor | None = None
     resolved_tails: torch.Tensor | None = None
+
+    @property
+    def device(self) -> torch.device:
+        return self.row_norms.device
+
+    @property
+    def resident_bytes(self) -> int:
+        """Bytes of device memory this weight holds."""
+        tensors = (self.code_payload, self.beta_payload, self.row_norms, self.beta_table, self.resolved_words,
+                   self.resolved_tails)
+        return sum(t.numel() * t.element_size() for t in tensors if t is not None)
 
 
 # --------------------------------------------------------------------------------------
@@ -320,9 +333,11 @@ def resolve_weight(code_payload: torch.Tensor, beta_payload: torch.Tensor, *, ro
 
 
 def prepare_fused_linear(record: Any, *, device: torch.device | str = "cuda",
-                         resolve: bool = True) -> PreparedNQRTLinear:
+                         resolve: bool = True, keep_streams: bool = False) -> PreparedNQRTLinear:
     """Copy only the packed NQRT streams and compact metadata to the target GPU, and (unless
-    `resolve=False`) derive the resolved form of the weight from them."""
+    `resolve=False`) derive the resolved form of the weight from them.  Once a weight is resolved
+    every kernel reads that form, so the device copies of the streams are dropped (6 bits per weight
+    resident instead of 10.25) unless `keep_streams` asks for both."""
     for attribute in ("indices", "row_norms", "betas", "feature_count", "dither_seed",
                       "dither_algorithm", "codec_semantics"):
         if not hasattr(record, attribute):
@@ -341,6 +356,8 @@ def prepare_fused_linear(record: Any, *, device: torch.device | str = "cuda",
             and record.feature_count % 32 == 0 and len(record.betas) == 4):
         words, tails = resolve_weight(codes, beta_ids, rows=record.indices.shape[0],
                                       features=record.feature_count, dither_seed=record.dither_seed)
+        if not keep_streams:
+            codes = beta_ids = None
     return PreparedNQRTLinear(
         record=record,
         code_payload=codes,
@@ -370,7 +387,7 @@ def dequantize_rows_packed(codes: torch.Tensor, beta_ids: torch.Tensor, norms: t
 
 
 def dequantize_record(record: Any, *, device: torch.device | str = "cuda") -> torch.Tensor:
-    prepared = prepare_fused_linear(record, device=device)
+    prepared = prepare_fused_linear(record, device=device, resolve=False)
     rows = record.indices.shape[0]
     return dequantize_rows_packed(prepared.code_payload, prepared.beta_payload, prepared.row_norms,
                                   prepared.beta_table, rows=rows, features=record.feature_count,
@@ -394,14 +411,20 @@ def decode_packed_a4(activation: PreparedNQA4Activation,
 # predicates
 # --------------------------------------------------------------------------------------
 
+def _pointer(tensor: torch.Tensor | None) -> int | None:
+    return None if tensor is None else tensor.data_ptr()
+
+
 def _common_ok(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear,
                feature_multiple: int, row_multiple: int) -> bool:
     record = weight.record
-    tensors = (activation.code_payload, activation.beta_payload, activation.row_norms,
-               activation.beta_table, weight.code_payload, weight.beta_payload,
-               weight.row_norms, weight.beta_table)
+    streams = (weight.code_payload, weight.beta_payload)
+    resolved = (weight.resolved_words, weight.resolved_tails)
+    tensors = (activation.code_payload, activation.beta_payload, activation.row_norms, activation.beta_table,
+               weight.row_norms, weight.beta_table, *(t for t in streams + resolved if t is not None))
     return bool(
-        activation.feature_count == record.feature_count
+        (all(t is not None for t in streams) or all(t is not None for t in resolved))
+        and activation.feature_count == record.feature_count
         and activation.q == 14 and activation.code_width == 4 and activation.beta_width == 2
         and activation.beta_table.numel() == 4
         and record.feature_count % feature_multiple == 0
@@ -483,10 +506,8 @@ def _gemv(activation: PreparedNQA4Activation, weight: PreparedNQRTLinear, *, spl
     _native.check(launch(
         activation.code_payload.data_ptr(), activation.beta_payload.data_ptr(),
         activation.row_norms.data_ptr(), activation.beta_table.data_ptr(),
-        None if decoded is None else decoded.data_ptr(), weight.code_payload.data_ptr(),
-        weight.beta_payload.data_ptr(),
-        None if weight.resolved_words is None else weight.resolved_words.data_ptr(),
-        None if weight.resolved_tails is None else weight.resolved_tails.data_ptr(),
+        None if decoded is None else decoded.data_ptr(), _pointer(weight.code_payload), _pointer(weight.beta_payload),
+        _pointer(weight.resolved_words), _pointer(weight.resolved_tails),
         weight.row_norms.data_ptr(), weight.beta_table.data_ptr(), m, k, n, 0,
         int(weight.record.dither_seed), split_k, out.data_ptr(), _native.dtype_tag(output_dtype),
         None if workspace is None else workspace.data_ptr(), need, _native.stream_handle(device)))
@@ -607,11 +628,9 @@ def decode_weight_bf16(weight: PreparedNQRTLinear, *, out: torch.Tensor | None =
         out = torch.empty((n, k), dtype=torch.bfloat16, device=device)
     elif tuple(out.shape) != (n, k) or out.dtype != torch.bfloat16 or not out.is_contiguous() or out.device != device:
         raise ValueError("out must be a contiguous BF16 [N, K] tensor on the weight's device")
-    resolved = weight.resolved_words is not None
     _native.check(_native.library().nq_w4a4_decode_weight(
-        weight.code_payload.data_ptr(), weight.beta_payload.data_ptr(),
-        weight.resolved_words.data_ptr() if resolved else None,
-        weight.resolved_tails.data_ptr() if resolved else None,
+        _pointer(weight.code_payload), _pointer(weight.beta_payload), _pointer(weight.resolved_words),
+        _pointer(weight.resolved_tails),
         weight.row_norms.data_ptr(), weight.beta_table.data_ptr(), n, k, 0, int(weight.record.dither_seed),
         out.data_ptr(), _native.stream_handle(device)))
     return out

@@ -168,6 +168,12 @@ def test_dispatch_counters_and_m_routes(tiny):
              layer.w4a4_cuda_mma_chunked_staged_dispatch_count)
     assert tuple(b - a for a, b in zip(base, after)) == (1, 1, 1, 1, 1)
     assert layer.prepared and layer.packed_device_bytes > 0
+    # a resolved weight keeps 6 bytes per block of eight weights, its row norms and the beta table on the
+    # device: the NQRT4 streams it was derived from are not resident
+    state = layer._prepared
+    assert state.code_payload is None and state.beta_payload is None
+    weights = layer.out_features * layer.in_features
+    assert layer.packed_device_bytes == weights * 6 // 8 + 4 * layer.out_features + 16
 
 
 def test_fused_rotation_matches_separate_rotation(oracle):

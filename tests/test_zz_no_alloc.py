@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 def _case(oracle, rt, m, k, n_out, seed):
     from test_gpu_gemv import _record, _references
     _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=3000 + k + n_out, dither_seed=seed)
-    weight = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
+    weight = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda", keep_streams=True)
     x = torch.from_numpy(oracle.hadamard(student_t_rows(m, k, seed=4001 + m).numpy())).to(torch.bfloat16).cuda()
     activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS)
     ref32, _ = _references(oracle, activation, rt, wc, wb, wn, seed)
@@ -76,7 +76,7 @@ def test_static_scratch_gemv_allocates_no_device_memory(oracle):
     out = torch.empty((m, n), dtype=torch.float32, device="cuda")
     arguments = [
         activation.code_payload.data_ptr(), activation.beta_payload.data_ptr(), activation.row_norms.data_ptr(),
-        activation.beta_table.data_ptr(), None, weight.code_payload.data_ptr(), weight.beta_payload.data_ptr(),
+        activation.beta_table.data_ptr(), None, None, None,
         weight.resolved_words.data_ptr(), weight.resolved_tails.data_ptr(), weight.row_norms.data_ptr(),
         weight.beta_table.data_ptr(), m, k, n, 0, seed, 4, out.data_ptr(), _native.NQ_F32,
         _native.stream_handle(out.device)]
