@@ -320,8 +320,15 @@ __device__ __forceinline__ float resolved_scale(const ResolvedScales &scales, ui
 // multiplies by -B and adds -3, which leaves the complement of (v B + 1) << 1, whose top 18 bits
 // are 2^18 - 1 - U.  The last shift-xor of lcg31_mix_v1 only touches bits 0..14 of the value: two
 // of the 18 bits used here (13 and 14), which then carry an unmixed but equally uniform bit.
-// The eight counters of a block share bits 16..30 unless the block straddles a multiple of 2^16
-// (or of 2^31): those blocks take the counter-by-counter form of the first shift-xor.
+// The counters of a block are seed + 8 block + j, so a block's eight counters lie in at most two
+// aligned groups of eight counters [8 g, 8 g + 8), and which of its weights fall into the second one
+// depends on seed & 7 alone, the same for every block of a tensor.  Inside an aligned group the
+// counters differ in their low three bits only and share bits 16..30 (a group never straddles a
+// multiple of 2^16 or of 2^31), so the first shift-xor of a whole group is one value
+// T = x ^ (x >> 16), x = 8 g, and counter 8 g + i enters the hash as T ^ i.  A run of consecutive
+// blocks therefore costs one T per aligned group it touches and one xor with a constant per weight,
+// with no special case; seed & 7 is uniform, so the eight patterns are the arms of a scalar switch
+// (resolved_dither_bits_run, for lanes that own two or more neighbouring blocks).
 
 // From t_j = counter_j ^ (counter_j >> 16) to the float pattern's dither part: 2^18 - 1 - U_j in
 // bits 0..17 under the exponent of 2^23 (the funnel shift that takes the hash's top 18 bits brings
@@ -337,8 +344,52 @@ __device__ __forceinline__ void resolved_hash_bits(const uint32_t (&t)[8], uint3
     }
 }
 
-// The part of the decode that needs no memory: bits[j] as resolved_hash_bits leaves them, from the
-// block's first counter.
+// t[b][j] for the kBlocks consecutive blocks whose first counter is counter_plus_seed (bit 31 of a
+// value is not meaningful: the hash multiplies modulo 2^31 on values shifted left by one).
+template <int kBlocks, int kShift>
+__device__ __forceinline__ void resolved_hash_inputs_shifted(const uint32_t (&group)[kBlocks + 1], uint32_t (&t)[kBlocks][8]) {
+#pragma unroll
+    for (int b = 0; b < kBlocks; b++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) t[b][j] = group[b + ((kShift + j) >> 3)] ^ (uint32_t)((kShift + j) & 7);
+}
+
+template <int kBlocks>
+__device__ __forceinline__ void resolved_hash_inputs(uint32_t counter_plus_seed, uint32_t (&t)[kBlocks][8]) {
+    const uint32_t shift = (uint32_t)__builtin_amdgcn_readfirstlane((int)(counter_plus_seed & 7u));   // seed & 7
+    const uint32_t first = counter_plus_seed - shift;
+    uint32_t group[kBlocks + 1];
+#pragma unroll
+    for (int g = 0; g <= kBlocks; g++) {
+        const uint32_t x = first + 8u * (uint32_t)g;
+        group[g] = x ^ ((x >> 16) & 0x7fffu);
+    }
+    switch (shift) {
+        case 0: resolved_hash_inputs_shifted<kBlocks, 0>(group, t); break;
+        case 1: resolved_hash_inputs_shifted<kBlocks, 1>(group, t); break;
+        case 2: resolved_hash_inputs_shifted<kBlocks, 2>(group, t); break;
+        case 3: resolved_hash_inputs_shifted<kBlocks, 3>(group, t); break;
+        case 4: resolved_hash_inputs_shifted<kBlocks, 4>(group, t); break;
+        case 5: resolved_hash_inputs_shifted<kBlocks, 5>(group, t); break;
+        case 6: resolved_hash_inputs_shifted<kBlocks, 6>(group, t); break;
+        default: resolved_hash_inputs_shifted<kBlocks, 7>(group, t); break;
+    }
+}
+
+// The part of the decode that needs no memory: bits[b][j] as resolved_hash_bits leaves them, for
+// kBlocks consecutive blocks of one lane from the first block's first counter.
+template <int kBlocks>
+__device__ __forceinline__ void resolved_dither_bits_run(uint32_t counter_plus_seed, uint32_t (&bits)[kBlocks][8]) {
+    uint32_t t[kBlocks][8];
+    resolved_hash_inputs<kBlocks>(counter_plus_seed, t);
+#pragma unroll
+    for (int b = 0; b < kBlocks; b++) resolved_hash_bits(t[b], bits[b]);
+}
+
+// One block by itself: its eight counters share bits 16..30 unless the block straddles a multiple of
+// 2^16 (or of 2^31), which takes the counter-by-counter form of the first shift-xor.  (For a single
+// block the test is cheaper than the switch of the run form, which ends the basic block and with it
+// the overlap of this block's arithmetic with the next block's loads.)
 __device__ __forceinline__ void resolved_dither_bits(uint32_t counter_plus_seed, uint32_t (&bits)[8]) {
     const uint32_t base = counter_plus_seed & 0x7fffffffu;
     const uint32_t high = base >> 16;
@@ -354,29 +405,6 @@ __device__ __forceinline__ void resolved_dither_bits(uint32_t counter_plus_seed,
         for (int j = 0; j < 8; j++) t[j] = (base + (uint32_t)j) ^ high;
     }
     resolved_hash_bits(t, bits);
-}
-
-// The same for kBlocks consecutive blocks of one lane (counters counter_plus_seed .. + 8 kBlocks - 1), with
-// one test for the whole run, taken by the wavefront as a whole: a run that stays inside one stretch of
-// 2^16 counters in every lane shares the bits 16..30 of all its counters.  Same values as kBlocks calls
-// of resolved_dither_bits.
-template <int kBlocks>
-__device__ __forceinline__ void resolved_dither_bits_run(uint32_t counter_plus_seed, uint32_t (&bits)[kBlocks][8]) {
-    const uint32_t base = counter_plus_seed & 0x7fffffffu;
-    const bool leaves_its_stretch = (base & 0xffffu) > 0x10000u - 8u * kBlocks;
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(leaves_its_stretch) != 0, 0)) {
-#pragma unroll
-        for (int b = 0; b < kBlocks; b++) resolved_dither_bits(counter_plus_seed + 8u * b, bits[b]);
-        return;
-    }
-    const uint32_t high = base >> 16;
-#pragma unroll
-    for (int b = 0; b < kBlocks; b++) {
-        uint32_t t[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) t[j] = (base + (uint32_t)(8 * b + j)) ^ high;
-        resolved_hash_bits(t, bits[b]);
-    }
 }
 
 // The part that needs the stored block: out[j] = (s_j - u_j) * 2^17 * scale.  A weight's float

@@ -280,11 +280,28 @@ w4a4_gemv_mfma_kernel(const uint4 *__restrict__ act, GemvWeights w, int m_rows, 
                 acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
                                                                  __builtin_bit_cast(bf16x8, b[r][t]), acc[r], 0, 0, 0);
         };
+        // R = 1: the dither parts of two neighbouring blocks at a time (three aligned groups of counters
+        // instead of four); R = 2 has no registers to spare for that
+        if constexpr (R == 1) {
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            float v[8];
-            decode_resolved(word[t], tail[t], first_counter + 8u * t, resolved_scale(scaled_beta, word[t]), v);
-            multiply(t, v);
+            for (int half = 0; half < 2; half++) {
+                uint32_t bits[2][8];
+                resolved_dither_bits_run<2>(first_counter + 16u * half, bits);
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    const int t = 2 * half + i;
+                    float v[8];
+                    resolved_apply(word[t], tail[t], bits[i], resolved_scale(scaled_beta, word[t]), v);
+                    multiply(t, v);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                float v[8];
+                decode_resolved(word[t], tail[t], first_counter + 8u * t, resolved_scale(scaled_beta, word[t]), v);
+                multiply(t, v);
+            }
         }
     }
     // accumulator i of lane l: A row 4 (l / 16) + i = (range, channel), token l % 16; the row's own
