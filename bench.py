@@ -96,7 +96,8 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--library", default=None,
                         help="another build of libnqhip.so to load (the measuring build that --only encode_phases needs: "
                              "python -m nestquant_aiinfra_amd.build --define NQ_PHASE_STAMPS --output PATH)")
-    parser.add_argument("--only", choices=("tpot", "gemm", "attention", "encode", "rowlinear", "encode_phases", "attention_phases"), default=None,
+    parser.add_argument("--only", choices=("tpot", "gemm", "attention", "encode", "rowlinear", "encode_phases", "attention_phases",
+                                           "gemv_phases", "pair_phases"), default=None,
                         help="run one of the extra measurements alone (for profiling) and print its JSON")
     parser.add_argument("--skip-extras", action="store_true",
                         help="only the headline GEMV workload (no prefill GEMM, attention, TPOT)")
@@ -406,6 +407,104 @@ def encode_phases_extra(rt, device):
                 "encode_parts_ns": {"load_scale_divide": s[5] - s[3], "nearest_point_and_code": s[6] - s[5],
                                     "decode_and_error": s[7] - s[6], "argmin_and_stores": s[4] - s[7]},
             }
+    return results
+
+
+def _rotating_weights(rt, device, name, k, n, wseed, dseed, copies):
+    import torch
+    g = torch.Generator().manual_seed(wseed)
+    w = hadamard_gpu((0.02 * torch.randn(n, k, generator=g)).to(device))
+    record = rt.quantize_weight_nqrt4(w, q=Q, betas=WEIGHT_BETAS, dither_seed=dseed, tensor_name=name)
+    base = rt.prepare_fused_linear(record, device=device)
+    return [base] + [rt.PreparedNQRTLinear(record, None, None, base.row_norms, base.beta_table,
+                                           base.resolved_words.clone(), base.resolved_tails.clone())
+                     for _ in range(copies - 1)]
+
+
+def _stamps(lib, entry, count):
+    import ctypes
+    from nestquant_aiinfra_amd import _native
+    if not hasattr(lib, entry):
+        sys.exit(f"bench.py: this measurement needs a library built with --define NQ_PHASE_STAMPS (see --library): no {entry}")
+    call = getattr(lib, entry)
+    call.restype, call.argtypes = ctypes.c_int, [ctypes.c_void_p]
+    stamps = (ctypes.c_ulonglong * count)()
+    _native.check(call(stamps))
+    return [int(v) * 10 for v in stamps]                          # 100 MHz ticks -> ns
+
+
+def gemv_phases_extra(rt, device):
+    """Where one launch of the vector-unit GEMV (resolved weights, one row) spends its time: the
+    stamps of lane 0 of workgroup 0 in a measuring build (--library), beside the launch-to-launch
+    time of the same call in a graph over weights that rotate through more than the caches hold."""
+    import torch
+    from nestquant_aiinfra_amd import _native
+    lib = _native.library()
+    table = torch.tensor(ACTIVATION_BETAS, dtype=torch.float32, device=device)
+    results = {}
+    for name, k, n, wseed, dseed in SHAPES:
+        weights = _rotating_weights(rt, device, name, k, n, wseed, dseed, 48)
+        for m in (1, 4):
+            x = torch.randn(m, k, generator=torch.Generator().manual_seed(60 + m)).to(torch.bfloat16).to(device)
+            activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS, beta_table=table, hadamard=True)
+            linear = rt.linear_packed_w4a4_gemv_m1 if m == 1 else rt.linear_packed_w4a4_mma_small_m
+            call = lambda i: linear(activation, weights[i % len(weights)])
+            seconds = time_graph(call, len(weights))
+            flush = torch.empty(128 << 20, dtype=torch.float32, device=device).fill_(1.0)      # cold caches
+            torch.cuda.synchronize()
+            call(7)
+            s = _stamps(lib, "nq_debug_gemv_stamps", 16)
+            del flush
+            results[f"{name}_m{m}"] = {
+                "launch_ns": round(seconds * 1e9), "first_workgroup_ns": s[6] - s[0],
+                "setup_and_first_requests_ns": s[1] - s[0], "first_block_decoded_ns": s[2] - s[1],
+                "remaining_steps_ns": s[3] - s[2], "lane_sums_ns": s[4] - s[3], "barrier_ns": s[5] - s[4],
+                "fold_and_store_ns": s[6] - s[5]}
+    return results
+
+
+def pair_phases_extra(rt, device):
+    """The one-launch input stage + linear(s) of a 1B decode step, pair by pair: launch-to-launch time in
+    a graph over rotating weights, and the stamps the first and last encoder workgroup and the first and
+    last consumer workgroup leave in a measuring build (--library), in ns from the earliest of them."""
+    import torch
+    from nestquant_aiinfra_amd import _native
+    lib = _native.library()
+    table = torch.tensor(ACTIVATION_BETAS, dtype=torch.float32, device=device)
+    pairs = {"qkv": ("rmsnorm", [(2048, 2048), (512, 2048), (512, 2048)]), "gate_up": ("rmsnorm", [(8192, 2048), (8192, 2048)]),
+             "down": ("swiglu", [(2048, 8192)]), "o": ("swiglu", [(2048, 2048)])}
+    results, copies = {}, 24
+    for name, (mode, shapes) in pairs.items():
+        sets = [_rotating_weights(rt, device, f"{name}{i}", k, n, 1100 + i, 20261201 + i, copies) for i, (n, k) in enumerate(shapes)]
+        groups = [[members[c] for members in sets] for c in range(copies)]
+        k = shapes[0][1]
+        for m in (1, 8):
+            g = torch.Generator().manual_seed(70 + m)
+            x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(device)
+            other = torch.randn(m, k, generator=g).to(torch.bfloat16).to(device)
+            norm_weight = torch.ones(k, dtype=torch.bfloat16, device=device)
+            extra = dict(residual=other, norm_weight=norm_weight, eps=1e-5) if mode == "rmsnorm" else dict(gate=other)
+            sync = rt.StageLinearSync(device, sets=256)
+            one = lambda i: rt.fused_stage_linear(x, groups[i % copies], sync, mode=mode, beta_table=table, **extra)[0]
+            def two(i):
+                activation = rt.fused_input_stage(x, mode=mode, beta_table=table, **extra)[0]
+                return rt.linear_packed_w4a4_gemv_grouped(activation, groups[i % copies], output_dtype=torch.bfloat16)
+            two_launches = time_graph(two, 2 * copies)
+            one_launch = time_graph(one, 2 * copies)
+            sync.reset()
+            flush = torch.empty(128 << 20, dtype=torch.float32, device=device).fill_(1.0)
+            torch.cuda.synchronize()
+            one(5)
+            s = _stamps(lib, "nq_debug_pair_stamps", 32)
+            del flush
+            origin = min(s[0], s[8], s[16], s[24])
+            role = lambda slot, names: {label: s[8 * slot + i] - origin for i, label in enumerate(names)}
+            producer = ("start", "encoded", "stores_acknowledged", "behind_barrier")
+            consumer = ("start", "weights_decoded", "flags_seen", "multiplied", "stored")
+            results[f"{name}_m{m}"] = {
+                "two_launches_ns": round(two_launches * 1e9), "one_launch_ns": round(one_launch * 1e9),
+                "timed_out": sync.timed_out, "first_encoder": role(0, producer), "last_encoder": role(1, producer),
+                "first_consumer": role(2, consumer), "last_consumer": role(3, consumer)}
     return results
 
 
@@ -780,7 +879,9 @@ def main() -> None:
                  "attention": lambda: attention_extra(device), "encode": lambda: encode_extra(rt, device),
                  "rowlinear": lambda: row_linear_extra(rt, device),
                  "encode_phases": lambda: encode_phases_extra(rt, device),
-                 "attention_phases": lambda: attention_phases_extra(device)}[args.only]()
+                 "attention_phases": lambda: attention_phases_extra(device),
+                 "gemv_phases": lambda: gemv_phases_extra(rt, device),
+                 "pair_phases": lambda: pair_phases_extra(rt, device)}[args.only]()
         print(json.dumps({args.only: extra}))
         return
 

@@ -25,6 +25,21 @@
 
 #include <math.h>
 
+#ifdef NQ_PHASE_STAMPS
+// Measuring builds only: lane 0 of workgroup (0, 0) of the vector-unit kernel leaves the 100 MHz
+// wall clock at its phase boundaries (start, first requests issued, first block decoded, loop
+// done, lane sums in LDS, behind the barrier, output stored).
+namespace nq { __device__ unsigned long long g_gemv_stamps[16]; }
+#define NQ_GEMV_STAMP(i) do { if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) nq::g_gemv_stamps[i] = wall_clock64(); } while (0)
+extern "C" int nq_debug_gemv_stamps(unsigned long long *out16) {
+    if (hipDeviceSynchronize() != hipSuccess) return NQ_ERR_LAUNCH;
+    return hipMemcpyFromSymbol(out16, HIP_SYMBOL(nq::g_gemv_stamps), 16 * sizeof(unsigned long long)) == hipSuccess
+               ? NQ_OK : NQ_ERR_LAUNCH;
+}
+#else
+#define NQ_GEMV_STAMP(i) do { } while (0)
+#endif
+
 namespace nq {
 
 constexpr int kGemvThreads = 256;
@@ -46,6 +61,7 @@ gemv_rows(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8
           uint32_t seed_plus_offset, float sqrt_k, float *__restrict__ out_f32,
           uint16_t *__restrict__ out_bf16) {
     __shared__ float partial[kGemvWaves * 4][R][M];        // one entry per 16-lane row of every wavefront
+    NQ_GEMV_STAMP(0);
     const int tid = threadIdx.x, lane = tid & 63;
     const int blocks_per_row = k_size >> 3;
     const int slice_blocks = k_slice >> 3;
@@ -86,6 +102,7 @@ gemv_rows(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8
         for (int m = 0; m < M; m++)
             if (m < m_rows) a_next[m] = act[(int64_t)m * blocks_per_row + slice_first_block + tid];
     }
+    NQ_GEMV_STAMP(1);
     for (int b = tid; b < slice_blocks; b += kGemvThreads) {
         uint32_t word[R], side[R];
         uint4 a[M];
@@ -129,7 +146,11 @@ gemv_rows(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8
                 acc[r][m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a[m].w), w[3], acc[r][m], false);
             }
         }
+#ifdef NQ_PHASE_STAMPS
+        if (b == tid) { asm volatile("" :: "v"(acc[0][0])); NQ_GEMV_STAMP(2); }
+#endif
     }
+    NQ_GEMV_STAMP(3);
     // sums over the 16 lanes of every row with register-only lane exchanges (fixed order)
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -139,7 +160,9 @@ gemv_rows(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8
             if ((lane & 15) == 0) partial[tid >> 4][r][m] = v;
         }
     }
+    NQ_GEMV_STAMP(4);
     __syncthreads();
+    NQ_GEMV_STAMP(5);
     // row partials in index order
     if (tid < R * M) {
         const int r = tid / M, m = tid - r * M;
@@ -154,6 +177,7 @@ gemv_rows(const uint4 *__restrict__ act,          // decoded BF16 [m_rows][K / 8
                 out_bf16[(int64_t)m * n_size + n] = f32_to_bf16(total);
         }
     }
+    NQ_GEMV_STAMP(6);
 }
 
 template <int M, int R, bool kResolved>
