@@ -829,15 +829,24 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 def extra_rooflines(extra):
     """One roofline object per secondary kernel, from the measurements already taken: the prefill
-    GEMM at its largest row count against the dense BF16 matrix-core peak, decode attention and the
+    GEMM at 128, 384 and 4096 rows against the dense BF16 matrix-core peak, decode attention and the
     decode-size encoder against HBM."""
-    gemm = extra["prefill_gemm"]["gate_proj_m4096"]
-    attention = extra["nqkv_attention"]
+    def gemm_object(name, m, note):
+        row = extra["prefill_gemm"][f"{name}_m{m}"]
+        k, n = (2048, 8192) if name == "gate_proj" else (8192, 2048)
+        return {"bound": "mfma", "workload": f"{name} K{k} N{n} M{m} ({note})", "achieved": row["TFLOPs"],
+                "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": row["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS,
+                "launch_us": row["us"]}
+    fused, once = "weight decoded inside the product's launch", "decode of the weight included"
     encoders = {name: extra["e8_encode"][name] for name in ("a4_bf16_m1_n2048", "a4_bf16_m1_n8192", "a4_bf16_m4096_n8192")}
+    attention = extra["nqkv_attention"]
     return {
-        "prefill_gemm": {"bound": "mfma", "workload": "gate_proj K2048 N8192 M4096 (decode of the weight included)",
-                         "achieved": gemm["TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": gemm["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, "launch_us": gemm["us"]},
+        # the reference's own prefill row counts (128 and 384 rows), then a long prompt
+        "prefill_gemm": gemm_object("gate_proj", 128, fused),
+        "prefill_gemm_m384": gemm_object("gate_proj", 384, once),
+        "prefill_gemm_down_m128": gemm_object("down_proj", 128, fused),
+        "prefill_gemm_down_m384": gemm_object("down_proj", 384, once),
+        "prefill_gemm_m4096": gemm_object("gate_proj", 4096, once),
         "nqkv_attention": {"bound": "hbm", "workload": "batch 8, 32 / 8 heads, D 64, contexts uniform in [128, 4096]",
                            "achieved": attention["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                            "frac": attention["hbm_frac"], "launch_us": attention["us"],
