@@ -595,7 +595,15 @@ def rope_gpu(x, positions, theta=500000.0):
 
 def attention_extra(device):
     """Paged NQKV4 decode attention: 32 / 8 heads, D 64, batch 8, contexts uniform in [128, 4096],
-    RoPE (theta = 500000) on keys and queries before their Hadamard."""
+    RoPE (theta = 500000) on keys and queries before their Hadamard.  Measured on pools that keep the
+    decode hints (four more bits per block, the runner's default) and, under `without_hints`, on the six
+    streams of the reference's format alone; the algorithmic bytes are those of the six streams either way."""
+    results = _attention_measurements(device, hints=True)
+    results["without_hints"] = _attention_measurements(device, hints=False)
+    return results
+
+
+def _attention_measurements(device, hints):
     import torch
     from nestquant_aiinfra_amd.runtime import nqkv
     key_betas = tuple(v / 14 for v in (3.50, 4.58, 6.47, 17.06))
@@ -604,7 +612,7 @@ def attention_extra(device):
     lengths = torch.randint(128, 4097, (8,), generator=g).tolist()
     manager = nqkv.BatchedNQKVCacheManager(capacity=8, num_layers=4, num_kv_heads=8, head_dim=64, max_cache_len=4096,
                                            page_size=16, q=Q, key_betas=key_betas, value_betas=value_betas,
-                                           dtype=torch.bfloat16, device=device)
+                                           dtype=torch.bfloat16, device=device, hints=hints)
     width = max(lengths)
     for slot in range(8):
         manager.register(slot, slot=slot)

@@ -412,7 +412,30 @@ int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_dtype, cons
                   const float *key_betas_dev, int key_beta_count, const float *value_betas_dev,
                   int value_beta_count, void *hot_keys_dev, void *hot_values_dev, int batch, int tokens,
                   int slots, int max_pages, int kv_heads, int head_dim, int page_size, int rotate_keys,
-                  const void *rope_cos_dev, const void *rope_sin_dev, void *stream);
+                  const void *rope_cos_dev, const void *rope_sin_dev, uint8_t *key_hints_dev,
+                  uint8_t *value_hints_dev, void *stream);
+
+/*
+ * Decode hints: an optional seventh and eighth stream of the page pool, beside the six of the
+ * reference's format (which stay bit-identical): four bits per 8-value block, two blocks per byte,
+ * [pages][page_size * kv_heads * head_dim / 16] bytes for keys and for values.  A block's hint
+ * records the two decisions its undithered decode takes inside Q_E8(G c / 14): bit 0 = the
+ * half-integer coset wins, bits 1..3 = the coordinate that the parity correction of that coset's D8
+ * search moves.  With the hints a reader decodes a block with about 140 instead of 280 vector
+ * instructions and gets the same floats bit for bit (nq_nqkv_verify_hints checks every code word).
+ * Writers (nq_nqkv_write, nq_nqkv_append_attention_decode) fill the hints of every page they pack when
+ * given the two pointers; readers (nq_nqkv_attention_decode, nq_nqkv_append_attention_decode,
+ * nq_nqkv_attention_prefill) use them when given; NULL, NULL is the path without hints.  Hints
+ * must belong to the code words beside them: a pool filled by other means gets them from
+ * nq_nqkv_page_hints (`blocks` code words -> blocks / 2 bytes; code stream 8-byte aligned).
+ * nq_nqkv_verify_hints decodes the `count` code words from index `first` on (digits below 14; all
+ * 14^8 of them are 0 .. 1475789055) with and without their hint and adds the number of blocks that
+ * differ to *mismatches_dev (a self-check; the tests run it over the whole range).
+ * No counterpart in the reference (its kernels search both cosets in every decode,
+ * nestquant/runtime/nqkv_attention_k1.py:243-342).
+ */
+int nq_nqkv_page_hints(const uint8_t *codes_dev, int64_t blocks, uint8_t *hints_dev, void *stream);
+int nq_nqkv_verify_hints(int64_t first, int64_t count, uint64_t *mismatches_dev, void *stream);
 
 /*
  * Paged NQKV4 decode attention for a ragged batch: for batch row r with slot s (clamped to
@@ -445,7 +468,7 @@ int nq_nqkv_attention_decode(
     const void *hot_values_dev, const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch,
     int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
     int rotate_query, const void *rope_cos_dev, const void *rope_sin_dev, void *out_dev, void *workspace_dev,
-    size_t workspace_bytes, void *stream);
+    size_t workspace_bytes, const uint8_t *key_hints_dev, const uint8_t *value_hints_dev, void *stream);
 
 size_t nq_nqkv_attention_workspace_bytes(int batch, int q_heads, int head_dim, int max_pages);
 
@@ -478,7 +501,7 @@ int nq_nqkv_append_attention_decode(
     const uint8_t *cache_active_dev, void *hot_keys_dev, void *hot_values_dev, const int32_t *slot_ids_dev,
     const uint8_t *active_mask_dev, int batch, int slots, int max_pages, int q_heads, int kv_heads, int head_dim,
     int page_size, float scale, int rotate, const void *rope_cos_dev, const void *rope_sin_dev, void *out_dev,
-    void *workspace_dev, size_t workspace_bytes, void *stream);
+    void *workspace_dev, size_t workspace_bytes, uint8_t *key_hints_dev, uint8_t *value_hints_dev, void *stream);
 
 /*
  * The second stage of the decode attention done where its result is consumed.  With
@@ -563,7 +586,8 @@ int nq_nqkv_attention_prefill(
     const int32_t *sequence_lengths_dev, const void *hot_keys_dev, const void *hot_values_dev,
     const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, const int32_t *counts_dev, int uniform_count,
     int batch, int tokens, int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size,
-    float scale, void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
+    float scale, void *out_dev, void *workspace_dev, size_t workspace_bytes, const uint8_t *key_hints_dev,
+    const uint8_t *value_hints_dev, void *stream);
 
 /*
  * Bytes of the optional workspace of nq_nqkv_attention_prefill (0 when the launch has enough

@@ -28,6 +28,8 @@ _DTYPE_TAGS = {torch.float32: NQ_F32, torch.bfloat16: NQ_BF16, torch.float16: NQ
 _c = ctypes
 _ptr, _i32, _i64, _size = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_size_t
 
+ABI_VERSION = 2          # what nq_abi_version() of a matching library returns
+
 # name -> (restype, argtypes); must list every symbol include/nqhip.h declares
 SIGNATURES = {
     "nq_abi_version": (_i32, []),
@@ -61,12 +63,14 @@ SIGNATURES = {
     "nq_decode_step_begin": (_i32, [_ptr, _ptr, _i32, _i32, _i32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i32,
                                     _ptr, _ptr, _ptr, _i64, _i32, _ptr, _ptr]),
     "nq_nqkv_write": (_i32, [_ptr, _ptr, _i32, _ptr, _ptr, _ptr, _i32, _ptr, _ptr] + [_ptr] * 6
-                      + [_ptr, _i32, _ptr, _i32, _ptr, _ptr] + [_i32] * 8 + [_ptr, _ptr, _ptr]),
+                      + [_ptr, _i32, _ptr, _i32, _ptr, _ptr] + [_i32] * 8 + [_ptr, _ptr, _ptr, _ptr, _ptr]),
+    "nq_nqkv_page_hints": (_i32, [_ptr, _i64, _ptr, _ptr]),
+    "nq_nqkv_verify_hints": (_i32, [_i64, _i64, _ptr, _ptr]),
     "nq_nqkv_attention_decode": (_i32, [_ptr, _i32] + [_ptr] * 17 + [_i32] * 7 + [_c.c_float, _i32, _ptr, _ptr,
-                                                                                _ptr, _ptr, _size, _ptr]),
+                                                                                _ptr, _ptr, _size, _ptr, _ptr, _ptr]),
     "nq_nqkv_append_attention_decode": (_i32, [_ptr] * 10 + [_ptr, _i32, _ptr, _i32] + [_ptr] * 9 + [_i32] * 7
-                                        + [_c.c_float, _i32, _ptr, _ptr, _ptr, _ptr, _size, _ptr]),
-    "nq_nqkv_attention_prefill": (_i32, [_ptr] * 19 + [_i32] * 9 + [_c.c_float, _ptr, _ptr, _size, _ptr]),
+                                        + [_c.c_float, _i32, _ptr, _ptr, _ptr, _ptr, _size, _ptr, _ptr, _ptr]),
+    "nq_nqkv_attention_prefill": (_i32, [_ptr] * 19 + [_i32] * 9 + [_c.c_float, _ptr, _ptr, _size, _ptr, _ptr, _ptr]),
     "nq_nqkv_attention_prefill_workspace_bytes": (_size, [_i32] * 5),
     "nq_nqkv_attention_workspace_bytes": (_size, [_i32, _i32, _i32, _i32]),
     "nq_nqkv_attention_parts": (_i32, [_i32, _i32]),
@@ -103,6 +107,11 @@ def library() -> ctypes.CDLL:
         function = getattr(lib, name)
         function.restype = restype
         function.argtypes = argtypes
+    built = lib.nq_abi_version()
+    if built != ABI_VERSION:
+        raise NativeLibraryMissing(
+            f"{LIBRARY_PATH} was built for ABI version {built}, this binding speaks version {ABI_VERSION}: "
+            "rebuild it with `python -m nestquant_aiinfra_amd.build`")
     _LIB = lib
     return lib
 

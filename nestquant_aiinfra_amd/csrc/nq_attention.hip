@@ -68,6 +68,9 @@ struct AttentionArgs {
     const uint16_t *new_key, *new_value;          // BF16 [batch, kv_heads, D], the key before RoPE and rotation
     const int32_t *sequence_lengths;              // [slots], this step's token already counted
     int key_beta_count, rotate_keys;
+    // optional decode hints [pages][P * kv_heads * D / 16], two blocks per byte (see decode_codeword_hinted):
+    // read by every launch, written by a kWrites launch for the page it completes; null for none
+    const uint8_t *key_hints, *value_hints;
 };
 
 // Rotary embedding ((x * cos) + (rotate_half(x) * sin) in BF16 tensor arithmetic), then optionally
@@ -208,6 +211,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     __shared__ float tail_scale[kWrites ? 2 * P : 1], tail_norm[kWrites ? 2 * P : 1];
     __shared__ uint32_t tail_code[kWrites ? 2 * P : 1][kWrites ? kBlocks : 1];
     __shared__ uint32_t tail_ids[kWrites ? 2 * P : 1][kWrites ? kBlocks / 4 : 1];
+    __shared__ uint32_t tail_hint[kWrites ? 2 * P : 1][kWrites ? kBlocks / 2 : 1];
 
     const int tid = threadIdx.x;
     NQ_STAMP(0);
@@ -298,6 +302,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     }
 
     // ---- third loads: the packed operands of all passes, keys and values --------------------------------
+    const bool hinted = a.key_hints != nullptr;
     bool pass_valid[kPasses];
     uint32_t k_code[kPasses], k_ids[kPasses], v_code[kPasses], v_ids[kPasses];
     float k_norm[kPasses], v_norm[kPasses];
@@ -318,6 +323,10 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
             v_code[pass] = a.value_codes[word];
             v_ids[pass] = a.value_beta_ids[word >> 2];
             v_norm[pass] = a.value_norms[norm];
+            if (hinted) {                        // the hint byte of the block's pair rides above the beta byte
+                k_ids[pass] |= (uint32_t)a.key_hints[word >> 1] << 8;
+                v_ids[pass] |= (uint32_t)a.value_hints[word >> 1] << 8;
+            }
         }
     }
     int64_t new_page = -1;
@@ -408,6 +417,16 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
             quantize_staged_pairs<false>(&tail[0][0], tail_scale, D, 14.0f, 1.0f / 14.0f, betas_of, a.key_beta_count,
                                          0u, 0, 2 * P * kBlocks * 4, sink);
             __syncthreads();
+            if (hinted) {                                // the new page's decode hints, from its code words
+                if (tid < 2 * P * (kBlocks / 2)) {
+                    const int r = tid / (kBlocks / 2), pair = tid % (kBlocks / 2);
+                    const uint32_t byte = hint_of_codeword(tail_code[r][2 * pair]) | (hint_of_codeword(tail_code[r][2 * pair + 1]) << 4);
+                    tail_hint[r][pair] = byte;
+                    if (new_page >= 0)
+                        const_cast<uint8_t *>(r < P ? a.key_hints : a.value_hints)[sink.word(r, 2 * pair) >> 1] = (uint8_t)byte;
+                }
+                __syncthreads();
+            }
         }
     }
     if (empty) {                                         // the row's cache is switched off: the append was all
@@ -420,6 +439,10 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     if (appends && packs && pass_valid[0]) {
         k_code[0] = tail_code[token][blk]; k_ids[0] = tail_ids[token][blk >> 2]; k_norm[0] = tail_norm[token];
         v_code[0] = tail_code[P + token][blk]; v_ids[0] = tail_ids[P + token][blk >> 2]; v_norm[0] = tail_norm[P + token];
+        if (hinted) {
+            k_ids[0] |= tail_hint[token][blk >> 1] << 8;
+            v_ids[0] |= tail_hint[P + token][blk >> 1] << 8;
+        }
     }
     const bool bf16_rows = is_hot && !packs;             // the pass reads BF16 rows, not codes
     float q[G][8];
@@ -448,7 +471,8 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
                 unpack_bf16_row(hot_k, k);
             }
         } else if (valid) {
-            decode_codeword<false>(k_code[pass], 14.0f, 0u, k);
+            if (hinted) decode_codeword_hinted(k_code[pass], (k_ids[pass] >> (8 + 4 * (blk & 1))) & 15u, k);
+            else decode_codeword<false>(k_code[pass], 14.0f, 0u, k);
             const float beta = key_beta[(k_ids[pass] >> (2 * (blk & 3))) & 3];     // word index % 4 == blk % 4
             const float back = k_norm[pass] / sqrt_d;
 #pragma unroll
@@ -512,7 +536,8 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
                 unpack_bf16_row(hot_v, v);
             }
         } else if (valid) {
-            decode_codeword<false>(v_code[pass], 14.0f, 0u, v);
+            if (hinted) decode_codeword_hinted(v_code[pass], (v_ids[pass] >> (8 + 4 * (blk & 1))) & 15u, v);
+            else decode_codeword<false>(v_code[pass], 14.0f, 0u, v);
             const float beta = value_beta[(v_ids[pass] >> (2 * (blk & 3))) & 3];
             const float back = v_norm[pass] / sqrt_d;
 #pragma unroll
@@ -660,9 +685,11 @@ int launch_decode_attention(
     const void *hot_values_dev, const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch,
     int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
     int rotate_query, const void *rope_cos_dev, const void *rope_sin_dev, void *out_dev, void *workspace_dev,
-    size_t workspace_bytes, void *stream) {
+    size_t workspace_bytes, const uint8_t *key_hints_dev, const uint8_t *value_hints_dev, void *stream) {
     NQ_REQUIRE(batch >= 1 && slots >= 1 && max_pages >= 1, NQ_ERR_SHAPE,
                "%s: batch, slots and max_pages must be positive", entry);
+    NQ_REQUIRE((key_hints_dev == nullptr) == (value_hints_dev == nullptr), NQ_ERR_ARGUMENT,
+               "%s: key and value hint streams come together", entry);
     NQ_REQUIRE(kv_heads >= 1 && q_heads >= kv_heads && q_heads % kv_heads == 0, NQ_ERR_SHAPE,
                "%s: q_heads must be a positive multiple of kv_heads", entry);
     const int group = q_heads / kv_heads;
@@ -698,6 +725,7 @@ int launch_decode_attention(
     a.key_codes = reinterpret_cast<const uint32_t *>(key_codes_dev);
     a.value_codes = reinterpret_cast<const uint32_t *>(value_codes_dev);
     a.key_beta_ids = key_beta_ids_dev; a.value_beta_ids = value_beta_ids_dev;
+    a.key_hints = key_hints_dev; a.value_hints = value_hints_dev;
     a.key_norms = key_norms_dev; a.value_norms = value_norms_dev;
     a.key_betas = key_betas_dev; a.value_betas = value_betas_dev;
     a.page_indices = page_indices_dev; a.page_counts = page_counts_dev;
@@ -778,13 +806,14 @@ extern "C" int nq_nqkv_attention_decode(
     const void *hot_values_dev, const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch,
     int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
     int rotate_query, const void *rope_cos_dev, const void *rope_sin_dev, void *out_dev, void *workspace_dev,
-    size_t workspace_bytes, void *stream) {
+    size_t workspace_bytes, const uint8_t *key_hints_dev, const uint8_t *value_hints_dev, void *stream) {
     return launch_decode_attention(
         "nq_nqkv_attention_decode", nullptr, query_dev, query_dtype, key_codes_dev, key_beta_ids_dev, key_norms_dev,
         value_codes_dev, value_beta_ids_dev, value_norms_dev, key_betas_dev, value_betas_dev, page_indices_dev,
         page_counts_dev, last_page_lens_dev, hot_lengths_dev, cache_active_dev, hot_keys_dev, hot_values_dev,
         slot_ids_dev, active_mask_dev, batch, slots, max_pages, q_heads, kv_heads, head_dim, page_size, scale,
-        rotate_query, rope_cos_dev, rope_sin_dev, out_dev, workspace_dev, workspace_bytes, stream);
+        rotate_query, rope_cos_dev, rope_sin_dev, out_dev, workspace_dev, workspace_bytes, key_hints_dev, value_hints_dev,
+        stream);
 }
 
 extern "C" int nq_nqkv_append_attention_decode(
@@ -796,12 +825,12 @@ extern "C" int nq_nqkv_append_attention_decode(
     const uint8_t *cache_active_dev, void *hot_keys_dev, void *hot_values_dev, const int32_t *slot_ids_dev,
     const uint8_t *active_mask_dev, int batch, int slots, int max_pages, int q_heads, int kv_heads, int head_dim,
     int page_size, float scale, int rotate, const void *rope_cos_dev, const void *rope_sin_dev, void *out_dev,
-    void *workspace_dev, size_t workspace_bytes, void *stream) {
+    void *workspace_dev, size_t workspace_bytes, uint8_t *key_hints_dev, uint8_t *value_hints_dev, void *stream) {
     const AppendOperands append{key_dev, value_dev, sequence_lengths_dev, key_beta_count, value_beta_count, rotate};
     return launch_decode_attention(
         "nq_nqkv_append_attention_decode", &append, query_dev, NQ_BF16, key_codes_dev, key_beta_ids_dev, key_norms_dev,
         value_codes_dev, value_beta_ids_dev, value_norms_dev, key_betas_dev, value_betas_dev, page_indices_dev,
         page_counts_dev, last_page_lens_dev, hot_lengths_dev, cache_active_dev, hot_keys_dev, hot_values_dev,
         slot_ids_dev, active_mask_dev, batch, slots, max_pages, q_heads, kv_heads, head_dim, page_size, scale,
-        rotate, rope_cos_dev, rope_sin_dev, out_dev, workspace_dev, workspace_bytes, stream);
+        rotate, rope_cos_dev, rope_sin_dev, out_dev, workspace_dev, workspace_bytes, key_hints_dev, value_hints_dev, stream);
 }

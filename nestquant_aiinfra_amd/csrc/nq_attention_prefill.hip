@@ -48,6 +48,7 @@ struct PrefillAttentionArgs {
     uint16_t *out;                     // BF16 [batch, tokens, q_heads, D]
     const uint32_t *key_codes, *value_codes;
     const uint8_t *key_beta_ids, *value_beta_ids;
+    const uint8_t *key_hints, *value_hints;        // optional decode hints, two blocks per byte (decode_codeword_hinted)
     const float *key_norms, *value_norms, *key_betas, *value_betas;
     const int32_t *page_indices, *page_counts, *last_page_lens, *hot_lengths, *sequence_lengths;
     const uint16_t *hot_keys, *hot_values;
@@ -175,6 +176,8 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     const uint32_t lane_word = (uint32_t)(row_in_page * kBlocks + dec_blk);
     const uint32_t *side_codes = decodes_values ? a.value_codes : a.key_codes;
     const uint8_t *side_ids = decodes_values ? a.value_beta_ids : a.key_beta_ids;
+    const uint8_t *side_hints = decodes_values ? a.value_hints : a.key_hints;
+    const bool hinted = side_hints != nullptr;
     const float *side_norms = decodes_values ? a.value_norms : a.key_norms;
     const float *side_betas = decodes_values ? a.value_betas : a.key_betas;
     const uint16_t *side_hot = (decodes_values ? a.hot_values : a.hot_keys) +
@@ -187,11 +190,14 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     auto request_cold = [&](int ordinal) {               // operands of this lane's block of a full cold page
         const uint32_t page = (uint32_t)slot_pages[ordinal];
         const uint32_t word = page * page_words + lane_word;
-        return ColdOperands{side_codes[word], (uint32_t)side_ids[word >> 2], side_norms[page * page_rows + (uint32_t)row_in_page]};
+        // the hint byte of the block's pair rides above the beta byte
+        const uint32_t ids = (uint32_t)side_ids[word >> 2] | (hinted ? (uint32_t)side_hints[word >> 1] << 8 : 0u);
+        return ColdOperands{side_codes[word], ids, side_norms[page * page_rows + (uint32_t)row_in_page]};
     };
     auto decode_cold = [&](const ColdOperands &operands) {
         float v[8];
-        decode_codeword<false>(operands.code, 14.0f, 0u, v);
+        if (hinted) decode_codeword_hinted(operands.code, (operands.ids >> (8 + 4 * (dec_blk & 1))) & 15u, v);
+        else decode_codeword<false>(operands.code, 14.0f, 0u, v);
         const float beta = beta_table[(operands.ids >> (2 * (dec_blk & 3))) & 3];
         const float back = operands.norm / sqrt_d;
         const bf16x2 h0 = pack_bf16x2((v[0] * beta) * back, (v[1] * beta) * back);
@@ -413,9 +419,12 @@ extern "C" int nq_nqkv_attention_prefill(
     const int32_t *sequence_lengths_dev, const void *hot_keys_dev, const void *hot_values_dev,
     const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, const int32_t *counts_dev, int uniform_count,
     int batch, int tokens, int slots, int max_pages, int q_heads, int kv_heads, int head_dim, int page_size,
-    float scale, void *out_dev, void *workspace_dev, size_t workspace_bytes, void *stream) {
+    float scale, void *out_dev, void *workspace_dev, size_t workspace_bytes, const uint8_t *key_hints_dev,
+    const uint8_t *value_hints_dev, void *stream) {
     NQ_REQUIRE(batch >= 1 && tokens >= 1 && slots >= 1 && max_pages >= 1, NQ_ERR_SHAPE,
                "nq_nqkv_attention_prefill: batch, tokens, slots and max_pages must be positive");
+    NQ_REQUIRE((key_hints_dev == nullptr) == (value_hints_dev == nullptr), NQ_ERR_ARGUMENT,
+               "nq_nqkv_attention_prefill: key and value hint streams come together");
     NQ_REQUIRE(kv_heads >= 1 && q_heads >= kv_heads && q_heads % kv_heads == 0, NQ_ERR_SHAPE,
                "nq_nqkv_attention_prefill: q_heads must be a positive multiple of kv_heads");
     const int group = q_heads / kv_heads;
@@ -440,6 +449,7 @@ extern "C" int nq_nqkv_attention_prefill(
     a.key_codes = reinterpret_cast<const uint32_t *>(key_codes_dev);
     a.value_codes = reinterpret_cast<const uint32_t *>(value_codes_dev);
     a.key_beta_ids = key_beta_ids_dev; a.value_beta_ids = value_beta_ids_dev;
+    a.key_hints = key_hints_dev; a.value_hints = value_hints_dev;
     a.key_norms = key_norms_dev; a.value_norms = value_norms_dev;
     a.key_betas = key_betas_dev; a.value_betas = value_betas_dev;
     a.page_indices = page_indices_dev; a.page_counts = page_counts_dev; a.last_page_lens = last_page_lens_dev;

@@ -10,6 +10,6 @@ char *error_buffer() {
 
 }  // namespace nq
 
-extern "C" int nq_abi_version(void) { return 1; }
+extern "C" int nq_abi_version(void) { return 2; }
 
 extern "C" const char *nq_last_error(void) { return nq::error_buffer(); }

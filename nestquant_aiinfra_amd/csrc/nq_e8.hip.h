@@ -183,6 +183,98 @@ __device__ __forceinline__ void reduce_coset_point(const float (&p)[8], float q,
     for (int j = 0; j < 8; j++) out[j] = p[j] - q * k[j]; // exact
 }
 
+// ---------------------------------------------------------------------------------------
+// Hinted decode of an undithered block.
+//
+// decode_codeword<false> spends most of its instructions on decisions that the code word fixes:
+// which coset of E8 the point Q_E8(p / 14) lies in and which coordinate the parity correction of
+// that coset's D8 search moves.  A writer that has just made the code word can store both in four
+// bits (bit 0: the half-integer coset; bits 1..3: the coordinate), and a reader then needs neither
+// the other coset's search, nor the scans for the largest residual, nor the two distance sums.
+// Whether a correction happens at all is the parity of the rounded coordinates, and its direction
+// the sign of the chosen coordinate's residual, both cheap to recompute.  The quotient p / 14 stays
+// the correctly rounded one and the coset's offset is subtracted from it as the search does: a
+// single multiply-add p * RN(1/14) - 1/2 would round the exact tie p = 14 the other way (checked on
+// the CPU over every coordinate a coset point can have).  Same values as
+// decode_codeword<false>(word, 14, 0, out), bit for bit, for every code word (nq_nqkv_verify_hints).
+__device__ __forceinline__ uint32_t e8_nearest_hint(const float (&x)[8]) {
+    // e8_nearest(x) once more, keeping the decisions instead of the point
+    float ea[8], sum_a = 0.0f, eb[8], sum_b = 0.0f, a[8], b[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        a[j] = __builtin_rintf(x[j]);
+        ea[j] = x[j] - a[j];
+        sum_a = sum_a + a[j];
+        const float xm = x[j] - 0.5f;
+        b[j] = __builtin_rintf(xm);
+        eb[j] = xm - b[j];
+        sum_b = sum_b + b[j];
+    }
+    const float max_a = max_abs8(ea), max_b = max_abs8(eb);
+    const float moved_a = max_a - 1.0f, alt_a = moved_a * moved_a;
+    bool done_a = !is_odd(sum_a), done_b = !is_odd(sum_b);
+    float dist_a = 0.0f, dist_b = 0.0f;
+    uint32_t index_a = 0u, index_b = 0u;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const bool top_a = fabsf(ea[j]) == max_a, hit_a = top_a && !done_a;
+        done_a = done_a || top_a;
+        dist_a = dist_a + (hit_a ? alt_a : ea[j] * ea[j]);
+        index_a = hit_a ? (uint32_t)j : index_a;
+        const bool top_b = fabsf(eb[j]) == max_b, hit_b = top_b && !done_b;
+        done_b = done_b || top_b;
+        const float half_point = b[j] + 0.5f;
+        const float point = hit_b ? half_point + __builtin_copysignf(1.0f, eb[j]) : half_point;
+        const float t = x[j] - point;
+        dist_b = dist_b + t * t;
+        index_b = hit_b ? (uint32_t)j : index_b;
+    }
+    const bool pick_a = dist_a < dist_b;
+    return pick_a ? index_a << 1 : (index_b << 1) | 1u;
+}
+
+// The hint of a stored block: the decisions decode_codeword<false>(word, 14, 0, .) takes.
+__device__ __forceinline__ uint32_t hint_of_codeword(uint32_t word) {
+    float c[8], p[8], z[8];
+    unpack_codeword(word, c);
+    e8_coset_point(c, p);
+#pragma unroll
+    for (int j = 0; j < 8; j++) z[j] = div_by_14(p[j]);
+    return e8_nearest_hint(z);
+}
+
+__device__ __forceinline__ void decode_codeword_hinted(uint32_t word, uint32_t hint, float (&out)[8]) {
+    float c[8], p[8], xm[8], r[8];
+    unpack_codeword(word, c);
+    e8_coset_point(c, p);
+    const bool half_coset = (hint & 1u) != 0u;
+    const float minus_half = half_coset ? -0.5f : 0.0f;
+    const float minus_origin = half_coset ? -7.0f : 0.0f;          // 14 times the coset's offset
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        xm[j] = div_by_14(p[j]) + minus_half;
+        r[j] = __builtin_rintf(xm[j]);
+        sum = sum + r[j];
+    }
+    // the residual of the hinted coordinate, picked out of the eight by the index's bits
+    const bool bit0 = (hint & 2u) != 0u, bit1 = (hint & 4u) != 0u, bit2 = (hint & 8u) != 0u;
+    float e[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) e[j] = xm[j] - r[j];
+    const float e01 = bit0 ? e[1] : e[0], e23 = bit0 ? e[3] : e[2], e45 = bit0 ? e[5] : e[4], e67 = bit0 ? e[7] : e[6];
+    const float e03 = bit1 ? e23 : e01, e47 = bit1 ? e67 : e45;
+    const float chosen = bit2 ? e47 : e03;
+    // 14 times the step of the corrected coordinate, zero when the sum is even
+    const float step = is_odd(sum) ? __builtin_copysignf(14.0f, chosen) : 0.0f;
+    const uint32_t index = (hint >> 1) & 7u;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float plain = __builtin_fmaf(-14.0f, r[j], p[j] + minus_origin);      // exact: small half-integers
+        out[j] = index == (uint32_t)j ? plain - step : plain;
+    }
+}
+
 // x * c + a modulo 2^32.  On gfx950 the 32-bit multiply issues at the rate of the other
 // three-operand integer instructions (measured: v_mul_lo_u32 2.0 ns per wavefront instruction and
 // SIMD, v_dot2_u32_u16 1.9, v_lshl_add_u32 1.8, v_add_u32 1.1), so one multiply and one add beat

@@ -107,6 +107,7 @@ struct KvWriteArgs {
     const float *key_betas, *value_betas;
     uint16_t *hot_keys, *hot_values;        // BF16 [slots, P, kv_heads, D]
     const uint16_t *rope_cos, *rope_sin;    // optional BF16 [batch, tokens, D]: rotary embedding of the new keys
+    uint8_t *key_hints, *value_hints;       // optional [pages][P * kv_heads * D / 16]: decode hints, two blocks per byte
     int batch, tokens, uniform_count, slots, max_pages, kv_heads, key_beta_count, value_beta_count, rotate_keys;
 };
 
@@ -256,7 +257,44 @@ __global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
         // a lane per (block, beta) pair, which is what a many-page prompt pays for
         quantize_staged_blocks(&rows[0][0], row_scale, D, 14.0f, 1.0f / 14.0f, betas_of, a.key_beta_count, 0,
                                2 * P * kBlocks, sink);
+        if (a.key_hints) {
+            // the decode hints of the page's blocks, from the code words this workgroup has just stored
+            __syncthreads();
+            for (int i = tid; i < 2 * P * (kBlocks / 2); i += kKvThreads) {
+                const int which = i / (P * (kBlocks / 2)), rem = i % (P * (kBlocks / 2));
+                const int64_t word = sink.word(rem / (kBlocks / 2), 2 * (rem % (kBlocks / 2)));
+                const uint2 pair = *reinterpret_cast<const uint2 *>((which ? a.value_codes : a.key_codes) + word);
+                (which ? a.value_hints : a.key_hints)[word >> 1] =
+                    (uint8_t)(hint_of_codeword(pair.x) | (hint_of_codeword(pair.y) << 4));
+            }
+        }
     }
+}
+
+// Decode hints of a stream of undithered code words (a page brought in from a container, a test).
+__global__ void __launch_bounds__(256) page_hints_kernel(const uint2 *__restrict__ codes, int64_t pairs, uint8_t *__restrict__ hints) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= pairs) return;
+    const uint2 pair = codes[i];
+    hints[i] = (uint8_t)(hint_of_codeword(pair.x) | (hint_of_codeword(pair.y) << 4));
+}
+
+// Every code word with digits below 14 whose index lies in [first, first + count): the hinted decode
+// against the plain one; mismatching blocks are counted.
+__global__ void __launch_bounds__(256) verify_hints_kernel(int64_t first, int64_t count, unsigned long long *mismatches) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    int64_t index = first + i;
+    uint32_t word = 0u;
+#pragma unroll
+    for (int j = 0; j < 8; j++) { word |= (uint32_t)(index % 14) << (4 * j); index /= 14; }
+    float plain[8], hinted[8];
+    decode_codeword<false>(word, 14.0f, 0u, plain);
+    decode_codeword_hinted(word, hint_of_codeword(word), hinted);
+    bool same = true;
+#pragma unroll
+    for (int j = 0; j < 8; j++) same = same && __float_as_uint(plain[j]) == __float_as_uint(hinted[j]);
+    if (!same) atomicAdd(mismatches, 1ull);
 }
 
 }  // namespace nq
@@ -322,9 +360,14 @@ extern "C" int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_
                              const float *key_betas_dev, int key_beta_count, const float *value_betas_dev,
                              int value_beta_count, void *hot_keys_dev, void *hot_values_dev, int batch, int tokens,
                              int slots, int max_pages, int kv_heads, int head_dim, int page_size, int rotate_keys,
-                             const void *rope_cos_dev, const void *rope_sin_dev, void *stream) {
+                             const void *rope_cos_dev, const void *rope_sin_dev, uint8_t *key_hints_dev,
+                             uint8_t *value_hints_dev, void *stream) {
     NQ_REQUIRE(batch >= 1 && tokens >= 1 && slots >= 1 && max_pages >= 1 && kv_heads >= 1, NQ_ERR_SHAPE,
                "nq_nqkv_write: batch, tokens, slots, max_pages and kv_heads must be positive");
+    NQ_REQUIRE((key_hints_dev == nullptr) == (value_hints_dev == nullptr), NQ_ERR_ARGUMENT,
+               "nq_nqkv_write: key and value hint streams come together");
+    NQ_REQUIRE(!key_hints_dev || (nq::aligned(key_codes_dev, 8) && nq::aligned(value_codes_dev, 8)), NQ_ERR_ARGUMENT,
+               "nq_nqkv_write: with hint streams the code streams need 8-byte alignment");
     NQ_REQUIRE(head_dim == 64 && page_size == 16, NQ_ERR_SHAPE,
                "nq_nqkv_write: built for head_dim 64 and 16-token pages (got %d, %d)", head_dim, page_size);
     NQ_REQUIRE(kv_dtype == NQ_BF16, NQ_ERR_ARGUMENT, "nq_nqkv_write: keys and values must be BF16");
@@ -358,9 +401,34 @@ extern "C" int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_
                "nq_nqkv_write: rotary cos and sin tables come together");
     a.rope_cos = reinterpret_cast<const uint16_t *>(rope_cos_dev);
     a.rope_sin = reinterpret_cast<const uint16_t *>(rope_sin_dev);
+    a.key_hints = key_hints_dev; a.value_hints = value_hints_dev;
     // `tokens` new rows starting anywhere inside a page touch at most this many pages
     const int touched = (tokens + page_size - 2) / page_size + 1;
     hipLaunchKernelGGL((nq::kv_write_kernel<64, 16>), dim3((unsigned)touched, (unsigned)(batch * kv_heads)),
                        dim3(nq::kKvThreads), 0, (hipStream_t)stream, a);
     return nq::check_launch("nq_nqkv_write");
+}
+
+extern "C" int nq_nqkv_page_hints(const uint8_t *codes_dev, int64_t blocks, uint8_t *hints_dev, void *stream) {
+    NQ_REQUIRE(blocks >= 0 && blocks % 2 == 0, NQ_ERR_SHAPE, "nq_nqkv_page_hints: an even number of blocks (two per hint byte)");
+    if (blocks == 0) return NQ_OK;
+    NQ_REQUIRE(codes_dev && hints_dev && nq::aligned(codes_dev, 8), NQ_ERR_ARGUMENT,
+               "nq_nqkv_page_hints: needs the code words (8-byte aligned) and the hint bytes");
+    const int64_t pairs = blocks / 2, grid = (pairs + 255) / 256;
+    NQ_REQUIRE(grid <= 0x7fffffff, NQ_ERR_SHAPE, "nq_nqkv_page_hints: too many blocks");
+    hipLaunchKernelGGL(nq::page_hints_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<const uint2 *>(codes_dev), pairs, hints_dev);
+    return nq::check_launch("nq_nqkv_page_hints");
+}
+
+extern "C" int nq_nqkv_verify_hints(int64_t first, int64_t count, uint64_t *mismatches_dev, void *stream) {
+    const int64_t all = 14ll * 14 * 14 * 14 * 14 * 14 * 14 * 14;
+    NQ_REQUIRE(first >= 0 && count >= 1 && first + count <= all, NQ_ERR_SHAPE,
+               "nq_nqkv_verify_hints: the range must lie inside the 14^8 code words");
+    NQ_REQUIRE(mismatches_dev && nq::aligned(mismatches_dev, 8), NQ_ERR_ARGUMENT, "nq_nqkv_verify_hints: needs the counter");
+    const int64_t grid = (count + 255) / 256;
+    NQ_REQUIRE(grid <= 0x7fffffff, NQ_ERR_SHAPE, "nq_nqkv_verify_hints: at most 2^31 workgroups of 256 code words per call");
+    hipLaunchKernelGGL(nq::verify_hints_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, first, count,
+                       reinterpret_cast<unsigned long long *>(mismatches_dev));
+    return nq::check_launch("nq_nqkv_verify_hints");
 }

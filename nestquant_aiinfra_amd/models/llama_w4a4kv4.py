@@ -64,7 +64,7 @@ def build_w4a4kv4_runner(model: nn.Module, checkpoint: str | Path, *, capacity: 
                          enable_m1_down_splitk: bool = False,
                          fused_decode: bool | None = None, fused_prefill: bool | None = None,
                          packed_prefill: bool = False, expand_weights: bool = False,
-                         stage_linear_pairs=None) -> BatchedNQKVLlamaRunner:
+                         stage_linear_pairs=None, decode_hints: bool = True) -> BatchedNQKVLlamaRunner:
     """Swap the projections of `model` (BF16, on the GPU, eval mode) for packed W4A4 modules
     read from `checkpoint` and attach a batched NQKV4 cache; returns the runner."""
     reader = NQMCFileReader(checkpoint)
@@ -75,17 +75,20 @@ def build_w4a4kv4_runner(model: nn.Module, checkpoint: str | Path, *, capacity: 
     return attach_w4a4kv4_cache(model, capacity=capacity, max_cache_len=max_cache_len, page_size=page_size,
                                 key_betas=key_betas, value_betas=value_betas, fused_decode=fused_decode,
                                 fused_prefill=fused_prefill, packed_prefill=packed_prefill,
-                                expand_weights=expand_weights, stage_linear_pairs=stage_linear_pairs)
+                                expand_weights=expand_weights, stage_linear_pairs=stage_linear_pairs,
+                                decode_hints=decode_hints)
 
 
 def attach_w4a4kv4_cache(model: nn.Module, *, capacity: int, max_cache_len: int, page_size: int = 16,
                          key_betas: Sequence[float] = KEY_BETAS, value_betas: Sequence[float] = VALUE_BETAS,
                          fused_decode: bool | None = None, fused_prefill: bool | None = None,
                          packed_prefill: bool = False, expand_weights: bool = False,
-                         stage_linear_pairs=None) -> BatchedNQKVLlamaRunner:
+                         stage_linear_pairs=None, decode_hints: bool = True) -> BatchedNQKVLlamaRunner:
     """A batched NQKV4 cache of `capacity` slots and its runner over a model whose projections are
     already packed modules (an engine of another capacity over the same weights: the packed weights
-    are shared, the attention modules point at the newest cache)."""
+    are shared, the attention modules point at the newest cache).  `decode_hints`: the page pools keep
+    four more bits per block so that the attention kernels skip the lattice searches of the KV decode
+    (same outputs bit for bit; 10.5 % more pool memory)."""
     config = model.config
     head_dim = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
     device = next(model.parameters()).device
@@ -93,7 +96,7 @@ def attach_w4a4kv4_cache(model: nn.Module, *, capacity: int, max_cache_len: int,
         capacity=capacity, num_layers=config.num_hidden_layers, num_query_heads=config.num_attention_heads,
         num_kv_heads=config.num_key_value_heads, head_dim=head_dim, max_cache_len=max_cache_len,
         page_size=page_size, q=14, key_betas=key_betas, value_betas=value_betas, dtype=torch.bfloat16, device=device,
-        packed_prefill=packed_prefill)
+        packed_prefill=packed_prefill, decode_hints=decode_hints)
     install_batched_nqkv_llama_backend(model, cache)
     return BatchedNQKVLlamaRunner(model, cache, fused_decode=fused_decode, fused_prefill=fused_prefill,
                                   expand_weights=expand_weights, stage_linear_pairs=stage_linear_pairs)

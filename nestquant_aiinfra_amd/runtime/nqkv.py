@@ -169,7 +169,8 @@ class NQKVPagePool:
     def __init__(self, *, capacity: int, page_size: int, num_kv_heads: int, head_dim: int, q: int,
                  betas: Sequence[float] | None = None, key_betas: Sequence[float] | None = None,
                  value_betas: Sequence[float] | None = None,
-                 output_dtype: torch.dtype = torch.bfloat16, device: torch.device | str = "cuda") -> None:
+                 output_dtype: torch.dtype = torch.bfloat16, device: torch.device | str = "cuda",
+                 hints: bool = False) -> None:
         _positive(capacity=capacity, page_size=page_size, num_kv_heads=num_kv_heads, head_dim=head_dim)
         if head_dim % 8:
             raise ValueError("head_dim must be divisible by 8")
@@ -200,6 +201,15 @@ class NQKVPagePool:
         for side in ("key", "value"):
             for kind, (width, dtype) in self._stream_shapes.items():
                 setattr(self, f"{side}_{kind}", torch.zeros((capacity, width), dtype=dtype, device=where))
+        # Decode hints (not part of the reference's page format): four bits per block beside the six
+        # streams, written by the kernels that pack a page and read by the attention kernels, which
+        # then skip the lattice searches of the undithered decode.  Same decoded values bit for bit.
+        self.key_hints = self.value_hints = None
+        if hints:
+            if q != 14 or (rows * head_dim // 8) % 2:
+                raise ValueError("decode hints need q = 14 and an even number of blocks per page")
+            self.key_hints = torch.zeros((capacity, rows * head_dim // 16), dtype=torch.uint8, device=where)
+            self.value_hints = torch.zeros_like(self.key_hints)
         self.beta_table = torch.tensor(key_table, dtype=torch.float32, device=where)
         self.value_beta_table = self.beta_table if shared_table else torch.tensor(value_table, dtype=torch.float32,
                                                                                   device=where)
@@ -224,6 +234,8 @@ class NQKVPagePool:
         held = [getattr(self, name) for name in self._STREAMS] + [self.beta_table]
         if self.value_beta_table is not self.beta_table:
             held.append(self.value_beta_table)
+        if self.key_hints is not None:
+            held += [self.key_hints, self.value_hints]
         return sum(tensor.numel() * tensor.element_size() for tensor in held)
 
     # -- ownership ---------------------------------------------------------------------------
@@ -271,6 +283,11 @@ class NQKVPagePool:
             raise ValueError("prepared NQKV payload sizes do not match the pool")
         for slot, stream in zip(slots, incoming):
             slot.copy_(stream)
+        if self.key_hints is not None:                   # a page from elsewhere: its hints from its code words
+            lib, stream_handle = _native.library(), _native.stream_handle(self.device)
+            for codes, hints in ((self.key_codes, self.key_hints), (self.value_codes, self.value_hints)):
+                _native.check(lib.nq_nqkv_page_hints(codes[page_id].data_ptr(), codes.shape[1] // 4,
+                                                     hints[page_id].data_ptr(), stream_handle))
         self._pages[page_id].valid_tokens = page.valid_tokens
 
     def store(self, handle: NQKVPageHandle, page) -> None:
@@ -292,6 +309,12 @@ class NQKVPagePool:
         if not tokens:
             raise RuntimeError("NQKV page has not been stored")
         return self.page_view(page_id, tokens)
+
+    def hint_pointers(self) -> tuple[int | None, int | None]:
+        """The two hint streams as the C ABI takes them (None, None without hints)."""
+        if self.key_hints is None:
+            return None, None
+        return self.key_hints.data_ptr(), self.value_hints.data_ptr()
 
     def page_view(self, page_id: int, valid_tokens: int) -> PreparedNQKVPage:
         return PreparedNQKVPage(
@@ -457,7 +480,7 @@ class NQKVHotColdCache:
             pool.beta_table.data_ptr(), pool.beta_table.numel(), pool.value_beta_table.data_ptr(),
             pool.value_beta_table.numel(), self.hot_keys.data_ptr(), self.hot_values.data_ptr(),
             1, tokens, self.max_sequences, self.max_pages_per_sequence, pool.num_kv_heads, pool.head_dim,
-            pool.page_size, 0, None, None, stream))
+            pool.page_size, 0, None, None, *pool.hint_pointers(), stream))
         for handle in handles:
             logical.commit_graph_page(sequence_id, handle)
         self._hot_tokens[slot] = (held + tokens) % pool.page_size
@@ -530,7 +553,7 @@ def launch_nqkv_decode_attention(query: torch.Tensor, cache: NQKVHotColdCache, *
         batch, cache.max_sequences, cache.max_pages_per_sequence, heads, pool.num_kv_heads, dim, pool.page_size,
         attention_scale, int(rotate_query), None if rope is None else rope[0].data_ptr(),
         None if rope is None else rope[1].data_ptr(), workspace.output.data_ptr() if merge else None,
-        workspace.buffer.data_ptr(), workspace.buffer.numel(),
+        workspace.buffer.data_ptr(), workspace.buffer.numel(), *pool.hint_pointers(),
         _native.stream_handle(query.device)))
     return workspace.output if merge else None
 
@@ -655,7 +678,7 @@ def nqkv_prefill_attention(query: torch.Tensor, cache: NQKVHotColdCache, *, slot
         slot_ids.data_ptr(), active_mask.data_ptr(), None if counts is None else counts.data_ptr(),
         0 if uniform_count is None else int(uniform_count), batch, tokens, cache.max_sequences,
         cache.max_pages_per_sequence, heads, pool.num_kv_heads, dim, pool.page_size, attention_scale,
-        out.data_ptr(), None if workspace is None else workspace.data_ptr(), need,
+        out.data_ptr(), None if workspace is None else workspace.data_ptr(), need, *pool.hint_pointers(),
         _native.stream_handle(query.device)))
     return out
 
@@ -708,7 +731,7 @@ def _launch_append_hot_k1_graph_safe(key: torch.Tensor, value: torch.Tensor, cac
         pool.beta_table.data_ptr(), pool.beta_table.numel(), pool.value_beta_table.data_ptr(),
         pool.value_beta_table.numel(), cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(),
         batch, 1, cache.max_sequences, cache.max_pages_per_sequence, pool.num_kv_heads, pool.head_dim, pool.page_size,
-        0, None, None, stream))
+        0, None, None, *pool.hint_pointers(), stream))
 
 
 def append_hot_k1_graph_safe(key: torch.Tensor, value: torch.Tensor, cache: NQKVHotColdCache, *,
@@ -770,7 +793,9 @@ class BatchedNQKVCacheManager:
 
     def __init__(self, *, capacity: int, num_layers: int, num_kv_heads: int, head_dim: int,
                  max_cache_len: int, page_size: int, q: int, key_betas: Sequence[float],
-                 value_betas: Sequence[float], dtype: torch.dtype, device: torch.device | str) -> None:
+                 value_betas: Sequence[float], dtype: torch.dtype, device: torch.device | str,
+                 hints: bool = False) -> None:
+        """`hints`: every layer's pool also keeps the decode hints (NQKVPagePool), four bits per block."""
         if dtype != torch.bfloat16:
             raise ValueError("the NQKV hot tails and writer are BF16")
         self.capacity, self.num_layers, self.page_size = capacity, num_layers, page_size
@@ -788,7 +813,7 @@ class BatchedNQKVCacheManager:
             NQKVHotColdCache(
                 NQKVPagePool(capacity=capacity * self.max_pages, page_size=page_size, num_kv_heads=num_kv_heads,
                              head_dim=head_dim, q=q, key_betas=key_betas, value_betas=value_betas,
-                             output_dtype=dtype, device=target),
+                             output_dtype=dtype, device=target, hints=hints),
                 self.metadata, max_sequences=capacity, max_pages_per_sequence=self.max_pages)
             for _ in range(num_layers)
         ]
@@ -914,7 +939,7 @@ class BatchedNQKVCacheManager:
             pool.value_beta_table.numel(), cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(),
             rows, tokens, self.capacity, self.max_pages, pool.num_kv_heads, pool.head_dim, self.page_size,
             int(rotate_keys), None if rope is None else rope[0].data_ptr(),
-            None if rope is None else rope[1].data_ptr(), _native.stream_handle(self.device)))
+            None if rope is None else rope[1].data_ptr(), *pool.hint_pointers(), _native.stream_handle(self.device)))
 
     def append_and_attend(self, layer_index: int, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, *,
                           attention_scale: float, workspace: BatchedNQKVAttentionWorkspace, rotate: bool = False,
@@ -947,7 +972,8 @@ class BatchedNQKVCacheManager:
             self.step_active.data_ptr(), rows, self.capacity, self.max_pages, heads, pool.num_kv_heads, dim,
             self.page_size, attention_scale, int(rotate), None if rope is None else rope[0].data_ptr(),
             None if rope is None else rope[1].data_ptr(), workspace.output.data_ptr() if merge else None,
-            workspace.buffer.data_ptr(), workspace.buffer.numel(), _native.stream_handle(self.device)))
+            workspace.buffer.data_ptr(), workspace.buffer.numel(), *pool.hint_pointers(),
+            _native.stream_handle(self.device)))
         return workspace.output if merge else None
 
     def resident_bytes(self) -> int:

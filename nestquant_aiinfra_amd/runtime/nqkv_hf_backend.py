@@ -35,10 +35,12 @@ class BatchedNQKVLlamaCache(Cache):
     def __init__(self, *, capacity: int, num_layers: int, num_query_heads: int, num_kv_heads: int,
                  head_dim: int, max_cache_len: int, page_size: int, q: int, key_betas: Sequence[float],
                  value_betas: Sequence[float], dtype: torch.dtype, device: torch.device | str,
-                 packed_prefill: bool = False) -> None:
+                 packed_prefill: bool = False, decode_hints: bool = False) -> None:
         """`packed_prefill` (an extension): prefill chunks attend to the packed cache instead of
         the BF16 keys and values of the chunk, so long prompts can be fed in pieces.  A chunk
-        written into a slot that already holds tokens always takes that route."""
+        written into a slot that already holds tokens always takes that route.  `decode_hints` (an
+        extension): the pools keep four more bits per block, with which the attention kernels skip the
+        lattice searches of the KV decode (same outputs bit for bit)."""
         super().__init__(layers=[])
         for name, value in (("capacity", capacity), ("num_layers", num_layers),
                             ("num_query_heads", num_query_heads), ("num_kv_heads", num_kv_heads),
@@ -50,7 +52,7 @@ class BatchedNQKVLlamaCache(Cache):
         self.manager = BatchedNQKVCacheManager(
             capacity=capacity, num_layers=num_layers, num_kv_heads=num_kv_heads, head_dim=head_dim,
             max_cache_len=max_cache_len, page_size=page_size, q=q, key_betas=key_betas,
-            value_betas=value_betas, dtype=dtype, device=device)
+            value_betas=value_betas, dtype=dtype, device=device, hints=decode_hints)
         self.capacity, self.num_layers = capacity, num_layers
         self.num_query_heads, self.num_kv_heads, self.head_dim = num_query_heads, num_kv_heads, head_dim
         self._max_cache_len = max_cache_len

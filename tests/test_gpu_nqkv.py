@@ -691,5 +691,5 @@ def test_decode_attention_refuses_a_misaligned_query(kv):
         meta.hot_lengths.data_ptr(), meta.active_mask.data_ptr(), cache.hot_keys.data_ptr(), cache.hot_values.data_ptr(),
         slot_ids.data_ptr(), active.data_ptr(), 1, cache.max_sequences, cache.max_pages_per_sequence, 32, pool.num_kv_heads,
         DIM, pool.page_size, 0.125, 0, None, None, workspace.output.data_ptr(), workspace.buffer.data_ptr(),
-        workspace.buffer.numel(), _native.stream_handle(shifted.device))
+        workspace.buffer.numel(), None, None, _native.stream_handle(shifted.device))
     assert status == _native.NQ_ERR_ARGUMENT and b"16-byte alignment" in _native.library().nq_last_error()

@@ -232,3 +232,24 @@ def test_division_through_the_reciprocal_is_ieee_exact(oracle):
     betas += [1.0 / 3.0, 0.7, 1.9999999, 1.0000001, 3.1415927]
     for beta in betas:
         assert oracle.count_reciprocal_division_mismatches(float(np.float32(beta))) == 0, beta
+
+
+def test_hinted_decode_needs_the_exact_quotient():
+    """The hinted KV decode rounds p / 14 - h (h = 0 or 1/2) per coordinate.  A single fused multiply-add
+    p * RN(1/14) - h in place of the correctly rounded quotient would be cheaper, and is wrong: for the
+    coset-point coordinate p = 14 in the half-integer coset the exact value is the tie 0.5 (rounds to 0),
+    the fused form gives 0.50000006 (rounds to 1).  This test keeps the counter-example, and checks that it
+    is the only kind: every disagreement over the coordinates a coset point can have (multiples of 1/2;
+    code digits up to 15 give [-15, 37.5]) sits on an exact tie of the reference's form."""
+    c = np.float32(1.0) / np.float32(14.0)
+    disagreements = []
+    for twice in range(-30, 76):
+        p = np.float32(twice / 2.0)
+        exact = p / np.float32(14.0)                               # IEEE division, correctly rounded
+        for half in (np.float32(0.0), np.float32(0.5)):
+            reference = np.float32(exact - half)
+            fused = np.float32(np.float64(p) * np.float64(c) - np.float64(half))   # one rounding of the exact value
+            if np.rint(reference) != np.rint(fused):
+                disagreements.append((float(p), float(half)))
+                assert abs(float(reference) - np.floor(float(reference))) == 0.5
+    assert (14.0, 0.5) in disagreements
