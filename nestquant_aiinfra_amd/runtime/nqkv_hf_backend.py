@@ -392,6 +392,9 @@ class BatchedNQKVLlamaRunner:
         self.batch_size, self.max_cache_len = cache.capacity, cache.max_cache_len
         self._generation = [0] * self.batch_size
         self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor, torch.Tensor]] = {}
+        # (rows, width) -> captured fused prefill with last-token logits: graph, tokens, positions, keep, logits
+        self._prefill_graphs: dict[tuple[int, int], tuple] = {}
+        self.prefill_graph_replay_counts: dict[tuple[int, int], int] = {}
         self._greedy: dict[int, tuple[torch.Tensor, ...]] = {}       # width -> (history, cursors, sampler scratch)
         self.graph_replay_counts: dict[int, int] = {}
         self._decode_state: tuple | None = None      # (width, slots) the step tensors were last set for
@@ -540,6 +543,17 @@ class BatchedNQKVLlamaRunner:
         if last_token_logits:
             keep = torch.tensor([length - 1 for length in lengths], dtype=torch.long, device=self.device)
         try:
+            captured = None
+            if keep is not None and not self.cache._continuation and not self.cache.packed_prefill:
+                captured = self._prefill_graphs.get((rows, width))
+            if captured is not None:
+                graph, graph_ids, graph_positions, graph_keep, logits = captured
+                graph_ids.copy_(input_ids)
+                graph_positions.copy_(positions)
+                graph_keep.copy_(keep)
+                graph.replay()
+                self.prefill_graph_replay_counts[(rows, width)] += 1
+                return logits.clone()
             if self.fused_prefill is not None:
                 return self.fused_prefill(input_ids, positions, keep=keep)
             output = self.model(input_ids=input_ids, position_ids=positions, past_key_values=self.cache, use_cache=True)
@@ -549,6 +563,50 @@ class BatchedNQKVLlamaRunner:
         if keep is not None:
             return output.logits[torch.arange(rows, device=self.device), keep].unsqueeze(1)
         return output.logits
+
+    @torch.inference_mode()
+    def capture_prefill(self, *, rows: int, width: int) -> None:
+        """Capture the fused prefill of `rows` fresh prompts of up to `width` tokens (the form with the last
+        token's logits only, which is what an engine asks for) as one HIP graph.  A prompt of 128 tokens is
+        bound by the host issuing its 270 launches; replayed from a graph it is bound by its kernels.
+        `prefill_slots(..., last_token_logits=True)` then replays the graph whenever it is called with
+        exactly [rows, width] tokens for slots that hold nothing yet; the row lengths may be anything up
+        to `width` (they are read on the device).  Captured on rows that write nothing, so the cache is
+        left as it was; same logits and cache contents as the un-captured call, bit for bit."""
+        if self.fused_prefill is None:
+            raise RuntimeError("capture_prefill needs the fused prefill step (fused_prefill=None or True on a model that qualifies)")
+        if not 1 <= rows <= self.batch_size or not 1 <= width <= self.max_cache_len:
+            raise ValueError("rows must be in [1, capacity] and width in [1, max_cache_len]")
+        if self.cache.packed_prefill:
+            raise RuntimeError("a cache with packed_prefill attends over the cache in every prefill: nothing to capture")
+        cache, manager = self.cache, self.cache.manager
+        meta = manager.metadata
+        saved = [t.clone() for t in (meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths)]
+        ids = torch.zeros((rows, width), dtype=torch.long, device=self.device)
+        positions = torch.arange(width, device=self.device).repeat(rows, 1)
+        keep = torch.zeros(rows, dtype=torch.long, device=self.device)
+        manager.step_slot_ids[:rows].copy_(torch.arange(rows, dtype=torch.int32))
+        manager.step_counts[:rows].zero_()
+        manager.step_active[:rows].zero_()                   # inactive rows: the writer stores nothing
+        cache._rows, cache._tokens, cache._continuation = rows, width, False
+        self._decode_state = None
+        stream = torch.cuda.Stream(device=self.device)
+        stream.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(stream):
+            for _ in range(2):
+                manager.begin_step(rows=rows, uniform_count=None)
+                self.fused_prefill(ids, positions, keep=keep)
+            stream.synchronize()
+            manager.begin_step(rows=rows, uniform_count=None)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                logits = self.fused_prefill(ids, positions, keep=keep)
+        torch.cuda.current_stream(self.device).wait_stream(stream)
+        for tensor, value in zip((meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths), saved):
+            tensor.copy_(value)
+        cache._tokens = None
+        self._prefill_graphs[(rows, width)] = (graph, ids, positions, keep, logits)
+        self.prefill_graph_replay_counts[(rows, width)] = 0
 
     def release_slots(self, slots: Sequence[int]) -> None:
         self.cache.release_slots(slots)

@@ -206,3 +206,62 @@ def test_fused_rotation_matches_separate_rotation(oracle):
     k = torch.randn(3, 2, 7, 64, device="cuda").to(torch.bfloat16)
     assert torch.equal(rt.hadamard_cuda(k, compute_dtype=torch.float32), hadamard(k.float()).to(torch.bfloat16))
     assert relative_error(bits(rt.hadamard_cuda(k.float())), oracle.hadamard(bits(k.float()))) < 1e-6
+
+
+def test_captured_prefill_equals_the_uncaptured_one(tiny):
+    """`capture_prefill(rows, width)` replays the fused prefill as one graph: the same last-token logits and
+    the same cache (pools, hot tails, tables) as the un-captured call, for ragged lengths that change from
+    call to call; other shapes and continuation chunks keep the un-captured path."""
+    model, runner, *_ = tiny
+    cache = runner.cache
+    pools = [layer.pool for layer in cache.manager.layers]
+    meta = cache.manager.metadata
+
+    def state():
+        tensors = [getattr(pool, name).clone() for pool in pools
+                   for name in ("key_codes", "key_betas", "key_norms", "value_codes", "value_betas", "value_norms")]
+        tensors += [t.clone() for layer in cache.manager.layers for t in (layer.hot_keys, layer.hot_values)]
+        tensors += [t.clone() for t in (meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths)]
+        return tensors
+
+    def wipe():                                          # pages of released slots keep their bytes: start both passes from zeros
+        for pool in pools:
+            for name in ("key_codes", "key_betas", "key_norms", "value_codes", "value_betas", "value_norms", "key_hints",
+                         "value_hints"):
+                if getattr(pool, name) is not None:
+                    getattr(pool, name).zero_()
+        for layer in cache.manager.layers:
+            layer.hot_keys.zero_()
+            layer.hot_values.zero_()
+
+    runner.release_slots([s for s in range(4) if cache.manager.sequence_id(s) is not None])
+    cases = [([1, 3], [40, 23]), ([0, 2], [17, 48]), ([2, 1], [48, 1])]
+    eager = []
+    wipe()
+    for seed, (slots, lengths) in enumerate(cases):
+        ids = _prompt(2, 48, 6100 + seed)
+        logits = runner.prefill_slots(ids, slots=slots, lengths=lengths, last_token_logits=True).clone()
+        eager.append((logits, state()))
+        runner.release_slots(slots)
+    before = state()
+    runner.capture_prefill(rows=2, width=48)
+    assert all(torch.equal(a, b) for a, b in zip(before, state()))          # capturing leaves the cache alone
+    wipe()
+    for seed, (slots, lengths) in enumerate(cases):
+        ids = _prompt(2, 48, 6100 + seed)
+        logits = runner.prefill_slots(ids, slots=slots, lengths=lengths, last_token_logits=True)
+        want_logits, want_state = eager[seed]
+        assert torch.equal(logits, want_logits), seed
+        assert all(torch.equal(a, b) for a, b in zip(state(), want_state)), seed
+        runner.release_slots(slots)
+    assert runner.prefill_graph_replay_counts[(2, 48)] == 3
+    # another width, all-position logits and a chunk into slots that hold tokens do not take the graph
+    ids = _prompt(2, 40, 6200)
+    runner.prefill_slots(ids, slots=[0, 1], lengths=[40, 12], last_token_logits=True)
+    runner.prefill_slots(_prompt(2, 48, 6201), slots=[0, 1], lengths=[30, 48], last_token_logits=True)   # continuation
+    runner.release_slots([0, 1])
+    runner.prefill_slots(_prompt(2, 48, 6202), slots=[0, 1], lengths=[30, 48])
+    runner.release_slots([0, 1])
+    assert runner.prefill_graph_replay_counts[(2, 48)] == 3
+    with pytest.raises(ValueError, match="rows must be in"):
+        runner.capture_prefill(rows=9, width=16)
