@@ -93,6 +93,11 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     constexpr int kTileTokens = kSets * kSetTokens;      // query tokens per workgroup
     constexpr int kKeyRow = D + 8;                       // BF16 elements per key row: 144 bytes, conflict-free 16-byte reads
     __shared__ __attribute__((aligned(16))) uint16_t k_page[2][2][P][kKeyRow];   // [buffer][page of the pair][token][dim]
+    // What the BF16 rounding of a decoded key leaves behind, as a second BF16 value: the scores take both
+    // parts (two matrix instructions instead of one).  Of the roundings on this kernel's way (keys, softmax
+    // weights and values to BF16 for the matrix cores, the output to BF16) the keys' moves the result most:
+    // it sits in the exponent of every weight.
+    __shared__ __attribute__((aligned(16))) uint16_t k_rest[2][2][P][kKeyRow];
     // transposed: [dim][token], rows of 40 bytes, and the rows of dims 32..63 keep their two halves of
     // eight tokens swapped: the 64 lanes of a decode wavefront (8 tokens x 8 blocks) that store one
     // value each then hit 16 banks instead of 4, and the 8-byte fragment reads stay aligned
@@ -194,20 +199,28 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
         const uint32_t ids = (uint32_t)side_ids[word >> 2] | (hinted ? (uint32_t)side_hints[word >> 1] << 8 : 0u);
         return ColdOperands{side_codes[word], ids, side_norms[page * page_rows + (uint32_t)row_in_page]};
     };
+    struct Staged { uint4 value, rest; };               // eight BF16 values, and for keys what their rounding left
     auto decode_cold = [&](const ColdOperands &operands) {
         float v[8];
         if (hinted) decode_codeword_hinted(operands.code, (operands.ids >> (8 + 4 * (dec_blk & 1))) & 15u, v);
         else decode_codeword<false>(operands.code, 14.0f, 0u, v);
         const float beta = beta_table[(operands.ids >> (2 * (dec_blk & 3))) & 3];
         const float back = operands.norm / sqrt_d;
-        const bf16x2 h0 = pack_bf16x2((v[0] * beta) * back, (v[1] * beta) * back);
-        const bf16x2 h1 = pack_bf16x2((v[2] * beta) * back, (v[3] * beta) * back);
-        const bf16x2 h2 = pack_bf16x2((v[4] * beta) * back, (v[5] * beta) * back);
-        const bf16x2 h3 = pack_bf16x2((v[6] * beta) * back, (v[7] * beta) * back);
-        return make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
-                          __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = (v[j] * beta) * back;
+        uint32_t head[4], rest[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 4; j++) head[j] = __builtin_bit_cast(uint32_t, pack_bf16x2(v[2 * j], v[2 * j + 1]));
+        if (!decodes_values) {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                rest[j] = __builtin_bit_cast(uint32_t, pack_bf16x2(v[2 * j] - __uint_as_float(head[j] << 16),
+                                                                   v[2 * j + 1] - __uint_as_float(head[j] & 0xffff0000u)));
+        }
+        return Staged{make_uint4(head[0], head[1], head[2], head[3]), make_uint4(rest[0], rest[1], rest[2], rest[3])};
     };
-    auto write_page = [&](int buf, int half, const uint4 packed) {
+    auto write_page = [&](int buf, int half, const Staged &staged) {
+        const uint4 packed = staged.value;
         if (decodes_values) {
             const uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
 #pragma unroll
@@ -217,6 +230,7 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
             }
         } else {
             *reinterpret_cast<uint4 *>(&k_page[buf][half][dec_token][dec_blk * 8]) = packed;
+            *reinterpret_cast<uint4 *>(&k_rest[buf][half][dec_token][dec_blk * 8]) = staged.rest;
         }
     };
     auto tokens_of = [&](int ordinal) {
@@ -228,13 +242,16 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     // kMasked = false when all 32 tokens exist and are visible to every vector of the tile
     auto attend = [&](auto masked, int buf, int first) {
         constexpr bool kMasked = decltype(masked)::value;
-        bf16x8 k_frag[2][2];
+        bf16x8 k_frag[2][2], k_rest_frag[2][2];
 #pragma unroll
         for (int half = 0; half < 2; half++)
 #pragma unroll
-            for (int step = 0; step < 2; step++)
+            for (int step = 0; step < 2; step++) {
                 k_frag[half][step] = __builtin_bit_cast(
                     bf16x8, *reinterpret_cast<const uint4 *>(&k_page[buf][half][lane & 15][32 * step + 8 * quarter]));
+                k_rest_frag[half][step] = __builtin_bit_cast(
+                    bf16x8, *reinterpret_cast<const uint4 *>(&k_rest[buf][half][lane & 15][32 * step + 8 * quarter]));
+            }
         bf16x8 v_frag[4];
 #pragma unroll
         for (int tile = 0; tile < 4; tile++) {
@@ -250,8 +267,10 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
             for (int half = 0; half < 2; half++) {
                 floatx4 st = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int step = 0; step < 2; step++)
+                for (int step = 0; step < 2; step++) {
+                    st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_rest_frag[half][step], q_frag[i][step], st, 0, 0, 0);
                     st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag[half][step], q_frag[i][step], st, 0, 0, 0);
+                }
                 const int tokens_here = kMasked ? tokens_of(first + half) : P;
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
@@ -312,12 +331,12 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     for (int first = fast_pages; first < pages_needed; first += 2, trip++) {
         {
             const int ordinal = first + dec_half;
-            uint4 packed = make_uint4(0, 0, 0, 0);
+            Staged staged{make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
             if (dec_token < tokens_of(ordinal)) {
-                if (ordinal < page_count) packed = decode_cold(request_cold(ordinal));
-                else packed = *reinterpret_cast<const uint4 *>(side_hot);
+                if (ordinal < page_count) staged = decode_cold(request_cold(ordinal));
+                else staged.value = *reinterpret_cast<const uint4 *>(side_hot);      // BF16 rows: nothing left behind
             }
-            write_page(trip & 1, dec_half, packed);
+            write_page(trip & 1, dec_half, staged);
         }
         __syncthreads();
         attend(std::true_type{}, trip & 1, first);

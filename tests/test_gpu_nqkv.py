@@ -368,7 +368,7 @@ def test_prefill_attention_over_the_packed_cache(kv, oracle, q_heads, split_cont
     decode = kv.nqkv_decode_attention_batched_k1(
         query[:, counts[i] - 1].contiguous(), manager.layers[0], slot_ids=manager.step_slot_ids[:4].clone(),
         active_mask=torch.tensor([True, False, False, False], device="cuda"))
-    assert relative_error(_f32(out[i, counts[i] - 1]), _f32(decode[0])) <= 2e-2
+    assert relative_error(_f32(out[i, counts[i] - 1]), _f32(decode[0])) <= 1e-2
 
 
 def test_prefill_attention_with_the_context_split_over_workgroups(kv, oracle):

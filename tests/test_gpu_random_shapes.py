@@ -6,8 +6,9 @@ The fixed cases of the other files pin the shapes the model uses; these pin what
 Bars: codes, beta ids, norms and the BF16 decode of the encoder bit-exact; linears <= 1e-2 against
 the oracle's FP32 product and <= 2e-3 against its product of BF16-rounded operands (5e-3 for
 K <= 256, where a single weight that rounds to the neighbouring BF16 value weighs that much);
-decode attention <= 1e-2; prefill attention <= 2e-2 (its products run on the matrix cores with BF16
-weights and values, and a head whose value terms cancel loses that much of the result)."""
+decode and prefill attention <= 1e-2 (the prefill kernel's products run on the matrix cores with BF16
+operands: its scores take each decoded key as two BF16 parts, without which a head whose value terms
+cancel reached 1.3e-2)."""
 
 import numpy as np
 import pytest
@@ -171,7 +172,7 @@ def test_kv_writer_and_attention_over_random_batches(kv, oracle, sweep_seed):
                 for t in (0, tokens - 1):
                     visible = lengths[row] - tokens + t + 1
                     ref = oracle.attention_dense(_f32(queries[row, t].cpu()), views[s][0][:visible], views[s][1][:visible])
-                    assert relative_error(_f32(got[row, t]), ref) <= 2e-2, ("prefill attention", split, row, t, case)
+                    assert relative_error(_f32(got[row, t]), ref) <= 1e-2, ("prefill attention", split, row, t, case)
 
 
 @pytest.mark.parametrize("sweep_seed", [3, 41])
