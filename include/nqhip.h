@@ -371,6 +371,26 @@ int nq_nqkv_advance(const int32_t *slot_ids_dev, const uint8_t *active_mask_dev,
                     int32_t *hot_lengths_dev, void *stream);
 
 /*
+ * The head of a step that writes prompts (or further chunks of them) in one launch.  `record` is
+ * int32 [3, batch] as the host describes the step: row r writes its first record[1][r] tokens
+ * (clamped to [0, width]) into slot record[0][r]; record[2][r] != 0 says the slot starts a new
+ * sequence, whose four table entries restart at zero and whose cache_active flag is set.  The
+ * launch leaves the row state where nq_nqkv_write and the attention entries read it
+ * (step_slot_ids, step_counts int32 [batch]; step_active uint8 [batch] = the row writes something),
+ * fills positions[r, c] = tokens the slot held + c (int64 [batch, width], may be NULL) and
+ * last_token[r] = count - 1 (int64 [batch], 0 for a row that writes nothing; may be NULL), and
+ * advances the tables as nq_nqkv_advance does.  Rows must name distinct slots.  Replaces, for a
+ * prompt step, the slot reset, the row-state copies and the metadata update of
+ * nestquant/runtime/nqkv_batched_hf_backend.py:147-280 and nqkv_batch_manager.py:394-422, 245-285
+ * (about twenty small launches and copies through the tensor library).
+ */
+int nq_prompt_step_begin(const int32_t *record_dev, int batch, int width, int slots, int page_size,
+                         int max_tokens, int32_t *step_slot_ids_dev, int32_t *step_counts_dev,
+                         uint8_t *step_active_dev, int32_t *sequence_lengths_dev, int32_t *page_counts_dev,
+                         int32_t *last_page_lens_dev, int32_t *hot_lengths_dev, uint8_t *cache_active_dev,
+                         int64_t *positions_dev, int64_t *last_token_dev, void *stream);
+
+/*
  * The head of a decode step in one launch: nq_nqkv_advance with a count of one token per row,
  * embedded[r] = embedding[tokens[r]] (BF16 rows of `hidden` values; a token outside [0, vocab)
  * embeds as zero) and the rotary embedding's rows of positions[r] (clamped to the table):

@@ -60,6 +60,7 @@ SIGNATURES = {
     "nq_bf16_gemm": (_i32, [_ptr, _ptr, _i64, _i64, _i64, _ptr, _i32, _i32, _ptr, _size, _ptr]),
     "nq_bf16_gemm_split": (_i32, [_ptr, _ptr, _i64, _i64, _ptr, _ptr, _i32, _i32, _ptr]),
     "nq_nqkv_advance": (_i32, [_ptr, _ptr, _ptr, _i32, _i32, _i32, _i32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "nq_prompt_step_begin": (_i32, [_ptr] + [_i32] * 5 + [_ptr] * 11),
     "nq_decode_step_begin": (_i32, [_ptr, _ptr, _i32, _i32, _i32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i32,
                                     _ptr, _ptr, _ptr, _i64, _i32, _ptr, _ptr]),
     "nq_nqkv_write": (_i32, [_ptr, _ptr, _i32, _ptr, _ptr, _ptr, _i32, _ptr, _ptr] + [_ptr] * 6

@@ -49,6 +49,51 @@ kv_advance_kernel(const int32_t *__restrict__ slot_ids, const uint8_t *__restric
     hot_lengths[slot] = length % page_size;
 }
 
+// One launch at the head of a step that writes prompts: workgroup r takes row r of `record` (the host's
+// description of the step: slot, tokens to write, whether the slot starts a new sequence), resets a new
+// sequence's tables, leaves the step's row state where the writer and the attention read it, fills the
+// row's positions and the index of its last token, and advances the slot's tables as kv_advance_kernel.
+struct PromptBeginArgs {
+    const int32_t *record;          // [3][batch]: slot, count, fresh
+    int batch, width, slots, page_size, max_tokens;
+    int32_t *step_slot_ids, *step_counts;
+    uint8_t *step_active;
+    int32_t *sequence_lengths, *page_counts, *last_page_lens, *hot_lengths;
+    uint8_t *cache_active;
+    int64_t *positions;             // [batch][width], or null
+    int64_t *last_token;            // [batch], or null
+};
+
+__global__ void __launch_bounds__(256) prompt_begin_kernel(PromptBeginArgs a) {
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const int slot = a.record[r];
+    int count = a.record[a.batch + r];
+    const bool fresh = a.record[2 * a.batch + r] != 0;
+    const bool known = slot >= 0 && slot < a.slots;
+    if (count < 0) count = 0;
+    if (count > a.width) count = a.width;
+    // every lane reads the length before lane 0 stores the new one (a new sequence starts at zero)
+    const int start = known && !fresh ? a.sequence_lengths[slot] : 0;
+    __syncthreads();
+    if (a.positions)
+        for (int c = tid; c < a.width; c += blockDim.x) a.positions[(int64_t)r * a.width + c] = (int64_t)start + c;
+    if (tid != 0) return;
+    a.step_slot_ids[r] = slot;
+    a.step_counts[r] = count;
+    a.step_active[r] = count > 0;
+    if (a.last_token) a.last_token[r] = count > 0 ? count - 1 : 0;
+    if (!known) return;
+    if (fresh) a.cache_active[slot] = 1;
+    if (!fresh && count == 0) return;
+    int length = start;
+    if (length + count > a.max_tokens) count = a.max_tokens - length;   // clamp at capacity
+    length += count;
+    a.sequence_lengths[slot] = length;
+    a.page_counts[slot] = length / a.page_size;
+    a.last_page_lens[slot] = length >= a.page_size ? a.page_size : 0;
+    a.hot_lengths[slot] = length % a.page_size;
+}
+
 // One launch at the head of a decode step: workgroup r advances row r's tables by one token
 // (as kv_advance_kernel), copies the embedding row of its input token and the rotary
 // embedding's cos and sin rows of its position.
@@ -314,6 +359,28 @@ extern "C" int nq_nqkv_advance(const int32_t *slot_ids_dev, const uint8_t *activ
                        slot_ids_dev, active_mask_dev, counts_dev, uniform_count, batch, slots, page_size, max_tokens,
                        sequence_lengths_dev, page_counts_dev, last_page_lens_dev, hot_lengths_dev);
     return nq::check_launch("nq_nqkv_advance");
+}
+
+extern "C" int nq_prompt_step_begin(const int32_t *record_dev, int batch, int width, int slots, int page_size,
+                                    int max_tokens, int32_t *step_slot_ids_dev, int32_t *step_counts_dev,
+                                    uint8_t *step_active_dev, int32_t *sequence_lengths_dev, int32_t *page_counts_dev,
+                                    int32_t *last_page_lens_dev, int32_t *hot_lengths_dev, uint8_t *cache_active_dev,
+                                    int64_t *positions_dev, int64_t *last_token_dev, void *stream) {
+    NQ_REQUIRE(batch >= 1 && batch <= 65535 && width >= 1 && slots >= 1 && page_size >= 1 && max_tokens >= 1,
+               NQ_ERR_SHAPE,
+               "nq_prompt_step_begin: batch (at most 65535), width, slots, page_size and max_tokens must be positive");
+    NQ_REQUIRE(record_dev && step_slot_ids_dev && step_counts_dev && step_active_dev && sequence_lengths_dev &&
+                   page_counts_dev && last_page_lens_dev && hot_lengths_dev && cache_active_dev,
+               NQ_ERR_ARGUMENT, "nq_prompt_step_begin: null pointer");
+    nq::PromptBeginArgs a;
+    a.record = record_dev;
+    a.batch = batch; a.width = width; a.slots = slots; a.page_size = page_size; a.max_tokens = max_tokens;
+    a.step_slot_ids = step_slot_ids_dev; a.step_counts = step_counts_dev; a.step_active = step_active_dev;
+    a.sequence_lengths = sequence_lengths_dev; a.page_counts = page_counts_dev;
+    a.last_page_lens = last_page_lens_dev; a.hot_lengths = hot_lengths_dev; a.cache_active = cache_active_dev;
+    a.positions = positions_dev; a.last_token = last_token_dev;
+    hipLaunchKernelGGL(nq::prompt_begin_kernel, dim3((unsigned)batch), dim3(256), 0, (hipStream_t)stream, a);
+    return nq::check_launch("nq_prompt_step_begin");
 }
 
 extern "C" int nq_decode_step_begin(const int32_t *slot_ids_dev, const uint8_t *active_mask_dev, int batch, int slots,

@@ -339,6 +339,9 @@ class BatchedNQKVMetadata:
     hot_lengths: torch.Tensor
     sequence_lengths: torch.Tensor
     active_mask: torch.Tensor
+    # the four per-slot counters as rows of one int32 [4, capacity] tensor (None when they were
+    # allocated one by one): a run of slots is then reset with one fill instead of four
+    counters: torch.Tensor | None = None
 
     @classmethod
     def create(cls, *, capacity: int, max_pages_per_sequence: int,
@@ -347,14 +350,14 @@ class BatchedNQKVMetadata:
             if isinstance(value, bool) or not isinstance(value, int) or value < 1:
                 raise ValueError(f"{name} must be a positive integer")
         target = torch.device(device)
-        zeros = lambda: torch.zeros(capacity, dtype=torch.int32, device=target)   # noqa: E731
+        counters = torch.zeros((4, capacity), dtype=torch.int32, device=target)
         return cls(
             slot_ids=torch.arange(capacity, dtype=torch.int32, device=target),
             page_indptr=torch.arange(0, (capacity + 1) * max_pages_per_sequence, max_pages_per_sequence,
                                      dtype=torch.int32, device=target),
             page_indices=torch.full((capacity, max_pages_per_sequence), -1, dtype=torch.int32, device=target),
-            page_counts=zeros(), last_page_lens=zeros(), hot_lengths=zeros(), sequence_lengths=zeros(),
-            active_mask=torch.zeros(capacity, dtype=torch.bool, device=target),
+            page_counts=counters[0], last_page_lens=counters[1], hot_lengths=counters[2], sequence_lengths=counters[3],
+            active_mask=torch.zeros(capacity, dtype=torch.bool, device=target), counters=counters,
         )
 
     def pointers(self) -> tuple[int, ...]:
@@ -824,13 +827,20 @@ class BatchedNQKVCacheManager:
         self.step_counts = torch.zeros(capacity, dtype=torch.int32, device=target)
         self._step_rows = capacity
         self._step_uniform: int | None = 1
+        # a prompt step's description on its way to the device: pinned host words, their device copy, and
+        # the event that says the last copy has left the host words
+        self._prompt_record: torch.Tensor | None = None
+        self._prompt_stage: torch.Tensor | None = None
+        self._prompt_stage_free: torch.cuda.Event | None = None
 
     # -- slots ---------------------------------------------------------------------------
     def register(self, sequence_id: Hashable, *, slot: int) -> None:
         self.register_batch([(sequence_id, slot)])
 
-    def register_batch(self, assignments: Sequence[tuple[Hashable, int]]) -> None:
-        """All-or-nothing: every assignment is checked before the first slot is taken."""
+    def register_batch(self, assignments: Sequence[tuple[Hashable, int]], *, reset_tables: bool = True) -> None:
+        """All-or-nothing: every assignment is checked before the first slot is taken.  With
+        `reset_tables=False` the slots' device tables are left to the `begin_prompt_step` that must
+        follow and name these slots as fresh."""
         assignments = list(assignments)
         slots = [slot for _, slot in assignments]
         names = [name for name, _ in assignments]
@@ -842,11 +852,12 @@ class BatchedNQKVCacheManager:
             raise RuntimeError("slot is already occupied")          # nqkv_batch_manager.py:398-399
         for name, slot in assignments:
             self._sequence_of_slot[slot] = name
-        self._reset_slot_tables(slots, active=True)
+        if reset_tables:
+            self._reset_slot_tables(slots, active=True)
 
     def _reset_slot_tables(self, slots: Sequence[int], *, active: bool) -> None:
         """Zero lengths and counts of `slots` and set their activity flag: one fill per table and run
-        of neighbouring slots (a batch admitted into slots 0..b-1 costs five launches, not 5 b)."""
+        of neighbouring slots (a batch admitted into slots 0..b-1 costs two launches, not 5 b)."""
         ordered = sorted(slots)
         meta = self.metadata
         start = 0
@@ -856,8 +867,11 @@ class BatchedNQKVCacheManager:
                 stop += 1
             first, last = ordered[start], ordered[stop] + 1
             meta.active_mask[first:last] = active
-            for tensor in (meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths):
-                tensor[first:last] = 0
+            if meta.counters is not None:
+                meta.counters[:, first:last] = 0
+            else:
+                for tensor in (meta.sequence_lengths, meta.page_counts, meta.last_page_lens, meta.hot_lengths):
+                    tensor[first:last] = 0
             start = stop + 1
 
     def release_slots(self, slots: Sequence[int]) -> tuple[Hashable, ...]:
@@ -888,6 +902,41 @@ class BatchedNQKVCacheManager:
             0 if uniform_count is None else uniform_count, rows, self.capacity, self.page_size, self.max_tokens,
             meta.sequence_lengths.data_ptr(), meta.page_counts.data_ptr(), meta.last_page_lens.data_ptr(),
             meta.hot_lengths.data_ptr(), _native.stream_handle(self.device)))
+
+    def begin_prompt_step(self, *, slot_ids: Sequence[int], counts: Sequence[int], fresh: Sequence[bool], width: int,
+                          positions: torch.Tensor | None = None, last_token: torch.Tensor | None = None) -> None:
+        """The head of a step that writes prompts, as one copy and one launch: row i writes its first
+        counts[i] tokens into slot_ids[i]; `fresh[i]` restarts that slot's tables at zero and marks it
+        active (a sequence registered with `reset_tables=False`).  Leaves step_slot_ids / step_counts /
+        step_active as `set_batch_state` would, advances the tables as `begin_step` and fills, when
+        given, positions [rows, width] (tokens held + column) and last_token [rows] (count - 1), both
+        int64 on the device.  Host lists go to the device through pinned words, so nothing here waits."""
+        rows = len(slot_ids)
+        if not 1 <= rows <= self.capacity or len(counts) != rows or len(fresh) != rows:
+            raise ValueError("slot_ids, counts and fresh must describe 1..capacity rows")
+        for name, tensor, shape in (("positions", positions, (rows, width)), ("last_token", last_token, (rows,))):
+            if tensor is not None and (tensor.dtype != torch.int64 or tuple(tensor.shape) != shape
+                                       or not tensor.is_contiguous() or tensor.device != self.device):
+                raise ValueError(f"{name} must be contiguous int64 {shape} on the cache's device")
+        if self._prompt_record is None:
+            self._prompt_record = torch.zeros(3 * self.capacity, dtype=torch.int32, device=self.device)
+            self._prompt_stage = torch.zeros(3 * self.capacity, dtype=torch.int32, pin_memory=True)
+            self._prompt_stage_free = torch.cuda.Event()
+        else:
+            self._prompt_stage_free.synchronize()             # the previous step's copy has read the words
+        words = [int(s) for s in slot_ids] + [int(c) for c in counts] + [int(bool(f)) for f in fresh]
+        self._prompt_stage[:3 * rows] = torch.tensor(words, dtype=torch.int32)
+        self._prompt_record[:3 * rows].copy_(self._prompt_stage[:3 * rows], non_blocking=True)
+        self._prompt_stage_free.record(torch.cuda.current_stream(self.device))
+        self._step_rows, self._step_uniform = rows, None
+        meta = self.metadata
+        _native.check(_native.library().nq_prompt_step_begin(
+            self._prompt_record.data_ptr(), rows, width, self.capacity, self.page_size, self.max_tokens,
+            self.step_slot_ids.data_ptr(), self.step_counts.data_ptr(), self.step_active.data_ptr(),
+            meta.sequence_lengths.data_ptr(), meta.page_counts.data_ptr(), meta.last_page_lens.data_ptr(),
+            meta.hot_lengths.data_ptr(), meta.active_mask.data_ptr(),
+            None if positions is None else positions.data_ptr(),
+            None if last_token is None else last_token.data_ptr(), _native.stream_handle(self.device)))
 
     def begin_decode_step(self, *, rows: int, tokens: torch.Tensor, embedding: torch.Tensor,
                           positions: torch.Tensor, rotary: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:

@@ -71,9 +71,9 @@ class BatchedNQKVLlamaCache(Cache):
         self.manager.register(sequence_id, slot=slot)
         self._host_lengths[slot] = 0
 
-    def register_batch(self, assignments: Sequence[tuple[Hashable, int]]) -> None:
+    def register_batch(self, assignments: Sequence[tuple[Hashable, int]], *, reset_tables: bool = True) -> None:
         assignments = list(assignments)
-        self.manager.register_batch(assignments)
+        self.manager.register_batch(assignments, reset_tables=reset_tables)
         for _, slot in assignments:
             self._host_lengths[slot] = 0
 
@@ -85,7 +85,8 @@ class BatchedNQKVLlamaCache(Cache):
     # -- step state ------------------------------------------------------------------------
     def set_batch_state(self, *, slot_ids: Sequence[int] | None = None, counts: Sequence[int] | None = None,
                         active_mask: torch.Tensor | None = None, write_mask: torch.Tensor | None = None,
-                        width: int | None = None) -> None:
+                        width: int | None = None, fresh: Sequence[int] | None = None,
+                        positions: torch.Tensor | None = None, last_token: torch.Tensor | None = None) -> None:
         """Eager (prefill) step.  Two forms:
           * slot_ids / counts: row i writes its first counts[i] tokens into slot_ids[i] (`width`, when
             given, bounds every count);
@@ -93,7 +94,9 @@ class BatchedNQKVLlamaCache(Cache):
             bool [capacity] and bool [capacity, width]; row r is slot r and writes the prefix of
             `write_mask[r]` (masks that are not prefixes are rejected).
         Validates before anything changes, copies the row state to the fixed step tensors and advances
-        the device tables."""
+        the device tables.  With `fresh` (first form, `width` given: the slots among slot_ids whose
+        sequences were registered with `reset_tables=False`) all of that is one copy and one launch
+        (`BatchedNQKVCacheManager.begin_prompt_step`), which also fills `positions` and `last_token`."""
         if write_mask is not None or active_mask is not None:
             if slot_ids is not None or counts is not None:
                 raise ValueError("give slot_ids / counts or active_mask / write_mask, not both")
@@ -131,13 +134,23 @@ class BatchedNQKVLlamaCache(Cache):
                 raise RuntimeError("sequence would exceed max_cache_len")
         self._continuation = any(self._host_lengths[slot] > 0 and count > 0 for slot, count in zip(slot_ids, counts))
         m = self.manager
-        m.step_slot_ids[:rows].copy_(torch.tensor(slot_ids, dtype=torch.int32))
-        m.step_counts[:rows].copy_(torch.tensor(counts, dtype=torch.int32))
-        m.step_active[:rows].copy_(torch.tensor([c > 0 for c in counts]))
+        if fresh is not None:
+            if width is None:
+                raise ValueError("the one-launch form needs `width`")
+            starting = set(int(slot) for slot in fresh)
+            m.begin_prompt_step(slot_ids=slot_ids, counts=counts, fresh=[slot in starting for slot in slot_ids],
+                                width=width, positions=positions, last_token=last_token)
+        else:
+            if positions is not None or last_token is not None:
+                raise ValueError("positions / last_token are filled by the one-launch form (`fresh`) only")
+            m.step_slot_ids[:rows].copy_(torch.tensor(slot_ids, dtype=torch.int32))
+            m.step_counts[:rows].copy_(torch.tensor(counts, dtype=torch.int32))
+            m.step_active[:rows].copy_(torch.tensor([c > 0 for c in counts]))
         for slot, count in zip(slot_ids, counts):
             self._host_lengths[slot] += count
         self._rows, self._tokens = rows, max(counts)
-        m.begin_step(rows=rows, uniform_count=None)
+        if fresh is None:
+            m.begin_step(rows=rows, uniform_count=None)
 
     def fail_closed(self, slots: Sequence[int]) -> None:
         """After a forward that raised: the step's table advance is not backed by keys and values in
@@ -516,10 +529,8 @@ class BatchedNQKVLlamaRunner:
         for slot, length in zip(slots, lengths):
             if self.cache._host_lengths[slot] + length > self.max_cache_len:
                 raise RuntimeError("sequence would exceed max_cache_len")
-        if positions is None:
-            starts = torch.tensor([self.cache._host_lengths[s] for s in slots], device=self.device)
-            positions = starts[:, None] + torch.arange(width, device=self.device)[None, :]
-        else:
+        one_launch = positions is None          # the step's head as one copy and one launch, positions included
+        if positions is not None:
             if positions.dtype != torch.long or tuple(positions.shape) != (rows, width) or positions.device != self.device:
                 raise ValueError("positions must be torch.long [rows, width] on the model device")
             written = torch.arange(width, device=self.device)[None, :] < torch.tensor(lengths, device=self.device)[:, None]
@@ -536,21 +547,37 @@ class BatchedNQKVLlamaRunner:
         fresh = [slot for slot in slots if self.cache.manager.sequence_id(slot) is None]
         for slot in fresh:
             self._generation[slot] += 1
-        self.cache.register_batch([(f"slot-{slot}-generation-{self._generation[slot]}", slot) for slot in fresh])
+        self.cache.register_batch([(f"slot-{slot}-generation-{self._generation[slot]}", slot) for slot in fresh],
+                                  reset_tables=not one_launch)
         self._decode_state = None
-        self.cache.set_batch_state(slot_ids=slots, counts=lengths, width=width)
+        continuation = any(self.cache._host_lengths[slot] > 0 and length > 0 for slot, length in zip(slots, lengths))
+        captured = None
+        if last_token_logits and not continuation and not self.cache.packed_prefill:
+            captured = self._prefill_graphs.get((rows, width))
         keep = None
-        if last_token_logits:
-            keep = torch.tensor([length - 1 for length in lengths], dtype=torch.long, device=self.device)
+        if one_launch:
+            if captured is not None:
+                positions, keep = captured[2], captured[3]           # the graph's own inputs, filled in place
+            else:
+                positions = torch.empty((rows, width), dtype=torch.long, device=self.device)
+                keep = torch.empty(rows, dtype=torch.long, device=self.device) if last_token_logits else None
+            try:
+                self.cache.set_batch_state(slot_ids=slots, counts=lengths, width=width, fresh=fresh,
+                                           positions=positions, last_token=keep)
+            except Exception:
+                self.cache.release_slots(fresh)                      # registered above, tables never reset
+                raise
+        else:
+            self.cache.set_batch_state(slot_ids=slots, counts=lengths, width=width)
+            if last_token_logits:
+                keep = torch.tensor([length - 1 for length in lengths], dtype=torch.long, device=self.device)
         try:
-            captured = None
-            if keep is not None and not self.cache._continuation and not self.cache.packed_prefill:
-                captured = self._prefill_graphs.get((rows, width))
             if captured is not None:
                 graph, graph_ids, graph_positions, graph_keep, logits = captured
                 graph_ids.copy_(input_ids)
-                graph_positions.copy_(positions)
-                graph_keep.copy_(keep)
+                if not one_launch:
+                    graph_positions.copy_(positions)
+                    graph_keep.copy_(keep)
                 graph.replay()
                 self.prefill_graph_replay_counts[(rows, width)] += 1
                 return logits.clone()

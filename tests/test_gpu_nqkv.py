@@ -558,6 +558,57 @@ def test_decode_step_begin_is_advance_plus_two_gathers():
     assert torch.equal(rotary_rows, rotary.index_select(1, positions.view(-1).clamp(0, max_pos - 1)))
 
 
+def test_prompt_step_begin_equals_reset_copies_and_advance(kv):
+    """A scripted run of prompt steps (new sequences into free slots, further chunks into slots that hold
+    tokens, rows that write nothing, slots released and taken again, a slot filled to capacity) through two
+    managers: one resets, copies and advances with tensor operations and nq_nqkv_advance, the other does the
+    step's head as one copy and one launch.  Tables, row state, positions and last-token indices agree."""
+    rng = np.random.default_rng(4242)
+    capacity, max_len = 8, 96
+    plain, fused = _manager(kv, capacity, max_len), _manager(kv, capacity, max_len)
+    held = [None] * capacity                                   # tokens per slot on the host, None = free
+    generation = 0
+    for step in range(120):
+        rows = int(rng.integers(1, capacity + 1))
+        slots = [int(s) for s in rng.permutation(capacity)[:rows]]
+        width = int(rng.choice([1, 7, 16, 33, 96]))
+        fresh = [s for s in slots if held[s] is None]
+        counts = []
+        for s in slots:
+            room = max_len - (held[s] or 0)
+            counts.append(int(min(room, rng.integers(0, width + 1))) if rng.random() > 0.15 else 0)
+        generation += 1
+        for manager, reset in ((plain, True), (fused, False)):
+            manager.register_batch([((generation, s), s) for s in fresh], reset_tables=reset)
+        starts = torch.tensor([held[s] or 0 for s in slots])
+        plain.step_slot_ids[:rows].copy_(torch.tensor(slots, dtype=torch.int32))
+        plain.step_counts[:rows].copy_(torch.tensor(counts, dtype=torch.int32))
+        plain.step_active[:rows].copy_(torch.tensor([c > 0 for c in counts]))
+        plain.begin_step(rows=rows, uniform_count=None)
+        positions = torch.full((rows, width), -1, dtype=torch.long, device="cuda")
+        last = torch.full((rows,), -1, dtype=torch.long, device="cuda")
+        fused.begin_prompt_step(slot_ids=slots, counts=counts, fresh=[s in fresh for s in slots], width=width,
+                                positions=positions, last_token=last)
+        for s, c in zip(slots, counts):
+            held[s] = (held[s] or 0) + c
+        for name in ("sequence_lengths", "page_counts", "last_page_lens", "hot_lengths", "active_mask"):
+            assert torch.equal(getattr(fused.metadata, name), getattr(plain.metadata, name)), (step, name)
+        for name in ("step_slot_ids", "step_counts", "step_active"):
+            assert torch.equal(getattr(fused, name)[:rows], getattr(plain, name)[:rows]), (step, name)
+        assert fused.metadata.sequence_lengths.tolist() == [h or 0 for h in held]
+        assert torch.equal(positions.cpu(), starts[:, None] + torch.arange(width)[None, :]), step
+        assert last.tolist() == [max(c - 1, 0) for c in counts]
+        gone = [s for s in range(capacity) if held[s] is not None and rng.random() < 0.2]
+        for manager in (plain, fused):
+            manager.release_slots(gone)
+        for s in gone:
+            held[s] = None
+    assert max(h or 0 for h in held) <= max_len
+    with pytest.raises(ValueError, match="int64"):
+        fused.begin_prompt_step(slot_ids=[0], counts=[0], fresh=[False], width=4,
+                                positions=torch.zeros((1, 4), dtype=torch.int32, device="cuda"))
+
+
 @pytest.mark.parametrize("q_heads,max_len,steps", [(32, 256, 40), (8, 256, 20), (64, 64, 34), (16, 1024, 20),
                                                    (32, 2048, 20), (32, 16384, 18)])
 def test_append_inside_the_attention_launch_equals_writer_then_attention(kv, oracle, q_heads, max_len, steps):
