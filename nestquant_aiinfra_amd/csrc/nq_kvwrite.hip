@@ -156,8 +156,13 @@ struct KvWriteArgs {
     int batch, tokens, uniform_count, slots, max_pages, kv_heads, key_beta_count, value_beta_count, rotate_keys;
 };
 
-template <int D, int P>
-__global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
+// kPairs: one lane per (block, beta) pair on 4 x 256 lanes instead of one lane per block with its betas in
+// turn: three times the lanes for a third of a lane's instructions, the same bits.  A launch of few
+// workgroups (the pages of one short prompt) is bound by the length of that chain, a launch of many
+// by the instructions in all.
+template <int D, int P, bool kPairs>
+__global__ void __launch_bounds__(kPairs ? 4 * kKvThreads : kKvThreads) kv_write_kernel(KvWriteArgs a) {
+    constexpr int kThreads = kPairs ? 4 * kKvThreads : kKvThreads;
     constexpr int kBlocks = D / 8;
     __shared__ float rows[2 * P][D];             // K tokens 0..P-1, then V tokens
     __shared__ float row_scale[2 * P], row_norm[2 * P];
@@ -196,7 +201,7 @@ __global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
         const int page_tokens = complete ? P : length - page_start;      // tokens of this page that exist
         const int first_new = start > page_start ? start - page_start : 0;
         // stage the page's tokens as float32: hot tail first, then the new rows
-        for (int i = tid; i < 2 * P * (D / 8); i += kKvThreads) {
+        for (int i = tid; i < 2 * P * (D / 8); i += kThreads) {
             const int which = i / (P * (D / 8)), rem = i % (P * (D / 8));
             const int t = rem / (D / 8), c = rem % (D / 8);
             float *dst = &rows[which * P + t][c * 8];
@@ -222,7 +227,7 @@ __global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
             // rotary position embedding of the new key rows in BF16 tensor arithmetic:
             // (k * cos) + (rotate_half(k) * sin), every product and the sum rounded to BF16
             const int new_rows = page_tokens - first_new;
-            for (int i = tid; i < new_rows * (D / 2); i += kKvThreads) {
+            for (int i = tid; i < new_rows * (D / 2); i += kThreads) {
                 const int r = first_new + i / (D / 2), k = i % (D / 2);
                 const int64_t at = ((int64_t)row * a.tokens + (page_start + r - start)) * D;
                 const float c_lo = bf16_to_f32(a.rope_cos[at + k]), c_hi = bf16_to_f32(a.rope_cos[at + k + D / 2]);
@@ -238,7 +243,7 @@ __global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
             // hadamard(key.float()).to(bfloat16) (nestquant/runtime/nqkv_batched_hf_backend.py:381)
             const int new_rows = page_tokens - first_new;
             for (int width = 1; width < D; width <<= 1) {
-                for (int i = tid; i < new_rows * (D / 2); i += kKvThreads) {
+                for (int i = tid; i < new_rows * (D / 2); i += kThreads) {
                     const int r = first_new + i / (D / 2), k = i % (D / 2);
                     const int x = (k / width) * 2 * width + (k % width), y = x + width;
                     const float left = rows[r][x], right = rows[r][y];
@@ -248,7 +253,7 @@ __global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
                 __syncthreads();
             }
             const float inv = 1.0f / sqrt_d;
-            for (int i = tid; i < new_rows * D; i += kKvThreads) {
+            for (int i = tid; i < new_rows * D; i += kThreads) {
                 float &v = rows[first_new + i / D][i % D];
                 v = bf16_to_f32(f32_to_bf16(v * inv));
             }
@@ -256,7 +261,7 @@ __global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
         }
         if (!complete) {
             // trailing partial page: the new rows of this head go to the hot tail
-            for (int i = tid; i < 2 * (page_tokens - first_new) * (D / 8); i += kKvThreads) {
+            for (int i = tid; i < 2 * (page_tokens - first_new) * (D / 8); i += kThreads) {
                 const int which = i / ((page_tokens - first_new) * (D / 8)), rem = i % ((page_tokens - first_new) * (D / 8));
                 const int t = first_new + rem / (D / 8), c = rem % (D / 8);
                 const float *src = &rows[which * P + t][c * 8];
@@ -300,12 +305,16 @@ __global__ void __launch_bounds__(kKvThreads) kv_write_kernel(KvWriteArgs a) {
         // one lane per block, its betas in turn (the 2 P x 8 blocks of the page's key and value rows are the
         // workgroup's 256 lanes; a wavefront holds rows of one kind): fewer instructions per block than
         // a lane per (block, beta) pair, which is what a many-page prompt pays for
-        quantize_staged_blocks(&rows[0][0], row_scale, D, 14.0f, 1.0f / 14.0f, betas_of, a.key_beta_count, 0,
-                               2 * P * kBlocks, sink);
+        if (kPairs)
+            quantize_staged_pairs<false>(&rows[0][0], row_scale, D, 14.0f, 1.0f / 14.0f, betas_of, a.key_beta_count, 0u,
+                                         0, 2 * P * kBlocks * 4, sink);
+        else
+            quantize_staged_blocks(&rows[0][0], row_scale, D, 14.0f, 1.0f / 14.0f, betas_of, a.key_beta_count, 0,
+                                   2 * P * kBlocks, sink);
         if (a.key_hints) {
             // the decode hints of the page's blocks, from the code words this workgroup has just stored
             __syncthreads();
-            for (int i = tid; i < 2 * P * (kBlocks / 2); i += kKvThreads) {
+            for (int i = tid; i < 2 * P * (kBlocks / 2); i += kThreads) {
                 const int which = i / (P * (kBlocks / 2)), rem = i % (P * (kBlocks / 2));
                 const int64_t word = sink.word(rem / (kBlocks / 2), 2 * (rem % (kBlocks / 2)));
                 const uint2 pair = *reinterpret_cast<const uint2 *>((which ? a.value_codes : a.key_codes) + word);
@@ -471,8 +480,13 @@ extern "C" int nq_nqkv_write(const void *key_dev, const void *value_dev, int kv_
     a.key_hints = key_hints_dev; a.value_hints = value_hints_dev;
     // `tokens` new rows starting anywhere inside a page touch at most this many pages
     const int touched = (tokens + page_size - 2) / page_size + 1;
-    hipLaunchKernelGGL((nq::kv_write_kernel<64, 16>), dim3((unsigned)touched, (unsigned)(batch * kv_heads)),
-                       dim3(nq::kKvThreads), 0, (hipStream_t)stream, a);
+    // up to two workgroups per compute unit: the launch waits for one workgroup's chain of instructions
+    if ((int64_t)touched * batch * kv_heads <= 512 && key_beta_count <= 4 && value_beta_count <= 4)
+        hipLaunchKernelGGL((nq::kv_write_kernel<64, 16, true>), dim3((unsigned)touched, (unsigned)(batch * kv_heads)),
+                           dim3(4 * nq::kKvThreads), 0, (hipStream_t)stream, a);
+    else
+        hipLaunchKernelGGL((nq::kv_write_kernel<64, 16, false>), dim3((unsigned)touched, (unsigned)(batch * kv_heads)),
+                           dim3(nq::kKvThreads), 0, (hipStream_t)stream, a);
     return nq::check_launch("nq_nqkv_write");
 }
 
