@@ -97,8 +97,10 @@ def parse_args() -> argparse.Namespace:
                         help="another build of libnqhip.so to load (the measuring build that --only encode_phases needs: "
                              "python -m nestquant_aiinfra_amd.build --define NQ_PHASE_STAMPS --output PATH)")
     parser.add_argument("--only", choices=("tpot", "gemm", "attention", "encode", "rowlinear", "encode_phases", "attention_phases",
-                                           "gemv_phases", "pair_phases"), default=None,
+                                           "gemv_phases", "pair_phases", "prompt"), default=None,
                         help="run one of the extra measurements alone (for profiling) and print its JSON")
+    parser.add_argument("--prompt-shape", default=None,
+                        help="ROWSxWIDTH: the one prompt shape --only prompt runs (default: 1x128, 8x128 and 1x384)")
     parser.add_argument("--skip-extras", action="store_true",
                         help="only the headline GEMV workload (no prefill GEMM, attention, TPOT)")
     return parser.parse_args()
@@ -846,6 +848,55 @@ def tpot_extra(device, batches=(1, 2, 4, 8), prompt=128, generate=128):
     return results
 
 
+def prompt_extra(device, shapes=((1, 128), (8, 128), (1, 384)), repeats=10):
+    """Prompts into empty slots of the random-init Llama-3.2-1B runner, replayed from their captured graphs
+    (the last token's logits only, as an engine asks for them): median GPU time from the first host
+    operation of `prefill_slots` to the end of the graph, and the wall time to the sampled token.
+    The mode a kernel trace of a prompt is taken from."""
+    import tempfile
+
+    import torch
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from nestquant_aiinfra_amd.models import llama_w4a4kv4 as asm
+
+    torch.manual_seed(5001)
+    config = LlamaConfig(hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, num_attention_heads=32,
+                         num_key_value_heads=8, head_dim=64, vocab_size=128256, max_position_embeddings=4096,
+                         rope_theta=500000.0, tie_word_embeddings=True)
+    with torch.device(device):
+        model = LlamaForCausalLM(config).to(torch.bfloat16).eval()
+    results = {}
+    with tempfile.TemporaryDirectory() as folder:
+        path = os.path.join(folder, "llama1b_random.nqmc")
+        asm.write_w4_checkpoint(model, path)
+        runner = asm.build_w4a4kv4_runner(model, path, capacity=max(rows for rows, _ in shapes),
+                                          max_cache_len=max(width for _, width in shapes) + 64)
+        g = torch.Generator().manual_seed(5003)
+        for rows, width in shapes:
+            ids = torch.randint(0, config.vocab_size, (rows, width), generator=g).to(device)
+            slots = list(range(rows))
+            for _ in range(2):                               # the first prompt also prepares the weights
+                runner.prefill_slots(ids, slots=slots, lengths=[width] * rows, last_token_logits=True)
+                runner.release_slots(slots)
+            runner.capture_prefill(rows=rows, width=width)
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            gpu_ms, wall_ms = [], []
+            for _ in range(repeats):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                begin.record()
+                logits = runner.prefill_slots(ids, slots=slots, lengths=[width] * rows, last_token_logits=True)
+                end.record()
+                logits[:, 0].argmax(-1).tolist()
+                wall_ms.append((time.perf_counter() - t0) * 1e3)
+                gpu_ms.append(begin.elapsed_time(end))
+                runner.release_slots(slots)
+            results[f"{rows}x{width}"] = {"gpu_ms_p50": sorted(gpu_ms)[len(gpu_ms) // 2],
+                                          "wall_ms_to_token_p50": sorted(wall_ms)[len(wall_ms) // 2],
+                                          "graph_replays": runner.prefill_graph_replay_counts[(rows, width)]}
+    return results
+
+
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
@@ -912,7 +963,10 @@ def main() -> None:
                  "encode_phases": lambda: encode_phases_extra(rt, device),
                  "attention_phases": lambda: attention_phases_extra(device),
                  "gemv_phases": lambda: gemv_phases_extra(rt, device),
-                 "pair_phases": lambda: pair_phases_extra(rt, device)}[args.only]()
+                 "pair_phases": lambda: pair_phases_extra(rt, device),
+                 "prompt": lambda: prompt_extra(device, **(
+                     {"shapes": (tuple(int(v) for v in args.prompt_shape.split("x")),)} if args.prompt_shape else {}))
+                 }[args.only]()
         print(json.dumps({args.only: extra}))
         return
 
