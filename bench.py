@@ -203,6 +203,28 @@ def time_kernel_alone(rt, case, copies, launches_per_graph=None):
     return begin.elapsed_time(end) * 1e-3 / (repeats * count)
 
 
+def one_launch_per_case_extra(rt, cases, copies, step_bytes):
+    """The headline step with every case's encoder and linear in one launch (`fused_stage_linear`, mode
+    "rotated_rows": the form a decode step's pairs run in), one fill per step clearing the flag words: the
+    same outputs bit for bit (checked here), time per step from graphs over the same rotating weights."""
+    import torch
+    device = cases[0]["x"].device
+    sync = rt.StageLinearSync(device)
+
+    def one(case, copy):
+        return rt.fused_stage_linear(case["x"], [case["weights"][copy]], sync, mode="rotated_rows",
+                                     beta_table=case["table"])[0][0]
+
+    same = all(torch.equal(one(case, 0).reshape(-1), run_case(rt, case, 0).reshape(-1)) for case in cases)
+
+    def step(i):
+        sync.begin_step()
+        return [one(case, i % copies) for case in cases]
+    seconds = time_graph(step, copies)
+    return {"us_per_step": seconds * 1e6, "GBps": step_bytes / seconds / 1e9, "equals_two_launches": bool(same),
+            "waits_ran_out": bool(sync.timed_out)}
+
+
 def cpu_baseline_torch(cases, budget_s: float):
     """The same four-linear step with whole-tensor torch operations on the CPU, as the reference's own
     CPU path evaluates it: one encode + decode pass per beta over the full tensor, argmin over the
@@ -1015,6 +1037,7 @@ def main() -> None:
     }
     if not args.skip_extras:
         del graphs, keep
+        result["extra"]["one_launch_per_case"] = one_launch_per_case_extra(rt, cases, copies, step_bytes)
         for case in cases:
             case["weights"] = case["weights"][:1]
         torch.cuda.empty_cache()

@@ -545,7 +545,9 @@ int nq_attention_output_stage(const void *workspace_dev, int64_t rows, int q_hea
 /*
  * A decode step's input stage and the packed linear(s) that consume its rows, in one launch: what
  * nq_fused_input_stage (mode 1: residual + RMSNorm, mode 2: SiLU(gate) * x) or
- * nq_attention_output_stage (mode 3: attention merge) with the Hadamard rotation and q = 14 leaves
+ * nq_attention_output_stage (mode 3: attention merge) with the Hadamard rotation and q = 14, or
+ * nq_quantize_rows of the BF16 rows x_dev themselves (mode 0: rotated first, what
+ * FusedNQRTLinear.forward does with its input; mode 4: as they are, rows that were rotated already), leaves
  * in codes / beta ids / norms / decoded BF16 rows, followed by nq_w4a4_gemv_grouped of `count`
  * (1..4) resolved weights on those rows; all outputs bit for bit those of the two calls.  The first
  * rows * slices workgroups of the grid run the encoder; the others decode their weights while the

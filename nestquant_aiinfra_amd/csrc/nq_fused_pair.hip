@@ -499,8 +499,10 @@ extern "C" int nq_fused_stage_linear(
     void *stream) {
     NQ_REQUIRE(rows >= 1 && rows <= 16, NQ_ERR_SHAPE, "nq_fused_stage_linear: between 1 and 16 rows (a decode step)");
     NQ_REQUIRE(n == 2048 || n == 8192, NQ_ERR_SHAPE, "nq_fused_stage_linear: rows of 2048 or 8192 values, got %lld", (long long)n);
-    NQ_REQUIRE(mode == 1 || mode == 2 || mode == 3, NQ_ERR_ARGUMENT,
-               "nq_fused_stage_linear: mode must be 1 (residual + RMSNorm), 2 (SiLU(gate) * x) or 3 (attention merge)");
+    NQ_REQUIRE(mode >= 0 && mode <= 4, NQ_ERR_ARGUMENT,
+               "nq_fused_stage_linear: mode must be 0 (the rows as they are), 1 (residual + RMSNorm), 2 (SiLU(gate) * x), "
+               "3 (attention merge) or 4 (the rows as they are, already rotated)");
+    NQ_REQUIRE((mode != 0 && mode != 4) || x_dev, NQ_ERR_ARGUMENT, "nq_fused_stage_linear: modes 0 and 4 need the rows");
     NQ_REQUIRE(mode != 1 || (x_dev && norm_weight_dev && eps >= 0.0f && eps < 1.0f), NQ_ERR_ARGUMENT,
                "nq_fused_stage_linear: mode 1 needs the rows, the norm weight and an eps in [0, 1)");
     NQ_REQUIRE(mode != 2 || (x_dev && gate_dev), NQ_ERR_ARGUMENT, "nq_fused_stage_linear: mode 2 needs the rows and the gate rows");
@@ -583,7 +585,7 @@ extern "C" int nq_fused_stage_linear(
     e.norms = norms_dev;
     e.decoded = reinterpret_cast<uint4 *>(decoded_bf16_dev);
     e.slices = slices;
-    e.rotate = 1;
+    e.rotate = mode == 4 ? 0 : 1;
     e.prologue.residual = reinterpret_cast<const uint16_t *>(residual_dev);
     e.prologue.weight = reinterpret_cast<const uint16_t *>(norm_weight_dev);
     e.prologue.gate = reinterpret_cast<const uint16_t *>(gate_dev);
@@ -611,10 +613,12 @@ extern "C" int nq_fused_stage_linear(
 #define NQ_LAUNCH_PAIR(PRO, FORM) \
     launch_pair<PRO, FORM>(e, w, consumer, m_tile, r, producers, groups, late, m, sqrt_k, out_is_f32, sync, lds_bytes, s)
     if (k == 8192) {
+        if (mode == 0 || mode == 4) return NQ_LAUNCH_PAIR(0, nq::kFirstLanes);
         if (mode == 1) return NQ_LAUNCH_PAIR(1, nq::kFirstLanes);
         if (mode == 2) return NQ_LAUNCH_PAIR(2, nq::kFirstLanes);
         return NQ_LAUNCH_PAIR(3, nq::kFirstLanes);
     }
+    if (mode == 0 || mode == 4) return NQ_LAUNCH_PAIR(0, nq::kEightLanes);
     if (mode == 1) return NQ_LAUNCH_PAIR(1, nq::kEightLanes);
     if (mode == 2) return NQ_LAUNCH_PAIR(2, nq::kEightLanes);
     return NQ_LAUNCH_PAIR(3, nq::kEightLanes);

@@ -803,12 +803,13 @@ def fused_stage_linear(inputs: torch.Tensor | None, weights: Sequence[PreparedNQ
                        ) -> tuple[list[torch.Tensor], PreparedNQA4Activation, torch.Tensor | None, torch.Tensor | None]:
     """`fused_input_stage` (mode "rmsnorm" / "swiglu") or `attention_output_stage` (mode "attention", the
     rows then come from `attention_workspace`, a BatchedNQKVAttentionWorkspace whose first stage has run)
-    with the Hadamard rotation, followed by `linear_packed_w4a4_gemv_grouped` of `weights` on the encoded
+    with the Hadamard rotation, or the encoder alone on the rows themselves (mode "rows": rotated first, as
+    `quantize_activation_cuda(..., hadamard=True)`; mode "rotated_rows": as they are), followed by `linear_packed_w4a4_gemv_grouped` of `weights` on the encoded
     rows, as one launch whose linear workgroups decode their weights while the encoder runs.  Returns
     (outputs, packed activation, residual sum when `want_residual`, staged rows when `want_staged`): the
     same bits as the two calls.  `sync` orders the launch among its neighbours on the stream."""
-    if mode not in ("rmsnorm", "swiglu", "attention"):
-        raise ValueError("mode must be 'rmsnorm', 'swiglu' or 'attention'")
+    if mode not in ("rmsnorm", "swiglu", "attention", "rows", "rotated_rows"):
+        raise ValueError("mode must be 'rmsnorm', 'swiglu', 'attention', 'rows' or 'rotated_rows'")
     bf16 = torch.bfloat16
     if mode == "attention":
         if attention_workspace is None:
@@ -838,6 +839,8 @@ def fused_stage_linear(inputs: torch.Tensor | None, weights: Sequence[PreparedNQ
             raise ValueError("mode 'rmsnorm' needs a norm weight of the feature size")
         if mode == "swiglu" and gate is None:
             raise ValueError("mode 'swiglu' needs the gate rows")
+        if mode in ("rows", "rotated_rows") and (want_staged or want_residual or residual is not None or gate is not None):
+            raise ValueError("modes 'rows' and 'rotated_rows' have no staged rows, residual or gate")
     if not can_use_fused_stage_linear(rows, n, weights):
         raise ValueError("rows, K or weights are outside what the fused stage + linear launch takes")
     if beta_table is None or beta_table.numel() != 4:
@@ -861,7 +864,8 @@ def fused_stage_linear(inputs: torch.Tensor | None, weights: Sequence[PreparedNQ
 
     parts = 0 if mode != "attention" else lib.nq_nqkv_attention_parts(rows, attention_workspace.max_pages)
     _native.check(lib.nq_fused_stage_linear(
-        ptr(inputs) if mode != "attention" else None, rows, n, {"rmsnorm": 1, "swiglu": 2, "attention": 3}[mode],
+        ptr(inputs) if mode != "attention" else None, rows, n,
+        {"rows": 0, "rmsnorm": 1, "swiglu": 2, "attention": 3, "rotated_rows": 4}[mode],
         ptr(residual), ptr(residual_out), ptr(norm_weight), float(eps), ptr(gate),
         attention_workspace.buffer.data_ptr() if mode == "attention" else None,
         attention_workspace.query_heads if mode == "attention" else 0, parts, ptr(staged), beta_table.data_ptr(), 4,

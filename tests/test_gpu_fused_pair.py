@@ -75,6 +75,34 @@ def test_stage_and_linear_in_one_launch_equal_two_launches(rt, name, k, sizes, r
     assert not sync.timed_out
 
 
+@pytest.mark.parametrize("rows", [1, 2, 5, 8, 16])
+@pytest.mark.parametrize("name,k,sizes", PAIRS)
+def test_encoder_and_linear_in_one_launch_equal_two_launches(rt, name, k, sizes, rows):
+    """The rows themselves as the input stage (what a packed linear module does with its input: rotate,
+    encode, multiply): modes "rows" and "rotated_rows" against `quantize_activation_cuda` with and without
+    the rotation followed by the grouped linear, bit for bit."""
+    if k == 8192 and rows > 8:
+        pytest.skip("rows of 8192 values: up to eight per launch")
+    weights = _weights(rt, k, sizes, seed=len(name))
+    sync = rt.StageLinearSync(torch.device("cuda"))
+    g = torch.Generator().manual_seed(300 * rows + k % 89)
+    x = (torch.randn(rows, k, generator=g) * (1.0 + 3.0 * (torch.rand(rows, 1, generator=g) > 0.5))).to(torch.bfloat16).cuda()
+    for mode, rotate in (("rows", True), ("rotated_rows", False)):
+        expect_activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS, beta_table=_table(), hadamard=rotate)
+        for dtype in (torch.bfloat16, torch.float32):
+            expect = rt.linear_packed_w4a4_gemv_grouped(expect_activation, weights, output_dtype=dtype)
+            for repeat in range(2):
+                outs, activation, residual, staged = rt.fused_stage_linear(x, weights, sync, mode=mode, beta_table=_table(),
+                                                                            output_dtype=dtype)
+                assert residual is None and staged is None
+                assert _same_activation(activation, expect_activation), (mode, dtype)
+                for out, want in zip(outs, expect):
+                    assert out.shape == want.shape and torch.equal(out, want), (mode, dtype)
+    assert not sync.timed_out
+    with pytest.raises(ValueError, match="staged"):
+        rt.fused_stage_linear(x, weights, sync, mode="rows", beta_table=_table(), want_staged=True)
+
+
 @pytest.mark.parametrize("rows", [1, 4, 8])
 def test_attention_merge_and_o_proj_in_one_launch(rt, rows):
     from nestquant_aiinfra_amd.runtime import nqkv
