@@ -81,8 +81,8 @@ def test_encoder_and_linear_in_one_launch_equal_two_launches(rt, name, k, sizes,
     """The rows themselves as the input stage (what a packed linear module does with its input: rotate,
     encode, multiply): modes "rows" and "rotated_rows" against `quantize_activation_cuda` with and without
     the rotation followed by the grouped linear, bit for bit."""
-    if k == 8192 and rows > 8:
-        pytest.skip("rows of 8192 values: up to eight per launch")
+    if k == 8192:
+        rows = min(rows, 7)                              # rows of 8192 values: up to eight per launch
     weights = _weights(rt, k, sizes, seed=len(name))
     sync = rt.StageLinearSync(torch.device("cuda"))
     g = torch.Generator().manual_seed(300 * rows + k % 89)
