@@ -55,14 +55,18 @@ struct GemmWeights {
 // blocks (words / tails, see nq_e8.hip.h) instead of NQRT4 code words and beta bytes.
 // FP32 results (partial sums of K slab blockIdx.y, or the output itself) are laid out weight by
 // weight: out_f32[(slab * n_total + first channel of the weight) * m_rows + m * channels + n].
-template <int TILES, bool kResolved>
+// CT: tiles of 32 channels per workgroup.  Every workgroup reads the whole activation of its K slab from
+// L2, and those reads are what a launch of many channel tiles waits for (a 128-row gate + up launch: 512
+// workgroups x 512 KB); with CT = 2 a decode lane takes two blocks per trip (channels c and c + 32) and a
+// multiplying wavefront uses each activation fragment for both tiles, so half as many workgroups read it.
+template <int TILES, bool kResolved, int CT = 1>
 __global__ void __launch_bounds__(kGemmThreads)
 w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
                  GemmWeights weights, int m_rows, int k_size, int n_total, int k_slab, float sqrt_k,
                  float *__restrict__ out_f32) {
-    __shared__ uint4 b_tile[2][kGemmBK / 16][64];          // 2 x 8 K-steps x 64 lanes x 16 B = 16 KiB
+    __shared__ uint4 b_tile[2][CT][kGemmBK / 16][64];      // 2 x CT x 8 K-steps x 64 lanes x 16 B = CT x 16 KiB
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int channel0 = blockIdx.x * kGemmBN;
+    const int channel0 = blockIdx.x * (kGemmBN * CT);
     const int group = (channel0 >= weights.end[0]) + (channel0 >= weights.end[1]) + (channel0 >= weights.end[2]);
     const int group_first = group ? weights.end[group - 1] : 0;
     const int n0 = channel0 - group_first, n_size = weights.end[group] - group_first;
@@ -76,14 +80,21 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
     const int k_begin = blockIdx.y * k_slab;
     const int blocks_per_row = k_size >> 3;
 
-    // decode role: channel n0 + tid / 16, block tid % 16 of the current 128-wide step.
+    // decode role: channel n0 + 32 c + tid / 16 of every tile c, block tid % 16 of the current 128-wide step.
     // Channels past the end repeat the last one; their results are never stored.
-    const int dec_n = n0 + (tid >> 4) < n_size ? n0 + (tid >> 4) : n_size - 1, dec_kb = tid & 15;
-    const float unit = w_norms[dec_n] / sqrt_k;
-    const float wscale = kResolved ? unit * kResolvedUnit : unit;
+    const int dec_kb = tid & 15;
     const float wbeta[4] = {w_betas[0], w_betas[1], w_betas[2], w_betas[3]};
-    const ResolvedScales scaled_beta = resolved_scales(wbeta, wscale);
-    const int64_t dec_first = (int64_t)dec_n * blocks_per_row + (k_begin >> 3) + dec_kb;
+    float wscale[CT];
+    ResolvedScales scaled_beta[CT];
+    int64_t dec_first[CT];
+#pragma unroll
+    for (int c = 0; c < CT; c++) {
+        const int dec_n = n0 + kGemmBN * c + (tid >> 4) < n_size ? n0 + kGemmBN * c + (tid >> 4) : n_size - 1;
+        const float unit = w_norms[dec_n] / sqrt_k;
+        wscale[c] = kResolved ? unit * kResolvedUnit : unit;
+        scaled_beta[c] = resolved_scales(wbeta, wscale[c]);
+        dec_first[c] = (int64_t)dec_n * blocks_per_row + (k_begin >> 3) + dec_kb;
+    }
     // LDS entry of (K-step kk, fragment lane f): [kk][f ^ (2 (kk % 4) + f / 32)].  Eight neighbouring
     // decode lanes (one channel, blocks 8 i .. 8 i + 7, i.e. four K-steps x the two halves of the
     // fragment) then write eight different 16-byte bank groups, and for the readers the mask is a
@@ -91,8 +102,9 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
     const int dec_kk = dec_kb >> 1;
     const int dec_f = (tid >> 4) + 32 * (dec_kb & 1);
     const int dec_entry = dec_f ^ (2 * (dec_kk & 3) + (dec_kb & 1));
-    uint4 *dec_slot0 = &b_tile[0][dec_kk][dec_entry];
-    uint4 *dec_slot1 = &b_tile[1][dec_kk][dec_entry];
+    uint4 *dec_slot0 = &b_tile[0][0][dec_kk][dec_entry];
+    uint4 *dec_slot1 = &b_tile[1][0][dec_kk][dec_entry];
+    constexpr int kTileEntries = (kGemmBK / 16) * 64;
 
     // multiply role: A fragment rows of this lane, one per owned tile (rows past the end
     // repeat the last one; their results are never stored)
@@ -103,18 +115,24 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
         a_row[t] = act + (int64_t)(m < m_rows ? m : m_rows - 1) * k_size + k_begin + 8 * (lane >> 5);
     }
     const bool multiplies = wave * 32 < m_rows;
-    floatx16 acc[TILES];
+    floatx16 acc[TILES][CT];
 #pragma unroll
     for (int t = 0; t < TILES; t++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) acc[t][i] = 0.0f;
+        for (int c = 0; c < CT; c++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[t][c][i] = 0.0f;
 
     // Software pipeline, one barrier per trip: trip s multiplies step s - 1 (weights from
     // LDS, activation fragments requested one trip earlier) while it decodes step s, and
     // requests the code words of step s + 1 and the fragments of step s.
     const int steps = k_slab / kGemmBK;
-    uint32_t word_next = w_words[dec_first];
-    uint32_t side_next = kResolved ? (uint32_t)w_tails[dec_first] : (uint32_t)w_beta_ids[dec_first >> 2];
+    uint32_t word_next[CT], side_next[CT];
+#pragma unroll
+    for (int c = 0; c < CT; c++) {
+        word_next[c] = w_words[dec_first[c]];
+        side_next[c] = kResolved ? (uint32_t)w_tails[dec_first[c]] : (uint32_t)w_beta_ids[dec_first[c] >> 2];
+    }
     uint4 a_next[TILES][kGemmBK / 16];
 #pragma unroll
     for (int t = 0; t < TILES; t++)
@@ -122,16 +140,22 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
         for (int kk = 0; kk < kGemmBK / 16; kk++) a_next[t][kk] = make_uint4(0, 0, 0, 0);
 
     for (int s = 0; s <= steps; s++) {
-        const uint32_t word = word_next, side = side_next;
+        uint32_t word[CT], side[CT];
+#pragma unroll
+        for (int c = 0; c < CT; c++) { word[c] = word_next[c]; side[c] = side_next[c]; }
         uint4 a_now[TILES][kGemmBK / 16];
 #pragma unroll
         for (int t = 0; t < TILES; t++)
 #pragma unroll
             for (int kk = 0; kk < kGemmBK / 16; kk++) a_now[t][kk] = a_next[t][kk];
-        const int64_t g = dec_first + (int64_t)s * (kGemmBK / 8);
-        if (s + 1 < steps) {
-            word_next = w_words[g + kGemmBK / 8];
-            side_next = kResolved ? (uint32_t)w_tails[g + kGemmBK / 8] : (uint32_t)w_beta_ids[(g + kGemmBK / 8) >> 2];
+        int64_t g[CT];
+#pragma unroll
+        for (int c = 0; c < CT; c++) {
+            g[c] = dec_first[c] + (int64_t)s * (kGemmBK / 8);
+            if (s + 1 < steps) {
+                word_next[c] = w_words[g[c] + kGemmBK / 8];
+                side_next[c] = kResolved ? (uint32_t)w_tails[g[c] + kGemmBK / 8] : (uint32_t)w_beta_ids[(g[c] + kGemmBK / 8) >> 2];
+            }
         }
         if (s < steps && multiplies) {
 #pragma unroll
@@ -143,35 +167,45 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
         if (s > 0 && multiplies) {
 #pragma unroll
             for (int kk = 0; kk < kGemmBK / 16; kk++) {
-                const bf16x8 b = __builtin_bit_cast(bf16x8, b_tile[(s - 1) & 1][kk][lane ^ (2 * (kk & 3) + (lane >> 5))]);
 #pragma unroll
-                for (int t = 0; t < TILES; t++)
-                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[t][kk]), b, acc[t], 0, 0, 0);
+                for (int c = 0; c < CT; c++) {
+                    const bf16x8 b = __builtin_bit_cast(bf16x8, b_tile[(s - 1) & 1][c][kk][lane ^ (2 * (kk & 3) + (lane >> 5))]);
+#pragma unroll
+                    for (int t = 0; t < TILES; t++)
+                        acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[t][kk]), b,
+                                                                            acc[t][c], 0, 0, 0);
+                }
             }
         }
         if (s < steps) {
-            float v[8];
-            if (kResolved) {
-                decode_resolved(word, side, seed_plus_offset + (uint32_t)g * 8u, resolved_scale(scaled_beta, word), v);
-            } else {
-                decode_codeword<true>(word, 14.0f, seed_plus_offset + (uint32_t)g * 8u, v);
-                const float scale = wbeta[(side >> (2 * (g & 3))) & 3] * wscale;
 #pragma unroll
-                for (int j = 0; j < 8; j++) v[j] = v[j] * scale;
+            for (int c = 0; c < CT; c++) {
+                float v[8];
+                if (kResolved) {
+                    decode_resolved(word[c], side[c], seed_plus_offset + (uint32_t)g[c] * 8u,
+                                    resolved_scale(scaled_beta[c], word[c]), v);
+                } else {
+                    decode_codeword<true>(word[c], 14.0f, seed_plus_offset + (uint32_t)g[c] * 8u, v);
+                    const float scale = wbeta[(side[c] >> (2 * (g[c] & 3))) & 3] * wscale[c];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) v[j] = v[j] * scale;
+                }
+                const bf16x2 h0 = pack_bf16x2(v[0], v[1]), h1 = pack_bf16x2(v[2], v[3]);
+                const bf16x2 h2 = pack_bf16x2(v[4], v[5]), h3 = pack_bf16x2(v[6], v[7]);
+                ((s & 1) ? dec_slot1 : dec_slot0)[c * kTileEntries] =
+                    make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
+                               __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
             }
-            const bf16x2 h0 = pack_bf16x2(v[0], v[1]), h1 = pack_bf16x2(v[2], v[3]);
-            const bf16x2 h2 = pack_bf16x2(v[4], v[5]), h3 = pack_bf16x2(v[6], v[7]);
-            *((s & 1) ? dec_slot1 : dec_slot0) =
-                make_uint4(__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
-                           __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3));
         }
         __syncthreads();
     }
 
     // accumulator register r of lane l holds token row (r % 4) + 8 * (r / 4) + 4 * (l / 32)
     // of the tile and channel n0 + l % 32
-    const int n = n0 + (lane & 31);
-    if (n < n_size) {
+#pragma unroll
+    for (int c = 0; c < CT; c++) {
+        const int n = n0 + kGemmBN * c + (lane & 31);
+        if (n >= n_size) continue;
 #pragma unroll
         for (int t = 0; t < TILES; t++) {
             const int m_base = (wave + t * kGemmWaves) * 32 + 4 * (lane >> 5);
@@ -180,9 +214,9 @@ w4a4_gemm_kernel(const uint16_t *__restrict__ act,        // BF16 [m_rows][K]
                 const int m = m_base + (r & 3) + 8 * (r >> 2);
                 if (m < m_rows) {
                     if (out_f32)
-                        out_f32[((int64_t)blockIdx.y * n_total + group_first) * m_rows + (int64_t)m * n_size + n] = acc[t][r];
+                        out_f32[((int64_t)blockIdx.y * n_total + group_first) * m_rows + (int64_t)m * n_size + n] = acc[t][c][r];
                     else
-                        out_bf16[(int64_t)m * n_size + n] = f32_to_bf16(acc[t][r]);
+                        out_bf16[(int64_t)m * n_size + n] = f32_to_bf16(acc[t][c][r]);
                 }
             }
         }
@@ -285,8 +319,20 @@ int pick_gemm_split(int k, int n, int requested) {
 // One launch of the fused kernel over `rows` tokens and the n_total channels of `weights`.
 int launch_fused_gemm(const uint16_t *act, const nq::GemmWeights &weights, bool resolved, int rows, int k, int n_total,
                       int split, float *out_f32, hipStream_t s) {
-    const dim3 grid((unsigned)((n_total + nq::kGemmBN - 1) / nq::kGemmBN), (unsigned)split);
     const float sqrt_k = (float)sqrt((double)k);
+    // Two channel tiles per workgroup where that still leaves a workgroup for every compute unit and no
+    // K split is needed (the gate + up launch of a short prefill): half the reads of the activation, the
+    // same bits.  Measured on gate + up of the 1B model (us, 32- / 64-channel tiles): 96 rows 34.6 / 33.7,
+    // 128 rows 40.3 / 35.7, 200 rows 58.6 / 47.0, 256 rows 68.4 / 50.4; below 96 rows the launch waits for
+    // the decode of its slowest workgroup, and 512 workgroups share that better (64 rows: 27.8 / 30.3).
+    bool wide = resolved && rows >= 96 && rows <= 8 * 32 && split == 1 && n_total >= 64 * 256;
+    for (int g = 0; g < nq::kGemmMaxGroups; g++) wide = wide && (weights.end[g] % 64 == 0 || weights.end[g] == n_total);
+    if (wide) {
+        hipLaunchKernelGGL((nq::w4a4_gemm_kernel<1, true, 2>), dim3((unsigned)((n_total + 63) / 64), 1u),
+                           dim3(nq::kGemmThreads), 0, s, act, weights, rows, k, n_total, k, sqrt_k, out_f32);
+        return nq::check_launch("nq_w4a4_gemm");
+    }
+    const dim3 grid((unsigned)((n_total + nq::kGemmBN - 1) / nq::kGemmBN), (unsigned)split);
 #define NQ_LAUNCH_GEMM(TILES, RESOLVED)                                                                     \
     hipLaunchKernelGGL((nq::w4a4_gemm_kernel<TILES, RESOLVED>), grid, dim3(nq::kGemmThreads), 0, s, act,    \
                        weights, rows, k, n_total, k / split, sqrt_k, out_f32)

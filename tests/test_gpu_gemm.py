@@ -207,11 +207,14 @@ def test_grouped_prefill_linears_equal_one_call_per_weight(rt, oracle, m, k, siz
 
 
 @pytest.mark.parametrize("m,k,sizes", [(17, 512, (256, 64, 64)), (128, 2048, (2048, 512, 512)), (287, 1024, (512, 512)),
-                                       (40, 256, (32, 64, 96, 32)), (128, 2048, (8192, 8192)), (100, 8192, (64, 32))])
+                                       (40, 256, (32, 64, 96, 32)), (128, 2048, (8192, 8192)), (100, 8192, (64, 32)),
+                                       (96, 512, (8192, 8192)), (250, 256, (8192, 4096, 4160)), (95, 256, (8192, 8192))])
 def test_grouped_short_prefill_linears_equal_one_launch_per_weight(rt, oracle, m, k, sizes):
     """Below the decode-once size one launch of the fused kernel walks the channels of all the
     weights (`nq_w4a4_gemm_grouped`): every output is bit for bit what the kernel gives for its
-    weight alone with the K split the group runs with (the split follows the sum of the widths)."""
+    weight alone with the K split the group runs with (the split follows the sum of the widths).  A
+    group of 16384 channels or more at 96 to 256 rows runs with 64-channel tiles, a weight alone with
+    32-channel ones: the same bits."""
     from nestquant_aiinfra_amd.runtime.w4a4_linear import _gemm
     weights = []
     for i, n_out in enumerate(sizes):
