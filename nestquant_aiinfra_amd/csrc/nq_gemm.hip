@@ -316,20 +316,50 @@ int pick_gemm_split(int k, int n, int requested) {
     return split;
 }
 
+// The form of one launch of the fused kernel: 32- or 64-channel tiles, and the K slabs.
+// Two channel tiles per workgroup halve the reads of the activation, which every workgroup makes for
+// its whole K slab and which a launch of many tiles or of long rows waits for; they are taken from 96
+// rows on (below, the launch waits for the decode of its slowest workgroup, and twice the workgroups
+// share that better), where a workgroup for every compute unit is left
+//   * without a K split (gate + up of a short prefill; us, 32- / 64-channel tiles: 96 rows 34.6 / 33.7,
+//     128 rows 40.3 / 35.7, 200 rows 58.6 / 47.0, 256 rows 68.4 / 50.4, 64 rows 27.8 / 30.3), or
+//   * with twice the slabs when a row of the activation has 8192 values or more (down_proj: the halved
+//     reads outweigh the doubled partial sums).
+// A split the caller names is kept.  Every split gives the same bits in both forms.
+struct GemmPlan {
+    bool wide;
+    int split;
+};
+
+GemmPlan plan_fused_gemm(int rows, int k, int n_total, int requested, bool resolved, bool whole_tiles) {
+    GemmPlan plan{false, pick_gemm_split(k, n_total, requested)};
+    if (!resolved || !whole_tiles || rows < 96 || rows > 8 * 32) return plan;
+    const int tiles = (n_total + 63) / 64;
+    if (requested > 0) {
+        plan.wide = tiles * requested >= 256;
+        return plan;
+    }
+    int split = 1;
+    while (split < 16 && tiles * split < 256 && (k / (split * 2)) % nq::kGemmBK == 0) split *= 2;
+    if (tiles * split >= 256 && (split == 1 || k >= 8192)) plan = GemmPlan{true, split};
+    return plan;
+}
+
+// whether every weight of a launch but the last has a multiple of 64 channels (a workgroup's tiles lie in one weight)
+bool whole_wide_tiles(const nq::GemmWeights &weights, int n_total) {
+    bool whole = true;
+    for (int g = 0; g < nq::kGemmMaxGroups; g++) whole = whole && (weights.end[g] % 64 == 0 || weights.end[g] == n_total);
+    return whole;
+}
+
 // One launch of the fused kernel over `rows` tokens and the n_total channels of `weights`.
 int launch_fused_gemm(const uint16_t *act, const nq::GemmWeights &weights, bool resolved, int rows, int k, int n_total,
-                      int split, float *out_f32, hipStream_t s) {
+                      const GemmPlan &plan, float *out_f32, hipStream_t s) {
     const float sqrt_k = (float)sqrt((double)k);
-    // Two channel tiles per workgroup where that still leaves a workgroup for every compute unit and no
-    // K split is needed (the gate + up launch of a short prefill): half the reads of the activation, the
-    // same bits.  Measured on gate + up of the 1B model (us, 32- / 64-channel tiles): 96 rows 34.6 / 33.7,
-    // 128 rows 40.3 / 35.7, 200 rows 58.6 / 47.0, 256 rows 68.4 / 50.4; below 96 rows the launch waits for
-    // the decode of its slowest workgroup, and 512 workgroups share that better (64 rows: 27.8 / 30.3).
-    bool wide = resolved && rows >= 96 && rows <= 8 * 32 && split == 1 && n_total >= 64 * 256;
-    for (int g = 0; g < nq::kGemmMaxGroups; g++) wide = wide && (weights.end[g] % 64 == 0 || weights.end[g] == n_total);
-    if (wide) {
-        hipLaunchKernelGGL((nq::w4a4_gemm_kernel<1, true, 2>), dim3((unsigned)((n_total + 63) / 64), 1u),
-                           dim3(nq::kGemmThreads), 0, s, act, weights, rows, k, n_total, k, sqrt_k, out_f32);
+    const int split = plan.split;
+    if (plan.wide) {
+        hipLaunchKernelGGL((nq::w4a4_gemm_kernel<1, true, 2>), dim3((unsigned)((n_total + 63) / 64), (unsigned)split),
+                           dim3(nq::kGemmThreads), 0, s, act, weights, rows, k, n_total, k / split, sqrt_k, out_f32);
         return nq::check_launch("nq_w4a4_gemm");
     }
     const dim3 grid((unsigned)((n_total + nq::kGemmBN - 1) / nq::kGemmBN), (unsigned)split);
@@ -351,12 +381,14 @@ int launch_fused_gemm(const uint16_t *act, const nq::GemmWeights &weights, bool 
 
 extern "C" size_t nq_w4a4_gemm_workspace_bytes(int m, int k, int n, int split_k, int have_decoded_activation) {
     if (m < 1 || n < 1 || k < 1) return 0;
-    const int split = pick_gemm_split(k, n, split_k);
     size_t bytes = 0;
     if (!have_decoded_activation) bytes += nq::align256((size_t)m * k * 2);
     // the output dtype is not known here: enough for the decode-once scratch (BF16 output) and for the
     // fused kernel's partial sums (FP32 output) alike
     const int chunk = m < kChunkRows ? m : kChunkRows;
+    // (nor the weight's form: the larger of the two forms' splits)
+    const int narrow = pick_gemm_split(k, n, split_k), other = plan_fused_gemm(chunk, k, n, split_k, true, true).split;
+    const int split = narrow > other ? narrow : other;
     const size_t partials = split > 1 ? (size_t)split * (size_t)chunk * (size_t)n * sizeof(float) : 0;
     // decode-once: the BF16 weight, then the partial results of the dense product's own K split
     size_t scratch = 0;
@@ -398,10 +430,11 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
     NQ_REQUIRE(weight_offset >= 0 && weight_offset + (int64_t)n * (k / 8) <= ((int64_t)1 << 28),
                NQ_ERR_SHAPE, "nq_w4a4_gemm: block range exceeds the stateless dither counter space");
     const bool once = decodes_once(m, k, split_k) && out_dtype == NQ_BF16;
-    const int split = once ? 1 : pick_gemm_split(k, n, split_k);
+    const int chunk_rows = m < kChunkRows ? m : kChunkRows;
+    const GemmPlan plan = once ? GemmPlan{false, 1} : plan_fused_gemm(chunk_rows, k, n, split_k, resolved, true);
+    const int split = plan.split;
     NQ_REQUIRE(k % split == 0 && (k / split) % nq::kGemmBK == 0, NQ_ERR_SHAPE,
                "nq_w4a4_gemm: K / split_k = %d / %d must be a multiple of 128", k, split);
-    const int chunk_rows = m < kChunkRows ? m : kChunkRows;
     const size_t decoded_bytes = act_decoded_dev ? 0 : nq::align256((size_t)m * k * 2);
     const size_t need = decoded_bytes + (once ? nq::align256((size_t)n * k * 2)
                                               : (split > 1 ? (size_t)split * chunk_rows * n * sizeof(float) : 0));
@@ -444,7 +477,7 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
         char *out_chunk = reinterpret_cast<char *>(out_dev) + (size_t)m0 * out_row_bytes;
         float *target_f32 = split > 1 ? partials : (out_dtype == NQ_F32 ? (float *)out_chunk : nullptr);
         weights.out_bf16[0] = (split > 1 || out_dtype == NQ_F32) ? nullptr : (uint16_t *)out_chunk;
-        int status = launch_fused_gemm(act + (size_t)m0 * k, weights, resolved, rows, k, n, split, target_f32, s);
+        int status = launch_fused_gemm(act + (size_t)m0 * k, weights, resolved, rows, k, n, plan, target_f32, s);
         if (status != NQ_OK) return status;
         if (split > 1) {
             status = nq::launch_splitk_reduce(partials, split, (int64_t)rows * n, out_chunk, out_dtype, s);
@@ -456,7 +489,8 @@ extern "C" int nq_w4a4_gemm(const uint8_t *act_codes_dev, const uint8_t *act_bet
 
 extern "C" size_t nq_w4a4_gemm_grouped_workspace_bytes(int m, int k, int n_total) {
     if (m < 1 || n_total < 1 || k < 1) return 0;
-    const int split = pick_gemm_split(k, n_total, 0);
+    const int narrow = pick_gemm_split(k, n_total, 0), other = plan_fused_gemm(m, k, n_total, 0, true, true).split;
+    const int split = narrow > other ? narrow : other;
     return split > 1 ? (size_t)split * (size_t)m * (size_t)n_total * sizeof(float) : 0;
 }
 
@@ -507,7 +541,8 @@ extern "C" int nq_w4a4_gemm_grouped(const void *act_decoded_dev, int count, cons
         outputs.out[g] = outputs.out[count - 1];
         outputs.end[g] = (int64_t)m * n_total;
     }
-    const int split = pick_gemm_split(k, (int)n_total, 0);
+    const GemmPlan plan = plan_fused_gemm(m, k, (int)n_total, 0, true, whole_wide_tiles(weights, (int)n_total));
+    const int split = plan.split;
     const size_t need = split > 1 ? (size_t)split * m * n_total * sizeof(float) : 0;
     NQ_REQUIRE(need == 0 || (workspace_dev && workspace_bytes >= need), NQ_ERR_WORKSPACE,
                "nq_w4a4_gemm_grouped: needs a %zu-byte workspace, got %zu", need, workspace_bytes);
@@ -518,7 +553,7 @@ extern "C" int nq_w4a4_gemm_grouped(const void *act_decoded_dev, int count, cons
     if (split > 1)
         for (int g = 0; g < nq::kGemmMaxGroups; g++) weights.out_bf16[g] = nullptr;
     int status = launch_fused_gemm(reinterpret_cast<const uint16_t *>(act_decoded_dev), weights, true, m, k, (int)n_total,
-                                   split, partials, s);
+                                   plan, partials, s);
     if (status != NQ_OK || split == 1) return status;
     return nq::launch_splitk_reduce_grouped(partials, split, (int64_t)m * n_total, outputs, s);
 }
