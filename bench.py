@@ -360,6 +360,27 @@ def prefill_gemm_extra(rt, device):
             flops = 2.0 * m * k * n
             results[f"{name}_m{m}"] = {"us": seconds * 1e6, "TFLOPs": flops / seconds / 1e12,
                                        "mfma_frac": flops / seconds / 2.5e15, "encode_us": encode * 1e6}
+        if name == "gate_proj":
+            # gate and up of a layer as the model's prefill step launches them: one call for both weights
+            g = torch.Generator().manual_seed(wseed + 10)
+            w = hadamard_gpu((0.02 * torch.randn(n, k, generator=g)).to(device))
+            up_record = rt.quantize_weight_nqrt4(w, q=Q, betas=WEIGHT_BETAS, dither_seed=dseed + 10, tensor_name="up_proj")
+            up_base = rt.prepare_fused_linear(up_record, device=device)
+            ups = [up_base] + [rt.PreparedNQRTLinear(up_record, None, None, up_base.row_norms, up_base.beta_table,
+                                                     up_base.resolved_words.clone(), up_base.resolved_tails.clone())
+                               for _ in range(copies - 1)]
+            for m in (64, 128, 256, 384):
+                rng = np.random.default_rng(3001)
+                x = rng.standard_normal((m, k)).astype(np.float32)
+                x[:, rng.choice(k, size=k // 100, replace=False)] *= 20.0
+                x = torch.from_numpy(x).to(device).to(torch.bfloat16)
+                activation = rt.quantize_activation_cuda(x, q=Q, betas=ACTIVATION_BETAS, beta_table=table, hadamard=True)
+                seconds = time_graph(lambda i: rt.linear_packed_w4a4_gemm_grouped(
+                    activation, [weights[i % copies], ups[i % copies]]), copies)
+                flops = 2.0 * m * k * 2 * n
+                results[f"gate_up_m{m}"] = {"us": seconds * 1e6, "TFLOPs": flops / seconds / 1e12,
+                                            "mfma_frac": flops / seconds / 2.5e15}
+            del ups
     return results
 
 
@@ -939,6 +960,11 @@ def extra_rooflines(extra):
         # the reference's own prefill row counts (128 and 384 rows), then a long prompt
         "prefill_gemm": gemm_object("gate_proj", 128, fused),
         "prefill_gemm_m384": gemm_object("gate_proj", 384, once),
+        "prefill_gemm_gate_up_m128": {
+            "bound": "mfma", "workload": "gate_proj + up_proj K2048 N2x8192 M128 in one launch, as the prefill step runs them",
+            "achieved": extra["prefill_gemm"]["gate_up_m128"]["TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": extra["prefill_gemm"]["gate_up_m128"]["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS,
+            "launch_us": extra["prefill_gemm"]["gate_up_m128"]["us"]},
         "prefill_gemm_down_m128": gemm_object("down_proj", 128, fused),
         "prefill_gemm_down_m384": gemm_object("down_proj", 384, once),
         "prefill_gemm_m4096": gemm_object("gate_proj", 4096, once),
