@@ -235,3 +235,20 @@ def test_grouped_short_prefill_linears_equal_one_launch_per_weight(rt, oracle, m
     # the same call twice gives the same bits (the slabs are added in order)
     again = rt.linear_packed_w4a4_gemm_grouped(activation, weights)
     assert all(torch.equal(a, b) for a, b in zip(grouped, again))
+
+
+@pytest.mark.parametrize("m,k,n_out,split", [(128, 256, 16400, 0), (200, 128, 16417, 0), (96, 4096, 4100, 0), (130, 1024, 2050, 8)])
+def test_wide_tiles_on_ragged_widths_match_oracle(rt, oracle, m, k, n_out, split):
+    """The 64-channel tiles of the fused kernel (96 to 256 rows; 16384 channels and more, rows of 4096
+    values and more with K slabs, or a split that leaves 256 workgroups) where the last workgroup holds
+    a few channels only: against the oracle's product, FP32 and BF16 outputs."""
+    seed = 20300000 + n_out
+    _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=9100 + n_out % 97, dither_seed=seed)
+    weight = rt.prepare_fused_linear(_record(rt, wc, wb, wn, k, seed), device="cuda")
+    activation = _activation(rt, oracle, m, k, seed=9200 + m)
+    ref32, ref16 = _references(oracle, activation, rt, wc, wb, wn, seed)
+    y = rt._gemm(activation, weight, output_dtype=torch.float32, split_k=split)
+    assert relative_error(bits(y), ref32) <= TOLERANCE
+    assert relative_error(bits(y), ref16) <= BF16_TOLERANCE
+    y16 = rt._gemm(activation, weight, output_dtype=torch.bfloat16, split_k=split)
+    assert torch.equal(y16, y.to(torch.bfloat16))
