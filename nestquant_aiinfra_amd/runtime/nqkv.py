@@ -921,7 +921,8 @@ class BatchedNQKVCacheManager:
         if self._prompt_record is None:
             self._prompt_record = torch.zeros(3 * self.capacity, dtype=torch.int32, device=self.device)
             self._prompt_stage = torch.zeros(3 * self.capacity, dtype=torch.int32, pin_memory=True)
-            self._prompt_stage_free = torch.cuda.Event()
+            with torch.cuda.device(self.device):
+                self._prompt_stage_free = torch.cuda.Event()
         else:
             self._prompt_stage_free.synchronize()             # the previous step's copy has read the words
         words = [int(s) for s in slot_ids] + [int(c) for c in counts] + [int(bool(f)) for f in fresh]
