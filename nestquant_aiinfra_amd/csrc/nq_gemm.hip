@@ -320,13 +320,15 @@ int pick_gemm_split(int k, int n, int requested) {
 // Two channel tiles per workgroup halve the reads of the activation, which every workgroup makes for
 // its whole K slab and which a launch of many tiles or of long rows waits for; they are taken from 96
 // rows on (below, the launch waits for the decode of its slowest workgroup, and twice the workgroups
-// share that better), where a workgroup for every compute unit is left
+// share that better), where enough workgroups are left
 //   * without a K split (gate + up of a short prefill; us, 32- / 64-channel tiles: 96 rows 34.6 / 33.7,
 //     128 rows 40.3 / 35.7, 200 rows 58.6 / 47.0, 256 rows 68.4 / 50.4, 64 rows 27.8 / 30.3), or
 //   * with twice the slabs when a row of the activation has 4096 values or more (down_proj, K = 8192:
 //     128 rows 26.7 / 24.8, 256 rows 40.1 / 33.5; a 4096 x 4096 weight at 256 rows 41.2 / 33.8): the halved
 //     reads outweigh the doubled partial sums, which they do not for rows of 2048 values (q/k/v at 128
-//     rows 17.6 / 22.0, o_proj 13.1 / 14.6).
+//     rows 17.6 / 22.0, o_proj 13.1 / 14.6), or
+//   * with the slabs of the 32-channel form where 192 workgroups remain (q/k/v: 128 rows 17.6 / 16.6,
+//     256 rows 27.8 / 23.1; not o_proj, 128 workgroups: 12.9 / 14.4).
 // A split the caller names is kept.  Every split gives the same bits in both forms.
 struct GemmPlan {
     bool wide;
@@ -338,12 +340,13 @@ GemmPlan plan_fused_gemm(int rows, int k, int n_total, int requested, bool resol
     if (!resolved || !whole_tiles || rows < 96 || rows > 8 * 32) return plan;
     const int tiles = (n_total + 63) / 64;
     if (requested > 0) {
-        plan.wide = tiles * requested >= 256;
+        plan.wide = tiles * requested >= 192;
         return plan;
     }
     int split = 1;
     while (split < 16 && tiles * split < 256 && (k / (split * 2)) % nq::kGemmBK == 0) split *= 2;
     if (tiles * split >= 256 && (split == 1 || k >= 4096)) plan = GemmPlan{true, split};
+    else if (tiles * plan.split >= 192) plan.wide = true;
     return plan;
 }
 
