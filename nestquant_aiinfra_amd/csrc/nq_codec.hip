@@ -655,6 +655,10 @@ constexpr int64_t kBulkElements = 1 << 21;
 // 13.5 / 42.1 against 14.6 / 47.5; 1024 rows: 21.5 / 84.0 against the many-row kernel's 21.5 / 77.5)
 constexpr int64_t kLanesKernelRows = 192;
 constexpr int64_t kBlockLanesRows = 512;
+// (rows of 8192 values: two 1024-lane workgroups a row, one workgroup per compute unit, so 128 rows fill
+// the chip and 192 rows took two rounds: 34.3 us against 19.3 for 128; with a lane per block, one workgroup
+// a row, they are one round again)
+int64_t every_lane_rows(int n) { return n > 4096 ? 128 : kLanesKernelRows; }
 
 template <typename T, bool kDithered, int kPrologue = 0>
 int launch_quantize(const void *x, int64_t rows, int n, int q, const float *betas, int beta_count,
@@ -669,14 +673,14 @@ int launch_quantize(const void *x, int64_t rows, int n, int q, const float *beta
     constexpr bool kBf16 = std::is_same<T, uint16_t>::value, kF32 = std::is_same<T, float>::value;
     const bool lanes_input = kBf16 || (kF32 && kPrologue == 0 && hadamard_stage_dtype < 0);
     if ((kBf16 || kF32) && lanes_input && !kDithered && q == 14 && (n == 2048 || n == 4096 || n == 8192) &&
-        nq::aligned(x, 16) && (kPrologue != 3 || rows <= 16) && (kBf16 || rows > kLanesKernelRows) &&
+        nq::aligned(x, 16) && (kPrologue != 3 || rows <= 16) && (kBf16 || rows > every_lane_rows(n)) &&
         (rows <= kBlockLanesRows || rows * (int64_t)n < kBulkElements)) {
         // decode step: a workgroup of n / 8 lanes encodes n / 256 blocks per pass with eight lanes per
         // (block, beta) pair: 32 slices of one pass each while that keeps the launch within one
         // workgroup per compute unit (n <= 4096); an 8192-value row keeps one lane per pair, slices of
         // 256 pairs.  Prefill chunk: every lane one pair, four slices a row (two, when four would put
         // more than two 1024-lane workgroups on a compute unit).
-        const int form = rows > kLanesKernelRows ? nq::kBlockLanes
+        const int form = rows > every_lane_rows(n) ? nq::kBlockLanes
                          : (rows > 16 ? nq::kEveryLane : (n > 4096 ? nq::kFirstLanes : nq::kEightLanes));
         int slices = n > 4096 ? n / 512 : (rows * 32 <= 256 ? 32 : 16);
         if (form == nq::kEveryLane) slices = n <= 2048 || rows * 4 * (n / 2048) <= 1024 ? 4 : 2;
