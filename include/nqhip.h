@@ -261,7 +261,7 @@ int nq_w4a4_gemv_grouped(const void *act_decoded_dev, int count, const uint32_t 
  * weight tile is decoded once per call into double-buffered LDS as MFMA B fragments; ragged
  * M is padded to a multiple of 32 with zero rows inside the kernel and M above 512 is
  * processed in chunks of 512 rows.  split_k in {0 (library picks), 1, 2, 4, 8, 16}.
- * From 288 rows on, with split_k = 0 and BF16 output, the weight is instead decoded once into a
+ * From 257 rows on, with split_k = 0 and BF16 output, the weight is instead decoded once into a
  * BF16 scratch [N, K] inside the workspace (nq_w4a4_decode_weight) and multiplied by
  * nq_bf16_gemm; nq_w4a4_gemm_workspace_bytes includes that scratch.
  * Requires q = 14, K % 128 == 0, (K / split_k) % 128 == 0.

@@ -303,7 +303,7 @@ constexpr int kChunkRows = 512;    // 8 wavefronts x 2 tiles x 32 rows
 // From this many rows on (BF16 output, automatic split) the weight is decoded once into a BF16
 // scratch [N][K] in the workspace and a dense BF16 GEMM multiplies: the fused kernel decodes a
 // block once per 512 rows and re-reads the activation once per 32 channels.
-constexpr int kDecodeOnceRows = 288;
+constexpr int kDecodeOnceRows = 257;
 
 bool decodes_once(int m, int k, int split_k) { return split_k == 0 && m >= kDecodeOnceRows && k % 128 == 0; }
 

@@ -609,9 +609,10 @@ def linear_packed_w4a4_mma_small_m_splitk_probe(activation: PreparedNQA4Activati
 
 # From this many rows on (BF16 output, automatic split) nq_w4a4_gemm decodes the weight once into a
 # BF16 scratch inside its workspace and multiplies with the dense matrix-core GEMM of the library
-# (nq_bf16_gemm); below, the fused kernel decodes inside the multiply.  Measured crossover on MI355X
-# at the 1B shapes: between 256 and 384 rows.
-DECODE_ONCE_ROWS = 288
+# (nq_bf16_gemm); below, the fused kernel decodes inside the multiply.  Measured on MI355X at the 1B
+# shapes: gate + up 50 us at 256 rows on the fused kernel, 101 us at 257 (a second token tile per
+# wavefront), 68 us on this route.
+DECODE_ONCE_ROWS = 257
 # up to this many rows a linear over resolved weights (K a multiple of 128) takes the decode GEMV,
 # which from five rows on multiplies on the matrix cores
 MATRIX_CORE_GEMV_ROWS = 16
@@ -901,7 +902,7 @@ def can_use_w4a4_gemm_grouped(activation: PreparedNQA4Activation, weights: Seque
 def linear_packed_w4a4_gemm_grouped(activation: PreparedNQA4Activation, weights: Sequence[PreparedNQRTLinear], *,
                                     checked: bool = False) -> list[torch.Tensor]:
     """The linears of the weights that share one activation (q, k and v; gate and up) in a prefill,
-    as one product.  From 288 rows on every weight is decoded once into its rows of one BF16 scratch
+    as one product.  From 257 rows on every weight is decoded once into its rows of one BF16 scratch
     and one dense matrix-core GEMM over the stacked rows stores each projection's columns to a BF16
     [M, N_i] output of its own; below, one launch of the fused kernel walks the channels of all the
     weights.  Same values as one `linear_packed_w4a4_mma_chunked_staged` per weight.  `checked`:

@@ -206,7 +206,7 @@ def test_grouped_prefill_linears_equal_one_call_per_weight(rt, oracle, m, k, siz
     assert not rt.can_use_w4a4_gemm_grouped(activation, weights[:1])
 
 
-@pytest.mark.parametrize("m,k,sizes", [(17, 512, (256, 64, 64)), (128, 2048, (2048, 512, 512)), (287, 1024, (512, 512)),
+@pytest.mark.parametrize("m,k,sizes", [(17, 512, (256, 64, 64)), (128, 2048, (2048, 512, 512)), (256, 1024, (512, 512)),
                                        (40, 256, (32, 64, 96, 32)), (128, 2048, (8192, 8192)), (100, 8192, (64, 32)),
                                        (96, 512, (8192, 8192)), (250, 256, (8192, 4096, 4160)), (95, 256, (8192, 8192))])
 def test_grouped_short_prefill_linears_equal_one_launch_per_weight(rt, oracle, m, k, sizes):

@@ -95,7 +95,7 @@ def test_linears_over_random_shapes_match_oracle(rt, oracle, sweep_seed):
         if rng.integers(2):
             m = int(rng.integers(1, 17))                     # the decode kernels
         else:                                                # both prefill routes and their thresholds
-            m = int(rng.choice([17, 31, 32, 33, 64, 100, 128, 200, 287, 288, 300, 513, 600]))
+            m = int(rng.choice([17, 31, 32, 33, 64, 100, 128, 200, 256, 257, 300, 513, 600]))
         seed = int(rng.integers(1 << 31))
         case = (m, k, n_out, seed)
         _, wc, wb, wn = oracle_weight(oracle, n_out, k, seed=seed % 100000, dither_seed=seed)
@@ -412,9 +412,9 @@ def test_dense_gemm_and_grouped_linears_over_random_shapes(rt, oracle, sweep_see
             assert relative_error(bits(c.float()), ref) <= 2.0 ** -8, (tile, split, case)
     for _ in range(12):
         k = int(rng.choice([256, 512, 1024, 2048]))
-        m = int(rng.choice([17, 40, 100, 128, 287, 288, 300, 600]))
-        count = int(rng.integers(2, 5 if m < 288 else 4))
-        unit = 32 if m < 288 else 256
+        m = int(rng.choice([17, 40, 100, 128, 256, 257, 300, 600]))
+        count = int(rng.integers(2, 5 if m < rt.DECODE_ONCE_ROWS else 4))
+        unit = 32 if m < rt.DECODE_ONCE_ROWS else 256
         sizes = [unit * int(rng.integers(1, 4)) for _ in range(count)]
         case = (m, k, sizes)
         weights = []
@@ -432,7 +432,7 @@ def test_dense_gemm_and_grouped_linears_over_random_shapes(rt, oracle, sweep_see
         while split < 16 and tiles * split < 256 and (k // (split * 2)) % 128 == 0:
             split *= 2
         for out, weight in zip(grouped, weights):
-            alone = (rt._gemm(activation, weight, output_dtype=torch.bfloat16, split_k=split) if m < 288
+            alone = (rt._gemm(activation, weight, output_dtype=torch.bfloat16, split_k=split) if m < rt.DECODE_ONCE_ROWS
                      else rt.linear_packed_w4a4_mma_chunked_staged(activation, weight))
             assert torch.equal(out, alone), case
 
