@@ -552,7 +552,7 @@ int nq_attention_output_stage(const void *workspace_dev, int64_t rows, int q_hea
  * (1..4) resolved weights on those rows; all outputs bit for bit those of the two calls.  The first
  * rows * slices workgroups of the grid run the encoder; the others decode their weights while the
  * encoder is still busy, wait until every encoder workgroup has set its flag word, and then
- * multiply.  rows in [1, 16] (8 for n = 8192), n = K in {2048, 8192}, four betas.
+ * multiply.  rows in [1, 16], n = K in {2048, 8192}, four betas.
  *   flags_dev            nq_fused_stage_linear_flag_words(rows, n) words of device memory, 16-byte
  *                        aligned (the library keeps several copies of a launch's flags, each in a
  *                        memory channel of its own, because every consumer polls them at once; a poll

@@ -637,15 +637,30 @@ attention_merge_kernel(const float *__restrict__ part_max, const float *__restri
 
 namespace {
 
-// Pages per chunk, from measurements over batches of 1 to 8 and tables of 23 to 512 pages: a
-// workgroup's time is mostly the latency of its first loads up to 4 pages and grows from there,
-// while every further chunk adds workgroups (a second round on the chip beyond about 768) and a
-// part to merge.  Tables of up to 64 pages: 4; longer ones: 8; 16 only when even that would
-// launch more than 384 (row, chunk) pairs.
+// Pages per chunk, from measurements of the appending launch over batches of 1 to 16, tables of 21 to
+// 256 pages and contexts from 150 tokens to the whole table (a launch has one workgroup per (row,
+// chunk, KV head) of the table, whatever the rows hold: the host does not know their lengths).  A
+// workgroup alone on the chip takes 8.8 us with up to 4 pages, 9.7 with 8 and 11 to 13 with 16, mostly
+// the latency of its dependent loads; two workgroups on a compute unit share its vector units for the
+// decode of their pages, and every chunk is a part to merge.  With eight KV heads 32 (row, chunk)
+// pairs are one workgroup per compute unit: the smallest chunk that stays within that, else 8 pages
+// up to 100 pairs and 16 beyond (8 rows of a 64-page table at full length: 28.4, 20.1, 21.1 us with
+// 4, 8, 16 pages; 8 rows of a 256-page table with mixed lengths: 64.0, 39.7, 35.6 us).  A table of at
+// most 32 pages is filled to a good part by the rows of a step, so none of its workgroups is idle:
+// there 4 pages while two workgroups per compute unit hold the launch (9 rows of 21 pages: 10.2,
+// 13.8, 11.5 us at 150 tokens), then 16 while one does (10 rows: 13.6, 13.7, 11.4 us).
 int pages_per_chunk_for(int batch, int max_pages) {
-    if (max_pages <= 64) return 4;
-    if ((int64_t)batch * ((max_pages + 7) / 8) > 384) return nq::kAttnMaxPagesPerChunk;
-    return 8;
+#ifdef NQ_ATTN_FORCE_PAGES                       // measuring builds only
+    return NQ_ATTN_FORCE_PAGES;
+#endif
+    const auto pairs = [&](int pages) { return (int64_t)batch * ((max_pages + pages - 1) / pages + 1); };
+    if (pairs(4) <= 32) return 4;
+    if (pairs(8) <= 32) return 8;
+    if (max_pages <= 32) {
+        if (pairs(4) <= 64) return 4;
+        if (pairs(16) <= 32) return nq::kAttnMaxPagesPerChunk;
+    }
+    return pairs(8) <= 100 ? 8 : nq::kAttnMaxPagesPerChunk;
 }
 
 int chunks_for(int batch, int max_pages) {

@@ -480,7 +480,12 @@ int launch_pair(const nq::EncoderArgs &e, const nq::GemvWeights &w, int consumer
 
 namespace {
 // encoder workgroups of a launch: rows x slices (a multiple of four, at most 256)
-int pair_producers(int64_t rows, int64_t n) { return (int)(rows * (n > 4096 ? n / 512 : (rows * 32 <= 256 ? 32 : 16))); }
+int pair_producers(int64_t rows, int64_t n) {
+    // rows of 8192 values: slices of 512 values, one pass each, up to eight rows; slices of 1024 values
+    // beyond, so that the consumers still find free compute units beside the encoder
+    if (n > 4096) return (int)(rows * (rows <= 8 ? n / 512 : n / 1024));
+    return (int)(rows * (rows * 32 <= 256 ? 32 : 16));
+}
 }  // namespace
 
 extern "C" int nq_fused_stage_linear_flag_words(int64_t rows, int64_t n) {
@@ -536,7 +541,6 @@ extern "C" int nq_fused_stage_linear(
         total_n += w_n[i];
     }
     const int m = (int)rows;
-    NQ_REQUIRE(n != 8192 || m <= 8, NQ_ERR_SHAPE, "nq_fused_stage_linear: rows of 8192 values come at most eight at a time");
     const int consumer = pair_takes_matrix_cores(m, total_n) ? 1 : 0;
     const int producers = pair_producers(rows, n);
     const int slices = producers / m;

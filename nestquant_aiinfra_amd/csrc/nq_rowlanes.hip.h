@@ -457,8 +457,10 @@ row_lanes_encode(const void *__restrict__ x_any, int x_is_f32, int64_t rows, int
             NQ_STAMP(4);
             return;
         }
-        const int pairs_per_slice = kForm == kFirstLanes ? 256 : (n >> 1) / slices;
-        for (int at = tid; at < pairs_per_slice; at += (int)blockDim.x) {
+        // (kFirstLanes: the 256 lanes that are left take the slice 256 pairs at a time, once for slices of
+        // 512 values)
+        const int pairs_per_slice = (n >> 1) / slices, pairs_per_pass = kForm == kFirstLanes ? 256 : (int)blockDim.x;
+        for (int at = tid; at < pairs_per_slice; at += pairs_per_pass) {
             const int p = slice * pairs_per_slice + at, b = p >> 2;
             float raw[8];
 #pragma unroll

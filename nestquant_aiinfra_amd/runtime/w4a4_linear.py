@@ -790,9 +790,9 @@ class StageLinearSync:
 
 
 def can_use_fused_stage_linear(rows: int, k: int, weights: Sequence[PreparedNQRTLinear]) -> bool:
-    """Whether `fused_stage_linear` takes this decode-step pair: up to 16 rows of 2048 values or up to
-    8 of 8192, one to four resolved weights of that K."""
-    return ((k == 2048 and 1 <= rows <= 16) or (k == 8192 and 1 <= rows <= 8)) and 1 <= len(weights) <= 4 and all(
+    """Whether `fused_stage_linear` takes this decode-step pair: up to 16 rows of 2048 or
+    8192 values, one to four resolved weights of that K."""
+    return k in (2048, 8192) and 1 <= rows <= 16 and 1 <= len(weights) <= 4 and all(
         w.resolved_words is not None and w.record.feature_count == k for w in weights)
 
 

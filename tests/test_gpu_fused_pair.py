@@ -49,7 +49,7 @@ PAIRS = [("qkv", 2048, (2048, 512, 512)), ("o_proj", 2048, (2048,)), ("gate_up",
          ("down_proj", 8192, (2048,)), ("ragged", 2048, (136, 2050)), ("ragged_long", 8192, (520,))]
 
 
-@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 8, 9, 13, 16])
 @pytest.mark.parametrize("name,k,sizes", PAIRS)
 def test_stage_and_linear_in_one_launch_equal_two_launches(rt, name, k, sizes, rows):
     weights = _weights(rt, k, sizes, seed=len(name))
@@ -81,8 +81,8 @@ def test_encoder_and_linear_in_one_launch_equal_two_launches(rt, name, k, sizes,
     """The rows themselves as the input stage (what a packed linear module does with its input: rotate,
     encode, multiply): modes "rows" and "rotated_rows" against `quantize_activation_cuda` with and without
     the rotation followed by the grouped linear, bit for bit."""
-    if k == 8192:
-        rows = min(rows, 7)                              # rows of 8192 values: up to eight per launch
+    if k == 8192 and rows == 5:
+        rows = 11                                        # slices of 1024 values from nine rows on
     weights = _weights(rt, k, sizes, seed=len(name))
     sync = rt.StageLinearSync(torch.device("cuda"))
     g = torch.Generator().manual_seed(300 * rows + k % 89)
@@ -176,5 +176,6 @@ def test_fused_pair_argument_checks(rt):
                               beta_table=_table(), gate=torch.zeros(2, 4096, dtype=torch.bfloat16, device="cuda"))
     with pytest.raises(TypeError):
         rt.fused_stage_linear(x.float(), weights, sync, mode="swiglu", beta_table=_table(), gate=x.float())
-    assert not rt.can_use_fused_stage_linear(9, 8192, _weights(rt, 8192, (520,), seed=11))
+    assert rt.can_use_fused_stage_linear(9, 8192, _weights(rt, 8192, (520,), seed=11))
+    assert not rt.can_use_fused_stage_linear(17, 8192, _weights(rt, 8192, (520,), seed=11))
     assert rt.can_use_fused_stage_linear(16, 2048, weights)
