@@ -48,17 +48,16 @@ extern "C" int nq_debug_pair_stamps(unsigned long long *out32) {
 namespace nq {
 
 // Every consumer workgroup polls the flags at once, and polls of one cache line queue up at the one
-// memory channel that holds it: the flag words therefore exist in kFlagCopies copies, kFlagStride words
-// apart, a producer sets its word in all of them (one store instruction) and consumer g reads copy
-// g % kFlagCopies.
-#ifndef NQ_PAIR_FLAG_COPIES
-#define NQ_PAIR_FLAG_COPIES 16
-#endif
-constexpr int kFlagCopies = NQ_PAIR_FLAG_COPIES;
-constexpr int kFlagStride = 256;         // words: the most producer workgroups a launch has
+// memory channel that holds it: the flag words therefore exist in several copies, a producer sets
+// its word in all of them (one store instruction) and consumer g reads copy g % copies.  A launch of
+// up to 256 producers lays its kFlagWords out as 16 copies 256 words apart, a larger one (up to 512)
+// as 8 copies 512 words apart.
+constexpr int kFlagWords = 4096;
+constexpr int kMaxProducers = 512;
 
 struct PairSync {
-    uint32_t *flags;         // kFlagCopies x kFlagStride words, one per producer workgroup and copy, zero when the launch starts
+    uint32_t *flags;         // copies x stride = kFlagWords words, one per producer workgroup and copy, zero when the launch starts
+    int copies, stride;
     uint32_t *previous;      // the flag words of the launch before this one on the stream (cleared here), or null
     int previous_count;
     uint32_t *status;        // set to 1 when a consumer's wait runs out (device or pinned host memory)
@@ -124,24 +123,28 @@ __device__ __forceinline__ void load_pieces_device_scope(const uint4 *const (&at
 
 // All lanes of a consumer workgroup: true once every producer's flag is set, false when the first
 // wavefront's polls ran out (it has then written the status word).  Ends behind a barrier.  A poll is
-// one 16-byte load per lane: four flag words each, so that the up to 256 flags of a launch cost one
-// trip to memory per poll (a load per flag and lane in turn made a poll of 256 flags four trips long).
+// one 16-byte load per lane, two for more than 256 producers, both requested before either is waited
+// for: four flag words each, so that the flags of a launch cost one trip to memory per poll (a load
+// per flag and lane in turn made a poll of 256 flags four trips long).
 __device__ __forceinline__ bool wait_for_producers(const PairSync &sync, int producers) {
     __shared__ __align__(16) int ready_shared[4];        // a multiple of 16 bytes, like every static array here
     if (threadIdx.x < 64) {
         const int first = 4 * (int)threadIdx.x;
-        const uint32_t *flags = sync.flags + ((int)blockIdx.x % kFlagCopies) * kFlagStride;
+        const uint32_t *flags = sync.flags + ((int)blockIdx.x % sync.copies) * sync.stride;
         const bool polls = first < producers;             // the flag words come in multiples of four
+        const bool polls_twice = first + 256 < producers;
         int spins = 0;
         bool ready;
         for (;;) {
-            bool mine = true;
-            if (polls) {
-                u32x4 four;
+            u32x4 four = u32x4{1u, 1u, 1u, 1u}, more = u32x4{1u, 1u, 1u, 1u};
+            if (polls_twice)
+                asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:1024 sc1\n\t"
+                             "s_waitcnt vmcnt(0)" : "=&v"(four), "=&v"(more) : "v"(flags + first) : "memory");
+            else if (polls)
                 asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
                              : "=&v"(four) : "v"(flags + first) : "memory");
-                mine = four.x != 0u && four.y != 0u && four.z != 0u && four.w != 0u;
-            }
+            const bool mine = four.x != 0u && four.y != 0u && four.z != 0u && four.w != 0u && more.x != 0u &&
+                              more.y != 0u && more.z != 0u && more.w != 0u;
             ready = __builtin_amdgcn_ballot_w64(!mine) == 0;
             if (ready || ++spins > sync.spin_limit) break;
             __builtin_amdgcn_s_sleep(4);
@@ -419,7 +422,7 @@ fused_stage_linear_kernel(EncoderArgs e, GemvWeights w, int producers, int late_
         NQ_PAIR_STAMP(stamp_slot, 2);
         __syncthreads();
         NQ_PAIR_STAMP(stamp_slot, 3);
-        if (threadIdx.x < kFlagCopies) store_word_device_scope(sync.flags + (int)threadIdx.x * kFlagStride + block, 1u);
+        if ((int)threadIdx.x < sync.copies) store_word_device_scope(sync.flags + (int)threadIdx.x * sync.stride + block, 1u);
         // the groups of channels that found no free slot beside the others are the producers' second job
         if (block >= late_count) return;
         __builtin_amdgcn_s_setprio(0);
@@ -479,18 +482,21 @@ int launch_pair(const nq::EncoderArgs &e, const nq::GemvWeights &w, int consumer
 }  // namespace
 
 namespace {
-// encoder workgroups of a launch: rows x slices (a multiple of four, at most 256)
-int pair_producers(int64_t rows, int64_t n) {
+// encoder workgroups of a launch: rows x slices (a multiple of four, at most kMaxProducers); `tiles`:
+// the linear's workgroups when they take 16 channels each
+int pair_producers(int64_t rows, int64_t n, int64_t tiles) {
     // rows of 8192 values: slices of 512 values, one pass each, up to eight rows; slices of 1024 values
     // beyond, so that the consumers still find free compute units beside the encoder
     if (n > 4096) return (int)(rows * (rows <= 8 ? n / 512 : n / 1024));
-    return (int)(rows * (rows * 32 <= 256 ? 32 : 16));
+    // rows of 2048 values: 32 slices of one pass each up to eight rows, and beyond while the launch as
+    // a whole still fits the chip (four 256-lane workgroups per compute unit); else 16 of two passes
+    return (int)(rows * (rows * 32 <= 256 || rows * 32 + tiles <= 4 * kComputeUnits ? 32 : 16));
 }
 }  // namespace
 
 extern "C" int nq_fused_stage_linear_flag_words(int64_t rows, int64_t n) {
     if (rows < 1 || rows > 16 || (n != 2048 && n != 8192)) return 0;
-    return nq::kFlagCopies * nq::kFlagStride;
+    return nq::kFlagWords;
 }
 
 extern "C" int nq_fused_stage_linear(
@@ -542,7 +548,9 @@ extern "C" int nq_fused_stage_linear(
     }
     const int m = (int)rows;
     const int consumer = pair_takes_matrix_cores(m, total_n) ? 1 : 0;
-    const int producers = pair_producers(rows, n);
+    int64_t tiles = 0;
+    for (int i = 0; i < count; i++) tiles += (w_n[i] + 15) / 16;
+    const int producers = pair_producers(rows, n, tiles);
     const int slices = producers / m;
     const int lanes = k / 8, subgroups = lanes / nq::kPairSubgroup;
     // Every workgroup of the launch must be resident at once: a consumer that started after another
@@ -608,7 +616,9 @@ extern "C" int nq_fused_stage_linear(
     // whole decode behind the rest of the launch: as many of them as there are producers become the
     // producers' second job (an encoder workgroup is done long before the first consumer).
     const int late = groups + producers > slots ? (groups + producers - slots < producers ? groups + producers - slots : producers) : 0;
-    nq::PairSync sync{flags_dev, previous_flags_dev, previous_flag_words, status_dev, spin_limit};
+    const int flag_stride = producers > 256 ? nq::kMaxProducers : 256;
+    nq::PairSync sync{flags_dev, nq::kFlagWords / flag_stride, flag_stride, previous_flags_dev, previous_flag_words, status_dev,
+                      spin_limit};
     const size_t lds_bytes = (size_t)(8 * ((k >> 3) + 8) + k + 4 + 8) * sizeof(float);
     const float sqrt_k = (float)sqrt((double)k);
     const int m_tile = m == 1 ? 1 : (m == 2 ? 2 : 4);
