@@ -197,7 +197,7 @@ int nq_w4a4_resolve_weight(const uint8_t *w_codes_dev, const uint8_t *w_beta_ids
  *                    NULL when that is 0)
  * Requires q = 14, K % 32 == 0, (K / split_k) % 32 == 0, 1 <= M <= 8.  With resolved weights
  * (16-byte aligned words, 8-byte aligned tails), K % 128 == 0 and split_k 0 or 1, M up to 16: above
- * eight rows, from three rows on, and for any row count when N fills 512 tiles of 16 channels,
+ * eight rows, from two rows on, and for any row count when N fills 512 tiles of 16 channels,
  * the products run on the matrix cores (v_mfma_f32_16x16x32_bf16 fed from registers), still one
  * decode per block.
  * Replaces: run_m1 / run_m1_splitk_probe / run_small_m / run_small_m_splitk_probe of the

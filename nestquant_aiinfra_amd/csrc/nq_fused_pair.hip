@@ -454,7 +454,7 @@ namespace {
 constexpr int kComputeUnits = 256;
 
 // mirrors the choice nq_w4a4_gemv_grouped makes between its two kernels
-bool pair_takes_matrix_cores(int m, int64_t total_n) { return m >= 3 || total_n >= 16 * 512; }
+bool pair_takes_matrix_cores(int m, int64_t total_n) { return m >= NQ_MFMA_FROM_ROWS || total_n >= 16 * 512; }
 
 template <int kPrologue, int kForm>
 int launch_pair(const nq::EncoderArgs &e, const nq::GemvWeights &w, int consumer, int m_tile, int r, int producers,

@@ -397,10 +397,12 @@ namespace {
 // The matrix-core kernel (resolved weights, 16-byte aligned streams) works in tiles of 16 / R
 // channels: R = 2 interleaved K ranges (K a multiple of 256) when 16-channel tiles would number
 // fewer than 192, else R = 1.  (R = 4 was measured at more than twice the time of R = 2.)  Above eight rows it is the only decode kernel; below, it is taken
-// from three rows on, where it saves the per-token vector work (us, vector units / matrix cores, at 3
-// and 4 rows: q/k/v 7.5, 7.5 / 7.0, 7.1; down_proj 12.2, 12.1 / 11.1, 11.2; behind the encoder in one
-// launch: q/k/v 11.0, 11.1 / 9.6, 9.7; o_proj 10.6, 10.8 / 9.5, 9.6; down_proj 18.4, 18.5 / 17.3, 17.9;
-// at two rows the two are even), and for any row count when even
+// from two rows on (NQ_MFMA_FROM_ROWS), where it saves the per-token vector work (us, vector units /
+// matrix cores, at 3 and 4 rows: q/k/v 7.5, 7.5 / 7.0, 7.1; down_proj 12.2, 12.1 / 11.1, 11.2; behind
+// the encoder in one launch: q/k/v 11.0, 11.1 / 9.6, 9.7; o_proj 10.6, 10.8 / 9.5, 9.6; down_proj 18.4,
+// 18.5 / 17.3, 17.9; at two rows the kernels alone are even, and a 1B decode step of two rows takes
+// 1.235 ms on the vector units and 1.195 on the matrix cores; at one row 1.166 and 1.183), and for any
+// row count when even
 // R = 1 gives 512 tiles (gate/up), where it also beats the vector-unit kernel's reductions
 // (measured: 25.0 against 26.2 us at one row).
 constexpr int kMfmaGemvMaxRows = 16;
@@ -411,7 +413,7 @@ int mfma_gemv_ranges(int k, int64_t total_n) {
 
 bool takes_mfma_gemv(int m, int k, int64_t total_n, bool resolved) {
     if (!resolved || k % 128 != 0 || m > kMfmaGemvMaxRows) return false;
-    return m >= 3 || total_n >= 16 * 512;
+    return m >= NQ_MFMA_FROM_ROWS || total_n >= 16 * 512;
 }
 
 int launch_mfma_gemv(const void *act, const nq::GemvWeights &w, int ranges, int groups, int m, int k,

@@ -4,6 +4,11 @@
 #include "nq_e8.hip.h"
 #include "nq_host.h"
 
+// the row count from which the decode linears run on the matrix cores (measuring builds set another)
+#ifndef NQ_MFMA_FROM_ROWS
+#define NQ_MFMA_FROM_ROWS 2
+#endif
+
 namespace nq {
 
 

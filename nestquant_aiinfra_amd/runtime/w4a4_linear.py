@@ -614,7 +614,7 @@ def linear_packed_w4a4_mma_small_m_splitk_probe(activation: PreparedNQA4Activati
 # wavefront), 68 us on this route.
 DECODE_ONCE_ROWS = 257
 # up to this many rows a linear over resolved weights (K a multiple of 128) takes the decode GEMV,
-# which from three rows on multiplies on the matrix cores
+# which from two rows on multiplies on the matrix cores
 MATRIX_CORE_GEMV_ROWS = 16
 BF16_ROWS_LINEAR_MAX_ROWS = 16
 BF16_ROWS_LINEAR_K = (2048, 4096, 8192)
