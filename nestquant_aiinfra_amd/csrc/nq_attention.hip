@@ -219,10 +219,18 @@ __global__ void __launch_bounds__(kAttnThreads) attention_stage1_kernel(Attentio
     // A page stores the blocks of all KV heads of a token side by side, so the workgroups of one
     // (row, chunk) -- one per KV head -- fetch the same cache lines: they are numbered so that they
     // share an XCD and follow each other there (index = 8 * (kv_heads * (pair / 8) + head) + pair % 8).
+    // Pair p lands on XCD p % 8.  The pairs are numbered part by part, the rows of a part side by side
+    // and one place further round for every part (p = part * batch + (row + part) % batch): the rows'
+    // early chunks, the ones that every row has, then spread over the XCDs, and so do the chunks of a
+    // long row.  (Numbered row by row, chunk 0 of every row of a table of eight parts fell to XCD 0:
+    // 13.6 against 10 us for 8 rows of 150 tokens in a 25-page table.)  The hot tails, whose workgroups
+    // also append the step's token, are the first part.
     const int place = blockIdx.x >> 3, pair = (place / a.kv_heads) * 8 + (blockIdx.x & 7);
     const int g = place % a.kv_heads;
-    const int chunk = pair % (a.chunks + 1), row = pair / (a.chunks + 1);
-    if (row >= a.batch) return;                          // padding of the last group of eight pairs
+    const int order = pair / a.batch, seat = pair - order * a.batch;
+    if (order > a.chunks) return;                        // padding of the last group of eight pairs
+    const int row = (seat + a.batch - order % a.batch) % a.batch;
+    const int chunk = order == 0 ? a.chunks : order - 1;
     const bool is_hot = chunk == a.chunks;
     const bool appends = kWrites && is_hot;              // this workgroup owns the row's new token
     const int first_page = chunk * kAttnPagesPerChunk;
@@ -638,28 +646,21 @@ attention_merge_kernel(const float *__restrict__ part_max, const float *__restri
 namespace {
 
 // Pages per chunk, from measurements of the appending launch over batches of 1 to 16, tables of 21 to
-// 256 pages and contexts from 150 tokens to the whole table (a launch has one workgroup per (row,
+// 512 pages and contexts from 150 tokens to the whole table (a launch has one workgroup per (row,
 // chunk, KV head) of the table, whatever the rows hold: the host does not know their lengths).  A
-// workgroup alone on the chip takes 8.8 us with up to 4 pages, 9.7 with 8 and 11 to 13 with 16, mostly
+// workgroup alone on the chip takes 9 us with up to 4 pages, 10 with 8 and 11 to 13.5 with 16, mostly
 // the latency of its dependent loads; two workgroups on a compute unit share its vector units for the
 // decode of their pages, and every chunk is a part to merge.  With eight KV heads 32 (row, chunk)
-// pairs are one workgroup per compute unit: the smallest chunk that stays within that, else 8 pages
-// up to 100 pairs and 16 beyond (8 rows of a 64-page table at full length: 28.4, 20.1, 21.1 us with
-// 4, 8, 16 pages; 8 rows of a 256-page table with mixed lengths: 64.0, 39.7, 35.6 us).  A table of at
-// most 32 pages is filled to a good part by the rows of a step, so none of its workgroups is idle:
-// there 4 pages while two workgroups per compute unit hold the launch (9 rows of 21 pages: 10.2,
-// 13.8, 11.5 us at 150 tokens), then 16 while one does (10 rows: 13.6, 13.7, 11.4 us).
+// pairs are one workgroup per compute unit: 4 pages while the launch stays within that, 8 pages up
+// to 100 pairs, 16 beyond (us with 4 / 8 / 16 pages: 8 rows of a 21-page table, 150 tokens 9.3 /
+// 10.2 / 11.4, full 13.6 / 10.1 / 13.6; 8 rows of 64 pages full 27.1 / 18.5 / 17.4, half 16.9 / 12.5 /
+// 13.7; 8 rows of 256 pages with mixed lengths 52.5 / 33.2 / 32.1, full 89.6 / 50.0 / 42.1).
 int pages_per_chunk_for(int batch, int max_pages) {
 #ifdef NQ_ATTN_FORCE_PAGES                       // measuring builds only
     return NQ_ATTN_FORCE_PAGES;
 #endif
     const auto pairs = [&](int pages) { return (int64_t)batch * ((max_pages + pages - 1) / pages + 1); };
     if (pairs(4) <= 32) return 4;
-    if (pairs(8) <= 32) return 8;
-    if (max_pages <= 32) {
-        if (pairs(4) <= 64) return 4;
-        if (pairs(16) <= 32) return nq::kAttnMaxPagesPerChunk;
-    }
     return pairs(8) <= 100 ? 8 : nq::kAttnMaxPagesPerChunk;
 }
 

@@ -43,13 +43,13 @@ def test_host_side_validation_needs_no_gpu():
     status = lib.nq_dequantize_rows(None, None, None, None, 1, 64, 14, 1, -5, 0, None, 0, None)
     assert status == _native.NQ_ERR_ARGUMENT
     assert lib.nq_w4a4_gemv_workspace_bytes(1, 8192, 2048, 8, 1) == 8 * 2048 * 4
-    # the attention's partial results: the smallest chunk (4, 8, 16 pages) that keeps the launch within 32 (row, chunk)
-    # pairs, else 8 pages up to 100 pairs and 16 beyond; small tables 4 pages up to 64 pairs, then 16 within 32
+    # the attention's partial results: chunks of 4 pages while the launch stays within 32 (row, chunk) pairs,
+    # 8 pages up to 100 pairs, 16 beyond
     assert lib.nq_nqkv_attention_parts(8, 23) == 4 and lib.nq_nqkv_attention_parts(1, 64) == 17
     assert lib.nq_nqkv_attention_parts(8, 256) == 17 and lib.nq_nqkv_attention_parts(8, 400) == 26
     assert lib.nq_nqkv_attention_parts(1, 256) == 33 and lib.nq_nqkv_attention_parts(4, 21) == 7
-    assert lib.nq_nqkv_attention_parts(9, 21) == 7 and lib.nq_nqkv_attention_parts(10, 21) == 3
-    assert lib.nq_nqkv_attention_parts(12, 21) == 4 and lib.nq_nqkv_attention_parts(0, 5) == 0
+    assert lib.nq_nqkv_attention_parts(9, 21) == 4 and lib.nq_nqkv_attention_parts(16, 64) == 5
+    assert lib.nq_nqkv_attention_parts(12, 64) == 5 and lib.nq_nqkv_attention_parts(0, 5) == 0
     assert lib.nq_nqkv_attention_workspace_bytes(8, 32, 64, 23) == 8 * 32 * 4 * 66 * 4
     status = lib.nq_attention_output_stage(None, 8, 32, 128, 7, None, 14, None, 4, 1, None, None, None, None, None)
     assert status == _native.NQ_ERR_SHAPE and b"head_dim 128 is not 64" in lib.nq_last_error()
