@@ -108,9 +108,11 @@ __global__ void __launch_bounds__(kPrefillThreads) attention_prefill_kernel(Pref
     // The workgroups of one (row, token tile) -- one per KV head -- read the same cache lines of every
     // page (a page keeps the blocks of all KV heads of a token side by side): they are numbered so
     // that they share an XCD, hence an L2 (index = 8 * (kv_heads * (pair / 8) + head) + pair % 8;
-    // workgroups go to the eight XCDs in turn).
+    // workgroups go to the eight XCDs in turn).  A row's work is its context length, and the same eight
+    // pairs would meet the same XCD in every split of the context: the pairs of a group of eight move one
+    // place round per split, so that a long row's splits spread over the XCDs.
     const int tiles = (a.tokens + kTileTokens - 1) / kTileTokens;
-    const int place = blockIdx.x >> 3, pair = (place / a.kv_heads) * 8 + (blockIdx.x & 7);
+    const int place = blockIdx.x >> 3, pair = (place / a.kv_heads) * 8 + ((blockIdx.x + blockIdx.y) & 7);
     const int g = place % a.kv_heads, tile = pair % tiles, row = pair / tiles;
     if (row >= a.batch) return;                          // padding of the last group of eight pairs
     const int vec = 16 * wave + (lane & 15);             // this lane's query vector of every set (column of S^T and O^T)
