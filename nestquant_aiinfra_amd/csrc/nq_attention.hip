@@ -46,7 +46,6 @@ namespace nq {
 
 constexpr int kAttnThreads = 512;
 constexpr int kAttnMaxPagesPerChunk = 16;
-constexpr int kAttnMaxGroup = 8;
 
 struct AttentionArgs {
     const void *query;                 // [batch, q_heads, D]
