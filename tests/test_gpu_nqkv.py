@@ -295,14 +295,17 @@ def test_attention_ragged_batch_at_full_size(kv, oracle):
 
 
 @pytest.mark.parametrize("capacity,max_len,q_heads", [(4, 1024, 64), (8, 1024, 16), (1, 4096, 32), (2, 64, 8),
-                                                      (8, 6400, 32)])
+                                                      (8, 6400, 32), (3, 448, 32), (6, 400, 32), (12, 336, 16),
+                                                      (16, 1024, 32)])
 def test_attention_chunk_sizes(kv, oracle, capacity, max_len, q_heads):
-    """The context is cut into chunks of 4, 8 or 16 pages depending on batch and table width
-    (4 up to 64 pages, 16 from 8 x 400 pages): every chunk size, with contexts that end inside a
-    chunk, on a page edge and in the hot tail."""
+    """The context is cut into chunks of 4, 8 or 16 pages depending on batch and table width (4 pages
+    within 32 (row, chunk) pairs, 8 up to 100 pairs, 16 beyond), and the pairs are numbered part by
+    part and rotated: every chunk size, with contexts that end inside a chunk, on a page edge and in the
+    hot tail; eight parts a row (3 x 448), row counts that do not divide eight, more rows than XCDs."""
     rng = np.random.default_rng(capacity * max_len + q_heads)
     manager = _manager(kv, capacity=capacity, max_len=max_len)
-    lengths = [max_len, max_len // 2 + 5, 33, 16, max_len - 16, 7, 1, max_len // 4][:capacity]
+    lengths = [max_len, max_len // 2 + 5, 33, 16, max_len - 16, 7, 1, max_len // 4]
+    lengths = (lengths + [max(1, n - 3) for n in lengths])[:capacity]
     keys = [_bf16(oracle.hadamard(rng.standard_normal((n, HEADS, DIM)).astype(np.float32))) for n in lengths]
     values = [_bf16(rng.standard_normal((n, HEADS, DIM)).astype(np.float32)) for n in lengths]
     for s in range(capacity):
