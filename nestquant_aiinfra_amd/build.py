@@ -4,7 +4,9 @@
 
 `--define NQ_PHASE_STAMPS --output PATH` makes a measuring build beside the product library: the
 row encoder then stamps the wall clock at its phase boundaries (read with nq_debug_phase_stamps;
-`bench.py --only encode_phases --library PATH` prints the table).
+`bench.py --only encode_phases --library PATH` prints the table).  Two more names serve timing
+comparisons on one GPU: `NQ_ATTN_FORCE_PAGES=4|8|16` fixes the decode attention's pages per chunk,
+`NQ_MFMA_FROM_ROWS=N` the row count from which the decode linears run on the matrix cores.
 
 hipcc cross-compiles for gfx950 without a GPU.  Flags that are part of the contract:
   -ffp-contract=off   the codec's float32 operation order is specified; fused
